@@ -1,0 +1,43 @@
+// gemv_w8a32.h -- launch description of the int8 dequant GEMV kernel family.
+#pragma once
+
+#include "common.h"
+
+namespace bh {
+
+// What happens to the raw sums before they are stored.
+enum GemvEpilogue : int {
+  kEpiStore = 0,  // C = acc*scale (+ bias)
+  kEpiAccum = 1,  // C = C + acc*scale        (linalg.matmul accumulate / residual)
+  kEpiSiluMul = 2 // C = silu(acc0*s0) * (acc1*s1), two weight matrices
+};
+
+struct GemvArgs {
+  const float *A = nullptr;   // [M, K], row stride lda
+  int64_t lda = 0;
+  const int8_t *W0 = nullptr; // wave-tile packed [Kp, Np]
+  const int8_t *W1 = nullptr; // second matrix for kEpiSiluMul
+  const float *s0 = nullptr;  // [N]
+  const float *s1 = nullptr;
+  const float *bias = nullptr; // [N] or null; y = bias + acc*scale
+  float *C = nullptr;          // [M, N], row stride ldc
+  int64_t ldc = 0;
+  // Optional RMSNorm applied to A while it is staged:
+  //   x' = norm_w[k] * (x[k] * rsqrt(sum(x^2) * inv_k + eps))
+  const float *norm_w = nullptr;
+  float norm_eps = 0.f;
+  float norm_inv_k = 0.f;
+  int M = 1;
+  int64_t K = 0, N = 0;
+  int epilogue = kEpiStore;
+  void *workspace = nullptr;
+  size_t workspace_bytes = 0;
+};
+
+// Bytes of workspace a launch with these sizes may need (split-K partial sums
+// plus one arrival counter per block column).
+size_t gemv_workspace_bytes(int64_t M, int64_t K, int64_t N, bool dual);
+
+int launch_gemv(const GemvArgs &a, hipStream_t stream);
+
+} // namespace bh

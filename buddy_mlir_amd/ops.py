@@ -1,0 +1,99 @@
+"""Helpers that call libbuddy_hip.so on torch device tensors.
+
+torch is used for device memory and streams only; every computation here goes
+through the C ABI.  Nothing falls back to torch or to the CPU.
+"""
+from __future__ import annotations
+
+import torch
+
+from . import check, lib
+
+GEMV_ACCUMULATE = 1
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _dev(t: torch.Tensor, dtype) -> torch.Tensor:
+    if not t.is_cuda:
+        raise ValueError("expected a device tensor")
+    if t.dtype != dtype or not t.is_contiguous():
+        raise ValueError(f"expected contiguous {dtype}, got {t.dtype}")
+    return t
+
+
+def quantize_w8(w: torch.Tensor):
+    """Per-output-channel symmetric int8 quantization of W[K,N] on device."""
+    _dev(w, torch.float32)
+    K, N = w.shape
+    q = torch.empty((K, N), dtype=torch.int8, device=w.device)
+    s = torch.empty((N,), dtype=torch.float32, device=w.device)
+    check(lib().buddy_hip_quantize_w8(w.data_ptr(), K, N, q.data_ptr(),
+                                      s.data_ptr(), _stream()), "quantize_w8")
+    return q, s
+
+
+def pack_w8(q: torch.Tensor) -> torch.Tensor:
+    """Row-major int8 W[K,N] -> wave-tile packed bytes."""
+    _dev(q, torch.int8)
+    K, N = q.shape
+    nbytes = lib().buddy_hip_w8_packed_bytes(K, N)
+    out = torch.empty((nbytes,), dtype=torch.int8, device=q.device)
+    check(lib().buddy_hip_pack_w8(q.data_ptr(), K, N, out.data_ptr(), _stream()),
+          "pack_w8")
+    return out
+
+
+def unpack_w8(packed: torch.Tensor, K: int, N: int) -> torch.Tensor:
+    _dev(packed, torch.int8)
+    out = torch.empty((K, N), dtype=torch.int8, device=packed.device)
+    check(lib().buddy_hip_unpack_w8(packed.data_ptr(), K, N, out.data_ptr(),
+                                    _stream()), "unpack_w8")
+    return out
+
+
+class Workspace:
+    """Zero-initialised scratch for split-K partial sums."""
+
+    def __init__(self, nbytes: int, device="cuda"):
+        self.buf = torch.empty((max(nbytes, 16),), dtype=torch.uint8, device=device)
+        check(lib().buddy_hip_workspace_init(self.buf.data_ptr(), self.buf.numel(),
+                                             _stream()), "workspace_init")
+
+    @property
+    def ptr(self) -> int:
+        return self.buf.data_ptr()
+
+    @property
+    def nbytes(self) -> int:
+        return self.buf.numel()
+
+
+def gemv_workspace(M: int, K: int, N: int, device="cuda") -> Workspace:
+    return Workspace(lib().buddy_hip_gemv_workspace_bytes(M, K, N), device)
+
+
+def gemv_w8a32(x: torch.Tensor, packed: torch.Tensor, scale: torch.Tensor,
+               K: int, N: int, out: torch.Tensor | None = None,
+               accumulate: bool = False, workspace: Workspace | None = None):
+    """out[M,N] (+)= (x[M,K] . W[K,N]) * scale[N] with W wave-tile packed."""
+    _dev(x, torch.float32)
+    _dev(packed, torch.int8)
+    _dev(scale, torch.float32)
+    M = x.shape[0]
+    if x.shape != (M, K):
+        raise ValueError(f"x is {tuple(x.shape)}, expected ({M},{K})")
+    if out is None:
+        if accumulate:
+            raise ValueError("accumulate needs an output tensor")
+        out = torch.empty((M, N), dtype=torch.float32, device=x.device)
+    _dev(out, torch.float32)
+    if workspace is None:
+        workspace = gemv_workspace(M, K, N, x.device)
+    check(lib().buddy_hip_gemv_w8a32(
+        x.data_ptr(), packed.data_ptr(), scale.data_ptr(), out.data_ptr(), M, K,
+        N, GEMV_ACCUMULATE if accumulate else 0, workspace.ptr, workspace.nbytes,
+        _stream()), "gemv_w8a32")
+    return out

@@ -1,0 +1,289 @@
+"""ctypes/numpy binding of oracle/liboracle.so (the CPU checker).
+
+Test infrastructure: used by tests/, the smoke check and the benchmark's
+cpu_baseline leg only.
+"""
+from __future__ import annotations
+
+import ctypes
+import subprocess
+from ctypes import POINTER, Structure, c_float, c_int, c_int64, c_size_t, c_void_p
+from pathlib import Path
+
+import numpy as np
+
+ROOT = Path(__file__).resolve().parent.parent
+SO = ROOT / "oracle" / "liboracle.so"
+
+
+def build():
+    subprocess.run(["make", "-C", str(ROOT / "oracle"), "-s"], check=True)
+
+
+def _p(a):
+    return a.ctypes.data_as(c_void_p) if a is not None else None
+
+
+class Shape(Structure):
+    _fields_ = [(n, c_int64) for n in
+                ("layers", "hidden", "heads", "kv_heads", "head_dim", "inter",
+                 "vocab", "max_len")] + [("eps", c_float), ("attn_splits", c_int64)]
+
+
+class Layer(Structure):
+    _fields_ = [(n, c_void_p) for n in
+                ("ln1", "ln2", "wq", "wk", "wv", "wo", "sq", "sk", "sv", "so",
+                 "bq", "bk", "bv", "wg", "wu", "wd", "sg", "su", "sd")]
+
+
+class Model(Structure):
+    _fields_ = [("shape", Shape), ("embed", c_void_p), ("inv_freq", c_void_p),
+                ("layer", POINTER(Layer)), ("ln_f", c_void_p),
+                ("w_lm", c_void_p), ("s_lm", c_void_p)]
+
+
+class Oracle:
+    def __init__(self, lib):
+        self.lib = lib
+        lib.oracle_argmax_first.restype = c_int64
+        lib.oracle_decode_step.restype = c_int64
+        lib.oracle_num_threads.restype = c_int
+
+    # -- a1
+    def quantize_w8(self, W):
+        W = np.ascontiguousarray(W, dtype=np.float32)
+        K, N = W.shape
+        q = np.empty((K, N), np.int8)
+        s = np.empty((N,), np.float32)
+        self.lib.oracle_quantize_w8(_p(W), c_int64(K), c_int64(N), _p(q), _p(s))
+        return q, s
+
+    def quantize_w4(self, W):
+        W = np.ascontiguousarray(W, dtype=np.float32)
+        K, N = W.shape
+        q = np.empty((K, N), np.int8)
+        s = np.empty((N,), np.float32)
+        self.lib.oracle_quantize_w4(_p(W), c_int64(K), c_int64(N), _p(q), _p(s))
+        return q, s
+
+    # -- a3
+    def pack_panels(self, B, V=32):
+        B = np.ascontiguousarray(B)
+        K, N = B.shape
+        out = np.empty_like(B)
+        rc = self.lib.oracle_pack_panels(_p(B), c_int64(K), c_int64(N), c_int64(V),
+                                         c_size_t(B.itemsize), _p(out))
+        if rc:
+            raise ValueError("N not divisible by V")
+        return out
+
+    def unpack_panels(self, P, V=32):
+        P = np.ascontiguousarray(P)
+        K, N = P.shape
+        out = np.empty_like(P)
+        rc = self.lib.oracle_unpack_panels(_p(P), c_int64(K), c_int64(N),
+                                           c_int64(V), c_size_t(P.itemsize), _p(out))
+        if rc:
+            raise ValueError("N not divisible by V")
+        return out
+
+    # -- a4/a6
+    def gemv_packed_f32(self, A, flatB, C, K, N, V=32, zero_init=False):
+        A = np.ascontiguousarray(A, np.float32).reshape(-1)
+        flatB = np.ascontiguousarray(flatB, np.float32).reshape(-1)
+        C = np.array(C, np.float32).reshape(-1)
+        self.lib.oracle_gemv_packed_f32(_p(A), _p(flatB), _p(C), c_int64(K),
+                                        c_int64(N), c_int64(V), c_int(zero_init))
+        return C
+
+    def gemv_f32(self, A, B, C, V=32, zero_init=False):
+        B = np.ascontiguousarray(B, np.float32)
+        K, N = B.shape
+        A = np.ascontiguousarray(A, np.float32).reshape(-1)
+        C = np.array(C, np.float32).reshape(-1)
+        self.lib.oracle_gemv_f32(_p(A), _p(B), _p(C), c_int64(K), c_int64(N),
+                                 c_int64(V), c_int(zero_init))
+        return C
+
+    # -- a5
+    def dequant_gemv(self, A, W, scale, C=None):
+        W = np.ascontiguousarray(W, np.int8)
+        K, N = W.shape
+        A = np.ascontiguousarray(A, np.float32).reshape(-1)
+        scale = np.ascontiguousarray(scale, np.float32).reshape(-1)
+        C = np.zeros(N, np.float32) if C is None else np.array(C, np.float32).reshape(-1)
+        assert A.size == K and scale.size == N and C.size == N
+        self.lib.oracle_dequant_gemv_w8a32(_p(A), _p(W), _p(scale), _p(C),
+                                           c_int64(K), c_int64(N))
+        return C
+
+    def dequant_gemv_panels(self, A, Wp, scale, K, N, C=None):
+        Wp = np.ascontiguousarray(Wp, np.int8)
+        A = np.ascontiguousarray(A, np.float32).reshape(-1)
+        scale = np.ascontiguousarray(scale, np.float32).reshape(-1)
+        C = np.zeros(N, np.float32) if C is None else np.array(C, np.float32).reshape(-1)
+        self.lib.oracle_dequant_gemv_w8a32_panels(_p(A), _p(Wp), _p(scale), _p(C),
+                                                  c_int64(K), c_int64(N))
+        return C
+
+    # -- a7
+    def blis_gemm_f32(self, A, B, C):
+        A = np.ascontiguousarray(A, np.float32)
+        B = np.ascontiguousarray(B, np.float32)
+        C = np.array(C, np.float32)
+        M, K = A.shape
+        N = B.shape[1]
+        self.lib.oracle_blis_gemm_f32(_p(A), _p(B), _p(C), c_int64(M), c_int64(N),
+                                      c_int64(K))
+        return C
+
+    def blis_gemm_w8a32(self, A, W, scale, C=None):
+        A = np.ascontiguousarray(A, np.float32)
+        W = np.ascontiguousarray(W, np.int8)
+        scale = np.ascontiguousarray(scale, np.float32).reshape(-1)
+        M, K = A.shape
+        N = W.shape[1]
+        C = np.zeros((M, N), np.float32) if C is None else np.array(C, np.float32)
+        self.lib.oracle_blis_gemm_w8a32(_p(A), _p(W), _p(scale), _p(C), c_int64(M),
+                                        c_int64(N), c_int64(K))
+        return C
+
+    # -- a8
+    def gqa_decode_attention(self, q, kc, vc, mask, scale, num_splits=4):
+        q = np.ascontiguousarray(q, np.float32)
+        kc = np.ascontiguousarray(kc, np.float32)
+        vc = np.ascontiguousarray(vc, np.float32)
+        H, D = q.shape
+        HKV, L, _ = kc.shape
+        mask = None if mask is None else np.ascontiguousarray(mask, np.float32)
+        out = np.empty((H, D), np.float32)
+        lse = np.empty((H,), np.float32)
+        self.lib.oracle_gqa_decode_attention(
+            _p(q), _p(kc), _p(vc), _p(mask), _p(out), _p(lse), c_int64(H),
+            c_int64(HKV), c_int64(L), c_int64(D), c_float(scale),
+            c_int64(num_splits))
+        return out, lse
+
+    # -- a9
+    def prefill_flash_attention(self, q, k, v, mask, scale):
+        q = np.ascontiguousarray(q, np.float32)
+        k = np.ascontiguousarray(k, np.float32)
+        v = np.ascontiguousarray(v, np.float32)
+        H, Lq, D = q.shape
+        Lk = k.shape[1]
+        mask = None if mask is None else np.ascontiguousarray(mask, np.float32)
+        out = np.empty((H, Lq, D), np.float32)
+        self.lib.oracle_prefill_flash_attention(
+            _p(q), _p(k), _p(v), _p(mask), _p(out), c_int64(H), c_int64(Lq),
+            c_int64(Lk), c_int64(D), c_float(scale))
+        return out
+
+    # -- a10
+    def rmsnorm(self, x, w, eps=9.99999997e-7, inv_n=None):
+        x = np.ascontiguousarray(x, np.float32).reshape(-1)
+        w = np.ascontiguousarray(w, np.float32).reshape(-1)
+        n = x.size
+        inv_n = np.float32(1.0) / np.float32(n) if inv_n is None else inv_n
+        y = np.empty(n, np.float32)
+        self.lib.oracle_rmsnorm(_p(x), _p(w), _p(y), c_int64(n), c_float(inv_n),
+                                c_float(eps))
+        return y
+
+    def rope_cos_sin(self, inv_freq, pos):
+        inv_freq = np.ascontiguousarray(inv_freq, np.float32)
+        half = inv_freq.size
+        c = np.empty(2 * half, np.float32)
+        s = np.empty(2 * half, np.float32)
+        self.lib.oracle_rope_cos_sin(_p(inv_freq), c_int64(half), c_int64(pos),
+                                     _p(c), _p(s))
+        return c, s
+
+    def rope_apply(self, x, cosv, sinv):
+        x = np.array(x, np.float32)
+        H, D = x.shape
+        cosv = np.ascontiguousarray(cosv, np.float32)
+        sinv = np.ascontiguousarray(sinv, np.float32)
+        self.lib.oracle_rope_apply(_p(x), c_int64(H), c_int64(D), _p(cosv), _p(sinv))
+        return x
+
+    def silu_mul(self, g, u):
+        g = np.ascontiguousarray(g, np.float32).reshape(-1)
+        u = np.ascontiguousarray(u, np.float32).reshape(-1)
+        h = np.empty_like(g)
+        self.lib.oracle_silu_mul(_p(g), _p(u), _p(h), c_int64(g.size))
+        return h
+
+    # -- a11
+    def argmax_first(self, x):
+        x = np.ascontiguousarray(x, np.float32).reshape(-1)
+        return int(self.lib.oracle_argmax_first(_p(x), c_int64(x.size)))
+
+    # -- a14
+    def w8a8_quantize_activation(self, x):
+        x = np.ascontiguousarray(x, np.float32)
+        xq = np.empty(x.shape, np.int8)
+        s = c_float()
+        self.lib.oracle_w8a8_quantize_activation(_p(x), c_int64(x.size), _p(xq),
+                                                 ctypes.byref(s))
+        return xq, np.float32(s.value)
+
+    def w8a8_matmul(self, A, W, wscale):
+        A = np.ascontiguousarray(A, np.float32)
+        W = np.ascontiguousarray(W, np.int8)
+        wscale = np.ascontiguousarray(wscale, np.float32).reshape(-1)
+        M, K = A.shape
+        N = W.shape[1]
+        C = np.empty((M, N), np.float32)
+        acc = np.empty((M, N), np.int32)
+        self.lib.oracle_w8a8_matmul(_p(A), _p(W), _p(wscale), _p(C), _p(acc),
+                                    c_int64(M), c_int64(N), c_int64(K))
+        return C, acc
+
+    def num_threads(self):
+        return int(self.lib.oracle_num_threads())
+
+
+class OracleModel:
+    """Holds numpy weights and the ctypes structs that point at them."""
+
+    def __init__(self, oracle: Oracle, shape: dict, embed, inv_freq, layers, ln_f,
+                 w_lm, s_lm):
+        self.o = oracle
+        self.keep = [embed, inv_freq, ln_f, w_lm, s_lm, layers]
+        self.shape = shape
+        arr = (Layer * len(layers))()
+        for i, L in enumerate(layers):
+            for name, _ in Layer._fields_:
+                a = L.get(name)
+                setattr(arr[i], name, None if a is None else a.ctypes.data)
+        self.arr = arr
+        m = Model()
+        for k, v in shape.items():
+            setattr(m.shape, k, v)
+        m.embed = embed.ctypes.data
+        m.inv_freq = inv_freq.ctypes.data
+        m.layer = arr
+        m.ln_f = ln_f.ctypes.data
+        m.w_lm = w_lm.ctypes.data
+        m.s_lm = s_lm.ctypes.data
+        self.m = m
+
+    def decode_step(self, token, pos, kv):
+        V = self.shape["vocab"]
+        logits = np.empty(V, np.float32)
+        ptrs = (c_void_p * len(kv))(*[a.ctypes.data for a in kv])
+        tok = self.o.lib.oracle_decode_step(ctypes.byref(self.m), c_int64(token),
+                                            c_int64(pos), ptrs, _p(logits))
+        return int(tok), logits
+
+
+_cached = None
+
+
+def load() -> Oracle:
+    global _cached
+    if _cached is None:
+        if not SO.exists():
+            build()
+        _cached = Oracle(ctypes.CDLL(str(SO)))
+    return _cached
