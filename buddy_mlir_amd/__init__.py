@@ -87,10 +87,8 @@ def _declare(lib):
         "buddy_hip_pack_w8": (c_int, [vp, i64, i64, vp, vp]),
         "buddy_hip_unpack_w8": (c_int, [vp, i64, i64, vp, vp]),
         "buddy_hip_quantize_w8": (c_int, [vp, i64, i64, vp, vp, vp]),
-        "buddy_hip_gemv_workspace_bytes": (sz, [i64, i64, i64]),
-        "buddy_hip_workspace_init": (c_int, [vp, sz, vp]),
         "buddy_hip_gemv_w8a32": (c_int, [vp, vp, vp, vp, i64, i64, i64, c_uint,
-                                         vp, sz, vp]),
+                                         vp]),
         "buddy_hip_matmul_f32": (c_int, [vp, vp, vp, i64, i64, i64, c_uint, vp]),
         "_mlir_ciface_buddy_matmul_f32": (None, [vp, vp, vp]),
         "_mlir_ciface_buddy_dequant_matmul_i8_f32": (None, [vp, vp, vp, vp]),

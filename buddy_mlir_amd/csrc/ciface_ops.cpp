@@ -55,7 +55,7 @@ struct CachedWeight {
 struct OpContext {
   std::mutex mu;
   hipStream_t stream = nullptr;
-  DeviceBuffer a_buf, c_buf, w_stage, workspace;
+  DeviceBuffer a_buf, c_buf, w_stage;
   std::map<std::tuple<const void *, const void *, int64_t, int64_t>,
            CachedWeight>
       weights;
@@ -67,16 +67,6 @@ struct OpContext {
     if (hipGetDeviceCount(&n) != hipSuccess || n == 0)
       return fail(BUDDY_HIP_ERR_NO_DEVICE, "no HIP device available");
     BH_CHECK_HIP(hipStreamCreateWithFlags(&stream, hipStreamNonBlocking));
-    return BUDDY_HIP_OK;
-  }
-
-  int ensure_workspace(size_t bytes) {
-    if (bytes <= workspace.bytes)
-      return BUDDY_HIP_OK;
-    int rc = workspace.reserve(bytes);
-    if (rc)
-      return rc;
-    BH_CHECK_HIP(hipMemsetAsync(workspace.ptr, 0, workspace.bytes, stream));
     return BUDDY_HIP_OK;
   }
 };
@@ -221,9 +211,6 @@ int dequant_matmul(buddy_memref_f32_2d *A, buddy_memref_i8_2d *W,
                                     sizeof(float) * ldc, sizeof(float) * N, M,
                                     hipMemcpyHostToDevice, c.stream));
   }
-  rc = c.ensure_workspace(gemv_workspace_bytes(M, K, N, false));
-  if (rc)
-    return rc;
   for (int64_t m0 = 0; m0 < M; m0 += 16) {
     GemvArgs g;
     g.A = a_dev + m0 * K;
@@ -236,8 +223,6 @@ int dequant_matmul(buddy_memref_f32_2d *A, buddy_memref_i8_2d *W,
     g.K = K;
     g.N = N;
     g.epilogue = accumulate ? kEpiAccum : kEpiStore;
-    g.workspace = c.workspace.ptr;
-    g.workspace_bytes = c.workspace.bytes;
     rc = launch_gemv(g, c.stream);
     if (rc)
       return rc;

@@ -30,13 +30,7 @@ struct GemvArgs {
   int M = 1;
   int64_t K = 0, N = 0;
   int epilogue = kEpiStore;
-  void *workspace = nullptr;
-  size_t workspace_bytes = 0;
 };
-
-// Bytes of workspace a launch with these sizes may need (split-K partial sums
-// plus one arrival counter per block column).
-size_t gemv_workspace_bytes(int64_t M, int64_t K, int64_t N, bool dual);
 
 int launch_gemv(const GemvArgs &a, hipStream_t stream);
 

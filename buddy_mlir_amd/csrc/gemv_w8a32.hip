@@ -7,18 +7,22 @@
 //
 // The kernel is HBM-bound, so its shape follows the memory system:
 //  * weights live in 1 KiB wave tiles (16 channels x 64 k); one wavefront
-//    streams one channel group's K extent with 128-bit loads, 1 KiB per
-//    instruction, contiguous from tile to tile;
-//  * a workgroup is 4 wavefronts = 4 adjacent channel groups over the same k
-//    range, so the activation slice is staged in LDS once per 64 channels;
-//  * the k range is split over blockIdx.y when the matrix alone cannot fill
-//    256 CUs; partial sums meet in a workspace and the last workgroup to
-//    arrive (a ticket per block column) adds them in split order, so the result
-//    does not depend on arrival order;
-//  * the scale, bias, residual add and SiLU*up are applied to the finished sums
-//    in the same kernel, and RMSNorm can be applied to the activations while
-//    they are staged.
-// No MFMA: at M <= 16 the arithmetic is far below the bandwidth ridge.
+//    streams a contiguous run of tiles of one channel group with 128-bit
+//    loads, 1 KiB per instruction, the next batch of loads in flight while the
+//    current one is consumed;
+//  * a workgroup is G channel groups x KS k-slices of wavefronts.  Wide
+//    matrices (lm_head) use G=4, KS=1; narrow ones (down/o_proj) put up to 16
+//    wavefronts on one channel group so that 96 groups still keep ~1500
+//    wavefronts streaming.  The k-slices meet in LDS, in slice order, so the
+//    sum is deterministic and no workgroup ever waits for another one (cross-
+//    XCD traffic inside a kernel costs an L2 write-back on this part);
+//  * every wavefront stages its own slice of the activations in LDS
+//    (optionally multiplied by the RMSNorm weight, with the row's sum of
+//    squares gathered on the way; the common rsqrt factor is applied to the
+//    finished sums);
+//  * scale, bias, residual add and SiLU*up are applied to the finished sums in
+//    the same kernel.
+// No MFMA: at M = 1 the arithmetic is far below the bandwidth ridge.
 #include "gemv_w8a32.h"
 
 #include <cstdlib>
@@ -26,55 +30,61 @@
 namespace bh {
 namespace {
 
-constexpr int kWavesPerBlock = 4;
-constexpr int kThreads = kWavesPerBlock * kWave;
-constexpr int kMaxCounters = 4096;
-constexpr size_t kCounterBytes = kMaxCounters * sizeof(unsigned);
-constexpr size_t kMaxLdsBytes = 96 * 1024;
+constexpr int kMaxWaves = 16;            // wavefronts per workgroup
+constexpr int kXStride = 20;             // floats per (tile, k-group) in LDS:
+                                         // 16 used + 4 pad, conflict-free b128
+constexpr int kTileFloats = 4 * kXStride; // 80 floats of LDS per staged tile
+constexpr size_t kMaxLdsBytes = 144 * 1024;
 
 struct GemvPlan {
-  int64_t chunks, groups, np;
-  int bx, splits, cps;
-  size_t lds_bytes, partial_bytes;
+  int64_t chunks, groups;
+  int G, KS, waves, tiles_per_round, blocks;
+  size_t lds_bytes;
 };
 
-int target_blocks() {
+int target_waves() {
   static int v = [] {
-    const char *e = getenv("BUDDY_HIP_GEMV_TARGET_BLOCKS");
+    const char *e = getenv("BUDDY_HIP_GEMV_TARGET_WAVES");
     int t = e ? atoi(e) : 0;
-    return t > 0 ? t : 1024;
+    return t > 0 ? t : 2048;
   }();
   return v;
 }
 
 GemvPlan make_plan(int64_t M, int64_t K, int64_t N, bool dual) {
+  (void)dual;
   GemvPlan p;
   p.chunks = ceil_div(K, kTileK);
   p.groups = ceil_div(N, kTileN);
-  p.np = p.groups * kTileN;
-  p.bx = (int)ceil_div(p.groups, kWavesPerBlock);
-  // enough workgroups to cover 256 CUs several times over, but at least two
-  // tiles per wavefront
-  int64_t want = ceil_div(target_blocks(), p.bx);
-  int64_t max_by_work = p.chunks / 2 > 0 ? p.chunks / 2 : 1;
-  int64_t s = want < max_by_work ? want : max_by_work;
-  if (s < 1)
-    s = 1;
-  // the activation slice of one split must fit in LDS
-  const int64_t max_cps = (int64_t)(kMaxLdsBytes / (sizeof(float) * kTileK * M));
-  int64_t cps = ceil_div(p.chunks, s);
-  if (cps > max_cps)
-    cps = max_cps;
-  p.cps = (int)cps;
-  p.splits = (int)ceil_div(p.chunks, cps);
-  if (p.bx > kMaxCounters) { // never split matrices that wide
-    p.splits = 1;
-    p.cps = (int)p.chunks;
-  }
-  p.lds_bytes = sizeof(float) * (size_t)M * p.cps * kTileK + 64 * sizeof(float);
-  p.partial_bytes = p.splits > 1 ? sizeof(float) * (size_t)p.splits *
-                                       (dual ? 2 : 1) * M * p.np
-                                 : 0;
+  // k-slices per channel group: enough wavefronts to cover 256 CUs several
+  // times, but at least two tiles per wavefront
+  int ks = 1;
+  while (ks < kMaxWaves && p.groups * ks < target_waves() &&
+         p.chunks / (ks * 2) >= 2)
+    ks *= 2;
+  // four staged tiles per wavefront must fit in LDS for every row
+  auto red_bytes = [&](int waves) {
+    return sizeof(float) * waves * (size_t)M * (2 * 16 + 1);
+  };
+  auto round_bytes = [&](int waves, int64_t tiles) {
+    return sizeof(float) * kTileFloats * (size_t)M * waves * (size_t)tiles;
+  };
+  while (ks > 1 && round_bytes(ks < 4 ? 4 : ks, 4) + red_bytes(ks < 4 ? 4 : ks) >
+                       kMaxLdsBytes)
+    ks /= 2;
+  p.KS = ks;
+  p.waves = ks < 4 ? 4 : ks;
+  while (p.waves > ks && round_bytes(p.waves, 4) + red_bytes(p.waves) > kMaxLdsBytes)
+    p.waves /= 2; // fewer channel groups per workgroup
+  p.G = p.waves / ks;
+  p.blocks = (int)ceil_div(p.groups, p.G);
+  const int64_t tiles = ceil_div(p.chunks, ks);
+  int64_t cap = (int64_t)((kMaxLdsBytes - red_bytes(p.waves)) / round_bytes(p.waves, 1));
+  cap = cap / 4 * 4; // rounds are whole batches of four tiles
+  if (cap < 4)
+    cap = 4;
+  p.tiles_per_round = (int)(tiles < cap ? round_up(tiles, 4) : cap);
+  p.lds_bytes = round_bytes(p.waves, p.tiles_per_round) + red_bytes(p.waves);
   return p;
 }
 
@@ -83,11 +93,10 @@ struct KernelArgs {
   const int4 *W0, *W1;
   const float *s0, *s1, *bias, *norm_w;
   float *C;
-  float *partial;
-  unsigned *counters;
   int64_t lda, ldc;
   float norm_eps, norm_inv_k;
-  int K, N, np, groups, chunks, cps, splits;
+  int K, N, groups, chunks;
+  int G, KS, tiles_per_round;
   int rows; // valid rows; the kernel is compiled for the next power of two
 };
 
@@ -103,10 +112,10 @@ __device__ __forceinline__ float byte_to_float(int v, int j) {
   return (float)(signed char)(v >> (8 * j));
 }
 
-// acc[m] += sum_j x[m][j] * w[j] for the lane's 16 k values.
+// acc[m] += sum_j x[m][j] * w[j] for the lane's 16 k values of one tile.
 template <int M>
 __device__ __forceinline__ void fma_tile(const int4 &w, const float *xl,
-                                         int kspan, float (&acc)[M]) {
+                                         int row_stride, float (&acc)[M]) {
   float wf[16];
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
@@ -117,7 +126,7 @@ __device__ __forceinline__ void fma_tile(const int4 &w, const float *xl,
   }
 #pragma unroll
   for (int m = 0; m < M; ++m) {
-    const float4 *xv = reinterpret_cast<const float4 *>(xl + m * kspan);
+    const float4 *xv = reinterpret_cast<const float4 *>(xl + m * row_stride);
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
       const float4 x = xv[q];
@@ -152,105 +161,133 @@ __device__ __forceinline__ void finish(const KernelArgs &a, int m, int n,
 }
 
 template <int M, int EPI, bool NORM>
-__global__ void __launch_bounds__(kThreads) gemv_w8a32_kernel(KernelArgs a) {
+__global__ void __launch_bounds__(kMaxWaves *kWave)
+    gemv_w8a32_kernel(KernelArgs a) {
   constexpr bool DUAL = (EPI == kEpiSiluMul);
+  constexpr int U = 4; // weight loads in flight per matrix
   extern __shared__ float lds[];
   const int tid = threadIdx.x;
   const int wave = tid >> 6, lane = tid & 63;
-  const int g = blockIdx.x * kWavesPerBlock + wave;
-  const int split = blockIdx.y;
-  const int c0 = split * a.cps;
-  const int nch = min(a.cps, a.chunks - c0);
-  const int k0 = c0 * kTileK;
-  const int kspan = a.cps * kTileK;
-  float *xs = lds;
-  float *red = lds + M * kspan;
+  const int nwaves = a.G * a.KS;
+  const int gl = wave / a.KS, ks = wave % a.KS;
+  const int g = blockIdx.x * a.G + gl;
+  const bool live = g < a.groups;
+  // this wavefront's contiguous run of tiles
+  const int per = (a.chunks + a.KS - 1) / a.KS;
+  const int t0 = min(ks * per, a.chunks);
+  const int t1 = min(t0 + per, a.chunks);
+  const int TR = a.tiles_per_round;
+  const int row_stride = TR * kTileFloats;
+  float *xs = lds + (size_t)wave * M * row_stride;
+  float *red = lds + (size_t)nwaves * M * row_stride;
 
-  // ---- stage the activation slice (optionally RMS-normalised) ------------
-  float rms[M];
-#pragma unroll
-  for (int m = 0; m < M; ++m)
-    rms[m] = 1.0f;
-  if (NORM) {
-    // sum of squares over the whole row, every workgroup for itself
-    float ss[M];
-#pragma unroll
-    for (int m = 0; m < M; ++m) {
-      float s = 0.f;
-      for (int k = tid; k < (m < a.rows ? a.K : 0); k += kThreads) {
-        const float v = a.A[(int64_t)m * a.lda + k];
-        s = fmaf(v, v, s);
-      }
-      ss[m] = wave_sum(s);
-    }
-    if (lane == 0) {
-#pragma unroll
-      for (int m = 0; m < M; ++m)
-        red[wave * 16 + m] = ss[m];
-    }
-    __syncthreads();
-#pragma unroll
-    for (int m = 0; m < M; ++m) {
-      const float tot = (red[m] + red[16 + m]) + (red[32 + m] + red[48 + m]);
-      rms[m] = 1.0f / sqrtf(tot * a.norm_inv_k + a.norm_eps);
-    }
-  }
-  {
-    const int span = nch * kTileK;
-#pragma unroll
-    for (int m = 0; m < M; ++m) {
-      for (int kk = tid; kk < span; kk += kThreads) {
-        const int k = k0 + kk;
-        const bool live = k < a.K && m < a.rows;
-        float v = live ? a.A[(int64_t)m * a.lda + k] : 0.f;
-        if (NORM && live)
-          v = a.norm_w[k] * (v * rms[m]);
-        xs[m * kspan + kk] = v;
-      }
-    }
-  }
-  __syncthreads();
-
-  // ---- stream this wavefront's channel group -----------------------------
-  float acc0[M], acc1[M]; // acc1 is dead code unless DUAL
+  float acc0[M], acc1[M], ss[M]; // acc1 is dead code unless DUAL
 #pragma unroll
   for (int m = 0; m < M; ++m) {
     acc0[m] = 0.f;
     acc1[m] = 0.f;
+    ss[m] = 0.f;
+  }
+  const size_t wbase = ((size_t)(live ? g : 0) * a.chunks) * 64 + lane;
+  const int4 *w0 = a.W0 + wbase;
+  const int4 *w1 = DUAL ? a.W1 + wbase : a.W0 + wbase;
+  // where this lane's float4 of a 256-float staging load lands in LDS
+  const int st_off = ((lane >> 4) * 4 + ((lane & 15) >> 2)) * kXStride +
+                     (lane & 3) * 4;
+  const float *xl = xs + (lane >> 4) * kXStride;
+
+  const int nrounds = (per + TR - 1) / TR; // same for every wavefront
+  const int kend = min(a.K, t1 * kTileK);   // this wavefront's k range ends here
+  for (int rd = 0; rd < nrounds; ++rd) {
+    const int r0 = t0 + rd * TR;
+    const int r1 = min(r0 + TR, t1);
+    // ---- first batch of weight loads goes out before anything else -------
+    int4 wa[U], wb[U];
+    if (r0 < r1) {
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int t = min(r0 + u, a.chunks - 1);
+        wa[u] = load_stream(w0 + (size_t)t * 64);
+        if (DUAL)
+          wb[u] = load_stream(w1 + (size_t)t * 64);
+      }
+    }
+    // ---- stage this wavefront's slice of the activations -----------------
+    if (rd != 0)
+      __syncthreads(); // everyone is done with the previous round's LDS
+    for (int i = 0; i < (r1 - r0 + 3) / 4; ++i) {
+      const int k = (r0 + 4 * i) * kTileK + lane * 4;
+      float4 nw = make_float4(1.f, 1.f, 1.f, 1.f);
+      const bool in = k + 3 < kend;
+      if (NORM) {
+        if (in)
+          nw = *reinterpret_cast<const float4 *>(a.norm_w + k);
+        else
+          nw = make_float4(k < kend ? a.norm_w[k] : 0.f,
+                           k + 1 < kend ? a.norm_w[k + 1] : 0.f,
+                           k + 2 < kend ? a.norm_w[k + 2] : 0.f, 0.f);
+      }
+#pragma unroll
+      for (int m = 0; m < M; ++m) {
+        float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (m < a.rows) {
+          const float *src = a.A + (int64_t)m * a.lda + k;
+          if (in && ((reinterpret_cast<uintptr_t>(src) & 15) == 0))
+            v = *reinterpret_cast<const float4 *>(src);
+          else
+            v = make_float4(k < kend ? src[0] : 0.f, k + 1 < kend ? src[1] : 0.f,
+                            k + 2 < kend ? src[2] : 0.f,
+                            k + 3 < kend ? src[3] : 0.f);
+        }
+        if (NORM) {
+          ss[m] = fmaf(v.x, v.x, ss[m]);
+          ss[m] = fmaf(v.y, v.y, ss[m]);
+          ss[m] = fmaf(v.z, v.z, ss[m]);
+          ss[m] = fmaf(v.w, v.w, ss[m]);
+          v.x *= nw.x;
+          v.y *= nw.y;
+          v.z *= nw.z;
+          v.w *= nw.w;
+        }
+        *reinterpret_cast<float4 *>(xs + m * row_stride + i * 4 * kTileFloats +
+                                    st_off) = v;
+      }
+    }
+    __syncthreads();
+    // ---- stream the tiles, next batch in flight while this one is used ----
+    for (int t = r0; t < r1; t += U) {
+      int4 na[U], nb[U];
+      const bool more = t + U < r1;
+      if (more) {
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          const int tt = min(t + U + u, a.chunks - 1);
+          na[u] = load_stream(w0 + (size_t)tt * 64);
+          if (DUAL)
+            nb[u] = load_stream(w1 + (size_t)tt * 64);
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        if (t + u < r1) {
+          const float *x = xl + (t + u - r0) * kTileFloats;
+          fma_tile<M>(wa[u], x, row_stride, acc0);
+          if (DUAL)
+            fma_tile<M>(wb[u], x, row_stride, acc1);
+        }
+      }
+      if (more) {
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          wa[u] = na[u];
+          if (DUAL)
+            wb[u] = nb[u];
+        }
+      }
+    }
   }
 
-  if (g < a.groups) {
-    const size_t base = ((size_t)g * a.chunks + c0) * 64 + lane;
-    const int4 *w0 = a.W0 + base;
-    const int4 *w1 = DUAL ? a.W1 + base : nullptr;
-    const float *xl = xs + (lane >> 4) * 16;
-    constexpr int U = DUAL ? 2 : 4;
-    int c = 0;
-    for (; c + U <= nch; c += U) {
-      int4 wa[U], wb[DUAL ? U : 1];
-#pragma unroll
-      for (int u = 0; u < U; ++u) {
-        wa[u] = load_stream(w0 + (size_t)(c + u) * 64);
-        if (DUAL)
-          wb[u] = load_stream(w1 + (size_t)(c + u) * 64);
-      }
-#pragma unroll
-      for (int u = 0; u < U; ++u) {
-        fma_tile<M>(wa[u], xl + (c + u) * kTileK, kspan, acc0);
-        if (DUAL)
-          fma_tile<M>(wb[u], xl + (c + u) * kTileK, kspan, acc1);
-      }
-    }
-    for (; c < nch; ++c) {
-      const int4 wa = load_stream(w0 + (size_t)c * 64);
-      fma_tile<M>(wa, xl + c * kTileK, kspan, acc0);
-      if (DUAL) {
-        const int4 wb = load_stream(w1 + (size_t)c * 64);
-        fma_tile<M>(wb, xl + c * kTileK, kspan, acc1);
-      }
-    }
-  }
-  // the four 16-lane rows hold the four k sub-ranges of the same channels
+  // the four 16-lane rows hold four k sub-ranges of the same 16 channels
 #pragma unroll
   for (int m = 0; m < M; ++m) {
     acc0[m] += __shfl_xor(acc0[m], 16, 64);
@@ -259,60 +296,65 @@ __global__ void __launch_bounds__(kThreads) gemv_w8a32_kernel(KernelArgs a) {
       acc1[m] += __shfl_xor(acc1[m], 16, 64);
       acc1[m] += __shfl_xor(acc1[m], 32, 64);
     }
+    if (NORM)
+      ss[m] = wave_sum(ss[m]);
   }
-  const int n = g * kTileN + lane;
 
-  if (a.splits == 1) {
-    if (lane < kTileN && g < a.groups && n < a.N) {
+  // ---- k-slices of one channel group meet in LDS, in slice order ----------
+  if (a.KS > 1) {
+    float *mine = red + (size_t)wave * M * 33;
+    if (lane < 16) {
+#pragma unroll
+      for (int m = 0; m < M; ++m) {
+        mine[m * 33 + lane] = acc0[m];
+        if (DUAL)
+          mine[m * 33 + 16 + lane] = acc1[m];
+      }
+    }
+    if (NORM && lane == 0) {
 #pragma unroll
       for (int m = 0; m < M; ++m)
-        if (m < a.rows)
-          finish<EPI>(a, m, n, acc0[m], DUAL ? acc1[m] : 0.f);
+        mine[m * 33 + 32] = ss[m];
     }
-    return;
+    __syncthreads();
+    if (ks != 0)
+      return;
+    if (lane < 16) {
+#pragma unroll
+      for (int m = 0; m < M; ++m) {
+        float r0 = 0.f, r1 = 0.f, rs = 0.f;
+        for (int s = 0; s < a.KS; ++s) {
+          const float *o = red + (size_t)(wave + s) * M * 33 + m * 33;
+          r0 += o[lane];
+          if (DUAL)
+            r1 += o[16 + lane];
+          if (NORM)
+            rs += o[32];
+        }
+        acc0[m] = r0;
+        acc1[m] = r1;
+        ss[m] = rs;
+      }
+    }
   }
-
-  // ---- split-K: publish partial sums, last arrival reduces ---------------
-  constexpr int NMAT = DUAL ? 2 : 1;
-  if (lane < kTileN && g < a.groups) {
+  const int n = g * kTileN + lane;
+  if (lane < kTileN && live && n < a.N) {
 #pragma unroll
     for (int m = 0; m < M; ++m) {
-      a.partial[((size_t)(split * NMAT + 0) * M + m) * a.np + n] = acc0[m];
-      if (DUAL)
-        a.partial[((size_t)(split * NMAT + 1) * M + m) * a.np + n] = acc1[m];
+      if (m < a.rows) {
+        float v0 = acc0[m], v1 = acc1[m];
+        if (NORM) {
+          // x' = w (.) (x * r) with r = rsqrt(mean(x^2) + eps): r is common to
+          // the whole row, so it multiplies the finished sum
+          // (subgraph0_decode_simplify.mlir:60-72)
+          const float r = 1.0f / sqrtf(ss[m] * a.norm_inv_k + a.norm_eps);
+          v0 *= r;
+          v1 *= r;
+        }
+        finish<EPI>(a, m, n, v0, v1);
+      }
     }
   }
-  __threadfence();
-  __syncthreads();
-  __shared__ int is_last;
-  if (tid == 0) {
-    const unsigned t = atomicAdd(&a.counters[blockIdx.x], 1u);
-    is_last = (t == (unsigned)a.splits - 1);
-  }
-  __syncthreads();
-  if (!is_last)
-    return;
-  __threadfence();
-  const int nb = blockIdx.x * kWavesPerBlock * kTileN;
-  for (int idx = tid; idx < M * kWavesPerBlock * kTileN; idx += kThreads) {
-    const int m = idx / (kWavesPerBlock * kTileN);
-    const int nn = nb + idx % (kWavesPerBlock * kTileN);
-    if (nn >= a.N || m >= a.rows)
-      continue;
-    float r0 = 0.f, r1 = 0.f;
-    for (int s = 0; s < a.splits; ++s) {
-      r0 += __hip_atomic_load(
-          &a.partial[((size_t)(s * NMAT + 0) * M + m) * a.np + nn],
-          __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      if (DUAL)
-        r1 += __hip_atomic_load(
-            &a.partial[((size_t)(s * NMAT + 1) * M + m) * a.np + nn],
-            __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
-    finish<EPI>(a, m, nn, r0, r1);
-  }
-  if (tid == 0)
-    a.counters[blockIdx.x] = 0; // leave the workspace ready for the next launch
 }
 
 template <int M, int EPI, bool NORM>
@@ -322,10 +364,10 @@ int launch_one(const KernelArgs &ka, const GemvPlan &p, hipStream_t stream) {
   if (!attr_set) {
     BH_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
                                      hipFuncAttributeMaxDynamicSharedMemorySize,
-                                     (int)(kMaxLdsBytes + 1024)));
+                                     (int)(kMaxLdsBytes + 4096)));
     attr_set = true;
   }
-  hipLaunchKernelGGL(kernel, dim3(p.bx, p.splits), dim3(kThreads), p.lds_bytes,
+  hipLaunchKernelGGL(kernel, dim3(p.blocks), dim3(p.waves * kWave), p.lds_bytes,
                      stream, ka);
   BH_CHECK_HIP(hipGetLastError());
   return BUDDY_HIP_OK;
@@ -349,17 +391,11 @@ int launch_m(const GemvArgs &a, const KernelArgs &ka, const GemvPlan &p,
   return fail(BUDDY_HIP_ERR_ARG, "gemv: unknown epilogue %d", a.epilogue);
 }
 
-} // namespace
-
-size_t gemv_workspace_bytes(int64_t M, int64_t K, int64_t N, bool dual) {
-  if (M < 1 || K < 1 || N < 1)
-    return 0;
-  // rows beyond 16 are processed in slabs of at most 16
-  const int64_t mc = M > 16 ? 16 : M;
-  const int64_t m = mc <= 2 ? mc : mc <= 4 ? 4 : mc <= 8 ? 8 : 16;
-  const GemvPlan p = make_plan(m, K, N, dual);
-  return kCounterBytes + p.partial_bytes;
+int compiled_rows(int64_t M) {
+  return M <= 2 ? (int)M : M <= 4 ? 4 : M <= 8 ? 8 : 16;
 }
+
+} // namespace
 
 int launch_gemv(const GemvArgs &a, hipStream_t stream) {
   BH_REQUIRE(a.A && a.W0 && a.s0 && a.C, "gemv: null pointer");
@@ -372,16 +408,12 @@ int launch_gemv(const GemvArgs &a, hipStream_t stream) {
   BH_REQUIRE((reinterpret_cast<uintptr_t>(a.W0) & 15) == 0 &&
                  (reinterpret_cast<uintptr_t>(a.W1) & 15) == 0,
              "gemv: packed weights must be 16-byte aligned");
+  BH_REQUIRE(!a.norm_w || (reinterpret_cast<uintptr_t>(a.norm_w) & 15) == 0,
+             "gemv: norm weight must be 16-byte aligned");
   // the kernel is compiled for 1, 2, 4, 8 and 16 rows; extra rows are zero-
   // filled in LDS and never stored
-  const int mt = a.M <= 2 ? a.M : a.M <= 4 ? 4 : a.M <= 8 ? 8 : 16;
+  const int mt = compiled_rows(a.M);
   const GemvPlan p = make_plan(mt, a.K, a.N, dual);
-  if (p.splits > 1) {
-    if (!a.workspace || a.workspace_bytes < kCounterBytes + p.partial_bytes)
-      return fail(BUDDY_HIP_ERR_WORKSPACE,
-                  "gemv: workspace of %zu bytes needed, %zu given",
-                  kCounterBytes + p.partial_bytes, a.workspace_bytes);
-  }
   KernelArgs ka;
   ka.A = a.A;
   ka.W0 = reinterpret_cast<const int4 *>(a.W0);
@@ -391,52 +423,34 @@ int launch_gemv(const GemvArgs &a, hipStream_t stream) {
   ka.bias = a.bias;
   ka.norm_w = a.norm_w;
   ka.C = a.C;
-  ka.counters = reinterpret_cast<unsigned *>(a.workspace);
-  ka.partial = a.workspace ? reinterpret_cast<float *>(
-                                 static_cast<char *>(a.workspace) + kCounterBytes)
-                           : nullptr;
   ka.lda = a.lda;
   ka.ldc = a.ldc;
   ka.norm_eps = a.norm_eps;
   ka.norm_inv_k = a.norm_inv_k;
   ka.K = (int)a.K;
   ka.N = (int)a.N;
-  ka.np = (int)p.np;
   ka.groups = (int)p.groups;
   ka.chunks = (int)p.chunks;
-  ka.cps = p.cps;
-  ka.splits = p.splits;
+  ka.G = p.G;
+  ka.KS = p.KS;
+  ka.tiles_per_round = p.tiles_per_round;
   ka.rows = a.M;
-  if (a.M == 1) return launch_m<1>(a, ka, p, stream);
-  if (a.M == 2) return launch_m<2>(a, ka, p, stream);
-  if (a.M <= 4) return launch_m<4>(a, ka, p, stream);
-  if (a.M <= 8) return launch_m<8>(a, ka, p, stream);
-  if (a.M <= 16) return launch_m<16>(a, ka, p, stream);
-  return fail(BUDDY_HIP_ERR_ARG, "gemv: M=%d outside 1..16", a.M);
+  switch (mt) {
+  case 1: return launch_m<1>(a, ka, p, stream);
+  case 2: return launch_m<2>(a, ka, p, stream);
+  case 4: return launch_m<4>(a, ka, p, stream);
+  case 8: return launch_m<8>(a, ka, p, stream);
+  default: return launch_m<16>(a, ka, p, stream);
+  }
 }
 
 } // namespace bh
 
 extern "C" {
 
-size_t buddy_hip_gemv_workspace_bytes(int64_t M, int64_t K, int64_t N) {
-  return bh::gemv_workspace_bytes(M, K, N, true);
-}
-
-int buddy_hip_workspace_init(void *workspace, size_t workspace_bytes,
-                             buddy_hip_stream stream) {
-  BH_REQUIRE(workspace || workspace_bytes == 0, "workspace_init: null pointer");
-  if (workspace_bytes == 0)
-    return BUDDY_HIP_OK;
-  BH_CHECK_HIP(
-      hipMemsetAsync(workspace, 0, workspace_bytes, bh::as_stream(stream)));
-  return BUDDY_HIP_OK;
-}
-
 int buddy_hip_gemv_w8a32(const float *A, const int8_t *packed,
                          const float *scale, float *C, int64_t M, int64_t K,
-                         int64_t N, unsigned flags, void *workspace,
-                         size_t workspace_bytes, buddy_hip_stream stream) {
+                         int64_t N, unsigned flags, buddy_hip_stream stream) {
   BH_REQUIRE(M >= 1, "gemv_w8a32: M=%lld", (long long)M);
   // rows beyond 16 go in slabs; each slab streams the weights once
   for (int64_t m0 = 0; m0 < M; m0 += 16) {
@@ -452,8 +466,6 @@ int buddy_hip_gemv_w8a32(const float *A, const int8_t *packed,
     a.N = N;
     a.epilogue = (flags & BUDDY_HIP_GEMV_ACCUMULATE) ? bh::kEpiAccum
                                                      : bh::kEpiStore;
-    a.workspace = workspace;
-    a.workspace_bytes = workspace_bytes;
     int rc = bh::launch_gemv(a, bh::as_stream(stream));
     if (rc)
       return rc;

@@ -54,30 +54,9 @@ def unpack_w8(packed: torch.Tensor, K: int, N: int) -> torch.Tensor:
     return out
 
 
-class Workspace:
-    """Zero-initialised scratch for split-K partial sums."""
-
-    def __init__(self, nbytes: int, device="cuda"):
-        self.buf = torch.empty((max(nbytes, 16),), dtype=torch.uint8, device=device)
-        check(lib().buddy_hip_workspace_init(self.buf.data_ptr(), self.buf.numel(),
-                                             _stream()), "workspace_init")
-
-    @property
-    def ptr(self) -> int:
-        return self.buf.data_ptr()
-
-    @property
-    def nbytes(self) -> int:
-        return self.buf.numel()
-
-
-def gemv_workspace(M: int, K: int, N: int, device="cuda") -> Workspace:
-    return Workspace(lib().buddy_hip_gemv_workspace_bytes(M, K, N), device)
-
-
 def gemv_w8a32(x: torch.Tensor, packed: torch.Tensor, scale: torch.Tensor,
                K: int, N: int, out: torch.Tensor | None = None,
-               accumulate: bool = False, workspace: Workspace | None = None):
+               accumulate: bool = False):
     """out[M,N] (+)= (x[M,K] . W[K,N]) * scale[N] with W wave-tile packed."""
     _dev(x, torch.float32)
     _dev(packed, torch.int8)
@@ -90,10 +69,7 @@ def gemv_w8a32(x: torch.Tensor, packed: torch.Tensor, scale: torch.Tensor,
             raise ValueError("accumulate needs an output tensor")
         out = torch.empty((M, N), dtype=torch.float32, device=x.device)
     _dev(out, torch.float32)
-    if workspace is None:
-        workspace = gemv_workspace(M, K, N, x.device)
     check(lib().buddy_hip_gemv_w8a32(
         x.data_ptr(), packed.data_ptr(), scale.data_ptr(), out.data_ptr(), M, K,
-        N, GEMV_ACCUMULATE if accumulate else 0, workspace.ptr, workspace.nbytes,
-        _stream()), "gemv_w8a32")
+        N, GEMV_ACCUMULATE if accumulate else 0, _stream()), "gemv_w8a32")
     return out

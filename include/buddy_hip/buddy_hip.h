@@ -20,8 +20,7 @@
  * is `void` by the reference's convention; failures also print one
  * `[buddy_hip] ...` line to stderr and are queryable with
  * buddy_hip_last_error().  Nothing unwinds through this boundary.
- * Calls on one stream are ordered; calls that share a workspace must not
- * overlap.
+ * Calls on one stream are ordered.
  */
 #ifndef BUDDY_HIP_H
 #define BUDDY_HIP_H
@@ -38,8 +37,7 @@ enum {
   BUDDY_HIP_OK = 0,
   BUDDY_HIP_ERR_ARG = 1,     /* shape / pointer / size check failed */
   BUDDY_HIP_ERR_HIP = 2,     /* a HIP runtime call failed */
-  BUDDY_HIP_ERR_NO_DEVICE = 3,
-  BUDDY_HIP_ERR_WORKSPACE = 4 /* workspace missing or too small */
+  BUDDY_HIP_ERR_NO_DEVICE = 3
 };
 
 /* ---- library ---------------------------------------------------------- */
@@ -81,15 +79,9 @@ enum {
                                    without it C = ... and C need not be
                                    initialised */
 };
-size_t buddy_hip_gemv_workspace_bytes(int64_t M, int64_t K, int64_t N);
 int buddy_hip_gemv_w8a32(const float *A, const int8_t *packed,
                          const float *scale, float *C, int64_t M, int64_t K,
-                         int64_t N, unsigned flags, void *workspace,
-                         size_t workspace_bytes, buddy_hip_stream stream);
-/* workspace must be zero-filled once before its first use (the kernels leave
- * it zeroed again); buddy_hip_workspace_init does that. */
-int buddy_hip_workspace_init(void *workspace, size_t workspace_bytes,
-                             buddy_hip_stream stream);
+                         int64_t N, unsigned flags, buddy_hip_stream stream);
 
 /* ---- plain f32 matmul ---------------------------------------------------
  * C (+)= A[M,K] * B[K,N], all dense row-major device pointers.  The f32
