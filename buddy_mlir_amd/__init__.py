@@ -89,6 +89,29 @@ def _declare(lib):
         "buddy_hip_quantize_w8": (c_int, [vp, i64, i64, vp, vp, vp]),
         "buddy_hip_gemv_w8a32": (c_int, [vp, vp, vp, vp, i64, i64, i64, c_uint,
                                          vp]),
+        "buddy_hip_linear_w8a32": (c_int, [vp, vp]),
+        "buddy_hip_rmsnorm": (c_int, [vp, vp, vp, c_int, c_int, c_float, vp]),
+        "buddy_hip_rope": (c_int, [vp, vp, vp, c_int, c_int, vp]),
+        "buddy_hip_silu_mul": (c_int, [vp, vp, vp, i64, vp]),
+        "buddy_hip_argmax_workspace_bytes": (sz, []),
+        "buddy_hip_argmax": (c_int, [vp, c_int, vp, vp, vp]),
+        "buddy_hip_attn_decode_workspace_bytes": (sz, [c_int, c_int]),
+        "buddy_hip_gqa_decode_attention": (c_int, [vp, vp, vp, vp, vp, vp, c_int,
+                                                   c_int, c_int, c_int, c_float,
+                                                   vp, sz, vp]),
+        "buddy_hip_session_create": (vp, [vp, vp]),
+        "buddy_hip_session_destroy": (None, [vp]),
+        "buddy_hip_session_set_globals": (c_int, [vp, vp, vp, vp, vp, vp]),
+        "buddy_hip_session_set_layer": (c_int, [vp, c_int, vp]),
+        "buddy_hip_session_set_kv": (c_int, [vp, c_int, vp]),
+        "buddy_hip_session_get_kv": (c_int, [vp, c_int, vp]),
+        "buddy_hip_session_use_graph": (c_int, [vp, c_int]),
+        "buddy_hip_session_decode": (c_int, [vp, c_int, c_int, vp, vp]),
+        "buddy_hip_session_decode_greedy": (c_int, [vp, c_int, c_int, c_int, vp]),
+        "buddy_hip_session_set_state": (c_int, [vp, c_int, c_int]),
+        "buddy_hip_session_enqueue_steps": (c_int, [vp, c_int]),
+        "buddy_hip_session_logits": (vp, [vp]),
+        "buddy_hip_session_stream": (vp, [vp]),
         "buddy_hip_matmul_f32": (c_int, [vp, vp, vp, i64, i64, i64, c_uint, vp]),
         "_mlir_ciface_buddy_matmul_f32": (None, [vp, vp, vp]),
         "_mlir_ciface_buddy_dequant_matmul_i8_f32": (None, [vp, vp, vp, vp]),

@@ -1,0 +1,24 @@
+// attn.h -- launch descriptions of the attention kernels.
+#pragma once
+
+#include "common.h"
+
+namespace bh {
+
+struct AttnDecodeArgs {
+  const float *qkv = nullptr;      // [heads*D | kv_heads*D | kv_heads*D], pre-RoPE
+  const float *inv_freq = nullptr; // [D/2]
+  const int *pos_ptr = nullptr;    // device scalar: index of the current token
+  float *kcache = nullptr;         // [kv_heads, max_len, D]
+  float *vcache = nullptr;
+  float *out = nullptr;            // [heads*D]
+  int heads = 0, kv_heads = 0, head_dim = 0, max_len = 0;
+  float scale = 0.f;
+  void *workspace = nullptr; // flash-decoding partials
+  size_t workspace_bytes = 0;
+};
+
+size_t attn_decode_workspace_bytes(int heads, int max_len);
+int launch_attn_decode(const AttnDecodeArgs &a, hipStream_t stream);
+
+} // namespace bh

@@ -1,0 +1,308 @@
+// attn_decode.hip -- GQA decode attention over a device-resident f32 KV cache,
+// with RoPE and the KV-cache write fused in.
+//
+// Replaces, for one decode step of one layer:
+//   * RoPE on q and k   (examples/BuddyDeepSeekR1/subgraph0_decode_simplify.mlir
+//                        :51-59 angles, :88-107 rotate-half)
+//   * cache[0, h, pos, :] = k' / v                       (same file :108-142)
+//   * gqa_attention_fused_op  (frontend/Python/ops/tosa.py:14130-14600):
+//     softmax(scale * q.K^T + mask) V with mask = 0 for k <= pos, -inf beyond,
+//     computed as flash-decoding partials over k ranges plus a combine.
+//
+// Differences from the reference kernel that follow from the hardware:
+//   * the cache is scanned up to pos only (masked positions contribute exactly
+//     zero in the reference, so skipping them changes nothing);
+//   * one workgroup serves all query heads of a KV head, so K and V rows are
+//     read once per group, not once per query head;
+//   * the k range is cut into chunks of 32 positions (more, smaller partials
+//     than the reference's 4): a decode step has only ~2 MB of KV per layer and
+//     is latency bound, so the chunks are what spreads it over the CUs.
+// Partials meet in a small workspace and a second kernel folds them in chunk
+// order with the reference's own combine rule.
+#include "attn.h"
+
+namespace bh {
+namespace {
+
+constexpr int kChunk = 32;       // cache positions per workgroup
+constexpr int kThreads = 256;
+constexpr int kMaxGroup = 8;     // query heads per KV head
+constexpr int kD = 128;          // head_dim this kernel is written for
+constexpr float kSeedM = -1.0e30f; // tosa.py:13971
+
+struct AttnArgs {
+  const float *qkv;      // [heads*D | kv_heads*D | kv_heads*D]
+  const float *inv_freq; // [D/2]
+  const int *pos_ptr;    // device scalar: index of the current token
+  float *kcache, *vcache; // [kv_heads, max_len, D]
+  float *part_acc;       // [heads, nchunks, D]
+  float *part_ml;        // [heads, nchunks, 2]
+  float *out;            // [heads*D]
+  int heads, kv_heads, group, max_len, nchunks;
+  float scale;
+};
+
+__global__ void __launch_bounds__(kThreads) attn_decode_partial(AttnArgs a) {
+  __shared__ float q_s[kMaxGroup][kD];
+  __shared__ float knew_s[kD], vnew_s[kD];
+  __shared__ float cos_s[kD / 2], sin_s[kD / 2];
+  __shared__ float sc_s[kMaxGroup][kChunk];
+  __shared__ float red_s[kThreads / 32][kMaxGroup][kD];
+  __shared__ float m_s[kMaxGroup], l_s[kMaxGroup];
+
+  const int tid = threadIdx.x;
+  const int chunk = blockIdx.x, kvh = blockIdx.y;
+  const int pos = *a.pos_ptr;
+  const int p0 = chunk * kChunk;
+  const int G = a.group;
+  const int h0 = kvh * G;
+
+  if (p0 > pos) { // nothing visible in this chunk: an empty partial
+    for (int i = tid; i < G * kD; i += kThreads)
+      a.part_acc[((size_t)(h0 + i / kD) * a.nchunks + chunk) * kD + i % kD] = 0.f;
+    if (tid < G) {
+      a.part_ml[((size_t)(h0 + tid) * a.nchunks + chunk) * 2 + 0] = kSeedM;
+      a.part_ml[((size_t)(h0 + tid) * a.nchunks + chunk) * 2 + 1] = 0.f;
+    }
+    return;
+  }
+  const int p1 = min(p0 + kChunk, pos + 1);
+  const int np = p1 - p0;
+  const bool has_new = pos >= p0 && pos < p1;
+
+  // ---- RoPE tables for this position -------------------------------------
+  if (tid < kD / 2) {
+    const float ang = a.inv_freq[tid] * (float)pos;
+    cos_s[tid] = cosf(ang);
+    sin_s[tid] = sinf(ang);
+  }
+  __syncthreads();
+  // q' = q*cos + cat(-q[64:], q[:64])*sin for the G heads of this KV head
+  for (int i = tid; i < G * kD; i += kThreads) {
+    const int h = i / kD, j = i % kD, jj = j & (kD / 2 - 1);
+    const float *q = a.qkv + (size_t)(h0 + h) * kD;
+    const float rot = j < kD / 2 ? -q[j + kD / 2] : q[j - kD / 2];
+    q_s[h][j] = q[j] * cos_s[jj] + rot * sin_s[jj];
+  }
+  if (has_new && tid < kD) {
+    const int j = tid, jj = j & (kD / 2 - 1);
+    const float *k = a.qkv + (size_t)a.heads * kD + (size_t)kvh * kD;
+    const float *v = k + (size_t)a.kv_heads * kD;
+    const float rot = j < kD / 2 ? -k[j + kD / 2] : k[j - kD / 2];
+    const float kn = k[j] * cos_s[jj] + rot * sin_s[jj];
+    knew_s[j] = kn;
+    vnew_s[j] = v[j];
+    a.kcache[((size_t)kvh * a.max_len + pos) * kD + j] = kn;
+    a.vcache[((size_t)kvh * a.max_len + pos) * kD + j] = v[j];
+  }
+  __syncthreads();
+
+  // ---- scores: 8 threads per position, 16 dims each ----------------------
+  {
+    const int p = tid >> 3, part = tid & 7;
+    float dot[kMaxGroup];
+#pragma unroll
+    for (int h = 0; h < kMaxGroup; ++h)
+      dot[h] = 0.f;
+    if (p < np) {
+      const bool is_new = (p0 + p == pos);
+      const float *krow = is_new ? knew_s
+                                 : a.kcache + ((size_t)kvh * a.max_len + p0 + p) * kD;
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        const int d = part * 16 + c * 4;
+        const float4 kv = *reinterpret_cast<const float4 *>(krow + d);
+#pragma unroll
+        for (int h = 0; h < kMaxGroup; ++h) {
+          if (h < G) {
+            const float4 qv = *reinterpret_cast<const float4 *>(&q_s[h][d]);
+            dot[h] = fmaf(qv.x, kv.x, dot[h]);
+            dot[h] = fmaf(qv.y, kv.y, dot[h]);
+            dot[h] = fmaf(qv.z, kv.z, dot[h]);
+            dot[h] = fmaf(qv.w, kv.w, dot[h]);
+          }
+        }
+      }
+    }
+#pragma unroll
+    for (int h = 0; h < kMaxGroup; ++h) {
+      dot[h] += __shfl_xor(dot[h], 1, 64);
+      dot[h] += __shfl_xor(dot[h], 2, 64);
+      dot[h] += __shfl_xor(dot[h], 4, 64);
+    }
+    if (part == 0 && p < kChunk) {
+#pragma unroll
+      for (int h = 0; h < kMaxGroup; ++h)
+        if (h < G)
+          sc_s[h][p] = p < np ? dot[h] * a.scale : -INFINITY;
+    }
+  }
+  __syncthreads();
+
+  // ---- per-head max, exp, sum over the chunk: one 32-lane half per head ----
+  {
+    const int h = tid >> 5, p = tid & 31;
+    if (h < G) {
+      const float s = sc_s[h][p];
+      float m = s;
+#pragma unroll
+      for (int o = 16; o > 0; o >>= 1)
+        m = fmaxf(m, __shfl_xor(m, o, 64));
+      const float e = expf(s - m); // -inf -> 0 for the positions beyond pos
+      float l = e;
+#pragma unroll
+      for (int o = 16; o > 0; o >>= 1)
+        l += __shfl_xor(l, o, 64);
+      sc_s[h][p] = e;
+      if (p == 0) {
+        m_s[h] = m;
+        l_s[h] = l;
+      }
+    }
+  }
+  __syncthreads();
+
+  // ---- acc[h][d] = sum_p e[h][p] * V[p][d]: 32 threads across d, 8 rows of p
+  {
+    const int dq = tid & 31, pg = tid >> 5;
+    float acc[kMaxGroup][4];
+#pragma unroll
+    for (int h = 0; h < kMaxGroup; ++h)
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        acc[h][j] = 0.f;
+    for (int p = pg; p < np; p += kThreads / 32) {
+      const bool is_new = (p0 + p == pos);
+      const float *vrow = is_new ? vnew_s
+                                 : a.vcache + ((size_t)kvh * a.max_len + p0 + p) * kD;
+      const float4 v = *reinterpret_cast<const float4 *>(vrow + dq * 4);
+#pragma unroll
+      for (int h = 0; h < kMaxGroup; ++h) {
+        if (h < G) {
+          const float e = sc_s[h][p];
+          acc[h][0] = fmaf(v.x, e, acc[h][0]);
+          acc[h][1] = fmaf(v.y, e, acc[h][1]);
+          acc[h][2] = fmaf(v.z, e, acc[h][2]);
+          acc[h][3] = fmaf(v.w, e, acc[h][3]);
+        }
+      }
+    }
+#pragma unroll
+    for (int h = 0; h < kMaxGroup; ++h)
+      if (h < G)
+        *reinterpret_cast<float4 *>(&red_s[pg][h][dq * 4]) =
+            make_float4(acc[h][0], acc[h][1], acc[h][2], acc[h][3]);
+  }
+  __syncthreads();
+  for (int i = tid; i < G * kD; i += kThreads) {
+    const int h = i / kD, d = i % kD;
+    float s = 0.f;
+#pragma unroll
+    for (int g = 0; g < kThreads / 32; ++g)
+      s += red_s[g][h][d];
+    a.part_acc[((size_t)(h0 + h) * a.nchunks + chunk) * kD + d] = s;
+  }
+  if (tid < G) {
+    a.part_ml[((size_t)(h0 + tid) * a.nchunks + chunk) * 2 + 0] = m_s[tid];
+    a.part_ml[((size_t)(h0 + tid) * a.nchunks + chunk) * 2 + 1] = l_s[tid];
+  }
+}
+
+// Folds the partials of one head in chunk order with the reference's combine
+// (tosa.py:14485-14568): m_new = max(m_run, m_s); a = exp(m_run - m_new);
+// b = exp(m_s - m_new); l = l*a + l_s*b; acc = acc_s*b + acc*a; out = acc / l.
+__global__ void __launch_bounds__(kD) attn_decode_combine(AttnArgs a) {
+  const int h = blockIdx.x, d = threadIdx.x;
+  const int pos = *a.pos_ptr;
+  const int used = min(a.nchunks, pos / kChunk + 1);
+  float m_run = kSeedM, l_run = 0.f, acc = 0.f;
+  for (int s = 0; s < used; ++s) {
+    const float m_c = a.part_ml[((size_t)h * a.nchunks + s) * 2 + 0];
+    const float l_c = a.part_ml[((size_t)h * a.nchunks + s) * 2 + 1];
+    const float m_new = m_c > m_run ? m_c : m_run;
+    const float al = expf(m_run - m_new);
+    const float be = expf(m_c - m_new);
+    l_run = l_run * al + l_c * be;
+    const float rescaled = acc * al;
+    acc = fmaf(a.part_acc[((size_t)h * a.nchunks + s) * kD + d], be, rescaled);
+    m_run = m_new;
+  }
+  a.out[(size_t)h * kD + d] = acc / l_run;
+}
+
+} // namespace
+
+size_t attn_decode_workspace_bytes(int heads, int max_len) {
+  const int nchunks = (int)ceil_div(max_len, kChunk);
+  return sizeof(float) * (size_t)heads * nchunks * (kD + 2);
+}
+
+int launch_attn_decode(const AttnDecodeArgs &in, hipStream_t stream) {
+  BH_REQUIRE(in.qkv && in.inv_freq && in.pos_ptr && in.kcache && in.vcache &&
+                 in.out && in.workspace,
+             "attn_decode: null pointer");
+  BH_REQUIRE(in.head_dim == kD, "attn_decode: head_dim %d (only %d is built)",
+             in.head_dim, kD);
+  BH_REQUIRE(in.kv_heads > 0 && in.heads % in.kv_heads == 0 &&
+                 in.heads / in.kv_heads <= kMaxGroup,
+             "attn_decode: heads=%d kv_heads=%d unsupported", in.heads,
+             in.kv_heads);
+  BH_REQUIRE(in.max_len > 0, "attn_decode: max_len=%d", in.max_len);
+  BH_REQUIRE(in.workspace_bytes >=
+                 attn_decode_workspace_bytes(in.heads, in.max_len),
+             "attn_decode: workspace of %zu bytes needed, %zu given",
+             attn_decode_workspace_bytes(in.heads, in.max_len),
+             in.workspace_bytes);
+  AttnArgs a;
+  a.qkv = in.qkv;
+  a.inv_freq = in.inv_freq;
+  a.pos_ptr = in.pos_ptr;
+  a.kcache = in.kcache;
+  a.vcache = in.vcache;
+  a.heads = in.heads;
+  a.kv_heads = in.kv_heads;
+  a.group = in.heads / in.kv_heads;
+  a.max_len = in.max_len;
+  a.nchunks = (int)ceil_div(in.max_len, kChunk);
+  a.scale = in.scale;
+  a.part_acc = static_cast<float *>(in.workspace);
+  a.part_ml = a.part_acc + (size_t)in.heads * a.nchunks * kD;
+  a.out = in.out;
+  hipLaunchKernelGGL(attn_decode_partial, dim3(a.nchunks, in.kv_heads),
+                     dim3(kThreads), 0, stream, a);
+  hipLaunchKernelGGL(attn_decode_combine, dim3(in.heads), dim3(kD), 0, stream, a);
+  BH_CHECK_HIP(hipGetLastError());
+  return BUDDY_HIP_OK;
+}
+
+} // namespace bh
+
+extern "C" {
+
+size_t buddy_hip_attn_decode_workspace_bytes(int heads, int max_len) {
+  return bh::attn_decode_workspace_bytes(heads, max_len);
+}
+
+int buddy_hip_gqa_decode_attention(const float *qkv, const float *inv_freq,
+                                   const int *pos, float *kcache, float *vcache,
+                                   float *out, int heads, int kv_heads,
+                                   int head_dim, int max_len, float scale,
+                                   void *workspace, size_t workspace_bytes,
+                                   buddy_hip_stream stream) {
+  bh::AttnDecodeArgs a;
+  a.qkv = qkv;
+  a.inv_freq = inv_freq;
+  a.pos_ptr = pos;
+  a.kcache = kcache;
+  a.vcache = vcache;
+  a.out = out;
+  a.heads = heads;
+  a.kv_heads = kv_heads;
+  a.head_dim = head_dim;
+  a.max_len = max_len;
+  a.scale = scale;
+  a.workspace = workspace;
+  a.workspace_bytes = workspace_bytes;
+  return bh::launch_attn_decode(a, bh::as_stream(stream));
+}
+}

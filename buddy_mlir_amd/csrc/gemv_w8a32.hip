@@ -448,6 +448,33 @@ int launch_gemv(const GemvArgs &a, hipStream_t stream) {
 
 extern "C" {
 
+int buddy_hip_linear_w8a32(const buddy_hip_linear_desc *d,
+                           buddy_hip_stream stream) {
+  BH_REQUIRE(d, "linear_w8a32: null descriptor");
+  bh::GemvArgs a;
+  a.A = d->A;
+  a.lda = d->lda;
+  a.W0 = d->W0;
+  a.W1 = d->W1;
+  a.s0 = d->scale0;
+  a.s1 = d->scale1;
+  a.bias = d->bias;
+  a.norm_w = d->norm_w;
+  a.norm_eps = d->norm_eps;
+  a.norm_inv_k = d->K > 0 ? 1.0f / (float)d->K : 0.f;
+  a.C = d->C;
+  a.ldc = d->ldc;
+  a.M = (int)d->M;
+  a.K = d->K;
+  a.N = d->N;
+  a.epilogue = d->epilogue;
+  BH_REQUIRE(d->M >= 1 && d->M <= 16, "linear_w8a32: M=%lld outside 1..16",
+             (long long)d->M);
+  BH_REQUIRE(!(d->bias && d->epilogue != BUDDY_HIP_EPI_STORE),
+             "linear_w8a32: bias only with the STORE epilogue");
+  return bh::launch_gemv(a, bh::as_stream(stream));
+}
+
 int buddy_hip_gemv_w8a32(const float *A, const int8_t *packed,
                          const float *scale, float *C, int64_t M, int64_t K,
                          int64_t N, unsigned flags, buddy_hip_stream stream) {

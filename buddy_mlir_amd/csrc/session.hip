@@ -1,0 +1,527 @@
+// session.hip -- a Qwen2-shaped int8 (w8a32) decoder resident on one GPU.
+//
+// Takes the place of the generated ModelSession + compiled forward_decode
+// (tools/buddy-codegen/gen_session.py:1381-1452 calling
+// _mlir_ciface_forward_decode, whose body is the op sequence of
+// examples/BuddyDeepSeekR1/subgraph0_decode_simplify.mlir:46-260,4986-5004) and
+// of the greedy part of the decode loop
+// (runtime/llm/TextGeneration.cpp:215-266, Sampler.h:101-104).
+//
+// Weights are repacked once into wave tiles and stay in HBM together with the
+// f32 KV cache; a decode step is 6 kernels per layer on one stream:
+//   [RMSNorm + q|k|v GEMV] -> [RoPE + KV write + attention partials] ->
+//   [combine] -> [o_proj GEMV + residual] -> [RMSNorm + gate|up GEMV + SiLU*mul]
+//   -> [down GEMV + residual]
+// followed by [RMSNorm + lm_head GEMV], a two-stage argmax and a bookkeeping
+// kernel.  Token id, position and step counter live in device memory, so the
+// whole step is captured once into a hipGraph and replayed; greedy decoding
+// feeds the argmax straight into the next step's embedding gather without a
+// host round trip.
+#include "attn.h"
+#include "elementwise.h"
+#include "gemv_w8a32.h"
+
+#include <cmath>
+#include <cstring>
+#include <new>
+#include <vector>
+
+namespace bh {
+namespace {
+
+struct PackedLinear {
+  int8_t *w = nullptr; // wave tiles
+  float *s = nullptr;  // scales
+  float *b = nullptr;  // bias or null
+  int64_t K = 0, N = 0;
+};
+
+struct Layer {
+  float *ln1 = nullptr, *ln2 = nullptr;
+  PackedLinear qkv, o, gate, up, down;
+  float *kc = nullptr, *vc = nullptr; // [kv_heads, max_len, D]
+  bool set = false;
+};
+
+__global__ void advance_kernel(int *state) {
+  // state: [0] token, [1] pos, [2] step
+  if (threadIdx.x == 0) {
+    state[1] += 1;
+    state[2] += 1;
+  }
+}
+
+} // namespace
+
+struct Session {
+  buddy_hip_model_shape shape{};
+  hipStream_t stream = nullptr;
+  bool own_stream = false;
+  std::vector<Layer> layers;
+  const float *embed = nullptr; // borrowed: [vocab, hidden] f32
+  float *ln_f = nullptr, *inv_freq = nullptr;
+  PackedLinear lm;
+  // activations
+  float *x = nullptr, *qkv = nullptr, *att = nullptr, *h = nullptr,
+        *logits = nullptr;
+  void *attn_ws = nullptr, *amax_ws = nullptr;
+  size_t attn_ws_bytes = 0;
+  int *state = nullptr;     // device: token, pos, step
+  int *token_log = nullptr; // device: greedy tokens by step
+  int token_log_cap = 0;
+  int *host_state = nullptr; // pinned staging for token/pos/step
+  hipGraph_t graph = nullptr;
+  hipGraphExec_t graph_exec = nullptr;
+  bool use_graph = true;
+  std::vector<void *> owned;
+
+  template <typename T> int alloc(T **p, size_t n) {
+    void *q = nullptr;
+    BH_CHECK_HIP(hipMalloc(&q, n * sizeof(T)));
+    owned.push_back(q);
+    *p = static_cast<T *>(q);
+    return BUDDY_HIP_OK;
+  }
+
+  int pack_into(const int8_t *W, const float *scale, const float *bias,
+                int64_t K, int64_t N, int8_t *dst_w, float *dst_s, float *dst_b) {
+    int rc = buddy_hip_pack_w8(W, K, N, dst_w, stream);
+    if (rc)
+      return rc;
+    BH_CHECK_HIP(hipMemcpyAsync(dst_s, scale, sizeof(float) * N,
+                                hipMemcpyDefault, stream));
+    if (bias && dst_b)
+      BH_CHECK_HIP(hipMemcpyAsync(dst_b, bias, sizeof(float) * N,
+                                  hipMemcpyDefault, stream));
+    return BUDDY_HIP_OK;
+  }
+
+  int make_linear(PackedLinear &L, const int8_t *W, const float *scale,
+                  int64_t K, int64_t N) {
+    BH_REQUIRE(W && scale, "session: null weight or scale");
+    L.K = K;
+    L.N = N;
+    int rc = alloc(&L.w, buddy_hip_w8_packed_bytes(K, N));
+    if (rc)
+      return rc;
+    rc = alloc(&L.s, (size_t)N);
+    if (rc)
+      return rc;
+    return pack_into(W, scale, nullptr, K, N, L.w, L.s, nullptr);
+  }
+
+  void drop_graph() {
+    if (graph_exec)
+      (void)hipGraphExecDestroy(graph_exec);
+    if (graph)
+      (void)hipGraphDestroy(graph);
+    graph_exec = nullptr;
+    graph = nullptr;
+  }
+
+  int gemv(const float *A, const PackedLinear &W0, const PackedLinear *W1,
+           const float *norm_w, float *C, int epi) {
+    GemvArgs g;
+    g.A = A;
+    g.lda = W0.K;
+    g.W0 = W0.w;
+    g.s0 = W0.s;
+    if (W1) {
+      g.W1 = W1->w;
+      g.s1 = W1->s;
+    }
+    g.bias = epi == kEpiStore ? W0.b : nullptr;
+    g.norm_w = norm_w;
+    g.norm_eps = shape.rms_eps;
+    g.norm_inv_k = 1.0f / (float)W0.K;
+    g.C = C;
+    g.ldc = W0.N;
+    g.M = 1;
+    g.K = W0.K;
+    g.N = W0.N;
+    g.epilogue = epi;
+    return launch_gemv(g, stream);
+  }
+
+  // Enqueues one decode step (reads token/pos from device state).
+  int enqueue_step() {
+    const auto &S = shape;
+    int rc = launch_embedding(embed, state, S.hidden, S.vocab, x, stream);
+    if (rc)
+      return rc;
+    const float scale = (float)(1.0 / std::sqrt((double)S.head_dim));
+    for (int i = 0; i < S.layers; ++i) {
+      Layer &L = layers[(size_t)i];
+      if ((rc = gemv(x, L.qkv, nullptr, L.ln1, qkv, kEpiStore)))
+        return rc;
+      AttnDecodeArgs a;
+      a.qkv = qkv;
+      a.inv_freq = inv_freq;
+      a.pos_ptr = state + 1;
+      a.kcache = L.kc;
+      a.vcache = L.vc;
+      a.out = att;
+      a.heads = S.heads;
+      a.kv_heads = S.kv_heads;
+      a.head_dim = S.head_dim;
+      a.max_len = S.max_len;
+      a.scale = scale;
+      a.workspace = attn_ws;
+      a.workspace_bytes = attn_ws_bytes;
+      if ((rc = launch_attn_decode(a, stream)))
+        return rc;
+      if ((rc = gemv(att, L.o, nullptr, nullptr, x, kEpiAccum)))
+        return rc;
+      if ((rc = gemv(x, L.gate, &L.up, L.ln2, h, kEpiSiluMul)))
+        return rc;
+      if ((rc = gemv(h, L.down, nullptr, nullptr, x, kEpiAccum)))
+        return rc;
+    }
+    if ((rc = gemv(x, lm, nullptr, ln_f, logits, kEpiStore)))
+      return rc;
+    if ((rc = launch_argmax(logits, S.vocab, amax_ws, state, token_log,
+                            state + 2, stream)))
+      return rc;
+    hipLaunchKernelGGL(advance_kernel, dim3(1), dim3(64), 0, stream, state);
+    BH_CHECK_HIP(hipGetLastError());
+    return BUDDY_HIP_OK;
+  }
+
+  int ready() const {
+    if (!embed || !ln_f || !lm.w)
+      return fail(BUDDY_HIP_ERR_ARG, "session: embedding / head not set");
+    for (size_t i = 0; i < layers.size(); ++i)
+      if (!layers[i].set)
+        return fail(BUDDY_HIP_ERR_ARG, "session: layer %zu not set", i);
+    return BUDDY_HIP_OK;
+  }
+
+  int run_step() {
+    if (!use_graph)
+      return enqueue_step();
+    if (!graph_exec) {
+      BH_CHECK_HIP(hipStreamBeginCapture(stream, hipStreamCaptureModeThreadLocal));
+      int rc = enqueue_step();
+      hipError_t e = hipStreamEndCapture(stream, &graph);
+      if (rc)
+        return rc;
+      if (e != hipSuccess)
+        return fail(BUDDY_HIP_ERR_HIP, "hipStreamEndCapture: %s",
+                    hipGetErrorString(e));
+      BH_CHECK_HIP(hipGraphInstantiate(&graph_exec, graph, nullptr, nullptr, 0));
+    }
+    BH_CHECK_HIP(hipGraphLaunch(graph_exec, stream));
+    return BUDDY_HIP_OK;
+  }
+
+  int set_state(int token, int pos, int step) {
+    host_state[0] = token;
+    host_state[1] = pos;
+    host_state[2] = step;
+    BH_CHECK_HIP(hipMemcpyAsync(state, host_state, 3 * sizeof(int),
+                                hipMemcpyHostToDevice, stream));
+    // the pinned staging words are reused by the next call
+    BH_CHECK_HIP(hipStreamSynchronize(stream));
+    return BUDDY_HIP_OK;
+  }
+};
+
+} // namespace bh
+
+using bh::Session;
+
+extern "C" {
+
+buddy_hip_session *buddy_hip_session_create(const buddy_hip_model_shape *shape,
+                                            buddy_hip_stream stream) {
+  if (!shape) {
+    bh::fail(BUDDY_HIP_ERR_ARG, "session_create: null shape");
+    return nullptr;
+  }
+  const auto &S = *shape;
+  if (S.layers <= 0 || S.hidden <= 0 || S.heads <= 0 || S.kv_heads <= 0 ||
+      S.head_dim != 128 || S.inter <= 0 || S.vocab <= 0 || S.max_len <= 0 ||
+      S.heads % S.kv_heads != 0 || S.heads / S.kv_heads > 8) {
+    bh::fail(BUDDY_HIP_ERR_ARG,
+             "session_create: unsupported shape (head_dim must be 128, at most "
+             "8 query heads per KV head)");
+    return nullptr;
+  }
+  if (buddy_hip_device_count() == 0) {
+    bh::fail(BUDDY_HIP_ERR_NO_DEVICE, "session_create: no HIP device");
+    return nullptr;
+  }
+  Session *s = new (std::nothrow) Session();
+  if (!s)
+    return nullptr;
+  s->shape = S;
+  s->stream = bh::as_stream(stream);
+  if (!s->stream) {
+    if (hipStreamCreateWithFlags(&s->stream, hipStreamNonBlocking) != hipSuccess) {
+      bh::fail(BUDDY_HIP_ERR_HIP, "session_create: cannot create a stream");
+      delete s;
+      return nullptr;
+    }
+    s->own_stream = true;
+  }
+  s->layers.resize((size_t)S.layers);
+  const size_t QN = (size_t)S.heads * S.head_dim, KVN = (size_t)S.kv_heads * S.head_dim;
+  int rc = 0;
+  rc |= s->alloc(&s->x, (size_t)S.hidden);
+  rc |= s->alloc(&s->qkv, QN + 2 * KVN);
+  rc |= s->alloc(&s->att, QN);
+  rc |= s->alloc(&s->h, (size_t)S.inter);
+  rc |= s->alloc(&s->logits, (size_t)S.vocab);
+  rc |= s->alloc(&s->ln_f, (size_t)S.hidden);
+  rc |= s->alloc(&s->inv_freq, (size_t)S.head_dim / 2);
+  rc |= s->alloc(&s->state, 4);
+  s->token_log_cap = 65536;
+  rc |= s->alloc(&s->token_log, (size_t)s->token_log_cap);
+  s->attn_ws_bytes = bh::attn_decode_workspace_bytes(S.heads, S.max_len);
+  rc |= s->alloc((char **)&s->attn_ws, s->attn_ws_bytes);
+  rc |= s->alloc((char **)&s->amax_ws, bh::argmax_workspace_bytes());
+  for (auto &L : s->layers) {
+    rc |= s->alloc(&L.kc, KVN * (size_t)S.max_len);
+    rc |= s->alloc(&L.vc, KVN * (size_t)S.max_len);
+    rc |= s->alloc(&L.ln1, (size_t)S.hidden);
+    rc |= s->alloc(&L.ln2, (size_t)S.hidden);
+  }
+  if (!rc && hipHostMalloc((void **)&s->host_state, 4 * sizeof(int)) != hipSuccess)
+    rc = bh::fail(BUDDY_HIP_ERR_HIP, "session_create: pinned alloc failed");
+  if (!rc) {
+    for (auto &L : s->layers) {
+      if (hipMemsetAsync(L.kc, 0, sizeof(float) * KVN * S.max_len, s->stream) != hipSuccess ||
+          hipMemsetAsync(L.vc, 0, sizeof(float) * KVN * S.max_len, s->stream) != hipSuccess)
+        rc = bh::fail(BUDDY_HIP_ERR_HIP, "session_create: cache clear failed");
+    }
+    if (hipMemsetAsync(s->state, 0, 4 * sizeof(int), s->stream) != hipSuccess)
+      rc = BUDDY_HIP_ERR_HIP;
+    (void)hipStreamSynchronize(s->stream);
+  }
+  if (rc) {
+    buddy_hip_session_destroy(reinterpret_cast<buddy_hip_session *>(s));
+    return nullptr;
+  }
+  return reinterpret_cast<buddy_hip_session *>(s);
+}
+
+void buddy_hip_session_destroy(buddy_hip_session *hs) {
+  Session *s = reinterpret_cast<Session *>(hs);
+  if (!s)
+    return;
+  if (s->stream)
+    (void)hipStreamSynchronize(s->stream);
+  s->drop_graph();
+  for (void *p : s->owned)
+    (void)hipFree(p);
+  if (s->host_state)
+    (void)hipHostFree(s->host_state);
+  if (s->own_stream)
+    (void)hipStreamDestroy(s->stream);
+  delete s;
+}
+
+int buddy_hip_session_set_globals(buddy_hip_session *hs, const float *embed,
+                                  const float *inv_freq, const float *ln_f,
+                                  const int8_t *w_lm, const float *s_lm) {
+  Session *s = reinterpret_cast<Session *>(hs);
+  BH_REQUIRE(s && embed && inv_freq && ln_f && w_lm && s_lm,
+             "session_set_globals: null argument");
+  const auto &S = s->shape;
+  s->embed = embed;
+  BH_CHECK_HIP(hipMemcpyAsync(s->inv_freq, inv_freq, sizeof(float) * S.head_dim / 2,
+                              hipMemcpyDefault, s->stream));
+  BH_CHECK_HIP(hipMemcpyAsync(s->ln_f, ln_f, sizeof(float) * S.hidden,
+                              hipMemcpyDefault, s->stream));
+  if (!s->lm.w) {
+    int rc = s->make_linear(s->lm, w_lm, s_lm, S.hidden, S.vocab);
+    if (rc)
+      return rc;
+  } else {
+    int rc = s->pack_into(w_lm, s_lm, nullptr, S.hidden, S.vocab, s->lm.w,
+                          s->lm.s, nullptr);
+    if (rc)
+      return rc;
+  }
+  BH_CHECK_HIP(hipStreamSynchronize(s->stream));
+  return BUDDY_HIP_OK;
+}
+
+int buddy_hip_session_set_layer(buddy_hip_session *hs, int index,
+                                const buddy_hip_layer_weights *w) {
+  Session *s = reinterpret_cast<Session *>(hs);
+  BH_REQUIRE(s && w, "session_set_layer: null argument");
+  const auto &S = s->shape;
+  BH_REQUIRE(index >= 0 && index < S.layers, "session_set_layer: index %d", index);
+  BH_REQUIRE(w->ln1 && w->ln2 && w->wq && w->wk && w->wv && w->wo && w->wg &&
+                 w->wu && w->wd && w->sq && w->sk && w->sv && w->so && w->sg &&
+                 w->su && w->sd,
+             "session_set_layer: null weight");
+  BH_REQUIRE((w->bq != nullptr) == (w->bk != nullptr) &&
+                 (w->bq != nullptr) == (w->bv != nullptr),
+             "session_set_layer: q/k/v biases must come together");
+  bh::Layer &L = s->layers[(size_t)index];
+  const int64_t H = S.hidden, QN = (int64_t)S.heads * S.head_dim,
+                KVN = (int64_t)S.kv_heads * S.head_dim, I = S.inter;
+  int rc = 0;
+  if (!L.set) {
+    // q|k|v share one packed matrix: channel groups are independent, so the
+    // three packed blocks simply follow each other
+    L.qkv.K = H;
+    L.qkv.N = QN + 2 * KVN;
+    rc |= s->alloc(&L.qkv.w, buddy_hip_w8_packed_bytes(H, L.qkv.N));
+    rc |= s->alloc(&L.qkv.s, (size_t)L.qkv.N);
+    if (w->bq)
+      rc |= s->alloc(&L.qkv.b, (size_t)L.qkv.N);
+    L.o.K = QN; L.o.N = H;
+    L.gate.K = H; L.gate.N = I;
+    L.up.K = H; L.up.N = I;
+    L.down.K = I; L.down.N = H;
+    for (bh::PackedLinear *P : {&L.o, &L.gate, &L.up, &L.down}) {
+      rc |= s->alloc(&P->w, buddy_hip_w8_packed_bytes(P->K, P->N));
+      rc |= s->alloc(&P->s, (size_t)P->N);
+    }
+    if (rc)
+      return rc;
+  }
+  BH_REQUIRE(QN % 16 == 0 && KVN % 16 == 0, "session_set_layer: head sizes");
+  const size_t kp = (size_t)bh::round_up(H, bh::kTileK);
+  rc |= s->pack_into(w->wq, w->sq, w->bq, H, QN, L.qkv.w, L.qkv.s, L.qkv.b);
+  rc |= s->pack_into(w->wk, w->sk, w->bk, H, KVN, L.qkv.w + kp * QN,
+                     L.qkv.s + QN, L.qkv.b ? L.qkv.b + QN : nullptr);
+  rc |= s->pack_into(w->wv, w->sv, w->bv, H, KVN, L.qkv.w + kp * (QN + KVN),
+                     L.qkv.s + QN + KVN, L.qkv.b ? L.qkv.b + QN + KVN : nullptr);
+  rc |= s->pack_into(w->wo, w->so, nullptr, QN, H, L.o.w, L.o.s, nullptr);
+  rc |= s->pack_into(w->wg, w->sg, nullptr, H, I, L.gate.w, L.gate.s, nullptr);
+  rc |= s->pack_into(w->wu, w->su, nullptr, H, I, L.up.w, L.up.s, nullptr);
+  rc |= s->pack_into(w->wd, w->sd, nullptr, I, H, L.down.w, L.down.s, nullptr);
+  if (rc)
+    return rc;
+  BH_CHECK_HIP(hipMemcpyAsync(L.ln1, w->ln1, sizeof(float) * H, hipMemcpyDefault, s->stream));
+  BH_CHECK_HIP(hipMemcpyAsync(L.ln2, w->ln2, sizeof(float) * H, hipMemcpyDefault, s->stream));
+  BH_CHECK_HIP(hipStreamSynchronize(s->stream));
+  L.set = true;
+  return BUDDY_HIP_OK;
+}
+
+int buddy_hip_session_set_kv(buddy_hip_session *hs, int kv_index,
+                             const float *src) {
+  Session *s = reinterpret_cast<Session *>(hs);
+  BH_REQUIRE(s && src, "session_set_kv: null argument");
+  const auto &S = s->shape;
+  BH_REQUIRE(kv_index >= 0 && kv_index < 2 * S.layers, "session_set_kv: index %d",
+             kv_index);
+  bh::Layer &L = s->layers[(size_t)(kv_index / 2)];
+  float *dst = (kv_index & 1) ? L.vc : L.kc; // even = K, odd = V
+  BH_CHECK_HIP(hipMemcpyAsync(dst, src,
+                              sizeof(float) * (size_t)S.kv_heads * S.max_len * S.head_dim,
+                              hipMemcpyDefault, s->stream));
+  BH_CHECK_HIP(hipStreamSynchronize(s->stream));
+  return BUDDY_HIP_OK;
+}
+
+int buddy_hip_session_get_kv(buddy_hip_session *hs, int kv_index, float *dst) {
+  Session *s = reinterpret_cast<Session *>(hs);
+  BH_REQUIRE(s && dst, "session_get_kv: null argument");
+  const auto &S = s->shape;
+  BH_REQUIRE(kv_index >= 0 && kv_index < 2 * S.layers, "session_get_kv: index %d",
+             kv_index);
+  bh::Layer &L = s->layers[(size_t)(kv_index / 2)];
+  const float *src = (kv_index & 1) ? L.vc : L.kc;
+  BH_CHECK_HIP(hipMemcpyAsync(dst, src,
+                              sizeof(float) * (size_t)S.kv_heads * S.max_len * S.head_dim,
+                              hipMemcpyDefault, s->stream));
+  BH_CHECK_HIP(hipStreamSynchronize(s->stream));
+  return BUDDY_HIP_OK;
+}
+
+int buddy_hip_session_use_graph(buddy_hip_session *hs, int enable) {
+  Session *s = reinterpret_cast<Session *>(hs);
+  BH_REQUIRE(s, "session_use_graph: null session");
+  s->use_graph = enable != 0;
+  return BUDDY_HIP_OK;
+}
+
+int buddy_hip_session_decode(buddy_hip_session *hs, int token, int pos,
+                             float *logits_out, int *next_token) {
+  Session *s = reinterpret_cast<Session *>(hs);
+  BH_REQUIRE(s, "session_decode: null session");
+  int rc = s->ready();
+  if (rc)
+    return rc;
+  BH_REQUIRE(token >= 0 && token < s->shape.vocab, "session_decode: token %d", token);
+  BH_REQUIRE(pos >= 0 && pos < s->shape.max_len,
+             "session_decode: position %d outside the cache (max_len %d)", pos,
+             s->shape.max_len);
+  if ((rc = s->set_state(token, pos, 0)))
+    return rc;
+  if ((rc = s->run_step()))
+    return rc;
+  if (logits_out)
+    BH_CHECK_HIP(hipMemcpyAsync(logits_out, s->logits,
+                                sizeof(float) * s->shape.vocab, hipMemcpyDefault,
+                                s->stream));
+  BH_CHECK_HIP(hipMemcpyAsync(s->host_state, s->state, 3 * sizeof(int),
+                              hipMemcpyDeviceToHost, s->stream));
+  BH_CHECK_HIP(hipStreamSynchronize(s->stream));
+  if (next_token)
+    *next_token = s->host_state[0];
+  return BUDDY_HIP_OK;
+}
+
+int buddy_hip_session_decode_greedy(buddy_hip_session *hs, int first_token,
+                                    int start_pos, int steps, int *tokens_out) {
+  Session *s = reinterpret_cast<Session *>(hs);
+  BH_REQUIRE(s && tokens_out, "session_decode_greedy: null argument");
+  int rc = s->ready();
+  if (rc)
+    return rc;
+  BH_REQUIRE(first_token >= 0 && first_token < s->shape.vocab,
+             "session_decode_greedy: token %d", first_token);
+  BH_REQUIRE(steps > 0 && steps <= s->token_log_cap,
+             "session_decode_greedy: steps %d", steps);
+  BH_REQUIRE(start_pos >= 0 && start_pos + steps <= s->shape.max_len,
+             "session_decode_greedy: positions %d..%d outside the cache (max_len %d)",
+             start_pos, start_pos + steps - 1, s->shape.max_len);
+  if ((rc = s->set_state(first_token, start_pos, 0)))
+    return rc;
+  for (int i = 0; i < steps; ++i)
+    if ((rc = s->run_step()))
+      return rc;
+  BH_CHECK_HIP(hipMemcpyAsync(tokens_out, s->token_log, sizeof(int) * steps,
+                              hipMemcpyDefault, s->stream));
+  BH_CHECK_HIP(hipStreamSynchronize(s->stream));
+  return BUDDY_HIP_OK;
+}
+
+int buddy_hip_session_enqueue_steps(buddy_hip_session *hs, int steps) {
+  Session *s = reinterpret_cast<Session *>(hs);
+  BH_REQUIRE(s && steps > 0, "session_enqueue_steps: bad argument");
+  int rc = s->ready();
+  if (rc)
+    return rc;
+  for (int i = 0; i < steps; ++i)
+    if ((rc = s->run_step()))
+      return rc;
+  return BUDDY_HIP_OK;
+}
+
+int buddy_hip_session_set_state(buddy_hip_session *hs, int token, int pos) {
+  Session *s = reinterpret_cast<Session *>(hs);
+  BH_REQUIRE(s, "session_set_state: null session");
+  BH_REQUIRE(token >= 0 && token < s->shape.vocab && pos >= 0 &&
+                 pos < s->shape.max_len,
+             "session_set_state: token %d / position %d out of range", token, pos);
+  return s->set_state(token, pos, 0);
+}
+
+const float *buddy_hip_session_logits(buddy_hip_session *hs) {
+  Session *s = reinterpret_cast<Session *>(hs);
+  return s ? s->logits : nullptr;
+}
+
+buddy_hip_stream buddy_hip_session_stream(buddy_hip_session *hs) {
+  Session *s = reinterpret_cast<Session *>(hs);
+  return s ? reinterpret_cast<buddy_hip_stream>(s->stream) : nullptr;
+}
+}

@@ -83,6 +83,65 @@ int buddy_hip_gemv_w8a32(const float *A, const int8_t *packed,
                          const float *scale, float *C, int64_t M, int64_t K,
                          int64_t N, unsigned flags, buddy_hip_stream stream);
 
+/* Full form of the kernel above with the fusions a decoder layer uses.
+ * Every pointer is device memory. */
+typedef struct buddy_hip_linear_desc {
+  const float *A;       /* [M, K], row stride lda (>= K) */
+  int64_t lda;
+  const int8_t *W0;     /* wave-tile packed [K, N] */
+  const float *scale0;  /* [N] */
+  const int8_t *W1;     /* second matrix (epilogue SILU_MUL) or NULL */
+  const float *scale1;
+  const float *bias;    /* [N] or NULL: C = bias + acc*scale (epilogue STORE) */
+  const float *norm_w;  /* [K] or NULL: RMSNorm applied to A first
+                           (subgraph0_decode_simplify.mlir:60-72) */
+  float norm_eps;
+  float *C;             /* [M, N], row stride ldc (>= N) */
+  int64_t ldc;
+  int64_t M, K, N;      /* M in 1..16 */
+  int epilogue;         /* BUDDY_HIP_EPI_* */
+} buddy_hip_linear_desc;
+enum {
+  BUDDY_HIP_EPI_STORE = 0,   /* C = acc*scale (+ bias) */
+  BUDDY_HIP_EPI_ACCUM = 1,   /* C = C + acc*scale (residual add) */
+  BUDDY_HIP_EPI_SILU_MUL = 2 /* C = silu(acc0*scale0) * (acc1*scale1)
+                                (subgraph0_decode_simplify.mlir:225-232) */
+};
+int buddy_hip_linear_w8a32(const buddy_hip_linear_desc *desc,
+                           buddy_hip_stream stream);
+
+/* ---- element-wise pieces of a decoder layer ------------------------------
+ * Stand-alone forms of what the decode step runs fused; constants and op order
+ * from examples/BuddyDeepSeekR1/subgraph0_decode_simplify.mlir:51-72,88-107,
+ * 225-232.  `pos` is a device scalar. */
+int buddy_hip_rmsnorm(const float *x, const float *w, float *y, int rows, int n,
+                      float eps, buddy_hip_stream stream);
+int buddy_hip_rope(float *x, const float *inv_freq, const int *pos, int n_heads,
+                   int head_dim, buddy_hip_stream stream);
+int buddy_hip_silu_mul(const float *g, const float *u, float *h, int64_t n,
+                       buddy_hip_stream stream);
+/* Greedy sampling: the FIRST index of the maximum, like std::max_element
+ * (runtime/include/buddy/runtime/llm/Sampler.h:101-104). */
+size_t buddy_hip_argmax_workspace_bytes(void);
+int buddy_hip_argmax(const float *x, int n, void *workspace, int *out_index,
+                     buddy_hip_stream stream);
+
+/* ---- GQA decode attention -------------------------------------------------
+ * Replaces gqa_attention_fused_op (frontend/Python/ops/tosa.py:14130-14600)
+ * together with the RoPE and KV-cache write in front of it
+ * (subgraph0_decode_simplify.mlir:88-142).  qkv = [q | k | v] as the
+ * projections leave them (before RoPE); the kernel rotates q and k, writes k'
+ * and v into row *pos of the caches ([kv_heads, max_len, head_dim] f32 each)
+ * and attends over rows 0..*pos.  out: [heads*head_dim].  head_dim must be 128.
+ */
+size_t buddy_hip_attn_decode_workspace_bytes(int heads, int max_len);
+int buddy_hip_gqa_decode_attention(const float *qkv, const float *inv_freq,
+                                   const int *pos, float *kcache, float *vcache,
+                                   float *out, int heads, int kv_heads,
+                                   int head_dim, int max_len, float scale,
+                                   void *workspace, size_t workspace_bytes,
+                                   buddy_hip_stream stream);
+
 /* ---- plain f32 matmul ---------------------------------------------------
  * C (+)= A[M,K] * B[K,N], all dense row-major device pointers.  The f32
  * sibling of the kernel above (MatMulVectorizationDecode.cpp:142-175); the
@@ -90,6 +149,72 @@ int buddy_hip_gemv_w8a32(const float *A, const int8_t *packed,
 int buddy_hip_matmul_f32(const float *A, const float *B, float *C, int64_t M,
                          int64_t N, int64_t K, unsigned flags,
                          buddy_hip_stream stream);
+
+/* ---- resident decoder session ---------------------------------------------
+ * A Qwen2-shaped int8 (w8a32) decoder kept on one GPU: weights repacked into
+ * wave tiles, f32 KV cache, activations, and one hipGraph per decode step.
+ * Stands where the generated ModelSession and the compiled forward_decode
+ * stand in the reference (tools/buddy-codegen/gen_session.py:1381-1452;
+ * op order of examples/BuddyDeepSeekR1/subgraph0_decode_simplify.mlir:46-260,
+ * 4986-5004) and runs the greedy part of runtime/llm/TextGeneration.cpp:215-266
+ * on the device.  Field names follow the HF config, not the reference's
+ * (its `head_num` is kv_heads and its `hidden_size` is head_dim:
+ * tools/buddy-codegen/gen_config.py:288-299).  Not re-entrant per session. */
+typedef struct buddy_hip_model_shape {
+  int layers, hidden, heads, kv_heads, head_dim, inter, vocab;
+  int max_len;    /* KV cache capacity in positions */
+  float rms_eps;
+} buddy_hip_model_shape;
+
+/* One decoder layer as the importer leaves it: int8 W[K,N] row-major with
+ * K = in, N = out (frontend/Python/graph/transform/eliminate_weight_transpose
+ * .py:28-41) and f32 scale[N]; biases may be NULL (all three or none).
+ * Pointers are device memory and are read only during the call. */
+typedef struct buddy_hip_layer_weights {
+  const float *ln1, *ln2;
+  const int8_t *wq, *wk, *wv, *wo, *wg, *wu, *wd;
+  const float *sq, *sk, *sv, *so, *sg, *su, *sd;
+  const float *bq, *bk, *bv;
+} buddy_hip_layer_weights;
+
+typedef struct buddy_hip_session buddy_hip_session;
+
+/* stream NULL: the session creates its own.  Returns NULL on failure. */
+buddy_hip_session *buddy_hip_session_create(const buddy_hip_model_shape *shape,
+                                            buddy_hip_stream stream);
+void buddy_hip_session_destroy(buddy_hip_session *s);
+/* embed: f32 [vocab, hidden], borrowed (must outlive the session); the other
+ * arguments are copied / repacked: inv_freq f32 [head_dim/2], ln_f f32
+ * [hidden], lm_head int8 [hidden, vocab] + scale [vocab]. */
+int buddy_hip_session_set_globals(buddy_hip_session *s, const float *embed,
+                                  const float *inv_freq, const float *ln_f,
+                                  const int8_t *w_lm, const float *s_lm);
+int buddy_hip_session_set_layer(buddy_hip_session *s, int index,
+                                const buddy_hip_layer_weights *w);
+/* KV tensors in the reference's numbering: even index = K, odd = V of layer
+ * index/2 (runtime/include/buddy/runtime/llm/KVCacheManager.h:200-201), each
+ * f32 [kv_heads, max_len, head_dim]; src/dst may be host or device memory. */
+int buddy_hip_session_set_kv(buddy_hip_session *s, int kv_index, const float *src);
+int buddy_hip_session_get_kv(buddy_hip_session *s, int kv_index, float *dst);
+/* 1 (default): a decode step is replayed from a captured hipGraph; 0: launched
+ * kernel by kernel. */
+int buddy_hip_session_use_graph(buddy_hip_session *s, int enable);
+/* One decode step for `token` at cache row `pos` (ModelSession::decode).
+ * logits_out (host or device, vocab floats) and next_token may be NULL.
+ * next_token is the greedy choice (first maximum).  Synchronous. */
+int buddy_hip_session_decode(buddy_hip_session *s, int token, int pos,
+                             float *logits_out, int *next_token);
+/* `steps` greedy steps starting from first_token at start_pos; each step's
+ * argmax feeds the next step on the device.  tokens_out[i] = token chosen by
+ * step i.  Synchronous. */
+int buddy_hip_session_decode_greedy(buddy_hip_session *s, int first_token,
+                                    int start_pos, int steps, int *tokens_out);
+/* Asynchronous pieces of the call above, for timing: set the device-side
+ * (token, position), then enqueue steps on the session stream. */
+int buddy_hip_session_set_state(buddy_hip_session *s, int token, int pos);
+int buddy_hip_session_enqueue_steps(buddy_hip_session *s, int steps);
+const float *buddy_hip_session_logits(buddy_hip_session *s); /* device */
+buddy_hip_stream buddy_hip_session_stream(buddy_hip_session *s);
 
 /* ---- operator-level memref entry points --------------------------------
  * result = A * B, f32.  Same symbol and contract as

@@ -1,0 +1,273 @@
+"""GPU parity of the decode-step pieces and of whole decode steps against the
+CPU oracle: attention (with fused RoPE + KV write), fused linear epilogues,
+argmax, and the resident session (logits, KV rows written, greedy tokens)."""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+import buddy_mlir_amd as bma
+import oracle_lib
+from buddy_mlir_amd import ops, synthetic
+from buddy_mlir_amd.session import Shape
+from parity import check_close
+
+pytestmark = pytest.mark.gpu
+
+EPS = np.float32(1e-6)
+
+
+def dev(a, dtype=torch.float32):
+    return torch.from_numpy(np.ascontiguousarray(a)).to("cuda", dtype)
+
+
+def linear(bh, **kw):
+    class Desc(ctypes.Structure):
+        _fields_ = [("A", ctypes.c_void_p), ("lda", ctypes.c_int64),
+                    ("W0", ctypes.c_void_p), ("scale0", ctypes.c_void_p),
+                    ("W1", ctypes.c_void_p), ("scale1", ctypes.c_void_p),
+                    ("bias", ctypes.c_void_p), ("norm_w", ctypes.c_void_p),
+                    ("norm_eps", ctypes.c_float), ("C", ctypes.c_void_p),
+                    ("ldc", ctypes.c_int64), ("M", ctypes.c_int64),
+                    ("K", ctypes.c_int64), ("N", ctypes.c_int64),
+                    ("epilogue", ctypes.c_int)]
+    d = Desc()
+    for k, v in kw.items():
+        setattr(d, k, v.data_ptr() if isinstance(v, torch.Tensor) else v)
+    torch.cuda.synchronize()
+    bma.check(bh.buddy_hip_linear_w8a32(ctypes.byref(d), None), "linear")
+    torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize("M", [1, 4, 16])
+def test_mlp_block_matches_oracle(bh, oracle, M):
+    """h = SiLU(x.G) * (x.U); y = h.D -- the fused gate|up kernel and the down
+    projection.  M = 1 follows the decode GEMV kernel, M = 4 / 16 the BLIS
+    kernel, the only vectorised reference kernel for M > 1."""
+    H, I = 1536, 8960
+    qg, sg = synthetic.quantized_linear(H, I, 11)
+    qu, su = synthetic.quantized_linear(H, I, 12)
+    qd, sd = synthetic.quantized_linear(I, H, 13)
+    x = torch.randn((M, H), generator=torch.Generator(device="cuda").manual_seed(M),
+                    device="cuda")
+    h = torch.empty((M, I), device="cuda")
+    y = torch.empty((M, H), device="cuda")
+    linear(bh, A=x, lda=H, W0=ops.pack_w8(qg), scale0=sg, W1=ops.pack_w8(qu),
+           scale1=su, C=h, ldc=I, M=M, K=H, N=I, epilogue=2)
+    linear(bh, A=h, lda=I, W0=ops.pack_w8(qd), scale0=sd, C=y, ldc=H, M=M, K=I,
+           N=H, epilogue=0)
+    xh = x.cpu().numpy()
+    qg, sg, qu, su, qd, sd = (t.cpu().numpy() for t in (qg, sg, qu, su, qd, sd))
+    if M == 1:
+        g = oracle.dequant_gemv(xh[0], qg, sg)[None]
+        u = oracle.dequant_gemv(xh[0], qu, su)[None]
+    else:
+        g = oracle.blis_gemm_w8a32(xh, qg, sg)
+        u = oracle.blis_gemm_w8a32(xh, qu, su)
+    hh = np.stack([oracle.silu_mul(g[m], u[m]) for m in range(M)])
+    want = (oracle.dequant_gemv(hh[0], qd, sd)[None] if M == 1
+            else oracle.blis_gemm_w8a32(hh, qd, sd))
+    check_close(h.cpu().numpy(), hh)
+    check_close(y.cpu().numpy(), want)
+
+
+def test_norm_prologue_and_residual_epilogue(bh, oracle):
+    K, N = 1536, 2048
+    q, s = synthetic.quantized_linear(K, N, 21)
+    g = torch.Generator(device="cuda").manual_seed(3)
+    x = torch.randn((2, K), generator=g, device="cuda") * 3
+    w = 1 + 0.1 * torch.randn(K, generator=g, device="cuda")
+    bias = torch.randn(N, generator=g, device="cuda")
+    out = torch.empty((2, N), device="cuda")
+    linear(bh, A=x, lda=K, W0=ops.pack_w8(q), scale0=s, norm_w=w, norm_eps=float(EPS),
+           bias=bias, C=out, ldc=N, M=2, K=K, N=N, epilogue=0)
+    xh, wh, qh, sh, bh_ = (t.cpu().numpy() for t in (x, w, q, s, bias))
+    want = np.stack([bh_ + oracle.dequant_gemv(oracle.rmsnorm(xh[m], wh, EPS), qh, sh)
+                     for m in range(2)])
+    check_close(out.cpu().numpy(), want)
+    # residual: C += ...
+    c0 = torch.randn((2, N), generator=g, device="cuda")
+    c = c0.clone()
+    linear(bh, A=x, lda=K, W0=ops.pack_w8(q), scale0=s, C=c, ldc=N, M=2, K=K, N=N,
+           epilogue=1)
+    want = np.stack([oracle.dequant_gemv(xh[m], qh, sh, c0.cpu().numpy()[m])
+                     for m in range(2)])
+    check_close(c.cpu().numpy(), want)
+
+
+def test_standalone_elementwise_and_argmax(bh, oracle):
+    g = torch.Generator(device="cuda").manual_seed(5)
+    x = torch.randn((3, 1536), generator=g, device="cuda") * 2
+    w = 1 + 0.1 * torch.randn(1536, generator=g, device="cuda")
+    y = torch.empty_like(x)
+    torch.cuda.synchronize()
+    bma.check(bh.buddy_hip_rmsnorm(x.data_ptr(), w.data_ptr(), y.data_ptr(), 3, 1536,
+                                   float(EPS), None))
+    torch.cuda.synchronize()
+    for m in range(3):
+        check_close(y[m].cpu().numpy(), oracle.rmsnorm(x[m].cpu().numpy(), w.cpu().numpy(), EPS))
+    # RoPE
+    inv = synthetic.inv_freq(128)
+    qk = torch.randn((12, 128), generator=g, device="cuda")
+    want_in = qk.cpu().numpy()
+    pos = torch.tensor([777], dtype=torch.int32, device="cuda")
+    torch.cuda.synchronize()
+    bma.check(bh.buddy_hip_rope(qk.data_ptr(), inv.data_ptr(), pos.data_ptr(), 12, 128, None))
+    torch.cuda.synchronize()
+    c, s = oracle.rope_cos_sin(inv.cpu().numpy(), 777)
+    check_close(qk.cpu().numpy(), oracle.rope_apply(want_in, c, s))
+    # SiLU*mul
+    a = torch.randn(8960, generator=g, device="cuda") * 3
+    b = torch.randn(8960, generator=g, device="cuda")
+    h = torch.empty_like(a)
+    torch.cuda.synchronize()
+    bma.check(bh.buddy_hip_silu_mul(a.data_ptr(), b.data_ptr(), h.data_ptr(), 8960, None))
+    torch.cuda.synchronize()
+    check_close(h.cpu().numpy(), oracle.silu_mul(a.cpu().numpy(), b.cpu().numpy()))
+    # argmax: first maximum on ties
+    v = torch.randn(151936, generator=g, device="cuda")
+    v[[100, 5000, 151935]] = 50.0
+    ws = torch.empty(bh.buddy_hip_argmax_workspace_bytes(), dtype=torch.uint8, device="cuda")
+    out = torch.zeros(1, dtype=torch.int32, device="cuda")
+    torch.cuda.synchronize()
+    bma.check(bh.buddy_hip_argmax(v.data_ptr(), 151936, ws.data_ptr(), out.data_ptr(), None))
+    torch.cuda.synchronize()
+    assert int(out.item()) == 100 == oracle.argmax_first(v.cpu().numpy())
+
+
+@pytest.mark.parametrize("pos", [0, 8, 31, 32, 36, 612, 1023, 1087])
+def test_decode_attention_with_rope_and_kv_write(bh, oracle, pos):
+    """valid lengths 9/37/613/1024 are the reference's own check points
+    (frontend/Python/ops/tosa.py:14075-14080); 0/31/32 sit on chunk edges."""
+    H, HKV, D, L = 12, 2, 128, 1088
+    g = torch.Generator(device="cuda").manual_seed(pos + 1)
+    qkv = torch.randn((H + 2 * HKV) * D, generator=g, device="cuda")
+    kc = torch.randn((HKV, L, D), generator=g, device="cuda")
+    vc = torch.randn((HKV, L, D), generator=g, device="cuda")
+    kc[:, pos:, :] = 1e30  # rows at and beyond pos must not be read (pos is rewritten)
+    vc[:, pos:, :] = 1e30
+    inv = synthetic.inv_freq(D)
+    out = torch.empty(H * D, device="cuda")
+    pos_t = torch.tensor([pos], dtype=torch.int32, device="cuda")
+    nb = bh.buddy_hip_attn_decode_workspace_bytes(H, L)
+    ws = torch.empty(nb, dtype=torch.uint8, device="cuda")
+    kch, vch, qh = kc.cpu().numpy().copy(), vc.cpu().numpy().copy(), qkv.cpu().numpy()
+    scale = np.float32(0.0883883461)
+    torch.cuda.synchronize()
+    bma.check(bh.buddy_hip_gqa_decode_attention(
+        qkv.data_ptr(), inv.data_ptr(), pos_t.data_ptr(), kc.data_ptr(), vc.data_ptr(),
+        out.data_ptr(), H, HKV, D, L, float(scale), ws.data_ptr(), nb, None))
+    torch.cuda.synchronize()
+    # oracle: RoPE, cache write, then attention over the whole cache with the mask
+    c, s = oracle.rope_cos_sin(inv.cpu().numpy(), pos)
+    q = oracle.rope_apply(qh[:H * D].reshape(H, D), c, s)
+    k = oracle.rope_apply(qh[H * D:(H + HKV) * D].reshape(HKV, D), c, s)
+    v = qh[(H + HKV) * D:].reshape(HKV, D)
+    kch[:, pos, :] = k
+    vch[:, pos, :] = v
+    kch[:, pos + 1:, :] = 0  # the oracle multiplies masked rows by exactly 0
+    vch[:, pos + 1:, :] = 0
+    mask = np.where(np.arange(L) <= pos, 0.0, -np.inf).astype(np.float32)
+    want, _ = oracle.gqa_decode_attention(q, kch, vch, mask, scale, 4)
+    check_close(out.cpu().numpy().reshape(H, D), want)
+    # the new K/V rows landed in the cache, nothing else moved
+    check_close(kc[:, pos, :].cpu().numpy(), k)
+    np.testing.assert_array_equal(vc[:, pos, :].cpu().numpy(), v)
+    if pos:
+        np.testing.assert_array_equal(kc[:, :pos, :].cpu().numpy(), kch[:, :pos, :])
+
+
+def oracle_model(oracle, shape: Shape, host):
+    g = host["globals"]
+    od = dict(layers=shape.layers, hidden=shape.hidden, heads=shape.heads,
+              kv_heads=shape.kv_heads, head_dim=shape.head_dim, inter=shape.inter,
+              vocab=shape.vocab, max_len=shape.max_len, eps=shape.rms_eps,
+              attn_splits=4)
+    return oracle_lib.OracleModel(oracle, od, g["embed"], g["inv_freq"], host["layers"],
+                                  g["ln_f"], g["w_lm"], g["s_lm"])
+
+
+SMALL = Shape(layers=2, hidden=256, heads=4, kv_heads=2, head_dim=128, inter=512,
+              vocab=1024, max_len=128, rms_eps=1e-6)
+
+
+@pytest.mark.parametrize("graph", [False, True])
+def test_small_model_logits_kv_and_tokens(oracle, graph):
+    sess, host = synthetic.build_session(SMALL, context=40, keep_host=True, ln_jitter=0.1)
+    sess.use_graph(graph)
+    om = oracle_model(oracle, SMALL, host)
+    kv = [a.copy() for a in host["kv"]]
+    tok, toks_gpu, toks_cpu = 17, [], []
+    for step in range(12):
+        pos = 40 + step
+        nxt, logits = sess.decode(tok, pos)
+        otok, ologits = om.decode_step(tok, pos, kv)
+        check_close(logits, ologits)
+        toks_gpu.append(nxt)
+        toks_cpu.append(otok)
+        tok = otok
+    assert toks_gpu == toks_cpu
+    # every cache row the steps wrote matches the oracle's
+    for j in range(2 * SMALL.layers):
+        got = sess.get_kv(j)
+        check_close(got[:, 40:52, :], kv[j][:, 40:52, :])
+        np.testing.assert_array_equal(got[:, :40, :], host["kv"][j][:, :40, :])
+    sess.close()
+
+
+def test_small_model_greedy_feedback_matches_stepwise(oracle):
+    sess, host = synthetic.build_session(SMALL, context=16, keep_host=True, ln_jitter=0.1)
+    toks = sess.decode_greedy(5, 16, 24)
+    om = oracle_model(oracle, SMALL, host)
+    kv = [a.copy() for a in host["kv"]]
+    tok, want = 5, []
+    for step in range(24):
+        tok, _ = om.decode_step(tok, 16 + step, kv)
+        want.append(tok)
+    assert toks.tolist() == want
+    sess.close()
+
+
+def test_session_refuses_bad_arguments(bh):
+    sess, _ = synthetic.build_session(SMALL, context=0)
+    with pytest.raises(bma.BuddyHipError):
+        sess.decode(5, SMALL.max_len)  # position beyond the cache
+    with pytest.raises(bma.BuddyHipError):
+        sess.decode(SMALL.vocab, 0)  # token id out of range
+    with pytest.raises(bma.BuddyHipError):
+        sess.decode_greedy(1, SMALL.max_len - 3, 8)  # would run off the cache
+    sess.close()
+    bad = Shape(head_dim=64)
+    with pytest.raises(bma.BuddyHipError):
+        bma.session.DecoderSession(bad)
+
+
+@pytest.mark.timeout(900)
+def test_qwen2_1p5b_shape_64_greedy_steps(oracle):
+    """BASELINE config 3: 28 layers, hidden 1536, 12/2 heads, inter 8960, vocab
+    151936, context 1024, 64 greedy steps.  Token ids must match the oracle for
+    all 64 steps; logits are compared on the first and last step."""
+    shape = Shape()
+    sess, host = synthetic.build_session(shape, context=1024, keep_host=True)
+    first = int(synthetic.first_tokens(shape, 1)[0])
+    _, logits0 = sess.decode(first, 1024)  # step 0 once more, for its logits
+    toks = sess.decode_greedy(first, 1024, 64)
+    om = oracle_model(oracle, shape, host)
+    kv = host["kv"]
+    tok, want, margins = first, [], []
+    for step in range(64):
+        tok, logits = om.decode_step(tok, 1024 + step, kv)
+        if step == 0:
+            check_close(logits0, logits)
+        top2 = np.partition(logits, -2)[-2:]
+        margins.append(float(top2[1] - top2[0]))
+        want.append(tok)
+    got = toks.tolist()
+    diverge = next((i for i in range(64) if got[i] != want[i]), None)
+    assert diverge is None, (f"first divergence at step {diverge}, top-2 logit margin "
+                             f"there {margins[diverge]:.3e}")
+    # the 64 cache rows the run wrote, last layer
+    for j in (2 * shape.layers - 2, 2 * shape.layers - 1):
+        check_close(sess.get_kv(j)[:, 1024:1088, :], kv[j][:, 1024:1088, :])
+    sess.close()
