@@ -1,0 +1,218 @@
+#!/usr/bin/env python3
+"""Decode throughput of the int8 (w8a32) Qwen2-1.5B-shaped decoder on one
+MI355X, next to the CPU oracle timed on the same host.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+A step is one greedy decode step (one token) at batch 1 with the KV cache
+already holding 1024 positions; weights, KV cache and activations are resident
+in HBM before the timed region; each step's argmax feeds the next step on the
+device.  Prints one JSON line.
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+from pathlib import Path
+
+ROOT = Path(__file__).resolve().parent
+sys.path.insert(0, str(ROOT))
+sys.path.insert(0, str(ROOT / "tests"))
+
+HBM_PEAK_GBPS = 8000.0  # MI355X published HBM3E bandwidth
+CONTEXT = 1024
+
+
+def gate_up_bytes(hidden: int, inter: int) -> int:
+    """Algorithmic bytes of one fused RMSNorm + gate|up GEMV + SiLU*mul launch:
+    two int8 matrices, their scales, the activation row, the norm weight and
+    the output row."""
+    return 2 * hidden * inter + 2 * 4 * inter + 4 * hidden + 4 * hidden + 4 * inter
+
+
+def decode_step_bytes(shape, ctx: int) -> int:
+    """Algorithmic bytes of one decode step at context `ctx` (rows 0..ctx read)."""
+    H, I, V, L = shape.hidden, shape.inter, shape.vocab, shape.layers
+    QN, KVN = shape.heads * shape.head_dim, shape.kv_heads * shape.head_dim
+    w = L * (H * (QN + 2 * KVN) + QN * H + 3 * H * I) + H * V
+    scales = 4 * (L * (QN + 2 * KVN + H + 2 * I + H) + V)
+    kv = L * 2 * KVN * 4 * (ctx + 1)
+    norms = 4 * H * (2 * L + 1)
+    return w + scales + kv + norms + 4 * H + 4 * V
+
+
+def time_gate_up(bh, shape, sess_stream, layers, iters):
+    """Average duration of the dominant kernel (fused gate|up GEMV), launched
+    back to back over `layers` distinct weight sets (more than the 256 MB
+    last-level cache holds), timed with HIP events on the launch stream."""
+    import torch
+    from buddy_mlir_amd import check, ops, synthetic
+
+    class Desc(ctypes.Structure):
+        _fields_ = [("A", ctypes.c_void_p), ("lda", ctypes.c_int64),
+                    ("W0", ctypes.c_void_p), ("scale0", ctypes.c_void_p),
+                    ("W1", ctypes.c_void_p), ("scale1", ctypes.c_void_p),
+                    ("bias", ctypes.c_void_p), ("norm_w", ctypes.c_void_p),
+                    ("norm_eps", ctypes.c_float), ("C", ctypes.c_void_p),
+                    ("ldc", ctypes.c_int64), ("M", ctypes.c_int64),
+                    ("K", ctypes.c_int64), ("N", ctypes.c_int64),
+                    ("epilogue", ctypes.c_int)]
+
+    H, I = shape.hidden, shape.inter
+    sets = []
+    for i in range(layers):
+        qg, sg = synthetic.quantized_linear(H, I, 9000 + 2 * i)
+        qu, su = synthetic.quantized_linear(H, I, 9001 + 2 * i)
+        sets.append((ops.pack_w8(qg), sg, ops.pack_w8(qu), su))
+        del qg, qu
+    x = torch.randn((1, H), device="cuda")
+    w = torch.ones(H, device="cuda")
+    h = torch.empty((1, I), device="cuda")
+    descs = []
+    for pg, sg, pu, su in sets:
+        d = Desc()
+        d.A, d.lda, d.W0, d.scale0, d.W1, d.scale1 = (x.data_ptr(), H, pg.data_ptr(),
+                                                     sg.data_ptr(), pu.data_ptr(),
+                                                     su.data_ptr())
+        d.bias, d.norm_w, d.norm_eps = None, w.data_ptr(), shape.rms_eps
+        d.C, d.ldc, d.M, d.K, d.N, d.epilogue = h.data_ptr(), I, 1, H, I, 2
+        descs.append(d)
+    torch.cuda.synchronize()
+    stream = torch.cuda.ExternalStream(sess_stream)
+    for d in descs:
+        check(bh.buddy_hip_linear_w8a32(ctypes.byref(d), sess_stream))
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    stream.synchronize()
+    e0.record(stream)
+    for i in range(iters):
+        bh.buddy_hip_linear_w8a32(ctypes.byref(descs[i % layers]), sess_stream)
+    e1.record(stream)
+    e1.synchronize()
+    return e0.elapsed_time(e1) * 1e-3 / iters
+
+
+def cpu_baseline(shape, host, first_token, budget_s=12.0, max_steps=16):
+    """The CPU oracle (OpenMP restatement of the reference's kernels) on the
+    same weights: whole decode steps at context 1024 until ~budget_s is used."""
+    import oracle_lib
+
+    oracle = oracle_lib.load()
+    om = oracle_lib.model_from_host(oracle, shape, host)
+    kv = host["kv"]
+    tok = first_token
+    tok, _ = om.decode_step(tok, CONTEXT, kv)  # warm-up (page-in, thread start)
+    t0 = time.perf_counter()
+    n = 0
+    while n < max_steps:
+        tok, _ = om.decode_step(tok, CONTEXT + 1 + n, kv)
+        n += 1
+        if time.perf_counter() - t0 > budget_s:
+            break
+    dt = time.perf_counter() - t0
+    return {"value": n / dt, "unit": "tokens/s", "cores": oracle.num_threads(),
+            "kind": "port",
+            "sample": f"{n} decode steps at context {CONTEXT}, same weights, "
+                      f"{dt:.1f} s of CPU time"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=64)
+    ap.add_argument("--warmup", type=int, default=8)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-graph", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU's decode throughput; --gpus above 1 is "
+              "not supported in this build (nothing here uses a second GPU).",
+              file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    import buddy_mlir_amd as bma
+    from buddy_mlir_amd import synthetic
+    from buddy_mlir_amd.session import Shape
+
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    bh = bma.lib()
+    K, W = args.steps, args.warmup
+    max_len = (CONTEXT + W + K + 63) // 64 * 64
+    shape = Shape(max_len=max_len)
+    want_cpu = not args.no_cpu_baseline
+    sess, host = synthetic.build_session(shape, context=CONTEXT, keep_host=want_cpu)
+    sess.use_graph(not args.no_graph)
+    first = int(synthetic.first_tokens(shape, 1)[0])
+
+    stream = torch.cuda.ExternalStream(sess.stream)
+    sess.set_state(first, CONTEXT)
+    sess.enqueue_steps(W)
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    stream.synchronize()
+    t0 = time.perf_counter()
+    e0.record(stream)
+    sess.enqueue_steps(K)
+    e1.record(stream)
+    e1.synchronize()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    dev_s = e0.elapsed_time(e1) * 1e-3
+    step_s = max(dev_s, wall) / K  # the slower of the two clocks
+
+    # dominant kernel, measured live on its launch stream
+    gu_s = time_gate_up(bh, shape, sess.stream, layers=16, iters=160)
+    gu_b = gate_up_bytes(shape.hidden, shape.inter)
+    achieved = gu_b / gu_s / 1e9
+    step_b = decode_step_bytes(shape, CONTEXT + W + K // 2)
+
+    out = {
+        "metric": "decode_tokens_per_s",
+        "value": 1.0 / step_s,
+        "unit": "tokens/s",
+        "n_gpus": 1,
+        "steps": K,
+        "warmup": W,
+        "ms_per_step": step_s * 1e3,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {
+            "workload": "Qwen2-1.5B-shaped int8 weight-only (w8a32) decoder, one "
+                        "greedy decode step, batch 1, KV cache prefilled to 1024 "
+                        "positions (BASELINE configs[2])",
+            "layers": shape.layers, "hidden": shape.hidden, "heads": shape.heads,
+            "kv_heads": shape.kv_heads, "inter": shape.inter, "vocab": shape.vocab,
+            "context": CONTEXT, "hip_graph": not args.no_graph,
+        },
+        "decode_step_algorithmic_bytes": step_b,
+        "decode_step_hbm_gbps": step_b / step_s / 1e9,
+        "decode_step_hbm_frac": step_b / step_s / 1e9 / HBM_PEAK_GBPS,
+        "roofline": {
+            "kernel": "gemv_w8a32_kernel<1, 2, true> (RMSNorm + gate|up int8 GEMV "
+                      "+ SiLU*mul, 1536 -> 2 x 8960)",
+            "bound": "hbm",
+            "achieved": achieved,
+            "peak": HBM_PEAK_GBPS,
+            "unit": "GB/s",
+            "frac": achieved / HBM_PEAK_GBPS,
+            "algorithmic_bytes_per_launch": gu_b,
+            "avg_launch_us": gu_s * 1e6,
+            "traffic": None,
+        },
+    }
+    if want_cpu:
+        out["cpu_baseline"] = cpu_baseline(shape, host, first)
+    sess.close()
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

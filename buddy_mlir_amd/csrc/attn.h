@@ -5,6 +5,8 @@
 
 namespace bh {
 
+constexpr int kAttnChunk = 64; // cache positions per flash-decoding partial
+
 struct AttnDecodeArgs {
   const float *qkv = nullptr;      // [heads*D | kv_heads*D | kv_heads*D], pre-RoPE
   const float *inv_freq = nullptr; // [D/2]
@@ -16,7 +18,16 @@ struct AttnDecodeArgs {
   float scale = 0.f;
   void *workspace = nullptr; // flash-decoding partials
   size_t workspace_bytes = 0;
+  bool combine = true; // false: leave the partials for the consumer to fold
 };
+
+// Where the partials live inside the workspace.
+struct AttnPartials {
+  float *acc; // [heads, nchunks, head_dim]
+  float *ml;  // [heads, nchunks, 2] = (max, sum)
+  int nchunks;
+};
+AttnPartials attn_partials(void *workspace, int heads, int head_dim, int max_len);
 
 size_t attn_decode_workspace_bytes(int heads, int max_len);
 int launch_attn_decode(const AttnDecodeArgs &a, hipStream_t stream);

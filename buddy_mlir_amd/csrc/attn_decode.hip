@@ -14,17 +14,18 @@
 //     zero in the reference, so skipping them changes nothing);
 //   * one workgroup serves all query heads of a KV head, so K and V rows are
 //     read once per group, not once per query head;
-//   * the k range is cut into chunks of 32 positions (more, smaller partials
+//   * the k range is cut into chunks of 64 positions (more, smaller partials
 //     than the reference's 4): a decode step has only ~2 MB of KV per layer and
 //     is latency bound, so the chunks are what spreads it over the CUs.
-// Partials meet in a small workspace and a second kernel folds them in chunk
-// order with the reference's own combine rule.
+// Partials meet in a small workspace.  The decode step folds them while the
+// o_proj kernel stages its input; stand-alone callers get a second kernel that
+// folds them in chunk order with the reference's own combine rule.
 #include "attn.h"
 
 namespace bh {
 namespace {
 
-constexpr int kChunk = 32;       // cache positions per workgroup
+constexpr int kChunk = kAttnChunk; // cache positions per workgroup
 constexpr int kThreads = 256;
 constexpr int kMaxGroup = 8;     // query heads per KV head
 constexpr int kD = 128;          // head_dim this kernel is written for
@@ -70,11 +71,34 @@ __global__ void __launch_bounds__(kThreads) attn_decode_partial(AttnArgs a) {
   const int np = p1 - p0;
   const bool has_new = pos >= p0 && pos < p1;
 
+  // ---- the chunk's K and V rows are requested before anything else --------
+  // (rows that are not in the cache yet -- the current token's -- come from
+  // LDS later; their slots are loaded from row p0, which always exists)
+  const int sp = tid >> 2, spart = tid & 3; // scores: 4 threads per position
+  const int vq = tid & 31, vg = tid >> 5;   // P.V: 32 threads over d, 8 rows
+  float4 kreg[8], vreg[kChunk / 8];
+  {
+    const int prow = (sp < np && p0 + sp != pos) ? p0 + sp : p0;
+    const float *krow = a.kcache + ((size_t)kvh * a.max_len + prow) * kD + spart * 32;
+#pragma unroll
+    for (int c = 0; c < 8; ++c)
+      kreg[c] = *reinterpret_cast<const float4 *>(krow + c * 4);
+#pragma unroll
+    for (int i = 0; i < kChunk / 8; ++i) {
+      const int p = vg + 8 * i;
+      const int vrow = (p < np && p0 + p != pos) ? p0 + p : p0;
+      vreg[i] = *reinterpret_cast<const float4 *>(
+          a.vcache + ((size_t)kvh * a.max_len + vrow) * kD + vq * 4);
+    }
+  }
+
   // ---- RoPE tables for this position -------------------------------------
   if (tid < kD / 2) {
     const float ang = a.inv_freq[tid] * (float)pos;
-    cos_s[tid] = cosf(ang);
-    sin_s[tid] = sinf(ang);
+    float sn, cs;
+    sincosf(ang, &sn, &cs);
+    cos_s[tid] = cs;
+    sin_s[tid] = sn;
   }
   __syncthreads();
   // q' = q*cos + cat(-q[64:], q[:64])*sin for the G heads of this KV head
@@ -97,21 +121,20 @@ __global__ void __launch_bounds__(kThreads) attn_decode_partial(AttnArgs a) {
   }
   __syncthreads();
 
-  // ---- scores: 8 threads per position, 16 dims each ----------------------
+  // ---- scores: 4 threads per position, 32 dims each ----------------------
   {
-    const int p = tid >> 3, part = tid & 7;
+    const int p = sp, part = spart;
     float dot[kMaxGroup];
 #pragma unroll
     for (int h = 0; h < kMaxGroup; ++h)
       dot[h] = 0.f;
     if (p < np) {
       const bool is_new = (p0 + p == pos);
-      const float *krow = is_new ? knew_s
-                                 : a.kcache + ((size_t)kvh * a.max_len + p0 + p) * kD;
 #pragma unroll
-      for (int c = 0; c < 4; ++c) {
-        const int d = part * 16 + c * 4;
-        const float4 kv = *reinterpret_cast<const float4 *>(krow + d);
+      for (int c = 0; c < 8; ++c) {
+        const int d = part * 32 + c * 4;
+        const float4 kv =
+            is_new ? *reinterpret_cast<const float4 *>(knew_s + d) : kreg[c];
 #pragma unroll
         for (int h = 0; h < kMaxGroup; ++h) {
           if (h < G) {
@@ -128,9 +151,8 @@ __global__ void __launch_bounds__(kThreads) attn_decode_partial(AttnArgs a) {
     for (int h = 0; h < kMaxGroup; ++h) {
       dot[h] += __shfl_xor(dot[h], 1, 64);
       dot[h] += __shfl_xor(dot[h], 2, 64);
-      dot[h] += __shfl_xor(dot[h], 4, 64);
     }
-    if (part == 0 && p < kChunk) {
+    if (part == 0) {
 #pragma unroll
       for (int h = 0; h < kMaxGroup; ++h)
         if (h < G)
@@ -139,51 +161,46 @@ __global__ void __launch_bounds__(kThreads) attn_decode_partial(AttnArgs a) {
   }
   __syncthreads();
 
-  // ---- per-head max, exp, sum over the chunk: one 32-lane half per head ----
-  {
-    const int h = tid >> 5, p = tid & 31;
-    if (h < G) {
-      const float s = sc_s[h][p];
-      float m = s;
-#pragma unroll
-      for (int o = 16; o > 0; o >>= 1)
-        m = fmaxf(m, __shfl_xor(m, o, 64));
-      const float e = expf(s - m); // -inf -> 0 for the positions beyond pos
-      float l = e;
-#pragma unroll
-      for (int o = 16; o > 0; o >>= 1)
-        l += __shfl_xor(l, o, 64);
-      sc_s[h][p] = e;
-      if (p == 0) {
-        m_s[h] = m;
-        l_s[h] = l;
-      }
+  // ---- per-head max, exp, sum over the chunk: one wavefront per head -------
+  for (int h = tid >> 6; h < G; h += kThreads / 64) {
+    const int p = tid & 63;
+    const float s = sc_s[h][p];
+    const float m = wave_max(s);
+    const float e = expf(s - m); // -inf -> 0 for the positions beyond pos
+    const float l = wave_sum(e);
+    sc_s[h][p] = e;
+    if (p == 0) {
+      m_s[h] = m;
+      l_s[h] = l;
     }
   }
   __syncthreads();
 
   // ---- acc[h][d] = sum_p e[h][p] * V[p][d]: 32 threads across d, 8 rows of p
   {
-    const int dq = tid & 31, pg = tid >> 5;
+    const int dq = vq, pg = vg;
     float acc[kMaxGroup][4];
 #pragma unroll
     for (int h = 0; h < kMaxGroup; ++h)
 #pragma unroll
       for (int j = 0; j < 4; ++j)
         acc[h][j] = 0.f;
-    for (int p = pg; p < np; p += kThreads / 32) {
-      const bool is_new = (p0 + p == pos);
-      const float *vrow = is_new ? vnew_s
-                                 : a.vcache + ((size_t)kvh * a.max_len + p0 + p) * kD;
-      const float4 v = *reinterpret_cast<const float4 *>(vrow + dq * 4);
 #pragma unroll
-      for (int h = 0; h < kMaxGroup; ++h) {
-        if (h < G) {
-          const float e = sc_s[h][p];
-          acc[h][0] = fmaf(v.x, e, acc[h][0]);
-          acc[h][1] = fmaf(v.y, e, acc[h][1]);
-          acc[h][2] = fmaf(v.z, e, acc[h][2]);
-          acc[h][3] = fmaf(v.w, e, acc[h][3]);
+    for (int i = 0; i < kChunk / 8; ++i) {
+      const int p = pg + 8 * i;
+      if (p < np) {
+        const bool is_new = (p0 + p == pos);
+        const float4 v =
+            is_new ? *reinterpret_cast<const float4 *>(vnew_s + dq * 4) : vreg[i];
+#pragma unroll
+        for (int h = 0; h < kMaxGroup; ++h) {
+          if (h < G) {
+            const float e = sc_s[h][p];
+            acc[h][0] = fmaf(v.x, e, acc[h][0]);
+            acc[h][1] = fmaf(v.y, e, acc[h][1]);
+            acc[h][2] = fmaf(v.z, e, acc[h][2]);
+            acc[h][3] = fmaf(v.w, e, acc[h][3]);
+          }
         }
       }
     }
@@ -237,9 +254,17 @@ size_t attn_decode_workspace_bytes(int heads, int max_len) {
   return sizeof(float) * (size_t)heads * nchunks * (kD + 2);
 }
 
+AttnPartials attn_partials(void *workspace, int heads, int head_dim, int max_len) {
+  AttnPartials p;
+  p.nchunks = (int)ceil_div(max_len, kChunk);
+  p.acc = static_cast<float *>(workspace);
+  p.ml = p.acc + (size_t)heads * p.nchunks * head_dim;
+  return p;
+}
+
 int launch_attn_decode(const AttnDecodeArgs &in, hipStream_t stream) {
   BH_REQUIRE(in.qkv && in.inv_freq && in.pos_ptr && in.kcache && in.vcache &&
-                 in.out && in.workspace,
+                 (in.out || !in.combine) && in.workspace,
              "attn_decode: null pointer");
   BH_REQUIRE(in.head_dim == kD, "attn_decode: head_dim %d (only %d is built)",
              in.head_dim, kD);
@@ -265,12 +290,14 @@ int launch_attn_decode(const AttnDecodeArgs &in, hipStream_t stream) {
   a.max_len = in.max_len;
   a.nchunks = (int)ceil_div(in.max_len, kChunk);
   a.scale = in.scale;
-  a.part_acc = static_cast<float *>(in.workspace);
-  a.part_ml = a.part_acc + (size_t)in.heads * a.nchunks * kD;
+  const AttnPartials parts = attn_partials(in.workspace, in.heads, kD, in.max_len);
+  a.part_acc = parts.acc;
+  a.part_ml = parts.ml;
   a.out = in.out;
   hipLaunchKernelGGL(attn_decode_partial, dim3(a.nchunks, in.kv_heads),
                      dim3(kThreads), 0, stream, a);
-  hipLaunchKernelGGL(attn_decode_combine, dim3(in.heads), dim3(kD), 0, stream, a);
+  if (in.combine)
+    hipLaunchKernelGGL(attn_decode_combine, dim3(in.heads), dim3(kD), 0, stream, a);
   BH_CHECK_HIP(hipGetLastError());
   return BUDDY_HIP_OK;
 }

@@ -27,6 +27,12 @@ struct GemvArgs {
   const float *norm_w = nullptr;
   float norm_eps = 0.f;
   float norm_inv_k = 0.f;
+  // Alternative input: A = attention output folded on the fly from flash-
+  // decoding partials (acc [heads, nchunks, head_dim], ml [heads, nchunks, 2]),
+  // chunks 0 .. *pos_ptr / attn_chunk; A is ignored then.
+  const float *attn_acc = nullptr, *attn_ml = nullptr;
+  const int *pos_ptr = nullptr;
+  int attn_nchunks = 0, attn_chunk = 0, head_dim = 0;
   int M = 1;
   int64_t K = 0, N = 0;
   int epilogue = kEpiStore;

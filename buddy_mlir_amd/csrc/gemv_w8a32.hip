@@ -34,7 +34,8 @@ constexpr int kMaxWaves = 16;            // wavefronts per workgroup
 constexpr int kXStride = 20;             // floats per (tile, k-group) in LDS:
                                          // 16 used + 4 pad, conflict-free b128
 constexpr int kTileFloats = 4 * kXStride; // 80 floats of LDS per staged tile
-constexpr size_t kMaxLdsBytes = 144 * 1024;
+constexpr size_t kMaxLdsBytes = 144 * 1024; // hard limit of one workgroup
+constexpr size_t kLdsBudget = 40 * 1024;    // preferred, keeps ~4 workgroups per CU
 
 struct GemvPlan {
   int64_t chunks, groups;
@@ -79,7 +80,7 @@ GemvPlan make_plan(int64_t M, int64_t K, int64_t N, bool dual) {
   p.G = p.waves / ks;
   p.blocks = (int)ceil_div(p.groups, p.G);
   const int64_t tiles = ceil_div(p.chunks, ks);
-  int64_t cap = (int64_t)((kMaxLdsBytes - red_bytes(p.waves)) / round_bytes(p.waves, 1));
+  int64_t cap = (int64_t)(kLdsBudget / round_bytes(p.waves, 1));
   cap = cap / 4 * 4; // rounds are whole batches of four tiles
   if (cap < 4)
     cap = 4;
@@ -98,6 +99,10 @@ struct KernelArgs {
   int K, N, groups, chunks;
   int G, KS, tiles_per_round;
   int rows; // valid rows; the kernel is compiled for the next power of two
+  // activation provider 2: fold flash-decoding partials while staging
+  const float *attn_acc, *attn_ml;
+  const int *pos_ptr;
+  int attn_nchunks, attn_chunk, head_dim;
 };
 
 typedef int v4i __attribute__((ext_vector_type(4)));
@@ -160,10 +165,65 @@ __device__ __forceinline__ void finish(const KernelArgs &a, int m, int n,
   }
 }
 
-template <int M, int EPI, bool NORM>
+// Combined attention output for 4 consecutive k of one head, from the
+// flash-decoding partials (m, l, acc) of the chunks used so far:
+//   w_s = exp(m_s - max m); x = sum_s w_s acc_s / sum_s w_s l_s
+// (the combine of frontend/Python/ops/tosa.py:14485-14594, eight chunks at a
+// time so that their loads are in flight together).
+__device__ __forceinline__ float4 attn_combined(const KernelArgs &a, int k) {
+  constexpr int B = 8; // partials fetched per batch
+  const int h = k / a.head_dim, d = k % a.head_dim;
+  const int pos = *a.pos_ptr;
+  const int used = min(a.attn_nchunks, pos / a.attn_chunk + 1);
+  const float2 *ml = reinterpret_cast<const float2 *>(a.attn_ml) +
+                     (size_t)h * a.attn_nchunks;
+  const float *acc = a.attn_acc + (size_t)h * a.attn_nchunks * a.head_dim + d;
+  float4 r = make_float4(0.f, 0.f, 0.f, 0.f);
+  float m = -1.0e30f, l = 0.f;
+  for (int s0 = 0; s0 < used; s0 += B) {
+    float2 mlv[B];
+    float4 v[B];
+#pragma unroll
+    for (int j = 0; j < B; ++j) {
+      const int s = min(s0 + j, used - 1);
+      mlv[j] = ml[s];
+      v[j] = *reinterpret_cast<const float4 *>(acc + (size_t)s * a.head_dim);
+    }
+    float mb = m;
+#pragma unroll
+    for (int j = 0; j < B; ++j)
+      if (s0 + j < used)
+        mb = fmaxf(mb, mlv[j].x);
+    const float al = expf(m - mb); // rescale what was gathered so far
+    r.x *= al;
+    r.y *= al;
+    r.z *= al;
+    r.w *= al;
+    l *= al;
+    m = mb;
+#pragma unroll
+    for (int j = 0; j < B; ++j) {
+      if (s0 + j < used) {
+        const float w = expf(mlv[j].x - m);
+        l = fmaf(mlv[j].y, w, l);
+        r.x = fmaf(v[j].x, w, r.x);
+        r.y = fmaf(v[j].y, w, r.y);
+        r.z = fmaf(v[j].z, w, r.z);
+        r.w = fmaf(v[j].w, w, r.w);
+      }
+    }
+  }
+  const float inv = 1.0f / l;
+  return make_float4(r.x * inv, r.y * inv, r.z * inv, r.w * inv);
+}
+
+enum { kProPlain = 0, kProNorm = 1, kProAttn = 2 };
+
+template <int M, int EPI, int PRO>
 __global__ void __launch_bounds__(kMaxWaves *kWave)
     gemv_w8a32_kernel(KernelArgs a) {
   constexpr bool DUAL = (EPI == kEpiSiluMul);
+  constexpr bool NORM = (PRO == kProNorm);
   constexpr int U = 4; // weight loads in flight per matrix
   extern __shared__ float lds[];
   const int tid = threadIdx.x;
@@ -230,7 +290,10 @@ __global__ void __launch_bounds__(kMaxWaves *kWave)
 #pragma unroll
       for (int m = 0; m < M; ++m) {
         float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (m < a.rows) {
+        if (PRO == kProAttn) {
+          if (m == 0 && in)
+            v = attn_combined(a, k);
+        } else if (m < a.rows) {
           const float *src = a.A + (int64_t)m * a.lda + k;
           if (in && ((reinterpret_cast<uintptr_t>(src) & 15) == 0))
             v = *reinterpret_cast<const float4 *>(src);
@@ -357,9 +420,9 @@ __global__ void __launch_bounds__(kMaxWaves *kWave)
   }
 }
 
-template <int M, int EPI, bool NORM>
+template <int M, int EPI, int PRO>
 int launch_one(const KernelArgs &ka, const GemvPlan &p, hipStream_t stream) {
-  auto kernel = gemv_w8a32_kernel<M, EPI, NORM>;
+  auto kernel = gemv_w8a32_kernel<M, EPI, PRO>;
   static bool attr_set = false;
   if (!attr_set) {
     BH_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
@@ -377,16 +440,21 @@ template <int M>
 int launch_m(const GemvArgs &a, const KernelArgs &ka, const GemvPlan &p,
              hipStream_t stream) {
   const bool norm = a.norm_w != nullptr;
+  if (a.attn_acc) { // only the o_proj of a decode step: M = 1, residual add
+    if (M == 1 && a.epilogue == kEpiAccum)
+      return launch_one<1, kEpiAccum, kProAttn>(ka, p, stream);
+    return fail(BUDDY_HIP_ERR_ARG, "gemv: attention input needs M=1 + ACCUM");
+  }
   switch (a.epilogue) {
   case kEpiStore:
-    return norm ? launch_one<M, kEpiStore, true>(ka, p, stream)
-                : launch_one<M, kEpiStore, false>(ka, p, stream);
+    return norm ? launch_one<M, kEpiStore, kProNorm>(ka, p, stream)
+                : launch_one<M, kEpiStore, kProPlain>(ka, p, stream);
   case kEpiAccum:
-    return norm ? launch_one<M, kEpiAccum, true>(ka, p, stream)
-                : launch_one<M, kEpiAccum, false>(ka, p, stream);
+    return norm ? launch_one<M, kEpiAccum, kProNorm>(ka, p, stream)
+                : launch_one<M, kEpiAccum, kProPlain>(ka, p, stream);
   case kEpiSiluMul:
-    return norm ? launch_one<M, kEpiSiluMul, true>(ka, p, stream)
-                : launch_one<M, kEpiSiluMul, false>(ka, p, stream);
+    return norm ? launch_one<M, kEpiSiluMul, kProNorm>(ka, p, stream)
+                : launch_one<M, kEpiSiluMul, kProPlain>(ka, p, stream);
   }
   return fail(BUDDY_HIP_ERR_ARG, "gemv: unknown epilogue %d", a.epilogue);
 }
@@ -398,11 +466,16 @@ int compiled_rows(int64_t M) {
 } // namespace
 
 int launch_gemv(const GemvArgs &a, hipStream_t stream) {
-  BH_REQUIRE(a.A && a.W0 && a.s0 && a.C, "gemv: null pointer");
+  BH_REQUIRE((a.A || a.attn_acc) && a.W0 && a.s0 && a.C, "gemv: null pointer");
+  BH_REQUIRE(!a.attn_acc || (a.attn_ml && a.pos_ptr && a.attn_nchunks > 0 &&
+                             a.attn_chunk > 0 && a.head_dim > 0 &&
+                             a.head_dim % 4 == 0 && a.K % a.head_dim == 0),
+             "gemv: incomplete attention-partials input");
   BH_REQUIRE(a.M >= 1 && a.M <= 16, "gemv: M=%d outside 1..16", a.M);
   BH_REQUIRE(a.K > 0 && a.N > 0 && a.K < (1 << 30) && a.N < (1 << 30),
              "gemv: bad shape K=%lld N=%lld", (long long)a.K, (long long)a.N);
-  BH_REQUIRE(a.lda >= a.K && a.ldc >= a.N, "gemv: row stride below row length");
+  BH_REQUIRE((a.attn_acc || a.lda >= a.K) && a.ldc >= a.N,
+             "gemv: row stride below row length");
   const bool dual = a.epilogue == kEpiSiluMul;
   BH_REQUIRE(!dual || (a.W1 && a.s1), "gemv: SiLU*mul needs two matrices");
   BH_REQUIRE((reinterpret_cast<uintptr_t>(a.W0) & 15) == 0 &&
@@ -435,6 +508,12 @@ int launch_gemv(const GemvArgs &a, hipStream_t stream) {
   ka.KS = p.KS;
   ka.tiles_per_round = p.tiles_per_round;
   ka.rows = a.M;
+  ka.attn_acc = a.attn_acc;
+  ka.attn_ml = a.attn_ml;
+  ka.pos_ptr = a.pos_ptr;
+  ka.attn_nchunks = a.attn_nchunks;
+  ka.attn_chunk = a.attn_chunk;
+  ka.head_dim = a.head_dim;
   switch (mt) {
   case 1: return launch_m<1>(a, ka, p, stream);
   case 2: return launch_m<2>(a, ka, p, stream);

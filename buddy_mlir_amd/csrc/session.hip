@@ -8,10 +8,10 @@
 // (runtime/llm/TextGeneration.cpp:215-266, Sampler.h:101-104).
 //
 // Weights are repacked once into wave tiles and stay in HBM together with the
-// f32 KV cache; a decode step is 6 kernels per layer on one stream:
+// f32 KV cache; a decode step is 5 kernels per layer on one stream:
 //   [RMSNorm + q|k|v GEMV] -> [RoPE + KV write + attention partials] ->
-//   [combine] -> [o_proj GEMV + residual] -> [RMSNorm + gate|up GEMV + SiLU*mul]
-//   -> [down GEMV + residual]
+//   [fold partials + o_proj GEMV + residual] ->
+//   [RMSNorm + gate|up GEMV + SiLU*mul] -> [down GEMV + residual]
 // followed by [RMSNorm + lm_head GEMV], a two-stage argmax and a bookkeeping
 // kernel.  Token id, position and step counter live in device memory, so the
 // whole step is captured once into a hipGraph and replayed; greedy decoding
@@ -168,10 +168,30 @@ struct Session {
       a.scale = scale;
       a.workspace = attn_ws;
       a.workspace_bytes = attn_ws_bytes;
+      a.combine = false; // o_proj folds the partials while staging its input
       if ((rc = launch_attn_decode(a, stream)))
         return rc;
-      if ((rc = gemv(att, L.o, nullptr, nullptr, x, kEpiAccum)))
-        return rc;
+      {
+        const AttnPartials parts =
+            attn_partials(attn_ws, S.heads, S.head_dim, S.max_len);
+        GemvArgs g;
+        g.attn_acc = parts.acc;
+        g.attn_ml = parts.ml;
+        g.attn_nchunks = parts.nchunks;
+        g.attn_chunk = kAttnChunk;
+        g.head_dim = S.head_dim;
+        g.pos_ptr = state + 1;
+        g.W0 = L.o.w;
+        g.s0 = L.o.s;
+        g.C = x;
+        g.ldc = L.o.N;
+        g.M = 1;
+        g.K = L.o.K;
+        g.N = L.o.N;
+        g.epilogue = kEpiAccum;
+        if ((rc = launch_gemv(g, stream)))
+          return rc;
+      }
       if ((rc = gemv(x, L.gate, &L.up, L.ln2, h, kEpiSiluMul)))
         return rc;
       if ((rc = gemv(h, L.down, nullptr, nullptr, x, kEpiAccum)))

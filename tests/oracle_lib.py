@@ -277,6 +277,18 @@ class OracleModel:
         return int(tok), logits
 
 
+def model_from_host(oracle: Oracle, shape, host) -> OracleModel:
+    """OracleModel over the numpy copies made by
+    buddy_mlir_amd.synthetic.build_session(keep_host=True)."""
+    g = host["globals"]
+    od = dict(layers=shape.layers, hidden=shape.hidden, heads=shape.heads,
+              kv_heads=shape.kv_heads, head_dim=shape.head_dim, inter=shape.inter,
+              vocab=shape.vocab, max_len=shape.max_len, eps=shape.rms_eps,
+              attn_splits=4)
+    return OracleModel(oracle, od, g["embed"], g["inv_freq"], host["layers"],
+                       g["ln_f"], g["w_lm"], g["s_lm"])
+
+
 _cached = None
 
 

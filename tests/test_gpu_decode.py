@@ -179,13 +179,7 @@ def test_decode_attention_with_rope_and_kv_write(bh, oracle, pos):
 
 
 def oracle_model(oracle, shape: Shape, host):
-    g = host["globals"]
-    od = dict(layers=shape.layers, hidden=shape.hidden, heads=shape.heads,
-              kv_heads=shape.kv_heads, head_dim=shape.head_dim, inter=shape.inter,
-              vocab=shape.vocab, max_len=shape.max_len, eps=shape.rms_eps,
-              attn_splits=4)
-    return oracle_lib.OracleModel(oracle, od, g["embed"], g["inv_freq"], host["layers"],
-                                  g["ln_f"], g["w_lm"], g["s_lm"])
+    return oracle_lib.model_from_host(oracle, shape, host)
 
 
 SMALL = Shape(layers=2, hidden=256, heads=4, kv_heads=2, head_dim=128, inter=512,
