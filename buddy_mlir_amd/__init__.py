@@ -90,6 +90,7 @@ def _declare(lib):
         "buddy_hip_gemv_w8a32": (c_int, [vp, vp, vp, vp, i64, i64, i64, c_uint,
                                          vp]),
         "buddy_hip_linear_w8a32": (c_int, [vp, vp]),
+        "buddy_hip_gemm_w8a32": (c_int, [vp, vp, vp, vp, i64, i64, i64, c_uint, vp]),
         "buddy_hip_rmsnorm": (c_int, [vp, vp, vp, c_int, c_int, c_float, vp]),
         "buddy_hip_rope": (c_int, [vp, vp, vp, c_int, c_int, vp]),
         "buddy_hip_silu_mul": (c_int, [vp, vp, vp, i64, vp]),
@@ -99,6 +100,8 @@ def _declare(lib):
         "buddy_hip_gqa_decode_attention": (c_int, [vp, vp, vp, vp, vp, vp, c_int,
                                                    c_int, c_int, c_int, c_float,
                                                    vp, sz, vp]),
+        "buddy_hip_prefill_attention": (c_int, [vp, vp, vp, vp, vp, c_int, c_int, c_int,
+                                                c_int, c_int, c_float, vp]),
         "buddy_hip_session_create": (vp, [vp, vp]),
         "buddy_hip_session_destroy": (None, [vp]),
         "buddy_hip_session_set_globals": (c_int, [vp, vp, vp, vp, vp, vp]),
@@ -108,6 +111,8 @@ def _declare(lib):
         "buddy_hip_session_use_graph": (c_int, [vp, c_int]),
         "buddy_hip_session_decode": (c_int, [vp, c_int, c_int, vp, vp]),
         "buddy_hip_session_decode_greedy": (c_int, [vp, c_int, c_int, c_int, vp]),
+        "buddy_hip_session_prefill": (c_int, [vp, vp, c_int, c_int, vp, vp]),
+        "buddy_hip_session_set_prefill_precision": (c_int, [vp, c_int]),
         "buddy_hip_session_set_state": (c_int, [vp, c_int, c_int]),
         "buddy_hip_session_enqueue_steps": (c_int, [vp, c_int]),
         "buddy_hip_session_logits": (vp, [vp]),

@@ -29,6 +29,24 @@ struct AttnPartials {
 };
 AttnPartials attn_partials(void *workspace, int heads, int head_dim, int max_len);
 
+struct AttnPrefillArgs {
+  const float *q = nullptr;   // token t, head h at q + t*q_stride + h*q_hstride
+  const float *k = nullptr;   // [kv_heads, kv_stride rows, head_dim]
+  const float *v = nullptr;
+  const float *mask = nullptr; // additive [q_len, k_len]; null = causal
+  float *out = nullptr;        // token t, head h at out + t*o_stride + h*o_hstride
+  int64_t q_stride = 0, q_hstride = 0, o_stride = 0, o_hstride = 0, kv_stride = 0;
+  int heads = 0, kv_heads = 0, head_dim = 0, q_len = 0, k_len = 0;
+  float scale = 0.f;
+};
+int launch_attn_prefill(const AttnPrefillArgs &a, hipStream_t stream);
+// Rotates q in place for n_tokens rows of [q | k | v], writes rotated k and v
+// into cache rows start_pos .. start_pos + n_tokens - 1.
+int launch_rope_kv_write(float *qkv, int64_t row_stride, const float *inv_freq,
+                         float *kcache, float *vcache, int heads, int kv_heads,
+                         int head_dim, int max_len, int start_pos, int n_tokens,
+                         hipStream_t stream);
+
 size_t attn_decode_workspace_bytes(int heads, int max_len);
 int launch_attn_decode(const AttnDecodeArgs &a, hipStream_t stream);
 

@@ -19,6 +19,7 @@
 // host round trip.
 #include "attn.h"
 #include "elementwise.h"
+#include "gemm.h"
 #include "gemv_w8a32.h"
 
 #include <cmath>
@@ -42,6 +43,19 @@ struct Layer {
   float *kc = nullptr, *vc = nullptr; // [kv_heads, max_len, D]
   bool set = false;
 };
+
+// x[t, :] = table[token[t], :]
+__global__ void __launch_bounds__(256)
+embedding_rows_kernel(const float *__restrict__ table, const int *__restrict__ tokens,
+                      int64_t hidden, int64_t vocab, float *__restrict__ out) {
+  int64_t t = tokens[blockIdx.x];
+  if (t < 0 || t >= vocab)
+    t = 0;
+  const float *row = table + t * hidden;
+  float *dst = out + (int64_t)blockIdx.x * hidden;
+  for (int64_t i = threadIdx.x; i < hidden; i += 256)
+    dst[i] = row[i];
+}
 
 __global__ void advance_kernel(int *state) {
   // state: [0] token, [1] pos, [2] step
@@ -74,6 +88,12 @@ struct Session {
   hipGraphExec_t graph_exec = nullptr;
   bool use_graph = true;
   std::vector<void *> owned;
+  // prefill activations, grown on demand: rows = tokens per prefill call
+  int pf_rows = 0;
+  float *pf_x = nullptr, *pf_xn = nullptr, *pf_qkv = nullptr, *pf_att = nullptr,
+        *pf_g = nullptr, *pf_u = nullptr;
+  int *pf_tokens = nullptr;
+  int gemm_terms = 1; // bf16 terms per activation in the prefill matmuls
 
   template <typename T> int alloc(T **p, size_t n) {
     void *q = nullptr;
@@ -207,6 +227,102 @@ struct Session {
     return BUDDY_HIP_OK;
   }
 
+  int ensure_prefill_buffers(int rows) {
+    if (rows <= pf_rows)
+      return BUDDY_HIP_OK;
+    const auto &S = shape;
+    const size_t QN = (size_t)S.heads * S.head_dim, KVN = (size_t)S.kv_heads * S.head_dim;
+    for (float **p : {&pf_x, &pf_xn, &pf_qkv, &pf_att, &pf_g, &pf_u})
+      if (*p) {
+        (void)hipFree(*p);
+        *p = nullptr;
+      }
+    if (pf_tokens)
+      (void)hipFree(pf_tokens);
+    pf_rows = 0;
+    BH_CHECK_HIP(hipMalloc((void **)&pf_x, sizeof(float) * rows * S.hidden));
+    BH_CHECK_HIP(hipMalloc((void **)&pf_xn, sizeof(float) * rows * S.hidden));
+    BH_CHECK_HIP(hipMalloc((void **)&pf_qkv, sizeof(float) * rows * (QN + 2 * KVN)));
+    BH_CHECK_HIP(hipMalloc((void **)&pf_att, sizeof(float) * rows * QN));
+    BH_CHECK_HIP(hipMalloc((void **)&pf_g, sizeof(float) * rows * S.inter));
+    BH_CHECK_HIP(hipMalloc((void **)&pf_u, sizeof(float) * rows * S.inter));
+    BH_CHECK_HIP(hipMalloc((void **)&pf_tokens, sizeof(int) * rows));
+    pf_rows = rows;
+    return BUDDY_HIP_OK;
+  }
+
+  int gemm(const float *A, const PackedLinear &W, float *C, int64_t M, bool accumulate) {
+    GemmW8Args g;
+    g.A = A;
+    g.lda = W.K;
+    g.W = W.w;
+    g.scale = W.s;
+    g.bias = accumulate ? nullptr : W.b;
+    g.C = C;
+    g.ldc = W.N;
+    g.M = M;
+    g.K = W.K;
+    g.N = W.N;
+    g.accumulate = accumulate;
+    g.terms = gemm_terms;
+    return launch_gemm_w8(g, stream);
+  }
+
+  // Prompt processing for tokens already in pf_tokens: fills cache rows
+  // start_pos .. start_pos+n-1 and leaves the final hidden states in pf_x
+  // (op order of a layer: subgraph0_decode_simplify.mlir:60-232 over n rows).
+  int enqueue_prefill(int n, int start_pos) {
+    const auto &S = shape;
+    const int64_t QKV = (int64_t)(S.heads + 2 * S.kv_heads) * S.head_dim;
+    const float scale = (float)(1.0 / std::sqrt((double)S.head_dim));
+    hipLaunchKernelGGL(embedding_rows_kernel, dim3(n), dim3(256), 0, stream, embed,
+                       pf_tokens, (int64_t)S.hidden, (int64_t)S.vocab, pf_x);
+    BH_CHECK_HIP(hipGetLastError());
+    int rc;
+    for (int i = 0; i < S.layers; ++i) {
+      Layer &L = layers[(size_t)i];
+      if ((rc = launch_rmsnorm(pf_x, L.ln1, pf_xn, n, S.hidden, S.rms_eps, stream)))
+        return rc;
+      if ((rc = gemm(pf_xn, L.qkv, pf_qkv, n, false)))
+        return rc;
+      if ((rc = launch_rope_kv_write(pf_qkv, QKV, inv_freq, L.kc, L.vc, S.heads,
+                                     S.kv_heads, S.head_dim, S.max_len, start_pos,
+                                     n, stream)))
+        return rc;
+      AttnPrefillArgs a;
+      a.q = pf_qkv;
+      a.q_stride = QKV;
+      a.q_hstride = S.head_dim;
+      a.k = L.kc;
+      a.v = L.vc;
+      a.kv_stride = S.max_len;
+      a.out = pf_att;
+      a.o_stride = (int64_t)S.heads * S.head_dim;
+      a.o_hstride = S.head_dim;
+      a.heads = S.heads;
+      a.kv_heads = S.kv_heads;
+      a.head_dim = S.head_dim;
+      a.q_len = n;
+      a.k_len = start_pos + n;
+      a.scale = scale;
+      if ((rc = launch_attn_prefill(a, stream)))
+        return rc;
+      if ((rc = gemm(pf_att, L.o, pf_x, n, true)))
+        return rc;
+      if ((rc = launch_rmsnorm(pf_x, L.ln2, pf_xn, n, S.hidden, S.rms_eps, stream)))
+        return rc;
+      if ((rc = gemm(pf_xn, L.gate, pf_g, n, false)))
+        return rc;
+      if ((rc = gemm(pf_xn, L.up, pf_u, n, false)))
+        return rc;
+      if ((rc = launch_silu_mul(pf_g, pf_u, pf_g, (int64_t)n * S.inter, stream)))
+        return rc;
+      if ((rc = gemm(pf_g, L.down, pf_x, n, true)))
+        return rc;
+    }
+    return BUDDY_HIP_OK;
+  }
+
   int ready() const {
     if (!embed || !ln_f || !lm.w)
       return fail(BUDDY_HIP_ERR_ARG, "session: embedding / head not set");
@@ -334,6 +450,10 @@ void buddy_hip_session_destroy(buddy_hip_session *hs) {
   s->drop_graph();
   for (void *p : s->owned)
     (void)hipFree(p);
+  for (void *p : {(void *)s->pf_x, (void *)s->pf_xn, (void *)s->pf_qkv, (void *)s->pf_att,
+                  (void *)s->pf_g, (void *)s->pf_u, (void *)s->pf_tokens})
+    if (p)
+      (void)hipFree(p);
   if (s->host_state)
     (void)hipHostFree(s->host_state);
   if (s->own_stream)
@@ -511,6 +631,64 @@ int buddy_hip_session_decode_greedy(buddy_hip_session *hs, int first_token,
   BH_CHECK_HIP(hipMemcpyAsync(tokens_out, s->token_log, sizeof(int) * steps,
                               hipMemcpyDefault, s->stream));
   BH_CHECK_HIP(hipStreamSynchronize(s->stream));
+  return BUDDY_HIP_OK;
+}
+
+int buddy_hip_session_prefill(buddy_hip_session *hs, const int *tokens,
+                              int n_tokens, int start_pos, float *logits_out,
+                              int *next_token) {
+  Session *s = reinterpret_cast<Session *>(hs);
+  BH_REQUIRE(s && tokens, "session_prefill: null argument");
+  int rc = s->ready();
+  if (rc)
+    return rc;
+  const auto &S = s->shape;
+  BH_REQUIRE(n_tokens > 0 && start_pos >= 0 && start_pos + n_tokens <= S.max_len,
+             "session_prefill: tokens %d..%d outside the cache (max_len %d)",
+             start_pos, start_pos + n_tokens - 1, S.max_len);
+  if ((rc = s->ensure_prefill_buffers(n_tokens)))
+    return rc;
+  BH_CHECK_HIP(hipMemcpyAsync(s->pf_tokens, tokens, sizeof(int) * n_tokens,
+                              hipMemcpyDefault, s->stream));
+  if ((rc = s->enqueue_prefill(n_tokens, start_pos)))
+    return rc;
+  // logits of the last prompt token only: RMSNorm + lm_head as in a decode step
+  {
+    bh::GemvArgs g;
+    g.A = s->pf_x + (size_t)(n_tokens - 1) * S.hidden;
+    g.lda = S.hidden;
+    g.W0 = s->lm.w;
+    g.s0 = s->lm.s;
+    g.norm_w = s->ln_f;
+    g.norm_eps = S.rms_eps;
+    g.norm_inv_k = 1.0f / (float)S.hidden;
+    g.C = s->logits;
+    g.ldc = S.vocab;
+    g.M = 1;
+    g.K = S.hidden;
+    g.N = S.vocab;
+    g.epilogue = bh::kEpiStore;
+    if ((rc = bh::launch_gemv(g, s->stream)))
+      return rc;
+  }
+  if ((rc = bh::launch_argmax(s->logits, S.vocab, s->amax_ws, s->state, nullptr,
+                              nullptr, s->stream)))
+    return rc;
+  if (logits_out)
+    BH_CHECK_HIP(hipMemcpyAsync(logits_out, s->logits, sizeof(float) * S.vocab,
+                                hipMemcpyDefault, s->stream));
+  BH_CHECK_HIP(hipMemcpyAsync(s->host_state, s->state, sizeof(int),
+                              hipMemcpyDeviceToHost, s->stream));
+  BH_CHECK_HIP(hipStreamSynchronize(s->stream));
+  if (next_token)
+    *next_token = s->host_state[0];
+  return BUDDY_HIP_OK;
+}
+
+int buddy_hip_session_set_prefill_precision(buddy_hip_session *hs, int exact) {
+  Session *s = reinterpret_cast<Session *>(hs);
+  BH_REQUIRE(s, "session_set_prefill_precision: null session");
+  s->gemm_terms = exact ? 3 : 1;
   return BUDDY_HIP_OK;
 }
 

@@ -133,6 +133,21 @@ class DecoderSession:
             self._h, first_token, start_pos, steps, out.ctypes.data), "decode_greedy")
         return out
 
+    def prefill(self, tokens, start_pos: int = 0, want_logits: bool = True,
+                exact: bool = False):
+        """ModelSession::prefill: the prompt as one block.  Returns (greedy next
+        token, logits of the last prompt token)."""
+        toks = np.ascontiguousarray(tokens, np.int32)
+        check(self._lib.buddy_hip_session_set_prefill_precision(self._h, int(exact)),
+              "set_prefill_precision")
+        logits = np.empty(self.shape.vocab, np.float32) if want_logits else None
+        nxt = c_int(-1)
+        check(self._lib.buddy_hip_session_prefill(
+            self._h, toks.ctypes.data, toks.size, start_pos,
+            None if logits is None else logits.ctypes.data, ctypes.byref(nxt)),
+            "session_prefill")
+        return nxt.value, logits
+
     def set_state(self, token: int, pos: int):
         check(self._lib.buddy_hip_session_set_state(self._h, token, pos), "set_state")
 

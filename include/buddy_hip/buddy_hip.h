@@ -110,6 +110,19 @@ enum {
 int buddy_hip_linear_w8a32(const buddy_hip_linear_desc *desc,
                            buddy_hip_stream stream);
 
+/* ---- int8 dequant prefill matmul on the matrix cores ----------------------
+ * Replaces the BLIS-style kernel with dequantisation fused into B packing
+ * (midend/lib/Conversion/MatMulOptimization/MatMulBlisVectorization.cpp:351-360,
+ * 398-986): C[M,N] (+)= A[M,K] . (W[K,N] * scale[N]), any M.  `packed` is the
+ * same wave-tile copy the decode kernel reads.  Activations are cast to bf16
+ * (round to nearest even) and multiplied on MFMA with f32 accumulation; with
+ * BUDDY_HIP_GEMM_A_F32_EXACT each activation is carried as three bf16 terms,
+ * i.e. with all 24 significand bits.  BUDDY_HIP_GEMV_ACCUMULATE as above. */
+enum { BUDDY_HIP_GEMM_A_F32_EXACT = 2 };
+int buddy_hip_gemm_w8a32(const float *A, const int8_t *packed, const float *scale,
+                         float *C, int64_t M, int64_t K, int64_t N,
+                         unsigned flags, buddy_hip_stream stream);
+
 /* ---- element-wise pieces of a decoder layer ------------------------------
  * Stand-alone forms of what the decode step runs fused; constants and op order
  * from examples/BuddyDeepSeekR1/subgraph0_decode_simplify.mlir:51-72,88-107,
@@ -141,6 +154,18 @@ int buddy_hip_gqa_decode_attention(const float *qkv, const float *inv_freq,
                                    int head_dim, int max_len, float scale,
                                    void *workspace, size_t workspace_bytes,
                                    buddy_hip_stream stream);
+
+/* ---- prefill attention ----------------------------------------------------
+ * Replaces flash_attention_for_cpu_prefill_op
+ * (frontend/Python/ops/tosa.py:4326-4810).  q, out: [heads, q_len, head_dim];
+ * k, v: [kv_heads, k_len, head_dim] (the reference passes K/V repeated to
+ * kv_heads == heads; fewer KV heads are read in place).  mask: additive f32
+ * [q_len, k_len], or NULL for the causal mask in which query i sees keys
+ * 0 .. k_len - q_len + i.  head_dim must be 128. */
+int buddy_hip_prefill_attention(const float *q, const float *k, const float *v,
+                                const float *mask, float *out, int heads,
+                                int kv_heads, int head_dim, int q_len, int k_len,
+                                float scale, buddy_hip_stream stream);
 
 /* ---- plain f32 matmul ---------------------------------------------------
  * C (+)= A[M,K] * B[K,N], all dense row-major device pointers.  The f32
@@ -209,6 +234,17 @@ int buddy_hip_session_decode(buddy_hip_session *s, int token, int pos,
  * step i.  Synchronous. */
 int buddy_hip_session_decode_greedy(buddy_hip_session *s, int first_token,
                                     int start_pos, int steps, int *tokens_out);
+/* Prompt processing (ModelSession::prefill, gen_session.py:1345-1369): runs
+ * n_tokens tokens (host or device int array) through the decoder as one block,
+ * filling cache rows start_pos .. start_pos + n_tokens - 1, on the MFMA matmul
+ * and the causal attention kernel.  logits_out (vocab floats) and next_token
+ * are for the LAST prompt token, the only row the decode loop reads
+ * (runtime/llm/TextGeneration.cpp:191-194).  Synchronous. */
+int buddy_hip_session_prefill(buddy_hip_session *s, const int *tokens,
+                              int n_tokens, int start_pos, float *logits_out,
+                              int *next_token);
+/* 0 (default): prefill activations are cast to bf16; 1: carried exactly. */
+int buddy_hip_session_set_prefill_precision(buddy_hip_session *s, int exact);
 /* Asynchronous pieces of the call above, for timing: set the device-side
  * (token, position), then enqueue steps on the session stream. */
 int buddy_hip_session_set_state(buddy_hip_session *s, int token, int pos);

@@ -1,0 +1,135 @@
+"""GPU parity of the prefill path: the MFMA int8 dequant matmul against the
+oracle's BLIS restatement, the causal GQA attention against the oracle's
+flash-attention restatement, and block prefill of the resident session against
+token-by-token decode steps of the oracle."""
+import numpy as np
+import pytest
+import torch
+
+import buddy_mlir_amd as bma
+from buddy_mlir_amd import ops, synthetic
+from buddy_mlir_amd.session import Shape
+from parity import check_close
+from test_gpu_decode import SMALL, oracle_model
+
+pytestmark = pytest.mark.gpu
+
+SCALE = np.float32(0.0883883461)
+
+
+def bf16_round(a: np.ndarray) -> np.ndarray:
+    return torch.from_numpy(a).to(torch.bfloat16).to(torch.float32).numpy()
+
+
+GEMM_SHAPES = [(512, 1536, 1536), (512, 1536, 256), (512, 1536, 8960), (512, 8960, 1536),
+               (9, 4, 17), (65, 129, 257), (1, 64, 16), (130, 200, 130)]
+
+
+@pytest.mark.parametrize("M,K,N", GEMM_SHAPES)
+@pytest.mark.parametrize("exact", [False, True])
+def test_prefill_gemm_matches_blis_oracle(oracle, M, K, N, exact):
+    q, s = synthetic.quantized_linear(K, N, M + K + N)
+    packed = ops.pack_w8(q)
+    g = torch.Generator(device="cuda").manual_seed(M)
+    x = torch.randn((M, K), generator=g, device="cuda")
+    y = ops.gemm_w8a32(x, packed, s, K, N, exact=exact)
+    torch.cuda.synchronize()
+    xh = x.cpu().numpy()
+    # "activations cast to bf16": the oracle gets the same rounded activations
+    a_in = xh if exact else bf16_round(xh)
+    want = oracle.blis_gemm_w8a32(a_in, q.cpu().numpy(), s.cpu().numpy())
+    check_close(y.cpu().numpy(), want)
+
+
+def test_prefill_gemm_accumulates(oracle):
+    M, K, N = 100, 256, 96
+    q, s = synthetic.quantized_linear(K, N, 77)
+    g = torch.Generator(device="cuda").manual_seed(1)
+    x = torch.randn((M, K), generator=g, device="cuda")
+    c0 = torch.randn((M, N), generator=g, device="cuda")
+    c = c0.clone()
+    ops.gemm_w8a32(x, ops.pack_w8(q), s, K, N, out=c, accumulate=True, exact=True)
+    torch.cuda.synchronize()
+    want = oracle.blis_gemm_w8a32(x.cpu().numpy(), q.cpu().numpy(), s.cpu().numpy(),
+                                  c0.cpu().numpy())
+    check_close(c.cpu().numpy(), want)
+
+
+def run_attn(bh, q, k, v, mask, heads, kv_heads, Lq, Lk):
+    out = torch.empty_like(q)
+    torch.cuda.synchronize()
+    bma.check(bh.buddy_hip_prefill_attention(
+        q.data_ptr(), k.data_ptr(), v.data_ptr(), None if mask is None else mask.data_ptr(),
+        out.data_ptr(), heads, kv_heads, 128, Lq, Lk, float(SCALE), None))
+    torch.cuda.synchronize()
+    return out.cpu().numpy()
+
+
+@pytest.mark.parametrize("L", [16, 40, 512])
+def test_prefill_attention_reference_shape(bh, oracle, L):
+    """q, k, v all [12, L, 128] with an additive causal mask, the call shape of
+    flash_attention_for_cpu_prefill_op; also the implicit causal mask."""
+    H = 12
+    g = torch.Generator(device="cuda").manual_seed(L)
+    q, k, v = (torch.randn((H, L, 128), generator=g, device="cuda") for _ in range(3))
+    mh = np.where(np.tril(np.ones((L, L), bool)), 0.0, -np.inf).astype(np.float32)
+    want = oracle.prefill_flash_attention(q.cpu().numpy(), k.cpu().numpy(), v.cpu().numpy(),
+                                          mh, SCALE)
+    got_mask = run_attn(bh, q, k, v, torch.from_numpy(mh).cuda(), H, H, L, L)
+    got_causal = run_attn(bh, q, k, v, None, H, H, L, L)
+    check_close(got_mask, want)
+    check_close(got_causal, want)
+
+
+def test_prefill_attention_gqa_and_longer_keys(bh, oracle):
+    """2 KV heads read in place = 12 repeated heads; 37 queries over 100 keys
+    (a prompt continuing after 63 cached positions)."""
+    H, HKV, Lq, Lk = 12, 2, 37, 100
+    g = torch.Generator(device="cuda").manual_seed(5)
+    q = torch.randn((H, Lq, 128), generator=g, device="cuda")
+    k = torch.randn((HKV, Lk, 128), generator=g, device="cuda")
+    v = torch.randn((HKV, Lk, 128), generator=g, device="cuda")
+    kk = k.repeat_interleave(H // HKV, dim=0).cpu().numpy()
+    vv = v.repeat_interleave(H // HKV, dim=0).cpu().numpy()
+    qi = np.arange(Lq)[:, None] + (Lk - Lq)
+    mh = np.where(np.arange(Lk)[None, :] <= qi, 0.0, -np.inf).astype(np.float32)
+    want = oracle.prefill_flash_attention(q.cpu().numpy(), kk, vv, mh, SCALE)
+    check_close(run_attn(bh, q, k, v, None, H, HKV, Lq, Lk), want)
+
+
+@pytest.mark.parametrize("exact", [True, False])
+def test_small_model_block_prefill_equals_token_by_token(oracle, exact):
+    """Prefill of 40 prompt tokens as one block against 40 oracle decode steps:
+    last-token logits, greedy token and every cache row written; then decode
+    continues from the prefilled cache."""
+    sess, host = synthetic.build_session(SMALL, context=0, keep_host=True, ln_jitter=0.1)
+    om = oracle_model(oracle, SMALL, host)
+    kv = [a.copy() for a in host["kv"]]
+    toks = synthetic.first_tokens(SMALL, 40, seed=3).tolist()
+    for pos, t in enumerate(toks):
+        otok, ologits = om.decode_step(t, pos, kv)
+    nxt, logits = sess.prefill(toks, 0, exact=exact)
+    if exact:
+        check_close(logits, ologits)
+        assert nxt == otok
+        for j in range(2 * SMALL.layers):
+            check_close(sess.get_kv(j)[:, :40, :], kv[j][:, :40, :])
+        # decoding on from the prefilled cache
+        tok = otok
+        for step in range(6):
+            n2, lg = sess.decode(tok, 40 + step)
+            tok, olg = om.decode_step(tok, 40 + step, kv)
+            check_close(lg, olg)
+            assert n2 == tok
+    else:
+        # activations cast to bf16 in every matmul of every layer: compared at
+        # the looser bound that rounding allows
+        check_close(logits, ologits, rtol=5e-2, atol_frac=2e-2, normwise=2e-2)
+    sess.close()
+
+
+def test_session_prefill_refuses_overflow(bh):
+    sess, _ = synthetic.build_session(SMALL, context=0)
+    with pytest.raises(bma.BuddyHipError):
+        sess.prefill(list(range(10)), SMALL.max_len - 5)
+    sess.close()
