@@ -113,10 +113,19 @@ def _declare(lib):
         "buddy_hip_session_decode_greedy": (c_int, [vp, c_int, c_int, c_int, vp]),
         "buddy_hip_session_prefill": (c_int, [vp, vp, c_int, c_int, vp, vp]),
         "buddy_hip_session_set_prefill_precision": (c_int, [vp, c_int]),
+        "buddy_hip_session_prefill_all_logits": (c_int, [vp, vp, c_int, c_int, vp]),
+        "buddy_hip_session_adopt": (None, [vp, vp]),
+        "buddy_hip_w8a32_blob_sizes": (None, [vp, vp, vp]),
+        "buddy_hip_session_create_from_w8a32_blobs": (vp, [vp, vp, i64, vp, i64]),
+        "_mlir_ciface_forward_prefill": (None, [vp, vp, vp, vp]),
+        "_mlir_ciface_forward_decode": (None, [vp] * 88),
+        "buddy_hip_forward_reset": (None, []),
+        "buddy_hip_forward_invalidate_kv": (None, []),
         "buddy_hip_session_set_state": (c_int, [vp, c_int, c_int]),
         "buddy_hip_session_enqueue_steps": (c_int, [vp, c_int]),
         "buddy_hip_session_logits": (vp, [vp]),
         "buddy_hip_session_stream": (vp, [vp]),
+        "buddy_hip_gemv_f32": (c_int, [vp, vp, vp, vp, i64, i64, c_uint, vp]),
         "buddy_hip_matmul_f32": (c_int, [vp, vp, vp, i64, i64, i64, c_uint, vp]),
         "_mlir_ciface_buddy_matmul_f32": (None, [vp, vp, vp]),
         "_mlir_ciface_buddy_dequant_matmul_i8_f32": (None, [vp, vp, vp, vp]),

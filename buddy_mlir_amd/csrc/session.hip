@@ -28,6 +28,17 @@
 #include <vector>
 
 namespace bh {
+
+// defined in gemv_f32.hip / matmul_f32.hip
+int launch_gemv_f32(const float *x, const float *B, const float *bias, float *y,
+                    int64_t K, int64_t N, int64_t ldb, bool accumulate,
+                    hipStream_t stream);
+int launch_bias_rows(float *C, const float *bias, int64_t M, int64_t N,
+                     hipStream_t stream);
+int launch_matmul_f32(const float *A, const float *B, float *C, int64_t M,
+                      int64_t N, int64_t K, int64_t lda, int64_t ldb,
+                      int64_t ldc, bool accumulate, hipStream_t stream);
+
 namespace {
 
 struct PackedLinear {
@@ -40,6 +51,9 @@ struct PackedLinear {
 struct Layer {
   float *ln1 = nullptr, *ln2 = nullptr;
   PackedLinear qkv, o, gate, up, down;
+  // the reference's shipped w8a32 build keeps q/k/v in f32 with a bias
+  // (they import as AddMMOp, which the quantizer does not touch):
+  float *qkv_f32 = nullptr; // [hidden, q|k|v] dense, or null when int8
   float *kc = nullptr, *vc = nullptr; // [kv_heads, max_len, D]
   bool set = false;
 };
@@ -76,8 +90,8 @@ struct Session {
   float *ln_f = nullptr, *inv_freq = nullptr;
   PackedLinear lm;
   // activations
-  float *x = nullptr, *qkv = nullptr, *att = nullptr, *h = nullptr,
-        *logits = nullptr;
+  float *x = nullptr, *xn = nullptr, *qkv = nullptr, *att = nullptr,
+        *h = nullptr, *logits = nullptr;
   void *attn_ws = nullptr, *amax_ws = nullptr;
   size_t attn_ws_bytes = 0;
   int *state = nullptr;     // device: token, pos, step
@@ -93,7 +107,7 @@ struct Session {
   float *pf_x = nullptr, *pf_xn = nullptr, *pf_qkv = nullptr, *pf_att = nullptr,
         *pf_g = nullptr, *pf_u = nullptr;
   int *pf_tokens = nullptr;
-  int gemm_terms = 1; // bf16 terms per activation in the prefill matmuls
+  int gemm_terms = 3; // bf16 terms per activation in the prefill matmuls (3 = exact)
 
   template <typename T> int alloc(T **p, size_t n) {
     void *q = nullptr;
@@ -172,8 +186,15 @@ struct Session {
     const float scale = (float)(1.0 / std::sqrt((double)S.head_dim));
     for (int i = 0; i < S.layers; ++i) {
       Layer &L = layers[(size_t)i];
-      if ((rc = gemv(x, L.qkv, nullptr, L.ln1, qkv, kEpiStore)))
+      if (L.qkv_f32) {
+        if ((rc = launch_rmsnorm(x, L.ln1, xn, 1, S.hidden, S.rms_eps, stream)))
+          return rc;
+        if ((rc = launch_gemv_f32(xn, L.qkv_f32, L.qkv.b, qkv, L.qkv.K, L.qkv.N,
+                                  L.qkv.N, false, stream)))
+          return rc;
+      } else if ((rc = gemv(x, L.qkv, nullptr, L.ln1, qkv, kEpiStore))) {
         return rc;
+      }
       AttnDecodeArgs a;
       a.qkv = qkv;
       a.inv_freq = inv_freq;
@@ -283,8 +304,15 @@ struct Session {
       Layer &L = layers[(size_t)i];
       if ((rc = launch_rmsnorm(pf_x, L.ln1, pf_xn, n, S.hidden, S.rms_eps, stream)))
         return rc;
-      if ((rc = gemm(pf_xn, L.qkv, pf_qkv, n, false)))
+      if (L.qkv_f32) {
+        if ((rc = launch_bias_rows(pf_qkv, L.qkv.b, n, L.qkv.N, stream)))
+          return rc;
+        if ((rc = launch_matmul_f32(pf_xn, L.qkv_f32, pf_qkv, n, L.qkv.N, L.qkv.K,
+                                    L.qkv.K, L.qkv.N, L.qkv.N, true, stream)))
+          return rc;
+      } else if ((rc = gemm(pf_xn, L.qkv, pf_qkv, n, false))) {
         return rc;
+      }
       if ((rc = launch_rope_kv_write(pf_qkv, QKV, inv_freq, L.kc, L.vc, S.heads,
                                      S.kv_heads, S.head_dim, S.max_len, start_pos,
                                      n, stream)))
@@ -404,6 +432,7 @@ buddy_hip_session *buddy_hip_session_create(const buddy_hip_model_shape *shape,
   const size_t QN = (size_t)S.heads * S.head_dim, KVN = (size_t)S.kv_heads * S.head_dim;
   int rc = 0;
   rc |= s->alloc(&s->x, (size_t)S.hidden);
+  rc |= s->alloc(&s->xn, (size_t)S.hidden);
   rc |= s->alloc(&s->qkv, QN + 2 * KVN);
   rc |= s->alloc(&s->att, QN);
   rc |= s->alloc(&s->h, (size_t)S.inter);
@@ -493,10 +522,15 @@ int buddy_hip_session_set_layer(buddy_hip_session *hs, int index,
   BH_REQUIRE(s && w, "session_set_layer: null argument");
   const auto &S = s->shape;
   BH_REQUIRE(index >= 0 && index < S.layers, "session_set_layer: index %d", index);
-  BH_REQUIRE(w->ln1 && w->ln2 && w->wq && w->wk && w->wv && w->wo && w->wg &&
-                 w->wu && w->wd && w->sq && w->sk && w->sv && w->so && w->sg &&
-                 w->su && w->sd,
+  const bool f32_qkv = w->fq != nullptr;
+  BH_REQUIRE(w->ln1 && w->ln2 && w->wo && w->wg && w->wu && w->wd && w->so &&
+                 w->sg && w->su && w->sd,
              "session_set_layer: null weight");
+  BH_REQUIRE(f32_qkv ? (w->fk && w->fv && w->bq && !w->wq && !w->wk && !w->wv)
+                     : (w->wq && w->wk && w->wv && w->sq && w->sk && w->sv &&
+                        !w->fk && !w->fv),
+             "session_set_layer: q/k/v must be all int8 (+scales) or all f32 "
+             "(+biases)");
   BH_REQUIRE((w->bq != nullptr) == (w->bk != nullptr) &&
                  (w->bq != nullptr) == (w->bv != nullptr),
              "session_set_layer: q/k/v biases must come together");
@@ -509,8 +543,12 @@ int buddy_hip_session_set_layer(buddy_hip_session *hs, int index,
     // three packed blocks simply follow each other
     L.qkv.K = H;
     L.qkv.N = QN + 2 * KVN;
-    rc |= s->alloc(&L.qkv.w, buddy_hip_w8_packed_bytes(H, L.qkv.N));
-    rc |= s->alloc(&L.qkv.s, (size_t)L.qkv.N);
+    if (f32_qkv) {
+      rc |= s->alloc(&L.qkv_f32, (size_t)H * L.qkv.N);
+    } else {
+      rc |= s->alloc(&L.qkv.w, buddy_hip_w8_packed_bytes(H, L.qkv.N));
+      rc |= s->alloc(&L.qkv.s, (size_t)L.qkv.N);
+    }
     if (w->bq)
       rc |= s->alloc(&L.qkv.b, (size_t)L.qkv.N);
     L.o.K = QN; L.o.N = H;
@@ -526,11 +564,27 @@ int buddy_hip_session_set_layer(buddy_hip_session *hs, int index,
   }
   BH_REQUIRE(QN % 16 == 0 && KVN % 16 == 0, "session_set_layer: head sizes");
   const size_t kp = (size_t)bh::round_up(H, bh::kTileK);
-  rc |= s->pack_into(w->wq, w->sq, w->bq, H, QN, L.qkv.w, L.qkv.s, L.qkv.b);
-  rc |= s->pack_into(w->wk, w->sk, w->bk, H, KVN, L.qkv.w + kp * QN,
-                     L.qkv.s + QN, L.qkv.b ? L.qkv.b + QN : nullptr);
-  rc |= s->pack_into(w->wv, w->sv, w->bv, H, KVN, L.qkv.w + kp * (QN + KVN),
-                     L.qkv.s + QN + KVN, L.qkv.b ? L.qkv.b + QN + KVN : nullptr);
+  BH_REQUIRE(f32_qkv == (L.qkv_f32 != nullptr),
+             "session_set_layer: layer %d was created with the other q/k/v type", index);
+  if (f32_qkv) {
+    // [H, QN] | [H, KVN] | [H, KVN] side by side in one [H, QN + 2 KVN] matrix
+    const size_t ld = (size_t)L.qkv.N * sizeof(float);
+    BH_CHECK_HIP(hipMemcpy2DAsync(L.qkv_f32, ld, w->fq, QN * sizeof(float),
+                                  QN * sizeof(float), H, hipMemcpyDefault, s->stream));
+    BH_CHECK_HIP(hipMemcpy2DAsync(L.qkv_f32 + QN, ld, w->fk, KVN * sizeof(float),
+                                  KVN * sizeof(float), H, hipMemcpyDefault, s->stream));
+    BH_CHECK_HIP(hipMemcpy2DAsync(L.qkv_f32 + QN + KVN, ld, w->fv, KVN * sizeof(float),
+                                  KVN * sizeof(float), H, hipMemcpyDefault, s->stream));
+    BH_CHECK_HIP(hipMemcpyAsync(L.qkv.b, w->bq, QN * sizeof(float), hipMemcpyDefault, s->stream));
+    BH_CHECK_HIP(hipMemcpyAsync(L.qkv.b + QN, w->bk, KVN * sizeof(float), hipMemcpyDefault, s->stream));
+    BH_CHECK_HIP(hipMemcpyAsync(L.qkv.b + QN + KVN, w->bv, KVN * sizeof(float), hipMemcpyDefault, s->stream));
+  } else {
+    rc |= s->pack_into(w->wq, w->sq, w->bq, H, QN, L.qkv.w, L.qkv.s, L.qkv.b);
+    rc |= s->pack_into(w->wk, w->sk, w->bk, H, KVN, L.qkv.w + kp * QN,
+                       L.qkv.s + QN, L.qkv.b ? L.qkv.b + QN : nullptr);
+    rc |= s->pack_into(w->wv, w->sv, w->bv, H, KVN, L.qkv.w + kp * (QN + KVN),
+                       L.qkv.s + QN + KVN, L.qkv.b ? L.qkv.b + QN + KVN : nullptr);
+  }
   rc |= s->pack_into(w->wo, w->so, nullptr, QN, H, L.o.w, L.o.s, nullptr);
   rc |= s->pack_into(w->wg, w->sg, nullptr, H, I, L.gate.w, L.gate.s, nullptr);
   rc |= s->pack_into(w->wu, w->su, nullptr, H, I, L.up.w, L.up.s, nullptr);
@@ -683,6 +737,44 @@ int buddy_hip_session_prefill(buddy_hip_session *hs, const int *tokens,
   if (next_token)
     *next_token = s->host_state[0];
   return BUDDY_HIP_OK;
+}
+
+int buddy_hip_session_prefill_all_logits(buddy_hip_session *hs, const int *tokens,
+                                         int n_tokens, int start_pos,
+                                         float *logits_out) {
+  Session *s = reinterpret_cast<Session *>(hs);
+  BH_REQUIRE(s && tokens && logits_out, "session_prefill_all_logits: null argument");
+  int rc = s->ready();
+  if (rc)
+    return rc;
+  const auto &S = s->shape;
+  BH_REQUIRE(n_tokens > 0 && start_pos >= 0 && start_pos + n_tokens <= S.max_len,
+             "session_prefill_all_logits: tokens %d..%d outside the cache (max_len %d)",
+             start_pos, start_pos + n_tokens - 1, S.max_len);
+  if ((rc = s->ensure_prefill_buffers(n_tokens)))
+    return rc;
+  BH_CHECK_HIP(hipMemcpyAsync(s->pf_tokens, tokens, sizeof(int) * n_tokens,
+                              hipMemcpyDefault, s->stream));
+  if ((rc = s->enqueue_prefill(n_tokens, start_pos)))
+    return rc;
+  if ((rc = bh::launch_rmsnorm(s->pf_x, s->ln_f, s->pf_xn, n_tokens, S.hidden,
+                               S.rms_eps, s->stream)))
+    return rc;
+  float *dev_logits = nullptr;
+  BH_CHECK_HIP(hipMalloc((void **)&dev_logits, sizeof(float) * (size_t)n_tokens * S.vocab));
+  rc = s->gemm(s->pf_xn, s->lm, dev_logits, n_tokens, false);
+  if (!rc && hipMemcpyAsync(logits_out, dev_logits, sizeof(float) * (size_t)n_tokens * S.vocab,
+                            hipMemcpyDefault, s->stream) != hipSuccess)
+    rc = bh::fail(BUDDY_HIP_ERR_HIP, "session_prefill_all_logits: copy failed");
+  (void)hipStreamSynchronize(s->stream);
+  (void)hipFree(dev_logits);
+  return rc;
+}
+
+void buddy_hip_session_adopt(buddy_hip_session *hs, void *device_ptr) {
+  Session *s = reinterpret_cast<Session *>(hs);
+  if (s && device_ptr)
+    s->owned.push_back(device_ptr);
 }
 
 int buddy_hip_session_set_prefill_precision(buddy_hip_session *hs, int exact) {

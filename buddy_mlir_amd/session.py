@@ -25,7 +25,8 @@ class ModelShape(Structure):
 class LayerWeights(Structure):
     _fields_ = [(n, c_void_p) for n in
                 ("ln1", "ln2", "wq", "wk", "wv", "wo", "wg", "wu", "wd",
-                 "sq", "sk", "sv", "so", "sg", "su", "sd", "bq", "bk", "bv")]
+                 "sq", "sk", "sv", "so", "sg", "su", "sd", "bq", "bk", "bv",
+                 "fq", "fk", "fv")]
 
 
 @dataclass
@@ -134,7 +135,7 @@ class DecoderSession:
         return out
 
     def prefill(self, tokens, start_pos: int = 0, want_logits: bool = True,
-                exact: bool = False):
+                exact: bool = True):
         """ModelSession::prefill: the prompt as one block.  Returns (greedy next
         token, logits of the last prompt token)."""
         toks = np.ascontiguousarray(tokens, np.int32)

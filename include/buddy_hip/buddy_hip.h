@@ -200,6 +200,10 @@ typedef struct buddy_hip_layer_weights {
   const int8_t *wq, *wk, *wv, *wo, *wg, *wu, *wd;
   const float *sq, *sk, *sv, *so, *sg, *su, *sd;
   const float *bq, *bk, *bv;
+  /* q/k/v kept in f32 [K,N], as in the reference's shipped w8a32 build where
+   * they import as AddMMOp and are not quantized (docs/DecodeWeightPacking.md:
+   * 128-131): set all three plus the biases and leave wq/wk/wv/sq/sk/sv NULL. */
+  const float *fq, *fk, *fv;
 } buddy_hip_layer_weights;
 
 typedef struct buddy_hip_session buddy_hip_session;
@@ -243,7 +247,15 @@ int buddy_hip_session_decode_greedy(buddy_hip_session *s, int first_token,
 int buddy_hip_session_prefill(buddy_hip_session *s, const int *tokens,
                               int n_tokens, int start_pos, float *logits_out,
                               int *next_token);
-/* 0 (default): prefill activations are cast to bf16; 1: carried exactly. */
+/* The same with the logits of every row, [n_tokens, vocab] (host or device):
+ * what the compiled forward_prefill returns (PrefillABI, gen_session.py:908-911). */
+int buddy_hip_session_prefill_all_logits(buddy_hip_session *s, const int *tokens,
+                                         int n_tokens, int start_pos,
+                                         float *logits_out);
+/* Hands a device allocation to the session, which frees it when destroyed. */
+void buddy_hip_session_adopt(buddy_hip_session *s, void *device_ptr);
+/* 1 (default): prefill activations keep all f32 bits (three bf16 terms);
+ * 0: they are cast to bf16, one MFMA pass instead of three. */
 int buddy_hip_session_set_prefill_precision(buddy_hip_session *s, int exact);
 /* Asynchronous pieces of the call above, for timing: set the device-side
  * (token, position), then enqueue steps on the session stream. */
@@ -251,6 +263,65 @@ int buddy_hip_session_set_state(buddy_hip_session *s, int token, int pos);
 int buddy_hip_session_enqueue_steps(buddy_hip_session *s, int steps);
 const float *buddy_hip_session_logits(buddy_hip_session *s); /* device */
 buddy_hip_stream buddy_hip_session_stream(buddy_hip_session *s);
+
+/* y[N] = bias[N] + x[K] . B[K,N] in f32 (bias may be NULL): the decode GEMV
+ * of MatMulVectorizationDecode.cpp:142-175 followed by the q/k/v bias add. */
+int buddy_hip_gemv_f32(const float *x, const float *B, const float *bias,
+                       float *y, int64_t K, int64_t N, unsigned flags,
+                       buddy_hip_stream stream);
+
+/* ---- the reference's w8a32 weight package ---------------------------------
+ * Builds a session from the two flat blobs the reference's importer writes for
+ * the w8a32 variant (arg0-w8a32-f32.data, arg0-w8a32-i8.data;
+ * tools/buddy-codegen/gen_config.py:55-58).  Parameter order inside the blobs
+ * (argument list of examples/BuddyDeepSeekR1/subgraph0_decode_simplify.mlir:4,
+ * split by dtype, scalers appended in weight order --
+ * frontend/Python/graph/transform/quantization/quantize.py:561-590):
+ *   f32: embed[V,H], inv_freq[D/2], per layer { ln1[H], q_bias, q_w[H,QN],
+ *        k_bias, k_w[H,KVN], v_bias, v_w[H,KVN], ln2[H] }, ln_f[H],
+ *        per layer { s_o[H], s_gate[I], s_up[I], s_down[H] }, s_lm[V]
+ *   i8 : per layer { o_w[QN,H], gate[H,I], up[H,I], down[I,H] }, lm_head[H,V]
+ * For the Qwen2-1.5B shape these counts equal the reference's F32ParamsSize =
+ * 322338752 and I8ParamsSize = 1455489024
+ * (examples/BuddyDeepSeekR1/buddy-deepseek-r1-w8a32-main.cpp:32-33).
+ * Blobs may be host or device memory and are not referenced after the call. */
+void buddy_hip_w8a32_blob_sizes(const buddy_hip_model_shape *shape, int64_t *n_f32,
+                                int64_t *n_i8);
+buddy_hip_session *buddy_hip_session_create_from_w8a32_blobs(
+    const buddy_hip_model_shape *shape, const float *f32_params, int64_t n_f32,
+    const int8_t *i8_params, int64_t n_i8);
+
+/* ---- model-level memref entry points ---------------------------------------
+ * The two symbols the generated ModelSession resolves with dlsym
+ * (tools/buddy-codegen/gen_session.py:1127-1143) with the argument lists of
+ * PrefillFn / DecodeFn (gen_session.py:974-1007) for the 28-layer
+ * DeepSeek-R1-Distill-Qwen-1.5B w8a32 package: result block, f32 blob, int8
+ * blob, then tokens [1,max_len] (prefill) or token [1,1], cache_position [1],
+ * kv0, kv1 and 27 x (position copy, k, v) (decode).  `result` is the
+ * PrefillABI / DecodeABI block (gen_session.py:908-932).  Decode results alias
+ * the caller's KV and position buffers and hand over a malloc'd [1,1,vocab]
+ * logits buffer; prefill hands over malloc'd KV tensors and [1,max_len,vocab]
+ * logits.  The device session is built on the first call and reused while the
+ * blob addresses stay the same.  The KV cache is uploaded from the caller's
+ * tensors on the first decode that no prefill preceded; call
+ * buddy_hip_forward_invalidate_kv() after editing the host cache. */
+void _mlir_ciface_forward_prefill(void *result, buddy_memref_f32_1d *f32_params,
+                                  buddy_memref_i8_1d *i8_params,
+                                  buddy_memref_i64_2d *tokens);
+#define BUDDY_HIP_KV_(n) , buddy_memref_f32_4d *k##n, buddy_memref_f32_4d *v##n
+#define BUDDY_HIP_DKV_(n) , buddy_memref_i64_1d *d##n BUDDY_HIP_KV_(n)
+void _mlir_ciface_forward_decode(
+    void *result, buddy_memref_f32_1d *f32_params, buddy_memref_i8_1d *i8_params,
+    buddy_memref_i64_2d *token, buddy_memref_i64_1d *cache_position BUDDY_HIP_KV_(0)
+    BUDDY_HIP_DKV_(1) BUDDY_HIP_DKV_(2) BUDDY_HIP_DKV_(3) BUDDY_HIP_DKV_(4)
+    BUDDY_HIP_DKV_(5) BUDDY_HIP_DKV_(6) BUDDY_HIP_DKV_(7) BUDDY_HIP_DKV_(8)
+    BUDDY_HIP_DKV_(9) BUDDY_HIP_DKV_(10) BUDDY_HIP_DKV_(11) BUDDY_HIP_DKV_(12)
+    BUDDY_HIP_DKV_(13) BUDDY_HIP_DKV_(14) BUDDY_HIP_DKV_(15) BUDDY_HIP_DKV_(16)
+    BUDDY_HIP_DKV_(17) BUDDY_HIP_DKV_(18) BUDDY_HIP_DKV_(19) BUDDY_HIP_DKV_(20)
+    BUDDY_HIP_DKV_(21) BUDDY_HIP_DKV_(22) BUDDY_HIP_DKV_(23) BUDDY_HIP_DKV_(24)
+    BUDDY_HIP_DKV_(25) BUDDY_HIP_DKV_(26) BUDDY_HIP_DKV_(27));
+void buddy_hip_forward_reset(void);         /* drops the cached device session */
+void buddy_hip_forward_invalidate_kv(void); /* next decode re-uploads the KV cache */
 
 /* ---- operator-level memref entry points --------------------------------
  * result = A * B, f32.  Same symbol and contract as

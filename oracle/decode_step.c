@@ -19,6 +19,18 @@ static void linear(const float *x, const int8_t *W, const float *s,
       y[n] = bias[n] + y[n];
 }
 
+/* q/k/v of the shipped w8a32 build: f32 weights through the plain decode GEMV
+ * (MatMulVectorizationDecode.cpp:142-175) into a zero tensor, then bias + y
+ * (subgraph0_decode_simplify.mlir:73-85). */
+static void linear_f32(const float *x, const float *W, const float *bias, float *y,
+                       int64_t K, int64_t N) {
+  memset(y, 0, sizeof(float) * (size_t)N);
+  oracle_gemv_f32(x, W, y, K, N, 32, 0);
+  if (bias)
+    for (int64_t n = 0; n < N; ++n)
+      y[n] = bias[n] + y[n];
+}
+
 int64_t oracle_decode_step(const oracle_model *m, int64_t token, int64_t pos,
                            float **kv, float *logits) {
   const oracle_shape *S = &m->shape;
@@ -50,9 +62,15 @@ int64_t oracle_decode_step(const oracle_model *m, int64_t token, int64_t pos,
     const oracle_layer *W = &m->layer[L];
     float *Kc = kv[2 * L], *Vc = kv[2 * L + 1];
     oracle_rmsnorm(x, W->ln1, xn, H, inv_h, S->eps);
-    linear(xn, W->wq, W->sq, W->bq, q, H, QN);
-    linear(xn, W->wk, W->sk, W->bk, k, H, KVN);
-    linear(xn, W->wv, W->sv, W->bv, v, H, KVN);
+    if (W->wq) {
+      linear(xn, W->wq, W->sq, W->bq, q, H, QN);
+      linear(xn, W->wk, W->sk, W->bk, k, H, KVN);
+      linear(xn, W->wv, W->sv, W->bv, v, H, KVN);
+    } else {
+      linear_f32(xn, W->fq, W->bq, q, H, QN);
+      linear_f32(xn, W->fk, W->bk, k, H, KVN);
+      linear_f32(xn, W->fv, W->bv, v, H, KVN);
+    }
     oracle_rope_apply(q, S->heads, D, cosv, sinv);
     oracle_rope_apply(k, S->kv_heads, D, cosv, sinv);
     /* KV write: cache[0, h, pos, :] = k' / v (:108-142) */

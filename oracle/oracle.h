@@ -134,6 +134,9 @@ typedef struct {
   const float *bq, *bk, *bv;            /* [N] or NULL */
   const int8_t *wg, *wu, *wd;
   const float *sg, *su, *sd;
+  /* q/k/v kept in f32 [K,N] (the reference's shipped w8a32 build): used when
+   * wq is NULL, with the f32 decode GEMV and the bias add */
+  const float *fq, *fk, *fv;
 } oracle_layer;
 
 typedef struct {

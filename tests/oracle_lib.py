@@ -33,7 +33,8 @@ class Shape(Structure):
 class Layer(Structure):
     _fields_ = [(n, c_void_p) for n in
                 ("ln1", "ln2", "wq", "wk", "wv", "wo", "sq", "sk", "sv", "so",
-                 "bq", "bk", "bv", "wg", "wu", "wd", "sg", "su", "sd")]
+                 "bq", "bk", "bv", "wg", "wu", "wd", "sg", "su", "sd",
+                 "fq", "fk", "fv")]
 
 
 class Model(Structure):
