@@ -126,6 +126,11 @@ def _declare(lib):
         "buddy_hip_session_logits": (vp, [vp]),
         "buddy_hip_session_stream": (vp, [vp]),
         "buddy_hip_gemv_f32": (c_int, [vp, vp, vp, vp, i64, i64, c_uint, vp]),
+        "buddy_hip_pack_panels_f32": (c_int, [vp, i64, i64, c_int, vp, vp]),
+        "buddy_hip_unpack_panels_f32": (c_int, [vp, i64, i64, c_int, vp, vp]),
+        "buddy_hip_gemv_f32_panels": (c_int, [vp, vp, vp, i64, i64, c_uint, vp]),
+        "buddy_hip_w8a8_workspace_bytes": (sz, [i64, i64]),
+        "buddy_hip_w8a8_matmul": (c_int, [vp, vp, vp, vp, vp, i64, i64, i64, vp, sz, vp]),
         "buddy_hip_matmul_f32": (c_int, [vp, vp, vp, i64, i64, i64, c_uint, vp]),
         "_mlir_ciface_buddy_matmul_f32": (None, [vp, vp, vp]),
         "_mlir_ciface_buddy_dequant_matmul_i8_f32": (None, [vp, vp, vp, vp]),

@@ -1,0 +1,165 @@
+// gemv_w8a8.hip -- w8a8 matmul: dynamic per-tensor int8 activations times int8
+// weights with exact int32 partial sums.
+//
+// Replaces quantized_matmul_op / _quantize_activation_i8
+// (frontend/Python/ops/linalg.py:12728-12847):
+//   s_a  = max(absmax(x) * (1/127), 1e-10)            (:12737-12760)
+//   x_q  = clamp(f32(i32(x * (1/s_a))), -128, 127)     (:12761-12792; the TOSA
+//          f32 -> i32 cast rounds to nearest even)
+//   acc  = x_q (i8) . W (i8) -> i32                    (:12814-12831)
+//   y    = f32(acc) * (s_a * s_w[n])                   (:12833-12845)
+// The int8 weights are the same wave-tile packed copy the w8a32 kernels read;
+// the dot products run on v_dot4_i32_i8 (four multiply-adds per lane per
+// instruction), so the partial sums are exact integers whatever the order.
+#include "common.h"
+
+namespace bh {
+namespace {
+
+// absmax over the whole activation tensor, one workgroup
+__global__ void __launch_bounds__(1024)
+w8a8_quantize_kernel(const float *__restrict__ x, int64_t n, int M, int K, int Kp,
+                     int8_t *__restrict__ xq, float *__restrict__ scale_out) {
+  __shared__ float red[16];
+  __shared__ float s_inv;
+  float m = 0.f;
+  for (int64_t i = threadIdx.x; i < n; i += 1024)
+    m = fmaxf(m, fabsf(x[i]));
+  m = wave_max(m);
+  if ((threadIdx.x & 63) == 0)
+    red[threadIdx.x >> 6] = m;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    float t = red[0];
+    for (int w = 1; w < 16; ++w)
+      t = fmaxf(t, red[w]);
+    const float r127 = 1.0f / 127.0f;
+    float s = t * r127;
+    s = fmaxf(s, 1e-10f);
+    *scale_out = s;
+    s_inv = 1.0f / s;
+  }
+  __syncthreads();
+  const float inv = s_inv;
+  // rows are padded to Kp (a multiple of 64) with zeros
+  for (int64_t i = threadIdx.x; i < (int64_t)M * Kp; i += 1024) {
+    const int m_ = (int)(i / Kp), k = (int)(i % Kp);
+    float r = 0.f;
+    if (k < K) {
+      r = rintf(x[(int64_t)m_ * K + k] * inv);
+      r = fminf(fmaxf(r, -128.0f), 127.0f);
+    }
+    xq[i] = (int8_t)r;
+  }
+}
+
+template <int M>
+__global__ void __launch_bounds__(256)
+w8a8_gemv_kernel(const int4 *__restrict__ W, const int8_t *__restrict__ xq,
+                 const float *__restrict__ a_scale, const float *__restrict__ wscale,
+                 float *__restrict__ C, int32_t *__restrict__ acc_out, int rows,
+                 int N, int groups, int chunks, int Kp) {
+  // 4 wavefronts split the k range of one channel group
+  __shared__ int red[4][M][16];
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int g = blockIdx.x;
+  const int per = (chunks + 3) / 4;
+  const int t0 = min(wave * per, chunks), t1 = min(t0 + per, chunks);
+  int acc[M];
+#pragma unroll
+  for (int m = 0; m < M; ++m)
+    acc[m] = 0;
+  const int4 *w = W + ((size_t)g * chunks) * 64 + lane;
+  const int kg = lane >> 4;
+  for (int t = t0; t < t1; ++t) {
+    const int4 wv = w[(size_t)t * 64];
+#pragma unroll
+    for (int m = 0; m < M; ++m) {
+      if (m < rows) {
+        const int4 xv = *reinterpret_cast<const int4 *>(xq + (size_t)m * Kp + t * 64 + kg * 16);
+        int a = acc[m];
+        a = __builtin_amdgcn_sdot4(wv.x, xv.x, a, false);
+        a = __builtin_amdgcn_sdot4(wv.y, xv.y, a, false);
+        a = __builtin_amdgcn_sdot4(wv.z, xv.z, a, false);
+        a = __builtin_amdgcn_sdot4(wv.w, xv.w, a, false);
+        acc[m] = a;
+      }
+    }
+  }
+#pragma unroll
+  for (int m = 0; m < M; ++m) {
+    acc[m] += __shfl_xor(acc[m], 16, 64);
+    acc[m] += __shfl_xor(acc[m], 32, 64);
+  }
+  if (lane < 16) {
+#pragma unroll
+    for (int m = 0; m < M; ++m)
+      red[wave][m][lane] = acc[m];
+  }
+  __syncthreads();
+  if (wave == 0 && lane < 16) {
+    const int n = g * 16 + lane;
+    if (n < N) {
+      const float sa = *a_scale;
+#pragma unroll
+      for (int m = 0; m < M; ++m) {
+        if (m < rows) {
+          const int tot = red[0][m][lane] + red[1][m][lane] + red[2][m][lane] + red[3][m][lane];
+          if (acc_out)
+            acc_out[(size_t)m * N + n] = tot;
+          const float comb = sa * wscale[n];
+          C[(size_t)m * N + n] = (float)tot * comb;
+        }
+      }
+    }
+  }
+}
+
+} // namespace
+} // namespace bh
+
+extern "C" {
+
+size_t buddy_hip_w8a8_workspace_bytes(int64_t M, int64_t K) {
+  if (M <= 0 || K <= 0)
+    return 0;
+  return (size_t)(M * bh::round_up(K, 64)) + 64;
+}
+
+int buddy_hip_w8a8_matmul(const float *A, const int8_t *packed, const float *wscale,
+                          float *C, int32_t *acc_out, int64_t M, int64_t K,
+                          int64_t N, void *workspace, size_t workspace_bytes,
+                          buddy_hip_stream stream) {
+  BH_REQUIRE(A && packed && wscale && C && workspace, "w8a8_matmul: null pointer");
+  BH_REQUIRE(M >= 1 && M <= 16, "w8a8_matmul: M=%lld outside 1..16", (long long)M);
+  BH_REQUIRE(K > 0 && N > 0 && K < (1 << 30) && N < (1 << 30), "w8a8_matmul: bad shape");
+  BH_REQUIRE(workspace_bytes >= buddy_hip_w8a8_workspace_bytes(M, K),
+             "w8a8_matmul: workspace of %zu bytes needed, %zu given",
+             buddy_hip_w8a8_workspace_bytes(M, K), workspace_bytes);
+  BH_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 15) == 0 &&
+                 (reinterpret_cast<uintptr_t>(packed) & 15) == 0,
+             "w8a8_matmul: workspace and weights must be 16-byte aligned");
+  hipStream_t st = bh::as_stream(stream);
+  const int Kp = (int)bh::round_up(K, 64);
+  int8_t *xq = static_cast<int8_t *>(workspace);
+  float *scale = reinterpret_cast<float *>(xq + (size_t)M * Kp);
+  // the scale slot must be 4-byte aligned: M*Kp is a multiple of 64
+  hipLaunchKernelGGL(bh::w8a8_quantize_kernel, dim3(1), dim3(1024), 0, st, A, M * K,
+                     (int)M, (int)K, Kp, xq, scale);
+  const int groups = (int)bh::ceil_div(N, 16), chunks = Kp / 64;
+  const int4 *W = reinterpret_cast<const int4 *>(packed);
+#define BH_W8A8(MT)                                                            \
+  hipLaunchKernelGGL(bh::w8a8_gemv_kernel<MT>, dim3(groups), dim3(256), 0, st, W, \
+                     xq, scale, wscale, C, acc_out, (int)M, (int)N, groups,    \
+                     chunks, Kp)
+  if (M == 1)
+    BH_W8A8(1);
+  else if (M <= 4)
+    BH_W8A8(4);
+  else
+    BH_W8A8(16);
+#undef BH_W8A8
+  BH_CHECK_HIP(hipGetLastError());
+  return BUDDY_HIP_OK;
+}
+}

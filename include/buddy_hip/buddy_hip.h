@@ -270,6 +270,33 @@ int buddy_hip_gemv_f32(const float *x, const float *B, const float *bias,
                        float *y, int64_t K, int64_t N, unsigned flags,
                        buddy_hip_stream stream);
 
+/* ---- the reference's f32 panel packing -------------------------------------
+ * pack_decode_matmul_weights (frontend/Python/graph/transform/
+ * pack_decode_weights.py:94-108): flat[nt*K*V + k*V + v] = B[k, nt*V + v]; same
+ * bytes, same shape; N % V != 0 is refused (:95-99).  The GEMV reads that
+ * order directly (MatMulVectorizationDecodePacked.cpp:207-248, V = 32):
+ * y (+)= x[K] . B[K,N]; without BUDDY_HIP_GEMV_ACCUMULATE y need not be
+ * initialised (the zero-init case of :209-222). */
+int buddy_hip_pack_panels_f32(const float *B, int64_t K, int64_t N, int V,
+                              float *packed, buddy_hip_stream stream);
+int buddy_hip_unpack_panels_f32(const float *packed, int64_t K, int64_t N, int V,
+                                float *B, buddy_hip_stream stream);
+int buddy_hip_gemv_f32_panels(const float *x, const float *packed, float *y,
+                              int64_t K, int64_t N, unsigned flags,
+                              buddy_hip_stream stream);
+
+/* ---- w8a8: int8 activations x int8 weights, int32 partial sums -------------
+ * quantized_matmul_op (frontend/Python/ops/linalg.py:12728-12847): per-tensor
+ * dynamic activation scale s_a = max(absmax(A)/127, 1e-10), A_q = clamp(rint(
+ * A/s_a)), acc = A_q . W in int32 (exact), C = f32(acc) * (s_a * wscale[n]).
+ * `packed` is the wave-tile copy of W; acc_out (int32 [M,N]) may be NULL;
+ * M in 1..16.  workspace: buddy_hip_w8a8_workspace_bytes, 16-byte aligned. */
+size_t buddy_hip_w8a8_workspace_bytes(int64_t M, int64_t K);
+int buddy_hip_w8a8_matmul(const float *A, const int8_t *packed, const float *wscale,
+                          float *C, int32_t *acc_out, int64_t M, int64_t K,
+                          int64_t N, void *workspace, size_t workspace_bytes,
+                          buddy_hip_stream stream);
+
 /* ---- the reference's w8a32 weight package ---------------------------------
  * Builds a session from the two flat blobs the reference's importer writes for
  * the w8a32 variant (arg0-w8a32-f32.data, arg0-w8a32-i8.data;
