@@ -53,10 +53,54 @@ __global__ void __launch_bounds__(kThreads) attn_decode_partial(AttnArgs a) {
 
   const int tid = threadIdx.x;
   const int chunk = blockIdx.x, kvh = blockIdx.y;
-  const int pos = *a.pos_ptr;
   const int p0 = chunk * kChunk;
   const int G = a.group;
   const int h0 = kvh * G;
+
+  // ---- every load that does not need the position goes out first ----------
+  // The cache rows of the chunk exist whatever the position is (rows beyond it
+  // hold zeros or stale data and are masked by select, never multiplied in), so
+  // nothing below waits for the position to arrive.
+  const int sp = tid >> 2, spart = tid & 3; // scores: 4 threads per position
+  const int vq = tid & 31, vg = tid >> 5;   // P.V: 32 threads over d, 8 rows
+  float4 kreg[8], vreg[kChunk / 8];
+  {
+    const int prow = min(p0 + sp, a.max_len - 1);
+    const float *krow = a.kcache + ((size_t)kvh * a.max_len + prow) * kD + spart * 32;
+#pragma unroll
+    for (int c = 0; c < 8; ++c)
+      kreg[c] = *reinterpret_cast<const float4 *>(krow + c * 4);
+#pragma unroll
+    for (int i = 0; i < kChunk / 8; ++i) {
+      const int vrow = min(p0 + vg + 8 * i, a.max_len - 1);
+      vreg[i] = *reinterpret_cast<const float4 *>(
+          a.vcache + ((size_t)kvh * a.max_len + vrow) * kD + vq * 4);
+    }
+  }
+  // raw q of the G heads (3 values per thread at G = 6), raw k and v of the token
+  float qraw[(kMaxGroup * kD + kThreads - 1) / kThreads], qpair[(kMaxGroup * kD + kThreads - 1) / kThreads];
+#pragma unroll
+  for (int r = 0; r < (kMaxGroup * kD + kThreads - 1) / kThreads; ++r) {
+    const int i = tid + r * kThreads;
+    qraw[r] = 0.f;
+    qpair[r] = 0.f;
+    if (i < G * kD) {
+      const int h = i / kD, j = i % kD;
+      const float *q = a.qkv + (size_t)(h0 + h) * kD;
+      qraw[r] = q[j];
+      qpair[r] = j < kD / 2 ? -q[j + kD / 2] : q[j - kD / 2];
+    }
+  }
+  float kraw = 0.f, kpair = 0.f, vraw = 0.f;
+  if (tid < kD) {
+    const int j = tid;
+    const float *k = a.qkv + (size_t)a.heads * kD + (size_t)kvh * kD;
+    kraw = k[j];
+    kpair = j < kD / 2 ? -k[j + kD / 2] : k[j - kD / 2];
+    vraw = k[(size_t)a.kv_heads * kD + j];
+  }
+  const float inv_f = tid < kD / 2 ? a.inv_freq[tid] : 0.f;
+  const int pos = *a.pos_ptr;
 
   if (p0 > pos) { // nothing visible in this chunk: an empty partial
     for (int i = tid; i < G * kD; i += kThreads)
@@ -71,53 +115,30 @@ __global__ void __launch_bounds__(kThreads) attn_decode_partial(AttnArgs a) {
   const int np = p1 - p0;
   const bool has_new = pos >= p0 && pos < p1;
 
-  // ---- the chunk's K and V rows are requested before anything else --------
-  // (rows that are not in the cache yet -- the current token's -- come from
-  // LDS later; their slots are loaded from row p0, which always exists)
-  const int sp = tid >> 2, spart = tid & 3; // scores: 4 threads per position
-  const int vq = tid & 31, vg = tid >> 5;   // P.V: 32 threads over d, 8 rows
-  float4 kreg[8], vreg[kChunk / 8];
-  {
-    const int prow = (sp < np && p0 + sp != pos) ? p0 + sp : p0;
-    const float *krow = a.kcache + ((size_t)kvh * a.max_len + prow) * kD + spart * 32;
-#pragma unroll
-    for (int c = 0; c < 8; ++c)
-      kreg[c] = *reinterpret_cast<const float4 *>(krow + c * 4);
-#pragma unroll
-    for (int i = 0; i < kChunk / 8; ++i) {
-      const int p = vg + 8 * i;
-      const int vrow = (p < np && p0 + p != pos) ? p0 + p : p0;
-      vreg[i] = *reinterpret_cast<const float4 *>(
-          a.vcache + ((size_t)kvh * a.max_len + vrow) * kD + vq * 4);
-    }
-  }
-
   // ---- RoPE tables for this position -------------------------------------
   if (tid < kD / 2) {
-    const float ang = a.inv_freq[tid] * (float)pos;
     float sn, cs;
-    sincosf(ang, &sn, &cs);
+    sincosf(inv_f * (float)pos, &sn, &cs);
     cos_s[tid] = cs;
     sin_s[tid] = sn;
   }
   __syncthreads();
   // q' = q*cos + cat(-q[64:], q[:64])*sin for the G heads of this KV head
-  for (int i = tid; i < G * kD; i += kThreads) {
-    const int h = i / kD, j = i % kD, jj = j & (kD / 2 - 1);
-    const float *q = a.qkv + (size_t)(h0 + h) * kD;
-    const float rot = j < kD / 2 ? -q[j + kD / 2] : q[j - kD / 2];
-    q_s[h][j] = q[j] * cos_s[jj] + rot * sin_s[jj];
+#pragma unroll
+  for (int r = 0; r < (kMaxGroup * kD + kThreads - 1) / kThreads; ++r) {
+    const int i = tid + r * kThreads;
+    if (i < G * kD) {
+      const int h = i / kD, j = i % kD, jj = j & (kD / 2 - 1);
+      q_s[h][j] = qraw[r] * cos_s[jj] + qpair[r] * sin_s[jj];
+    }
   }
   if (has_new && tid < kD) {
     const int j = tid, jj = j & (kD / 2 - 1);
-    const float *k = a.qkv + (size_t)a.heads * kD + (size_t)kvh * kD;
-    const float *v = k + (size_t)a.kv_heads * kD;
-    const float rot = j < kD / 2 ? -k[j + kD / 2] : k[j - kD / 2];
-    const float kn = k[j] * cos_s[jj] + rot * sin_s[jj];
+    const float kn = kraw * cos_s[jj] + kpair * sin_s[jj];
     knew_s[j] = kn;
-    vnew_s[j] = v[j];
+    vnew_s[j] = vraw;
     a.kcache[((size_t)kvh * a.max_len + pos) * kD + j] = kn;
-    a.vcache[((size_t)kvh * a.max_len + pos) * kD + j] = v[j];
+    a.vcache[((size_t)kvh * a.max_len + pos) * kD + j] = vraw;
   }
   __syncthreads();
 
@@ -149,8 +170,7 @@ __global__ void __launch_bounds__(kThreads) attn_decode_partial(AttnArgs a) {
     }
 #pragma unroll
     for (int h = 0; h < kMaxGroup; ++h) {
-      dot[h] += __shfl_xor(dot[h], 1, 64);
-      dot[h] += __shfl_xor(dot[h], 2, 64);
+      dot[h] = quad_sum(dot[h]);
     }
     if (part == 0) {
 #pragma unroll

@@ -43,17 +43,44 @@ inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 inline int64_t round_up(int64_t a, int64_t b) { return ceil_div(a, b) * b; }
 
 #if defined(__HIPCC__)
-// Sum across the 64 lanes of a wavefront; every lane gets the total.
-__device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1)
-    v += __shfl_xor(v, o, 64);
+// Cross-lane reductions on DPP (data-parallel primitives: a VALU operand read
+// from another lane of the same row of 16, a few cycles) instead of
+// ds_bpermute round trips through the LDS crossbar.
+template <int CTRL> __device__ __forceinline__ float dpp_f(float v) {
+  return __int_as_float(
+      __builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, true));
+}
+// every lane gets the sum of its row of 16 lanes
+__device__ __forceinline__ float row16_sum(float v) {
+  v += dpp_f<0xB1>(v);  // quad_perm [1,0,3,2]
+  v += dpp_f<0x4E>(v);  // quad_perm [2,3,0,1]
+  v += dpp_f<0x141>(v); // row_half_mirror
+  v += dpp_f<0x140>(v); // row_mirror
   return v;
 }
+__device__ __forceinline__ float row16_max(float v) {
+  v = fmaxf(v, dpp_f<0xB1>(v));
+  v = fmaxf(v, dpp_f<0x4E>(v));
+  v = fmaxf(v, dpp_f<0x141>(v));
+  v = fmaxf(v, dpp_f<0x140>(v));
+  return v;
+}
+__device__ __forceinline__ float lane_f(float v, int lane) {
+  return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), lane));
+}
+// Sum across the 64 lanes of a wavefront; every lane gets the total.
+__device__ __forceinline__ float wave_sum(float v) {
+  v = row16_sum(v);
+  return (lane_f(v, 0) + lane_f(v, 16)) + (lane_f(v, 32) + lane_f(v, 48));
+}
 __device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1)
-    v = fmaxf(v, __shfl_xor(v, o, 64));
+  v = row16_max(v);
+  return fmaxf(fmaxf(lane_f(v, 0), lane_f(v, 16)), fmaxf(lane_f(v, 32), lane_f(v, 48)));
+}
+// sum over the 4 lanes of a quad / the 8 lanes of two adjacent quads
+__device__ __forceinline__ float quad_sum(float v) {
+  v += dpp_f<0xB1>(v);
+  v += dpp_f<0x4E>(v);
   return v;
 }
 #endif

@@ -41,6 +41,7 @@ struct GemvPlan {
   int64_t chunks, groups;
   int G, KS, waves, tiles_per_round, blocks;
   size_t lds_bytes;
+  bool deep; // >= 16 tiles per wavefront: worth eight loads in flight
 };
 
 int target_waves() {
@@ -86,6 +87,7 @@ GemvPlan make_plan(int64_t M, int64_t K, int64_t N, bool dual) {
     cap = 4;
   p.tiles_per_round = (int)(tiles < cap ? round_up(tiles, 4) : cap);
   p.lds_bytes = round_bytes(p.waves, p.tiles_per_round) + red_bytes(p.waves);
+  p.deep = tiles >= 16;
   return p;
 }
 
@@ -173,8 +175,10 @@ __device__ __forceinline__ void finish(const KernelArgs &a, int m, int n,
 __device__ __forceinline__ float4 attn_combined(const KernelArgs &a, int k) {
   constexpr int B = 8; // partials fetched per batch
   const int h = k / a.head_dim, d = k % a.head_dim;
-  const int pos = *a.pos_ptr;
-  const int used = min(a.attn_nchunks, pos / a.attn_chunk + 1);
+  // every chunk is folded: the ones beyond the position hold (m, l, acc) =
+  // (-1e30, 0, 0) and drop out with weight exp(-1e30 - m) = 0, so the loop does
+  // not have to wait for the position
+  const int used = a.attn_nchunks;
   const float2 *ml = reinterpret_cast<const float2 *>(a.attn_ml) +
                      (size_t)h * a.attn_nchunks;
   const float *acc = a.attn_acc + (size_t)h * a.attn_nchunks * a.head_dim + d;
@@ -219,12 +223,12 @@ __device__ __forceinline__ float4 attn_combined(const KernelArgs &a, int k) {
 
 enum { kProPlain = 0, kProNorm = 1, kProAttn = 2 };
 
-template <int M, int EPI, int PRO>
+template <int M, int EPI, int PRO, int U>
 __global__ void __launch_bounds__(kMaxWaves *kWave)
     gemv_w8a32_kernel(KernelArgs a) {
   constexpr bool DUAL = (EPI == kEpiSiluMul);
   constexpr bool NORM = (PRO == kProNorm);
-  constexpr int U = 4; // weight loads in flight per matrix
+  // U = weight loads in flight per matrix
   extern __shared__ float lds[];
   const int tid = threadIdx.x;
   const int wave = tid >> 6, lane = tid & 63;
@@ -420,9 +424,9 @@ __global__ void __launch_bounds__(kMaxWaves *kWave)
   }
 }
 
-template <int M, int EPI, int PRO>
-int launch_one(const KernelArgs &ka, const GemvPlan &p, hipStream_t stream) {
-  auto kernel = gemv_w8a32_kernel<M, EPI, PRO>;
+template <int M, int EPI, int PRO, int U>
+int launch_u(const KernelArgs &ka, const GemvPlan &p, hipStream_t stream) {
+  auto kernel = gemv_w8a32_kernel<M, EPI, PRO, U>;
   static bool attr_set = false;
   if (!attr_set) {
     BH_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
@@ -434,6 +438,14 @@ int launch_one(const KernelArgs &ka, const GemvPlan &p, hipStream_t stream) {
                      stream, ka);
   BH_CHECK_HIP(hipGetLastError());
   return BUDDY_HIP_OK;
+}
+
+template <int M, int EPI, int PRO>
+int launch_one(const KernelArgs &ka, const GemvPlan &p, hipStream_t stream) {
+  // long single-row, single-matrix streams keep eight tiles in flight
+  if (M == 1 && EPI != kEpiSiluMul && PRO != kProAttn && p.deep)
+    return launch_u<M, EPI, PRO, (M == 1 && EPI != kEpiSiluMul && PRO != kProAttn) ? 8 : 4>(ka, p, stream);
+  return launch_u<M, EPI, PRO, 4>(ka, p, stream);
 }
 
 template <int M>
