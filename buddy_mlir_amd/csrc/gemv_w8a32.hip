@@ -471,6 +471,11 @@ int launch_m(const GemvArgs &a, const KernelArgs &ka, const GemvPlan &p,
   return fail(BUDDY_HIP_ERR_ARG, "gemv: unknown epilogue %d", a.epilogue);
 }
 
+bool force_valu() {
+  static bool v = getenv("BUDDY_HIP_GEMV_FORCE_VALU") != nullptr;
+  return v;
+}
+
 int compiled_rows(int64_t M) {
   return M <= 2 ? (int)M : M <= 4 ? 4 : M <= 8 ? 8 : 16;
 }
@@ -495,6 +500,13 @@ int launch_gemv(const GemvArgs &a, hipStream_t stream) {
              "gemv: packed weights must be 16-byte aligned");
   BH_REQUIRE(!a.norm_w || (reinterpret_cast<uintptr_t>(a.norm_w) & 15) == 0,
              "gemv: norm weight must be 16-byte aligned");
+  // batches of 2..16 rows without a fused norm go to the matrix cores: always
+  // for wide matrices (one activation staging serves eight channel groups);
+  // narrow ones (k-slices inside the workgroup, activations restaged per slice)
+  // only from 6 rows up, below that the f32 FMA path is quicker
+  if (a.M >= 2 && !a.norm_w && !a.attn_acc && !force_valu() &&
+      (ceil_div(a.N, kTileN) >= 2048 / 4 || a.M >= 6))
+    return launch_gemv_mfma(a, stream);
   // the kernel is compiled for 1, 2, 4, 8 and 16 rows; extra rows are zero-
   // filled in LDS and never stored
   const int mt = compiled_rows(a.M);
