@@ -52,16 +52,6 @@ def time_gate_up(bh, shape, sess_stream, layers, iters):
     import torch
     from buddy_mlir_amd import check, ops, synthetic
 
-    class Desc(ctypes.Structure):
-        _fields_ = [("A", ctypes.c_void_p), ("lda", ctypes.c_int64),
-                    ("W0", ctypes.c_void_p), ("scale0", ctypes.c_void_p),
-                    ("W1", ctypes.c_void_p), ("scale1", ctypes.c_void_p),
-                    ("bias", ctypes.c_void_p), ("norm_w", ctypes.c_void_p),
-                    ("norm_eps", ctypes.c_float), ("C", ctypes.c_void_p),
-                    ("ldc", ctypes.c_int64), ("M", ctypes.c_int64),
-                    ("K", ctypes.c_int64), ("N", ctypes.c_int64),
-                    ("epilogue", ctypes.c_int)]
-
     H, I = shape.hidden, shape.inter
     sets = []
     for i in range(layers):
@@ -74,7 +64,7 @@ def time_gate_up(bh, shape, sess_stream, layers, iters):
     h = torch.empty((1, I), device="cuda")
     descs = []
     for pg, sg, pu, su in sets:
-        d = Desc()
+        d = ops.LinearDesc()
         d.A, d.lda, d.W0, d.scale0, d.W1, d.scale1 = (x.data_ptr(), H, pg.data_ptr(),
                                                      sg.data_ptr(), pu.data_ptr(),
                                                      su.data_ptr())
@@ -126,6 +116,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=8)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-graph", action="store_true")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run a 256 MiB device-to-device copy (a kernel of "
+                         "known traffic) for scaling hardware counters")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU's decode throughput; --gpus above 1 is "
@@ -208,6 +201,12 @@ def main():
             "traffic": None,
         },
     }
+    if args.calibrate_copy:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device="cuda")
+        dst = torch.empty_like(src)
+        for _ in range(4):
+            dst.copy_(src)
+        torch.cuda.synchronize()
     if want_cpu:
         out["cpu_baseline"] = cpu_baseline(shape, host, first)
     sess.close()

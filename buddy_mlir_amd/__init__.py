@@ -86,6 +86,9 @@ def _declare(lib):
         "buddy_hip_w8_packed_bytes": (sz, [i64, i64]),
         "buddy_hip_pack_w8": (c_int, [vp, i64, i64, vp, vp]),
         "buddy_hip_unpack_w8": (c_int, [vp, i64, i64, vp, vp]),
+        "buddy_hip_w8_packed_bytes_tiles": (sz, [i64, i64, c_int]),
+        "buddy_hip_pack_w8_tiles": (c_int, [vp, i64, i64, c_int, vp, vp]),
+        "buddy_hip_unpack_w8_tiles": (c_int, [vp, i64, i64, c_int, vp, vp]),
         "buddy_hip_quantize_w8": (c_int, [vp, i64, i64, vp, vp, vp]),
         "buddy_hip_gemv_w8a32": (c_int, [vp, vp, vp, vp, i64, i64, i64, c_uint,
                                          vp]),

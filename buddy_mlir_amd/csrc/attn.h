@@ -10,6 +10,9 @@ constexpr int kAttnChunk = 64; // cache positions per flash-decoding partial
 struct AttnDecodeArgs {
   const float *qkv = nullptr;      // [heads*D | kv_heads*D | kv_heads*D], pre-RoPE
   const float *inv_freq = nullptr; // [D/2]
+  // optional: [cos | sin] of the current position, D/2 values each, computed
+  // once per step; without it every workgroup evaluates them from inv_freq
+  const float *rope_table = nullptr;
   const int *pos_ptr = nullptr;    // device scalar: index of the current token
   float *kcache = nullptr;         // [kv_heads, max_len, D]
   float *vcache = nullptr;

@@ -34,6 +34,7 @@ constexpr float kSeedM = -1.0e30f; // tosa.py:13971
 struct AttnArgs {
   const float *qkv;      // [heads*D | kv_heads*D | kv_heads*D]
   const float *inv_freq; // [D/2]
+  const float *rope_table; // [cos | sin] of the position, or null
   const int *pos_ptr;    // device scalar: index of the current token
   float *kcache, *vcache; // [kv_heads, max_len, D]
   float *part_acc;       // [heads, nchunks, D]
@@ -99,7 +100,15 @@ __global__ void __launch_bounds__(kThreads) attn_decode_partial(AttnArgs a) {
     kpair = j < kD / 2 ? -k[j + kD / 2] : k[j - kD / 2];
     vraw = k[(size_t)a.kv_heads * kD + j];
   }
-  const float inv_f = tid < kD / 2 ? a.inv_freq[tid] : 0.f;
+  float inv_f = 0.f, tab_c = 0.f, tab_s = 0.f;
+  if (tid < kD / 2) {
+    if (a.rope_table) {
+      tab_c = a.rope_table[tid];
+      tab_s = a.rope_table[kD / 2 + tid];
+    } else {
+      inv_f = a.inv_freq[tid];
+    }
+  }
   const int pos = *a.pos_ptr;
 
   if (p0 > pos) { // nothing visible in this chunk: an empty partial
@@ -117,8 +126,9 @@ __global__ void __launch_bounds__(kThreads) attn_decode_partial(AttnArgs a) {
 
   // ---- RoPE tables for this position -------------------------------------
   if (tid < kD / 2) {
-    float sn, cs;
-    sincosf(inv_f * (float)pos, &sn, &cs);
+    float sn = tab_s, cs = tab_c;
+    if (!a.rope_table)
+      sincosf(inv_f * (float)pos, &sn, &cs);
     cos_s[tid] = cs;
     sin_s[tid] = sn;
   }
@@ -301,6 +311,7 @@ int launch_attn_decode(const AttnDecodeArgs &in, hipStream_t stream) {
   AttnArgs a;
   a.qkv = in.qkv;
   a.inv_freq = in.inv_freq;
+  a.rope_table = in.rope_table;
   a.pos_ptr = in.pos_ptr;
   a.kcache = in.kcache;
   a.vcache = in.vcache;

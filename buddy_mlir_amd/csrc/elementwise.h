@@ -20,4 +20,15 @@ size_t argmax_workspace_bytes();
 int launch_argmax(const float *x, int n, void *workspace, int *out_token,
                   int *token_log, int *step_ptr, hipStream_t stream);
 
+// First half of the argmax; *nparts_out candidates are left in the workspace.
+int launch_argmax_partial(const float *x, int n, void *workspace, int *nparts_out,
+                          hipStream_t stream);
+// Tail of a decode step (nparts > 0: pick + log the token; advance: pos/step += 1)
+// and head of the next one (x = embedding row of state[0], rope = [cos | sin] of
+// state[1]).  With nparts = 0 and advance = false it only prepares a step.
+int launch_finish_step(void *amax_workspace, int nparts, int *state, int *token_log,
+                       const float *table, int64_t hidden, int64_t vocab, float *x,
+                       const float *inv_freq, int head_dim, float *rope, bool advance,
+                       hipStream_t stream);
+
 } // namespace bh

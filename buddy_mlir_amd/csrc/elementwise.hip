@@ -134,7 +134,95 @@ argmax_final_kernel(const float *__restrict__ pv, const int *__restrict__ pi,
   }
 }
 
+// Last kernel of a decode step: picks the greedy token from the per-workgroup
+// candidates, logs it, advances position and step, then prepares the next step:
+// its embedding row and the cos/sin table of its position (shared by every
+// layer's attention kernel).  One workgroup.
+__global__ void __launch_bounds__(256)
+finish_step_kernel(const float *__restrict__ pv, const int *__restrict__ pi,
+                   int nparts, int *__restrict__ state, int *__restrict__ token_log,
+                   const float *__restrict__ table, int64_t hidden, int64_t vocab,
+                   float *__restrict__ x, const float *__restrict__ inv_freq,
+                   int half, float *__restrict__ rope, int advance) {
+  __shared__ float sv[4];
+  __shared__ int si[4];
+  __shared__ int s_tok, s_pos;
+  if (nparts > 0) {
+    float v = -INFINITY;
+    int idx = 0x7fffffff;
+    for (int i = threadIdx.x; i < nparts; i += 256)
+      amax_merge(v, idx, pv[i], pi[i]);
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1)
+      amax_merge(v, idx, __shfl_xor(v, o, 64), __shfl_xor(idx, o, 64));
+    if ((threadIdx.x & 63) == 0) {
+      sv[threadIdx.x >> 6] = v;
+      si[threadIdx.x >> 6] = idx;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      for (int w = 1; w < 4; ++w)
+        amax_merge(v, idx, sv[w], si[w]);
+      if (idx == 0x7fffffff)
+        idx = 0;
+      token_log[state[2]] = idx;
+      state[0] = idx;
+    }
+  }
+  if (threadIdx.x == 0) {
+    if (advance) {
+      state[1] += 1;
+      state[2] += 1;
+    }
+    s_tok = state[0];
+    s_pos = state[1];
+  }
+  __syncthreads();
+  int64_t t = s_tok;
+  if (t < 0 || t >= vocab)
+    t = 0;
+  const float *row = table + t * hidden;
+  for (int64_t i = threadIdx.x; i < hidden; i += 256)
+    x[i] = row[i];
+  if (threadIdx.x < half) {
+    float sn, cs;
+    sincosf(inv_freq[threadIdx.x] * (float)s_pos, &sn, &cs);
+    rope[threadIdx.x] = cs;
+    rope[half + threadIdx.x] = sn;
+  }
+}
+
 } // namespace
+
+int launch_finish_step(void *amax_workspace, int nparts, int *state, int *token_log,
+                       const float *table, int64_t hidden, int64_t vocab, float *x,
+                       const float *inv_freq, int head_dim, float *rope, bool advance,
+                       hipStream_t stream) {
+  BH_REQUIRE(state && table && x && inv_freq && rope && head_dim > 0 &&
+                 head_dim / 2 <= 256 && (nparts == 0 || (amax_workspace && token_log)),
+             "finish_step: bad argument");
+  const float *pv = static_cast<const float *>(amax_workspace);
+  const int *pi = reinterpret_cast<const int *>(pv + kArgmaxParts);
+  hipLaunchKernelGGL(finish_step_kernel, dim3(1), dim3(256), 0, stream, pv, pi, nparts,
+                     state, token_log, table, hidden, vocab, x, inv_freq, head_dim / 2,
+                     rope, advance ? 1 : 0);
+  BH_CHECK_HIP(hipGetLastError());
+  return BUDDY_HIP_OK;
+}
+
+int launch_argmax_partial(const float *x, int n, void *workspace, int *nparts_out,
+                          hipStream_t stream) {
+  BH_REQUIRE(x && workspace && n > 0, "argmax: bad argument");
+  float *pv = static_cast<float *>(workspace);
+  int *pi = reinterpret_cast<int *>(pv + kArgmaxParts);
+  int parts = (int)ceil_div(n, 1024);
+  if (parts > kArgmaxParts)
+    parts = kArgmaxParts;
+  hipLaunchKernelGGL(argmax_partial_kernel, dim3(parts), dim3(256), 0, stream, x, n, pv, pi);
+  BH_CHECK_HIP(hipGetLastError());
+  *nparts_out = parts;
+  return BUDDY_HIP_OK;
+}
 
 int launch_embedding(const float *table, const int *token, int64_t hidden,
                      int64_t vocab, float *out, hipStream_t stream) {

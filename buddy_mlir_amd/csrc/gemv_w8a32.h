@@ -33,6 +33,7 @@ struct GemvArgs {
   const float *attn_acc = nullptr, *attn_ml = nullptr;
   const int *pos_ptr = nullptr;
   int attn_nchunks = 0, attn_chunk = 0, head_dim = 0;
+  int tile_n = 16; // channels per packed tile: 16 (default), 8 or 4
   int M = 1;
   int64_t K = 0, N = 0;
   int epilogue = kEpiStore;

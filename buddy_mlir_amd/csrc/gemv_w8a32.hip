@@ -33,7 +33,8 @@ namespace {
 constexpr int kMaxWaves = 16;            // wavefronts per workgroup
 constexpr int kXStride = 20;             // floats per (tile, k-group) in LDS:
                                          // 16 used + 4 pad, conflict-free b128
-constexpr int kTileFloats = 4 * kXStride; // 80 floats of LDS per staged tile
+// LDS floats per staged tile: one padded run per 16 k values
+constexpr int tile_floats(int tn) { return (1024 / tn / 16) * kXStride; }
 constexpr size_t kMaxLdsBytes = 144 * 1024; // hard limit of one workgroup
 constexpr size_t kLdsBudget = 40 * 1024;    // preferred, keeps ~4 workgroups per CU
 
@@ -53,11 +54,11 @@ int target_waves() {
   return v;
 }
 
-GemvPlan make_plan(int64_t M, int64_t K, int64_t N, bool dual) {
+GemvPlan make_plan(int64_t M, int64_t K, int64_t N, bool dual, int tn) {
   (void)dual;
   GemvPlan p;
-  p.chunks = ceil_div(K, kTileK);
-  p.groups = ceil_div(N, kTileN);
+  p.chunks = ceil_div(K, 1024 / tn);
+  p.groups = ceil_div(N, tn);
   // k-slices per channel group: enough wavefronts to cover 256 CUs several
   // times, but at least two tiles per wavefront
   int ks = 1;
@@ -69,7 +70,7 @@ GemvPlan make_plan(int64_t M, int64_t K, int64_t N, bool dual) {
     return sizeof(float) * waves * (size_t)M * (2 * 16 + 1);
   };
   auto round_bytes = [&](int waves, int64_t tiles) {
-    return sizeof(float) * kTileFloats * (size_t)M * waves * (size_t)tiles;
+    return sizeof(float) * tile_floats(tn) * (size_t)M * waves * (size_t)tiles;
   };
   while (ks > 1 && round_bytes(ks < 4 ? 4 : ks, 4) + red_bytes(ks < 4 ? 4 : ks) >
                        kMaxLdsBytes)
@@ -99,7 +100,7 @@ struct KernelArgs {
   int64_t lda, ldc;
   float norm_eps, norm_inv_k;
   int K, N, groups, chunks;
-  int G, KS, tiles_per_round;
+  int G, KS, tiles_per_round, tile_n;
   int rows; // valid rows; the kernel is compiled for the next power of two
   // activation provider 2: fold flash-decoding partials while staging
   const float *attn_acc, *attn_ml;
@@ -173,7 +174,7 @@ __device__ __forceinline__ void finish(const KernelArgs &a, int m, int n,
 // (the combine of frontend/Python/ops/tosa.py:14485-14594, eight chunks at a
 // time so that their loads are in flight together).
 __device__ __forceinline__ float4 attn_combined(const KernelArgs &a, int k) {
-  constexpr int B = 8; // partials fetched per batch
+  constexpr int B = 9; // partials fetched per batch (two batches at 18 chunks)
   const int h = k / a.head_dim, d = k % a.head_dim;
   // every chunk is folded: the ones beyond the position hold (m, l, acc) =
   // (-1e30, 0, 0) and drop out with weight exp(-1e30 - m) = 0, so the loop does
@@ -223,9 +224,11 @@ __device__ __forceinline__ float4 attn_combined(const KernelArgs &a, int k) {
 
 enum { kProPlain = 0, kProNorm = 1, kProAttn = 2 };
 
-template <int M, int EPI, int PRO, int U>
+template <int M, int EPI, int PRO, int U, int TN>
 __global__ void __launch_bounds__(kMaxWaves *kWave)
     gemv_w8a32_kernel(KernelArgs a) {
+  constexpr int TK = 1024 / TN;           // k values per tile
+  constexpr int kTileFloats = tile_floats(TN);
   constexpr bool DUAL = (EPI == kEpiSiluMul);
   constexpr bool NORM = (PRO == kProNorm);
   // U = weight loads in flight per matrix
@@ -256,12 +259,11 @@ __global__ void __launch_bounds__(kMaxWaves *kWave)
   const int4 *w0 = a.W0 + wbase;
   const int4 *w1 = DUAL ? a.W1 + wbase : a.W0 + wbase;
   // where this lane's float4 of a 256-float staging load lands in LDS
-  const int st_off = ((lane >> 4) * 4 + ((lane & 15) >> 2)) * kXStride +
-                     (lane & 3) * 4;
-  const float *xl = xs + (lane >> 4) * kXStride;
+  const int st_off = (lane >> 2) * kXStride + (lane & 3) * 4;
+  const float *xl = xs + (lane / TN) * kXStride; // this lane's k sub-range
 
   const int nrounds = (per + TR - 1) / TR; // same for every wavefront
-  const int kend = min(a.K, t1 * kTileK);   // this wavefront's k range ends here
+  const int kend = min(a.K, t1 * TK);       // this wavefront's k range ends here
   for (int rd = 0; rd < nrounds; ++rd) {
     const int r0 = t0 + rd * TR;
     const int r1 = min(r0 + TR, t1);
@@ -270,17 +272,18 @@ __global__ void __launch_bounds__(kMaxWaves *kWave)
     if (r0 < r1) {
 #pragma unroll
       for (int u = 0; u < U; ++u) {
-        const int t = min(r0 + u, a.chunks - 1);
-        wa[u] = load_stream(w0 + (size_t)t * 64);
-        if (DUAL)
-          wb[u] = load_stream(w1 + (size_t)t * 64);
+        if (r0 + u < r1) { // never fetch a tile this wavefront will not use
+          wa[u] = load_stream(w0 + (size_t)(r0 + u) * 64);
+          if (DUAL)
+            wb[u] = load_stream(w1 + (size_t)(r0 + u) * 64);
+        }
       }
     }
     // ---- stage this wavefront's slice of the activations -----------------
     if (rd != 0)
       __syncthreads(); // everyone is done with the previous round's LDS
-    for (int i = 0; i < (r1 - r0 + 3) / 4; ++i) {
-      const int k = (r0 + 4 * i) * kTileK + lane * 4;
+    for (int i = 0; i < ((r1 - r0) * TK + 255) / 256; ++i) {
+      const int k = r0 * TK + i * 256 + lane * 4;
       float4 nw = make_float4(1.f, 1.f, 1.f, 1.f);
       const bool in = k + 3 < kend;
       if (NORM) {
@@ -316,7 +319,7 @@ __global__ void __launch_bounds__(kMaxWaves *kWave)
           v.z *= nw.z;
           v.w *= nw.w;
         }
-        *reinterpret_cast<float4 *>(xs + m * row_stride + i * 4 * kTileFloats +
+        *reinterpret_cast<float4 *>(xs + m * row_stride + i * 16 * kXStride +
                                     st_off) = v;
       }
     }
@@ -328,10 +331,11 @@ __global__ void __launch_bounds__(kMaxWaves *kWave)
       if (more) {
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-          const int tt = min(t + U + u, a.chunks - 1);
-          na[u] = load_stream(w0 + (size_t)tt * 64);
-          if (DUAL)
-            nb[u] = load_stream(w1 + (size_t)tt * 64);
+          if (t + U + u < r1) {
+            na[u] = load_stream(w0 + (size_t)(t + U + u) * 64);
+            if (DUAL)
+              nb[u] = load_stream(w1 + (size_t)(t + U + u) * 64);
+          }
         }
       }
 #pragma unroll
@@ -354,14 +358,14 @@ __global__ void __launch_bounds__(kMaxWaves *kWave)
     }
   }
 
-  // the four 16-lane rows hold four k sub-ranges of the same 16 channels
+  // lanes TN apart hold different k sub-ranges of the same channel
 #pragma unroll
   for (int m = 0; m < M; ++m) {
-    acc0[m] += __shfl_xor(acc0[m], 16, 64);
-    acc0[m] += __shfl_xor(acc0[m], 32, 64);
-    if (DUAL) {
-      acc1[m] += __shfl_xor(acc1[m], 16, 64);
-      acc1[m] += __shfl_xor(acc1[m], 32, 64);
+#pragma unroll
+    for (int o = TN; o < 64; o <<= 1) {
+      acc0[m] += __shfl_xor(acc0[m], o, 64);
+      if (DUAL)
+        acc1[m] += __shfl_xor(acc1[m], o, 64);
     }
     if (NORM)
       ss[m] = wave_sum(ss[m]);
@@ -370,7 +374,7 @@ __global__ void __launch_bounds__(kMaxWaves *kWave)
   // ---- k-slices of one channel group meet in LDS, in slice order ----------
   if (a.KS > 1) {
     float *mine = red + (size_t)wave * M * 33;
-    if (lane < 16) {
+    if (lane < TN) {
 #pragma unroll
       for (int m = 0; m < M; ++m) {
         mine[m * 33 + lane] = acc0[m];
@@ -386,7 +390,7 @@ __global__ void __launch_bounds__(kMaxWaves *kWave)
     __syncthreads();
     if (ks != 0)
       return;
-    if (lane < 16) {
+    if (lane < TN) {
 #pragma unroll
       for (int m = 0; m < M; ++m) {
         float r0 = 0.f, r1 = 0.f, rs = 0.f;
@@ -404,8 +408,8 @@ __global__ void __launch_bounds__(kMaxWaves *kWave)
       }
     }
   }
-  const int n = g * kTileN + lane;
-  if (lane < kTileN && live && n < a.N) {
+  const int n = g * TN + lane;
+  if (lane < TN && live && n < a.N) {
 #pragma unroll
     for (int m = 0; m < M; ++m) {
       if (m < a.rows) {
@@ -424,9 +428,9 @@ __global__ void __launch_bounds__(kMaxWaves *kWave)
   }
 }
 
-template <int M, int EPI, int PRO, int U>
-int launch_u(const KernelArgs &ka, const GemvPlan &p, hipStream_t stream) {
-  auto kernel = gemv_w8a32_kernel<M, EPI, PRO, U>;
+template <int M, int EPI, int PRO, int U, int TN>
+int launch_tn(const KernelArgs &ka, const GemvPlan &p, hipStream_t stream) {
+  auto kernel = gemv_w8a32_kernel<M, EPI, PRO, U, TN>;
   static bool attr_set = false;
   if (!attr_set) {
     BH_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
@@ -438,6 +442,21 @@ int launch_u(const KernelArgs &ka, const GemvPlan &p, hipStream_t stream) {
                      stream, ka);
   BH_CHECK_HIP(hipGetLastError());
   return BUDDY_HIP_OK;
+}
+
+// Narrow tiles (8 or 4 channels) exist for one-row launches of narrow matrices.
+template <int M, int EPI, int PRO, int U>
+int launch_u(const KernelArgs &ka, const GemvPlan &p, hipStream_t stream) {
+  if (M == 1 && EPI != kEpiSiluMul) {
+    if (ka.tile_n == 8)
+      return launch_tn<M, EPI, PRO, U, (M == 1 && EPI != kEpiSiluMul) ? 8 : 16>(ka, p, stream);
+    if (ka.tile_n == 4)
+      return launch_tn<M, EPI, PRO, U, (M == 1 && EPI != kEpiSiluMul) ? 4 : 16>(ka, p, stream);
+  }
+  if (ka.tile_n != 16)
+    return fail(BUDDY_HIP_ERR_ARG, "gemv: %d-channel tiles need M = 1 and one matrix",
+                ka.tile_n);
+  return launch_tn<M, EPI, PRO, U, 16>(ka, p, stream);
 }
 
 template <int M, int EPI, int PRO>
@@ -505,12 +524,14 @@ int launch_gemv(const GemvArgs &a, hipStream_t stream) {
   // narrow ones (k-slices inside the workgroup, activations restaged per slice)
   // only from 6 rows up, below that the f32 FMA path is quicker
   if (a.M >= 2 && !a.norm_w && !a.attn_acc && !force_valu() &&
-      (ceil_div(a.N, kTileN) >= 2048 / 4 || a.M >= 6))
+      a.tile_n == 16 && (ceil_div(a.N, kTileN) >= 2048 / 4 || a.M >= 6))
     return launch_gemv_mfma(a, stream);
   // the kernel is compiled for 1, 2, 4, 8 and 16 rows; extra rows are zero-
   // filled in LDS and never stored
   const int mt = compiled_rows(a.M);
-  const GemvPlan p = make_plan(mt, a.K, a.N, dual);
+  BH_REQUIRE(a.tile_n == 16 || a.tile_n == 8 || a.tile_n == 4,
+             "gemv: tile_n=%d (16, 8 or 4)", a.tile_n);
+  const GemvPlan p = make_plan(mt, a.K, a.N, dual, a.tile_n);
   KernelArgs ka;
   ka.A = a.A;
   ka.W0 = reinterpret_cast<const int4 *>(a.W0);
@@ -531,6 +552,7 @@ int launch_gemv(const GemvArgs &a, hipStream_t stream) {
   ka.G = p.G;
   ka.KS = p.KS;
   ka.tiles_per_round = p.tiles_per_round;
+  ka.tile_n = a.tile_n;
   ka.rows = a.M;
   ka.attn_acc = a.attn_acc;
   ka.attn_ml = a.attn_ml;
@@ -571,6 +593,7 @@ int buddy_hip_linear_w8a32(const buddy_hip_linear_desc *d,
   a.K = d->K;
   a.N = d->N;
   a.epilogue = d->epilogue;
+  a.tile_n = d->tile_n ? d->tile_n : 16;
   BH_REQUIRE(d->M >= 1 && d->M <= 16, "linear_w8a32: M=%lld outside 1..16",
              (long long)d->M);
   BH_REQUIRE(!(d->bias && d->epilogue != BUDDY_HIP_EPI_STORE),

@@ -54,15 +54,16 @@ quantize_kernel(const float *__restrict__ W, const float *__restrict__ scale,
 // One thread writes one lane's 16 bytes of one tile.
 __global__ void __launch_bounds__(256)
 pack_w8_kernel(const int8_t *__restrict__ W, int64_t K, int64_t N,
-               int64_t chunks, int64_t total_lanes, int8_t *__restrict__ P) {
+               int64_t chunks, int64_t total_lanes, int tn,
+               int8_t *__restrict__ P) {
   const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (t >= total_lanes)
     return;
   const int lane = (int)(t & 63);
   const int64_t tile = t >> 6;
   const int64_t c = tile % chunks, g = tile / chunks;
-  const int64_t n = g * kTileN + (lane & 15);
-  const int64_t kb = c * kTileK + (lane >> 4) * 16;
+  const int64_t n = g * tn + (lane % tn);
+  const int64_t kb = c * (1024 / tn) + (lane / tn) * 16;
   union {
     int8_t b[16];
     int4 v;
@@ -77,13 +78,14 @@ pack_w8_kernel(const int8_t *__restrict__ W, int64_t K, int64_t N,
 
 __global__ void __launch_bounds__(256)
 unpack_w8_kernel(const int8_t *__restrict__ P, int64_t K, int64_t N,
-                 int64_t chunks, int8_t *__restrict__ W) {
+                 int64_t chunks, int tn, int8_t *__restrict__ W) {
   const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= K * N)
     return;
   const int64_t k = i / N, n = i % N;
-  const int64_t g = n / kTileN, c = k / kTileK;
-  const int lane = (int)(((k % kTileK) / 16) * 16 + (n % kTileN));
+  const int tk = 1024 / tn;
+  const int64_t g = n / tn, c = k / tk;
+  const int lane = (int)(((k % tk) / 16) * tn + (n % tn));
   W[i] = P[((g * chunks + c) * 64 + lane) * 16 + (k % 16)];
 }
 
@@ -92,38 +94,56 @@ unpack_w8_kernel(const int8_t *__restrict__ P, int64_t K, int64_t N,
 
 extern "C" {
 
-size_t buddy_hip_w8_packed_bytes(int64_t K, int64_t N) {
-  if (K <= 0 || N <= 0)
+static bool valid_tile_n(int tn) { return tn == 16 || tn == 8 || tn == 4; }
+
+size_t buddy_hip_w8_packed_bytes_tiles(int64_t K, int64_t N, int tile_n) {
+  if (K <= 0 || N <= 0 || !valid_tile_n(tile_n))
     return 0;
-  return (size_t)(bh::round_up(K, bh::kTileK) * bh::round_up(N, bh::kTileN));
+  return (size_t)(bh::round_up(K, 1024 / tile_n) * bh::round_up(N, tile_n));
+}
+
+size_t buddy_hip_w8_packed_bytes(int64_t K, int64_t N) {
+  return buddy_hip_w8_packed_bytes_tiles(K, N, bh::kTileN);
+}
+
+int buddy_hip_pack_w8_tiles(const int8_t *W, int64_t K, int64_t N, int tile_n,
+                            int8_t *packed, buddy_hip_stream stream) {
+  BH_REQUIRE(W && packed, "pack_w8: null pointer");
+  BH_REQUIRE(K > 0 && N > 0, "pack_w8: bad shape K=%lld N=%lld", (long long)K,
+             (long long)N);
+  BH_REQUIRE(valid_tile_n(tile_n), "pack_w8: tile_n=%d (16, 8 or 4)", tile_n);
+  const int64_t chunks = bh::ceil_div(K, 1024 / tile_n);
+  const int64_t groups = bh::ceil_div(N, tile_n);
+  const int64_t lanes = groups * chunks * 64;
+  hipLaunchKernelGGL(bh::pack_w8_kernel, dim3((unsigned)bh::ceil_div(lanes, 256)),
+                     dim3(256), 0, bh::as_stream(stream), W, K, N, chunks,
+                     lanes, tile_n, packed);
+  BH_CHECK_HIP(hipGetLastError());
+  return BUDDY_HIP_OK;
 }
 
 int buddy_hip_pack_w8(const int8_t *W, int64_t K, int64_t N, int8_t *packed,
                       buddy_hip_stream stream) {
-  BH_REQUIRE(W && packed, "pack_w8: null pointer");
-  BH_REQUIRE(K > 0 && N > 0, "pack_w8: bad shape K=%lld N=%lld", (long long)K,
+  return buddy_hip_pack_w8_tiles(W, K, N, bh::kTileN, packed, stream);
+}
+
+int buddy_hip_unpack_w8_tiles(const int8_t *packed, int64_t K, int64_t N,
+                              int tile_n, int8_t *W, buddy_hip_stream stream) {
+  BH_REQUIRE(W && packed, "unpack_w8: null pointer");
+  BH_REQUIRE(K > 0 && N > 0, "unpack_w8: bad shape K=%lld N=%lld", (long long)K,
              (long long)N);
-  const int64_t chunks = bh::ceil_div(K, bh::kTileK);
-  const int64_t groups = bh::ceil_div(N, bh::kTileN);
-  const int64_t lanes = groups * chunks * 64;
-  hipLaunchKernelGGL(bh::pack_w8_kernel, dim3((unsigned)bh::ceil_div(lanes, 256)),
-                     dim3(256), 0, bh::as_stream(stream), W, K, N, chunks,
-                     lanes, packed);
+  BH_REQUIRE(valid_tile_n(tile_n), "unpack_w8: tile_n=%d (16, 8 or 4)", tile_n);
+  const int64_t chunks = bh::ceil_div(K, 1024 / tile_n);
+  hipLaunchKernelGGL(bh::unpack_w8_kernel,
+                     dim3((unsigned)bh::ceil_div(K * N, 256)), dim3(256), 0,
+                     bh::as_stream(stream), packed, K, N, chunks, tile_n, W);
   BH_CHECK_HIP(hipGetLastError());
   return BUDDY_HIP_OK;
 }
 
 int buddy_hip_unpack_w8(const int8_t *packed, int64_t K, int64_t N, int8_t *W,
                         buddy_hip_stream stream) {
-  BH_REQUIRE(W && packed, "unpack_w8: null pointer");
-  BH_REQUIRE(K > 0 && N > 0, "unpack_w8: bad shape K=%lld N=%lld", (long long)K,
-             (long long)N);
-  const int64_t chunks = bh::ceil_div(K, bh::kTileK);
-  hipLaunchKernelGGL(bh::unpack_w8_kernel,
-                     dim3((unsigned)bh::ceil_div(K * N, 256)), dim3(256), 0,
-                     bh::as_stream(stream), packed, K, N, chunks, W);
-  BH_CHECK_HIP(hipGetLastError());
-  return BUDDY_HIP_OK;
+  return buddy_hip_unpack_w8_tiles(packed, K, N, bh::kTileN, W, stream);
 }
 
 int buddy_hip_quantize_w8(const float *W, int64_t K, int64_t N, int8_t *q,

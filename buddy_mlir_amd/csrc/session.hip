@@ -41,6 +41,8 @@ int launch_matmul_f32(const float *A, const float *B, float *C, int64_t M,
 
 namespace {
 
+constexpr int kNarrowTile = 8;
+
 struct PackedLinear {
   int8_t *w = nullptr; // wave tiles
   float *s = nullptr;  // scales
@@ -54,6 +56,10 @@ struct Layer {
   // the reference's shipped w8a32 build keeps q/k/v in f32 with a bias
   // (they import as AddMMOp, which the quantizer does not touch):
   float *qkv_f32 = nullptr; // [hidden, q|k|v] dense, or null when int8
+  // down_proj has only hidden/16 channel groups (96 at 1536), fewer than the
+  // CUs: the decode step reads a second copy packed in 8-channel tiles, the
+  // prefill matmul the 16-channel one
+  int8_t *down_narrow = nullptr;
   float *kc = nullptr, *vc = nullptr; // [kv_heads, max_len, D]
   bool set = false;
 };
@@ -71,14 +77,6 @@ embedding_rows_kernel(const float *__restrict__ table, const int *__restrict__ t
     dst[i] = row[i];
 }
 
-__global__ void advance_kernel(int *state) {
-  // state: [0] token, [1] pos, [2] step
-  if (threadIdx.x == 0) {
-    state[1] += 1;
-    state[2] += 1;
-  }
-}
-
 } // namespace
 
 struct Session {
@@ -88,6 +86,7 @@ struct Session {
   std::vector<Layer> layers;
   const float *embed = nullptr; // borrowed: [vocab, hidden] f32
   float *ln_f = nullptr, *inv_freq = nullptr;
+  float *rope = nullptr; // [cos | sin] of the step's position
   PackedLinear lm;
   // activations
   float *x = nullptr, *xn = nullptr, *qkv = nullptr, *att = nullptr,
@@ -154,11 +153,12 @@ struct Session {
   }
 
   int gemv(const float *A, const PackedLinear &W0, const PackedLinear *W1,
-           const float *norm_w, float *C, int epi) {
+           const float *norm_w, float *C, int epi, const int8_t *narrow = nullptr) {
     GemvArgs g;
     g.A = A;
     g.lda = W0.K;
-    g.W0 = W0.w;
+    g.W0 = narrow ? narrow : W0.w;
+    g.tile_n = narrow ? kNarrowTile : 16;
     g.s0 = W0.s;
     if (W1) {
       g.W1 = W1->w;
@@ -179,10 +179,10 @@ struct Session {
 
   // Enqueues one decode step (reads token/pos from device state).
   int enqueue_step() {
+    // x and the RoPE table were prepared by the previous step's last kernel (or
+    // by prepare_step after the host set token and position)
     const auto &S = shape;
-    int rc = launch_embedding(embed, state, S.hidden, S.vocab, x, stream);
-    if (rc)
-      return rc;
+    int rc;
     const float scale = (float)(1.0 / std::sqrt((double)S.head_dim));
     for (int i = 0; i < S.layers; ++i) {
       Layer &L = layers[(size_t)i];
@@ -198,6 +198,7 @@ struct Session {
       AttnDecodeArgs a;
       a.qkv = qkv;
       a.inv_freq = inv_freq;
+      a.rope_table = rope;
       a.pos_ptr = state + 1;
       a.kcache = L.kc;
       a.vcache = L.vc;
@@ -235,17 +236,23 @@ struct Session {
       }
       if ((rc = gemv(x, L.gate, &L.up, L.ln2, h, kEpiSiluMul)))
         return rc;
-      if ((rc = gemv(h, L.down, nullptr, nullptr, x, kEpiAccum)))
+      if ((rc = gemv(h, L.down, nullptr, nullptr, x, kEpiAccum, L.down_narrow)))
         return rc;
     }
     if ((rc = gemv(x, lm, nullptr, ln_f, logits, kEpiStore)))
       return rc;
-    if ((rc = launch_argmax(logits, S.vocab, amax_ws, state, token_log,
-                            state + 2, stream)))
+    int nparts = 0;
+    if ((rc = launch_argmax_partial(logits, S.vocab, amax_ws, &nparts, stream)))
       return rc;
-    hipLaunchKernelGGL(advance_kernel, dim3(1), dim3(64), 0, stream, state);
-    BH_CHECK_HIP(hipGetLastError());
-    return BUDDY_HIP_OK;
+    return launch_finish_step(amax_ws, nparts, state, token_log, embed, S.hidden,
+                              S.vocab, x, inv_freq, S.head_dim, rope, true, stream);
+  }
+
+  // After the host wrote token/position: embedding row and RoPE table of the step.
+  int prepare_step() {
+    const auto &S = shape;
+    return launch_finish_step(amax_ws, 0, state, token_log, embed, S.hidden, S.vocab,
+                              x, inv_freq, S.head_dim, rope, false, stream);
   }
 
   int ensure_prefill_buffers(int rows) {
@@ -384,6 +391,9 @@ struct Session {
     host_state[2] = step;
     BH_CHECK_HIP(hipMemcpyAsync(state, host_state, 3 * sizeof(int),
                                 hipMemcpyHostToDevice, stream));
+    int rc = prepare_step();
+    if (rc)
+      return rc;
     // the pinned staging words are reused by the next call
     BH_CHECK_HIP(hipStreamSynchronize(stream));
     return BUDDY_HIP_OK;
@@ -439,6 +449,7 @@ buddy_hip_session *buddy_hip_session_create(const buddy_hip_model_shape *shape,
   rc |= s->alloc(&s->logits, (size_t)S.vocab);
   rc |= s->alloc(&s->ln_f, (size_t)S.hidden);
   rc |= s->alloc(&s->inv_freq, (size_t)S.head_dim / 2);
+  rc |= s->alloc(&s->rope, (size_t)S.head_dim);
   rc |= s->alloc(&s->state, 4);
   s->token_log_cap = 65536;
   rc |= s->alloc(&s->token_log, (size_t)s->token_log_cap);
@@ -559,6 +570,8 @@ int buddy_hip_session_set_layer(buddy_hip_session *hs, int index,
       rc |= s->alloc(&P->w, buddy_hip_w8_packed_bytes(P->K, P->N));
       rc |= s->alloc(&P->s, (size_t)P->N);
     }
+    rc |= s->alloc(&L.down_narrow,
+                   buddy_hip_w8_packed_bytes_tiles(I, H, bh::kNarrowTile));
     if (rc)
       return rc;
   }
@@ -589,6 +602,7 @@ int buddy_hip_session_set_layer(buddy_hip_session *hs, int index,
   rc |= s->pack_into(w->wg, w->sg, nullptr, H, I, L.gate.w, L.gate.s, nullptr);
   rc |= s->pack_into(w->wu, w->su, nullptr, H, I, L.up.w, L.up.s, nullptr);
   rc |= s->pack_into(w->wd, w->sd, nullptr, I, H, L.down.w, L.down.s, nullptr);
+  rc |= buddy_hip_pack_w8_tiles(w->wd, I, H, bh::kNarrowTile, L.down_narrow, s->stream);
   if (rc)
     return rc;
   BH_CHECK_HIP(hipMemcpyAsync(L.ln1, w->ln1, sizeof(float) * H, hipMemcpyDefault, s->stream));
@@ -802,6 +816,9 @@ int buddy_hip_session_set_state(buddy_hip_session *hs, int token, int pos) {
   BH_REQUIRE(token >= 0 && token < s->shape.vocab && pos >= 0 &&
                  pos < s->shape.max_len,
              "session_set_state: token %d / position %d out of range", token, pos);
+  int rc = s->ready();
+  if (rc)
+    return rc;
   return s->set_state(token, pos, 0);
 }
 

@@ -5,11 +5,61 @@ through the C ABI.  Nothing falls back to torch or to the CPU.
 """
 from __future__ import annotations
 
+import ctypes
+
 import torch
 
 from . import check, lib
 
 GEMV_ACCUMULATE = 1
+EPI_STORE, EPI_ACCUM, EPI_SILU_MUL = 0, 1, 2
+
+
+class LinearDesc(ctypes.Structure):
+    """ctypes mirror of buddy_hip_linear_desc."""
+    _fields_ = [("A", ctypes.c_void_p), ("lda", ctypes.c_int64),
+                ("W0", ctypes.c_void_p), ("scale0", ctypes.c_void_p),
+                ("W1", ctypes.c_void_p), ("scale1", ctypes.c_void_p),
+                ("bias", ctypes.c_void_p), ("norm_w", ctypes.c_void_p),
+                ("norm_eps", ctypes.c_float), ("C", ctypes.c_void_p),
+                ("ldc", ctypes.c_int64), ("M", ctypes.c_int64),
+                ("K", ctypes.c_int64), ("N", ctypes.c_int64),
+                ("epilogue", ctypes.c_int), ("tile_n", ctypes.c_int)]
+
+
+def linear_desc(**kw) -> LinearDesc:
+    d = LinearDesc()
+    for k, v in kw.items():
+        setattr(d, k, v.data_ptr() if isinstance(v, torch.Tensor) else v)
+    return d
+
+
+def linear_w8a32(stream=None, **kw):
+    """buddy_hip_linear_w8a32 with keyword fields of the descriptor."""
+    d = linear_desc(**kw)
+    check(lib().buddy_hip_linear_w8a32(ctypes.byref(d),
+                                       _stream() if stream is None else stream),
+          "linear_w8a32")
+
+
+def pack_w8_tiles(q: torch.Tensor, tile_n: int) -> torch.Tensor:
+    _dev(q, torch.int8)
+    K, N = q.shape
+    nbytes = lib().buddy_hip_w8_packed_bytes_tiles(K, N, tile_n)
+    if nbytes == 0:
+        raise ValueError(f"bad tile_n {tile_n}")
+    out = torch.empty((nbytes,), dtype=torch.int8, device=q.device)
+    check(lib().buddy_hip_pack_w8_tiles(q.data_ptr(), K, N, tile_n, out.data_ptr(),
+                                        _stream()), "pack_w8_tiles")
+    return out
+
+
+def unpack_w8_tiles(packed: torch.Tensor, K: int, N: int, tile_n: int) -> torch.Tensor:
+    _dev(packed, torch.int8)
+    out = torch.empty((K, N), dtype=torch.int8, device=packed.device)
+    check(lib().buddy_hip_unpack_w8_tiles(packed.data_ptr(), K, N, tile_n,
+                                          out.data_ptr(), _stream()), "unpack_w8_tiles")
+    return out
 
 
 def _stream() -> int:

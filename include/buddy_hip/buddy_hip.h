@@ -61,6 +61,16 @@ int buddy_hip_pack_w8(const int8_t *W, int64_t K, int64_t N, int8_t *packed,
                       buddy_hip_stream stream);
 int buddy_hip_unpack_w8(const int8_t *packed, int64_t K, int64_t N, int8_t *W,
                         buddy_hip_stream stream);
+/* Narrower tiles for narrow matrices at M = 1 (down / o_proj: 1536 outputs are
+ * only 96 groups of 16, fewer than the 256 CUs): a tile is tile_n channels x
+ * (1024 / tile_n) k, tile_n = 16 (as above), 8 or 4; lane L owns channel
+ * g*tile_n + L % tile_n and k = c*(1024/tile_n) + (L / tile_n)*16 + 0..15.
+ * Only buddy_hip_linear_w8a32 with M = 1 and one matrix reads these. */
+size_t buddy_hip_w8_packed_bytes_tiles(int64_t K, int64_t N, int tile_n);
+int buddy_hip_pack_w8_tiles(const int8_t *W, int64_t K, int64_t N, int tile_n,
+                            int8_t *packed, buddy_hip_stream stream);
+int buddy_hip_unpack_w8_tiles(const int8_t *packed, int64_t K, int64_t N,
+                              int tile_n, int8_t *W, buddy_hip_stream stream);
 
 /* ---- per-output-channel symmetric quantizer ----------------------------
  * tools/buddy-codegen/import_model.py:837-848,874-880 on device: W f32 [K,N],
@@ -100,6 +110,7 @@ typedef struct buddy_hip_linear_desc {
   int64_t ldc;
   int64_t M, K, N;      /* M in 1..16 */
   int epilogue;         /* BUDDY_HIP_EPI_* */
+  int tile_n;           /* channels per packed tile: 0 or 16 (default), 8, 4 */
 } buddy_hip_linear_desc;
 enum {
   BUDDY_HIP_EPI_STORE = 0,   /* C = acc*scale (+ bias) */

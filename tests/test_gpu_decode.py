@@ -23,20 +23,8 @@ def dev(a, dtype=torch.float32):
 
 
 def linear(bh, **kw):
-    class Desc(ctypes.Structure):
-        _fields_ = [("A", ctypes.c_void_p), ("lda", ctypes.c_int64),
-                    ("W0", ctypes.c_void_p), ("scale0", ctypes.c_void_p),
-                    ("W1", ctypes.c_void_p), ("scale1", ctypes.c_void_p),
-                    ("bias", ctypes.c_void_p), ("norm_w", ctypes.c_void_p),
-                    ("norm_eps", ctypes.c_float), ("C", ctypes.c_void_p),
-                    ("ldc", ctypes.c_int64), ("M", ctypes.c_int64),
-                    ("K", ctypes.c_int64), ("N", ctypes.c_int64),
-                    ("epilogue", ctypes.c_int)]
-    d = Desc()
-    for k, v in kw.items():
-        setattr(d, k, v.data_ptr() if isinstance(v, torch.Tensor) else v)
     torch.cuda.synchronize()
-    bma.check(bh.buddy_hip_linear_w8a32(ctypes.byref(d), None), "linear")
+    ops.linear_w8a32(stream=None, **kw)
     torch.cuda.synchronize()
 
 
@@ -86,6 +74,13 @@ def test_norm_prologue_and_residual_epilogue(bh, oracle):
     want = np.stack([bh_ + oracle.dequant_gemv(oracle.rmsnorm(xh[m], wh, EPS), qh, sh)
                      for m in range(2)])
     check_close(out.cpu().numpy(), want)
+    # narrow tiles (8 and 4 channels per tile) at M = 1: same result
+    for tn in (8, 4):
+        out1 = torch.empty((1, N), device="cuda")
+        linear(bh, A=x, lda=K, W0=ops.pack_w8_tiles(q, tn), scale0=s, norm_w=w,
+               norm_eps=float(EPS), bias=bias, C=out1, ldc=N, M=1, K=K, N=N, epilogue=0,
+               tile_n=tn)
+        check_close(out1.cpu().numpy()[0], want[0])
     # residual: C += ...
     c0 = torch.randn((2, N), generator=g, device="cuda")
     c = c0.clone()

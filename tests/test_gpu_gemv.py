@@ -52,6 +52,39 @@ def test_pack_roundtrip_and_layout(K, N):
     assert int(np.abs(ph.astype(np.int32)).sum()) == int(np.abs(qh.astype(np.int32)).sum())
 
 
+@pytest.mark.parametrize("tn", [8, 4])
+@pytest.mark.parametrize("K,N", [(256, 8), (8960, 1536), (1536, 1536), (300, 50), (1, 1)])
+def test_narrow_tile_layouts(oracle, K, N, tn):
+    g = torch.Generator(device="cuda").manual_seed(K + N + tn)
+    q = torch.randint(-128, 128, (K, N), generator=g, device="cuda", dtype=torch.int8)
+    p = ops.pack_w8_tiles(q, tn)
+    tk = 1024 // tn
+    assert p.numel() == ((K + tk - 1) // tk * tk) * ((N + tn - 1) // tn * tn)
+    np.testing.assert_array_equal(ops.unpack_w8_tiles(p, K, N, tn).cpu().numpy(),
+                                  q.cpu().numpy())
+    qh, ph = q.cpu().numpy(), p.cpu().numpy()
+    chunks = (K + tk - 1) // tk
+    rng = np.random.default_rng(1)
+    for _ in range(100):
+        k, n = int(rng.integers(K)), int(rng.integers(N))
+        lane = ((k % tk) // 16) * tn + n % tn
+        off = (((n // tn) * chunks + k // tk) * 64 + lane) * 16 + k % 16
+        assert ph[off] == qh[k, n]
+    # GEMV over the narrow tiles, plain and accumulating
+    s = torch.rand(N, generator=g, device="cuda") * 1e-3 + 1e-4
+    x = torch.randn((1, K), generator=g, device="cuda")
+    c0 = torch.randn((1, N), generator=g, device="cuda")
+    y = torch.empty((1, N), device="cuda")
+    c = c0.clone()
+    torch.cuda.synchronize()
+    ops.linear_w8a32(A=x, lda=K, W0=p, scale0=s, C=y, ldc=N, M=1, K=K, N=N, epilogue=0, tile_n=tn)
+    ops.linear_w8a32(A=x, lda=K, W0=p, scale0=s, C=c, ldc=N, M=1, K=K, N=N, epilogue=1, tile_n=tn)
+    torch.cuda.synchronize()
+    xh, sh = x.cpu().numpy()[0], s.cpu().numpy()
+    check_close(y.cpu().numpy()[0], oracle.dequant_gemv(xh, qh, sh))
+    check_close(c.cpu().numpy()[0], oracle.dequant_gemv(xh, qh, sh, c0.cpu().numpy()[0]))
+
+
 SHAPES = [(1536, 8960), (8960, 1536), (1536, 1536), (1536, 256), (64, 16), (100, 70),
           (1536, 151936), (4096, 4096)]
 
