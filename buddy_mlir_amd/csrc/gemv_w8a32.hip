@@ -5,23 +5,26 @@
 // :250-321 generates (parallel over 32-wide n panels, sequential k, scale
 // applied once after the reduction, result added to C).
 //
-// The kernel is HBM-bound, so its shape follows the memory system:
+// The kernels are HBM-bound, so their shape follows the memory system:
 //  * weights live in 1 KiB wave tiles (16 channels x 64 k); one wavefront
 //    streams a contiguous run of tiles of one channel group with 128-bit
-//    loads, 1 KiB per instruction, the next batch of loads in flight while the
-//    current one is consumed;
+//    loads, 1 KiB per instruction, several tiles in flight;
 //  * a workgroup is G channel groups x KS k-slices of wavefronts.  Wide
 //    matrices (lm_head) use G=4, KS=1; narrow ones (down/o_proj) put up to 16
 //    wavefronts on one channel group so that 96 groups still keep ~1500
 //    wavefronts streaming.  The k-slices meet in LDS, in slice order, so the
 //    sum is deterministic and no workgroup ever waits for another one (cross-
 //    XCD traffic inside a kernel costs an L2 write-back on this part);
-//  * every wavefront stages its own slice of the activations in LDS
-//    (optionally multiplied by the RMSNorm weight, with the row's sum of
-//    squares gathered on the way; the common rsqrt factor is applied to the
-//    finished sums);
+//  * activations never pass through LDS: a lane loads the one activation whose
+//    k equals its position in the tile and the multiply-add reads its
+//    neighbours' values through DPP row broadcasts (gemv_w8a32_bcast_kernel).
+//    RMSNorm is fused in (weight multiplied while consuming, the row's sum of
+//    squares gathered on the way, the common rsqrt factor applied to the
+//    finished sums), as is folding the attention partials (o_proj);
 //  * scale, bias, residual add and SiLU*up are applied to the finished sums in
-//    the same kernel.
+//    the same kernel; their operands are requested before the stream starts.
+// The 8- and 4-channel tile layouts keep the older kernel that stages the
+// activations in LDS (gemv_w8a32_kernel).
 // No MFMA: at M = 1 the arithmetic is far below the bandwidth ridge.
 #include "gemv_w8a32.h"
 
@@ -42,7 +45,6 @@ struct GemvPlan {
   int64_t chunks, groups;
   int G, KS, waves, tiles_per_round, blocks;
   size_t lds_bytes;
-  bool deep; // >= 16 tiles per wavefront: worth eight loads in flight
 };
 
 int target_waves() {
@@ -88,7 +90,6 @@ GemvPlan make_plan(int64_t M, int64_t K, int64_t N, bool dual, int tn) {
     cap = 4;
   p.tiles_per_round = (int)(tiles < cap ? round_up(tiles, 4) : cap);
   p.lds_bytes = round_bytes(p.waves, p.tiles_per_round) + red_bytes(p.waves);
-  p.deep = tiles >= 16;
   return p;
 }
 
@@ -153,18 +154,27 @@ __device__ __forceinline__ float silu(float g) {
   return g * sig;
 }
 
-template <int EPI>
-__device__ __forceinline__ void finish(const KernelArgs &a, int m, int n,
-                                       float raw0, float raw1) {
+// Per-channel operands of the epilogue.  They are fetched when the kernel
+// starts, so that their memory latency is hidden behind the weight stream
+// instead of following the reduction.
+template <int M>
+struct EpilogueOperands {
+  float s0, s1, bias;
+  float c[M];
+};
+
+template <int M, int EPI>
+__device__ __forceinline__ void finish(const KernelArgs &a, int m, int n, float raw0,
+                                       float raw1, const EpilogueOperands<M> &e) {
   float *c = a.C + (int64_t)m * a.ldc + n;
-  float v = raw0 * a.s0[n];
+  const float v = raw0 * e.s0;
   if (EPI == kEpiSiluMul) {
-    const float u = raw1 * a.s1[n];
+    const float u = raw1 * e.s1;
     *c = silu(v) * u;
   } else if (EPI == kEpiAccum) {
-    *c = *c + v;
+    *c = e.c[m] + v;
   } else {
-    *c = a.bias ? a.bias[n] + v : v;
+    *c = a.bias ? e.bias + v : v;
   }
 }
 
@@ -262,6 +272,10 @@ __global__ void __launch_bounds__(kMaxWaves *kWave)
   const int st_off = (lane >> 2) * kXStride + (lane & 3) * 4;
   const float *xl = xs + (lane / TN) * kXStride; // this lane's k sub-range
 
+  const int n = g * TN + lane;
+  const bool writer = ks == 0 && lane < TN && live && n < a.N;
+  EpilogueOperands<M> epi;
+
   const int nrounds = (per + TR - 1) / TR; // same for every wavefront
   const int kend = min(a.K, t1 * TK);       // this wavefront's k range ends here
   for (int rd = 0; rd < nrounds; ++rd) {
@@ -277,6 +291,19 @@ __global__ void __launch_bounds__(kMaxWaves *kWave)
           if (DUAL)
             wb[u] = load_stream(w1 + (size_t)(r0 + u) * 64);
         }
+      }
+    }
+    if (rd == 0 && writer) {
+      epi.s0 = a.s0[n];
+      if (DUAL)
+        epi.s1 = a.s1[n];
+      if (EPI == kEpiStore && a.bias)
+        epi.bias = a.bias[n];
+      if (EPI == kEpiAccum) {
+#pragma unroll
+        for (int m = 0; m < M; ++m)
+          if (m < a.rows)
+            epi.c[m] = a.C[(int64_t)m * a.ldc + n];
       }
     }
     // ---- stage this wavefront's slice of the activations -----------------
@@ -408,8 +435,7 @@ __global__ void __launch_bounds__(kMaxWaves *kWave)
       }
     }
   }
-  const int n = g * TN + lane;
-  if (lane < TN && live && n < a.N) {
+  if (writer) {
 #pragma unroll
     for (int m = 0; m < M; ++m) {
       if (m < a.rows) {
@@ -422,10 +448,345 @@ __global__ void __launch_bounds__(kMaxWaves *kWave)
           v0 *= r;
           v1 *= r;
         }
-        finish<EPI>(a, m, n, v0, v1);
+        finish<M, EPI>(a, m, n, v0, v1, epi);
       }
     }
   }
+}
+
+
+// ---------------------------------------------------------------------------
+// 16-channel tiles: activations stay in registers.
+//
+// In a 16 x 64 tile the 16 lanes of a DPP row (lanes 16r .. 16r+15) hold 16
+// different channels of the same 16 k values, k = 64c + 16r + j.  A lane that
+// loads x[64c + lane] therefore holds, for its row, exactly the 16 activations
+// the row needs, and `v_fmac_f32 ... row_newbcast:j` multiplies every lane's
+// j-th weight with the activation held by lane j of its own row.  No LDS
+// staging, no barrier before the stream, and the VALU issues two instructions
+// per weight (SDWA convert + DPP multiply-add) and nothing else.
+// ---------------------------------------------------------------------------
+
+// acc += sum_j x(lane j of this row) * (float)(int8 byte j of w), bytes in the
+// order x, y, z, w of the 16-byte word.  Convert and multiply-add are
+// interleaved over four rotating temporaries so that a tile in flight costs
+// four registers, not sixteen.  The leading wait states cover a preceding VALU
+// write of x (2) or of EXEC (5) before the first DPP read.
+__device__ __forceinline__ void fma_tile_row_bcast(float &acc, float x, const int4 &w) {
+  float t0, t1, t2, t3;
+  asm volatile(
+      "s_nop 4\n\t"
+      "v_cvt_f32_i32_sdwa %1, sext(%6) dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:BYTE_0\n\t"
+      "v_cvt_f32_i32_sdwa %2, sext(%6) dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:BYTE_1\n\t"
+      "v_cvt_f32_i32_sdwa %3, sext(%6) dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:BYTE_2\n\t"
+      "v_cvt_f32_i32_sdwa %4, sext(%6) dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:BYTE_3\n\t"
+      "v_fmac_f32_dpp %0, %5, %1 row_newbcast:0 row_mask:0xf bank_mask:0xf\n\t"
+      "v_cvt_f32_i32_sdwa %1, sext(%7) dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:BYTE_0\n\t"
+      "v_fmac_f32_dpp %0, %5, %2 row_newbcast:1 row_mask:0xf bank_mask:0xf\n\t"
+      "v_cvt_f32_i32_sdwa %2, sext(%7) dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:BYTE_1\n\t"
+      "v_fmac_f32_dpp %0, %5, %3 row_newbcast:2 row_mask:0xf bank_mask:0xf\n\t"
+      "v_cvt_f32_i32_sdwa %3, sext(%7) dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:BYTE_2\n\t"
+      "v_fmac_f32_dpp %0, %5, %4 row_newbcast:3 row_mask:0xf bank_mask:0xf\n\t"
+      "v_cvt_f32_i32_sdwa %4, sext(%7) dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:BYTE_3\n\t"
+      "v_fmac_f32_dpp %0, %5, %1 row_newbcast:4 row_mask:0xf bank_mask:0xf\n\t"
+      "v_cvt_f32_i32_sdwa %1, sext(%8) dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:BYTE_0\n\t"
+      "v_fmac_f32_dpp %0, %5, %2 row_newbcast:5 row_mask:0xf bank_mask:0xf\n\t"
+      "v_cvt_f32_i32_sdwa %2, sext(%8) dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:BYTE_1\n\t"
+      "v_fmac_f32_dpp %0, %5, %3 row_newbcast:6 row_mask:0xf bank_mask:0xf\n\t"
+      "v_cvt_f32_i32_sdwa %3, sext(%8) dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:BYTE_2\n\t"
+      "v_fmac_f32_dpp %0, %5, %4 row_newbcast:7 row_mask:0xf bank_mask:0xf\n\t"
+      "v_cvt_f32_i32_sdwa %4, sext(%8) dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:BYTE_3\n\t"
+      "v_fmac_f32_dpp %0, %5, %1 row_newbcast:8 row_mask:0xf bank_mask:0xf\n\t"
+      "v_cvt_f32_i32_sdwa %1, sext(%9) dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:BYTE_0\n\t"
+      "v_fmac_f32_dpp %0, %5, %2 row_newbcast:9 row_mask:0xf bank_mask:0xf\n\t"
+      "v_cvt_f32_i32_sdwa %2, sext(%9) dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:BYTE_1\n\t"
+      "v_fmac_f32_dpp %0, %5, %3 row_newbcast:10 row_mask:0xf bank_mask:0xf\n\t"
+      "v_cvt_f32_i32_sdwa %3, sext(%9) dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:BYTE_2\n\t"
+      "v_fmac_f32_dpp %0, %5, %4 row_newbcast:11 row_mask:0xf bank_mask:0xf\n\t"
+      "v_cvt_f32_i32_sdwa %4, sext(%9) dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:BYTE_3\n\t"
+      "v_fmac_f32_dpp %0, %5, %1 row_newbcast:12 row_mask:0xf bank_mask:0xf\n\t"
+      "v_fmac_f32_dpp %0, %5, %2 row_newbcast:13 row_mask:0xf bank_mask:0xf\n\t"
+      "v_fmac_f32_dpp %0, %5, %3 row_newbcast:14 row_mask:0xf bank_mask:0xf\n\t"
+      "v_fmac_f32_dpp %0, %5, %4 row_newbcast:15 row_mask:0xf bank_mask:0xf"
+      : "+v"(acc), "=&v"(t0), "=&v"(t1), "=&v"(t2), "=&v"(t3)
+      : "v"(x), "v"(w.x), "v"(w.y), "v"(w.z), "v"(w.w));
+}
+
+// acc[m] += ... for M rows that share the converted weights.
+__device__ __forceinline__ void fma16_row_bcast(float &acc, float x,
+                                                const float (&w)[16]) {
+  asm volatile(
+      "s_nop 4\n\t"
+      "v_fmac_f32_dpp %0, %1, %2 row_newbcast:0 row_mask:0xf bank_mask:0xf\n\t"
+      "v_fmac_f32_dpp %0, %1, %3 row_newbcast:1 row_mask:0xf bank_mask:0xf\n\t"
+      "v_fmac_f32_dpp %0, %1, %4 row_newbcast:2 row_mask:0xf bank_mask:0xf\n\t"
+      "v_fmac_f32_dpp %0, %1, %5 row_newbcast:3 row_mask:0xf bank_mask:0xf\n\t"
+      "v_fmac_f32_dpp %0, %1, %6 row_newbcast:4 row_mask:0xf bank_mask:0xf\n\t"
+      "v_fmac_f32_dpp %0, %1, %7 row_newbcast:5 row_mask:0xf bank_mask:0xf\n\t"
+      "v_fmac_f32_dpp %0, %1, %8 row_newbcast:6 row_mask:0xf bank_mask:0xf\n\t"
+      "v_fmac_f32_dpp %0, %1, %9 row_newbcast:7 row_mask:0xf bank_mask:0xf\n\t"
+      "v_fmac_f32_dpp %0, %1, %10 row_newbcast:8 row_mask:0xf bank_mask:0xf\n\t"
+      "v_fmac_f32_dpp %0, %1, %11 row_newbcast:9 row_mask:0xf bank_mask:0xf\n\t"
+      "v_fmac_f32_dpp %0, %1, %12 row_newbcast:10 row_mask:0xf bank_mask:0xf\n\t"
+      "v_fmac_f32_dpp %0, %1, %13 row_newbcast:11 row_mask:0xf bank_mask:0xf\n\t"
+      "v_fmac_f32_dpp %0, %1, %14 row_newbcast:12 row_mask:0xf bank_mask:0xf\n\t"
+      "v_fmac_f32_dpp %0, %1, %15 row_newbcast:13 row_mask:0xf bank_mask:0xf\n\t"
+      "v_fmac_f32_dpp %0, %1, %16 row_newbcast:14 row_mask:0xf bank_mask:0xf\n\t"
+      "v_fmac_f32_dpp %0, %1, %17 row_newbcast:15 row_mask:0xf bank_mask:0xf"
+      : "+v"(acc)
+      : "v"(x), "v"(w[0]), "v"(w[1]), "v"(w[2]), "v"(w[3]), "v"(w[4]), "v"(w[5]),
+        "v"(w[6]), "v"(w[7]), "v"(w[8]), "v"(w[9]), "v"(w[10]), "v"(w[11]),
+        "v"(w[12]), "v"(w[13]), "v"(w[14]), "v"(w[15]));
+}
+
+__device__ __forceinline__ void tile_to_float(const int4 &w, float (&wf)[16]) {
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    wf[j] = byte_to_float(w.x, j);
+    wf[4 + j] = byte_to_float(w.y, j);
+    wf[8 + j] = byte_to_float(w.z, j);
+    wf[12 + j] = byte_to_float(w.w, j);
+  }
+}
+
+// Combined attention output for one k (see attn_combined): the chunk weights
+// are common to the wavefront (one tile lies inside one head).
+__device__ __forceinline__ float attn_combined_one(const KernelArgs &a, int k) {
+  constexpr int B = 9;
+  const int h = __builtin_amdgcn_readfirstlane(k / a.head_dim), d = k % a.head_dim;
+  const int used = a.attn_nchunks;
+  const float2 *ml = reinterpret_cast<const float2 *>(a.attn_ml) +
+                     (size_t)h * a.attn_nchunks;
+  const float *acc = a.attn_acc + (size_t)h * a.attn_nchunks * a.head_dim + d;
+  float r = 0.f, m = -1.0e30f, l = 0.f;
+  for (int s0 = 0; s0 < used; s0 += B) {
+    float2 mlv[B];
+    float v[B];
+#pragma unroll
+    for (int j = 0; j < B; ++j) {
+      const int s = min(s0 + j, used - 1);
+      mlv[j] = ml[s];
+      v[j] = acc[(size_t)s * a.head_dim];
+    }
+    float mb = m;
+#pragma unroll
+    for (int j = 0; j < B; ++j)
+      if (s0 + j < used)
+        mb = fmaxf(mb, mlv[j].x);
+    const float al = expf(m - mb);
+    r *= al;
+    l *= al;
+    m = mb;
+#pragma unroll
+    for (int j = 0; j < B; ++j) {
+      if (s0 + j < used) {
+        const float w = expf(mlv[j].x - m);
+        l = fmaf(mlv[j].y, w, l);
+        r = fmaf(v[j], w, r);
+      }
+    }
+  }
+  return r * (1.0f / l);
+}
+
+// One tile's worth of operands of one wavefront.
+template <int M> struct TileOperands {
+  int4 w0, w1;
+  float x[M];
+  float nw;
+};
+
+template <int M, int PRO, bool DUAL>
+__device__ __forceinline__ void fetch_tile(const KernelArgs &a, const int4 *w0,
+                                           const int4 *w1, int t, int lane,
+                                           TileOperands<M> &o) {
+  o.w0 = load_stream(w0 + (size_t)t * 64);
+  if (DUAL)
+    o.w1 = load_stream(w1 + (size_t)t * 64);
+  // out-of-range lanes and rows read a valid address; the value is dropped when
+  // the tile is consumed.  Branch-free loads whose results are not touched here
+  // let the compiler keep an exact count of the loads in flight.
+  const int k = t * kTileK + lane;
+  const int kc = k < a.K ? k : a.K - 1;
+  if (PRO == kProNorm)
+    o.nw = a.norm_w[kc];
+#pragma unroll
+  for (int m = 0; m < M; ++m) {
+    if (PRO == kProAttn) {
+      o.x[m] = (m == 0 && k < a.K) ? attn_combined_one(a, k) : 0.f;
+    } else {
+      const int mc = m < a.rows ? m : a.rows - 1;
+      o.x[m] = a.A[(int64_t)mc * a.lda + kc];
+    }
+  }
+}
+
+// ONE: every wavefront's run of tiles fits in U, so all its loads go out at
+// once and nothing is double-buffered.
+template <int M, int EPI, int PRO, int U, bool ONE>
+__global__ void __launch_bounds__(kMaxWaves *kWave)
+    gemv_w8a32_bcast_kernel(KernelArgs a) {
+  constexpr bool DUAL = (EPI == kEpiSiluMul);
+  constexpr bool NORM = (PRO == kProNorm);
+  extern __shared__ float lds[]; // only the meeting place of the k-slices
+  const int tid = threadIdx.x;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+  const int gl = wave / a.KS, ks = wave % a.KS;
+  const int g = blockIdx.x * a.G + gl;
+  const bool live = g < a.groups;
+  const int per = (a.chunks + a.KS - 1) / a.KS;
+  const int t0 = min(ks * per, a.chunks);
+  const int t1 = min(t0 + per, a.chunks);
+
+  float acc0[M], acc1[M], ss[M];
+#pragma unroll
+  for (int m = 0; m < M; ++m) {
+    acc0[m] = 0.f;
+    acc1[m] = 0.f;
+    ss[m] = 0.f;
+  }
+  const size_t wbase = ((size_t)(live ? g : 0) * a.chunks) * 64 + lane;
+  const int4 *w0 = a.W0 + wbase;
+  const int4 *w1 = DUAL ? a.W1 + wbase : a.W0 + wbase;
+
+  // a ring of U tiles in flight: a slot is refilled as soon as it is consumed
+  TileOperands<M> slot[U];
+#pragma unroll
+  for (int u = 0; u < U; ++u)
+    if (t0 + u < t1)
+      fetch_tile<M, PRO, DUAL>(a, w0, w1, t0 + u, lane, slot[u]);
+
+  const int n = g * kTileN + lane;
+  const bool writer = ks == 0 && lane < kTileN && live && n < a.N;
+  EpilogueOperands<M> epi;
+  if (writer) {
+    epi.s0 = a.s0[n];
+    if (DUAL)
+      epi.s1 = a.s1[n];
+    if (EPI == kEpiStore && a.bias)
+      epi.bias = a.bias[n];
+    if (EPI == kEpiAccum) {
+#pragma unroll
+      for (int m = 0; m < M; ++m)
+        if (m < a.rows)
+          epi.c[m] = a.C[(int64_t)m * a.ldc + n];
+    }
+  }
+
+  for (int t = t0; t < (ONE ? min(t1, t0 + 1) : t1); t += U) {
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      if (t + u < t1) {
+        const TileOperands<M> &o = slot[u];
+        const bool in = (t + u) * kTileK + lane < a.K;
+        if (M == 1) {
+          float x = in ? o.x[0] : 0.f;
+          if (NORM) {
+            ss[0] = fmaf(x, x, ss[0]);
+            x *= o.nw;
+          }
+          fma_tile_row_bcast(acc0[0], x, o.w0);
+          if (DUAL)
+            fma_tile_row_bcast(acc1[0], x, o.w1);
+        } else {
+          float wf0[16], wf1[16];
+          tile_to_float(o.w0, wf0);
+          if (DUAL)
+            tile_to_float(o.w1, wf1);
+#pragma unroll
+          for (int m = 0; m < M; ++m) {
+            float x = (in && m < a.rows) ? o.x[m] : 0.f;
+            if (NORM) {
+              ss[m] = fmaf(x, x, ss[m]);
+              x *= o.nw;
+            }
+            fma16_row_bcast(acc0[m], x, wf0);
+            if (DUAL)
+              fma16_row_bcast(acc1[m], x, wf1);
+          }
+        }
+        if (!ONE && t + U + u < t1)
+          fetch_tile<M, PRO, DUAL>(a, w0, w1, t + U + u, lane, slot[u]);
+      }
+    }
+  }
+
+  // the four rows of a wavefront hold different k sub-ranges of the same channels
+#pragma unroll
+  for (int m = 0; m < M; ++m) {
+    acc0[m] += __shfl_xor(acc0[m], 16, 64);
+    acc0[m] += __shfl_xor(acc0[m], 32, 64);
+    if (DUAL) {
+      acc1[m] += __shfl_xor(acc1[m], 16, 64);
+      acc1[m] += __shfl_xor(acc1[m], 32, 64);
+    }
+    if (NORM)
+      ss[m] = wave_sum(ss[m]);
+  }
+
+  // ---- k-slices of one channel group meet in LDS, in slice order ----------
+  if (a.KS > 1) {
+    float *mine = lds + (size_t)wave * M * 33;
+    if (lane < kTileN) {
+#pragma unroll
+      for (int m = 0; m < M; ++m) {
+        mine[m * 33 + lane] = acc0[m];
+        if (DUAL)
+          mine[m * 33 + 16 + lane] = acc1[m];
+      }
+    }
+    if (NORM && lane == 0) {
+#pragma unroll
+      for (int m = 0; m < M; ++m)
+        mine[m * 33 + 32] = ss[m];
+    }
+    __syncthreads();
+    if (ks != 0)
+      return;
+    if (lane < kTileN) {
+#pragma unroll
+      for (int m = 0; m < M; ++m) {
+        float r0 = 0.f, r1 = 0.f, rs = 0.f;
+        for (int s = 0; s < a.KS; ++s) {
+          const float *o = lds + (size_t)(wave + s) * M * 33 + m * 33;
+          r0 += o[lane];
+          if (DUAL)
+            r1 += o[16 + lane];
+          if (NORM)
+            rs += o[32];
+        }
+        acc0[m] = r0;
+        acc1[m] = r1;
+        ss[m] = rs;
+      }
+    }
+  }
+  if (writer) {
+#pragma unroll
+    for (int m = 0; m < M; ++m) {
+      if (m < a.rows) {
+        float v0 = acc0[m], v1 = acc1[m];
+        if (NORM) {
+          // x' = w (.) (x * r) with r = rsqrt(mean(x^2) + eps): r is common to
+          // the whole row, so it multiplies the finished sum
+          // (subgraph0_decode_simplify.mlir:60-72)
+          const float r = 1.0f / sqrtf(ss[m] * a.norm_inv_k + a.norm_eps);
+          v0 *= r;
+          v1 *= r;
+        }
+        finish<M, EPI>(a, m, n, v0, v1, epi);
+      }
+    }
+  }
+}
+
+template <int M, int EPI, int PRO, int U, bool ONE>
+int launch_bcast(const KernelArgs &ka, const GemvPlan &p, hipStream_t stream) {
+  auto kernel = gemv_w8a32_bcast_kernel<M, EPI, PRO, U, ONE>;
+  hipLaunchKernelGGL(kernel, dim3(p.blocks), dim3(p.waves * kWave),
+                     sizeof(float) * p.waves * (size_t)M * 33, stream, ka);
+  BH_CHECK_HIP(hipGetLastError());
+  return BUDDY_HIP_OK;
 }
 
 template <int M, int EPI, int PRO, int U, int TN>
@@ -444,27 +805,32 @@ int launch_tn(const KernelArgs &ka, const GemvPlan &p, hipStream_t stream) {
   return BUDDY_HIP_OK;
 }
 
-// Narrow tiles (8 or 4 channels) exist for one-row launches of narrow matrices.
-template <int M, int EPI, int PRO, int U>
-int launch_u(const KernelArgs &ka, const GemvPlan &p, hipStream_t stream) {
-  if (M == 1 && EPI != kEpiSiluMul) {
-    if (ka.tile_n == 8)
-      return launch_tn<M, EPI, PRO, U, (M == 1 && EPI != kEpiSiluMul) ? 8 : 16>(ka, p, stream);
-    if (ka.tile_n == 4)
-      return launch_tn<M, EPI, PRO, U, (M == 1 && EPI != kEpiSiluMul) ? 4 : 16>(ka, p, stream);
-  }
-  if (ka.tile_n != 16)
-    return fail(BUDDY_HIP_ERR_ARG, "gemv: %d-channel tiles need M = 1 and one matrix",
-                ka.tile_n);
-  return launch_tn<M, EPI, PRO, U, 16>(ka, p, stream);
-}
-
+// 16-channel tiles run on the register-resident kernel; the 8- and 4-channel
+// layouts (one row, one matrix) on the LDS-staged one.
 template <int M, int EPI, int PRO>
 int launch_one(const KernelArgs &ka, const GemvPlan &p, hipStream_t stream) {
-  // long single-row, single-matrix streams keep eight tiles in flight
-  if (M == 1 && EPI != kEpiSiluMul && PRO != kProAttn && p.deep)
-    return launch_u<M, EPI, PRO, (M == 1 && EPI != kEpiSiluMul && PRO != kProAttn) ? 8 : 4>(ka, p, stream);
-  return launch_u<M, EPI, PRO, 4>(ka, p, stream);
+  constexpr bool kDual = EPI == kEpiSiluMul;
+  if (ka.tile_n != 16) {
+    constexpr bool kNarrowOk = M == 1 && !kDual;
+    if (!kNarrowOk)
+      return fail(BUDDY_HIP_ERR_ARG, "gemv: %d-channel tiles need M = 1 and one matrix",
+                  ka.tile_n);
+    if (ka.tile_n == 8)
+      return launch_tn<kNarrowOk ? 1 : M, kNarrowOk ? EPI : kEpiStore, PRO, 4, kNarrowOk ? 8 : 16>(ka, p, stream);
+    return launch_tn<kNarrowOk ? 1 : M, kNarrowOk ? EPI : kEpiStore, PRO, 4, kNarrowOk ? 4 : 16>(ka, p, stream);
+  }
+  if (M == 1) {
+    // short runs: every tile of a wavefront is requested at once
+    const int64_t tpw = ceil_div(p.chunks, p.KS); // tiles per wavefront
+    if (tpw <= 4)
+      return launch_bcast<1, EPI, PRO, 4, true>(ka, p, stream);
+    if (tpw <= 6)
+      return launch_bcast<1, EPI, PRO, 6, true>(ka, p, stream);
+    if (!kDual && tpw <= 9)
+      return launch_bcast<1, EPI, PRO, kDual ? 6 : 9, true>(ka, p, stream);
+  }
+  constexpr int kRing = M == 1 ? (kDual ? 6 : 8) : M <= 4 ? 4 : M == 8 ? 2 : 1;
+  return launch_bcast<M, EPI, PRO, kRing, false>(ka, p, stream);
 }
 
 template <int M>

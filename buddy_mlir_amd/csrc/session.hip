@@ -41,8 +41,6 @@ int launch_matmul_f32(const float *A, const float *B, float *C, int64_t M,
 
 namespace {
 
-constexpr int kNarrowTile = 8;
-
 struct PackedLinear {
   int8_t *w = nullptr; // wave tiles
   float *s = nullptr;  // scales
@@ -56,10 +54,6 @@ struct Layer {
   // the reference's shipped w8a32 build keeps q/k/v in f32 with a bias
   // (they import as AddMMOp, which the quantizer does not touch):
   float *qkv_f32 = nullptr; // [hidden, q|k|v] dense, or null when int8
-  // down_proj has only hidden/16 channel groups (96 at 1536), fewer than the
-  // CUs: the decode step reads a second copy packed in 8-channel tiles, the
-  // prefill matmul the 16-channel one
-  int8_t *down_narrow = nullptr;
   float *kc = nullptr, *vc = nullptr; // [kv_heads, max_len, D]
   bool set = false;
 };
@@ -153,12 +147,11 @@ struct Session {
   }
 
   int gemv(const float *A, const PackedLinear &W0, const PackedLinear *W1,
-           const float *norm_w, float *C, int epi, const int8_t *narrow = nullptr) {
+           const float *norm_w, float *C, int epi) {
     GemvArgs g;
     g.A = A;
     g.lda = W0.K;
-    g.W0 = narrow ? narrow : W0.w;
-    g.tile_n = narrow ? kNarrowTile : 16;
+    g.W0 = W0.w;
     g.s0 = W0.s;
     if (W1) {
       g.W1 = W1->w;
@@ -236,7 +229,7 @@ struct Session {
       }
       if ((rc = gemv(x, L.gate, &L.up, L.ln2, h, kEpiSiluMul)))
         return rc;
-      if ((rc = gemv(h, L.down, nullptr, nullptr, x, kEpiAccum, L.down_narrow)))
+      if ((rc = gemv(h, L.down, nullptr, nullptr, x, kEpiAccum)))
         return rc;
     }
     if ((rc = gemv(x, lm, nullptr, ln_f, logits, kEpiStore)))
@@ -570,8 +563,6 @@ int buddy_hip_session_set_layer(buddy_hip_session *hs, int index,
       rc |= s->alloc(&P->w, buddy_hip_w8_packed_bytes(P->K, P->N));
       rc |= s->alloc(&P->s, (size_t)P->N);
     }
-    rc |= s->alloc(&L.down_narrow,
-                   buddy_hip_w8_packed_bytes_tiles(I, H, bh::kNarrowTile));
     if (rc)
       return rc;
   }
@@ -602,7 +593,6 @@ int buddy_hip_session_set_layer(buddy_hip_session *hs, int index,
   rc |= s->pack_into(w->wg, w->sg, nullptr, H, I, L.gate.w, L.gate.s, nullptr);
   rc |= s->pack_into(w->wu, w->su, nullptr, H, I, L.up.w, L.up.s, nullptr);
   rc |= s->pack_into(w->wd, w->sd, nullptr, I, H, L.down.w, L.down.s, nullptr);
-  rc |= buddy_hip_pack_w8_tiles(w->wd, I, H, bh::kNarrowTile, L.down_narrow, s->stream);
   if (rc)
     return rc;
   BH_CHECK_HIP(hipMemcpyAsync(L.ln1, w->ln1, sizeof(float) * H, hipMemcpyDefault, s->stream));
