@@ -549,44 +549,63 @@ __device__ __forceinline__ void tile_to_float(const int4 &w, float (&wf)[16]) {
   }
 }
 
-// Combined attention output for one k (see attn_combined): the chunk weights
-// are common to the wavefront (one tile lies inside one head).
-__device__ __forceinline__ float attn_combined_one(const KernelArgs &a, int k) {
-  constexpr int B = 9;
-  const int h = __builtin_amdgcn_readfirstlane(k / a.head_dim), d = k % a.head_dim;
+// Combined attention output (see attn_combined) for the k = 64 t + lane of U
+// consecutive tiles of a wavefront.  A tile lies inside one head, so the chunk
+// weights exp(m_s - max m) are common to the wavefront: lane s computes the
+// weight of chunk s (one exp for up to 64 chunks) and the sum over the chunks
+// reads it from there.  The partials of all U tiles are requested together, 18
+// chunks at a time.
+template <int U>
+__device__ __forceinline__ void attn_fold_tiles(const KernelArgs &a, int t0, int t1,
+                                                int lane, float (&x)[U]) {
+  constexpr int B = 18;
   const int used = a.attn_nchunks;
-  const float2 *ml = reinterpret_cast<const float2 *>(a.attn_ml) +
-                     (size_t)h * a.attn_nchunks;
-  const float *acc = a.attn_acc + (size_t)h * a.attn_nchunks * a.head_dim + d;
-  float r = 0.f, m = -1.0e30f, l = 0.f;
-  for (int s0 = 0; s0 < used; s0 += B) {
-    float2 mlv[B];
-    float v[B];
+  const float2 *ml[U];
+  const float *acc[U];
+  float r[U], m[U], l[U];
 #pragma unroll
-    for (int j = 0; j < B; ++j) {
-      const int s = min(s0 + j, used - 1);
-      mlv[j] = ml[s];
-      v[j] = acc[(size_t)s * a.head_dim];
+  for (int u = 0; u < U; ++u) {
+    const int t = min(t0 + u, t1 - 1); // slots past the run repeat its last tile
+    const int k = min(t * kTileK + lane, a.K - 1);
+    const int h = __builtin_amdgcn_readfirstlane(k / a.head_dim), d = k % a.head_dim;
+    ml[u] = reinterpret_cast<const float2 *>(a.attn_ml) + (size_t)h * a.attn_nchunks;
+    acc[u] = a.attn_acc + (size_t)h * a.attn_nchunks * a.head_dim + d;
+    r[u] = 0.f;
+    m[u] = -1.0e30f;
+    l[u] = 0.f;
+  }
+  for (int c0 = 0; c0 < used; c0 += kWave) { // 64 chunks per pass
+    const int cnt = min(kWave, used - c0);
+    float w[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const float2 mine = ml[u][c0 + min(lane, cnt - 1)];
+      const bool valid = lane < cnt;
+      const float mb = fmaxf(m[u], wave_max(valid ? mine.x : -1.0e30f));
+      const float al = expf(m[u] - mb); // rescale what earlier passes gathered
+      w[u] = valid ? expf(mine.x - mb) : 0.f;
+      l[u] = fmaf(l[u], al, wave_sum(mine.y * w[u]));
+      r[u] *= al;
+      m[u] = mb;
     }
-    float mb = m;
+    for (int s0 = 0; s0 < cnt; s0 += B) {
+      float v[U][B];
 #pragma unroll
-    for (int j = 0; j < B; ++j)
-      if (s0 + j < used)
-        mb = fmaxf(mb, mlv[j].x);
-    const float al = expf(m - mb);
-    r *= al;
-    l *= al;
-    m = mb;
+      for (int u = 0; u < U; ++u)
 #pragma unroll
-    for (int j = 0; j < B; ++j) {
-      if (s0 + j < used) {
-        const float w = expf(mlv[j].x - m);
-        l = fmaf(mlv[j].y, w, l);
-        r = fmaf(v[j], w, r);
-      }
+        for (int j = 0; j < B; ++j)
+          v[u][j] = acc[u][(size_t)(c0 + min(s0 + j, cnt - 1)) * a.head_dim];
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+#pragma unroll
+        for (int j = 0; j < B; ++j)
+          if (s0 + j < cnt)
+            r[u] = fmaf(v[u][j], lane_f(w[u], s0 + j), r[u]);
     }
   }
-  return r * (1.0f / l);
+#pragma unroll
+  for (int u = 0; u < U; ++u)
+    x[u] = r[u] * (1.0f / l[u]);
 }
 
 // One tile's worth of operands of one wavefront.
@@ -596,7 +615,7 @@ template <int M> struct TileOperands {
   float nw;
 };
 
-template <int M, int PRO, bool DUAL>
+template <int M, int PRO, bool DUAL, bool FOLD_LATER = false>
 __device__ __forceinline__ void fetch_tile(const KernelArgs &a, const int4 *w0,
                                            const int4 *w1, int t, int lane,
                                            TileOperands<M> &o) {
@@ -613,7 +632,12 @@ __device__ __forceinline__ void fetch_tile(const KernelArgs &a, const int4 *w0,
 #pragma unroll
   for (int m = 0; m < M; ++m) {
     if (PRO == kProAttn) {
-      o.x[m] = (m == 0 && k < a.K) ? attn_combined_one(a, k) : 0.f;
+      if (!FOLD_LATER) {
+        float x1[1] = {0.f};
+        if (m == 0)
+          attn_fold_tiles<1>(a, t, t + 1, lane, x1);
+        o.x[m] = x1[0];
+      }
     } else {
       const int mc = m < a.rows ? m : a.rows - 1;
       o.x[m] = a.A[(int64_t)mc * a.lda + kc];
@@ -654,7 +678,22 @@ __global__ void __launch_bounds__(kMaxWaves *kWave)
 #pragma unroll
   for (int u = 0; u < U; ++u)
     if (t0 + u < t1)
-      fetch_tile<M, PRO, DUAL>(a, w0, w1, t0 + u, lane, slot[u]);
+      fetch_tile<M, PRO, DUAL, true>(a, w0, w1, t0 + u, lane, slot[u]);
+  if (PRO == kProAttn && t0 < t1) {
+    // four tiles per fold keep the partials of a batch in registers
+    float xf[(U + 3) / 4][4];
+#pragma unroll
+    for (int q = 0; q < (U + 3) / 4; ++q)
+      if (t0 + 4 * q < t1)
+        attn_fold_tiles<4>(a, t0 + 4 * q, t1, lane, xf[q]);
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      slot[u].x[0] = xf[u / 4][u % 4];
+#pragma unroll
+      for (int m = 1; m < M; ++m)
+        slot[u].x[m] = 0.f;
+    }
+  }
 
   const int n = g * kTileN + lane;
   const bool writer = ks == 0 && lane < kTileN && live && n < a.N;
