@@ -12,8 +12,10 @@
 // Differences from the reference kernel that follow from the hardware:
 //   * the cache is scanned up to pos only (masked positions contribute exactly
 //     zero in the reference, so skipping them changes nothing);
-//   * one workgroup serves all query heads of a KV head, so K and V rows are
-//     read once per group, not once per query head;
+//   * one workgroup serves one query head (the step is latency bound: many
+//     small workgroups beat few large ones), and the workgroups of the other
+//     query heads of the same KV head run on the same XCD, so K and V rows
+//     leave HBM once per group, not once per query head;
 //   * the k range is cut into chunks of 64 positions (more, smaller partials
 //     than the reference's 4): a decode step has only ~2 MB of KV per layer and
 //     is latency bound, so the chunks are what spreads it over the CUs.
@@ -28,6 +30,7 @@ namespace {
 constexpr int kChunk = kAttnChunk; // cache positions per workgroup
 constexpr int kThreads = 256;
 constexpr int kMaxGroup = 8;     // query heads per KV head
+constexpr int kHPB = 1;          // query heads per workgroup
 constexpr int kD = 128;          // head_dim this kernel is written for
 constexpr float kSeedM = -1.0e30f; // tosa.py:13971
 
@@ -42,21 +45,29 @@ struct AttnArgs {
   float *out;            // [heads*D]
   int heads, kv_heads, group, max_len, nchunks;
   float scale;
+  int pairs_padded; // (chunk, kv head) pairs rounded up to the XCD count
 };
 
+// One workgroup: 64 cache positions x kHPB query heads (one) of one KV head.  The
+// workgroups that share a chunk (different query heads, same K/V rows) get
+// linear ids that are equal modulo 8, so they run on the same XCD and the rows
+// come out of that XCD's L2 after the first of them has fetched them.
 __global__ void __launch_bounds__(kThreads) attn_decode_partial(AttnArgs a) {
-  __shared__ float q_s[kMaxGroup][kD];
+  __shared__ float q_s[kHPB][kD];
   __shared__ float knew_s[kD], vnew_s[kD];
-  __shared__ float cos_s[kD / 2], sin_s[kD / 2];
-  __shared__ float sc_s[kMaxGroup][kChunk];
-  __shared__ float red_s[kThreads / 32][kMaxGroup][kD];
-  __shared__ float m_s[kMaxGroup], l_s[kMaxGroup];
+  __shared__ float sc_s[kHPB][kChunk];
+  __shared__ float red_s[kThreads / 32][kHPB][kD];
+  __shared__ float m_s[kHPB], l_s[kHPB];
 
   const int tid = threadIdx.x;
-  const int chunk = blockIdx.x, kvh = blockIdx.y;
+  const int hb = blockIdx.x / a.pairs_padded, ckv = blockIdx.x % a.pairs_padded;
+  if (ckv >= a.nchunks * a.kv_heads)
+    return; // padding id
+  const int chunk = ckv % a.nchunks, kvh = ckv / a.nchunks;
   const int p0 = chunk * kChunk;
   const int G = a.group;
-  const int h0 = kvh * G;
+  const int nh = min(kHPB, G - hb * kHPB); // query heads of this workgroup
+  const int h0 = kvh * G + hb * kHPB;
 
   // ---- every load that does not need the position goes out first ----------
   // The cache rows of the chunk exist whatever the position is (rows beyond it
@@ -78,43 +89,35 @@ __global__ void __launch_bounds__(kThreads) attn_decode_partial(AttnArgs a) {
           a.vcache + ((size_t)kvh * a.max_len + vrow) * kD + vq * 4);
     }
   }
-  // raw q of the G heads (3 values per thread at G = 6), raw k and v of the token
-  float qraw[(kMaxGroup * kD + kThreads - 1) / kThreads], qpair[(kMaxGroup * kD + kThreads - 1) / kThreads];
-#pragma unroll
-  for (int r = 0; r < (kMaxGroup * kD + kThreads - 1) / kThreads; ++r) {
-    const int i = tid + r * kThreads;
-    qraw[r] = 0.f;
-    qpair[r] = 0.f;
-    if (i < G * kD) {
-      const int h = i / kD, j = i % kD;
-      const float *q = a.qkv + (size_t)(h0 + h) * kD;
-      qraw[r] = q[j];
-      qpair[r] = j < kD / 2 ? -q[j + kD / 2] : q[j - kD / 2];
-    }
+  // raw q of the workgroup's heads (one value per thread), raw k and v of the
+  // token; every thread rotates with the angle of its own j mod 64
+  const int qh = tid / kD, j = tid % kD, jj = j & (kD / 2 - 1);
+  float qraw = 0.f, qpair = 0.f;
+  if (qh < nh) {
+    const float *q = a.qkv + (size_t)(h0 + qh) * kD;
+    qraw = q[j];
+    qpair = j < kD / 2 ? -q[j + kD / 2] : q[j - kD / 2];
   }
   float kraw = 0.f, kpair = 0.f, vraw = 0.f;
   if (tid < kD) {
-    const int j = tid;
     const float *k = a.qkv + (size_t)a.heads * kD + (size_t)kvh * kD;
     kraw = k[j];
     kpair = j < kD / 2 ? -k[j + kD / 2] : k[j - kD / 2];
     vraw = k[(size_t)a.kv_heads * kD + j];
   }
-  float inv_f = 0.f, tab_c = 0.f, tab_s = 0.f;
-  if (tid < kD / 2) {
-    if (a.rope_table) {
-      tab_c = a.rope_table[tid];
-      tab_s = a.rope_table[kD / 2 + tid];
-    } else {
-      inv_f = a.inv_freq[tid];
-    }
+  float inv_f = 0.f, cs = 0.f, sn = 0.f;
+  if (a.rope_table) {
+    cs = a.rope_table[jj];
+    sn = a.rope_table[kD / 2 + jj];
+  } else {
+    inv_f = a.inv_freq[jj];
   }
   const int pos = *a.pos_ptr;
 
   if (p0 > pos) { // nothing visible in this chunk: an empty partial
-    for (int i = tid; i < G * kD; i += kThreads)
-      a.part_acc[((size_t)(h0 + i / kD) * a.nchunks + chunk) * kD + i % kD] = 0.f;
-    if (tid < G) {
+    if (qh < nh)
+      a.part_acc[((size_t)(h0 + qh) * a.nchunks + chunk) * kD + j] = 0.f;
+    if (tid < nh) {
       a.part_ml[((size_t)(h0 + tid) * a.nchunks + chunk) * 2 + 0] = kSeedM;
       a.part_ml[((size_t)(h0 + tid) * a.nchunks + chunk) * 2 + 1] = 0.f;
     }
@@ -124,40 +127,28 @@ __global__ void __launch_bounds__(kThreads) attn_decode_partial(AttnArgs a) {
   const int np = p1 - p0;
   const bool has_new = pos >= p0 && pos < p1;
 
-  // ---- RoPE tables for this position -------------------------------------
-  if (tid < kD / 2) {
-    float sn = tab_s, cs = tab_c;
-    if (!a.rope_table)
-      sincosf(inv_f * (float)pos, &sn, &cs);
-    cos_s[tid] = cs;
-    sin_s[tid] = sn;
-  }
-  __syncthreads();
-  // q' = q*cos + cat(-q[64:], q[:64])*sin for the G heads of this KV head
-#pragma unroll
-  for (int r = 0; r < (kMaxGroup * kD + kThreads - 1) / kThreads; ++r) {
-    const int i = tid + r * kThreads;
-    if (i < G * kD) {
-      const int h = i / kD, j = i % kD, jj = j & (kD / 2 - 1);
-      q_s[h][j] = qraw[r] * cos_s[jj] + qpair[r] * sin_s[jj];
-    }
-  }
+  // ---- RoPE: q' = q*cos + cat(-q[64:], q[:64])*sin, same for the new k ------
+  if (!a.rope_table)
+    sincosf(inv_f * (float)pos, &sn, &cs);
+  if (qh < nh)
+    q_s[qh][j] = qraw * cs + qpair * sn;
   if (has_new && tid < kD) {
-    const int j = tid, jj = j & (kD / 2 - 1);
-    const float kn = kraw * cos_s[jj] + kpair * sin_s[jj];
+    const float kn = kraw * cs + kpair * sn;
     knew_s[j] = kn;
     vnew_s[j] = vraw;
-    a.kcache[((size_t)kvh * a.max_len + pos) * kD + j] = kn;
-    a.vcache[((size_t)kvh * a.max_len + pos) * kD + j] = vraw;
+    if (hb == 0) { // one writer per cache row
+      a.kcache[((size_t)kvh * a.max_len + pos) * kD + j] = kn;
+      a.vcache[((size_t)kvh * a.max_len + pos) * kD + j] = vraw;
+    }
   }
   __syncthreads();
 
   // ---- scores: 4 threads per position, 32 dims each ----------------------
   {
     const int p = sp, part = spart;
-    float dot[kMaxGroup];
+    float dot[kHPB];
 #pragma unroll
-    for (int h = 0; h < kMaxGroup; ++h)
+    for (int h = 0; h < kHPB; ++h)
       dot[h] = 0.f;
     if (p < np) {
       const bool is_new = (p0 + p == pos);
@@ -167,8 +158,8 @@ __global__ void __launch_bounds__(kThreads) attn_decode_partial(AttnArgs a) {
         const float4 kv =
             is_new ? *reinterpret_cast<const float4 *>(knew_s + d) : kreg[c];
 #pragma unroll
-        for (int h = 0; h < kMaxGroup; ++h) {
-          if (h < G) {
+        for (int h = 0; h < kHPB; ++h) {
+          if (h < nh) {
             const float4 qv = *reinterpret_cast<const float4 *>(&q_s[h][d]);
             dot[h] = fmaf(qv.x, kv.x, dot[h]);
             dot[h] = fmaf(qv.y, kv.y, dot[h]);
@@ -179,21 +170,20 @@ __global__ void __launch_bounds__(kThreads) attn_decode_partial(AttnArgs a) {
       }
     }
 #pragma unroll
-    for (int h = 0; h < kMaxGroup; ++h) {
+    for (int h = 0; h < kHPB; ++h)
       dot[h] = quad_sum(dot[h]);
-    }
     if (part == 0) {
 #pragma unroll
-      for (int h = 0; h < kMaxGroup; ++h)
-        if (h < G)
+      for (int h = 0; h < kHPB; ++h)
+        if (h < nh)
           sc_s[h][p] = p < np ? dot[h] * a.scale : -INFINITY;
     }
   }
   __syncthreads();
 
   // ---- per-head max, exp, sum over the chunk: one wavefront per head -------
-  for (int h = tid >> 6; h < G; h += kThreads / 64) {
-    const int p = tid & 63;
+  if ((tid >> 6) < nh) {
+    const int h = tid >> 6, p = tid & 63;
     const float s = sc_s[h][p];
     const float m = wave_max(s);
     const float e = expf(s - m); // -inf -> 0 for the positions beyond pos
@@ -209,12 +199,12 @@ __global__ void __launch_bounds__(kThreads) attn_decode_partial(AttnArgs a) {
   // ---- acc[h][d] = sum_p e[h][p] * V[p][d]: 32 threads across d, 8 rows of p
   {
     const int dq = vq, pg = vg;
-    float acc[kMaxGroup][4];
+    float acc[kHPB][4];
 #pragma unroll
-    for (int h = 0; h < kMaxGroup; ++h)
+    for (int h = 0; h < kHPB; ++h)
 #pragma unroll
-      for (int j = 0; j < 4; ++j)
-        acc[h][j] = 0.f;
+      for (int c = 0; c < 4; ++c)
+        acc[h][c] = 0.f;
 #pragma unroll
     for (int i = 0; i < kChunk / 8; ++i) {
       const int p = pg + 8 * i;
@@ -223,8 +213,8 @@ __global__ void __launch_bounds__(kThreads) attn_decode_partial(AttnArgs a) {
         const float4 v =
             is_new ? *reinterpret_cast<const float4 *>(vnew_s + dq * 4) : vreg[i];
 #pragma unroll
-        for (int h = 0; h < kMaxGroup; ++h) {
-          if (h < G) {
+        for (int h = 0; h < kHPB; ++h) {
+          if (h < nh) {
             const float e = sc_s[h][p];
             acc[h][0] = fmaf(v.x, e, acc[h][0]);
             acc[h][1] = fmaf(v.y, e, acc[h][1]);
@@ -235,21 +225,20 @@ __global__ void __launch_bounds__(kThreads) attn_decode_partial(AttnArgs a) {
       }
     }
 #pragma unroll
-    for (int h = 0; h < kMaxGroup; ++h)
-      if (h < G)
+    for (int h = 0; h < kHPB; ++h)
+      if (h < nh)
         *reinterpret_cast<float4 *>(&red_s[pg][h][dq * 4]) =
             make_float4(acc[h][0], acc[h][1], acc[h][2], acc[h][3]);
   }
   __syncthreads();
-  for (int i = tid; i < G * kD; i += kThreads) {
-    const int h = i / kD, d = i % kD;
+  if (qh < nh) {
     float s = 0.f;
 #pragma unroll
     for (int g = 0; g < kThreads / 32; ++g)
-      s += red_s[g][h][d];
-    a.part_acc[((size_t)(h0 + h) * a.nchunks + chunk) * kD + d] = s;
+      s += red_s[g][qh][j];
+    a.part_acc[((size_t)(h0 + qh) * a.nchunks + chunk) * kD + j] = s;
   }
-  if (tid < G) {
+  if (tid < nh) {
     a.part_ml[((size_t)(h0 + tid) * a.nchunks + chunk) * 2 + 0] = m_s[tid];
     a.part_ml[((size_t)(h0 + tid) * a.nchunks + chunk) * 2 + 1] = l_s[tid];
   }
@@ -325,7 +314,9 @@ int launch_attn_decode(const AttnDecodeArgs &in, hipStream_t stream) {
   a.part_acc = parts.acc;
   a.part_ml = parts.ml;
   a.out = in.out;
-  hipLaunchKernelGGL(attn_decode_partial, dim3(a.nchunks, in.kv_heads),
+  a.pairs_padded = (int)round_up((int64_t)a.nchunks * in.kv_heads, 8);
+  const int head_blocks = (a.group + kHPB - 1) / kHPB;
+  hipLaunchKernelGGL(attn_decode_partial, dim3(a.pairs_padded * head_blocks),
                      dim3(kThreads), 0, stream, a);
   if (in.combine)
     hipLaunchKernelGGL(attn_decode_combine, dim3(in.heads), dim3(kD), 0, stream, a);
