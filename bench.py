@@ -3,6 +3,7 @@
 MI355X, next to the CPU oracle timed on the same host.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W]
+    python bench.py --workload gemv|mlp|prefill|llama8b   (the other configurations)
 
 A step is one greedy decode step (one token) at batch 1 with the KV cache
 already holding 1024 positions; weights, KV cache and activations are resident
@@ -112,11 +113,264 @@ def cpu_baseline(shape, host, first_token, budget_s=12.0, max_steps=4096):
                       f"{dt:.1f} s of CPU time"}
 
 
+# ---------------------------------------------------------------------------
+# The other measured configurations (one JSON line each, same field names).
+# ---------------------------------------------------------------------------
+MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X published dense bf16
+
+
+def _time_launches(fn, iters, warm=8):
+    """Average seconds per call of fn(i), launched back to back on torch's
+    current stream and timed with HIP events on that stream."""
+    import torch
+
+    for i in range(warm):
+        fn(i)
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    e0.record()
+    for i in range(iters):
+        fn(i)
+    e1.record()
+    e1.synchronize()
+    return e0.elapsed_time(e1) * 1e-3 / iters
+
+
+def _random_packed(K, N, copies):
+    """`copies` wave-tile buffers of random int8 (timing only: any bytes do)."""
+    import torch
+
+    import buddy_mlir_amd as bma
+
+    nbytes = bma.lib().buddy_hip_w8_packed_bytes(K, N)
+    return [torch.randint(-127, 128, (nbytes,), dtype=torch.int8, device="cuda")
+            for _ in range(copies)]
+
+
+def _linear_fn(bh, sets, x, out, K, N, M, dual, norm_w, epilogue):
+    """Returns fn(i) that launches one fused linear on weight set i % len(sets)."""
+    import torch
+
+    from buddy_mlir_amd import ops
+
+    scale = torch.full((N,), 1e-3, device="cuda")
+    descs = []
+    for w in sets:
+        d = ops.LinearDesc()
+        d.A, d.lda = x.data_ptr(), K
+        d.W0, d.scale0 = w[0].data_ptr(), scale.data_ptr()
+        if dual:
+            d.W1, d.scale1 = w[1].data_ptr(), scale.data_ptr()
+        d.bias, d.norm_w, d.norm_eps = None, (norm_w.data_ptr() if norm_w is not None else None), 1e-6
+        d.C, d.ldc, d.M, d.K, d.N, d.epilogue = out.data_ptr(), N, M, K, N, epilogue
+        descs.append(d)
+    stream = torch.cuda.current_stream().cuda_stream
+    keep = (scale, descs)
+
+    def fn(i, keep=keep):
+        rc = bh.buddy_hip_linear_w8a32(ctypes.byref(descs[i % len(descs)]), stream)
+        if rc:
+            raise RuntimeError("linear_w8a32 failed")
+    return fn
+
+
+def _linear_bytes(K, N, M, dual, norm):
+    return (2 if dual else 1) * (K * N + 4 * N) + 4 * M * (K + N) + (4 * K if norm else 0)
+
+
+def bench_gemv(bh, args):
+    """configs[0]: one int8 GEMV 1536 -> 8960 at M = 1, weights rotated over 48
+    copies (HBM-cold, 660 MB) and over one copy (cache-warm)."""
+    import torch
+
+    K, N = 1536, 8960
+    x = torch.randn((1, K), device="cuda")
+    y = torch.empty((1, N), device="cuda")
+    by = _linear_bytes(K, N, 1, False, False)
+    res = {}
+    for name, copies in (("hbm_cold", 48), ("cache_warm", 1)):
+        sets = [(w,) for w in _random_packed(K, N, copies)]
+        fn = _linear_fn(bh, sets, x, y, K, N, 1, False, None, 0)
+        t = _time_launches(fn, 960)
+        res[name] = {"us": t * 1e6, "gbps": by / t / 1e9, "frac": by / t / 1e9 / HBM_PEAK_GBPS}
+        del sets
+    t = res["hbm_cold"]["us"] * 1e-6
+    return {
+        "metric": "int8_gemv_hbm_gbps", "value": res["hbm_cold"]["gbps"], "unit": "GB/s",
+        "n_gpus": 1, "steps": 960, "warmup": 8, "ms_per_step": t * 1e3,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": "single int8 weight-only GEMV x[1,1536] . W[1536,8960] "
+                               "(BASELINE configs[0]), 48 rotating weight copies"},
+        "detail": res,
+        "roofline": {"kernel": "gemv_w8a32_bcast_kernel<1, 0, 0, 6, true>", "bound": "hbm",
+                     "achieved": res["hbm_cold"]["gbps"], "peak": HBM_PEAK_GBPS,
+                     "unit": "GB/s", "frac": res["hbm_cold"]["frac"],
+                     "algorithmic_bytes_per_launch": by, "avg_launch_us": t * 1e6,
+                     "traffic": None},
+    }
+
+
+def bench_mlp(bh, args):
+    """configs[1]: h = SiLU(x G) * (x U), y = h D at M in {1, 4, 16}: two launches
+    (fused gate|up, then down), 12 rotating weight sets (496 MB)."""
+    import torch
+
+    H, I = 1536, 8960
+    gu = _random_packed(H, I, 24)
+    dn = _random_packed(I, H, 12)
+    res = {}
+    for M in (1, 4, 16):
+        x = torch.randn((M, H), device="cuda")
+        h = torch.empty((M, I), device="cuda")
+        y = torch.zeros((M, H), device="cuda")
+        f1 = _linear_fn(bh, [(gu[2 * i], gu[2 * i + 1]) for i in range(12)], x, h, H, I, M, True, None, 2)
+        f2 = _linear_fn(bh, [(w,) for w in dn], h, y, I, H, M, False, None, 0)
+
+        def fn(i):
+            f1(i)
+            f2(i)
+        t = _time_launches(fn, 480)
+        by = 3 * H * I + 4 * (2 * I + H) + 4 * M * 2 * H  # the survey's formula
+        res[f"M={M}"] = {"us": t * 1e6, "gbps": by / t / 1e9,
+                         "frac": by / t / 1e9 / HBM_PEAK_GBPS}
+    t = res["M=1"]["us"] * 1e-6
+    return {
+        "metric": "int8_mlp_hbm_gbps", "value": res["M=1"]["gbps"], "unit": "GB/s",
+        "n_gpus": 1, "steps": 480, "warmup": 8, "ms_per_step": t * 1e3,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": "int8 MLP block 1536 -> 8960 -> 1536 at M in {1,4,16} "
+                               "(BASELINE configs[1]); value is M=1"},
+        "detail": res,
+        "roofline": {"kernel": "gate|up + down GEMV pair", "bound": "hbm",
+                     "achieved": res["M=1"]["gbps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": res["M=1"]["frac"], "traffic": None},
+    }
+
+
+def bench_prefill(bh, args):
+    """configs[3]: a 512-token prompt through all 28 layers (int8 weights
+    converted to bf16 in LDS, MFMA with f32 accumulators, causal GQA
+    attention).  Activations as one bf16 term (the configuration's wording) and
+    as three exact terms (what the parity bar needs)."""
+    import numpy as np
+    import torch
+
+    from buddy_mlir_amd import synthetic
+    from buddy_mlir_amd.session import Shape
+
+    M = 512
+    shape = Shape(max_len=M + 64)
+    sess, _ = synthetic.build_session(shape, context=0)
+    toks = synthetic.first_tokens(shape, M)
+    H, I, L = shape.hidden, shape.inter, shape.layers
+    QN, KVN = shape.heads * shape.head_dim, shape.kv_heads * shape.head_dim
+    gemm_flop = 2 * M * L * (H * (QN + 2 * KVN) + QN * H + 3 * H * I)
+    attn_flop = L * shape.heads * M * M * shape.head_dim * 2 * 2 // 2
+    res = {}
+    for name, exact in (("bf16_1term", False), ("f32_exact_3term", True)):
+        sess.prefill(toks, 0, want_logits=False, exact=exact)  # warm-up
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        n = 5
+        for _ in range(n):
+            sess.prefill(toks, 0, want_logits=False, exact=exact)
+        torch.cuda.synchronize()
+        t = (time.perf_counter() - t0) / n
+        res[name] = {"ms": t * 1e3, "tokens_per_s": M / t,
+                     "gemm_tflops": gemm_flop / t / 1e12,
+                     "mfma_frac": gemm_flop / t / 1e12 / MFMA_BF16_PEAK_TFLOPS}
+    sess.close()
+    t = res["bf16_1term"]["ms"] * 1e-3
+    return {
+        "metric": "prefill_tokens_per_s", "value": M / t, "unit": "tokens/s",
+        "n_gpus": 1, "steps": 5, "warmup": 1, "ms_per_step": t * 1e3,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": "prefill of 512 tokens, Qwen2-1.5B shape, 28 layers "
+                               "(BASELINE configs[3]); value is the 1-term bf16 mode; "
+                               "time includes attention, norms and the last-row lm_head"},
+        "detail": res, "gemm_flop": gemm_flop, "attention_flop": attn_flop,
+        "roofline": {"kernel": "gemm_w8_bf16_kernel<1>", "bound": "mfma",
+                     "achieved": res["bf16_1term"]["gemm_tflops"], "peak": MFMA_BF16_PEAK_TFLOPS,
+                     "unit": "TFLOP/s", "frac": res["bf16_1term"]["mfma_frac"], "traffic": None},
+    }
+
+
+def bench_llama8b(bh, args):
+    """configs[4]: the decode GEMVs of a Llama-3-8B-shaped step, 32 layers of
+    distinct weights (q|k|v, o, gate|up fused, down) plus lm_head: 7.5 GB of int8
+    streamed once per sweep, at M = 1 and M = 8."""
+    import torch
+
+    H, I, V, L = 4096, 14336, 128256, 32
+    QKV = 4096 + 2 * 1024
+    mats = []  # (name, K, N, dual, count)
+    layers = []
+    for _ in range(L):
+        layers.append({
+            "qkv": _random_packed(H, QKV, 1), "o": _random_packed(H, H, 1),
+            "gu": _random_packed(H, I, 2), "down": _random_packed(I, H, 1)})
+    lm = _random_packed(H, V, 1)
+    res = {}
+    for M in (1, 8):
+        x = torch.randn((M, H), device="cuda")
+        hbuf = torch.empty((M, I), device="cuda")
+        qkv = torch.empty((M, QKV), device="cuda")
+        y = torch.zeros((M, H), device="cuda")
+        logits = torch.empty((M, V), device="cuda")
+        nw = torch.ones(H, device="cuda") if M == 1 else None  # fused norm at M = 1
+        f_qkv = _linear_fn(bh, [(l["qkv"][0],) for l in layers], x, qkv, H, QKV, M, False, nw, 0)
+        f_o = _linear_fn(bh, [(l["o"][0],) for l in layers], x, y, H, H, M, False, None, 1)
+        f_gu = _linear_fn(bh, [tuple(l["gu"]) for l in layers], x, hbuf, H, I, M, True, nw, 2)
+        f_dn = _linear_fn(bh, [(l["down"][0],) for l in layers], hbuf, y, I, H, M, False, None, 1)
+        f_lm = _linear_fn(bh, [(lm[0],)], x, logits, H, V, M, False, nw, 0)
+
+        def sweep(_):
+            for i in range(L):
+                f_qkv(i)
+                f_o(i)
+                f_gu(i)
+                f_dn(i)
+            f_lm(0)
+        t = _time_launches(sweep, 10, warm=2)
+        by = (L * (_linear_bytes(H, QKV, M, False, M == 1) + _linear_bytes(H, H, M, False, False)
+                   + _linear_bytes(H, I, M, True, M == 1) + _linear_bytes(I, H, M, False, False))
+              + _linear_bytes(H, V, M, False, M == 1))
+        per = {}
+        for nm, f, k, n, dual in (("qkv", f_qkv, H, QKV, False), ("o", f_o, H, H, False),
+                                  ("gate|up", f_gu, H, I, True), ("down", f_dn, I, H, False),
+                                  ("lm_head", f_lm, H, V, False)):
+            tt = _time_launches(f, 128)
+            b = _linear_bytes(k, n, M, dual, False)
+            per[nm] = {"us": tt * 1e6, "gbps": b / tt / 1e9, "frac": b / tt / 1e9 / HBM_PEAK_GBPS}
+        res[f"M={M}"] = {"sweep_ms": t * 1e3, "bytes": by, "gbps": by / t / 1e9,
+                         "frac": by / t / 1e9 / HBM_PEAK_GBPS, "per_matrix": per}
+    r1 = res["M=1"]
+    return {
+        "metric": "int8_gemv_sweep_hbm_gbps", "value": r1["gbps"], "unit": "GB/s",
+        "n_gpus": 1, "steps": 10, "warmup": 2, "ms_per_step": r1["sweep_ms"],
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": "Llama-3-8B-shaped decode GEMV sweep, 32 layers + lm_head, "
+                               "161 dependent launches (BASELINE configs[4]); value is M=1"},
+        "detail": res,
+        "roofline": {"kernel": "gemv_w8a32_bcast_kernel (all shapes of the sweep)",
+                     "bound": "hbm", "achieved": r1["gbps"], "peak": HBM_PEAK_GBPS,
+                     "unit": "GB/s", "frac": r1["frac"], "traffic": None},
+    }
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=64)
     ap.add_argument("--warmup", type=int, default=8)
+    ap.add_argument("--workload", default="decode",
+                    choices=["decode", "gemv", "mlp", "prefill", "llama8b"],
+                    help="decode (default): the full decode step the headline metric "
+                         "is quoted on; the others measure the remaining configurations")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-graph", action="store_true")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -137,6 +391,11 @@ def main():
 
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     bh = bma.lib()
+    if args.workload != "decode":
+        fn = {"gemv": bench_gemv, "mlp": bench_mlp, "prefill": bench_prefill,
+              "llama8b": bench_llama8b}[args.workload]
+        print(json.dumps(fn(bh, args)))
+        return
     K, W = args.steps, args.warmup
     max_len = (CONTEXT + W + K + 63) // 64 * 64
     shape = Shape(max_len=max_len)
@@ -192,7 +451,7 @@ def main():
         "decode_step_hbm_gbps": step_b / step_s / 1e9,
         "decode_step_hbm_frac": step_b / step_s / 1e9 / HBM_PEAK_GBPS,
         "roofline": {
-            "kernel": "gemv_w8a32_kernel<1, 2, 1, 4, 16> (RMSNorm + gate|up int8 GEMV "
+            "kernel": "gemv_w8a32_bcast_kernel<1, 2, 1, 6, true> (RMSNorm + gate|up int8 GEMV "
                       "+ SiLU*mul, 1536 -> 2 x 8960)",
             "bound": "hbm",
             "achieved": achieved,

@@ -20,4 +20,8 @@ struct GemmW8Args {
 
 int launch_gemm_w8(const GemmW8Args &a, hipStream_t stream);
 
+// The matmul keeps a bf16 copy of its activations in a grow-only device buffer
+// per stream; a stream's owner drops it before destroying the stream.
+void release_gemm_staging(hipStream_t stream);
+
 } // namespace bh

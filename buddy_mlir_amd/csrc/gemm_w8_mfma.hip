@@ -7,27 +7,36 @@
 //
 // Shape of the kernel:
 //  * the weights are read from the same wave-tile packed copy the decode GEMV
-//    streams (one resident copy serves prefill and decode);
-//  * a workgroup owns a 128 x 128 tile of C; per 64-wide k slab it converts the
-//    int8 tile to bf16 while storing it to LDS (|q| <= 128 is exact in bf16; the
-//    per-channel scale is applied once to the f32 accumulators, where the
-//    reference multiplies every element before the FMA) and the f32 activations
-//    to bf16 (one, two or three bf16 terms: one term is "activations cast to
-//    bf16", three terms carry all 24 significand bits of the f32 input);
-//  * four wavefronts each hold a 64 x 64 block of C as 2 x 2 MFMA 32x32x16 bf16
-//    accumulators (f32), fragments come from LDS with 16-byte reads;
-//  * the next slab's global loads are in flight while the current slab is
-//    multiplied.
+//    streams (one resident copy serves prefill and decode).  A lane's 16 bytes
+//    of a 16 x 64 tile are, as they lie, two 8-wide operand fragments of
+//    v_mfma_f32_16x16x32_bf16 (rows = the tile's 16 channels): they go from
+//    global memory to registers, are converted to bf16 (|q| <= 128 is exact)
+//    and fed to the matrix core.  No LDS on the way;
+//  * the activations are converted once per call to bf16 terms (one term =
+//    "activations cast to bf16"; three terms carry all 24 significand bits of
+//    the f32 input) in a [term][row][k] buffer.  A lane's fragment of the other
+//    operand (columns = 16 activation rows) is 32 contiguous bytes of that
+//    buffer, so it is loaded straight from L2 as well;
+//  * a wavefront owns 64 rows x 64 channels of C (4 x 4 accumulators); the four
+//    wavefronts of a workgroup split K and meet in LDS, in slice order;
+//  * workgroup ids are laid out so that the row blocks of one column tile run
+//    on the same XCD (ids equal modulo 8) and share the weight tiles in its L2;
+//  * the per-channel scale is applied once to the f32 accumulators, where the
+//    reference multiplies every element before the FMA.
 #include "gemm.h"
+
+#include <map>
+#include <mutex>
 
 namespace bh {
 namespace {
 
-constexpr int BM = 128, BN = 128, BK = 64;
-constexpr int LDSK = BK + 8; // bf16 elements per LDS row, padded against conflicts
+constexpr int kRowsPerWave = 64;   // 4 row blocks of 16
+constexpr int kGroupsPerWave = 4;  // 4 channel groups of 16
+constexpr int kSlices = 4;         // k-slices = wavefronts per workgroup
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned short u16;
 
 __device__ __forceinline__ u16 bf16_rne(float x) {
@@ -47,159 +56,224 @@ __device__ __forceinline__ unsigned q2_to_bf16x2(int v, int j) {
   const float b = (float)(signed char)(v >> (8 * j + 8));
   return (__float_as_uint(a) >> 16) | (__float_as_uint(b) & 0xffff0000u);
 }
+__device__ __forceinline__ bf16x8 frag_from(int lo, int hi) {
+  union {
+    uint4 u;
+    bf16x8 v;
+  } x;
+  x.u = make_uint4(q2_to_bf16x2(lo, 0), q2_to_bf16x2(lo, 2), q2_to_bf16x2(hi, 0),
+                   q2_to_bf16x2(hi, 2));
+  return x.v;
+}
+__device__ __forceinline__ bf16x8 as_frag(const uint4 &u) {
+  union {
+    uint4 u;
+    bf16x8 v;
+  } x;
+  x.u = u;
+  return x.v;
+}
+
+// A[M, K] f32 -> terms x [Mp, Kp] bf16, zero padded; term t holds the bf16
+// rounding of what the terms before it left over.
+__global__ void __launch_bounds__(256)
+activations_to_bf16(const float *__restrict__ A, int64_t lda, int M, int K, int Mp,
+                    int Kp, int terms, u16 *__restrict__ out) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; // 8 k per thread
+  const int kq = Kp / 8;
+  if (i >= (int64_t)Mp * kq)
+    return;
+  const int m = (int)(i / kq), k0 = (int)(i % kq) * 8;
+  float r[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e)
+    r[e] = (m < M && k0 + e < K) ? A[(int64_t)m * lda + k0 + e] : 0.f;
+  for (int t = 0; t < terms; ++t) {
+    u16 h[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      h[e] = bf16_rne(r[e]);
+      r[e] -= bf16_to_f32(h[e]);
+    }
+    *reinterpret_cast<uint4 *>(out + ((size_t)t * Mp + m) * Kp + k0) =
+        make_uint4(pack2(h[0], h[1]), pack2(h[2], h[3]), pack2(h[4], h[5]),
+                   pack2(h[6], h[7]));
+  }
+}
 
 struct GemmArgs {
-  const float *A;
+  const u16 *Abf; // [terms][Mp][Kp]
   const int4 *W;
   const float *scale;
   const float *bias;
   float *C;
-  int64_t lda, ldc;
-  int M, K, N, groups, chunks;
+  int64_t ldc;
+  int M, N, Mp, Kp, groups, chunks;
+  int ncols, cols_padded; // column tiles of 64 channels; padded to the XCD count
   int accumulate;
 };
 
+template <int TERMS> struct ChunkOperands {
+  int4 w[kGroupsPerWave];
+  uint4 a[TERMS][4][2]; // [term][row block][k half]
+};
+
 template <int TERMS>
-__global__ void __launch_bounds__(256) gemm_w8_bf16_kernel(GemmArgs a) {
-  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-  u16(*As)[BM][LDSK] = reinterpret_cast<u16(*)[BM][LDSK]>(smem);
-  u16(*Bs)[LDSK] = reinterpret_cast<u16(*)[LDSK]>(smem + sizeof(u16) * TERMS * BM * LDSK);
-
-  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
-  const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
-  const int wm = wave >> 1, wn = wave & 1;
-
-  // global -> register staging assignments
-  const int arow = tid >> 1, ahalf = tid & 1;   // A: 32 consecutive k of a row
-  const int btile = tid >> 6;                   // B: tiles btile and btile + 4
-  const int bch = lane & 15, bkg = lane >> 4;
-
-  f32x16 acc[2][2];
+__device__ __forceinline__ void load_chunk(const int4 *const (&wp)[kGroupsPerWave],
+                                           const u16 *ap, size_t term_stride,
+                                           size_t rb_stride, int c,
+                                           ChunkOperands<TERMS> &o) {
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int g = 0; g < kGroupsPerWave; ++g)
+    o.w[g] = wp[g][(size_t)c * 64];
 #pragma unroll
-    for (int j = 0; j < 2; ++j)
+  for (int t = 0; t < TERMS; ++t)
 #pragma unroll
-      for (int e = 0; e < 16; ++e)
-        acc[i][j][e] = 0.f;
-
-  float4 areg[8];
-  int4 breg[2];
-  auto load_global = [&](int c) {
-    const int k0 = c * BK + ahalf * 32;
-    const int m = m0 + arow;
-    const float *src = a.A + (int64_t)m * a.lda + k0;
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const int k = k0 + i * 4;
-      if (m < a.M && k + 3 < a.K && ((reinterpret_cast<uintptr_t>(src + i * 4) & 15) == 0))
-        areg[i] = *reinterpret_cast<const float4 *>(src + i * 4);
-      else if (m < a.M)
-        areg[i] = make_float4(k < a.K ? src[i * 4] : 0.f,
-                              k + 1 < a.K ? src[i * 4 + 1] : 0.f,
-                              k + 2 < a.K ? src[i * 4 + 2] : 0.f,
-                              k + 3 < a.K ? src[i * 4 + 3] : 0.f);
-      else
-        areg[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int rb = 0; rb < 4; ++rb) {
+      const uint4 *src = reinterpret_cast<const uint4 *>(
+          ap + t * term_stride + rb * rb_stride + (size_t)c * kTileK);
+      o.a[t][rb][0] = src[0];
+      o.a[t][rb][1] = src[1];
     }
+}
+
+template <int TERMS>
+__global__ void __launch_bounds__(kSlices *kWave) gemm_w8_bf16_kernel(GemmArgs a) {
+  extern __shared__ __attribute__((aligned(16))) float red[]; // [slice][64][lane]
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int col = blockIdx.x % a.cols_padded, rbk = blockIdx.x / a.cols_padded;
+  if (col >= a.ncols)
+    return; // padding id
+  const int m0 = rbk * kRowsPerWave, g0 = col * kGroupsPerWave;
+  const int per = (a.chunks + kSlices - 1) / kSlices;
+  const int c0 = min(wave * per, a.chunks), c1 = min(c0 + per, a.chunks);
+
+  f32x4 acc[kGroupsPerWave][4];
 #pragma unroll
-    for (int t = 0; t < 2; ++t) {
-      const int g = n0 / 16 + btile + 4 * t;
-      breg[t] = g < a.groups ? a.W[((size_t)g * a.chunks + c) * 64 + lane]
-                             : make_int4(0, 0, 0, 0);
-    }
-  };
-  auto store_lds = [&]() {
-    // A: f32 -> TERMS bf16 terms
+  for (int g = 0; g < kGroupsPerWave; ++g)
 #pragma unroll
-    for (int i = 0; i < 8; i += 2) {
-      const float v[8] = {areg[i].x, areg[i].y, areg[i].z, areg[i].w,
-                          areg[i + 1].x, areg[i + 1].y, areg[i + 1].z, areg[i + 1].w};
-      float r[8];
+    for (int rb = 0; rb < 4; ++rb)
+      acc[g][rb] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  const int4 *wp[kGroupsPerWave];
 #pragma unroll
-      for (int e = 0; e < 8; ++e)
-        r[e] = v[e];
+  for (int g = 0; g < kGroupsPerWave; ++g) // groups past the end repeat the last one
+    wp[g] = a.W + ((size_t)min(g0 + g, a.groups - 1) * a.chunks) * 64 + lane;
+  const size_t term_stride = (size_t)a.Mp * a.Kp, rb_stride = (size_t)16 * a.Kp;
+  const u16 *ap = a.Abf + (size_t)(m0 + (lane & 15)) * a.Kp + (lane >> 4) * 16;
+
+  ChunkOperands<TERMS> cur, nxt;
+  if (c0 < c1)
+    load_chunk<TERMS>(wp, ap, term_stride, rb_stride, c0, cur);
+  for (int c = c0; c < c1; ++c) {
+    if (c + 1 < c1)
+      load_chunk<TERMS>(wp, ap, term_stride, rb_stride, c + 1, nxt);
 #pragma unroll
-      for (int t = 0; t < TERMS; ++t) {
-        u16 h[8];
+    for (int g = 0; g < kGroupsPerWave; ++g) {
+      const bf16x8 w0 = frag_from(cur.w[g].x, cur.w[g].y);
+      const bf16x8 w1 = frag_from(cur.w[g].z, cur.w[g].w);
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          h[e] = bf16_rne(r[e]);
-          r[e] = r[e] - bf16_to_f32(h[e]);
+      for (int t = 0; t < TERMS; ++t)
+#pragma unroll
+        for (int rb = 0; rb < 4; ++rb) {
+          acc[g][rb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+              w0, as_frag(cur.a[t][rb][0]), acc[g][rb], 0, 0, 0);
+          acc[g][rb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+              w1, as_frag(cur.a[t][rb][1]), acc[g][rb], 0, 0, 0);
         }
-        *reinterpret_cast<uint4 *>(&As[t][arow][ahalf * 32 + i * 4]) =
-            make_uint4(pack2(h[0], h[1]), pack2(h[2], h[3]), pack2(h[4], h[5]),
-                       pack2(h[6], h[7]));
-      }
     }
-    // B: int8 -> bf16, row = channel, 16 consecutive k
-#pragma unroll
-    for (int t = 0; t < 2; ++t) {
-      const int ch = (btile + 4 * t) * 16 + bch;
-      const int4 w = breg[t];
-      uint4 lo = make_uint4(q2_to_bf16x2(w.x, 0), q2_to_bf16x2(w.x, 2),
-                            q2_to_bf16x2(w.y, 0), q2_to_bf16x2(w.y, 2));
-      uint4 hi = make_uint4(q2_to_bf16x2(w.z, 0), q2_to_bf16x2(w.z, 2),
-                            q2_to_bf16x2(w.w, 0), q2_to_bf16x2(w.w, 2));
-      *reinterpret_cast<uint4 *>(&Bs[ch][bkg * 16]) = lo;
-      *reinterpret_cast<uint4 *>(&Bs[ch][bkg * 16 + 8]) = hi;
-    }
-  };
-
-  load_global(0);
-  for (int c = 0; c < a.chunks; ++c) {
-    __syncthreads(); // previous slab fully consumed
-    store_lds();
-    __syncthreads();
-    if (c + 1 < a.chunks)
-      load_global(c + 1);
-#pragma unroll
-    for (int ks = 0; ks < BK / 16; ++ks) {
-      const int kk = ks * 16 + (lane >> 5) * 8;
-      bf16x8 bf[2];
-#pragma unroll
-      for (int j = 0; j < 2; ++j)
-        bf[j] = *reinterpret_cast<const bf16x8 *>(&Bs[wn * 64 + j * 32 + (lane & 31)][kk]);
-#pragma unroll
-      for (int t = 0; t < TERMS; ++t) {
-#pragma unroll
-        for (int i = 0; i < 2; ++i) {
-          const bf16x8 af =
-              *reinterpret_cast<const bf16x8 *>(&As[t][wm * 64 + i * 32 + (lane & 31)][kk]);
-#pragma unroll
-          for (int j = 0; j < 2; ++j)
-            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af, bf[j], acc[i][j], 0, 0, 0);
-        }
-      }
-    }
+    if (c + 1 < c1)
+      cur = nxt;
   }
 
-  // epilogue: scale per channel, optional bias / accumulate
+  // ---- the k-slices meet in LDS; wavefront w finishes channel group w ------
+  float *mine = red + (size_t)wave * 64 * kWave;
 #pragma unroll
-  for (int j = 0; j < 2; ++j) {
-    const int n = n0 + wn * 64 + j * 32 + (lane & 31);
-    if (n >= a.N)
+  for (int g = 0; g < kGroupsPerWave; ++g)
+#pragma unroll
+    for (int rb = 0; rb < 4; ++rb)
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        mine[((g * 4 + rb) * 4 + r) * kWave + lane] = acc[g][rb][r];
+  __syncthreads();
+  const int g = wave;
+  if (g0 + g >= a.groups)
+    return;
+  // lane holds channels n..n+3 of row m for each row block
+  const int n = (g0 + g) * kTileN + (lane >> 4) * 4;
+  float s[4], b[4];
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    s[r] = n + r < a.N ? a.scale[n + r] : 0.f;
+    b[r] = (a.bias && n + r < a.N) ? a.bias[n + r] : 0.f;
+  }
+  const bool vec = n + 3 < a.N && (a.ldc & 3) == 0 &&
+                   (reinterpret_cast<uintptr_t>(a.C) & 15) == 0;
+#pragma unroll
+  for (int rb = 0; rb < 4; ++rb) {
+    const int m = m0 + rb * 16 + (lane & 15);
+    float v[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      float sum = 0.f;
+#pragma unroll
+      for (int sl = 0; sl < kSlices; ++sl)
+        sum += red[((size_t)sl * 64 + (g * 4 + rb) * 4 + r) * kWave + lane];
+      v[r] = sum * s[r];
+    }
+    if (m >= a.M)
       continue;
-    const float s = a.scale[n];
-    const float b = a.bias ? a.bias[n] : 0.f;
-#pragma unroll
-    for (int i = 0; i < 2; ++i) {
-#pragma unroll
-      for (int e = 0; e < 16; ++e) {
-        const int m = m0 + wm * 64 + i * 32 + (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3);
-        if (m < a.M) {
-          float *c = a.C + (int64_t)m * a.ldc + n;
-          const float v = acc[i][j][e] * s;
-          *c = a.accumulate ? *c + v : b + v;
-        }
+    float *c = a.C + (int64_t)m * a.ldc + n;
+    if (vec) {
+      float4 o = make_float4(v[0], v[1], v[2], v[3]);
+      if (a.accumulate) {
+        const float4 p = *reinterpret_cast<const float4 *>(c);
+        o = make_float4(p.x + o.x, p.y + o.y, p.z + o.z, p.w + o.w);
+      } else {
+        o = make_float4(b[0] + o.x, b[1] + o.y, b[2] + o.z, b[3] + o.w);
       }
+      *reinterpret_cast<float4 *>(c) = o;
+    } else {
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        if (n + r < a.N)
+          c[r] = a.accumulate ? c[r] + v[r] : b[r] + v[r];
     }
   }
 }
 
+// bf16 staging of the activations: one grow-only device buffer per stream, so
+// that calls on different streams do not share it.  Calls on one stream are
+// ordered, and the buffer is only read by the matmul that follows the
+// conversion on that stream.
+struct Staging {
+  u16 *ptr = nullptr;
+  size_t bytes = 0;
+};
+std::mutex g_staging_mutex;
+std::map<hipStream_t, Staging> g_staging;
+
+int staging_for(hipStream_t stream, size_t bytes, u16 **out) {
+  std::lock_guard<std::mutex> lock(g_staging_mutex);
+  Staging &s = g_staging[stream];
+  if (s.bytes < bytes) {
+    if (s.ptr) {
+      BH_CHECK_HIP(hipStreamSynchronize(stream)); // an earlier matmul may still read it
+      BH_CHECK_HIP(hipFree(s.ptr));
+      s.ptr = nullptr;
+      s.bytes = 0;
+    }
+    BH_CHECK_HIP(hipMalloc(reinterpret_cast<void **>(&s.ptr), bytes));
+    s.bytes = bytes;
+  }
+  *out = s.ptr;
+  return BUDDY_HIP_OK;
+}
+
 template <int TERMS>
-int launch_terms(const GemmArgs &a, dim3 grid, hipStream_t stream) {
-  constexpr size_t lds = sizeof(u16) * LDSK * (size_t)(TERMS * BM + BN);
+int launch_terms(const GemmArgs &a, unsigned blocks, hipStream_t stream) {
+  constexpr size_t lds = sizeof(float) * kSlices * 64 * kWave;
   auto kernel = gemm_w8_bf16_kernel<TERMS>;
   static bool attr_set = false;
   if (!attr_set) {
@@ -208,7 +282,7 @@ int launch_terms(const GemmArgs &a, dim3 grid, hipStream_t stream) {
                                      (int)lds));
     attr_set = true;
   }
-  hipLaunchKernelGGL(kernel, grid, dim3(256), lds, stream, a);
+  hipLaunchKernelGGL(kernel, dim3(blocks), dim3(kSlices * kWave), lds, stream, a);
   BH_CHECK_HIP(hipGetLastError());
   return BUDDY_HIP_OK;
 }
@@ -217,8 +291,8 @@ int launch_terms(const GemmArgs &a, dim3 grid, hipStream_t stream) {
 
 int launch_gemm_w8(const GemmW8Args &in, hipStream_t stream) {
   BH_REQUIRE(in.A && in.W && in.scale && in.C, "gemm_w8: null pointer");
-  BH_REQUIRE(in.M > 0 && in.K > 0 && in.N > 0 && in.M < (1 << 30) &&
-                 in.K < (1 << 30) && in.N < (1 << 30),
+  BH_REQUIRE(in.M > 0 && in.K > 0 && in.N > 0 && in.M < (1 << 24) &&
+                 in.K < (1 << 24) && in.N < (1 << 24),
              "gemm_w8: bad shape M=%lld K=%lld N=%lld", (long long)in.M,
              (long long)in.K, (long long)in.N);
   BH_REQUIRE(in.lda >= in.K && in.ldc >= in.N, "gemm_w8: row stride below row length");
@@ -227,25 +301,48 @@ int launch_gemm_w8(const GemmW8Args &in, hipStream_t stream) {
   BH_REQUIRE((reinterpret_cast<uintptr_t>(in.W) & 15) == 0,
              "gemm_w8: packed weights must be 16-byte aligned");
   GemmArgs a;
-  a.A = in.A;
   a.W = reinterpret_cast<const int4 *>(in.W);
   a.scale = in.scale;
   a.bias = in.bias;
   a.C = in.C;
-  a.lda = in.lda;
   a.ldc = in.ldc;
   a.M = (int)in.M;
-  a.K = (int)in.K;
   a.N = (int)in.N;
   a.groups = (int)ceil_div(in.N, kTileN);
   a.chunks = (int)ceil_div(in.K, kTileK);
+  a.Mp = (int)round_up(in.M, kRowsPerWave);
+  a.Kp = a.chunks * kTileK;
+  a.ncols = (int)ceil_div(a.groups, kGroupsPerWave);
+  a.cols_padded = (int)round_up(a.ncols, 8);
   a.accumulate = in.accumulate ? 1 : 0;
-  const dim3 grid((unsigned)ceil_div(in.N, BN), (unsigned)ceil_div(in.M, BM));
+  u16 *abf = nullptr;
+  int rc = staging_for(stream, sizeof(u16) * in.terms * (size_t)a.Mp * a.Kp, &abf);
+  if (rc)
+    return rc;
+  a.Abf = abf;
+  const int64_t threads = (int64_t)a.Mp * (a.Kp / 8);
+  hipLaunchKernelGGL(activations_to_bf16, dim3((unsigned)ceil_div(threads, 256)),
+                     dim3(256), 0, stream, in.A, in.lda, a.M, (int)in.K, a.Mp, a.Kp,
+                     in.terms, abf);
+  BH_CHECK_HIP(hipGetLastError());
+  const unsigned blocks = (unsigned)(a.cols_padded * (a.Mp / kRowsPerWave));
   switch (in.terms) {
-  case 1: return launch_terms<1>(a, grid, stream);
-  case 2: return launch_terms<2>(a, grid, stream);
-  default: return launch_terms<3>(a, grid, stream);
+  case 1: return launch_terms<1>(a, blocks, stream);
+  case 2: return launch_terms<2>(a, blocks, stream);
+  default: return launch_terms<3>(a, blocks, stream);
   }
+}
+
+void release_gemm_staging(hipStream_t stream) {
+  std::lock_guard<std::mutex> lock(g_staging_mutex);
+  auto it = g_staging.find(stream);
+  if (it == g_staging.end())
+    return;
+  if (it->second.ptr) {
+    (void)hipStreamSynchronize(stream);
+    (void)hipFree(it->second.ptr);
+  }
+  g_staging.erase(it);
 }
 
 } // namespace bh

@@ -489,6 +489,7 @@ void buddy_hip_session_destroy(buddy_hip_session *hs) {
       (void)hipFree(p);
   if (s->host_state)
     (void)hipHostFree(s->host_state);
+  bh::release_gemm_staging(s->stream);
   if (s->own_stream)
     (void)hipStreamDestroy(s->stream);
   delete s;
