@@ -924,12 +924,13 @@ int launch_gemv(const GemvArgs &a, hipStream_t stream) {
              "gemv: packed weights must be 16-byte aligned");
   BH_REQUIRE(!a.norm_w || (reinterpret_cast<uintptr_t>(a.norm_w) & 15) == 0,
              "gemv: norm weight must be 16-byte aligned");
-  // batches of 2..16 rows without a fused norm go to the matrix cores: always
-  // for wide matrices (one activation staging serves eight channel groups);
-  // narrow ones (k-slices inside the workgroup, activations restaged per slice)
-  // only from 6 rows up, below that the f32 FMA path is quicker
-  if (a.M >= 2 && !a.norm_w && !a.attn_acc && !force_valu() &&
-      a.tile_n == 16 && (ceil_div(a.N, kTileN) >= 2048 / 4 || a.M >= 6))
+  // batches of 5..16 rows go to the matrix cores when the activations can be
+  // read as aligned 16-byte pieces; up to four rows the f32 FMA kernel (1 + M
+  // instructions per weight) is quicker, and it takes whatever is unaligned
+  if (a.M >= 5 && !a.attn_acc && !force_valu() && a.tile_n == 16 && a.K >= 4 &&
+      (a.K & 3) == 0 && (a.lda & 3) == 0 &&
+      (reinterpret_cast<uintptr_t>(a.A) & 15) == 0 &&
+      (!a.norm_w || (reinterpret_cast<uintptr_t>(a.norm_w) & 15) == 0))
     return launch_gemv_mfma(a, stream);
   // the kernel is compiled for 1, 2, 4, 8 and 16 rows; extra rows are zero-
   // filled in LDS and never stored

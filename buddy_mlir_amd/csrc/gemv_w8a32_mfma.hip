@@ -5,12 +5,24 @@
 // fire for m == 1 only (DequantMatMulVectorizationDecode.cpp:212-217) and the
 // BLIS kernel (MatMulBlisVectorization.cpp:398-986) is the one vectorised
 // kernel for M > 1.  On the GPU the f32 FMA pipe cannot keep up with HBM beyond
-// a few rows (2 + M instructions per weight byte), so the rows go through
+// a few rows (1 + M instructions per weight byte), so the rows go through
 // v_mfma_f32_16x16x32_bf16: the 16 channels of a wave tile are the MFMA's rows,
-// the batch rows its columns.  A lane's 16 weight bytes are two 8-wide A
-// fragments (exact in bf16); the activations are staged in LDS as three bf16
-// terms (all 24 significand bits), so six MFMAs consume one 1 KiB tile.  The
-// weights stream exactly as in the one-row kernel, from the same packed copy.
+// the batch rows its columns.
+//  * A lane's 16 weight bytes are, as they lie in the tile, two 8-wide operand
+//    fragments (exact in bf16).
+//  * The other operand of lane l is x[row l % 16][16 consecutive k]: 64
+//    contiguous bytes of the activation matrix, loaded straight from L2 and cut
+//    into three truncated bf16 terms that add up to the f32 value exactly, so
+//    the products are the f32 ones and only the order of summation differs.
+//    No LDS staging, no barrier before the stream.
+//  * A wavefront converts the activations of a 64-k chunk once and uses them
+//    for SPAN channel groups (six MFMAs per 1 KiB tile), so activation traffic
+//    from L2 stays below the weight stream.
+//  * The weights stream exactly as in the one-row kernel, from the same packed
+//    copy; k-slices of a workgroup meet in LDS in slice order.
+//  * RMSNorm can be fused in: the weight multiplies the activation before it is
+//    cut into terms, each lane gathers the squares of what it loads, and the
+//    row's rsqrt factor multiplies the finished sums.
 #include "gemv_w8a32.h"
 
 namespace bh {
@@ -19,21 +31,19 @@ namespace {
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef int v4i __attribute__((ext_vector_type(4)));
-typedef unsigned short u16;
 
-constexpr int kWaves = 8;
-constexpr int kThreads = kWaves * kWave;
-constexpr int kTerms = 3;
-constexpr int kCols = 16;       // batch rows = MFMA columns
-constexpr int kSpanTiles = 8;   // tiles staged per round, over all k-slices
+constexpr int kMaxWavesMfma = 8; // 512 threads: up to 256 registers per lane
 
 struct MfmaArgs {
   const float *A;
   const int4 *W0, *W1;
-  const float *s0, *s1, *bias;
+  const float *s0, *s1, *bias, *norm_w;
   float *C;
   int64_t lda, ldc;
-  int K, N, groups, chunks, G, KS, TR, rows;
+  float norm_eps, norm_inv_k;
+  int K, N, groups, chunks, spans; // spans = ceil(groups / SPAN)
+  int GS, KS;                      // spans x k-slices of wavefronts per workgroup
+  int rows;
 };
 
 __device__ __forceinline__ int4 load_stream(const int4 *p) {
@@ -59,160 +69,232 @@ __device__ __forceinline__ float silu(float g) {
   return g * sig;
 }
 
-template <int EPI>
-__global__ void __launch_bounds__(kThreads) gemv_w8a32_mfma_kernel(MfmaArgs a) {
-  constexpr bool DUAL = (EPI == kEpiSiluMul);
-  constexpr int U = DUAL ? 2 : 4;
-  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
-  const int gl = wave / a.KS, ks = wave % a.KS;
-  const int g = blockIdx.x * a.G + gl;
-  const bool live = g < a.groups;
-  const int per = (a.chunks + a.KS - 1) / a.KS; // tiles per k-slice
-  const int t0 = min(ks * per, a.chunks), t1 = min(t0 + per, a.chunks);
-  const int TR = a.TR;
-  const int span = a.KS * TR * kTileK;   // staged k per row and round
-  const int rs = span + 8;               // row stride in bf16 elements
-  u16 *xs = reinterpret_cast<u16 *>(smem); // [kTerms][kCols][rs]
-  float *red = reinterpret_cast<float *>(smem + sizeof(u16) * kTerms * kCols * rs);
-
-  f32x4 acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = {0.f, 0.f, 0.f, 0.f};
-  const size_t wbase = ((size_t)(live ? g : 0) * a.chunks) * 64 + lane;
-  const int4 *w0 = a.W0 + wbase;
-  const int4 *w1 = DUAL ? a.W1 + wbase : a.W0 + wbase;
-  const int m = lane & 15, kg = lane >> 4;
-  const int nrounds = (per + TR - 1) / TR;
-
-  for (int rd = 0; rd < nrounds; ++rd) {
-    const int r0 = t0 + rd * TR, r1 = min(r0 + TR, t1);
-    int4 wa[U], wb[U];
-    if (r0 < r1) {
+// 8 f32 -> three bf16x8 terms, each the truncation of what the ones before it
+// left over (8 + 8 + 8 significand bits: the sum is the f32 value).
+__device__ __forceinline__ void split3(const float (&x)[8], bf16x8 (&t)[3]) {
+  float r[8];
 #pragma unroll
-      for (int u = 0; u < U; ++u) {
-        const int t = min(r0 + u, a.chunks - 1);
-        wa[u] = load_stream(w0 + (size_t)t * 64);
-        if (DUAL)
-          wb[u] = load_stream(w1 + (size_t)t * 64);
-      }
+  for (int e = 0; e < 8; ++e)
+    r[e] = x[e];
+#pragma unroll
+  for (int term = 0; term < 3; ++term) {
+    unsigned h[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      h[e] = __float_as_uint(r[e]) & 0xffff0000u;
+      r[e] -= __uint_as_float(h[e]);
     }
-    if (rd != 0)
-      __syncthreads();
-    // stage: slice s of the round covers tiles s*per + rd*TR .. + TR
-    for (int i = tid; i < kCols * (span / 4); i += kThreads) {
-      const int row = i / (span / 4), q = i % (span / 4);
-      const int kk = q * 4; // position inside the staged span
-      const int s = kk / (TR * kTileK), within = kk % (TR * kTileK);
-      const int sl0 = min(s * per, a.chunks);
-      const int kend = min(a.K, min(sl0 + per, a.chunks) * kTileK);
-      const int k = (sl0 + rd * TR) * kTileK + within;
-      float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-      if (row < a.rows && k < kend) {
-        const float *src = a.A + (int64_t)row * a.lda + k;
-        if (k + 3 < kend && ((reinterpret_cast<uintptr_t>(src) & 15) == 0))
-          v = *reinterpret_cast<const float4 *>(src);
-        else
-          v = make_float4(src[0], k + 1 < kend ? src[1] : 0.f,
-                          k + 2 < kend ? src[2] : 0.f, k + 3 < kend ? src[3] : 0.f);
-      }
-      // three truncated bf16 terms: each residual is exactly representable
-      float r[4] = {v.x, v.y, v.z, v.w};
+    union {
+      uint4 u;
+      bf16x8 v;
+    } p;
+    p.u = make_uint4((h[0] >> 16) | h[1], (h[2] >> 16) | h[3], (h[4] >> 16) | h[5],
+                     (h[6] >> 16) | h[7]);
+    t[term] = p.v;
+  }
+}
+
+// A clamped load near the end of a row is shifted: put the values of the 16-k
+// run that starts at k back on their k and zero what lies beyond K.
+__device__ __forceinline__ void fix_row_end(float (&v)[16], int k, int K) {
 #pragma unroll
-      for (int t = 0; t < kTerms; ++t) {
-        unsigned h[4];
+  for (int q = 0; q < 4; ++q) {
+    const int kq = k + 4 * q, sh = kq - min(kq, K - 4);
+    if (sh != 0) {
+      const float o[4] = {v[4 * q], v[4 * q + 1], v[4 * q + 2], v[4 * q + 3]};
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          h[e] = __float_as_uint(r[e]) & 0xffff0000u;
-          r[e] -= __uint_as_float(h[e]);
-        }
-        *reinterpret_cast<uint2 *>(xs + ((size_t)t * kCols + row) * rs + kk) =
-            make_uint2((h[0] >> 16) | h[1], (h[2] >> 16) | h[3]);
-      }
-    }
-    __syncthreads();
-    const u16 *xrow = xs + (size_t)m * rs + ks * TR * kTileK + kg * 16;
-    for (int t = r0; t < r1; t += U) {
-      int4 na[U], nb[U];
-      const bool more = t + U < r1;
-      if (more) {
+      for (int e = 0; e < 4; ++e) {
+        float r = 0.f;
 #pragma unroll
-        for (int u = 0; u < U; ++u) {
-          const int tt = min(t + U + u, a.chunks - 1);
-          na[u] = load_stream(w0 + (size_t)tt * 64);
-          if (DUAL)
-            nb[u] = load_stream(w1 + (size_t)tt * 64);
-        }
-      }
-#pragma unroll
-      for (int u = 0; u < U; ++u) {
-        if (t + u < r1) {
-          const u16 *xt = xrow + (t + u - r0) * kTileK;
-          const bf16x8 a_lo = frag_from(wa[u].x, wa[u].y), a_hi = frag_from(wa[u].z, wa[u].w);
-          bf16x8 b_lo, b_hi;
-          if (DUAL) {
-            b_lo = frag_from(wb[u].x, wb[u].y);
-            b_hi = frag_from(wb[u].z, wb[u].w);
-          }
-#pragma unroll
-          for (int term = 0; term < kTerms; ++term) {
-            const u16 *xp = xt + (size_t)term * kCols * rs;
-            const bf16x8 x_lo = *reinterpret_cast<const bf16x8 *>(xp);
-            const bf16x8 x_hi = *reinterpret_cast<const bf16x8 *>(xp + 8);
-            acc0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_lo, x_lo, acc0, 0, 0, 0);
-            acc0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_hi, x_hi, acc0, 0, 0, 0);
-            if (DUAL) {
-              acc1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(b_lo, x_lo, acc1, 0, 0, 0);
-              acc1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(b_hi, x_hi, acc1, 0, 0, 0);
-            }
-          }
-        }
-      }
-      if (more) {
-#pragma unroll
-        for (int u = 0; u < U; ++u) {
-          wa[u] = na[u];
-          if (DUAL)
-            wb[u] = nb[u];
-        }
+        for (int d = 1; d < 4; ++d)
+          if (e + d < 4 && sh == d)
+            r = o[e + d < 4 ? e + d : 0];
+        v[4 * q + e] = r;
       }
     }
   }
+}
 
-  // k-slices of one channel group meet in LDS, in slice order
-  if (a.KS > 1) {
-    __syncthreads(); // staging area no longer read
-    float *mine = red + (size_t)wave * 64 * 8;
+template <int SPAN, bool DUAL, bool NORM> struct ChunkRegs {
+  int4 w0[SPAN];
+  int4 w1[DUAL ? SPAN : 1];
+  float4 x[4];  // 16 consecutive k of this lane's row
+  float4 nw[NORM ? 4 : 1];
+};
+
+template <int SPAN, bool DUAL, bool NORM>
+__device__ __forceinline__ void load_chunk(const MfmaArgs &a, const int4 *w0,
+                                           const int4 *w1,
+                                           const size_t (&gofs)[SPAN],
+                                           const float *xrow, int kofs, int c,
+                                           ChunkRegs<SPAN, DUAL, NORM> &o) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      mine[lane * 8 + i] = acc0[i];
-      if (DUAL)
-        mine[lane * 8 + 4 + i] = acc1[i];
+  for (int s = 0; s < SPAN; ++s) {
+    o.w0[s] = load_stream(w0 + gofs[s] + (size_t)c * 64);
+    if (DUAL)
+      o.w1[s] = load_stream(w1 + gofs[s] + (size_t)c * 64);
+  }
+  // activations: branch-free, clamped inside the row; what lies beyond K is
+  // multiplied with zero-padded weights (and masked for the sum of squares)
+  const int k = c * kTileK + kofs;
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    const int kq = min(k + 4 * q, a.K - 4);
+    o.x[q] = *reinterpret_cast<const float4 *>(xrow + kq);
+    if (NORM)
+      o.nw[q] = *reinterpret_cast<const float4 *>(a.norm_w + kq);
+  }
+}
+
+template <int EPI, int SPAN, bool NORM>
+__global__ void __launch_bounds__(kMaxWavesMfma *kWave)
+    gemv_w8a32_mfma_kernel(MfmaArgs a) {
+  constexpr bool DUAL = (EPI == kEpiSiluMul);
+  constexpr int NA = DUAL ? 2 * SPAN : SPAN; // accumulators per lane
+  extern __shared__ __attribute__((aligned(16))) float red[];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int sl = wave / a.KS, ks = wave % a.KS;
+  const int span = blockIdx.x * a.GS + sl;
+  const bool live = span < a.spans;
+  const int g0 = (live ? span : 0) * SPAN;
+  const int per = (a.chunks + a.KS - 1) / a.KS;
+  const int c0 = min(ks * per, a.chunks), c1 = min(c0 + per, a.chunks);
+  const int m = lane & 15, kg = lane >> 4;
+
+  f32x4 acc0[SPAN], acc1[DUAL ? SPAN : 1];
+#pragma unroll
+  for (int s = 0; s < SPAN; ++s) {
+    acc0[s] = f32x4{0.f, 0.f, 0.f, 0.f};
+    if (DUAL)
+      acc1[s] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+  float ss = 0.f;
+  // groups past the end of the matrix repeat the last one (never stored)
+  size_t gofs[SPAN];
+#pragma unroll
+  for (int s = 0; s < SPAN; ++s)
+    gofs[s] = (size_t)min(g0 + s, a.groups - 1) * a.chunks * 64;
+  const int4 *w0 = a.W0 + lane;
+  const int4 *w1 = (DUAL ? a.W1 : a.W0) + lane;
+  const float *xrow = a.A + (int64_t)min(m, a.rows - 1) * a.lda;
+  const int kofs = kg * 16;
+
+  ChunkRegs<SPAN, DUAL, NORM> cur, nxt;
+  if (c0 < c1)
+    load_chunk<SPAN, DUAL, NORM>(a, w0, w1, gofs, xrow, kofs, c0, cur);
+  for (int c = c0; c < c1; ++c) {
+    if (c + 1 < c1)
+      load_chunk<SPAN, DUAL, NORM>(a, w0, w1, gofs, xrow, kofs, c + 1, nxt);
+    // this lane's 16 activations -> 2 halves x 3 bf16 terms
+    float xv[16] = {cur.x[0].x, cur.x[0].y, cur.x[0].z, cur.x[0].w,
+                    cur.x[1].x, cur.x[1].y, cur.x[1].z, cur.x[1].w,
+                    cur.x[2].x, cur.x[2].y, cur.x[2].z, cur.x[2].w,
+                    cur.x[3].x, cur.x[3].y, cur.x[3].z, cur.x[3].w};
+    const int k = c * kTileK + kofs;
+    fix_row_end(xv, k, a.K);
+    if (NORM) {
+      float nv[16] = {cur.nw[0].x, cur.nw[0].y, cur.nw[0].z, cur.nw[0].w,
+                      cur.nw[NORM ? 1 : 0].x, cur.nw[NORM ? 1 : 0].y, cur.nw[NORM ? 1 : 0].z, cur.nw[NORM ? 1 : 0].w,
+                      cur.nw[NORM ? 2 : 0].x, cur.nw[NORM ? 2 : 0].y, cur.nw[NORM ? 2 : 0].z, cur.nw[NORM ? 2 : 0].w,
+                      cur.nw[NORM ? 3 : 0].x, cur.nw[NORM ? 3 : 0].y, cur.nw[NORM ? 3 : 0].z, cur.nw[NORM ? 3 : 0].w};
+      fix_row_end(nv, k, a.K);
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        ss = fmaf(xv[e], xv[e], ss);
+        xv[e] *= nv[e];
+      }
     }
+    bf16x8 xlo[3], xhi[3];
+    {
+      const float lo[8] = {xv[0], xv[1], xv[2], xv[3], xv[4], xv[5], xv[6], xv[7]};
+      const float hi[8] = {xv[8], xv[9], xv[10], xv[11], xv[12], xv[13], xv[14], xv[15]};
+      split3(lo, xlo);
+      split3(hi, xhi);
+    }
+#pragma unroll
+    for (int s = 0; s < SPAN; ++s) {
+      const bf16x8 a_lo = frag_from(cur.w0[s].x, cur.w0[s].y);
+      const bf16x8 a_hi = frag_from(cur.w0[s].z, cur.w0[s].w);
+#pragma unroll
+      for (int t = 0; t < 3; ++t) {
+        acc0[s] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_lo, xlo[t], acc0[s], 0, 0, 0);
+        acc0[s] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_hi, xhi[t], acc0[s], 0, 0, 0);
+      }
+      if (DUAL) {
+        const bf16x8 b_lo = frag_from(cur.w1[DUAL ? s : 0].x, cur.w1[DUAL ? s : 0].y);
+        const bf16x8 b_hi = frag_from(cur.w1[DUAL ? s : 0].z, cur.w1[DUAL ? s : 0].w);
+#pragma unroll
+        for (int t = 0; t < 3; ++t) {
+          acc1[DUAL ? s : 0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(b_lo, xlo[t], acc1[DUAL ? s : 0], 0, 0, 0);
+          acc1[DUAL ? s : 0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(b_hi, xhi[t], acc1[DUAL ? s : 0], 0, 0, 0);
+        }
+      }
+    }
+    if (c + 1 < c1)
+      cur = nxt;
+  }
+  if (NORM) { // the four lanes that share a row hold different k
+    ss += __shfl_xor(ss, 16, 64);
+    ss += __shfl_xor(ss, 32, 64);
+  }
+
+  // ---- k-slices meet in LDS, in slice order --------------------------------
+  constexpr int kPerWave = (NA * 4 + 1) * kWave; // floats per wavefront
+  if (a.KS > 1) {
+    float *mine = red + (size_t)wave * kPerWave;
+#pragma unroll
+    for (int s = 0; s < SPAN; ++s)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        mine[(s * 4 + i) * kWave + lane] = acc0[s][i];
+        if (DUAL)
+          mine[((SPAN + s) * 4 + i) * kWave + lane] = acc1[DUAL ? s : 0][i];
+      }
+    if (NORM)
+      mine[NA * 4 * kWave + lane] = ss;
     __syncthreads();
     if (ks != 0)
       return;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      float r0 = 0.f, r1 = 0.f;
-      for (int s = 0; s < a.KS; ++s) {
-        const float *o = red + (size_t)(wave + s) * 64 * 8 + lane * 8;
-        r0 += o[i];
+    for (int s = 0; s < SPAN; ++s)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        float r0 = 0.f, r1 = 0.f;
+        for (int q = 0; q < a.KS; ++q) {
+          const float *o = red + (size_t)(wave + q) * kPerWave;
+          r0 += o[(s * 4 + i) * kWave + lane];
+          if (DUAL)
+            r1 += o[((SPAN + s) * 4 + i) * kWave + lane];
+        }
+        acc0[s][i] = r0;
         if (DUAL)
-          r1 += o[4 + i];
+          acc1[DUAL ? s : 0][i] = r1;
       }
-      acc0[i] = r0;
-      acc1[i] = r1;
+    if (NORM) {
+      float r = 0.f;
+      for (int q = 0; q < a.KS; ++q)
+        r += red[(size_t)(wave + q) * kPerWave + NA * 4 * kWave + lane];
+      ss = r;
     }
   }
-  // lane holds batch row m and channels kg*4 .. kg*4+3 of the group
-  if (live && m < a.rows) {
+  // lane holds batch row m and channels kg*4 .. kg*4+3 of each group
+  if (!live || m >= a.rows)
+    return;
+  const float rn = NORM ? 1.0f / sqrtf(ss * a.norm_inv_k + a.norm_eps) : 1.0f;
+#pragma unroll
+  for (int s = 0; s < SPAN; ++s) {
+    const int g = g0 + s;
+    if (g >= a.groups)
+      continue;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int n = g * kTileN + kg * 4 + i;
       if (n < a.N) {
         float *c = a.C + (int64_t)m * a.ldc + n;
-        const float v = acc0[i] * a.s0[n];
+        const float v = acc0[s][i] * rn * a.s0[n];
         if (EPI == kEpiSiluMul)
-          *c = silu(v) * (acc1[i] * a.s1[n]);
+          *c = silu(v) * (acc1[DUAL ? s : 0][i] * rn * a.s1[n]);
         else if (EPI == kEpiAccum)
           *c = *c + v;
         else
@@ -222,24 +304,43 @@ __global__ void __launch_bounds__(kThreads) gemv_w8a32_mfma_kernel(MfmaArgs a) {
   }
 }
 
-template <int EPI>
-int launch_epi(const MfmaArgs &ka, int blocks, size_t lds, hipStream_t stream) {
-  auto kernel = gemv_w8a32_mfma_kernel<EPI>;
+template <int EPI, int SPAN, bool NORM>
+int launch_kernel(const MfmaArgs &ka, int blocks, hipStream_t stream) {
+  constexpr int NA = (EPI == kEpiSiluMul) ? 2 * SPAN : SPAN;
+  const int waves = ka.GS * ka.KS;
+  const size_t lds = ka.KS > 1 ? sizeof(float) * waves * (size_t)(NA * 4 + 1) * kWave : 0;
+  auto kernel = gemv_w8a32_mfma_kernel<EPI, SPAN, NORM>;
   static bool attr_set = false;
   if (!attr_set) {
     BH_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
                                      hipFuncAttributeMaxDynamicSharedMemorySize,
-                                     96 * 1024));
+                                     144 * 1024));
     attr_set = true;
   }
-  hipLaunchKernelGGL(kernel, dim3(blocks), dim3(kThreads), lds, stream, ka);
+  hipLaunchKernelGGL(kernel, dim3(blocks), dim3(waves * kWave), lds, stream, ka);
   BH_CHECK_HIP(hipGetLastError());
   return BUDDY_HIP_OK;
 }
 
+template <int EPI, int SPAN>
+int launch_norm(const MfmaArgs &ka, int blocks, hipStream_t stream) {
+  return ka.norm_w ? launch_kernel<EPI, SPAN, true>(ka, blocks, stream)
+                   : launch_kernel<EPI, SPAN, false>(ka, blocks, stream);
+}
+
+template <int SPAN>
+int launch_span(const MfmaArgs &ka, int epilogue, int blocks, hipStream_t stream) {
+  switch (epilogue) {
+  case kEpiStore: return launch_norm<kEpiStore, SPAN>(ka, blocks, stream);
+  case kEpiAccum: return launch_norm<kEpiAccum, SPAN>(ka, blocks, stream);
+  case kEpiSiluMul: return launch_norm<kEpiSiluMul, SPAN>(ka, blocks, stream);
+  }
+  return fail(BUDDY_HIP_ERR_ARG, "gemv: unknown epilogue %d", epilogue);
+}
+
 } // namespace
 
-// Small-batch path of launch_gemv (2 <= M <= 16, no fused RMSNorm).
+// Small-batch path of launch_gemv (2 <= M <= 16).
 int launch_gemv_mfma(const GemvArgs &a, hipStream_t stream) {
   MfmaArgs ka;
   ka.A = a.A;
@@ -248,6 +349,9 @@ int launch_gemv_mfma(const GemvArgs &a, hipStream_t stream) {
   ka.s0 = a.s0;
   ka.s1 = a.s1;
   ka.bias = a.bias;
+  ka.norm_w = a.norm_w;
+  ka.norm_eps = a.norm_eps;
+  ka.norm_inv_k = a.norm_inv_k;
   ka.C = a.C;
   ka.lda = a.lda;
   ka.ldc = a.ldc;
@@ -256,24 +360,24 @@ int launch_gemv_mfma(const GemvArgs &a, hipStream_t stream) {
   ka.groups = (int)ceil_div(a.N, kTileN);
   ka.chunks = (int)ceil_div(a.K, kTileK);
   ka.rows = a.M;
-  // k-slices inside the workgroup when the matrix is narrow
+  const bool dual = a.epilogue == kEpiSiluMul;
+  // channel groups per wavefront: four, two when that leaves too few wavefronts
+  // to cover the chip even with 16 k-slices
+  int span = 4;
+  if (ceil_div(ka.groups, 4) * kMaxWavesMfma < 1024)
+    span = 2;
+  ka.spans = (int)ceil_div(ka.groups, span);
+  // k-slices: enough wavefronts for 256 CUs, at least two chunks each; the
+  // meeting place of a two-matrix launch must fit in LDS
   int ks = 1;
-  while (ks < kWaves && ks < kSpanTiles / 2 && (int64_t)ka.groups * ks < 2048 &&
-         ka.chunks / (ks * 2) >= 2)
+  const int ks_max = dual && span == 4 ? 8 : kMaxWavesMfma;
+  while (ks < ks_max && (int64_t)ka.spans * ks < 2048 && ka.chunks / (ks * 2) >= 2)
     ks *= 2;
   ka.KS = ks;
-  ka.G = kWaves / ks;
-  ka.TR = kSpanTiles / ks;
-  const int blocks = (int)ceil_div(ka.groups, ka.G);
-  const int span = kSpanTiles * kTileK;
-  const size_t lds = sizeof(u16) * kTerms * kCols * (span + 8) +
-                     sizeof(float) * kWaves * 64 * 8;
-  switch (a.epilogue) {
-  case kEpiStore: return launch_epi<kEpiStore>(ka, blocks, lds, stream);
-  case kEpiAccum: return launch_epi<kEpiAccum>(ka, blocks, lds, stream);
-  case kEpiSiluMul: return launch_epi<kEpiSiluMul>(ka, blocks, lds, stream);
-  }
-  return fail(BUDDY_HIP_ERR_ARG, "gemv: unknown epilogue %d", a.epilogue);
+  ka.GS = ks < 4 ? 4 / ks : 1;
+  const int blocks = (int)ceil_div(ka.spans, ka.GS);
+  return span == 4 ? launch_span<4>(ka, a.epilogue, blocks, stream)
+                   : launch_span<2>(ka, a.epilogue, blocks, stream);
 }
 
 } // namespace bh

@@ -91,6 +91,43 @@ def test_norm_prologue_and_residual_epilogue(bh, oracle):
     check_close(c.cpu().numpy(), want)
 
 
+@pytest.mark.parametrize("M", [3, 9, 16])
+@pytest.mark.parametrize("K,N", [(1536, 2048), (8960, 1536), (200, 48)])
+def test_small_batch_fusions(bh, oracle, M, K, N):
+    """RMSNorm + bias, residual add and SiLU*mul at batch sizes that run on the
+    f32 FMA kernel (M <= 4) and on the matrix-core kernel (M >= 5)."""
+    q, s = synthetic.quantized_linear(K, N, 31)
+    q2, s2 = synthetic.quantized_linear(K, N, 32)
+    g = torch.Generator(device="cuda").manual_seed(100 + M)
+    x = torch.randn((M, K), generator=g, device="cuda") * 2
+    w = 1 + 0.1 * torch.randn(K, generator=g, device="cuda")
+    bias = torch.randn(N, generator=g, device="cuda")
+    p, p2 = ops.pack_w8(q), ops.pack_w8(q2)
+    xh, wh, qh, sh, q2h, s2h, bh_ = (t.cpu().numpy() for t in (x, w, q, s, q2, s2, bias))
+    xn = np.stack([oracle.rmsnorm(xh[m], wh, EPS) for m in range(M)])
+    # norm + bias
+    out = torch.empty((M, N), device="cuda")
+    linear(bh, A=x, lda=K, W0=p, scale0=s, norm_w=w, norm_eps=float(EPS), bias=bias,
+           C=out, ldc=N, M=M, K=K, N=N, epilogue=0)
+    want = np.stack([bh_ + oracle.dequant_gemv(xn[m], qh, sh) for m in range(M)])
+    check_close(out.cpu().numpy(), want)
+    # norm + SiLU(gate) * up
+    h = torch.empty((M, N), device="cuda")
+    linear(bh, A=x, lda=K, W0=p, scale0=s, W1=p2, scale1=s2, norm_w=w,
+           norm_eps=float(EPS), C=h, ldc=N, M=M, K=K, N=N, epilogue=2)
+    want = np.stack([oracle.silu_mul(oracle.dequant_gemv(xn[m], qh, sh),
+                                     oracle.dequant_gemv(xn[m], q2h, s2h))
+                     for m in range(M)])
+    check_close(h.cpu().numpy(), want)
+    # residual: C += ...
+    c0 = torch.randn((M, N), generator=g, device="cuda")
+    c = c0.clone()
+    linear(bh, A=x, lda=K, W0=p, scale0=s, C=c, ldc=N, M=M, K=K, N=N, epilogue=1)
+    want = np.stack([oracle.dequant_gemv(xh[m], qh, sh, c0.cpu().numpy()[m])
+                     for m in range(M)])
+    check_close(c.cpu().numpy(), want)
+
+
 def test_standalone_elementwise_and_argmax(bh, oracle):
     g = torch.Generator(device="cuda").manual_seed(5)
     x = torch.randn((3, 1536), generator=g, device="cuda") * 2

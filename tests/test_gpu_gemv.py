@@ -85,12 +85,14 @@ def test_narrow_tile_layouts(oracle, K, N, tn):
     check_close(c.cpu().numpy()[0], oracle.dequant_gemv(xh, qh, sh, c0.cpu().numpy()[0]))
 
 
+# (102, 70): K % 4 != 0 keeps every batch size on the f32 FMA kernel; (100, 70)
+# and (1100, 40) end a row inside a 16-k run of the matrix-core kernel
 SHAPES = [(1536, 8960), (8960, 1536), (1536, 1536), (1536, 256), (64, 16), (100, 70),
-          (1536, 151936), (4096, 4096)]
+          (102, 70), (1100, 40), (1536, 151936), (4096, 4096)]
 
 
 @pytest.mark.parametrize("K,N", SHAPES)
-@pytest.mark.parametrize("M", [1, 4, 16])
+@pytest.mark.parametrize("M", [1, 2, 4, 5, 8, 13, 16])
 def test_gemv_matches_oracle(oracle, K, N, M):
     if M > 1 and K * N > 1536 * 8960:
         pytest.skip("large shapes at M=1 only (CPU oracle time)")
