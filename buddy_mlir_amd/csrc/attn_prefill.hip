@@ -9,18 +9,21 @@
 //
 // The reference kernel is handed K and V already repeated to one copy per query
 // head (tosa.py:4578-4579,4700); here the KV head is h / group, so the cache is
-// read in place.  The causal structure is exploited: key tiles that lie wholly
-// in a query tile's future are skipped (they are exactly zero after softmax).
-// Arithmetic is f32 throughout.
+// read in place.  The causal structure is exploited: key blocks that lie wholly
+// in a query block's future are skipped (they are exactly zero after softmax).
+// Arithmetic is f32 throughout, on the f32 matrix cores.
 #include "attn.h"
 
 namespace bh {
 namespace {
 
 constexpr int kD = 128;
-constexpr int TQ = 32, TK = 32;  // query / key rows per tile
-constexpr int LDR = kD + 4;      // padded row length in LDS (floats)
+constexpr int kQB = 16;            // query rows per workgroup
+constexpr int kKB = 16;            // key positions per step of a wavefront
+constexpr int kAttnWaves = 4;      // wavefronts per workgroup; they split the keys
 constexpr float kSeedM = -1.0e30f; // tosa.py:4383
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 struct PrefillArgs {
   const float *q;   // token t, head h at q + t*q_stride + h*q_hstride
@@ -32,122 +35,179 @@ struct PrefillArgs {
   float scale;
 };
 
-__global__ void __launch_bounds__(256) attn_prefill_kernel(PrefillArgs a) {
-  __shared__ float q_s[TQ][LDR];
-  __shared__ float k_s[TK][LDR];
-  __shared__ float v_s[TK][LDR];
-  __shared__ float p_s[TQ][TK + 1];
+// One workgroup: 16 query rows of one head.  Its four wavefronts take the 16-key
+// blocks round robin, each with its own running (max, sum, output), and merge
+// at the end.  All products run on the f32 matrix cores (16x16x4), operands
+// straight from global memory in fragment layout:
+//   S^T[key, query] = K . Q^T   (contraction over d; a lane supplies d =
+//                                32*(lane/16) + j in step j, for K and Q alike)
+//   O^T[d, query]  += V^T . P^T (contraction over the key; the S^T accumulator
+//                                registers ARE the P^T operand of step r: a
+//                                lane holds keys 4*(lane/16) + r of query lane%16)
+// so the scores never leave the registers between the two products.
+__global__ void __launch_bounds__(kAttnWaves *kWave) attn_prefill_kernel(PrefillArgs a) {
+  __shared__ float o_s[kAttnWaves][32][kWave];
+  __shared__ float m_s[kAttnWaves][kQB], l_s[kAttnWaves][kQB];
 
-  const int tid = threadIdx.x;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int h = blockIdx.y, kvh = h / a.group;
-  const int q0 = blockIdx.x * TQ;
-  const int nq = min(TQ, a.q_len - q0);
-  const int qi = tid >> 3, sub = tid & 7; // 8 threads per query row
+  const int q0 = blockIdx.x * kQB;
+  const int nq = min(kQB, a.q_len - q0);
+  const int qi = lane & 15, lg = lane >> 4; // query of this lane; lane group
+  const int qrow = q0 + min(qi, nq - 1);    // rows past the end repeat the last
 
-  for (int i = tid; i < TQ * (kD / 4); i += 256) {
-    const int r = i / (kD / 4), c = (i % (kD / 4)) * 4;
-    float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-    if (r < nq)
-      v = *reinterpret_cast<const float4 *>(a.q + (int64_t)(q0 + r) * a.q_stride +
-                                            (int64_t)h * a.q_hstride + c);
-    *reinterpret_cast<float4 *>(&q_s[r][c]) = v;
-  }
-
-  float m_run = kSeedM, l_run = 0.f;
-  float acc[16];
+  // Q^T fragment: d = 32*lg + j
+  float qf[32];
+  {
+    const float *src = a.q + (int64_t)qrow * a.q_stride + (int64_t)h * a.q_hstride + lg * 32;
 #pragma unroll
-  for (int d = 0; d < 16; ++d)
-    acc[d] = 0.f;
-
-  // last key any query of this tile may see
+    for (int j = 0; j < 32; j += 4) {
+      const float4 v = *reinterpret_cast<const float4 *>(src + j);
+      qf[j] = v.x;
+      qf[j + 1] = v.y;
+      qf[j + 2] = v.z;
+      qf[j + 3] = v.w;
+    }
+  }
+  // last key any query of this workgroup may see
   const int k_last = a.mask ? a.k_len - 1
                             : min(a.k_len - 1, a.q_offset + q0 + nq - 1);
+  const int nblocks = k_last / kKB + 1;
   const float *kbase = a.k + (int64_t)kvh * a.kv_stride * kD;
   const float *vbase = a.v + (int64_t)kvh * a.kv_stride * kD;
 
-  for (int k0 = 0; k0 <= k_last; k0 += TK) {
-    const int nk = min(TK, a.k_len - k0);
-    __syncthreads(); // previous tile consumed (and q_s written, first time)
-    for (int i = tid; i < TK * (kD / 4); i += 256) {
-      const int r = i / (kD / 4), c = (i % (kD / 4)) * 4;
-      float4 kv = make_float4(0.f, 0.f, 0.f, 0.f), vv = kv;
-      if (r < nk) {
-        kv = *reinterpret_cast<const float4 *>(kbase + (int64_t)(k0 + r) * kD + c);
-        vv = *reinterpret_cast<const float4 *>(vbase + (int64_t)(k0 + r) * kD + c);
-      }
-      *reinterpret_cast<float4 *>(&k_s[r][c]) = kv;
-      *reinterpret_cast<float4 *>(&v_s[r][c]) = vv;
-    }
-    __syncthreads();
-    // scores of query qi against keys sub, sub+8, sub+16, sub+24
-    float s[4] = {0.f, 0.f, 0.f, 0.f};
-    for (int d = 0; d < kD; d += 4) {
-      const float4 qv = *reinterpret_cast<const float4 *>(&q_s[qi][d]);
+  float m_run = kSeedM, l_run = 0.f; // l_run: this lane's share of the row sum
+  f32x4 acc[8]; // O^T: acc[2*e + half][r] is d = 64*half + 4*(4*lg + r) + e
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const float4 kv = *reinterpret_cast<const float4 *>(&k_s[sub + 8 * j][d]);
-        s[j] = fmaf(qv.x, kv.x, s[j]);
-        s[j] = fmaf(qv.y, kv.y, s[j]);
-        s[j] = fmaf(qv.z, kv.z, s[j]);
-        s[j] = fmaf(qv.w, kv.w, s[j]);
-      }
+  for (int i = 0; i < 8; ++i)
+    acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  float4 kreg[8], vreg[8], knext[8], vnext[8];
+  auto load_block = [&](int b, float4 (&kr)[8], float4 (&vr)[8]) {
+    const int p0 = b * kKB;
+    // K fragment: key p0 + lane%16, d = 32*lg + 0..31
+    const float *ks = kbase + (int64_t)min(p0 + qi, a.k_len - 1) * kD + lg * 32;
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+      kr[j] = *reinterpret_cast<const float4 *>(ks + 4 * j);
+    // V^T fragments: key p0 + 4*lg + r, d = 64*half + 4*(lane%16) + 0..3
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const float *vs = vbase + (int64_t)min(p0 + 4 * lg + r, a.k_len - 1) * kD + 4 * qi;
+      vr[2 * r] = *reinterpret_cast<const float4 *>(vs);
+      vr[2 * r + 1] = *reinterpret_cast<const float4 *>(vs + 64);
     }
+  };
+  if (wave < nblocks)
+    load_block(wave, kreg, vreg);
+  for (int b = wave; b < nblocks; b += kAttnWaves) {
+    if (b + kAttnWaves < nblocks)
+      load_block(b + kAttnWaves, knext, vnext);
+    // ---- S^T block: keys x queries ------------------------------------------
+    f32x4 st = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      st = __builtin_amdgcn_mfma_f32_16x16x4f32(kreg[j].x, qf[4 * j], st, 0, 0, 0);
+      st = __builtin_amdgcn_mfma_f32_16x16x4f32(kreg[j].y, qf[4 * j + 1], st, 0, 0, 0);
+      st = __builtin_amdgcn_mfma_f32_16x16x4f32(kreg[j].z, qf[4 * j + 2], st, 0, 0, 0);
+      st = __builtin_amdgcn_mfma_f32_16x16x4f32(kreg[j].w, qf[4 * j + 3], st, 0, 0, 0);
+    }
+    // lane holds keys p0 + 4*lg + r of query q0 + qi
+    const int p0 = b * kKB;
+    float sc[4];
     float m_blk = -INFINITY;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int kj = sub + 8 * j, kp = k0 + kj;
-      float sc = s[j] * a.scale;
-      bool ok = qi < nq && kj < nk;
+    for (int r = 0; r < 4; ++r) {
+      const int kp = p0 + 4 * lg + r;
+      float v = st[r] * a.scale;
+      bool ok = qi < nq && kp < a.k_len;
       if (ok) {
         if (a.mask)
-          sc += a.mask[(int64_t)(q0 + qi) * a.k_len + kp];
+          v += a.mask[(int64_t)(q0 + qi) * a.k_len + kp];
         else
           ok = kp <= a.q_offset + q0 + qi;
       }
-      s[j] = ok ? sc : -INFINITY;
-      m_blk = fmaxf(m_blk, s[j]);
+      sc[r] = ok ? v : -INFINITY;
+      m_blk = fmaxf(m_blk, sc[r]);
     }
-    m_blk = fmaxf(m_blk, __shfl_xor(m_blk, 1, 64));
-    m_blk = fmaxf(m_blk, __shfl_xor(m_blk, 2, 64));
-    m_blk = fmaxf(m_blk, __shfl_xor(m_blk, 4, 64));
+    m_blk = fmaxf(m_blk, __shfl_xor(m_blk, 16, 64));
+    m_blk = fmaxf(m_blk, __shfl_xor(m_blk, 32, 64));
     const float m_new = fmaxf(m_run, m_blk); // m_run is finite, so m_new is
     const float alpha = expf(m_run - m_new);
+    float p[4];
     float l_blk = 0.f;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const float p = expf(s[j] - m_new);
-      p_s[qi][sub + 8 * j] = p;
-      l_blk += p;
+    for (int r = 0; r < 4; ++r) {
+      p[r] = expf(sc[r] - m_new);
+      l_blk += p[r];
     }
-    l_blk += __shfl_xor(l_blk, 1, 64);
-    l_blk += __shfl_xor(l_blk, 2, 64);
-    l_blk += __shfl_xor(l_blk, 4, 64);
     l_run = l_run * alpha + l_blk;
     m_run = m_new;
-    __syncthreads(); // p_s complete
-    // acc[d] for d = sub*16 .. +16
+    // ---- O^T += V^T . P^T -----------------------------------------------------
 #pragma unroll
-    for (int d = 0; d < 16; ++d)
-      acc[d] *= alpha;
-    for (int kj = 0; kj < nk; ++kj) {
-      const float p = p_s[qi][kj];
+    for (int i = 0; i < 8; ++i)
+      acc[i] *= alpha;
 #pragma unroll
-      for (int d = 0; d < 16; d += 4) {
-        const float4 vv = *reinterpret_cast<const float4 *>(&v_s[kj][sub * 16 + d]);
-        acc[d] = fmaf(vv.x, p, acc[d]);
-        acc[d + 1] = fmaf(vv.y, p, acc[d + 1]);
-        acc[d + 2] = fmaf(vv.z, p, acc[d + 2]);
-        acc[d + 3] = fmaf(vv.w, p, acc[d + 3]);
+    for (int r = 0; r < 4; ++r) {
+#pragma unroll
+      for (int half = 0; half < 2; ++half) {
+        const float4 vv = vreg[2 * r + half];
+        acc[0 + half] = __builtin_amdgcn_mfma_f32_16x16x4f32(vv.x, p[r], acc[0 + half], 0, 0, 0);
+        acc[2 + half] = __builtin_amdgcn_mfma_f32_16x16x4f32(vv.y, p[r], acc[2 + half], 0, 0, 0);
+        acc[4 + half] = __builtin_amdgcn_mfma_f32_16x16x4f32(vv.z, p[r], acc[4 + half], 0, 0, 0);
+        acc[6 + half] = __builtin_amdgcn_mfma_f32_16x16x4f32(vv.w, p[r], acc[6 + half], 0, 0, 0);
+      }
+    }
+    if (b + kAttnWaves < nblocks) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        kreg[j] = knext[j];
+        vreg[j] = vnext[j];
       }
     }
   }
-  if (qi < nq) {
-    float *o = a.out + (int64_t)(q0 + qi) * a.o_stride + (int64_t)h * a.o_hstride + sub * 16;
+  // this wavefront's row sums: the four lane groups hold different keys
+  l_run += __shfl_xor(l_run, 16, 64);
+  l_run += __shfl_xor(l_run, 32, 64);
+
+  // ---- merge the wavefronts (the reference's combine rule, in wave order) ----
 #pragma unroll
-    for (int d = 0; d < 16; d += 4)
-      *reinterpret_cast<float4 *>(o + d) =
-          make_float4(acc[d] / l_run, acc[d + 1] / l_run, acc[d + 2] / l_run,
-                      acc[d + 3] / l_run);
+  for (int i = 0; i < 8; ++i)
+#pragma unroll
+    for (int r = 0; r < 4; ++r)
+      o_s[wave][i * 4 + r][lane] = acc[i][r];
+  if (lg == 0) {
+    m_s[wave][qi] = m_run;
+    l_s[wave][qi] = l_run;
+  }
+  __syncthreads();
+  float m_all = m_s[0][qi];
+#pragma unroll
+  for (int w = 1; w < kAttnWaves; ++w)
+    m_all = fmaxf(m_all, m_s[w][qi]);
+  float wgt[kAttnWaves], l_all = 0.f;
+#pragma unroll
+  for (int w = 0; w < kAttnWaves; ++w) {
+    wgt[w] = expf(m_s[w][qi] - m_all);
+    l_all = fmaf(l_s[w][qi], wgt[w], l_all);
+  }
+  if (qi >= nq)
+    return;
+  const float inv = 1.0f / l_all;
+  float *o = a.out + (int64_t)(q0 + qi) * a.o_stride + (int64_t)h * a.o_hstride;
+  // wavefront w finishes accumulators 2w and 2w+1 (e = w, both halves)
+#pragma unroll
+  for (int half = 0; half < 2; ++half) {
+    const int i = 2 * wave + half;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      float sum = 0.f;
+#pragma unroll
+      for (int w = 0; w < kAttnWaves; ++w)
+        sum = fmaf(o_s[w][i * 4 + r][lane], wgt[w], sum);
+      o[64 * half + 4 * (4 * lg + r) + wave] = sum * inv;
+    }
   }
 }
 
@@ -219,8 +279,8 @@ int launch_attn_prefill(const AttnPrefillArgs &in, hipStream_t stream) {
   a.k_len = in.k_len;
   a.q_offset = in.k_len - in.q_len; // the last query sees every key
   a.scale = in.scale;
-  hipLaunchKernelGGL(attn_prefill_kernel, dim3((unsigned)ceil_div(in.q_len, TQ), in.heads),
-                     dim3(256), 0, stream, a);
+  hipLaunchKernelGGL(attn_prefill_kernel, dim3((unsigned)ceil_div(in.q_len, kQB), in.heads),
+                     dim3(kAttnWaves * kWave), 0, stream, a);
   BH_CHECK_HIP(hipGetLastError());
   return BUDDY_HIP_OK;
 }
