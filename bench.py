@@ -24,7 +24,7 @@ ROOT = Path(__file__).resolve().parent
 sys.path.insert(0, str(ROOT))
 sys.path.insert(0, str(ROOT / "tests"))
 
-GATE_UP_HBM_TRAFFIC_BYTES = 27903603
+GATE_UP_HBM_TRAFFIC_BYTES = 27916074
 HBM_PEAK_GBPS = 8000.0  # MI355X published HBM3E bandwidth
 CONTEXT = 1024
 
@@ -461,7 +461,7 @@ def main():
             "algorithmic_bytes_per_launch": gu_b,
             "avg_launch_us": gu_s * 1e6,
             # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-            # (13608.5 KiB x 1.99982 + 35 KiB x 1.0, factors from a 256 MiB copy);
+            # (13614.6 KiB x 1.99982 + 35 KiB x 1.0, factors from a 256 MiB copy);
             # a counter reading, not something this script can measure live
             "traffic": GATE_UP_HBM_TRAFFIC_BYTES,
         },
