@@ -243,6 +243,189 @@ __global__ void __launch_bounds__(kSlices *kWave) gemm_w8_bf16_kernel(GemmArgs a
   }
 }
 
+// Wide matrices (enough column tiles to fill the chip without splitting K):
+// a workgroup owns 64 rows x 256 channels, one 64-channel span per wavefront,
+// every wavefront runs the whole K.  The activation fragments of a chunk are the
+// same for the four wavefronts: wavefront w fetches row block w for everyone
+// and leaves it in LDS in fragment order (lane l of fragment f at f*1 KiB +
+// 16 l: conflict-free by construction), so the fragments cross L2 -> CU once per
+// workgroup.  Weights stay on the register path.
+//
+// Global loads run kRing - 2 chunks ahead of the matrix cores.  The compiler
+// sinks ordinary loads down to their first use (and then waits for them there),
+// so the loads of this loop are issued by hand and waited for by hand: a fetch
+// is kFetchLoads loads in a fixed order, vmcnt counts them in order, and each
+// wait names the registers it releases so that nothing reads them earlier.
+constexpr int kRing = 5;
+
+typedef int v4i32 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ void issue_load(v4i32 &dst, const void *p) {
+  asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(dst) : "v"(p) : "memory");
+}
+template <int TERMS> struct FetchRegs {
+  v4i32 w[kGroupsPerWave];
+  v4i32 a[TERMS][2];
+};
+// Waits until at most N loads are in flight; the registers of `f` are only
+// valid after it.
+template <int N, int TERMS> __device__ __forceinline__ void wait_loads(FetchRegs<TERMS> &f) {
+  static_assert(kGroupsPerWave == 4, "operand list below");
+  asm volatile("s_waitcnt vmcnt(%4)"
+               : "+v"(f.w[0]), "+v"(f.w[1]), "+v"(f.w[2]), "+v"(f.w[3])
+               : "n"(N)
+               : "memory");
+#pragma unroll
+  for (int t = 0; t < TERMS; ++t)
+    asm volatile("" : "+v"(f.a[t][0]), "+v"(f.a[t][1])::"memory");
+}
+__device__ __forceinline__ bf16x8 frag_from_v(int lo, int hi) { return frag_from(lo, hi); }
+
+template <int TERMS>
+__global__ void __launch_bounds__(kSlices *kWave) gemm_w8_bf16_wide_kernel(GemmArgs a) {
+  constexpr int L = kGroupsPerWave + 2 * TERMS; // loads per fetch
+  extern __shared__ __attribute__((aligned(16))) v4i32 frag_s[]; // [2][TERMS][8][64]
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int col = blockIdx.x % a.cols_padded, rbk = blockIdx.x / a.cols_padded;
+  if (col >= a.ncols)
+    return; // padding id
+  const int m0 = rbk * kRowsPerWave;
+  const int g0 = (col * kSlices + wave) * kGroupsPerWave;
+
+  f32x4 acc[kGroupsPerWave][4];
+#pragma unroll
+  for (int g = 0; g < kGroupsPerWave; ++g)
+#pragma unroll
+    for (int rb = 0; rb < 4; ++rb)
+      acc[g][rb] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  const int4 *wp[kGroupsPerWave];
+#pragma unroll
+  for (int g = 0; g < kGroupsPerWave; ++g) // groups past the end repeat the last one
+    wp[g] = a.W + ((size_t)min(g0 + g, a.groups - 1) * a.chunks) * 64 + lane;
+  const size_t term_stride = (size_t)a.Mp * a.Kp;
+  // this wavefront fetches row block `wave` of the activation tile
+  const u16 *ap = a.Abf + (size_t)(m0 + wave * 16 + (lane & 15)) * a.Kp + (lane >> 4) * 16;
+
+  FetchRegs<TERMS> ring[kRing];
+  // chunks past the end are fetched again from the last chunk (never used):
+  // every fetch is exactly L loads, which is what keeps the counts below exact
+  auto fetch = [&](int c, FetchRegs<TERMS> &f) {
+    const int cc = min(c, a.chunks - 1);
+#pragma unroll
+    for (int g = 0; g < kGroupsPerWave; ++g)
+      issue_load(f.w[g], wp[g] + (size_t)cc * 64);
+#pragma unroll
+    for (int t = 0; t < TERMS; ++t) {
+      const u16 *src = ap + t * term_stride + (size_t)cc * kTileK;
+      issue_load(f.a[t][0], src);
+      issue_load(f.a[t][1], src + 8);
+    }
+  };
+  auto stage = [&](const FetchRegs<TERMS> &f, int buf) { // own row block -> LDS
+#pragma unroll
+    for (int t = 0; t < TERMS; ++t) {
+      v4i32 *dst = frag_s + (((size_t)buf * TERMS + t) * 8 + wave * 2) * kWave + lane;
+      dst[0] = f.a[t][0];
+      dst[kWave] = f.a[t][1];
+    }
+  };
+#pragma unroll
+  for (int u = 0; u < kRing; ++u)
+    fetch(u, ring[u]);
+  wait_loads<(kRing - 1) * L, TERMS>(ring[0]); // chunk 0 has arrived
+  stage(ring[0], 0);
+  __syncthreads();
+  for (int c0 = 0; c0 < a.chunks; c0 += kRing) {
+#pragma unroll
+    for (int u = 0; u < kRing; ++u) {
+      const int c = c0 + u;
+      if (c < a.chunks) {
+        const int buf = c & 1;
+        FetchRegs<TERMS> &cur = ring[u];
+        FetchRegs<TERMS> &nxt = ring[(u + 1) % kRing];
+        // in flight: chunks c+1 .. c+kRing-1 (chunk c was waited for when it was
+        // staged).  Release chunk c+1 and put its row block into the other
+        // buffer, whose readers passed the barrier that closed chunk c-1.
+        wait_loads<(kRing - 2) * L, TERMS>(nxt);
+        stage(nxt, buf ^ 1);
+        bf16x8 wf[kGroupsPerWave][2];
+#pragma unroll
+        for (int g = 0; g < kGroupsPerWave; ++g) {
+          wf[g][0] = frag_from(cur.w[g].x, cur.w[g].y);
+          wf[g][1] = frag_from(cur.w[g].z, cur.w[g].w);
+        }
+#pragma unroll
+        for (int t = 0; t < TERMS; ++t)
+#pragma unroll
+          for (int rb = 0; rb < 4; ++rb) {
+            const v4i32 *src = frag_s + (((size_t)buf * TERMS + t) * 8 + rb * 2) * kWave + lane;
+            union {
+              v4i32 i;
+              bf16x8 v;
+            } a0, a1;
+            a0.i = src[0];
+            a1.i = src[kWave];
+#pragma unroll
+            for (int g = 0; g < kGroupsPerWave; ++g) {
+              acc[g][rb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[g][0], a0.v, acc[g][rb], 0, 0, 0);
+              acc[g][rb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[g][1], a1.v, acc[g][rb], 0, 0, 0);
+            }
+          }
+        // the registers of chunk c are free: fetch the chunk kRing further on
+        // (its weights were converted above; wf holds them now)
+        fetch(c + kRing, cur);
+        __syncthreads();
+      }
+    }
+  }
+  // loads of the repeated last chunk may still be in flight
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+
+  // ---- epilogue: lane holds channels n..n+3 of row m for each row block ------
+#pragma unroll
+  for (int g = 0; g < kGroupsPerWave; ++g) {
+    if (g0 + g >= a.groups)
+      continue;
+    const int n = (g0 + g) * kTileN + (lane >> 4) * 4;
+    float s[4], b[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      s[r] = n + r < a.N ? a.scale[n + r] : 0.f;
+      b[r] = (a.bias && n + r < a.N) ? a.bias[n + r] : 0.f;
+    }
+    const bool vec = n + 3 < a.N && (a.ldc & 3) == 0 &&
+                     (reinterpret_cast<uintptr_t>(a.C) & 15) == 0;
+#pragma unroll
+    for (int rb = 0; rb < 4; ++rb) {
+      const int m = m0 + rb * 16 + (lane & 15);
+      if (m >= a.M)
+        continue;
+      float v[4];
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        v[r] = acc[g][rb][r] * s[r];
+      float *c = a.C + (int64_t)m * a.ldc + n;
+      if (vec) {
+        float4 o = make_float4(v[0], v[1], v[2], v[3]);
+        if (a.accumulate) {
+          const float4 p = *reinterpret_cast<const float4 *>(c);
+          o = make_float4(p.x + o.x, p.y + o.y, p.z + o.z, p.w + o.w);
+        } else {
+          o = make_float4(b[0] + o.x, b[1] + o.y, b[2] + o.z, b[3] + o.w);
+        }
+        *reinterpret_cast<float4 *>(c) = o;
+      } else {
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+          if (n + r < a.N)
+            c[r] = a.accumulate ? c[r] + v[r] : b[r] + v[r];
+      }
+    }
+  }
+}
+
 // bf16 staging of the activations: one grow-only device buffer per stream, so
 // that calls on different streams do not share it.  Calls on one stream are
 // ordered, and the buffer is only read by the matmul that follows the
@@ -268,6 +451,15 @@ int staging_for(hipStream_t stream, size_t bytes, u16 **out) {
     s.bytes = bytes;
   }
   *out = s.ptr;
+  return BUDDY_HIP_OK;
+}
+
+template <int TERMS>
+int launch_wide(const GemmArgs &a, unsigned blocks, hipStream_t stream) {
+  constexpr size_t lds = sizeof(v4i32) * 2 * TERMS * 8 * kWave;
+  hipLaunchKernelGGL(gemm_w8_bf16_wide_kernel<TERMS>, dim3(blocks), dim3(kSlices * kWave),
+                     lds, stream, a);
+  BH_CHECK_HIP(hipGetLastError());
   return BUDDY_HIP_OK;
 }
 
@@ -325,6 +517,18 @@ int launch_gemm_w8(const GemmW8Args &in, hipStream_t stream) {
                      dim3(256), 0, stream, in.A, in.lda, a.M, (int)in.K, a.Mp, a.Kp,
                      in.terms, abf);
   BH_CHECK_HIP(hipGetLastError());
+  // wide matrices: a workgroup per 64 rows x 256 channels, no split of K
+  const int wide_cols = (int)ceil_div(a.groups, kGroupsPerWave * kSlices);
+  if ((int64_t)wide_cols * (a.Mp / kRowsPerWave) >= 200) {
+    a.ncols = wide_cols;
+    a.cols_padded = (int)round_up(wide_cols, 8);
+    const unsigned wb = (unsigned)(a.cols_padded * (a.Mp / kRowsPerWave));
+    switch (in.terms) {
+    case 1: return launch_wide<1>(a, wb, stream);
+    case 2: return launch_wide<2>(a, wb, stream);
+    default: return launch_wide<3>(a, wb, stream);
+    }
+  }
   const unsigned blocks = (unsigned)(a.cols_padded * (a.Mp / kRowsPerWave));
   switch (in.terms) {
   case 1: return launch_terms<1>(a, blocks, stream);
