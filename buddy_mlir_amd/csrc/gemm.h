@@ -16,6 +16,9 @@ struct GemmW8Args {
   int64_t M = 0, K = 0, N = 0;
   bool accumulate = false;
   int terms = 1; // bf16 terms per activation: 1 = cast to bf16, 3 = all f32 bits
+  // A (same pointer, shape, terms, contents) was the input of the previous
+  // matmul on this stream: its bf16 copy is still staged, skip the conversion
+  bool reuse_staged_a = false;
 };
 
 int launch_gemm_w8(const GemmW8Args &a, hipStream_t stream);

@@ -433,13 +433,25 @@ __global__ void __launch_bounds__(kSlices *kWave) gemm_w8_bf16_wide_kernel(GemmA
 struct Staging {
   u16 *ptr = nullptr;
   size_t bytes = 0;
+  // what the buffer holds
+  const float *src = nullptr;
+  int64_t lda = 0;
+  int M = 0, K = 0, terms = 0;
 };
 std::mutex g_staging_mutex;
 std::map<hipStream_t, Staging> g_staging;
 
-int staging_for(hipStream_t stream, size_t bytes, u16 **out) {
+int staging_for(hipStream_t stream, size_t bytes, const GemmW8Args &in, u16 **out,
+                bool *holds_input) {
   std::lock_guard<std::mutex> lock(g_staging_mutex);
   Staging &s = g_staging[stream];
+  *holds_input = in.reuse_staged_a && s.ptr && s.src == in.A && s.lda == in.lda &&
+                 s.M == (int)in.M && s.K == (int)in.K && s.terms == in.terms;
+  s.src = in.A;
+  s.lda = in.lda;
+  s.M = (int)in.M;
+  s.K = (int)in.K;
+  s.terms = in.terms;
   if (s.bytes < bytes) {
     if (s.ptr) {
       BH_CHECK_HIP(hipStreamSynchronize(stream)); // an earlier matmul may still read it
@@ -508,15 +520,19 @@ int launch_gemm_w8(const GemmW8Args &in, hipStream_t stream) {
   a.cols_padded = (int)round_up(a.ncols, 8);
   a.accumulate = in.accumulate ? 1 : 0;
   u16 *abf = nullptr;
-  int rc = staging_for(stream, sizeof(u16) * in.terms * (size_t)a.Mp * a.Kp, &abf);
+  bool staged = false;
+  int rc = staging_for(stream, sizeof(u16) * in.terms * (size_t)a.Mp * a.Kp, in, &abf,
+                       &staged);
   if (rc)
     return rc;
   a.Abf = abf;
-  const int64_t threads = (int64_t)a.Mp * (a.Kp / 8);
-  hipLaunchKernelGGL(activations_to_bf16, dim3((unsigned)ceil_div(threads, 256)),
-                     dim3(256), 0, stream, in.A, in.lda, a.M, (int)in.K, a.Mp, a.Kp,
-                     in.terms, abf);
-  BH_CHECK_HIP(hipGetLastError());
+  if (!staged) {
+    const int64_t threads = (int64_t)a.Mp * (a.Kp / 8);
+    hipLaunchKernelGGL(activations_to_bf16, dim3((unsigned)ceil_div(threads, 256)),
+                       dim3(256), 0, stream, in.A, in.lda, a.M, (int)in.K, a.Mp, a.Kp,
+                       in.terms, abf);
+    BH_CHECK_HIP(hipGetLastError());
+  }
   // wide matrices: a workgroup per 64 rows x 256 channels, no split of K
   const int wide_cols = (int)ceil_div(a.groups, kGroupsPerWave * kSlices);
   if ((int64_t)wide_cols * (a.Mp / kRowsPerWave) >= 200) {

@@ -272,7 +272,8 @@ struct Session {
     return BUDDY_HIP_OK;
   }
 
-  int gemm(const float *A, const PackedLinear &W, float *C, int64_t M, bool accumulate) {
+  int gemm(const float *A, const PackedLinear &W, float *C, int64_t M, bool accumulate,
+           bool same_input_as_before = false) {
     GemmW8Args g;
     g.A = A;
     g.lda = W.K;
@@ -286,6 +287,7 @@ struct Session {
     g.N = W.N;
     g.accumulate = accumulate;
     g.terms = gemm_terms;
+    g.reuse_staged_a = same_input_as_before;
     return launch_gemm_w8(g, stream);
   }
 
@@ -341,7 +343,7 @@ struct Session {
         return rc;
       if ((rc = gemm(pf_xn, L.gate, pf_g, n, false)))
         return rc;
-      if ((rc = gemm(pf_xn, L.up, pf_u, n, false)))
+      if ((rc = gemm(pf_xn, L.up, pf_u, n, false, true)))
         return rc;
       if ((rc = launch_silu_mul(pf_g, pf_u, pf_g, (int64_t)n * S.inter, stream)))
         return rc;
