@@ -115,35 +115,79 @@ __device__ __forceinline__ void fix_row_end(float (&v)[16], int k, int K) {
   }
 }
 
-template <int SPAN, bool DUAL, bool NORM> struct ChunkRegs {
-  int4 w0[SPAN];
-  int4 w1[DUAL ? SPAN : 1];
-  float4 x[4];  // 16 consecutive k of this lane's row
-  float4 nw[NORM ? 4 : 1];
+// The loads of the main loop are issued and waited for by hand: the compiler
+// sinks ordinary prefetch loads down to their first use and then waits for them
+// there.  A fetch is a fixed number of loads in a fixed order, vmcnt counts them
+// in order, and each wait names the registers it releases so that nothing reads
+// them earlier.
+typedef float v4f32 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ void issue_load(v4i &dst, const void *p) {
+  asm volatile("global_load_dwordx4 %0, %1, off nt" : "=v"(dst) : "v"(p) : "memory");
+}
+__device__ __forceinline__ void issue_load(v4f32 &dst, const void *p) {
+  asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(dst) : "v"(p) : "memory");
+}
+
+template <int SPAN, bool DUAL, bool NORM> struct FetchRegs {
+  v4i w0[SPAN];
+  v4i w1[DUAL ? SPAN : 1];
+  v4f32 x[4];  // 16 consecutive k of this lane's row
+  v4f32 nw[NORM ? 4 : 1];
 };
+template <int SPAN, bool DUAL, bool NORM> constexpr int fetch_loads() {
+  return SPAN * (DUAL ? 2 : 1) + 4 * (NORM ? 2 : 1);
+}
 
 template <int SPAN, bool DUAL, bool NORM>
-__device__ __forceinline__ void load_chunk(const MfmaArgs &a, const int4 *w0,
-                                           const int4 *w1,
-                                           const size_t (&gofs)[SPAN],
-                                           const float *xrow, int kofs, int c,
-                                           ChunkRegs<SPAN, DUAL, NORM> &o) {
+__device__ __forceinline__ void fetch_chunk(const MfmaArgs &a, const int4 *w0,
+                                            const int4 *w1,
+                                            const size_t (&gofs)[SPAN],
+                                            const float *xrow, int kofs, int c,
+                                            FetchRegs<SPAN, DUAL, NORM> &o) {
 #pragma unroll
   for (int s = 0; s < SPAN; ++s) {
-    o.w0[s] = load_stream(w0 + gofs[s] + (size_t)c * 64);
+    issue_load(o.w0[s], w0 + gofs[s] + (size_t)c * 64);
     if (DUAL)
-      o.w1[s] = load_stream(w1 + gofs[s] + (size_t)c * 64);
+      issue_load(o.w1[s], w1 + gofs[s] + (size_t)c * 64);
   }
-  // activations: branch-free, clamped inside the row; what lies beyond K is
-  // multiplied with zero-padded weights (and masked for the sum of squares)
+  // activations: clamped inside the row; the last chunk of a ragged row is
+  // put right when it is consumed
   const int k = c * kTileK + kofs;
 #pragma unroll
   for (int q = 0; q < 4; ++q) {
     const int kq = min(k + 4 * q, a.K - 4);
-    o.x[q] = *reinterpret_cast<const float4 *>(xrow + kq);
+    issue_load(o.x[q], xrow + kq);
     if (NORM)
-      o.nw[q] = *reinterpret_cast<const float4 *>(a.norm_w + kq);
+      issue_load(o.nw[q], a.norm_w + kq);
   }
+}
+
+// Waits until at most N loads are in flight; the registers of `f` are valid
+// only after it.
+template <int N, int SPAN, bool DUAL, bool NORM>
+__device__ __forceinline__ void wait_fetch(FetchRegs<SPAN, DUAL, NORM> &f) {
+  asm volatile("s_waitcnt vmcnt(%4)"
+               : "+v"(f.x[0]), "+v"(f.x[1]), "+v"(f.x[2]), "+v"(f.x[3])
+               : "n"(N)
+               : "memory");
+#pragma unroll
+  for (int s = 0; s < SPAN; ++s) {
+    asm volatile("" : "+v"(f.w0[s])::"memory");
+    if (DUAL)
+      asm volatile("" : "+v"(f.w1[DUAL ? s : 0])::"memory");
+  }
+  if (NORM) {
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+      asm volatile("" : "+v"(f.nw[NORM ? q : 0])::"memory");
+  }
+}
+
+// Fetches kept in flight: three, two when a fetch is wide (two matrices or a
+// fused norm) so that the ring stays inside 256 registers.
+template <int SPAN, bool DUAL, bool NORM> constexpr int kRingOf() {
+  return (DUAL || NORM || SPAN > 4) ? 2 : 3;
 }
 
 template <int EPI, int SPAN, bool NORM>
@@ -180,25 +224,39 @@ __global__ void __launch_bounds__(kMaxWavesMfma *kWave)
   const float *xrow = a.A + (int64_t)min(m, a.rows - 1) * a.lda;
   const int kofs = kg * 16;
 
-  ChunkRegs<SPAN, DUAL, NORM> cur, nxt;
-  if (c0 < c1)
-    load_chunk<SPAN, DUAL, NORM>(a, w0, w1, gofs, xrow, kofs, c0, cur);
-  for (int c = c0; c < c1; ++c) {
-    if (c + 1 < c1)
-      load_chunk<SPAN, DUAL, NORM>(a, w0, w1, gofs, xrow, kofs, c + 1, nxt);
+  constexpr int L = fetch_loads<SPAN, DUAL, NORM>();
+  constexpr int R = kRingOf<SPAN, DUAL, NORM>(); // fetches in flight
+  FetchRegs<SPAN, DUAL, NORM> ring[R];
+  // chunks past the end of the slice are fetched again from its last chunk
+  // (never used): every fetch is exactly L loads, which keeps the counts exact
+  const int clast = max(c1 - 1, 0);
+#pragma unroll
+  for (int u = 0; u < R; ++u)
+    fetch_chunk<SPAN, DUAL, NORM>(a, w0, w1, gofs, xrow, kofs, min(c0 + u, clast), ring[u]);
+  const bool ragged = (a.K & (kTileK - 1)) != 0;
+  for (int cb = c0; cb < c1; cb += R) {
+#pragma unroll
+    for (int u = 0; u < R; ++u) {
+      const int c = cb + u;
+      if (c >= c1)
+        continue;
+      FetchRegs<SPAN, DUAL, NORM> &cur = ring[u];
+      wait_fetch<(R - 1) * L, SPAN, DUAL, NORM>(cur); // chunk c has arrived
     // this lane's 16 activations -> 2 halves x 3 bf16 terms
     float xv[16] = {cur.x[0].x, cur.x[0].y, cur.x[0].z, cur.x[0].w,
                     cur.x[1].x, cur.x[1].y, cur.x[1].z, cur.x[1].w,
                     cur.x[2].x, cur.x[2].y, cur.x[2].z, cur.x[2].w,
                     cur.x[3].x, cur.x[3].y, cur.x[3].z, cur.x[3].w};
     const int k = c * kTileK + kofs;
-    fix_row_end(xv, k, a.K);
+    if (ragged && c == a.chunks - 1)
+      fix_row_end(xv, k, a.K);
     if (NORM) {
       float nv[16] = {cur.nw[0].x, cur.nw[0].y, cur.nw[0].z, cur.nw[0].w,
                       cur.nw[NORM ? 1 : 0].x, cur.nw[NORM ? 1 : 0].y, cur.nw[NORM ? 1 : 0].z, cur.nw[NORM ? 1 : 0].w,
                       cur.nw[NORM ? 2 : 0].x, cur.nw[NORM ? 2 : 0].y, cur.nw[NORM ? 2 : 0].z, cur.nw[NORM ? 2 : 0].w,
                       cur.nw[NORM ? 3 : 0].x, cur.nw[NORM ? 3 : 0].y, cur.nw[NORM ? 3 : 0].z, cur.nw[NORM ? 3 : 0].w};
-      fix_row_end(nv, k, a.K);
+      if (ragged && c == a.chunks - 1)
+        fix_row_end(nv, k, a.K);
 #pragma unroll
       for (int e = 0; e < 16; ++e) {
         ss = fmaf(xv[e], xv[e], ss);
@@ -231,9 +289,11 @@ __global__ void __launch_bounds__(kMaxWavesMfma *kWave)
         }
       }
     }
-    if (c + 1 < c1)
-      cur = nxt;
+      // the registers of chunk c are free: fetch the chunk R further on
+      fetch_chunk<SPAN, DUAL, NORM>(a, w0, w1, gofs, xrow, kofs, min(c + R, clast), cur);
+    }
   }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // repeated last chunks
   if (NORM) { // the four lanes that share a row hold different k
     ss += __shfl_xor(ss, 16, 64);
     ss += __shfl_xor(ss, 32, 64);
@@ -361,10 +421,13 @@ int launch_gemv_mfma(const GemvArgs &a, hipStream_t stream) {
   ka.chunks = (int)ceil_div(a.K, kTileK);
   ka.rows = a.M;
   const bool dual = a.epilogue == kEpiSiluMul;
-  // channel groups per wavefront: four, two when that leaves too few wavefronts
-  // to cover the chip even with 16 k-slices
+  // channel groups per wavefront (they share one conversion of the
+  // activations): eight for wide single-matrix launches, else four, two when
+  // that leaves too few wavefronts to cover the chip even with 8 k-slices
   int span = 4;
-  if (ceil_div(ka.groups, 4) * kMaxWavesMfma < 1024)
+  if (!dual && ceil_div(ka.groups, 8) >= 1024)
+    span = 8;
+  else if (ceil_div(ka.groups, 4) * kMaxWavesMfma < 1024)
     span = 2;
   ka.spans = (int)ceil_div(ka.groups, span);
   // k-slices: enough wavefronts for 256 CUs, at least two chunks each; the
@@ -376,6 +439,8 @@ int launch_gemv_mfma(const GemvArgs &a, hipStream_t stream) {
   ka.KS = ks;
   ka.GS = ks < 4 ? 4 / ks : 1;
   const int blocks = (int)ceil_div(ka.spans, ka.GS);
+  if (span == 8)
+    return launch_span<8>(ka, a.epilogue, blocks, stream);
   return span == 4 ? launch_span<4>(ka, a.epilogue, blocks, stream)
                    : launch_span<2>(ka, a.epilogue, blocks, stream);
 }
