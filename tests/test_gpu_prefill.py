@@ -22,7 +22,10 @@ def bf16_round(a: np.ndarray) -> np.ndarray:
 
 
 GEMM_SHAPES = [(512, 1536, 1536), (512, 1536, 256), (512, 1536, 8960), (512, 8960, 1536),
-               (9, 4, 17), (65, 129, 257), (1, 64, 16), (130, 200, 130)]
+               (9, 4, 17), (65, 129, 257), (1, 64, 16), (130, 200, 130),
+               # ragged in every dimension and wide enough for the kernel that does
+               # not split K (64 x 256 workgroup tiles)
+               (500, 200, 6500), (1000, 72, 3300)]
 
 
 @pytest.mark.parametrize("M,K,N", GEMM_SHAPES)
@@ -41,8 +44,8 @@ def test_prefill_gemm_matches_blis_oracle(oracle, M, K, N, exact):
     check_close(y.cpu().numpy(), want)
 
 
-def test_prefill_gemm_accumulates(oracle):
-    M, K, N = 100, 256, 96
+@pytest.mark.parametrize("M,K,N", [(100, 256, 96), (490, 136, 6600)])
+def test_prefill_gemm_accumulates(oracle, M, K, N):
     q, s = synthetic.quantized_linear(K, N, 77)
     g = torch.Generator(device="cuda").manual_seed(1)
     x = torch.randn((M, K), generator=g, device="cuda")
