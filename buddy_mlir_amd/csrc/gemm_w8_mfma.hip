@@ -25,6 +25,7 @@
 //    reference multiplies every element before the FMA.
 #include "gemm.h"
 
+#include <algorithm>
 #include <map>
 #include <mutex>
 
@@ -281,23 +282,25 @@ template <int N, int TERMS> __device__ __forceinline__ void wait_loads(FetchRegs
 }
 __device__ __forceinline__ bf16x8 frag_from_v(int lo, int hi) { return frag_from(lo, hi); }
 
-template <int TERMS>
+// RB = row blocks of 16 per workgroup (4 or 3: whichever leaves the shorter last
+// round of workgroups on the chip).
+template <int TERMS, int RB>
 __global__ void __launch_bounds__(kSlices *kWave) gemm_w8_bf16_wide_kernel(GemmArgs a) {
   constexpr int L = kGroupsPerWave + 2 * TERMS; // loads per fetch
-  extern __shared__ __attribute__((aligned(16))) v4i32 frag_s[]; // [2][TERMS][8][64]
+  extern __shared__ __attribute__((aligned(16))) v4i32 frag_s[]; // [2][TERMS][2 RB][64]
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int col = blockIdx.x % a.cols_padded, rbk = blockIdx.x / a.cols_padded;
   if (col >= a.ncols)
     return; // padding id
-  const int m0 = rbk * kRowsPerWave;
+  const int m0 = rbk * RB * 16;
   const int g0 = (col * kSlices + wave) * kGroupsPerWave;
 
-  f32x4 acc[kGroupsPerWave][4];
+  f32x4 acc[kGroupsPerWave][RB];
 #pragma unroll
   for (int g = 0; g < kGroupsPerWave; ++g)
 #pragma unroll
-    for (int rb = 0; rb < 4; ++rb)
+    for (int rb = 0; rb < RB; ++rb)
       acc[g][rb] = f32x4{0.f, 0.f, 0.f, 0.f};
 
   const int4 *wp[kGroupsPerWave];
@@ -305,8 +308,10 @@ __global__ void __launch_bounds__(kSlices *kWave) gemm_w8_bf16_wide_kernel(GemmA
   for (int g = 0; g < kGroupsPerWave; ++g) // groups past the end repeat the last one
     wp[g] = a.W + ((size_t)min(g0 + g, a.groups - 1) * a.chunks) * 64 + lane;
   const size_t term_stride = (size_t)a.Mp * a.Kp;
-  // this wavefront fetches row block `wave` of the activation tile
-  const u16 *ap = a.Abf + (size_t)(m0 + wave * 16 + (lane & 15)) * a.Kp + (lane >> 4) * 16;
+  // this wavefront fetches row block `wave` of the activation tile (with three
+  // row blocks the fourth wavefront repeats the third's loads and stages nothing)
+  const int my_rb = min(wave, RB - 1);
+  const u16 *ap = a.Abf + (size_t)(m0 + my_rb * 16 + (lane & 15)) * a.Kp + (lane >> 4) * 16;
 
   FetchRegs<TERMS> ring[kRing];
   // chunks past the end are fetched again from the last chunk (never used):
@@ -324,9 +329,11 @@ __global__ void __launch_bounds__(kSlices *kWave) gemm_w8_bf16_wide_kernel(GemmA
     }
   };
   auto stage = [&](const FetchRegs<TERMS> &f, int buf) { // own row block -> LDS
+    if (wave >= RB)
+      return;
 #pragma unroll
     for (int t = 0; t < TERMS; ++t) {
-      v4i32 *dst = frag_s + (((size_t)buf * TERMS + t) * 8 + wave * 2) * kWave + lane;
+      v4i32 *dst = frag_s + (((size_t)buf * TERMS + t) * 2 * RB + wave * 2) * kWave + lane;
       dst[0] = f.a[t][0];
       dst[kWave] = f.a[t][1];
     }
@@ -359,8 +366,8 @@ __global__ void __launch_bounds__(kSlices *kWave) gemm_w8_bf16_wide_kernel(GemmA
 #pragma unroll
         for (int t = 0; t < TERMS; ++t)
 #pragma unroll
-          for (int rb = 0; rb < 4; ++rb) {
-            const v4i32 *src = frag_s + (((size_t)buf * TERMS + t) * 8 + rb * 2) * kWave + lane;
+          for (int rb = 0; rb < RB; ++rb) {
+            const v4i32 *src = frag_s + (((size_t)buf * TERMS + t) * 2 * RB + rb * 2) * kWave + lane;
             union {
               v4i32 i;
               bf16x8 v;
@@ -398,7 +405,7 @@ __global__ void __launch_bounds__(kSlices *kWave) gemm_w8_bf16_wide_kernel(GemmA
     const bool vec = n + 3 < a.N && (a.ldc & 3) == 0 &&
                      (reinterpret_cast<uintptr_t>(a.C) & 15) == 0;
 #pragma unroll
-    for (int rb = 0; rb < 4; ++rb) {
+    for (int rb = 0; rb < RB; ++rb) {
       const int m = m0 + rb * 16 + (lane & 15);
       if (m >= a.M)
         continue;
@@ -466,11 +473,11 @@ int staging_for(hipStream_t stream, size_t bytes, const GemmW8Args &in, u16 **ou
   return BUDDY_HIP_OK;
 }
 
-template <int TERMS>
+template <int TERMS, int RB>
 int launch_wide(const GemmArgs &a, unsigned blocks, hipStream_t stream) {
-  constexpr size_t lds = sizeof(v4i32) * 2 * TERMS * 8 * kWave;
-  hipLaunchKernelGGL(gemm_w8_bf16_wide_kernel<TERMS>, dim3(blocks), dim3(kSlices * kWave),
-                     lds, stream, a);
+  constexpr size_t lds = sizeof(v4i32) * 2 * TERMS * 2 * RB * kWave;
+  hipLaunchKernelGGL((gemm_w8_bf16_wide_kernel<TERMS, RB>), dim3(blocks),
+                     dim3(kSlices * kWave), lds, stream, a);
   BH_CHECK_HIP(hipGetLastError());
   return BUDDY_HIP_OK;
 }
@@ -514,7 +521,8 @@ int launch_gemm_w8(const GemmW8Args &in, hipStream_t stream) {
   a.N = (int)in.N;
   a.groups = (int)ceil_div(in.N, kTileN);
   a.chunks = (int)ceil_div(in.K, kTileK);
-  a.Mp = (int)round_up(in.M, kRowsPerWave);
+  // padded rows cover the last 64-row block and the last 48-row block
+  a.Mp = (int)std::max(round_up(in.M, 64), round_up(in.M, 48));
   a.Kp = a.chunks * kTileK;
   a.ncols = (int)ceil_div(a.groups, kGroupsPerWave);
   a.cols_padded = (int)round_up(a.ncols, 8);
@@ -536,13 +544,26 @@ int launch_gemm_w8(const GemmW8Args &in, hipStream_t stream) {
   // wide matrices: a workgroup per 64 rows x 256 channels, no split of K
   const int wide_cols = (int)ceil_div(a.groups, kGroupsPerWave * kSlices);
   if ((int64_t)wide_cols * (a.Mp / kRowsPerWave) >= 200) {
+    // 64 or 48 rows per workgroup: the chip runs 256 workgroups at a time (one
+    // wavefront per SIMD), so the time is rounds x rows; ties go to 64 rows,
+    // which convert each weight tile fewer times
+    const int64_t wg4 = wide_cols * ceil_div(in.M, 64), wg3 = wide_cols * ceil_div(in.M, 48);
+    const bool three = ceil_div(wg3, 256) * 3 < ceil_div(wg4, 256) * 4;
+    const int rows = three ? 48 : 64;
     a.ncols = wide_cols;
     a.cols_padded = (int)round_up(wide_cols, 8);
-    const unsigned wb = (unsigned)(a.cols_padded * (a.Mp / kRowsPerWave));
+    const unsigned wb = (unsigned)(a.cols_padded * ceil_div(in.M, rows));
+    if (three) {
+      switch (in.terms) {
+      case 1: return launch_wide<1, 3>(a, wb, stream);
+      case 2: return launch_wide<2, 3>(a, wb, stream);
+      default: return launch_wide<3, 3>(a, wb, stream);
+      }
+    }
     switch (in.terms) {
-    case 1: return launch_wide<1>(a, wb, stream);
-    case 2: return launch_wide<2>(a, wb, stream);
-    default: return launch_wide<3>(a, wb, stream);
+    case 1: return launch_wide<1, 4>(a, wb, stream);
+    case 2: return launch_wide<2, 4>(a, wb, stream);
+    default: return launch_wide<3, 4>(a, wb, stream);
     }
   }
   const unsigned blocks = (unsigned)(a.cols_padded * (a.Mp / kRowsPerWave));
