@@ -102,6 +102,71 @@ activations_to_bf16(const float *__restrict__ A, int64_t lda, int M, int K, int 
   }
 }
 
+// 8 consecutive values of a row -> `terms` bf16 terms in the staging layout
+__device__ __forceinline__ void store_terms(float (&r)[8], int terms, u16 *out,
+                                            size_t term_stride) {
+  for (int t = 0; t < terms; ++t) {
+    u16 h[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      h[e] = bf16_rne(r[e]);
+      r[e] -= bf16_to_f32(h[e]);
+    }
+    *reinterpret_cast<uint4 *>(out + t * term_stride) =
+        make_uint4(pack2(h[0], h[1]), pack2(h[2], h[3]), pack2(h[4], h[5]),
+                   pack2(h[6], h[7]));
+  }
+}
+
+// One workgroup per row: y = w * (x * rsqrt(sum(x^2) / n + eps)) -> staging
+__global__ void __launch_bounds__(256)
+rmsnorm_to_staging_kernel(const float *__restrict__ x, const float *__restrict__ w, int n,
+                          float inv_n, float eps, int terms, int Mp, int Kp,
+                          u16 *__restrict__ out) {
+  __shared__ float red[4];
+  const int row = blockIdx.x;
+  const float *xr = x + (size_t)row * n;
+  float s = 0.f;
+  for (int i = threadIdx.x; i < n; i += 256)
+    s = fmaf(xr[i], xr[i], s);
+  s = wave_sum(s);
+  if ((threadIdx.x & 63) == 0)
+    red[threadIdx.x >> 6] = s;
+  __syncthreads();
+  const float tot = (red[0] + red[1]) + (red[2] + red[3]);
+  const float rs = 1.0f / sqrtf(tot * inv_n + eps);
+  for (int k0 = threadIdx.x * 8; k0 < Kp; k0 += 256 * 8) {
+    float r[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e)
+      r[e] = k0 + e < n ? w[k0 + e] * (xr[k0 + e] * rs) : 0.f;
+    store_terms(r, terms, out + (size_t)row * Kp + k0, (size_t)Mp * Kp);
+  }
+}
+
+__global__ void __launch_bounds__(256)
+silu_mul_to_staging_kernel(const float *__restrict__ g, const float *__restrict__ u,
+                           int rows, int n, int terms, int Mp, int Kp,
+                           u16 *__restrict__ out) {
+  const int kq = Kp / 8;
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= (int64_t)rows * kq)
+    return;
+  const int row = (int)(i / kq), k0 = (int)(i % kq) * 8;
+  float r[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    float v = 0.f;
+    if (k0 + e < n) {
+      const float gv = g[(size_t)row * n + k0 + e];
+      const float sig = 1.0f / (1.0f + expf(-gv));
+      v = (gv * sig) * u[(size_t)row * n + k0 + e];
+    }
+    r[e] = v;
+  }
+  store_terms(r, terms, out + (size_t)row * Kp + k0, (size_t)Mp * Kp);
+}
+
 struct GemmArgs {
   const u16 *Abf; // [terms][Mp][Kp]
   const int4 *W;
@@ -500,13 +565,46 @@ int launch_terms(const GemmArgs &a, unsigned blocks, hipStream_t stream) {
 
 } // namespace
 
+GemmStagingLayout gemm_staging_layout(int64_t M, int64_t K) {
+  GemmStagingLayout l;
+  // padded rows cover the last 64-row block and the last 48-row block
+  l.rows_padded = (int)std::max(round_up(M, 64), round_up(M, 48));
+  l.cols_padded = (int)round_up(K, kTileK);
+  return l;
+}
+
+int launch_rmsnorm_to_staging(const float *x, const float *w, int rows, int n, float eps,
+                              int terms, unsigned short *staged, hipStream_t stream) {
+  BH_REQUIRE(x && w && staged && rows > 0 && n > 0 && terms >= 1 && terms <= 3,
+             "rmsnorm_to_staging: bad argument");
+  const GemmStagingLayout l = gemm_staging_layout(rows, n);
+  hipLaunchKernelGGL(rmsnorm_to_staging_kernel, dim3(rows), dim3(256), 0, stream, x, w, n,
+                     1.0f / (float)n, eps, terms, l.rows_padded, l.cols_padded, staged);
+  BH_CHECK_HIP(hipGetLastError());
+  return BUDDY_HIP_OK;
+}
+
+int launch_silu_mul_to_staging(const float *g, const float *u, int rows, int n, int terms,
+                               unsigned short *staged, hipStream_t stream) {
+  BH_REQUIRE(g && u && staged && rows > 0 && n > 0 && terms >= 1 && terms <= 3,
+             "silu_mul_to_staging: bad argument");
+  const GemmStagingLayout l = gemm_staging_layout(rows, n);
+  const int64_t threads = (int64_t)rows * (l.cols_padded / 8);
+  hipLaunchKernelGGL(silu_mul_to_staging_kernel, dim3((unsigned)ceil_div(threads, 256)),
+                     dim3(256), 0, stream, g, u, rows, n, terms, l.rows_padded,
+                     l.cols_padded, staged);
+  BH_CHECK_HIP(hipGetLastError());
+  return BUDDY_HIP_OK;
+}
+
 int launch_gemm_w8(const GemmW8Args &in, hipStream_t stream) {
-  BH_REQUIRE(in.A && in.W && in.scale && in.C, "gemm_w8: null pointer");
+  BH_REQUIRE((in.A || in.staged) && in.W && in.scale && in.C, "gemm_w8: null pointer");
   BH_REQUIRE(in.M > 0 && in.K > 0 && in.N > 0 && in.M < (1 << 24) &&
                  in.K < (1 << 24) && in.N < (1 << 24),
              "gemm_w8: bad shape M=%lld K=%lld N=%lld", (long long)in.M,
              (long long)in.K, (long long)in.N);
-  BH_REQUIRE(in.lda >= in.K && in.ldc >= in.N, "gemm_w8: row stride below row length");
+  BH_REQUIRE((in.staged || in.lda >= in.K) && in.ldc >= in.N,
+             "gemm_w8: row stride below row length");
   BH_REQUIRE(in.terms >= 1 && in.terms <= 3, "gemm_w8: terms=%d outside 1..3", in.terms);
   BH_REQUIRE(!(in.bias && in.accumulate), "gemm_w8: bias with accumulate");
   BH_REQUIRE((reinterpret_cast<uintptr_t>(in.W) & 15) == 0,
@@ -521,15 +619,15 @@ int launch_gemm_w8(const GemmW8Args &in, hipStream_t stream) {
   a.N = (int)in.N;
   a.groups = (int)ceil_div(in.N, kTileN);
   a.chunks = (int)ceil_div(in.K, kTileK);
-  // padded rows cover the last 64-row block and the last 48-row block
-  a.Mp = (int)std::max(round_up(in.M, 64), round_up(in.M, 48));
-  a.Kp = a.chunks * kTileK;
+  const GemmStagingLayout layout = gemm_staging_layout(in.M, in.K);
+  a.Mp = layout.rows_padded;
+  a.Kp = layout.cols_padded;
   a.ncols = (int)ceil_div(a.groups, kGroupsPerWave);
   a.cols_padded = (int)round_up(a.ncols, 8);
   a.accumulate = in.accumulate ? 1 : 0;
-  u16 *abf = nullptr;
-  bool staged = false;
-  int rc = staging_for(stream, sizeof(u16) * in.terms * (size_t)a.Mp * a.Kp, in, &abf,
+  u16 *abf = const_cast<u16 *>(in.staged);
+  bool staged = in.staged != nullptr;
+  int rc = staged ? BUDDY_HIP_OK : staging_for(stream, sizeof(u16) * in.terms * (size_t)a.Mp * a.Kp, in, &abf,
                        &staged);
   if (rc)
     return rc;

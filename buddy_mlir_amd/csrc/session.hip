@@ -100,6 +100,7 @@ struct Session {
   float *pf_x = nullptr, *pf_xn = nullptr, *pf_qkv = nullptr, *pf_att = nullptr,
         *pf_g = nullptr, *pf_u = nullptr;
   int *pf_tokens = nullptr;
+  unsigned short *pf_xn_bf = nullptr, *pf_g_bf = nullptr; // bf16 matmul inputs
   int gemm_terms = 3; // bf16 terms per activation in the prefill matmuls (3 = exact)
 
   template <typename T> int alloc(T **p, size_t n) {
@@ -260,6 +261,11 @@ struct Session {
       }
     if (pf_tokens)
       (void)hipFree(pf_tokens);
+    for (unsigned short **p : {&pf_xn_bf, &pf_g_bf})
+      if (*p) {
+        (void)hipFree(*p);
+        *p = nullptr;
+      }
     pf_rows = 0;
     BH_CHECK_HIP(hipMalloc((void **)&pf_x, sizeof(float) * rows * S.hidden));
     BH_CHECK_HIP(hipMalloc((void **)&pf_xn, sizeof(float) * rows * S.hidden));
@@ -268,6 +274,10 @@ struct Session {
     BH_CHECK_HIP(hipMalloc((void **)&pf_g, sizeof(float) * rows * S.inter));
     BH_CHECK_HIP(hipMalloc((void **)&pf_u, sizeof(float) * rows * S.inter));
     BH_CHECK_HIP(hipMalloc((void **)&pf_tokens, sizeof(int) * rows));
+    // bf16 staging of the matmul inputs that the norm and SiLU kernels write
+    // directly (up to three terms)
+    BH_CHECK_HIP(hipMalloc((void **)&pf_xn_bf, gemm_staging_layout(rows, S.hidden).bytes(3)));
+    BH_CHECK_HIP(hipMalloc((void **)&pf_g_bf, gemm_staging_layout(rows, S.inter).bytes(3)));
     pf_rows = rows;
     return BUDDY_HIP_OK;
   }
@@ -290,6 +300,23 @@ struct Session {
     g.reuse_staged_a = same_input_as_before;
     return launch_gemm_w8(g, stream);
   }
+  // the same with the input already staged as bf16 terms
+  int gemm_staged(const unsigned short *staged, const PackedLinear &W, float *C, int64_t M,
+                  bool accumulate) {
+    GemmW8Args g;
+    g.staged = staged;
+    g.W = W.w;
+    g.scale = W.s;
+    g.bias = accumulate ? nullptr : W.b;
+    g.C = C;
+    g.ldc = W.N;
+    g.M = M;
+    g.K = W.K;
+    g.N = W.N;
+    g.accumulate = accumulate;
+    g.terms = gemm_terms;
+    return launch_gemm_w8(g, stream);
+  }
 
   // Prompt processing for tokens already in pf_tokens: fills cache rows
   // start_pos .. start_pos+n-1 and leaves the final hidden states in pf_x
@@ -304,16 +331,21 @@ struct Session {
     int rc;
     for (int i = 0; i < S.layers; ++i) {
       Layer &L = layers[(size_t)i];
-      if ((rc = launch_rmsnorm(pf_x, L.ln1, pf_xn, n, S.hidden, S.rms_eps, stream)))
-        return rc;
       if (L.qkv_f32) {
+        if ((rc = launch_rmsnorm(pf_x, L.ln1, pf_xn, n, S.hidden, S.rms_eps, stream)))
+          return rc;
         if ((rc = launch_bias_rows(pf_qkv, L.qkv.b, n, L.qkv.N, stream)))
           return rc;
         if ((rc = launch_matmul_f32(pf_xn, L.qkv_f32, pf_qkv, n, L.qkv.N, L.qkv.K,
                                     L.qkv.K, L.qkv.N, L.qkv.N, true, stream)))
           return rc;
-      } else if ((rc = gemm(pf_xn, L.qkv, pf_qkv, n, false))) {
-        return rc;
+      } else {
+        // the norm writes the matmul's bf16 input directly
+        if ((rc = launch_rmsnorm_to_staging(pf_x, L.ln1, n, S.hidden, S.rms_eps,
+                                            gemm_terms, pf_xn_bf, stream)))
+          return rc;
+        if ((rc = gemm_staged(pf_xn_bf, L.qkv, pf_qkv, n, false)))
+          return rc;
       }
       if ((rc = launch_rope_kv_write(pf_qkv, QKV, inv_freq, L.kc, L.vc, S.heads,
                                      S.kv_heads, S.head_dim, S.max_len, start_pos,
@@ -339,15 +371,17 @@ struct Session {
         return rc;
       if ((rc = gemm(pf_att, L.o, pf_x, n, true)))
         return rc;
-      if ((rc = launch_rmsnorm(pf_x, L.ln2, pf_xn, n, S.hidden, S.rms_eps, stream)))
+      if ((rc = launch_rmsnorm_to_staging(pf_x, L.ln2, n, S.hidden, S.rms_eps,
+                                          gemm_terms, pf_xn_bf, stream)))
         return rc;
-      if ((rc = gemm(pf_xn, L.gate, pf_g, n, false)))
+      if ((rc = gemm_staged(pf_xn_bf, L.gate, pf_g, n, false)))
         return rc;
-      if ((rc = gemm(pf_xn, L.up, pf_u, n, false, true)))
+      if ((rc = gemm_staged(pf_xn_bf, L.up, pf_u, n, false)))
         return rc;
-      if ((rc = launch_silu_mul(pf_g, pf_u, pf_g, (int64_t)n * S.inter, stream)))
+      if ((rc = launch_silu_mul_to_staging(pf_g, pf_u, n, S.inter, gemm_terms, pf_g_bf,
+                                           stream)))
         return rc;
-      if ((rc = gemm(pf_g, L.down, pf_x, n, true)))
+      if ((rc = gemm_staged(pf_g_bf, L.down, pf_x, n, true)))
         return rc;
     }
     return BUDDY_HIP_OK;
@@ -486,7 +520,8 @@ void buddy_hip_session_destroy(buddy_hip_session *hs) {
   for (void *p : s->owned)
     (void)hipFree(p);
   for (void *p : {(void *)s->pf_x, (void *)s->pf_xn, (void *)s->pf_qkv, (void *)s->pf_att,
-                  (void *)s->pf_g, (void *)s->pf_u, (void *)s->pf_tokens})
+                  (void *)s->pf_g, (void *)s->pf_u, (void *)s->pf_tokens,
+                  (void *)s->pf_xn_bf, (void *)s->pf_g_bf})
     if (p)
       (void)hipFree(p);
   if (s->host_state)
