@@ -153,16 +153,26 @@ silu_mul_to_staging_kernel(const float *__restrict__ g, const float *__restrict_
   if (i >= (int64_t)rows * kq)
     return;
   const int row = (int)(i / kq), k0 = (int)(i % kq) * 8;
-  float r[8];
+  float r[8], gv[8], uv[8];
+  const float *gr = g + (size_t)row * n + k0, *ur = u + (size_t)row * n + k0;
+  if (k0 + 7 < n && ((reinterpret_cast<uintptr_t>(gr) | reinterpret_cast<uintptr_t>(ur)) & 15) == 0) {
+    const float4 g0 = *reinterpret_cast<const float4 *>(gr), g1 = *reinterpret_cast<const float4 *>(gr + 4);
+    const float4 u0 = *reinterpret_cast<const float4 *>(ur), u1 = *reinterpret_cast<const float4 *>(ur + 4);
+    gv[0] = g0.x; gv[1] = g0.y; gv[2] = g0.z; gv[3] = g0.w;
+    gv[4] = g1.x; gv[5] = g1.y; gv[6] = g1.z; gv[7] = g1.w;
+    uv[0] = u0.x; uv[1] = u0.y; uv[2] = u0.z; uv[3] = u0.w;
+    uv[4] = u1.x; uv[5] = u1.y; uv[6] = u1.z; uv[7] = u1.w;
+  } else {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      gv[e] = k0 + e < n ? gr[e] : 0.f;
+      uv[e] = k0 + e < n ? ur[e] : 0.f;
+    }
+  }
 #pragma unroll
   for (int e = 0; e < 8; ++e) {
-    float v = 0.f;
-    if (k0 + e < n) {
-      const float gv = g[(size_t)row * n + k0 + e];
-      const float sig = 1.0f / (1.0f + expf(-gv));
-      v = (gv * sig) * u[(size_t)row * n + k0 + e];
-    }
-    r[e] = v;
+    const float sig = 1.0f / (1.0f + expf(-gv[e]));
+    r[e] = k0 + e < n ? (gv[e] * sig) * uv[e] : 0.f;
   }
   store_terms(r, terms, out + (size_t)row * Kp + k0, (size_t)Mp * Kp);
 }
