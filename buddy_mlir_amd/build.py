@@ -31,6 +31,30 @@ COMMON = [
 ]
 
 
+# Kernels of these files issue global loads through inline asm and wait for them
+# by hand.  The compiler believes such a load's result exists as soon as the
+# load is issued: if it spilled one of those registers it would store garbage
+# and hand the register to something else while the load is still in flight.
+# Their kernels must therefore use no scratch at all; the build checks it.
+NO_SCRATCH = {"gemm_w8_mfma.hip", "gemv_w8a32_mfma.hip"}
+
+
+def _check_no_scratch(src: Path, remarks: str) -> None:
+    name = None
+    bad = []
+    for line in remarks.splitlines():
+        if "Function Name:" in line:
+            name = line.split("Function Name:")[1].split("[")[0].strip()
+        elif "ScratchSize [bytes/lane]:" in line:
+            n = int(line.split("ScratchSize [bytes/lane]:")[1].split("[")[0])
+            if n:
+                bad.append(f"{name}: {n} bytes of scratch per lane")
+    if bad:
+        raise RuntimeError(
+            f"{src.name}: kernels with hand-issued loads must not spill:\n  "
+            + "\n  ".join(bad))
+
+
 def _hipcc() -> str:
     for cand in (os.environ.get("HIPCC"), "/opt/rocm/bin/hipcc", "hipcc"):
         if cand and (os.path.isabs(cand) and os.path.exists(cand) or not os.path.isabs(cand)):
@@ -53,9 +77,17 @@ def _compile(src: Path, force: bool) -> Path:
     if not force and obj.exists() and obj.stat().st_mtime >= newest:
         return obj
     cmd = [_hipcc(), *COMMON, "-x", "hip", "-c", str(src), "-o", str(obj)]
+    if src.name in NO_SCRATCH:
+        cmd.append("-Rpass-analysis=kernel-resource-usage")
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError(f"hipcc failed on {src.name}:\n{r.stdout}\n{r.stderr}")
+    if src.name in NO_SCRATCH:
+        try:
+            _check_no_scratch(src, r.stderr)
+        except RuntimeError:
+            obj.unlink(missing_ok=True)
+            raise
     return obj
 
 

@@ -393,7 +393,12 @@ int launch_span(const MfmaArgs &ka, int epilogue, int blocks, hipStream_t stream
   switch (epilogue) {
   case kEpiStore: return launch_norm<kEpiStore, SPAN>(ka, blocks, stream);
   case kEpiAccum: return launch_norm<kEpiAccum, SPAN>(ka, blocks, stream);
-  case kEpiSiluMul: return launch_norm<kEpiSiluMul, SPAN>(ka, blocks, stream);
+  case kEpiSiluMul:
+    // two matrices with eight groups each do not fit the register file (the
+    // fetch ring must never spill), so that variant is not built
+    if (SPAN > 4)
+      return fail(BUDDY_HIP_ERR_ARG, "gemv: SiLU*mul with %d groups per wavefront", SPAN);
+    return launch_norm<kEpiSiluMul, (SPAN > 4 ? 4 : SPAN)>(ka, blocks, stream);
   }
   return fail(BUDDY_HIP_ERR_ARG, "gemv: unknown epilogue %d", epilogue);
 }
