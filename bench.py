@@ -3,7 +3,7 @@
 MI355X, next to the CPU oracle timed on the same host.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W]
-    python bench.py --workload gemv|mlp|prefill|llama8b   (the other configurations)
+    python bench.py --workload gemv|mlp|prefill|llama8b|kvdiscard   (the other configurations)
 
 A step is one greedy decode step (one token) at batch 1 with the KV cache
 already holding 1024 positions; weights, KV cache and activations are resident
@@ -298,6 +298,45 @@ def bench_prefill(bh, args):
     }
 
 
+def bench_kvdiscard(bh, args):
+    """KV-cache overflow at the Qwen2-1.5B shape: 56 cache tensors
+    [2, 1088, 128] f32 full to the last row, keep 4 tokens, discard 256, move
+    and re-rotate the other 828 rows, clear the rest."""
+    import numpy as np
+    import torch
+
+    from buddy_mlir_amd import synthetic
+
+    heads, L, D, n = 2, 1088, 128, 56
+    keep, discard, count = 4, 256, 1088
+    tensors = [torch.randn((heads, L, D), device="cuda") for _ in range(n)]
+    ptrs = (ctypes.c_void_p * n)(*[t.data_ptr() for t in tensors])
+    f = np.ascontiguousarray(synthetic.inv_freq(D).cpu().numpy(), np.float32)
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def fn(i):
+        rc = bh.buddy_hip_kv_discard(ptrs, n, heads, L, D, keep, discard, count,
+                                     f.ctypes.data, stream)
+        if rc:
+            raise RuntimeError("kv_discard failed")
+    t = _time_launches(fn, 50, warm=3)
+    tail = count - keep - discard
+    by = n * heads * D * 4 * (2 * tail + (L - keep - tail))  # read + write tail, clear rest
+    return {
+        "metric": "kv_discard_hbm_gbps", "value": by / t / 1e9, "unit": "GB/s",
+        "n_gpus": 1, "steps": 50, "warmup": 3, "ms_per_step": t * 1e3,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": "KV-cache discard + key re-rotation, 56 tensors [2,1088,128], "
+                               "keep 4 / discard 256 / count 1088"},
+        "roofline": {"kernel": "kv_discard_kernel", "bound": "hbm",
+                     "achieved": by / t / 1e9, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": by / t / 1e9 / HBM_PEAK_GBPS,
+                     "algorithmic_bytes_per_launch": by, "avg_launch_us": t * 1e6,
+                     "traffic": None},
+    }
+
+
 def bench_llama8b(bh, args):
     """configs[4]: the decode GEMVs of a Llama-3-8B-shaped step, 32 layers of
     distinct weights (q|k|v, o, gate|up fused, down) plus lm_head: 7.5 GB of int8
@@ -368,7 +407,7 @@ def main():
     ap.add_argument("--steps", type=int, default=64)
     ap.add_argument("--warmup", type=int, default=8)
     ap.add_argument("--workload", default="decode",
-                    choices=["decode", "gemv", "mlp", "prefill", "llama8b"],
+                    choices=["decode", "gemv", "mlp", "prefill", "llama8b", "kvdiscard"],
                     help="decode (default): the full decode step the headline metric "
                          "is quoted on; the others measure the remaining configurations")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -393,7 +432,7 @@ def main():
     bh = bma.lib()
     if args.workload != "decode":
         fn = {"gemv": bench_gemv, "mlp": bench_mlp, "prefill": bench_prefill,
-              "llama8b": bench_llama8b}[args.workload]
+              "llama8b": bench_llama8b, "kvdiscard": bench_kvdiscard}[args.workload]
         print(json.dumps(fn(bh, args)))
         return
     K, W = args.steps, args.warmup

@@ -125,6 +125,10 @@ def _declare(lib):
         "buddy_hip_forward_reset": (None, []),
         "buddy_hip_forward_invalidate_kv": (None, []),
         "buddy_hip_session_set_state": (c_int, [vp, c_int, c_int]),
+        "buddy_hip_session_discard_kv": (c_int, [vp, c_int, c_int, c_int]),
+        "buddy_hip_kv_discard": (c_int, [vp, c_int, c_int, c_int, c_int, c_int, c_int,
+                                         c_int, vp, vp]),
+        "buddy_hip_forward_discard_kv": (c_int, [c_int, c_int, c_int]),
         "buddy_hip_session_enqueue_steps": (c_int, [vp, c_int]),
         "buddy_hip_session_logits": (vp, [vp]),
         "buddy_hip_session_stream": (vp, [vp]),

@@ -423,6 +423,15 @@ void buddy_hip_forward_reset(void) {
   bh::destroy_locked(m);
 }
 
+int buddy_hip_forward_discard_kv(int keep, int discard, int count) {
+  bh::ModelState &m = bh::state();
+  std::lock_guard<std::mutex> lock(m.mu);
+  if (!m.sess || !m.kv_on_device)
+    return bh::fail(BUDDY_HIP_ERR_ARG,
+                    "forward_discard_kv: no device-resident KV cache yet");
+  return buddy_hip_session_discard_kv(m.sess, keep, discard, count);
+}
+
 void buddy_hip_forward_invalidate_kv(void) {
   bh::ModelState &m = bh::state();
   std::lock_guard<std::mutex> lock(m.mu);

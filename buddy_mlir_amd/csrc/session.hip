@@ -21,6 +21,7 @@
 #include "elementwise.h"
 #include "gemm.h"
 #include "gemv_w8a32.h"
+#include "kv_cache.h"
 
 #include <cmath>
 #include <cstring>
@@ -81,6 +82,7 @@ struct Session {
   const float *embed = nullptr; // borrowed: [vocab, hidden] f32
   float *ln_f = nullptr, *inv_freq = nullptr;
   float *rope = nullptr; // [cos | sin] of the step's position
+  std::vector<float> inv_freq_host; // for the key re-rotation after a discard
   PackedLinear lm;
   // activations
   float *x = nullptr, *xn = nullptr, *qkv = nullptr, *att = nullptr,
@@ -542,6 +544,10 @@ int buddy_hip_session_set_globals(buddy_hip_session *hs, const float *embed,
   s->embed = embed;
   BH_CHECK_HIP(hipMemcpyAsync(s->inv_freq, inv_freq, sizeof(float) * S.head_dim / 2,
                               hipMemcpyDefault, s->stream));
+  s->inv_freq_host.resize((size_t)S.head_dim / 2);
+  BH_CHECK_HIP(hipMemcpyAsync(s->inv_freq_host.data(), inv_freq,
+                              sizeof(float) * S.head_dim / 2, hipMemcpyDefault,
+                              s->stream));
   BH_CHECK_HIP(hipMemcpyAsync(s->ln_f, ln_f, sizeof(float) * S.hidden,
                               hipMemcpyDefault, s->stream));
   if (!s->lm.w) {
@@ -853,6 +859,28 @@ int buddy_hip_session_set_state(buddy_hip_session *hs, int token, int pos) {
 const float *buddy_hip_session_logits(buddy_hip_session *hs) {
   Session *s = reinterpret_cast<Session *>(hs);
   return s ? s->logits : nullptr;
+}
+
+int buddy_hip_session_discard_kv(buddy_hip_session *hs, int keep, int discard,
+                                 int count) {
+  Session *s = reinterpret_cast<Session *>(hs);
+  BH_REQUIRE(s, "session_discard_kv: null session");
+  int rc = s->ready();
+  if (rc)
+    return rc;
+  const auto &S = s->shape;
+  std::vector<float *> tensors;
+  for (auto &L : s->layers) {
+    tensors.push_back(L.kc);
+    tensors.push_back(L.vc);
+  }
+  rc = bh::launch_kv_discard(tensors.data(), (int)tensors.size(), S.kv_heads, S.max_len,
+                             S.head_dim, keep, discard, count,
+                             s->inv_freq_host.data(), s->stream);
+  if (rc)
+    return rc;
+  BH_CHECK_HIP(hipStreamSynchronize(s->stream));
+  return BUDDY_HIP_OK;
 }
 
 buddy_hip_stream buddy_hip_session_stream(buddy_hip_session *hs) {

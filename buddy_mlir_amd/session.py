@@ -152,6 +152,11 @@ class DecoderSession:
     def set_state(self, token: int, pos: int):
         check(self._lib.buddy_hip_session_set_state(self._h, token, pos), "set_state")
 
+    def discard_kv(self, keep: int, discard: int, count: int):
+        """kvcache::discardKVCache + adjustKeyCacheRope on the device caches."""
+        check(self._lib.buddy_hip_session_discard_kv(self._h, keep, discard, count),
+              "session_discard_kv")
+
     def enqueue_steps(self, steps: int):
         check(self._lib.buddy_hip_session_enqueue_steps(self._h, steps), "enqueue_steps")
 

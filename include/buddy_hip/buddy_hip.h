@@ -275,6 +275,26 @@ int buddy_hip_session_enqueue_steps(buddy_hip_session *s, int steps);
 const float *buddy_hip_session_logits(buddy_hip_session *s); /* device */
 buddy_hip_stream buddy_hip_session_stream(buddy_hip_session *s);
 
+/* ---- KV-cache overflow ------------------------------------------------------
+ * kvcache::discardKVCache followed by kvcache::adjustKeyCacheRope
+ * (runtime/include/buddy/runtime/llm/KVCacheManager.h:150-194, :240-268), on
+ * caches that live on the device: keep the first `keep` tokens, drop the next
+ * `discard`, move the tail forward, zero the rest, and rotate the moved keys
+ * back by `discard` positions.  `count` is the token count before the call.
+ * tensors: host array of device pointers to [heads, max_len, head_dim] f32
+ * caches, even index = keys, odd = values (KVCacheManager.h:200-201,209).
+ * inv_freq: host pointer to head_dim/2 inverse RoPE frequencies; NULL moves
+ * without re-rotating.  Parameters the reference refuses (KVCacheManager.h
+ * :154-167) are refused here too and leave the caches untouched.  The moved
+ * bytes and the rotated keys equal the reference's bit for bit. */
+int buddy_hip_kv_discard(float *const *tensors, int num_tensors, int heads, int max_len,
+                         int head_dim, int keep, int discard, int count,
+                         const float *inv_freq, buddy_hip_stream stream);
+/* The same for a session's own caches; the caller continues decoding at
+ * position count - discard. */
+int buddy_hip_session_discard_kv(buddy_hip_session *s, int keep, int discard,
+                                 int count);
+
 /* y[N] = bias[N] + x[K] . B[K,N] in f32 (bias may be NULL): the decode GEMV
  * of MatMulVectorizationDecode.cpp:142-175 followed by the q/k/v bias add. */
 int buddy_hip_gemv_f32(const float *x, const float *B, const float *bias,
@@ -360,6 +380,10 @@ void _mlir_ciface_forward_decode(
     BUDDY_HIP_DKV_(25) BUDDY_HIP_DKV_(26) BUDDY_HIP_DKV_(27));
 void buddy_hip_forward_reset(void);         /* drops the cached device session */
 void buddy_hip_forward_invalidate_kv(void); /* next decode re-uploads the KV cache */
+/* discardKVCache + adjustKeyCacheRope on the device-resident cache of the
+ * session behind _mlir_ciface_forward_*: what the decode loop calls instead of
+ * editing its host tensors (TextGeneration.cpp:231-237). */
+int buddy_hip_forward_discard_kv(int keep, int discard, int count);
 
 /* ---- operator-level memref entry points --------------------------------
  * result = A * B, f32.  Same symbol and contract as

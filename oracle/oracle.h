@@ -156,6 +156,17 @@ int64_t oracle_decode_step(const oracle_model *m, int64_t token, int64_t pos,
 
 int oracle_num_threads(void);
 
+/* ---- KV-cache overflow handling (kv_cache.c) -------------------------------
+ * runtime/include/buddy/runtime/llm/KVCacheManager.h:150-194, :200-268.
+ * Pinned by: numpy slicing of the same move, rotation by -d composed with the
+ * RoPE of position p equals the RoPE of position p - d, rotation by -d then +d
+ * is the identity within rounding. */
+int oracle_kv_discard(float *cache, int64_t heads, int64_t max_len, int64_t dim,
+                      int64_t keep, int64_t discard, int64_t count);
+void oracle_kv_adjust_rope(float *kcache, int64_t heads, int64_t max_len, int64_t dim,
+                           int64_t keep, int64_t discard, int64_t count,
+                           const float *inv_freq);
+
 #ifdef __cplusplus
 }
 #endif

@@ -207,6 +207,23 @@ class Oracle:
         self.lib.oracle_rope_apply(_p(x), c_int64(H), c_int64(D), _p(cosv), _p(sinv))
         return x
 
+    def kv_discard(self, cache, keep, discard, count):
+        """discardKVCache on one [heads, max_len, dim] tensor; returns (rc, new)."""
+        c = np.array(cache, np.float32)
+        H, L, D = c.shape
+        rc = self.lib.oracle_kv_discard(_p(c), c_int64(H), c_int64(L), c_int64(D),
+                                        c_int64(keep), c_int64(discard), c_int64(count))
+        return rc, c
+
+    def kv_adjust_rope(self, kcache, keep, discard, count, inv_freq):
+        c = np.array(kcache, np.float32)
+        H, L, D = c.shape
+        inv_freq = np.ascontiguousarray(inv_freq, np.float32)
+        self.lib.oracle_kv_adjust_rope(_p(c), c_int64(H), c_int64(L), c_int64(D),
+                                       c_int64(keep), c_int64(discard), c_int64(count),
+                                       _p(inv_freq))
+        return c
+
     def silu_mul(self, g, u):
         g = np.ascontiguousarray(g, np.float32).reshape(-1)
         u = np.ascontiguousarray(u, np.float32).reshape(-1)
