@@ -3,7 +3,7 @@
 MI355X, next to the CPU oracle timed on the same host.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W]
-    python bench.py --workload gemv|mlp|prefill|llama8b|kvdiscard   (the other configurations)
+    python bench.py --workload gemv|mlp|prefill|llama8b|kvdiscard|w4a16   (the other configurations)
 
 A step is one greedy decode step (one token) at batch 1 with the KV cache
 already holding 1024 positions; weights, KV cache and activations are resident
@@ -337,6 +337,45 @@ def bench_kvdiscard(bh, args):
     }
 
 
+def bench_w4a16(bh, args):
+    """The reference's int4 weight-only decode GEMV (f16 activations and
+    accumulator, k in order) at 1536 -> 8960 and 8960 -> 1536, 24 weight copies."""
+    import torch
+
+    res = {}
+    for K, N in ((1536, 8960), (8960, 1536)):
+        copies = 24
+        packs = [torch.randint(-128, 128, (K, N // 2), dtype=torch.int8, device="cuda")
+                 for _ in range(copies)]
+        a = torch.randn(K, device="cuda").half()
+        sc = torch.full((N,), 0.01, device="cuda").half()
+        c = torch.zeros(N, device="cuda").half()
+        stream = torch.cuda.current_stream().cuda_stream
+
+        def fn(i):
+            rc = bh.buddy_hip_gemv_w4a16(a.data_ptr(), packs[i % copies].data_ptr(),
+                                         sc.data_ptr(), c.data_ptr(), K, N, stream)
+            if rc:
+                raise RuntimeError("gemv_w4a16 failed")
+        t = _time_launches(fn, 240)
+        by = K * N // 2 + 2 * K + 2 * N + 4 * N
+        res[f"{K}->{N}"] = {"us": t * 1e6, "gbps": by / t / 1e9, "frac": by / t / 1e9 / HBM_PEAK_GBPS,
+                            "bytes": by}
+    r = res["1536->8960"]
+    return {
+        "metric": "int4_gemv_hbm_gbps", "value": r["gbps"], "unit": "GB/s", "n_gpus": 1,
+        "steps": 240, "warmup": 8, "ms_per_step": r["us"] * 1e-3, "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
+        "config": {"workload": "W4A16 decode GEMV, reference order of f16 operations; "
+                               "value is 1536 -> 8960"},
+        "detail": res,
+        "roofline": {"kernel": "w4a16_gemv_kernel", "bound": "hbm", "achieved": r["gbps"],
+                     "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": r["frac"],
+                     "algorithmic_bytes_per_launch": r["bytes"], "avg_launch_us": r["us"],
+                     "traffic": None},
+    }
+
+
 def bench_llama8b(bh, args):
     """configs[4]: the decode GEMVs of a Llama-3-8B-shaped step, 32 layers of
     distinct weights (q|k|v, o, gate|up fused, down) plus lm_head: 7.5 GB of int8
@@ -407,7 +446,7 @@ def main():
     ap.add_argument("--steps", type=int, default=64)
     ap.add_argument("--warmup", type=int, default=8)
     ap.add_argument("--workload", default="decode",
-                    choices=["decode", "gemv", "mlp", "prefill", "llama8b", "kvdiscard"],
+                    choices=["decode", "gemv", "mlp", "prefill", "llama8b", "kvdiscard", "w4a16"],
                     help="decode (default): the full decode step the headline metric "
                          "is quoted on; the others measure the remaining configurations")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -432,7 +471,7 @@ def main():
     bh = bma.lib()
     if args.workload != "decode":
         fn = {"gemv": bench_gemv, "mlp": bench_mlp, "prefill": bench_prefill,
-              "llama8b": bench_llama8b, "kvdiscard": bench_kvdiscard}[args.workload]
+              "llama8b": bench_llama8b, "kvdiscard": bench_kvdiscard, "w4a16": bench_w4a16}[args.workload]
         print(json.dumps(fn(bh, args)))
         return
     K, W = args.steps, args.warmup

@@ -146,10 +146,11 @@ int buddy_hip_unpack_w8(const int8_t *packed, int64_t K, int64_t N, int8_t *W,
   return buddy_hip_unpack_w8_tiles(packed, K, N, bh::kTileN, W, stream);
 }
 
-int buddy_hip_quantize_w8(const float *W, int64_t K, int64_t N, int8_t *q,
-                          float *scale, buddy_hip_stream stream) {
-  BH_REQUIRE(W && q && scale, "quantize_w8: null pointer");
-  BH_REQUIRE(K > 0 && N > 0, "quantize_w8: bad shape K=%lld N=%lld",
+static int quantize_per_channel(const float *W, int64_t K, int64_t N, int8_t *q,
+                                float *scale, float qmax, float lo, float hi,
+                                buddy_hip_stream stream) {
+  BH_REQUIRE(W && q && scale, "quantize: null pointer");
+  BH_REQUIRE(K > 0 && N > 0, "quantize: bad shape K=%lld N=%lld",
              (long long)K, (long long)N);
   hipStream_t st = bh::as_stream(stream);
   BH_CHECK_HIP(hipMemsetAsync(scale, 0, sizeof(float) * (size_t)N, st));
@@ -161,11 +162,21 @@ int buddy_hip_quantize_w8(const float *W, int64_t K, int64_t N, int8_t *q,
                      reinterpret_cast<unsigned *>(scale));
   hipLaunchKernelGGL(bh::finalize_scale_kernel,
                      dim3((unsigned)bh::ceil_div(N, 256)), dim3(256), 0, st,
-                     scale, N, 127.0f);
+                     scale, N, qmax);
   hipLaunchKernelGGL(bh::quantize_kernel,
                      dim3((unsigned)bh::ceil_div(K * N, 256)), dim3(256), 0, st,
-                     W, scale, K, N, q, -128.0f, 127.0f);
+                     W, scale, K, N, q, lo, hi);
   BH_CHECK_HIP(hipGetLastError());
   return BUDDY_HIP_OK;
+}
+
+int buddy_hip_quantize_w8(const float *W, int64_t K, int64_t N, int8_t *q,
+                          float *scale, buddy_hip_stream stream) {
+  return quantize_per_channel(W, K, N, q, scale, 127.0f, -128.0f, 127.0f, stream);
+}
+
+int buddy_hip_quantize_w4(const float *W, int64_t K, int64_t N, int8_t *q,
+                          float *scale, buddy_hip_stream stream) {
+  return quantize_per_channel(W, K, N, q, scale, 7.0f, -8.0f, 7.0f, stream);
 }
 }

@@ -78,6 +78,23 @@ int buddy_hip_unpack_w8_tiles(const int8_t *packed, int64_t K, int64_t N,
 int buddy_hip_quantize_w8(const float *W, int64_t K, int64_t N, int8_t *q,
                           float *scale, buddy_hip_stream stream);
 
+/* ---- int4 weight-only decode path (W4A16) -------------------------------
+ * The same recipe with amax/7 and a clamp to [-8, 7]
+ * (tools/buddy-codegen/import_model.py:800-802,838-842), the nibble packing of
+ * import_model.py:810-815 (element 2i in the low nibble, 2i+1 in the high one;
+ * for a row-major [K,N] matrix: even channel low, odd channel high), and the
+ * decode GEMV of Int4DequantMatMulVectorizationDecode.cpp:385-468:
+ *   C[n] = C[n] + (sum_k A[k] * w[k][n]) * scale[n]
+ * with f16 A [K], scale [N] and C [N] (bit patterns) and packed [K, N/2]
+ * bytes.  The sum runs in the reference's order, rounded to f16 after every
+ * step, so the result is the reference's bit for bit. */
+int buddy_hip_quantize_w4(const float *W, int64_t K, int64_t N, int8_t *q,
+                          float *scale, buddy_hip_stream stream);
+int buddy_hip_pack_int4(const int8_t *q, int64_t count, int8_t *packed,
+                        buddy_hip_stream stream);
+int buddy_hip_gemv_w4a16(const uint16_t *A, const int8_t *packed, const uint16_t *scale,
+                         uint16_t *C, int64_t K, int64_t N, buddy_hip_stream stream);
+
 /* ---- int8 dequant decode GEMV / small-batch matmul ---------------------
  * Replaces the kernel that
  * midend/lib/Conversion/MatMulOptimization/DequantMatMulVectorizationDecode.cpp

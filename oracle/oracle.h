@@ -167,6 +167,22 @@ void oracle_kv_adjust_rope(float *kcache, int64_t heads, int64_t max_len, int64_
                            int64_t keep, int64_t discard, int64_t count,
                            const float *inv_freq);
 
+/* ---- int4 weight-only decode path, W4A16 (w4a16.c) -------------------------
+ * tools/buddy-codegen/import_model.py:810-815 (nibble packing),
+ * Int4DequantMatMulVectorizationDecode.cpp:385-468 (kernel, f16 throughout).
+ * f16 values travel as their bit patterns (uint16_t).
+ * Pinned by: numpy.float16 for the conversions; a numpy.float16 emulation of the
+ * sequential f16 accumulation; the reference example's inputs
+ * (examples/BuddyMatmul/int4-dequant-matmul-vectorization-decode.mlir:177-190:
+ * A = 1, bytes = 2, scale = 1 -> [8, 0, 8, 0]); pack/unpack round trip over all
+ * 256 byte values. */
+void oracle_f32_to_f16(const float *x, int64_t n, uint16_t *y);
+void oracle_f16_to_f32(const uint16_t *x, int64_t n, float *y);
+int oracle_pack_int4(const int8_t *q, int64_t n, int8_t *packed);
+void oracle_unpack_int4(const int8_t *packed, int64_t n, int8_t *q);
+void oracle_w4a16_gemv(const uint16_t *a, const int8_t *packed, const uint16_t *scale,
+                       uint16_t *c, int64_t K, int64_t N);
+
 #ifdef __cplusplus
 }
 #endif

@@ -207,6 +207,37 @@ class Oracle:
         self.lib.oracle_rope_apply(_p(x), c_int64(H), c_int64(D), _p(cosv), _p(sinv))
         return x
 
+    # -- W4A16 (f16 values are numpy.float16 arrays; bits go through uint16 views)
+    def f32_to_f16(self, x):
+        x = np.ascontiguousarray(x, np.float32).reshape(-1)
+        y = np.empty(x.size, np.uint16)
+        self.lib.oracle_f32_to_f16(_p(x), c_int64(x.size), _p(y))
+        return y.view(np.float16)
+
+    def pack_int4(self, q):
+        q = np.ascontiguousarray(q, np.int8)
+        out = np.empty(q.size // 2, np.int8)
+        rc = self.lib.oracle_pack_int4(_p(q), c_int64(q.size), _p(out))
+        assert rc == 0
+        return out.reshape(q.shape[:-1] + (q.shape[-1] // 2,))
+
+    def unpack_int4(self, packed):
+        packed = np.ascontiguousarray(packed, np.int8)
+        out = np.empty(packed.size * 2, np.int8)
+        self.lib.oracle_unpack_int4(_p(packed), c_int64(out.size), _p(out))
+        return out.reshape(packed.shape[:-1] + (packed.shape[-1] * 2,))
+
+    def w4a16_gemv(self, a, packed, scale, c=None):
+        """a [K] f16, packed [K, N/2] int8, scale [N] f16, c [N] f16 (or zeros)."""
+        a = np.ascontiguousarray(a, np.float16).reshape(-1)
+        packed = np.ascontiguousarray(packed, np.int8)
+        K, N = packed.shape[0], packed.shape[1] * 2
+        scale = np.ascontiguousarray(scale, np.float16).reshape(-1)
+        out = np.zeros(N, np.float16) if c is None else np.array(c, np.float16).reshape(-1)
+        self.lib.oracle_w4a16_gemv(_p(a.view(np.uint16)), _p(packed), _p(scale.view(np.uint16)),
+                                   _p(out.view(np.uint16)), c_int64(K), c_int64(N))
+        return out
+
     def kv_discard(self, cache, keep, discard, count):
         """discardKVCache on one [heads, max_len, dim] tensor; returns (rc, new)."""
         c = np.array(cache, np.float32)
