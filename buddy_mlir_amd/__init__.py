@@ -136,6 +136,10 @@ def _declare(lib):
         "buddy_hip_session_logits": (vp, [vp]),
         "buddy_hip_session_stream": (vp, [vp]),
         "buddy_hip_gemv_f32": (c_int, [vp, vp, vp, vp, i64, i64, c_uint, vp]),
+        "buddy_hip_f32_tiles_bytes": (sz, [i64, i64]),
+        "buddy_hip_tile_f32": (c_int, [vp, i64, i64, vp, vp]),
+        "buddy_hip_gemv_f32_tiles": (c_int, [vp, vp, vp, vp, c_float, vp, i64, i64, c_uint,
+                                             vp]),
         "buddy_hip_pack_panels_f32": (c_int, [vp, i64, i64, c_int, vp, vp]),
         "buddy_hip_unpack_panels_f32": (c_int, [vp, i64, i64, c_int, vp, vp]),
         "buddy_hip_gemv_f32_panels": (c_int, [vp, vp, vp, i64, i64, c_uint, vp]),

@@ -8,63 +8,197 @@
 // build the q/k/v projections are this kernel followed by a bias add
 // (examples/BuddyDeepSeekR1/subgraph0_decode_simplify.mlir:73-85).
 //
-// B is row-major with N contiguous, so lanes run along n: a wavefront reads
-// four rows x 64 columns per 128-bit load; the 16 wavefronts of a workgroup
-// take interleaved rows of the same 64 columns and meet in LDS.
+// B is row-major with N contiguous.  The matrix is narrow for this chip (2048
+// columns at the q|k|v shape) and a sum over k must stay inside a workgroup (no
+// cross-workgroup reduction: it would cost an L2 write-back), so a workgroup
+// owns only 16 columns -- one 64-byte piece of every row -- and all of K: 128
+// workgroups at N = 2048.  A wavefront load reads 16 rows x 64 bytes (4 lanes of
+// float4 per row); the 8 wavefronts take interleaved 16-row blocks, all their
+// loads in flight at once, and meet in LDS in a fixed order.
+// RMSNorm can be fused in like in the int8 kernel: the norm weight multiplies x
+// as it is used, the sum of squares is gathered on the way (by the lanes of
+// column group 0 only, so every k counts once) and the rsqrt factor multiplies
+// the finished sums.
 #include "common.h"
 
 namespace bh {
 namespace {
 
-constexpr int kWaves = 16;
+constexpr int kWaves = 8;
+constexpr int kCols = 16;          // columns per workgroup
+constexpr int kRowsPerLoad = 16;   // rows per wavefront load
+constexpr int kUnroll = 6;         // loads in flight per lane
 
 __global__ void __launch_bounds__(kWaves * 64)
 gemv_f32_kernel(const float *__restrict__ x, const float *__restrict__ B,
-                const float *__restrict__ bias, float *__restrict__ y, int K,
-                int N, int64_t ldb, int accumulate) {
-  __shared__ float4 red[kWaves][64];
-  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
-  const int col = blockIdx.x * 64 + (lane & 15) * 4; // 4 columns per lane
-  const int rsub = lane >> 4;                        // 4 rows per wavefront load
-  float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
-  const bool full = col + 3 < N && ((ldb & 3) == 0) &&
+                const float *__restrict__ bias, const float *__restrict__ norm_w,
+                float norm_eps, float norm_inv_k, float *__restrict__ y, int K, int N,
+                int64_t ldb, int accumulate) {
+  __shared__ float red[kWaves][kCols + 1];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int c4 = lane & 3, rsub = lane >> 2; // float4 column group, row in a load
+  const int col = blockIdx.x * kCols + c4 * 4;
+  const bool full = blockIdx.x * kCols + kCols <= N && ((ldb & 3) == 0) &&
                     ((reinterpret_cast<uintptr_t>(B) & 15) == 0);
-  for (int k = wave * 4 + rsub; k < K; k += kWaves * 4) {
-    const float xv = x[k];
-    const float *row = B + (int64_t)k * ldb + col;
-    float4 b;
-    if (full)
-      b = *reinterpret_cast<const float4 *>(row);
-    else
-      b = make_float4(col < N ? row[0] : 0.f, col + 1 < N ? row[1] : 0.f,
-                      col + 2 < N ? row[2] : 0.f, col + 3 < N ? row[3] : 0.f);
-    acc.x = fmaf(xv, b.x, acc.x);
-    acc.y = fmaf(xv, b.y, acc.y);
-    acc.z = fmaf(xv, b.z, acc.z);
-    acc.w = fmaf(xv, b.w, acc.w);
+  float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+  float ss = 0.f;
+  // row blocks wave, wave + kWaves, ... of 16 rows each, kUnroll at a time
+  for (int kb = wave * kRowsPerLoad; kb < K; kb += kWaves * kRowsPerLoad * kUnroll) {
+    float4 b[kUnroll];
+    float xv[kUnroll], nw[kUnroll];
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+      const int k = kb + u * kWaves * kRowsPerLoad + rsub;
+      const int kc = min(k, K - 1); // rows past the end repeat the last, times zero
+      const float *row = B + (int64_t)kc * ldb + col;
+      if (full)
+        b[u] = *reinterpret_cast<const float4 *>(row);
+      else
+        b[u] = make_float4(col < N ? row[0] : 0.f, col + 1 < N ? row[1] : 0.f,
+                           col + 2 < N ? row[2] : 0.f, col + 3 < N ? row[3] : 0.f);
+      xv[u] = k < K ? x[kc] : 0.f;
+      nw[u] = norm_w ? norm_w[kc] : 1.f;
+    }
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+      if (norm_w && c4 == 0)
+        ss = fmaf(xv[u], xv[u], ss);
+      const float xs = xv[u] * nw[u];
+      acc.x = fmaf(xs, b[u].x, acc.x);
+      acc.y = fmaf(xs, b[u].y, acc.y);
+      acc.z = fmaf(xs, b[u].z, acc.z);
+      acc.w = fmaf(xs, b[u].w, acc.w);
+    }
   }
-  red[wave][lane] = acc;
+  // the 16 row lanes of a column group hold different k: lanes 4 apart ... 32 apart
+#pragma unroll
+  for (int o = 4; o < 64; o <<= 1) {
+    acc.x += __shfl_xor(acc.x, o, 64);
+    acc.y += __shfl_xor(acc.y, o, 64);
+    acc.z += __shfl_xor(acc.z, o, 64);
+    acc.w += __shfl_xor(acc.w, o, 64);
+    ss += __shfl_xor(ss, o, 64);
+  }
+  if (lane < 4) {
+    red[wave][lane * 4 + 0] = acc.x;
+    red[wave][lane * 4 + 1] = acc.y;
+    red[wave][lane * 4 + 2] = acc.z;
+    red[wave][lane * 4 + 3] = acc.w;
+    if (lane == 0)
+      red[wave][kCols] = ss;
+  }
   __syncthreads();
-  if (tid < 16) { // 16 lanes x 4 columns = the workgroup's 64 columns
-    float4 s = make_float4(0.f, 0.f, 0.f, 0.f);
-    for (int w = 0; w < kWaves; ++w)
-      for (int r = 0; r < 4; ++r) {
-        const float4 v = red[w][r * 16 + tid];
-        s.x += v.x;
-        s.y += v.y;
-        s.z += v.z;
-        s.w += v.w;
-      }
-    const int c0 = blockIdx.x * 64 + tid * 4;
-    const float out[4] = {s.x, s.y, s.z, s.w};
-    for (int j = 0; j < 4; ++j) {
-      const int n = c0 + j;
-      if (n < N) {
-        float v = out[j];
-        if (bias)
-          v = bias[n] + v; // tosa.add(bias, matmul)
-        y[n] = accumulate ? y[n] + v : v;
-      }
+  if (tid < kCols) {
+    float s = 0.f, sq = 0.f;
+    for (int w = 0; w < kWaves; ++w) {
+      s += red[w][tid];
+      sq += red[w][kCols];
+    }
+    const int n = blockIdx.x * kCols + tid;
+    if (n < N) {
+      float v = s;
+      if (norm_w) // x' = w (.) (x * r): r is common to the row
+        v *= 1.0f / sqrtf(sq * norm_inv_k + norm_eps);
+      if (bias)
+        v = bias[n] + v; // tosa.add(bias, matmul)
+      y[n] = accumulate ? y[n] + v : v;
+    }
+  }
+}
+
+// ---- the same product over 1 KiB tiles --------------------------------------
+// A device-side re-layout for matrices the library owns (the model path's f32
+// q|k|v weights): tile = 32 rows x 8 columns, row-major inside, tiles of one
+// 8-column strip contiguous along k, zero padded:
+//   T[((n/8) * ceil(K/32) + k/32) * 256 + (k%32) * 8 + n%8] = B[k, n].
+// A wavefront load is one whole tile (lane = float4: row lane/2, half lane%2), a
+// workgroup streams one contiguous strip, and a 2048-column matrix gives 256
+// workgroups instead of 128 with 64-byte pieces of 8 KB-apart rows.
+constexpr int kTileCols = 8, kTileRows = 32, kTileUnroll = 6;
+
+__global__ void __launch_bounds__(256)
+tile_f32_kernel(const float *__restrict__ B, int K, int N, int64_t ldb,
+                float *__restrict__ T, int64_t total) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= total)
+    return;
+  const int blocks = (K + kTileRows - 1) / kTileRows;
+  const int c = (int)(i & 7), r = (int)((i >> 3) & 31);
+  const int64_t tile = i >> 8;
+  const int64_t k = (tile % blocks) * kTileRows + r, n = (tile / blocks) * kTileCols + c;
+  T[i] = (k < K && n < N) ? B[k * ldb + n] : 0.f;
+}
+
+__global__ void __launch_bounds__(kWaves * 64)
+gemv_f32_tiles_kernel(const float *__restrict__ x, const float *__restrict__ T,
+                      const float *__restrict__ bias, const float *__restrict__ norm_w,
+                      float norm_eps, float norm_inv_k, float *__restrict__ y, int K,
+                      int N, int accumulate) {
+  __shared__ float red[kWaves][kTileCols + 1];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int half = lane & 1, row = lane >> 1;
+  const int blocks = (K + kTileRows - 1) / kTileRows;
+  const float4 *strip = reinterpret_cast<const float4 *>(T) +
+                        (int64_t)blockIdx.x * blocks * 64 + lane;
+  float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+  float ss = 0.f;
+  for (int b0 = wave; b0 < blocks; b0 += kWaves * kTileUnroll) {
+    float4 b[kTileUnroll];
+    float xv[kTileUnroll], nw[kTileUnroll];
+#pragma unroll
+    for (int u = 0; u < kTileUnroll; ++u) {
+      const int blk = b0 + u * kWaves;
+      const int bc = min(blk, blocks - 1); // past the end: the last tile again, x = 0
+      b[u] = strip[(int64_t)bc * 64];
+      const int k = blk * kTileRows + row;
+      const int kc = min(k, K - 1);
+      xv[u] = (blk < blocks && k < K) ? x[kc] : 0.f;
+      nw[u] = norm_w ? norm_w[kc] : 1.f;
+    }
+#pragma unroll
+    for (int u = 0; u < kTileUnroll; ++u) {
+      if (norm_w && half == 0)
+        ss = fmaf(xv[u], xv[u], ss);
+      const float xs = xv[u] * nw[u];
+      acc.x = fmaf(xs, b[u].x, acc.x);
+      acc.y = fmaf(xs, b[u].y, acc.y);
+      acc.z = fmaf(xs, b[u].z, acc.z);
+      acc.w = fmaf(xs, b[u].w, acc.w);
+    }
+  }
+#pragma unroll
+  for (int o = 2; o < 64; o <<= 1) {
+    acc.x += __shfl_xor(acc.x, o, 64);
+    acc.y += __shfl_xor(acc.y, o, 64);
+    acc.z += __shfl_xor(acc.z, o, 64);
+    acc.w += __shfl_xor(acc.w, o, 64);
+    ss += __shfl_xor(ss, o, 64);
+  }
+  if (lane < 2) {
+    red[wave][lane * 4 + 0] = acc.x;
+    red[wave][lane * 4 + 1] = acc.y;
+    red[wave][lane * 4 + 2] = acc.z;
+    red[wave][lane * 4 + 3] = acc.w;
+    if (lane == 0)
+      red[wave][kTileCols] = ss;
+  }
+  __syncthreads();
+  if (tid < kTileCols) {
+    float s = 0.f, sq = 0.f;
+    for (int w = 0; w < kWaves; ++w) {
+      s += red[w][tid];
+      sq += red[w][kTileCols];
+    }
+    const int n = blockIdx.x * kTileCols + tid;
+    if (n < N) {
+      float v = s;
+      if (norm_w)
+        v *= 1.0f / sqrtf(sq * norm_inv_k + norm_eps);
+      if (bias)
+        v = bias[n] + v;
+      y[n] = accumulate ? y[n] + v : v;
     }
   }
 }
@@ -79,16 +213,54 @@ bias_rows_kernel(float *__restrict__ C, const float *__restrict__ bias, int64_t 
 
 } // namespace
 
-int launch_gemv_f32(const float *x, const float *B, const float *bias, float *y,
-                    int64_t K, int64_t N, int64_t ldb, bool accumulate,
-                    hipStream_t stream) {
+int launch_gemv_f32_norm(const float *x, const float *B, const float *bias,
+                         const float *norm_w, float norm_eps, float *y, int64_t K,
+                         int64_t N, int64_t ldb, bool accumulate, hipStream_t stream) {
   BH_REQUIRE(x && B && y, "gemv_f32: null pointer");
   BH_REQUIRE(K > 0 && N > 0 && K < (1 << 30) && N < (1 << 30) && ldb >= N,
              "gemv_f32: bad shape K=%lld N=%lld ldb=%lld", (long long)K,
              (long long)N, (long long)ldb);
-  hipLaunchKernelGGL(gemv_f32_kernel, dim3((unsigned)ceil_div(N, 64)),
-                     dim3(kWaves * 64), 0, stream, x, B, bias, y, (int)K, (int)N,
-                     ldb, accumulate ? 1 : 0);
+  hipLaunchKernelGGL(gemv_f32_kernel, dim3((unsigned)ceil_div(N, kCols)),
+                     dim3(kWaves * 64), 0, stream, x, B, bias, norm_w, norm_eps,
+                     1.0f / (float)K, y, (int)K, (int)N, ldb, accumulate ? 1 : 0);
+  BH_CHECK_HIP(hipGetLastError());
+  return BUDDY_HIP_OK;
+}
+
+int launch_gemv_f32(const float *x, const float *B, const float *bias, float *y,
+                    int64_t K, int64_t N, int64_t ldb, bool accumulate,
+                    hipStream_t stream) {
+  return launch_gemv_f32_norm(x, B, bias, nullptr, 0.f, y, K, N, ldb, accumulate, stream);
+}
+
+int64_t f32_tiles_elems(int64_t K, int64_t N) {
+  return round_up(K, kTileRows) * round_up(N, kTileCols);
+}
+
+int launch_tile_f32(const float *B, int64_t K, int64_t N, int64_t ldb, float *T,
+                    hipStream_t stream) {
+  BH_REQUIRE(B && T, "tile_f32: null pointer");
+  BH_REQUIRE(K > 0 && N > 0 && K < (1 << 30) && N < (1 << 30) && ldb >= N,
+             "tile_f32: bad shape K=%lld N=%lld ldb=%lld", (long long)K, (long long)N,
+             (long long)ldb);
+  const int64_t total = f32_tiles_elems(K, N);
+  hipLaunchKernelGGL(tile_f32_kernel, dim3((unsigned)ceil_div(total, 256)), dim3(256), 0,
+                     stream, B, (int)K, (int)N, ldb, T, total);
+  BH_CHECK_HIP(hipGetLastError());
+  return BUDDY_HIP_OK;
+}
+
+int launch_gemv_f32_tiles(const float *x, const float *T, const float *bias,
+                          const float *norm_w, float norm_eps, float *y, int64_t K,
+                          int64_t N, bool accumulate, hipStream_t stream) {
+  BH_REQUIRE(x && T && y, "gemv_f32_tiles: null pointer");
+  BH_REQUIRE(K > 0 && N > 0 && K < (1 << 30) && N < (1 << 30),
+             "gemv_f32_tiles: bad shape K=%lld N=%lld", (long long)K, (long long)N);
+  BH_REQUIRE((reinterpret_cast<uintptr_t>(T) & 15) == 0,
+             "gemv_f32_tiles: tiles must be 16-byte aligned");
+  hipLaunchKernelGGL(gemv_f32_tiles_kernel, dim3((unsigned)ceil_div(N, kTileCols)),
+                     dim3(kWaves * 64), 0, stream, x, T, bias, norm_w, norm_eps,
+                     1.0f / (float)K, y, (int)K, (int)N, accumulate ? 1 : 0);
   BH_CHECK_HIP(hipGetLastError());
   return BUDDY_HIP_OK;
 }
@@ -112,5 +284,26 @@ int buddy_hip_gemv_f32(const float *x, const float *B, const float *bias,
   return bh::launch_gemv_f32(x, B, bias, y, K, N, N,
                              (flags & BUDDY_HIP_GEMV_ACCUMULATE) != 0,
                              bh::as_stream(stream));
+}
+}
+
+extern "C" {
+size_t buddy_hip_f32_tiles_bytes(int64_t K, int64_t N) {
+  if (K <= 0 || N <= 0)
+    return 0;
+  return (size_t)bh::f32_tiles_elems(K, N) * sizeof(float);
+}
+
+int buddy_hip_tile_f32(const float *B, int64_t K, int64_t N, float *tiles,
+                       buddy_hip_stream stream) {
+  return bh::launch_tile_f32(B, K, N, N, tiles, bh::as_stream(stream));
+}
+
+int buddy_hip_gemv_f32_tiles(const float *x, const float *tiles, const float *bias,
+                             const float *norm_w, float norm_eps, float *y, int64_t K,
+                             int64_t N, unsigned flags, buddy_hip_stream stream) {
+  return bh::launch_gemv_f32_tiles(x, tiles, bias, norm_w, norm_eps, y, K, N,
+                                   (flags & BUDDY_HIP_GEMV_ACCUMULATE) != 0,
+                                   bh::as_stream(stream));
 }
 }

@@ -31,6 +31,11 @@
 namespace bh {
 
 // defined in gemv_f32.hip / matmul_f32.hip
+int launch_tile_f32(const float *B, int64_t K, int64_t N, int64_t ldb, float *T,
+                    hipStream_t stream);
+int launch_gemv_f32_tiles(const float *x, const float *T, const float *bias,
+                          const float *norm_w, float norm_eps, float *y, int64_t K,
+                          int64_t N, bool accumulate, hipStream_t stream);
 int launch_gemv_f32(const float *x, const float *B, const float *bias, float *y,
                     int64_t K, int64_t N, int64_t ldb, bool accumulate,
                     hipStream_t stream);
@@ -55,6 +60,7 @@ struct Layer {
   // the reference's shipped w8a32 build keeps q/k/v in f32 with a bias
   // (they import as AddMMOp, which the quantizer does not touch):
   float *qkv_f32 = nullptr; // [hidden, q|k|v] dense, or null when int8
+  float *qkv_f32_tiles = nullptr; // the same matrix in 1 KiB tiles for the decode GEMV
   float *kc = nullptr, *vc = nullptr; // [kv_heads, max_len, D]
   bool set = false;
 };
@@ -183,10 +189,8 @@ struct Session {
     for (int i = 0; i < S.layers; ++i) {
       Layer &L = layers[(size_t)i];
       if (L.qkv_f32) {
-        if ((rc = launch_rmsnorm(x, L.ln1, xn, 1, S.hidden, S.rms_eps, stream)))
-          return rc;
-        if ((rc = launch_gemv_f32(xn, L.qkv_f32, L.qkv.b, qkv, L.qkv.K, L.qkv.N,
-                                  L.qkv.N, false, stream)))
+        if ((rc = launch_gemv_f32_tiles(x, L.qkv_f32_tiles, L.qkv.b, L.ln1, S.rms_eps,
+                                        qkv, L.qkv.K, L.qkv.N, false, stream)))
           return rc;
       } else if ((rc = gemv(x, L.qkv, nullptr, L.ln1, qkv, kEpiStore))) {
         return rc;
@@ -593,6 +597,7 @@ int buddy_hip_session_set_layer(buddy_hip_session *hs, int index,
     L.qkv.N = QN + 2 * KVN;
     if (f32_qkv) {
       rc |= s->alloc(&L.qkv_f32, (size_t)H * L.qkv.N);
+      rc |= s->alloc(&L.qkv_f32_tiles, buddy_hip_f32_tiles_bytes(H, L.qkv.N) / sizeof(float));
     } else {
       rc |= s->alloc(&L.qkv.w, buddy_hip_w8_packed_bytes(H, L.qkv.N));
       rc |= s->alloc(&L.qkv.s, (size_t)L.qkv.N);
@@ -623,6 +628,8 @@ int buddy_hip_session_set_layer(buddy_hip_session *hs, int index,
                                   KVN * sizeof(float), H, hipMemcpyDefault, s->stream));
     BH_CHECK_HIP(hipMemcpy2DAsync(L.qkv_f32 + QN + KVN, ld, w->fv, KVN * sizeof(float),
                                   KVN * sizeof(float), H, hipMemcpyDefault, s->stream));
+    if ((rc = bh::launch_tile_f32(L.qkv_f32, H, L.qkv.N, L.qkv.N, L.qkv_f32_tiles, s->stream)))
+      return rc;
     BH_CHECK_HIP(hipMemcpyAsync(L.qkv.b, w->bq, QN * sizeof(float), hipMemcpyDefault, s->stream));
     BH_CHECK_HIP(hipMemcpyAsync(L.qkv.b + QN, w->bk, KVN * sizeof(float), hipMemcpyDefault, s->stream));
     BH_CHECK_HIP(hipMemcpyAsync(L.qkv.b + QN + KVN, w->bv, KVN * sizeof(float), hipMemcpyDefault, s->stream));

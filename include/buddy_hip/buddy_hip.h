@@ -318,6 +318,22 @@ int buddy_hip_gemv_f32(const float *x, const float *B, const float *bias,
                        float *y, int64_t K, int64_t N, unsigned flags,
                        buddy_hip_stream stream);
 
+/* The same product over a device-side tile layout, for f32 matrices that stay
+ * resident (the model path's f32 q|k|v weights): 32-row x 8-column tiles of
+ * 1 KiB, zero padded, T[((n/8)*ceil(K/32) + k/32)*256 + (k%32)*8 + n%8] =
+ * B[k,n] with B dense row-major.  It plays the part that the panel packing of
+ * MatMulVectorizationDecodePacked.cpp:207-248 plays on the CPU (each worker
+ * streams one contiguous run), sized for wavefront loads.  With norm_w the
+ * RMSNorm of examples/BuddyDeepSeekR1/subgraph0_decode_simplify.mlir:38-58 is
+ * applied to x on the way: y = bias + (norm_w (.) x * rsqrt(mean(x^2) + eps)) . B.
+ * tiles: buddy_hip_f32_tiles_bytes(K, N) bytes, 16-byte aligned. */
+size_t buddy_hip_f32_tiles_bytes(int64_t K, int64_t N);
+int buddy_hip_tile_f32(const float *B, int64_t K, int64_t N, float *tiles,
+                       buddy_hip_stream stream);
+int buddy_hip_gemv_f32_tiles(const float *x, const float *tiles, const float *bias,
+                             const float *norm_w, float norm_eps, float *y, int64_t K,
+                             int64_t N, unsigned flags, buddy_hip_stream stream);
+
 /* ---- the reference's f32 panel packing -------------------------------------
  * pack_decode_matmul_weights (frontend/Python/graph/transform/
  * pack_decode_weights.py:94-108): flat[nt*K*V + k*V + v] = B[k, nt*V + v]; same

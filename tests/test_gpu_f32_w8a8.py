@@ -34,6 +34,46 @@ def test_f32_gemv_with_bias(bh, oracle, K, N):
     check_close(y.cpu().numpy(), want)
 
 
+@pytest.mark.parametrize("norm", [False, True])
+@pytest.mark.parametrize("K,N", [(1536, 2048), (1536, 256), (128, 64), (100, 70), (33, 9),
+                                 (8960, 1536), (1, 1)])
+def test_f32_gemv_over_tiles(bh, oracle, K, N, norm):
+    g = torch.Generator(device="cuda").manual_seed(K + 2 * N)
+    x = torch.randn(K, generator=g, device="cuda")
+    B = torch.randn((K, N), generator=g, device="cuda") * 0.02
+    bias = torch.randn(N, generator=g, device="cuda")
+    nw = torch.rand(K, generator=g, device="cuda") + 0.5
+    eps = 1e-6
+    nbytes = bh.buddy_hip_f32_tiles_bytes(K, N)
+    assert nbytes == ((K + 31) // 32 * 32) * ((N + 7) // 8 * 8) * 4
+    T = torch.full((nbytes // 4,), float("nan"), device="cuda")
+    y = torch.empty(N, device="cuda")
+    torch.cuda.synchronize()
+    sync_check(bh.buddy_hip_tile_f32(B.data_ptr(), K, N, T.data_ptr(), None))
+    # closed form of the layout, padding zero
+    Th, Bh = T.cpu().numpy(), B.cpu().numpy()
+    blocks = (K + 31) // 32
+    rng = np.random.default_rng(K)
+    for _ in range(200):
+        k, n = int(rng.integers(K)), int(rng.integers(N))
+        assert Th[((n // 8) * blocks + k // 32) * 256 + (k % 32) * 8 + n % 8] == Bh[k, n]
+    assert not np.isnan(Th).any() and np.count_nonzero(Th) == np.count_nonzero(Bh)
+    sync_check(bh.buddy_hip_gemv_f32_tiles(x.data_ptr(), T.data_ptr(), bias.data_ptr(),
+                                           nw.data_ptr() if norm else None, eps,
+                                           y.data_ptr(), K, N, 0, None))
+    xh = x.cpu().numpy()
+    if norm:
+        xh = oracle.rmsnorm(xh, nw.cpu().numpy(), eps)
+    want = bias.cpu().numpy() + oracle.gemv_f32(xh, Bh, np.zeros(N, np.float32), 32, True)
+    check_close(y.cpu().numpy(), want)
+    # accumulate flag: y += ..., deterministic
+    y2 = y.clone()
+    sync_check(bh.buddy_hip_gemv_f32_tiles(x.data_ptr(), T.data_ptr(), None,
+                                           nw.data_ptr() if norm else None, eps,
+                                           y2.data_ptr(), K, N, 1, None))
+    check_close(y2.cpu().numpy(), y.cpu().numpy() + (want - bias.cpu().numpy()))
+
+
 @pytest.mark.parametrize("K,N", [(128, 64), (1536, 8960), (1536, 256)])
 def test_panel_pack_and_packed_gemv(bh, oracle, K, N):
     g = torch.Generator(device="cuda").manual_seed(K)
