@@ -16,12 +16,16 @@ struct GemmW8Args {
   int64_t M = 0, K = 0, N = 0;
   bool accumulate = false;
   int terms = 1; // bf16 terms per activation: 1 = cast to bf16, 3 = all f32 bits
+  // 2 or 3: carry the activations as that many int8 digit planes (fixed point
+  // relative to each row's maximum) and multiply on the int8 matrix cores;
+  // 0: bf16 terms as above
+  int digits = 0;
   // A (same pointer, shape, terms, contents) was the input of the previous
   // matmul on this stream: its bf16 copy is still staged, skip the conversion
   bool reuse_staged_a = false;
-  // Caller-provided bf16 staging of A (written by one of the producers below for
-  // exactly this M, K and terms): no conversion, A itself is not read.
-  const unsigned short *staged = nullptr;
+  // Caller-provided staging of A (written by one of the producers below for
+  // exactly this M, K and terms / digits): no conversion, A itself is not read.
+  const void *staged = nullptr;
 };
 
 // Layout of a bf16 staging buffer: [terms][rows_padded][cols_padded] bf16, term t
@@ -32,6 +36,11 @@ struct GemmStagingLayout {
   size_t bytes(int terms) const {
     return sizeof(unsigned short) * (size_t)terms * rows_padded * cols_padded;
   }
+  // digit planes: [digits][rows_padded][cols_padded] int8, then the row steps
+  // (f32 [rows_padded])
+  size_t bytes_digits(int digits) const {
+    return (size_t)digits * rows_padded * cols_padded + sizeof(float) * (size_t)rows_padded;
+  }
 };
 GemmStagingLayout gemm_staging_layout(int64_t M, int64_t K);
 // Producers that write their result straight into a staging buffer:
@@ -41,6 +50,15 @@ int launch_rmsnorm_to_staging(const float *x, const float *w, int rows, int n, f
                               int terms, unsigned short *staged, hipStream_t stream);
 int launch_silu_mul_to_staging(const float *g, const float *u, int rows, int n, int terms,
                                unsigned short *staged, hipStream_t stream);
+// the same producers for digit planes, and the plain conversion of A
+int launch_rmsnorm_to_digits(const float *x, const float *w, int rows, int n, float eps,
+                             int digits, void *staged, hipStream_t stream);
+int launch_silu_mul_to_digits(const float *g, const float *u, int rows, int n, int digits,
+                              void *staged, hipStream_t stream);
+int launch_activations_to_digits(const float *A, int64_t lda, int64_t M, int64_t K,
+                                 int digits, void *staged, hipStream_t stream);
+// the matmul over digit planes (called by launch_gemm_w8 when digits != 0)
+int launch_gemm_w8_digits(const GemmW8Args &a, const void *planes, hipStream_t stream);
 
 int launch_gemm_w8(const GemmW8Args &a, hipStream_t stream);
 

@@ -523,17 +523,20 @@ struct Staging {
 std::mutex g_staging_mutex;
 std::map<hipStream_t, Staging> g_staging;
 
+// what the staged copy holds: bf16 terms (1..3) or digit planes (16 + digits)
+int precision_key(const GemmW8Args &in) { return in.digits ? 16 + in.digits : in.terms; }
+
 int staging_for(hipStream_t stream, size_t bytes, const GemmW8Args &in, u16 **out,
                 bool *holds_input) {
   std::lock_guard<std::mutex> lock(g_staging_mutex);
   Staging &s = g_staging[stream];
   *holds_input = in.reuse_staged_a && s.ptr && s.src == in.A && s.lda == in.lda &&
-                 s.M == (int)in.M && s.K == (int)in.K && s.terms == in.terms;
+                 s.M == (int)in.M && s.K == (int)in.K && s.terms == precision_key(in);
   s.src = in.A;
   s.lda = in.lda;
   s.M = (int)in.M;
   s.K = (int)in.K;
-  s.terms = in.terms;
+  s.terms = precision_key(in);
   if (s.bytes < bytes) {
     if (s.ptr) {
       BH_CHECK_HIP(hipStreamSynchronize(stream)); // an earlier matmul may still read it
@@ -616,6 +619,11 @@ int launch_gemm_w8(const GemmW8Args &in, hipStream_t stream) {
   BH_REQUIRE((in.staged || in.lda >= in.K) && in.ldc >= in.N,
              "gemm_w8: row stride below row length");
   BH_REQUIRE(in.terms >= 1 && in.terms <= 3, "gemm_w8: terms=%d outside 1..3", in.terms);
+  BH_REQUIRE(in.digits == 0 || (in.digits >= 2 && in.digits <= 3),
+             "gemm_w8: digits=%d outside 2..3", in.digits);
+  BH_REQUIRE(in.digits == 0 || in.K <= (1 << 17),
+             "gemm_w8: K=%lld beyond 2^17 would overflow the int32 sums of the digit planes",
+             (long long)in.K);
   BH_REQUIRE(!(in.bias && in.accumulate), "gemm_w8: bias with accumulate");
   BH_REQUIRE((reinterpret_cast<uintptr_t>(in.W) & 15) == 0,
              "gemm_w8: packed weights must be 16-byte aligned");
@@ -635,12 +643,19 @@ int launch_gemm_w8(const GemmW8Args &in, hipStream_t stream) {
   a.ncols = (int)ceil_div(a.groups, kGroupsPerWave);
   a.cols_padded = (int)round_up(a.ncols, 8);
   a.accumulate = in.accumulate ? 1 : 0;
-  u16 *abf = const_cast<u16 *>(in.staged);
+  u16 *abf = static_cast<u16 *>(const_cast<void *>(in.staged));
   bool staged = in.staged != nullptr;
-  int rc = staged ? BUDDY_HIP_OK : staging_for(stream, sizeof(u16) * in.terms * (size_t)a.Mp * a.Kp, in, &abf,
-                       &staged);
+  const size_t staging_bytes =
+      in.digits ? layout.bytes_digits(in.digits) : layout.bytes(in.terms);
+  int rc = staged ? BUDDY_HIP_OK : staging_for(stream, staging_bytes, in, &abf, &staged);
   if (rc)
     return rc;
+  if (in.digits) {
+    if (!staged &&
+        (rc = launch_activations_to_digits(in.A, in.lda, in.M, in.K, in.digits, abf, stream)))
+      return rc;
+    return launch_gemm_w8_digits(in, abf, stream);
+  }
   a.Abf = abf;
   if (!staged) {
     const int64_t threads = (int64_t)a.Mp * (a.Kp / 8);
@@ -713,6 +728,7 @@ int buddy_hip_gemm_w8a32(const float *A, const int8_t *packed, const float *scal
   a.N = N;
   a.accumulate = (flags & BUDDY_HIP_GEMV_ACCUMULATE) != 0;
   a.terms = (flags & BUDDY_HIP_GEMM_A_F32_EXACT) ? 3 : 1;
+  a.digits = (flags & BUDDY_HIP_GEMM_A_I8_DIGITS) ? 3 : 0;
   return bh::launch_gemm_w8(a, bh::as_stream(stream));
 }
 }

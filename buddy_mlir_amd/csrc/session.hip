@@ -23,6 +23,7 @@
 #include "gemv_w8a32.h"
 #include "kv_cache.h"
 
+#include <algorithm>
 #include <cmath>
 #include <cstring>
 #include <new>
@@ -110,6 +111,7 @@ struct Session {
   int *pf_tokens = nullptr;
   unsigned short *pf_xn_bf = nullptr, *pf_g_bf = nullptr; // bf16 matmul inputs
   int gemm_terms = 3; // bf16 terms per activation in the prefill matmuls (3 = exact)
+  int gemm_digits = 3; // int8 digit planes instead of bf16 terms when not 0
 
   template <typename T> int alloc(T **p, size_t n) {
     void *q = nullptr;
@@ -282,8 +284,10 @@ struct Session {
     BH_CHECK_HIP(hipMalloc((void **)&pf_tokens, sizeof(int) * rows));
     // bf16 staging of the matmul inputs that the norm and SiLU kernels write
     // directly (up to three terms)
-    BH_CHECK_HIP(hipMalloc((void **)&pf_xn_bf, gemm_staging_layout(rows, S.hidden).bytes(3)));
-    BH_CHECK_HIP(hipMalloc((void **)&pf_g_bf, gemm_staging_layout(rows, S.inter).bytes(3)));
+    const GemmStagingLayout lx = gemm_staging_layout(rows, S.hidden),
+                            lg = gemm_staging_layout(rows, S.inter);
+    BH_CHECK_HIP(hipMalloc((void **)&pf_xn_bf, std::max(lx.bytes(3), lx.bytes_digits(3))));
+    BH_CHECK_HIP(hipMalloc((void **)&pf_g_bf, std::max(lg.bytes(3), lg.bytes_digits(3))));
     pf_rows = rows;
     return BUDDY_HIP_OK;
   }
@@ -303,6 +307,7 @@ struct Session {
     g.N = W.N;
     g.accumulate = accumulate;
     g.terms = gemm_terms;
+    g.digits = gemm_digits;
     g.reuse_staged_a = same_input_as_before;
     return launch_gemm_w8(g, stream);
   }
@@ -321,7 +326,23 @@ struct Session {
     g.N = W.N;
     g.accumulate = accumulate;
     g.terms = gemm_terms;
+    g.digits = gemm_digits;
     return launch_gemm_w8(g, stream);
+  }
+  // RMSNorm rows / SiLU(g) * u written straight into the matmul's input format
+  int norm_to_staging(const float *x, const float *w, int rows, unsigned short *staged) {
+    const auto &S = shape;
+    if (gemm_digits)
+      return launch_rmsnorm_to_digits(x, w, rows, S.hidden, S.rms_eps, gemm_digits, staged,
+                                      stream);
+    return launch_rmsnorm_to_staging(x, w, rows, S.hidden, S.rms_eps, gemm_terms, staged,
+                                     stream);
+  }
+  int silu_mul_to_staging(const float *g, const float *u, int rows, unsigned short *staged) {
+    const auto &S = shape;
+    if (gemm_digits)
+      return launch_silu_mul_to_digits(g, u, rows, S.inter, gemm_digits, staged, stream);
+    return launch_silu_mul_to_staging(g, u, rows, S.inter, gemm_terms, staged, stream);
   }
 
   // Prompt processing for tokens already in pf_tokens: fills cache rows
@@ -347,8 +368,7 @@ struct Session {
           return rc;
       } else {
         // the norm writes the matmul's bf16 input directly
-        if ((rc = launch_rmsnorm_to_staging(pf_x, L.ln1, n, S.hidden, S.rms_eps,
-                                            gemm_terms, pf_xn_bf, stream)))
+        if ((rc = norm_to_staging(pf_x, L.ln1, n, pf_xn_bf)))
           return rc;
         if ((rc = gemm_staged(pf_xn_bf, L.qkv, pf_qkv, n, false)))
           return rc;
@@ -377,15 +397,13 @@ struct Session {
         return rc;
       if ((rc = gemm(pf_att, L.o, pf_x, n, true)))
         return rc;
-      if ((rc = launch_rmsnorm_to_staging(pf_x, L.ln2, n, S.hidden, S.rms_eps,
-                                          gemm_terms, pf_xn_bf, stream)))
+      if ((rc = norm_to_staging(pf_x, L.ln2, n, pf_xn_bf)))
         return rc;
       if ((rc = gemm_staged(pf_xn_bf, L.gate, pf_g, n, false)))
         return rc;
       if ((rc = gemm_staged(pf_xn_bf, L.up, pf_u, n, false)))
         return rc;
-      if ((rc = launch_silu_mul_to_staging(pf_g, pf_u, n, S.inter, gemm_terms, pf_g_bf,
-                                           stream)))
+      if ((rc = silu_mul_to_staging(pf_g, pf_u, n, pf_g_bf)))
         return rc;
       if ((rc = gemm_staged(pf_g_bf, L.down, pf_x, n, true)))
         return rc;
@@ -832,10 +850,13 @@ void buddy_hip_session_adopt(buddy_hip_session *hs, void *device_ptr) {
     s->owned.push_back(device_ptr);
 }
 
-int buddy_hip_session_set_prefill_precision(buddy_hip_session *hs, int exact) {
+int buddy_hip_session_set_prefill_precision(buddy_hip_session *hs, int mode) {
   Session *s = reinterpret_cast<Session *>(hs);
   BH_REQUIRE(s, "session_set_prefill_precision: null session");
-  s->gemm_terms = exact ? 3 : 1;
+  BH_REQUIRE(mode >= 0 && mode <= 2, "session_set_prefill_precision: mode %d outside 0..2",
+             mode);
+  s->gemm_terms = mode == 1 ? 3 : 1;
+  s->gemm_digits = mode == 2 ? 3 : 0;
   return BUDDY_HIP_OK;
 }
 

@@ -145,8 +145,14 @@ int buddy_hip_linear_w8a32(const buddy_hip_linear_desc *desc,
  * same wave-tile copy the decode kernel reads.  Activations are cast to bf16
  * (round to nearest even) and multiplied on MFMA with f32 accumulation; with
  * BUDDY_HIP_GEMM_A_F32_EXACT each activation is carried as three bf16 terms,
- * i.e. with all 24 significand bits.  BUDDY_HIP_GEMV_ACCUMULATE as above. */
-enum { BUDDY_HIP_GEMM_A_F32_EXACT = 2 };
+ * i.e. with all 24 significand bits.  With BUDDY_HIP_GEMM_A_I8_DIGITS the
+ * activations become fixed point instead -- per row a power-of-two step s with
+ * |a| / s < 2^22, rint(a / s) written as three balanced base-256 digits -- and
+ * the int8 weights are multiplied as they are on the int8 matrix cores, with
+ * exact int32 sums: the only rounding is that of a, at most 2^-23 of the row's
+ * largest magnitude (NaN and infinity do not survive it; K <= 2^17).
+ * BUDDY_HIP_GEMV_ACCUMULATE as above. */
+enum { BUDDY_HIP_GEMM_A_F32_EXACT = 2, BUDDY_HIP_GEMM_A_I8_DIGITS = 4 };
 int buddy_hip_gemm_w8a32(const float *A, const int8_t *packed, const float *scale,
                          float *C, int64_t M, int64_t K, int64_t N,
                          unsigned flags, buddy_hip_stream stream);
@@ -282,9 +288,11 @@ int buddy_hip_session_prefill_all_logits(buddy_hip_session *s, const int *tokens
                                          float *logits_out);
 /* Hands a device allocation to the session, which frees it when destroyed. */
 void buddy_hip_session_adopt(buddy_hip_session *s, void *device_ptr);
-/* 1 (default): prefill activations keep all f32 bits (three bf16 terms);
- * 0: they are cast to bf16, one MFMA pass instead of three. */
-int buddy_hip_session_set_prefill_precision(buddy_hip_session *s, int exact);
+/* How the prefill matmuls carry their f32 activations:
+ * 1: all f32 bits (three bf16 terms); 0: cast to bf16, one MFMA pass instead of
+ * three; 2 (default): three int8 digit planes on the int8 matrix cores, 23 bits
+ * below each row's largest magnitude (BUDDY_HIP_GEMM_A_I8_DIGITS). */
+int buddy_hip_session_set_prefill_precision(buddy_hip_session *s, int mode);
 /* Asynchronous pieces of the call above, for timing: set the device-side
  * (token, position), then enqueue steps on the session stream. */
 int buddy_hip_session_set_state(buddy_hip_session *s, int token, int pos);

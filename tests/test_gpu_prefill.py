@@ -28,30 +28,80 @@ GEMM_SHAPES = [(512, 1536, 1536), (512, 1536, 256), (512, 1536, 8960), (512, 896
                (500, 200, 6500), (1000, 72, 3300)]
 
 
+def fixed_point_round(a: np.ndarray, digits: int = 3):
+    """What the int8 matmul multiplies: per row the smallest power-of-two step s
+    with max|a| / s < 2^(8 digits - 2), and rint(a / s) * s."""
+    mx = np.abs(a).max(axis=1, keepdims=True).astype(np.float64)
+    e = np.floor(np.log2(np.where(mx > 0, mx, 1.0))) + 1 - (8 * digits - 2)
+    step = np.exp2(np.maximum(e, -126))
+    return (np.rint(a.astype(np.float64) / step) * step).astype(np.float32), step
+
+
 @pytest.mark.parametrize("M,K,N", GEMM_SHAPES)
-@pytest.mark.parametrize("exact", [False, True])
-def test_prefill_gemm_matches_blis_oracle(oracle, M, K, N, exact):
+@pytest.mark.parametrize("mode", ["bf16", "exact", "digits"])
+def test_prefill_gemm_matches_blis_oracle(oracle, M, K, N, mode):
     q, s = synthetic.quantized_linear(K, N, M + K + N)
     packed = ops.pack_w8(q)
     g = torch.Generator(device="cuda").manual_seed(M)
     x = torch.randn((M, K), generator=g, device="cuda")
-    y = ops.gemm_w8a32(x, packed, s, K, N, exact=exact)
+    if mode == "digits" and M > 2:
+        x[1] *= 1e-30   # rows of very different magnitude: the step is per row
+        x[2, 0] = 300.0  # one large element in a row of small ones
+    y = ops.gemm_w8a32(x, packed, s, K, N, exact=mode == "exact", digits=mode == "digits")
     torch.cuda.synchronize()
     xh = x.cpu().numpy()
+    if mode == "digits":
+        # against the plain f32 input at the stated bar, per row (rows differ by
+        # 30 orders of magnitude) ...
+        want = oracle.blis_gemm_w8a32(xh, q.cpu().numpy(), s.cpu().numpy())
+        got = y.cpu().numpy()
+        for m in range(M):
+            check_close(got[m], want[m])
+        # ... and against the oracle fed the same fixed-point activations, where
+        # what is left is summation order only
+        a_in, _ = fixed_point_round(xh)
+        want = oracle.blis_gemm_w8a32(a_in, q.cpu().numpy(), s.cpu().numpy())
+        for m in range(M):
+            check_close(got[m], want[m], normwise=4e-6)
+        return
     # "activations cast to bf16": the oracle gets the same rounded activations
-    a_in = xh if exact else bf16_round(xh)
+    a_in = xh if mode == "exact" else bf16_round(xh)
     want = oracle.blis_gemm_w8a32(a_in, q.cpu().numpy(), s.cpu().numpy())
     check_close(y.cpu().numpy(), want)
 
 
+@pytest.mark.parametrize("M,K", [(1, 64), (5, 100), (70, 1536), (48, 8960)])
+def test_digit_planes_are_the_rounded_fixed_point(M, K):
+    """W = 127 I with scale 1/127 copies the activations: what comes out is
+    rint(a / s) * s exactly, row by row."""
+    g = torch.Generator(device="cuda").manual_seed(K)
+    x = torch.randn((M, K), generator=g, device="cuda") * 3.0
+    x[0, 0] = 0.0
+    if M > 1:
+        x[1] = 0.0  # an all-zero row
+        x[M - 1] *= 2.0 ** -100
+    q = (torch.eye(K, device="cuda") * 127).to(torch.int8)
+    s = torch.full((K,), 1.0 / 127.0, device="cuda")
+    y = ops.gemm_w8a32(x, ops.pack_w8(q), s, K, K, digits=True)
+    torch.cuda.synchronize()
+    want, step = fixed_point_round(x.cpu().numpy())
+    got = y.cpu().numpy().astype(np.float64)
+    # 127 * (1/127 rounded to f32) is 1 to within 1 ulp of f32
+    np.testing.assert_allclose(got, want, rtol=2e-7, atol=0)
+    xh = x.cpu().numpy().astype(np.float64)
+    assert (np.abs(got - xh) <= 0.5 * step + 2e-7 * np.abs(xh)).all()
+
+
+@pytest.mark.parametrize("exact", [True, False])
 @pytest.mark.parametrize("M,K,N", [(100, 256, 96), (490, 136, 6600)])
-def test_prefill_gemm_accumulates(oracle, M, K, N):
+def test_prefill_gemm_accumulates(oracle, M, K, N, exact):
     q, s = synthetic.quantized_linear(K, N, 77)
     g = torch.Generator(device="cuda").manual_seed(1)
     x = torch.randn((M, K), generator=g, device="cuda")
     c0 = torch.randn((M, N), generator=g, device="cuda")
     c = c0.clone()
-    ops.gemm_w8a32(x, ops.pack_w8(q), s, K, N, out=c, accumulate=True, exact=True)
+    ops.gemm_w8a32(x, ops.pack_w8(q), s, K, N, out=c, accumulate=True, exact=exact,
+                   digits=not exact)
     torch.cuda.synchronize()
     want = oracle.blis_gemm_w8a32(x.cpu().numpy(), q.cpu().numpy(), s.cpu().numpy(),
                                   c0.cpu().numpy())
@@ -100,8 +150,8 @@ def test_prefill_attention_gqa_and_longer_keys(bh, oracle):
     check_close(run_attn(bh, q, k, v, None, H, HKV, Lq, Lk), want)
 
 
-@pytest.mark.parametrize("exact", [True, False])
-def test_small_model_block_prefill_equals_token_by_token(oracle, exact):
+@pytest.mark.parametrize("precision", ["digits", "exact", "bf16"])
+def test_small_model_block_prefill_equals_token_by_token(oracle, precision):
     """Prefill of 40 prompt tokens as one block against 40 oracle decode steps:
     last-token logits, greedy token and every cache row written; then decode
     continues from the prefilled cache."""
@@ -111,8 +161,8 @@ def test_small_model_block_prefill_equals_token_by_token(oracle, exact):
     toks = synthetic.first_tokens(SMALL, 40, seed=3).tolist()
     for pos, t in enumerate(toks):
         otok, ologits = om.decode_step(t, pos, kv)
-    nxt, logits = sess.prefill(toks, 0, exact=exact)
-    if exact:
+    nxt, logits = sess.prefill(toks, 0, precision=precision)
+    if precision != "bf16":
         check_close(logits, ologits)
         assert nxt == otok
         for j in range(2 * SMALL.layers):
