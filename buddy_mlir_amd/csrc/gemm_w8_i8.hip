@@ -26,9 +26,11 @@
 // contiguous bytes of a plane row.
 //
 // Two workgroup shapes, as for bf16: 64 rows x 64 channels with K split over the
-// four wavefronts (narrow matrices), and 64 or 48 rows x 256 channels with the
-// activation fragments shared through LDS (wide matrices).
+// four wavefronts (narrow matrices), and 64 or 48 rows x 256 or 320 channels with
+// the activation fragments shared through LDS (wide matrices).
 #include "gemm.h"
+
+#include <algorithm>
 
 namespace bh {
 namespace {
@@ -47,31 +49,71 @@ __device__ __forceinline__ float digit_step(float mx, int D) {
   return __uint_as_float((unsigned)(e + 127) << 23);
 }
 
+// Row sources: four consecutive values k0..k0+3 of the row (zero past its end).
+__device__ __forceinline__ void load4(const float *p, int k0, int n, float (&v)[4]) {
+  if (k0 + 3 < n && (reinterpret_cast<uintptr_t>(p + k0) & 15) == 0) {
+    const float4 q = *reinterpret_cast<const float4 *>(p + k0);
+    v[0] = q.x; v[1] = q.y; v[2] = q.z; v[3] = q.w;
+  } else {
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+      v[e] = k0 + e < n ? p[k0 + e] : 0.f;
+  }
+}
 struct PlainRow {
   const float *a;
-  __device__ __forceinline__ float operator()(int k) const { return a[k]; }
+  int n;
+  __device__ __forceinline__ void operator()(int k0, float (&v)[4]) const {
+    load4(a, k0, n, v);
+  }
 };
 struct NormRow { // w * (x * rs)
   const float *x, *w;
   float rs;
-  __device__ __forceinline__ float operator()(int k) const { return w[k] * (x[k] * rs); }
+  int n;
+  __device__ __forceinline__ void operator()(int k0, float (&v)[4]) const {
+    float xv[4], wv[4];
+    load4(x, k0, n, xv);
+    load4(w, k0, n, wv);
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+      v[e] = wv[e] * (xv[e] * rs);
+  }
 };
 struct SiluMulRow { // silu(g) * u
   const float *g, *u;
-  __device__ __forceinline__ float operator()(int k) const {
-    const float gv = g[k];
-    const float sig = 1.0f / (1.0f + expf(-gv));
-    return (gv * sig) * u[k];
+  int n;
+  __device__ __forceinline__ void operator()(int k0, float (&v)[4]) const {
+    float gv[4], uv[4];
+    load4(g, k0, n, gv);
+    load4(u, k0, n, uv);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const float sig = 1.0f / (1.0f + expf(-gv[e]));
+      v[e] = (gv[e] * sig) * uv[e];
+    }
   }
 };
 
+// Rows of up to this many values are kept in LDS between the pass that finds the
+// row maximum and the pass that writes the digits; longer rows are computed twice.
+constexpr int kRowCache = 12288;
+
 // One workgroup of 256 threads writes row `row` of every plane and its step.
+// A thread owns the same groups of four values in both passes.
 template <class F>
 __device__ __forceinline__ void row_to_digits(const F &f, int n, int row, int D, int Mp,
-                                              int Kp, int8_t *planes, float *red) {
+                                              int Kp, int8_t *planes, float *red,
+                                              float *cache) {
+  const bool cached = Kp <= kRowCache;
   float mx = 0.f;
-  for (int k = threadIdx.x; k < n; k += 256)
-    mx = fmaxf(mx, fabsf(f(k)));
+  for (int k0 = threadIdx.x * 4; k0 < Kp; k0 += 256 * 4) {
+    float v[4];
+    f(k0, v);
+    mx = fmaxf(fmaxf(mx, fmaxf(fabsf(v[0]), fabsf(v[1]))), fmaxf(fabsf(v[2]), fabsf(v[3])));
+    if (cached)
+      *reinterpret_cast<float4 *>(cache + k0) = make_float4(v[0], v[1], v[2], v[3]);
+  }
   mx = wave_max(mx);
   __syncthreads(); // red may still be read by the caller's own reduction
   if ((threadIdx.x & 63) == 0)
@@ -85,10 +127,17 @@ __device__ __forceinline__ void row_to_digits(const F &f, int n, int row, int D,
     steps[row] = step;
   const size_t plane = (size_t)Mp * Kp;
   for (int k0 = threadIdx.x * 4; k0 < Kp; k0 += 256 * 4) {
+    float v[4];
+    if (cached) {
+      const float4 q = *reinterpret_cast<const float4 *>(cache + k0);
+      v[0] = q.x; v[1] = q.y; v[2] = q.z; v[3] = q.w;
+    } else {
+      f(k0, v);
+    }
     int X[4];
 #pragma unroll
     for (int e = 0; e < 4; ++e)
-      X[e] = k0 + e < n ? (int)rintf(f(k0 + e) * inv) : 0;
+      X[e] = (int)rintf(v[e] * inv);
     int8_t *dst = planes + (size_t)row * Kp + k0;
     for (int j = 0; j < D; ++j) {
       unsigned word = 0;
@@ -108,6 +157,7 @@ __global__ void __launch_bounds__(256)
 activations_to_digits_kernel(const float *__restrict__ A, int64_t lda, int M, int K, int D,
                              int Mp, int Kp, int8_t *__restrict__ planes) {
   __shared__ float red[4];
+  extern __shared__ __attribute__((aligned(16))) float row_cache[];
   const int row = blockIdx.x;
   if (row >= M) { // padding rows: zero digits, step 1
     for (int j = 0; j < D; ++j)
@@ -117,7 +167,8 @@ activations_to_digits_kernel(const float *__restrict__ A, int64_t lda, int M, in
       reinterpret_cast<float *>(planes + (size_t)D * Mp * Kp)[row] = 1.0f;
     return;
   }
-  row_to_digits(PlainRow{A + (int64_t)row * lda}, K, row, D, Mp, Kp, planes, red);
+  row_to_digits(PlainRow{A + (int64_t)row * lda, K}, K, row, D, Mp, Kp, planes, red,
+                row_cache);
 }
 
 __global__ void __launch_bounds__(256)
@@ -125,6 +176,7 @@ rmsnorm_to_digits_kernel(const float *__restrict__ x, const float *__restrict__ 
                          float inv_n, float eps, int D, int Mp, int Kp,
                          int8_t *__restrict__ planes) {
   __shared__ float red[4];
+  extern __shared__ __attribute__((aligned(16))) float row_cache[];
   const int row = blockIdx.x;
   const float *xr = x + (size_t)row * n;
   float s = 0.f;
@@ -136,16 +188,17 @@ rmsnorm_to_digits_kernel(const float *__restrict__ x, const float *__restrict__ 
   __syncthreads();
   const float tot = (red[0] + red[1]) + (red[2] + red[3]);
   const float rs = 1.0f / sqrtf(tot * inv_n + eps);
-  row_to_digits(NormRow{xr, w, rs}, n, row, D, Mp, Kp, planes, red);
+  row_to_digits(NormRow{xr, w, rs, n}, n, row, D, Mp, Kp, planes, red, row_cache);
 }
 
 __global__ void __launch_bounds__(256)
 silu_mul_to_digits_kernel(const float *__restrict__ g, const float *__restrict__ u, int n,
                           int D, int Mp, int Kp, int8_t *__restrict__ planes) {
   __shared__ float red[4];
+  extern __shared__ __attribute__((aligned(16))) float row_cache[];
   const int row = blockIdx.x;
-  row_to_digits(SiluMulRow{g + (size_t)row * n, u + (size_t)row * n}, n, row, D, Mp, Kp,
-                planes, red);
+  row_to_digits(SiluMulRow{g + (size_t)row * n, u + (size_t)row * n, n}, n, row, D, Mp, Kp,
+                planes, red, row_cache);
 }
 
 // ---- the matmul ----------------------------------------------------------------
@@ -307,63 +360,76 @@ __global__ void __launch_bounds__(kSlices *kWave) gemm_w8_i8_kernel(GemmI8Args a
   }
 }
 
-// Wide matrices: 16 RB rows x 256 channels per workgroup, one 64-channel span per
-// wavefront, every wavefront runs the whole K.  Wavefront w fetches the digit
-// fragments of row block w for everyone and leaves them in LDS in fragment order
-// (lane l at 16 l: conflict-free).  Weights go from global memory to registers
-// to the matrix core.
+// Wide matrices: 16 RB rows x 64 GPW channels per workgroup (GPW channel groups
+// per wavefront), every wavefront runs the whole K.  Wavefront w fetches the
+// digit fragments of row block w for everyone and leaves them in LDS in fragment
+// order (lane l at 16 l: conflict-free).  Weights go from global memory to
+// registers to the matrix core.
 //
-// Global loads run kRing - 2 chunks ahead of the matrix cores.  The compiler
-// sinks ordinary loads down to their first use (and then waits for them there),
-// so the loads of this loop are issued by hand and waited for by hand: a fetch
-// is 4 + D loads in a fixed order, vmcnt counts them in order, and each wait
-// names the registers it releases so that nothing reads them earlier.  The ring
-// registers must never be spilled (a reload would read a register while its load
-// is in flight): the build refuses scratch use in this file.
-constexpr int kRing = 5;
+// The loop is a pipeline of three stages so that the matrix cores never wait:
+//  * global loads run kRing - 2 chunks ahead.  The compiler sinks ordinary loads
+//    down to their first use (and then waits for them there), so they are issued
+//    by hand and waited for by hand: a fetch is GPW + D loads in a fixed order,
+//    vmcnt counts them in order, and each wait names the registers it releases
+//    so that nothing reads them earlier.  The ring registers must never be
+//    spilled (a reload would read a register while its load is in flight): the
+//    build refuses scratch use in this file;
+//  * the fragments of chunk c + 2 go to LDS at the top of chunk c (three
+//    buffers), so the barrier that closes chunk c publishes them a whole chunk
+//    before they are wanted;
+//  * the fragments of the next digit plane (or of the next chunk's first one)
+//    are read from LDS into the second half of a two-slot register buffer while
+//    the matrix instructions of the current plane run.
+template <int GPW> struct RingDepth { static constexpr int value = GPW > 4 ? 4 : 5; };
 
 __device__ __forceinline__ void issue_load(v4i32 &dst, const void *p) {
   asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(dst) : "v"(p) : "memory");
 }
-template <int D> struct FetchRegs {
-  v4i32 w[kGroupsPerWave];
+template <int D, int GPW> struct FetchRegs {
+  v4i32 w[GPW];
   v4i32 a[D];
 };
-template <int N, int D> __device__ __forceinline__ void wait_loads(FetchRegs<D> &f) {
-  static_assert(kGroupsPerWave == 4, "operand list below");
-  asm volatile("s_waitcnt vmcnt(%4)"
-               : "+v"(f.w[0]), "+v"(f.w[1]), "+v"(f.w[2]), "+v"(f.w[3])
-               : "n"(N)
-               : "memory");
+// Waits until at most N loads are in flight; the registers of `f` are only valid
+// after it.
+template <int N, int D, int GPW>
+__device__ __forceinline__ void wait_loads(FetchRegs<D, GPW> &f) {
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+#pragma unroll
+  for (int g = 0; g < GPW; ++g)
+    asm volatile("" : "+v"(f.w[g])::"memory");
 #pragma unroll
   for (int j = 0; j < D; ++j)
     asm volatile("" : "+v"(f.a[j])::"memory");
 }
 
-template <int D, int RB>
+template <int D, int RB, int GPW>
 __global__ void __launch_bounds__(kSlices *kWave) gemm_w8_i8_wide_kernel(GemmI8Args a) {
-  constexpr int L = kGroupsPerWave + D; // loads per fetch
-  extern __shared__ __attribute__((aligned(16))) v4i32 frag_s[]; // [2][D][RB][64]
+  constexpr int kRing = RingDepth<GPW>::value;
+  constexpr int L = GPW + D; // loads per fetch
+  // chunks per unrolled pass: a multiple of the ring, and an even number of
+  // digit steps so that the two-slot fragment buffer is back where it started
+  constexpr int kPass = (kRing * D) % 2 == 0 ? kRing : 2 * kRing;
+  extern __shared__ __attribute__((aligned(16))) v4i32 frag_s[]; // [3][D][RB][64]
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int col = blockIdx.x % a.cols_padded, rbk = blockIdx.x / a.cols_padded;
   if (col >= a.ncols)
     return; // padding id
   const int m0 = rbk * RB * 16;
-  const int g0 = (col * kSlices + wave) * kGroupsPerWave;
+  const int g0 = (col * kSlices + wave) * GPW;
 
-  v4i32 acc[kGroupsPerWave][RB][D];
+  v4i32 acc[GPW][RB][D];
 #pragma unroll
-  for (int g = 0; g < kGroupsPerWave; ++g)
+  for (int g = 0; g < GPW; ++g)
 #pragma unroll
     for (int rb = 0; rb < RB; ++rb)
 #pragma unroll
       for (int j = 0; j < D; ++j)
         acc[g][rb][j] = v4i32{0, 0, 0, 0};
 
-  const v4i32 *wp[kGroupsPerWave];
+  const v4i32 *wp[GPW];
 #pragma unroll
-  for (int g = 0; g < kGroupsPerWave; ++g) // groups past the end repeat the last one
+  for (int g = 0; g < GPW; ++g) // groups past the end repeat the last one
     wp[g] = reinterpret_cast<const v4i32 *>(a.W) +
             ((size_t)min(g0 + g, a.groups - 1) * a.chunks) * 64 + lane;
   const size_t plane = (size_t)a.Mp * a.Kp;
@@ -372,66 +438,75 @@ __global__ void __launch_bounds__(kSlices *kWave) gemm_w8_i8_wide_kernel(GemmI8A
   const int my_rb = min(wave, RB - 1);
   const int8_t *ap = a.planes + (size_t)(m0 + my_rb * 16 + (lane & 15)) * a.Kp + (lane >> 4) * 16;
 
-  FetchRegs<D> ring[kRing];
+  FetchRegs<D, GPW> ring[kRing];
   // chunks past the end are fetched again from the last chunk (never used):
   // every fetch is exactly L loads, which is what keeps the counts below exact
-  auto fetch = [&](int c, FetchRegs<D> &f) {
+  auto fetch = [&](int c, FetchRegs<D, GPW> &f) {
     const int cc = min(c, a.chunks - 1);
 #pragma unroll
-    for (int g = 0; g < kGroupsPerWave; ++g)
+    for (int g = 0; g < GPW; ++g)
       issue_load(f.w[g], wp[g] + (size_t)cc * 64);
 #pragma unroll
     for (int j = 0; j < D; ++j)
       issue_load(f.a[j], ap + j * plane + (size_t)cc * kTileK);
   };
-  auto stage = [&](const FetchRegs<D> &f, int buf) { // own row block -> LDS
+  auto stage = [&](const FetchRegs<D, GPW> &f, int buf) { // own row block -> LDS
     if (wave >= RB)
       return;
 #pragma unroll
     for (int j = 0; j < D; ++j)
       frag_s[(((size_t)buf * D + j) * RB + wave) * kWave + lane] = f.a[j];
   };
+  auto read_frags = [&](v4i32(&dst)[RB], int buf, int j) {
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb)
+      dst[rb] = frag_s[(((size_t)buf * D + j) * RB + rb) * kWave + lane];
+  };
 #pragma unroll
   for (int u = 0; u < kRing; ++u)
     fetch(u, ring[u]);
-  wait_loads<(kRing - 1) * L, D>(ring[0]); // chunk 0 has arrived
+  wait_loads<(kRing - 1) * L, D, GPW>(ring[0]); // chunk 0 has arrived
   stage(ring[0], 0);
+  wait_loads<(kRing - 2) * L, D, GPW>(ring[1]);
+  stage(ring[1], 1);
   __syncthreads();
-  for (int c0 = 0; c0 < a.chunks; c0 += kRing) {
+  v4i32 af[2][RB];
+  read_frags(af[0], 0, 0);
+  int buf = 0; // LDS buffer of chunk c: c % 3
+  for (int c0 = 0; c0 < a.chunks; c0 += kPass) {
 #pragma unroll
-    for (int u = 0; u < kRing; ++u) {
+    for (int u = 0; u < kPass; ++u) {
       const int c = c0 + u;
       if (c < a.chunks) {
-        const int buf = c & 1;
-        FetchRegs<D> &cur = ring[u];
-        FetchRegs<D> &nxt = ring[(u + 1) % kRing];
-        // in flight: chunks c+1 .. c+kRing-1 (chunk c was waited for when it was
-        // staged).  Release chunk c+1 and put its row block into the other
-        // buffer, whose readers passed the barrier that closed chunk c-1.
-        wait_loads<(kRing - 2) * L, D>(nxt);
-        stage(nxt, buf ^ 1);
-        // all fragments of the chunk first, one wait, then nothing but matrix
-        // instructions (left alone the compiler reads two fragments at a time
-        // and the matrix cores idle through every LDS round trip)
-        v4i32 af[D][RB];
+        FetchRegs<D, GPW> &cur = ring[u % kRing];
+        FetchRegs<D, GPW> &ahead = ring[(u + 2) % kRing];
+        const int buf1 = buf == 2 ? 0 : buf + 1, buf2 = buf1 == 2 ? 0 : buf1 + 1;
+        // in flight: chunks c+2 .. c+kRing-1.  Release chunk c+2 and put its row
+        // block into the buffer that held chunk c-1, whose readers passed the
+        // barrier that closed chunk c-1.
+        wait_loads<(kRing - 3) * L, D, GPW>(ahead);
+        stage(ahead, buf2);
 #pragma unroll
-        for (int j = 0; j < D; ++j)
-#pragma unroll
-          for (int rb = 0; rb < RB; ++rb)
-            af[j][rb] = frag_s[(((size_t)buf * D + j) * RB + rb) * kWave + lane];
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int j = 0; j < D; ++j)
+        for (int j = 0; j < D; ++j) {
+          const int p = (u * D + j) & 1; // slot of this digit step's fragments
+          if (j + 1 < D)
+            read_frags(af[p ^ 1], buf, j + 1);
+          else
+            read_frags(af[p ^ 1], buf1, 0);
+          __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
           for (int rb = 0; rb < RB; ++rb)
 #pragma unroll
-            for (int g = 0; g < kGroupsPerWave; ++g)
-              acc[g][rb][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(cur.w[g], af[j][rb],
+            for (int g = 0; g < GPW; ++g)
+              acc[g][rb][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(cur.w[g], af[p][rb],
                                                                     acc[g][rb][j], 0, 0, 0);
+          __builtin_amdgcn_sched_barrier(0);
+        }
         // the matrix cores have read the registers of chunk c when the next
         // instruction issues: fetch the chunk kRing further on into them
         fetch(c + kRing, cur);
         __syncthreads();
+        buf = buf1;
       }
     }
   }
@@ -440,40 +515,75 @@ __global__ void __launch_bounds__(kSlices *kWave) gemm_w8_i8_wide_kernel(GemmI8A
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 #pragma unroll
   for (int u = 0; u < kRing; ++u)
-    wait_loads<0, D>(ring[u]);
+    wait_loads<0, D, GPW>(ring[u]);
 
+  // ---- epilogue ---------------------------------------------------------
+  // A lane's accumulator registers are 4 channels of one row: stored as they are,
+  // a store instruction would write 64-byte pieces of 16 rows.  Each wavefront
+  // turns its 16 x (16 GPW) tile around in its own part of LDS (free now: every
+  // wavefront is past the last barrier of the loop) and writes whole row
+  // segments, 64 GPW bytes each.
+  constexpr int kPad = GPW * 16 + 4; // floats per tile row in LDS
+  float *tile = reinterpret_cast<float *>(frag_s) + wave * (16 * kPad);
+  float s[GPW][4], b[GPW][4];
 #pragma unroll
-  for (int g = 0; g < kGroupsPerWave; ++g) {
-    if (g0 + g >= a.groups)
-      continue;
+  for (int g = 0; g < GPW; ++g) {
     const int n = (g0 + g) * kTileN + (lane >> 4) * 4;
-    float s[4], b[4];
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
-      s[r] = n + r < a.N ? a.scale[n + r] : 0.f;
-      b[r] = (a.bias && n + r < a.N) ? a.bias[n + r] : 0.f;
+      s[g][r] = n + r < a.N ? a.scale[n + r] : 0.f;
+      b[g][r] = (a.bias && n + r < a.N) ? a.bias[n + r] : 0.f;
     }
-    const bool vec = n + 3 < a.N && (a.ldc & 3) == 0 &&
-                     (reinterpret_cast<uintptr_t>(a.C) & 15) == 0;
+  }
+  const int n0 = g0 * kTileN;
+  const bool vec = (a.ldc & 3) == 0 && (reinterpret_cast<uintptr_t>(a.C) & 15) == 0;
 #pragma unroll
-    for (int rb = 0; rb < RB; ++rb) {
-      const int m = m0 + rb * 16 + (lane & 15);
-      if (m >= a.M)
+  for (int rb = 0; rb < RB; ++rb) {
+    const int mr = m0 + rb * 16 + (lane & 15);
+    const float step = mr < a.M ? a.steps[mr] : 0.f;
+#pragma unroll
+    for (int g = 0; g < GPW; ++g) {
+      float4 o;
+      o.x = b[g][0] + (combine<D>(acc[g][rb], 0) * step) * s[g][0];
+      o.y = b[g][1] + (combine<D>(acc[g][rb], 1) * step) * s[g][1];
+      o.z = b[g][2] + (combine<D>(acc[g][rb], 2) * step) * s[g][2];
+      o.w = b[g][3] + (combine<D>(acc[g][rb], 3) * step) * s[g][3];
+      *reinterpret_cast<float4 *>(tile + (lane & 15) * kPad + g * 16 + (lane >> 4) * 4) = o;
+    }
+#pragma unroll
+    for (int i = 0; i < GPW; ++i) { // 16 rows x 4 GPW float4 = 64 GPW lanes' worth
+      const int idx = lane + 64 * i;
+      const int row = idx / (GPW * 4), c4 = idx % (GPW * 4);
+      const float4 o = *reinterpret_cast<const float4 *>(tile + row * kPad + c4 * 4);
+      const int m = m0 + rb * 16 + row, n = n0 + c4 * 4;
+      if (m >= a.M || n >= a.N)
         continue;
-      float v[4];
+      float *c = a.C + (int64_t)m * a.ldc + n;
+      if (vec && n + 3 < a.N) {
+        float4 q = o;
+        if (a.accumulate) {
+          const float4 p = *reinterpret_cast<const float4 *>(c);
+          q = make_float4(p.x + q.x, p.y + q.y, p.z + q.z, p.w + q.w);
+        }
+        *reinterpret_cast<float4 *>(c) = q;
+      } else {
+        const float v[4] = {o.x, o.y, o.z, o.w};
 #pragma unroll
-      for (int r = 0; r < 4; ++r)
-        v[r] = combine<D>(acc[g][rb], r);
-      store_row(a, m, n, a.steps[m], v, s, b, vec);
+        for (int r = 0; r < 4; ++r)
+          if (n + r < a.N)
+            c[r] = a.accumulate ? c[r] + v[r] : v[r];
+      }
     }
   }
 }
 
-template <int D, int RB>
+template <int D, int RB, int GPW>
 int launch_wide(const GemmI8Args &a, unsigned blocks, hipStream_t stream) {
-  constexpr size_t lds = sizeof(v4i32) * 2 * D * RB * kWave;
-  hipLaunchKernelGGL((gemm_w8_i8_wide_kernel<D, RB>), dim3(blocks), dim3(kSlices * kWave),
-                     lds, stream, a);
+  // three fragment buffers in the loop, four output tiles in the epilogue
+  constexpr size_t lds = std::max(sizeof(v4i32) * 3 * D * RB * kWave,
+                                  sizeof(float) * kSlices * 16 * (GPW * 16 + 4));
+  hipLaunchKernelGGL((gemm_w8_i8_wide_kernel<D, RB, GPW>), dim3(blocks),
+                     dim3(kSlices * kWave), lds, stream, a);
   BH_CHECK_HIP(hipGetLastError());
   return BUDDY_HIP_OK;
 }
@@ -494,13 +604,19 @@ template <int D> int launch_split(const GemmI8Args &a, unsigned blocks, hipStrea
 
 } // namespace
 
+namespace {
+size_t row_cache_bytes(int cols_padded) {
+  return cols_padded <= kRowCache ? sizeof(float) * (size_t)cols_padded : 0;
+}
+} // namespace
+
 int launch_activations_to_digits(const float *A, int64_t lda, int64_t M, int64_t K,
                                  int digits, void *staged, hipStream_t stream) {
   BH_REQUIRE(A && staged && M > 0 && K > 0 && digits >= 2 && digits <= 3 && lda >= K,
              "activations_to_digits: bad argument");
   const GemmStagingLayout l = gemm_staging_layout(M, K);
   hipLaunchKernelGGL(activations_to_digits_kernel, dim3((unsigned)l.rows_padded), dim3(256),
-                     0, stream, A, lda, (int)M, (int)K, digits, l.rows_padded,
+                     row_cache_bytes(l.cols_padded), stream, A, lda, (int)M, (int)K, digits, l.rows_padded,
                      l.cols_padded, static_cast<int8_t *>(staged));
   BH_CHECK_HIP(hipGetLastError());
   return BUDDY_HIP_OK;
@@ -511,7 +627,8 @@ int launch_rmsnorm_to_digits(const float *x, const float *w, int rows, int n, fl
   BH_REQUIRE(x && w && staged && rows > 0 && n > 0 && digits >= 2 && digits <= 3,
              "rmsnorm_to_digits: bad argument");
   const GemmStagingLayout l = gemm_staging_layout(rows, n);
-  hipLaunchKernelGGL(rmsnorm_to_digits_kernel, dim3(rows), dim3(256), 0, stream, x, w, n,
+  hipLaunchKernelGGL(rmsnorm_to_digits_kernel, dim3(rows), dim3(256),
+                     row_cache_bytes(l.cols_padded), stream, x, w, n,
                      1.0f / (float)n, eps, digits, l.rows_padded, l.cols_padded,
                      static_cast<int8_t *>(staged));
   BH_CHECK_HIP(hipGetLastError());
@@ -523,7 +640,8 @@ int launch_silu_mul_to_digits(const float *g, const float *u, int rows, int n, i
   BH_REQUIRE(g && u && staged && rows > 0 && n > 0 && digits >= 2 && digits <= 3,
              "silu_mul_to_digits: bad argument");
   const GemmStagingLayout l = gemm_staging_layout(rows, n);
-  hipLaunchKernelGGL(silu_mul_to_digits_kernel, dim3(rows), dim3(256), 0, stream, g, u, n,
+  hipLaunchKernelGGL(silu_mul_to_digits_kernel, dim3(rows), dim3(256),
+                     row_cache_bytes(l.cols_padded), stream, g, u, n,
                      digits, l.rows_padded, l.cols_padded, static_cast<int8_t *>(staged));
   BH_CHECK_HIP(hipGetLastError());
   return BUDDY_HIP_OK;
@@ -548,24 +666,40 @@ int launch_gemm_w8_digits(const GemmW8Args &in, const void *planes, hipStream_t 
   a.groups = (int)ceil_div(in.N, kTileN);
   a.chunks = (int)ceil_div(in.K, kTileK);
   a.accumulate = in.accumulate ? 1 : 0;
-  // wide matrices: a workgroup per 64 (48) rows x 256 channels, no split of K
-  const int wide_cols = (int)ceil_div(a.groups, kGroupsPerWave * kSlices);
-  if ((int64_t)wide_cols * (a.Mp / 64) >= 200) {
-    // the chip runs 256 workgroups at a time (one wavefront per SIMD), so the
-    // time is rounds x rows; ties go to 64 rows
-    const int64_t wg4 = wide_cols * ceil_div(in.M, 64), wg3 = wide_cols * ceil_div(in.M, 48);
-    const bool three = ceil_div(wg3, 256) * 3 < ceil_div(wg4, 256) * 4;
-    a.ncols = wide_cols;
-    a.cols_padded = (int)round_up(wide_cols, 8);
-    const unsigned wb = (unsigned)(a.cols_padded * ceil_div(in.M, three ? 48 : 64));
-    if (three) {
-      if (in.digits == 2)
-        return launch_wide<2, 3>(a, wb, stream);
-      return launch_wide<3, 3>(a, wb, stream);
+  // Wide matrices: a workgroup per 16 RB rows x 64 GPW channels, no split of K.
+  // The chip runs 256 workgroups at a time (one wavefront per SIMD), so a launch
+  // costs rounds x (tile work + the fill and drain of a workgroup's pipeline, about
+  // three tile units); of the shapes that fill at least 160 CUs the cheapest
+  // wins, ties go to the larger tile (fewer reads of the operands).
+  int best_gpw = 0, best_rb = 0;
+  int64_t best_cost = 0;
+  for (int gpw : {5, 4})
+    for (int rb : {4, 3}) {
+      const int64_t tiles = ceil_div(a.groups, gpw * kSlices) * ceil_div(in.M, 16 * rb);
+      if (tiles < 160)
+        continue;
+      const int64_t cost = ceil_div(tiles, 256) * (gpw * rb + 3);
+      if (!best_gpw || cost < best_cost) {
+        best_gpw = gpw;
+        best_rb = rb;
+        best_cost = cost;
+      }
     }
-    if (in.digits == 2)
-      return launch_wide<2, 4>(a, wb, stream);
-    return launch_wide<3, 4>(a, wb, stream);
+  if (best_gpw) {
+    a.ncols = (int)ceil_div(a.groups, best_gpw * kSlices);
+    a.cols_padded = (int)round_up(a.ncols, 8);
+    const unsigned wb = (unsigned)(a.cols_padded * ceil_div(in.M, 16 * best_rb));
+    const int key = in.digits * 100 + best_rb * 10 + best_gpw;
+    switch (key) {
+    case 234: return launch_wide<2, 3, 4>(a, wb, stream);
+    case 235: return launch_wide<2, 3, 5>(a, wb, stream);
+    case 244: return launch_wide<2, 4, 4>(a, wb, stream);
+    case 245: return launch_wide<2, 4, 5>(a, wb, stream);
+    case 334: return launch_wide<3, 3, 4>(a, wb, stream);
+    case 335: return launch_wide<3, 3, 5>(a, wb, stream);
+    case 344: return launch_wide<3, 4, 4>(a, wb, stream);
+    default: return launch_wide<3, 4, 5>(a, wb, stream);
+    }
   }
   a.ncols = (int)ceil_div(a.groups, kGroupsPerWave);
   a.cols_padded = (int)round_up(a.ncols, 8);
