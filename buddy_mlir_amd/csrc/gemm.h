@@ -62,6 +62,9 @@ int launch_gemm_w8_digits(const GemmW8Args &a, const void *planes, hipStream_t s
 
 int launch_gemm_w8(const GemmW8Args &a, hipStream_t stream);
 
+// split-K workspace of the int8 matmul (dropped together with the staging)
+void release_gemm_i8_workspace(hipStream_t stream);
+
 // The matmul keeps a bf16 copy of its activations in a grow-only device buffer
 // per stream; a stream's owner drops it before destroying the stream.
 void release_gemm_staging(hipStream_t stream);

@@ -31,11 +31,12 @@
 #include "gemm.h"
 
 #include <algorithm>
+#include <map>
+#include <mutex>
 
 namespace bh {
 namespace {
 
-constexpr int kGroupsPerWave = 4; // channel groups of 16 per wavefront
 constexpr int kSlices = 4;        // wavefronts per workgroup
 
 typedef int v4i32 __attribute__((ext_vector_type(4)));
@@ -212,7 +213,12 @@ struct GemmI8Args {
   float *C;
   int64_t ldc;
   int M, N, Mp, Kp, groups, chunks;
-  int ncols, cols_padded; // column tiles; ids padded to the XCD count
+  int ncols;       // column tiles
+  int cols_padded; // ids per row tile: column tiles x slices, padded to the XCD count
+  // K split over `slices` workgroups per tile, chunks_per_slice chunks each
+  // (the last may hold fewer, never none); partial is only used when slices > 1
+  int slices, chunks_per_slice;
+  float *partial;     // [tile][slice][wavefront][row block][16][16 GPW]
   int accumulate;
 };
 
@@ -225,6 +231,8 @@ template <int D> __device__ __forceinline__ float combine(const v4i32 (&acc)[D],
     v = fmaf(v, 256.0f, (float)acc[j][r]);
   return v;
 }
+
+constexpr int kSplitGroups = 4; // channel groups of 16 per workgroup of the split kernel
 
 // lane holds channels n..n+3 of row m: C = step[m] * scale[n] * v (+ bias | + C)
 __device__ __forceinline__ void store_row(const GemmI8Args &a, int m, int n, float step,
@@ -253,16 +261,16 @@ __device__ __forceinline__ void store_row(const GemmI8Args &a, int m, int n, flo
 }
 
 template <int D> struct ChunkOperands {
-  v4i32 w[kGroupsPerWave];
+  v4i32 w[kSplitGroups];
   v4i32 a[D][4]; // [digit][row block]
 };
 
 template <int D>
-__device__ __forceinline__ void load_chunk(const v4i32 *const (&wp)[kGroupsPerWave],
+__device__ __forceinline__ void load_chunk(const v4i32 *const (&wp)[kSplitGroups],
                                            const int8_t *ap, size_t plane, size_t rb_stride,
                                            int c, ChunkOperands<D> &o) {
 #pragma unroll
-  for (int g = 0; g < kGroupsPerWave; ++g)
+  for (int g = 0; g < kSplitGroups; ++g)
     o.w[g] = wp[g][(size_t)c * 64];
 #pragma unroll
   for (int j = 0; j < D; ++j)
@@ -282,22 +290,22 @@ __global__ void __launch_bounds__(kSlices *kWave) gemm_w8_i8_kernel(GemmI8Args a
   const int col = blockIdx.x % a.cols_padded, rbk = blockIdx.x / a.cols_padded;
   if (col >= a.ncols)
     return; // padding id
-  const int m0 = rbk * 64, g0 = col * kGroupsPerWave;
+  const int m0 = rbk * 64, g0 = col * kSplitGroups;
   const int per = (a.chunks + kSlices - 1) / kSlices;
   const int c0 = min(wave * per, a.chunks), c1 = min(c0 + per, a.chunks);
 
-  v4i32 acc[kGroupsPerWave][4][D];
+  v4i32 acc[kSplitGroups][4][D];
 #pragma unroll
-  for (int g = 0; g < kGroupsPerWave; ++g)
+  for (int g = 0; g < kSplitGroups; ++g)
 #pragma unroll
     for (int rb = 0; rb < 4; ++rb)
 #pragma unroll
       for (int j = 0; j < D; ++j)
         acc[g][rb][j] = v4i32{0, 0, 0, 0};
 
-  const v4i32 *wp[kGroupsPerWave];
+  const v4i32 *wp[kSplitGroups];
 #pragma unroll
-  for (int g = 0; g < kGroupsPerWave; ++g) // groups past the end repeat the last one
+  for (int g = 0; g < kSplitGroups; ++g) // groups past the end repeat the last one
     wp[g] = reinterpret_cast<const v4i32 *>(a.W) +
             ((size_t)min(g0 + g, a.groups - 1) * a.chunks) * 64 + lane;
   const size_t plane = (size_t)a.Mp * a.Kp, rb_stride = (size_t)16 * a.Kp;
@@ -314,7 +322,7 @@ __global__ void __launch_bounds__(kSlices *kWave) gemm_w8_i8_kernel(GemmI8Args a
 #pragma unroll
       for (int rb = 0; rb < 4; ++rb)
 #pragma unroll
-        for (int g = 0; g < kGroupsPerWave; ++g)
+        for (int g = 0; g < kSplitGroups; ++g)
           acc[g][rb][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(cur.w[g], cur.a[j][rb],
                                                                 acc[g][rb][j], 0, 0, 0);
     if (c + 1 < c1)
@@ -323,7 +331,7 @@ __global__ void __launch_bounds__(kSlices *kWave) gemm_w8_i8_kernel(GemmI8Args a
 
   float *mine = red + (size_t)wave * 64 * kWave;
 #pragma unroll
-  for (int g = 0; g < kGroupsPerWave; ++g)
+  for (int g = 0; g < kSplitGroups; ++g)
 #pragma unroll
     for (int rb = 0; rb < 4; ++rb)
 #pragma unroll
@@ -380,6 +388,15 @@ __global__ void __launch_bounds__(kSlices *kWave) gemm_w8_i8_kernel(GemmI8Args a
 //  * the fragments of the next digit plane (or of the next chunk's first one)
 //    are read from LDS into the second half of a two-slot register buffer while
 //    the matrix instructions of the current plane run.
+//
+// Matrices too narrow to fill the chip with such tiles split K over several
+// workgroups per tile instead of shrinking the tile (a 64 x 64 tile reads its
+// operands four times as often from L2, and that, not the matrix cores, is what
+// bounds it).  Every slice writes its unscaled sums to a workspace and a second
+// small kernel adds the slices in slice order, applies the scales and writes C.
+// (Finishing a tile inside the kernel, by the workgroup that arrives last at a
+// counter, needs device-scope fences; on this chip they write back and
+// invalidate a whole L2 each time and slowed the running workgroups threefold.)
 template <int GPW> struct RingDepth { static constexpr int value = GPW > 4 ? 4 : 5; };
 
 __device__ __forceinline__ void issue_load(v4i32 &dst, const void *p) {
@@ -412,11 +429,16 @@ __global__ void __launch_bounds__(kSlices *kWave) gemm_w8_i8_wide_kernel(GemmI8A
   extern __shared__ __attribute__((aligned(16))) v4i32 frag_s[]; // [3][D][RB][64]
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int col = blockIdx.x % a.cols_padded, rbk = blockIdx.x / a.cols_padded;
-  if (col >= a.ncols)
+  // ids equal modulo 8 run on the same XCD: the row tiles of one (column tile,
+  // K slice) pair do, and share its weights in that XCD's L2
+  const int unit = blockIdx.x % a.cols_padded, rbk = blockIdx.x / a.cols_padded;
+  if (unit >= a.ncols * a.slices)
     return; // padding id
+  const int col = unit % a.ncols, slice = unit / a.ncols;
   const int m0 = rbk * RB * 16;
   const int g0 = (col * kSlices + wave) * GPW;
+  const int cb = slice * a.chunks_per_slice;
+  const int nch = min(a.chunks_per_slice, a.chunks - cb); // chunks of this slice, >= 1
 
   v4i32 acc[GPW][RB][D];
 #pragma unroll
@@ -431,18 +453,19 @@ __global__ void __launch_bounds__(kSlices *kWave) gemm_w8_i8_wide_kernel(GemmI8A
 #pragma unroll
   for (int g = 0; g < GPW; ++g) // groups past the end repeat the last one
     wp[g] = reinterpret_cast<const v4i32 *>(a.W) +
-            ((size_t)min(g0 + g, a.groups - 1) * a.chunks) * 64 + lane;
+            ((size_t)min(g0 + g, a.groups - 1) * a.chunks + cb) * 64 + lane;
   const size_t plane = (size_t)a.Mp * a.Kp;
   // this wavefront fetches row block `wave` of the activation tile (with three
   // row blocks the fourth wavefront repeats the third's loads and stages nothing)
   const int my_rb = min(wave, RB - 1);
-  const int8_t *ap = a.planes + (size_t)(m0 + my_rb * 16 + (lane & 15)) * a.Kp + (lane >> 4) * 16;
+  const int8_t *ap = a.planes + (size_t)(m0 + my_rb * 16 + (lane & 15)) * a.Kp +
+                     (size_t)cb * kTileK + (lane >> 4) * 16;
 
   FetchRegs<D, GPW> ring[kRing];
   // chunks past the end are fetched again from the last chunk (never used):
   // every fetch is exactly L loads, which is what keeps the counts below exact
   auto fetch = [&](int c, FetchRegs<D, GPW> &f) {
-    const int cc = min(c, a.chunks - 1);
+    const int cc = min(c, nch - 1);
 #pragma unroll
     for (int g = 0; g < GPW; ++g)
       issue_load(f.w[g], wp[g] + (size_t)cc * 64);
@@ -473,11 +496,11 @@ __global__ void __launch_bounds__(kSlices *kWave) gemm_w8_i8_wide_kernel(GemmI8A
   v4i32 af[2][RB];
   read_frags(af[0], 0, 0);
   int buf = 0; // LDS buffer of chunk c: c % 3
-  for (int c0 = 0; c0 < a.chunks; c0 += kPass) {
+  for (int c0 = 0; c0 < nch; c0 += kPass) {
 #pragma unroll
     for (int u = 0; u < kPass; ++u) {
       const int c = c0 + u;
-      if (c < a.chunks) {
+      if (c < nch) {
         FetchRegs<D, GPW> &cur = ring[u % kRing];
         FetchRegs<D, GPW> &ahead = ring[(u + 2) % kRing];
         const int buf1 = buf == 2 ? 0 : buf + 1, buf2 = buf1 == 2 ? 0 : buf1 + 1;
@@ -525,6 +548,32 @@ __global__ void __launch_bounds__(kSlices *kWave) gemm_w8_i8_wide_kernel(GemmI8A
   // segments, 64 GPW bytes each.
   constexpr int kPad = GPW * 16 + 4; // floats per tile row in LDS
   float *tile = reinterpret_cast<float *>(frag_s) + wave * (16 * kPad);
+  const int n0 = g0 * kTileN;
+  const bool vec = (a.ldc & 3) == 0 && (reinterpret_cast<uintptr_t>(a.C) & 15) == 0;
+  if (a.slices > 1) {
+    // unscaled sums of this slice; reduce_slices_kernel finishes the tile
+    constexpr int kSub = 16 * GPW * 16; // floats of one wavefront's row block
+    const int tile_id = rbk * a.ncols + col;
+    float *mine = a.partial +
+                  ((((size_t)tile_id * a.slices + slice) * kSlices + wave) * RB) * kSub;
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb) {
+#pragma unroll
+      for (int g = 0; g < GPW; ++g) {
+        const float4 o = make_float4(combine<D>(acc[g][rb], 0), combine<D>(acc[g][rb], 1),
+                                     combine<D>(acc[g][rb], 2), combine<D>(acc[g][rb], 3));
+        *reinterpret_cast<float4 *>(tile + (lane & 15) * kPad + g * 16 + (lane >> 4) * 4) = o;
+      }
+#pragma unroll
+      for (int i = 0; i < GPW; ++i) {
+        const int idx = lane + 64 * i;
+        const int row = idx / (GPW * 4), c4 = idx % (GPW * 4);
+        *reinterpret_cast<float4 *>(mine + (size_t)rb * kSub + idx * 4) =
+            *reinterpret_cast<const float4 *>(tile + row * kPad + c4 * 4);
+      }
+    }
+    return;
+  }
   float s[GPW][4], b[GPW][4];
 #pragma unroll
   for (int g = 0; g < GPW; ++g) {
@@ -535,8 +584,6 @@ __global__ void __launch_bounds__(kSlices *kWave) gemm_w8_i8_wide_kernel(GemmI8A
       b[g][r] = (a.bias && n + r < a.N) ? a.bias[n + r] : 0.f;
     }
   }
-  const int n0 = g0 * kTileN;
-  const bool vec = (a.ldc & 3) == 0 && (reinterpret_cast<uintptr_t>(a.C) & 15) == 0;
 #pragma unroll
   for (int rb = 0; rb < RB; ++rb) {
     const int mr = m0 + rb * 16 + (lane & 15);
@@ -577,6 +624,36 @@ __global__ void __launch_bounds__(kSlices *kWave) gemm_w8_i8_wide_kernel(GemmI8A
   }
 }
 
+// C (+)= step[m] * scale[n] * sum over slices of the unscaled sums, slice order.
+__global__ void __launch_bounds__(256)
+reduce_slices_kernel(GemmI8Args a, int rb_per_tile, int gpw) {
+  const int n4 = (a.N + 3) / 4;
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= (int64_t)a.M * n4)
+    return;
+  const int m = (int)(i / n4), n = (int)(i % n4) * 4;
+  const int span = 16 * gpw; // channels per wavefront
+  const int rbk = m / (16 * rb_per_tile), rb = (m / 16) % rb_per_tile, row = m % 16;
+  const int col = n / (kSlices * span), wave = (n / span) % kSlices, ch = n % span;
+  const int sub = 16 * span;
+  const size_t slice_stride = (size_t)kSlices * rb_per_tile * sub;
+  const float *p = a.partial + ((size_t)(rbk * a.ncols + col) * a.slices) * slice_stride +
+                   ((size_t)wave * rb_per_tile + rb) * sub + row * span + ch;
+  float v[4] = {0.f, 0.f, 0.f, 0.f};
+  for (int sl = 0; sl < a.slices; ++sl) {
+    const float4 q = *reinterpret_cast<const float4 *>(p + sl * slice_stride);
+    v[0] += q.x; v[1] += q.y; v[2] += q.z; v[3] += q.w;
+  }
+  const float step = a.steps[m];
+  float *c = a.C + (int64_t)m * a.ldc + n;
+#pragma unroll
+  for (int r = 0; r < 4; ++r)
+    if (n + r < a.N) {
+      const float o = (a.bias ? a.bias[n + r] : 0.f) + (v[r] * step) * a.scale[n + r];
+      c[r] = a.accumulate ? c[r] + o : o;
+    }
+}
+
 template <int D, int RB, int GPW>
 int launch_wide(const GemmI8Args &a, unsigned blocks, hipStream_t stream) {
   // three fragment buffers in the loop, four output tiles in the epilogue
@@ -584,20 +661,6 @@ int launch_wide(const GemmI8Args &a, unsigned blocks, hipStream_t stream) {
                                   sizeof(float) * kSlices * 16 * (GPW * 16 + 4));
   hipLaunchKernelGGL((gemm_w8_i8_wide_kernel<D, RB, GPW>), dim3(blocks),
                      dim3(kSlices * kWave), lds, stream, a);
-  BH_CHECK_HIP(hipGetLastError());
-  return BUDDY_HIP_OK;
-}
-
-template <int D> int launch_split(const GemmI8Args &a, unsigned blocks, hipStream_t stream) {
-  constexpr size_t lds = sizeof(float) * kSlices * 64 * kWave;
-  auto kernel = gemm_w8_i8_kernel<D>;
-  static bool attr_set = false;
-  if (!attr_set) {
-    BH_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
-                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-    attr_set = true;
-  }
-  hipLaunchKernelGGL(kernel, dim3(blocks), dim3(kSlices * kWave), lds, stream, a);
   BH_CHECK_HIP(hipGetLastError());
   return BUDDY_HIP_OK;
 }
@@ -647,6 +710,72 @@ int launch_silu_mul_to_digits(const float *g, const float *u, int rows, int n, i
   return BUDDY_HIP_OK;
 }
 
+namespace {
+
+// Split-K workspace: one grow-only device buffer per stream (calls on one stream
+// are ordered; calls on different streams must not share it).
+struct Workspace {
+  char *ptr = nullptr;
+  size_t bytes = 0;
+};
+std::mutex g_workspace_mutex;
+std::map<hipStream_t, Workspace> g_workspace;
+
+int workspace_for(hipStream_t stream, size_t bytes, char **out) {
+  std::lock_guard<std::mutex> lock(g_workspace_mutex);
+  Workspace &w = g_workspace[stream];
+  if (w.bytes < bytes) {
+    if (w.ptr) {
+      BH_CHECK_HIP(hipStreamSynchronize(stream)); // an earlier matmul may still use it
+      BH_CHECK_HIP(hipFree(w.ptr));
+      w.ptr = nullptr;
+      w.bytes = 0;
+    }
+    BH_CHECK_HIP(hipMalloc(reinterpret_cast<void **>(&w.ptr), bytes));
+    w.bytes = bytes;
+  }
+  *out = w.ptr;
+  return BUDDY_HIP_OK;
+}
+
+template <int D> int launch_split(const GemmI8Args &a, unsigned blocks, hipStream_t stream) {
+  constexpr size_t lds = sizeof(float) * kSlices * 64 * kWave;
+  auto kernel = gemm_w8_i8_kernel<D>;
+  static bool attr_set = false;
+  if (!attr_set) {
+    BH_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    attr_set = true;
+  }
+  hipLaunchKernelGGL(kernel, dim3(blocks), dim3(kSlices * kWave), lds, stream, a);
+  BH_CHECK_HIP(hipGetLastError());
+  return BUDDY_HIP_OK;
+}
+
+template <int D> int launch_shape(int rb, int gpw, const GemmI8Args &a, unsigned blocks,
+                                  hipStream_t stream) {
+  switch (rb * 10 + gpw) {
+  case 34: return launch_wide<D, 3, 4>(a, blocks, stream);
+  case 35: return launch_wide<D, 3, 5>(a, blocks, stream);
+  case 44: return launch_wide<D, 4, 4>(a, blocks, stream);
+  default: return launch_wide<D, 4, 5>(a, blocks, stream);
+  }
+}
+
+} // namespace
+
+void release_gemm_i8_workspace(hipStream_t stream) {
+  std::lock_guard<std::mutex> lock(g_workspace_mutex);
+  auto it = g_workspace.find(stream);
+  if (it == g_workspace.end())
+    return;
+  if (it->second.ptr) {
+    (void)hipStreamSynchronize(stream);
+    (void)hipFree(it->second.ptr);
+  }
+  g_workspace.erase(it);
+}
+
 // `planes` holds the digit planes and row steps of the activations (written by
 // one of the producers above for exactly this M, K and digit count).
 int launch_gemm_w8_digits(const GemmW8Args &in, const void *planes, hipStream_t stream) {
@@ -666,47 +795,77 @@ int launch_gemm_w8_digits(const GemmW8Args &in, const void *planes, hipStream_t 
   a.groups = (int)ceil_div(in.N, kTileN);
   a.chunks = (int)ceil_div(in.K, kTileK);
   a.accumulate = in.accumulate ? 1 : 0;
-  // Wide matrices: a workgroup per 16 RB rows x 64 GPW channels, no split of K.
-  // The chip runs 256 workgroups at a time (one wavefront per SIMD), so a launch
-  // costs rounds x (tile work + the fill and drain of a workgroup's pipeline, about
-  // three tile units); of the shapes that fill at least 160 CUs the cheapest
-  // wins, ties go to the larger tile (fewer reads of the operands).
-  int best_gpw = 0, best_rb = 0;
-  int64_t best_cost = 0;
+  a.partial = nullptr;
+  a.slices = 1;
+  // Three schemes, chosen by a model of their cost in microseconds (fitted to
+  // measurements at the Qwen2-1.5B shapes and M = 512):
+  //  * wide tiles, whole K per workgroup: the chip runs 256 workgroups at a time
+  //    (one wavefront per SIMD); a workgroup costs its matrix instructions
+  //    (12.5 ns each per SIMD, sustained) plus about 7 us of pipeline fill, drain
+  //    and stores; a launch costs rounds x that;
+  //  * wide tiles with K split over s workgroups: 2 us more per workgroup for the
+  //    partial sums, and the second kernel (3 us + its bytes at 3 TB/s);
+  //  * 64 x 64 tiles, K split over the wavefronts: bound by L2 -> CU traffic,
+  //    16 KiB per workgroup and chunk at about 6 TB/s.
+  int best_gpw = 0, best_rb = 0, best_s = 0;
+  double best_cost = 0;
   for (int gpw : {5, 4})
     for (int rb : {4, 3}) {
-      const int64_t tiles = ceil_div(a.groups, gpw * kSlices) * ceil_div(in.M, 16 * rb);
-      if (tiles < 160)
-        continue;
-      const int64_t cost = ceil_div(tiles, 256) * (gpw * rb + 3);
-      if (!best_gpw || cost < best_cost) {
-        best_gpw = gpw;
-        best_rb = rb;
-        best_cost = cost;
+      const int64_t ncols = ceil_div(a.groups, gpw * kSlices), rows = ceil_div(in.M, 16 * rb);
+      for (int s = 1; s <= 16; ++s) {
+        // workgroups of the busiest XCD (32 CUs each): the (column tile, slice)
+        // pairs are dealt round robin, each with all its row tiles
+        const int64_t per_xcd = ceil_div(ncols * s, 8) * rows;
+        if (s > 1 && per_xcd > 32)
+          break;
+        const int64_t cps = ceil_div(a.chunks, s);
+        if (ceil_div(a.chunks, cps) != s)
+          continue; // the last slice would be empty
+        const double wg = 0.0125 * (double)(cps * gpw * rb * in.digits) + 7.0 + (s > 1 ? 2.0 : 0.0);
+        double cost = (double)ceil_div(per_xcd, 32) * wg;
+        if (s > 1)
+          cost += 3.0 + 4.0 * (double)(ncols * rows * s) * (kSlices * rb * 16 * gpw * 16) / 3e6;
+        if (!best_gpw || cost < best_cost - 1e-9) {
+          best_gpw = gpw;
+          best_rb = rb;
+          best_s = s;
+          best_cost = cost;
+        }
       }
     }
-  if (best_gpw) {
-    a.ncols = (int)ceil_div(a.groups, best_gpw * kSlices);
+  const int64_t split_wgs = ceil_div(a.groups, kSplitGroups) * (a.Mp / 64);
+  const double split_cost = 1.0 + (double)split_wgs * a.chunks * 16384.0 / 6e6;
+  if (split_cost < best_cost) {
+    a.ncols = (int)ceil_div(a.groups, kSplitGroups);
     a.cols_padded = (int)round_up(a.ncols, 8);
-    const unsigned wb = (unsigned)(a.cols_padded * ceil_div(in.M, 16 * best_rb));
-    const int key = in.digits * 100 + best_rb * 10 + best_gpw;
-    switch (key) {
-    case 234: return launch_wide<2, 3, 4>(a, wb, stream);
-    case 235: return launch_wide<2, 3, 5>(a, wb, stream);
-    case 244: return launch_wide<2, 4, 4>(a, wb, stream);
-    case 245: return launch_wide<2, 4, 5>(a, wb, stream);
-    case 334: return launch_wide<3, 3, 4>(a, wb, stream);
-    case 335: return launch_wide<3, 3, 5>(a, wb, stream);
-    case 344: return launch_wide<3, 4, 4>(a, wb, stream);
-    default: return launch_wide<3, 4, 5>(a, wb, stream);
-    }
+    const unsigned blocks = (unsigned)(a.cols_padded * (a.Mp / 64));
+    if (in.digits == 2)
+      return launch_split<2>(a, blocks, stream);
+    return launch_split<3>(a, blocks, stream);
   }
-  a.ncols = (int)ceil_div(a.groups, kGroupsPerWave);
-  a.cols_padded = (int)round_up(a.ncols, 8);
-  const unsigned blocks = (unsigned)(a.cols_padded * (a.Mp / 64));
-  if (in.digits == 2)
-    return launch_split<2>(a, blocks, stream);
-  return launch_split<3>(a, blocks, stream);
+  a.ncols = (int)ceil_div(a.groups, best_gpw * kSlices);
+  a.cols_padded = (int)round_up((int64_t)a.ncols * best_s, 8);
+  const int row_tiles = (int)ceil_div(in.M, 16 * best_rb);
+  a.slices = best_s;
+  a.chunks_per_slice = (int)ceil_div(a.chunks, best_s);
+  if (best_s > 1) {
+    const size_t tile_floats = (size_t)kSlices * best_rb * 16 * best_gpw * 16;
+    const size_t bytes = sizeof(float) * tile_floats * best_s * (size_t)a.ncols * row_tiles;
+    char *ws = nullptr;
+    if (int rc = workspace_for(stream, bytes, &ws))
+      return rc;
+    a.partial = reinterpret_cast<float *>(ws);
+  }
+  const unsigned blocks = (unsigned)(a.cols_padded * row_tiles);
+  int rc = in.digits == 2 ? launch_shape<2>(best_rb, best_gpw, a, blocks, stream)
+                          : launch_shape<3>(best_rb, best_gpw, a, blocks, stream);
+  if (rc || best_s == 1)
+    return rc;
+  const int64_t threads = (int64_t)a.M * ((a.N + 3) / 4);
+  hipLaunchKernelGGL(reduce_slices_kernel, dim3((unsigned)ceil_div(threads, 256)), dim3(256), 0,
+                     stream, a, best_rb, best_gpw);
+  BH_CHECK_HIP(hipGetLastError());
+  return BUDDY_HIP_OK;
 }
 
 } // namespace bh

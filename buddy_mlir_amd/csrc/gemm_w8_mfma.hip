@@ -698,6 +698,7 @@ int launch_gemm_w8(const GemmW8Args &in, hipStream_t stream) {
 }
 
 void release_gemm_staging(hipStream_t stream) {
+  release_gemm_i8_workspace(stream);
   std::lock_guard<std::mutex> lock(g_staging_mutex);
   auto it = g_staging.find(stream);
   if (it == g_staging.end())
