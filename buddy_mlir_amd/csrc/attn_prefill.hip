@@ -14,6 +14,8 @@
 // Arithmetic is f32 throughout, on the f32 matrix cores.
 #include "attn.h"
 
+#include <type_traits>
+
 namespace bh {
 namespace {
 
@@ -39,31 +41,37 @@ struct PrefillArgs {
 // blocks round robin, each with its own running (max, sum, output), and merge
 // at the end.  All products run on the f32 matrix cores (16x16x4), operands
 // straight from global memory in fragment layout:
-//   S^T[key, query] = K . Q^T   (contraction over d; a lane supplies d =
-//                                32*(lane/16) + j in step j, for K and Q alike)
+//   S^T[key, query] = K . Q^T   (contraction over d; in step 4J + e a lane
+//                                supplies d = 16 J + 4 (lane/16) + e, for K and
+//                                Q alike: the four lane groups of a load read 64
+//                                contiguous bytes of a row, so a K load touches
+//                                16 pieces of memory and not 64)
 //   O^T[d, query]  += V^T . P^T (contraction over the key; the S^T accumulator
 //                                registers ARE the P^T operand of step r: a
 //                                lane holds keys 4*(lane/16) + r of query lane%16)
 // so the scores never leave the registers between the two products.
-__global__ void __launch_bounds__(kAttnWaves *kWave) attn_prefill_kernel(PrefillArgs a) {
+__global__ void __launch_bounds__(kAttnWaves *kWave) __attribute__((amdgpu_waves_per_eu(2, 2)))
+attn_prefill_kernel(PrefillArgs a) {
   __shared__ float o_s[kAttnWaves][32][kWave];
   __shared__ float m_s[kAttnWaves][kQB], l_s[kAttnWaves][kQB];
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int h = blockIdx.y, kvh = h / a.group;
-  const int q0 = blockIdx.x * kQB;
+  // workgroups start in id order: the last query blocks, which see the most
+  // keys, come first for every head, the short ones fill the gaps at the end
+  const int h = blockIdx.x, kvh = h / a.group;
+  const int q0 = ((int)gridDim.y - 1 - (int)blockIdx.y) * kQB;
   const int nq = min(kQB, a.q_len - q0);
   const int qi = lane & 15, lg = lane >> 4; // query of this lane; lane group
   const int qrow = q0 + min(qi, nq - 1);    // rows past the end repeat the last
 
-  // Q^T fragment: d = 32*lg + j
+  // Q^T fragment: qf[4J + e] is d = 16 J + 4 lg + e
   float qf[32];
   {
-    const float *src = a.q + (int64_t)qrow * a.q_stride + (int64_t)h * a.q_hstride + lg * 32;
+    const float *src = a.q + (int64_t)qrow * a.q_stride + (int64_t)h * a.q_hstride + lg * 4;
 #pragma unroll
     for (int j = 0; j < 32; j += 4) {
-      const float4 v = *reinterpret_cast<const float4 *>(src + j);
+      const float4 v = *reinterpret_cast<const float4 *>(src + 4 * j);
       qf[j] = v.x;
       qf[j + 1] = v.y;
       qf[j + 2] = v.z;
@@ -83,36 +91,56 @@ __global__ void __launch_bounds__(kAttnWaves *kWave) attn_prefill_kernel(Prefill
   for (int i = 0; i < 8; ++i)
     acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  float4 kreg[8], vreg[8], knext[8], vnext[8];
-  auto load_block = [&](int b, float4 (&kr)[8], float4 (&vr)[8]) {
-    const int p0 = b * kKB;
-    // K fragment: key p0 + lane%16, d = 32*lg + 0..31
-    const float *ks = kbase + (int64_t)min(p0 + qi, a.k_len - 1) * kD + lg * 32;
+  // K and V of a key block: 16 loads, issued by hand one block ahead of the
+  // block being multiplied (the compiler sinks ordinary loads down to their
+  // first use, which leaves the matrix cores waiting out every L2 round trip).
+  // A fetch is always exactly 16 loads -- blocks past the end fetch the last
+  // block again -- so that vmcnt(16) means "everything but the newest fetch has
+  // arrived".  The registers of a fetch are only read after such a wait names
+  // them; the build refuses scratch use in this file.
+  struct Frag {
+    f32x4 k[8], v[8];
+  };
+  auto issue = [](f32x4 &dst, const float *p) {
+    asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(dst) : "v"(p) : "memory");
+  };
+  auto fetch = [&](int b, Frag &f) {
+    const int p0 = min(b, nblocks - 1) * kKB;
+    // K fragment: key p0 + lane%16, k[J] is d = 16 J + 4 lg + 0..3
+    const float *ks = kbase + (int64_t)min(p0 + qi, a.k_len - 1) * kD + lg * 4;
 #pragma unroll
     for (int j = 0; j < 8; ++j)
-      kr[j] = *reinterpret_cast<const float4 *>(ks + 4 * j);
+      issue(f.k[j], ks + 16 * j);
     // V^T fragments: key p0 + 4*lg + r, d = 64*half + 4*(lane%16) + 0..3
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
       const float *vs = vbase + (int64_t)min(p0 + 4 * lg + r, a.k_len - 1) * kD + 4 * qi;
-      vr[2 * r] = *reinterpret_cast<const float4 *>(vs);
-      vr[2 * r + 1] = *reinterpret_cast<const float4 *>(vs + 64);
+      issue(f.v[2 * r], vs);
+      issue(f.v[2 * r + 1], vs + 64);
     }
   };
-  if (wave < nblocks)
-    load_block(wave, kreg, vreg);
-  for (int b = wave; b < nblocks; b += kAttnWaves) {
-    if (b + kAttnWaves < nblocks)
-      load_block(b + kAttnWaves, knext, vnext);
-    // ---- S^T block: keys x queries ------------------------------------------
-    f32x4 st = {0.f, 0.f, 0.f, 0.f};
+  auto arrived = [](Frag &f, auto n_in_flight) { // at most N loads still in flight
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(decltype(n_in_flight)::value) : "memory");
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
-      st = __builtin_amdgcn_mfma_f32_16x16x4f32(kreg[j].x, qf[4 * j], st, 0, 0, 0);
-      st = __builtin_amdgcn_mfma_f32_16x16x4f32(kreg[j].y, qf[4 * j + 1], st, 0, 0, 0);
-      st = __builtin_amdgcn_mfma_f32_16x16x4f32(kreg[j].z, qf[4 * j + 2], st, 0, 0, 0);
-      st = __builtin_amdgcn_mfma_f32_16x16x4f32(kreg[j].w, qf[4 * j + 3], st, 0, 0, 0);
+      asm volatile("" : "+v"(f.k[j])::"memory");
+      asm volatile("" : "+v"(f.v[j])::"memory");
     }
+  };
+  auto block = [&](const Frag &f, int b) {
+    // ---- S^T block: keys x queries ------------------------------------------
+    // four independent partial sums: a matrix instruction that adds to the
+    // result of the one before it cannot issue until that one has finished
+    f32x4 sp[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+      sp[e] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        sp[e] = __builtin_amdgcn_mfma_f32_16x16x4f32(f.k[j][e], qf[4 * j + e], sp[e], 0, 0, 0);
+    const f32x4 st = (sp[0] + sp[1]) + (sp[2] + sp[3]);
     // lane holds keys p0 + 4*lg + r of query q0 + qi
     const int p0 = b * kKB;
     float sc[4];
@@ -152,21 +180,29 @@ __global__ void __launch_bounds__(kAttnWaves *kWave) attn_prefill_kernel(Prefill
     for (int r = 0; r < 4; ++r) {
 #pragma unroll
       for (int half = 0; half < 2; ++half) {
-        const float4 vv = vreg[2 * r + half];
-        acc[0 + half] = __builtin_amdgcn_mfma_f32_16x16x4f32(vv.x, p[r], acc[0 + half], 0, 0, 0);
-        acc[2 + half] = __builtin_amdgcn_mfma_f32_16x16x4f32(vv.y, p[r], acc[2 + half], 0, 0, 0);
-        acc[4 + half] = __builtin_amdgcn_mfma_f32_16x16x4f32(vv.z, p[r], acc[4 + half], 0, 0, 0);
-        acc[6 + half] = __builtin_amdgcn_mfma_f32_16x16x4f32(vv.w, p[r], acc[6 + half], 0, 0, 0);
+        const f32x4 vv = f.v[2 * r + half];
+        acc[0 + half] = __builtin_amdgcn_mfma_f32_16x16x4f32(vv[0], p[r], acc[0 + half], 0, 0, 0);
+        acc[2 + half] = __builtin_amdgcn_mfma_f32_16x16x4f32(vv[1], p[r], acc[2 + half], 0, 0, 0);
+        acc[4 + half] = __builtin_amdgcn_mfma_f32_16x16x4f32(vv[2], p[r], acc[4 + half], 0, 0, 0);
+        acc[6 + half] = __builtin_amdgcn_mfma_f32_16x16x4f32(vv[3], p[r], acc[6 + half], 0, 0, 0);
       }
     }
-    if (b + kAttnWaves < nblocks) {
-#pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        kreg[j] = knext[j];
-        vreg[j] = vnext[j];
-      }
-    }
+  };
+  Frag fa, fb;
+  fetch(wave, fa);
+  for (int b = wave; b < nblocks; b += 2 * kAttnWaves) {
+    fetch(b + kAttnWaves, fb);
+    arrived(fa, std::integral_constant<int, 16>{});
+    block(fa, b);
+    fetch(b + 2 * kAttnWaves, fa);
+    arrived(fb, std::integral_constant<int, 16>{});
+    if (b + kAttnWaves < nblocks)
+      block(fb, b + kAttnWaves);
   }
+  // the last fetch (a repeated block) may still be in flight: its registers stay
+  // allocated until it has landed
+  arrived(fa, std::integral_constant<int, 0>{});
+  arrived(fb, std::integral_constant<int, 0>{});
   // this wavefront's row sums: the four lane groups hold different keys
   l_run += __shfl_xor(l_run, 16, 64);
   l_run += __shfl_xor(l_run, 32, 64);
@@ -279,7 +315,8 @@ int launch_attn_prefill(const AttnPrefillArgs &in, hipStream_t stream) {
   a.k_len = in.k_len;
   a.q_offset = in.k_len - in.q_len; // the last query sees every key
   a.scale = in.scale;
-  hipLaunchKernelGGL(attn_prefill_kernel, dim3((unsigned)ceil_div(in.q_len, kQB), in.heads),
+  BH_REQUIRE(ceil_div(in.q_len, kQB) <= 65535, "attn_prefill: q_len %d too long", in.q_len);
+  hipLaunchKernelGGL(attn_prefill_kernel, dim3(in.heads, (unsigned)ceil_div(in.q_len, kQB)),
                      dim3(kAttnWaves * kWave), 0, stream, a);
   BH_CHECK_HIP(hipGetLastError());
   return BUDDY_HIP_OK;
