@@ -3,7 +3,7 @@
 MI355X, next to the CPU oracle timed on the same host.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W]
-    python bench.py --workload gemv|mlp|prefill|llama8b|kvdiscard|w4a16   (the other configurations)
+    python bench.py --workload gemv|mlp|prefill|llama8b|kvdiscard|w4a16|model_abi   (the other configurations)
 
 A step is one greedy decode step (one token) at batch 1 with the KV cache
 already holding 1024 positions; weights, KV cache and activations are resident
@@ -300,7 +300,8 @@ def bench_prefill(bh, args):
         "detail": res, "gemm_flop": gemm_flop, "attention_flop": attn_flop,
         # algorithmic flops 2 M K N (each digit plane is not counted again)
         # over the time of the whole pass, against the dense int8 peak
-        "roofline": {"kernel": "gemm_w8_i8_wide_kernel<3,3> + gemm_w8_i8_kernel<3>",
+        "roofline": {"kernel": "gemm_w8_i8_wide_kernel<3, 4, 5> (gate, up), <3, 4, 4> (down), "
+                               "gemm_w8_i8_kernel<3> (q|k|v, o)",
                      "bound": "mfma", "achieved": res["i8_3digit"]["gemm_tflops"],
                      "peak": MFMA_I8_PEAK_TOPS, "unit": "TFLOP/s",
                      "frac": res["i8_3digit"]["mfma_frac"], "traffic": None},
@@ -449,13 +450,83 @@ def bench_llama8b(bh, args):
     }
 
 
+def bench_model_abi(bh, args):
+    """The reference's own decode entry point, `_mlir_ciface_forward_decode`
+    with its 88 memref arguments (two weight blobs, token, position, 56 KV
+    tensors), called token after token the way buddy-cli's runtime does: host
+    buffers in, malloc'd logits out, argmax on the host.  The library keeps
+    weights and KV caches resident on the device between calls."""
+    import numpy as np
+
+    import buddy_mlir_amd as bma
+    import test_gpu_model_abi as T
+    from buddy_mlir_amd.session import Shape
+
+    L = 1024
+    shape = Shape(max_len=L)
+    f32, i8, _ = T.make_blobs(bh, shape, seed=2)
+    mf = bma.MemRef(f32.ctypes.data, [f32.size])
+    mi = bma.MemRef(i8.ctypes.data, [i8.size], ctype=ctypes.c_int8)
+    kv = [np.random.default_rng(j).standard_normal((2, L, 128)).astype(np.float32)
+          for j in range(2 * shape.layers)]
+    kvm = [bma.MemRef(a.ctypes.data, [1, 2, L, 128]) for a in kv]
+    posbuf, tokbuf = np.zeros(1, np.int64), np.zeros((1, 1), np.int64)
+    dummies = [np.zeros(1, np.int64) for _ in range(shape.layers - 1)]
+    mpos = bma.MemRef(posbuf.ctypes.data, [1], ctype=ctypes.c_longlong)
+    mtok = bma.MemRef(tokbuf.ctypes.data, [1, 1], ctype=ctypes.c_longlong)
+    mdum = [bma.MemRef(d.ctypes.data, [1], ctype=ctypes.c_longlong) for d in dummies]
+    free = ctypes.CDLL(None).free
+    free.argtypes = [ctypes.c_void_p]
+
+    def step(pos, tok):
+        tokbuf[0, 0], posbuf[0] = tok, pos
+        for d in dummies:
+            d[0] = pos
+        res = T.DecodeResult()
+        a = [ctypes.byref(res), ctypes.byref(mf), ctypes.byref(mi), ctypes.byref(mtok),
+             ctypes.byref(mpos), ctypes.byref(kvm[0]), ctypes.byref(kvm[1])]
+        for i in range(shape.layers - 1):
+            a += [ctypes.byref(mdum[i]), ctypes.byref(kvm[2 + 2 * i]), ctypes.byref(kvm[3 + 2 * i])]
+        bh._mlir_ciface_forward_decode(*a)
+        if not res.logits.aligned:
+            raise RuntimeError(bh.buddy_hip_last_error())
+        lg = np.ctypeslib.as_array(res.logits.aligned, shape=(shape.vocab,))
+        nxt = int(lg.argmax())
+        free(ctypes.cast(res.logits.allocated, ctypes.c_void_p))
+        return nxt
+
+    tok = 5
+    for w in range(max(1, args.warmup)):  # the first call uploads and packs the blobs
+        tok = step(900 + w, tok)
+    n = max(1, min(args.steps, L - 901 - args.warmup))
+    t0 = time.perf_counter()
+    for s_ in range(n):
+        tok = step(900 + max(1, args.warmup) + s_, tok)
+    t = (time.perf_counter() - t0) / n
+    bh.buddy_hip_forward_reset()
+    return {
+        "metric": "decode_tokens_per_s", "value": 1.0 / t, "unit": "tokens/s",
+        "n_gpus": 1, "steps": n, "warmup": max(1, args.warmup), "ms_per_step": t * 1e3,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": "_mlir_ciface_forward_decode (the reference's 88-argument decode "
+                               "entry point), Qwen2-1.5B shape, context ~900, host buffers in and "
+                               "out, host argmax; PCIe-inclusive"},
+        "roofline": {"kernel": "whole call", "bound": "hbm",
+                     "achieved": decode_step_bytes(shape, 900) / t / 1e9, "peak": HBM_PEAK_GBPS,
+                     "unit": "GB/s", "frac": decode_step_bytes(shape, 900) / t / 1e9 / HBM_PEAK_GBPS,
+                     "traffic": None},
+    }
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=64)
     ap.add_argument("--warmup", type=int, default=8)
     ap.add_argument("--workload", default="decode",
-                    choices=["decode", "gemv", "mlp", "prefill", "llama8b", "kvdiscard", "w4a16"],
+                    choices=["decode", "gemv", "mlp", "prefill", "llama8b", "kvdiscard", "w4a16",
+                             "model_abi"],
                     help="decode (default): the full decode step the headline metric "
                          "is quoted on; the others measure the remaining configurations")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -480,7 +551,8 @@ def main():
     bh = bma.lib()
     if args.workload != "decode":
         fn = {"gemv": bench_gemv, "mlp": bench_mlp, "prefill": bench_prefill,
-              "llama8b": bench_llama8b, "kvdiscard": bench_kvdiscard, "w4a16": bench_w4a16}[args.workload]
+              "llama8b": bench_llama8b, "kvdiscard": bench_kvdiscard, "w4a16": bench_w4a16,
+              "model_abi": bench_model_abi}[args.workload]
         print(json.dumps(fn(bh, args)))
         return
     K, W = args.steps, args.warmup
