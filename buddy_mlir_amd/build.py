@@ -20,6 +20,8 @@ CSRC = PKG / "csrc"
 LIBDIR = PKG / "lib"
 OBJDIR = LIBDIR / "obj"
 LIB = LIBDIR / "libbuddy_hip.so"
+RUNNER_SRC = PKG / "runner" / "buddy_hip_run.cpp"
+RUNNER = LIBDIR / "buddy_hip_run"
 
 ARCH = "gfx950"
 # -packed-fp32-ops off: scalar float code must not be turned into v_pk_*_f32.
@@ -102,8 +104,15 @@ def build(force: bool = False, jobs: int = 8, verbose: bool = True) -> Path:
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError(f"link failed:\n{r.stdout}\n{r.stderr}")
+    # the command-line runner for the reference's w8a32 parameter files: plain
+    # C++ over the C interface, found next to the library at run time
+    cmd = [_hipcc(), "-O2", "-std=c++17", f"-I{ROOT / 'include'}", str(RUNNER_SRC),
+           f"-L{LIBDIR}", "-lbuddy_hip", "-Wl,-rpath,$ORIGIN", "-o", str(RUNNER)]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError(f"runner build failed:\n{r.stdout}\n{r.stderr}")
     if verbose:
-        print(f"built {LIB} from {len(srcs)} sources")
+        print(f"built {LIB} from {len(srcs)} sources, and {RUNNER.name}")
     return LIB
 
 
