@@ -242,6 +242,55 @@ def test_small_model_logits_kv_and_tokens(oracle, graph):
     sess.close()
 
 
+@pytest.mark.parametrize("pos", [4095, 4096, 8191])
+def test_decode_attention_long_context(bh, oracle, pos):
+    """Contexts far beyond the model's shipped 1024: more than 64 chunks per head."""
+    H, HKV, D, L = 4, 2, 128, 8192
+    g = torch.Generator(device="cuda").manual_seed(pos)
+    qkv = torch.randn((H + 2 * HKV) * D, generator=g, device="cuda")
+    kc = torch.randn((HKV, L, D), generator=g, device="cuda")
+    vc = torch.randn((HKV, L, D), generator=g, device="cuda")
+    inv = synthetic.inv_freq(D)
+    out = torch.empty(H * D, device="cuda")
+    pos_t = torch.tensor([pos], dtype=torch.int32, device="cuda")
+    nb = bh.buddy_hip_attn_decode_workspace_bytes(H, L)
+    ws = torch.empty(nb, dtype=torch.uint8, device="cuda")
+    kch, vch, qh = kc.cpu().numpy().copy(), vc.cpu().numpy().copy(), qkv.cpu().numpy()
+    scale = np.float32(0.0883883461)
+    torch.cuda.synchronize()
+    bma.check(bh.buddy_hip_gqa_decode_attention(
+        qkv.data_ptr(), inv.data_ptr(), pos_t.data_ptr(), kc.data_ptr(), vc.data_ptr(),
+        out.data_ptr(), H, HKV, D, L, float(scale), ws.data_ptr(), nb, None))
+    torch.cuda.synchronize()
+    c, s = oracle.rope_cos_sin(inv.cpu().numpy(), pos)
+    q = oracle.rope_apply(qh[:H * D].reshape(H, D), c, s)
+    kch[:, pos, :] = oracle.rope_apply(qh[H * D:(H + HKV) * D].reshape(HKV, D), c, s)
+    vch[:, pos, :] = qh[(H + HKV) * D:].reshape(HKV, D)
+    kch[:, pos + 1:, :] = 0
+    vch[:, pos + 1:, :] = 0
+    mask = np.where(np.arange(L) <= pos, 0.0, -np.inf).astype(np.float32)
+    want, _ = oracle.gqa_decode_attention(q, kch, vch, mask, scale, 4)
+    check_close(out.cpu().numpy().reshape(H, D), want)
+
+
+def test_small_model_decodes_at_long_context(oracle):
+    """A cache of 4352 positions (68 chunks of 64: the o_proj kernel folds them in
+    two passes) filled to 4300, then greedy steps against the oracle."""
+    shape = Shape(layers=2, hidden=256, heads=4, kv_heads=2, head_dim=128, inter=512,
+                  vocab=1024, max_len=4352, rms_eps=1e-6)
+    sess, host = synthetic.build_session(shape, context=4300, keep_host=True, ln_jitter=0.1)
+    om = oracle_model(oracle, shape, host)
+    kv = [a.copy() for a in host["kv"]]
+    tok = 9
+    for step in range(6):
+        nxt, logits = sess.decode(tok, 4300 + step)
+        otok, ologits = om.decode_step(tok, 4300 + step, kv)
+        check_close(logits, ologits)
+        assert nxt == otok
+        tok = otok
+    sess.close()
+
+
 def test_small_model_greedy_feedback_matches_stepwise(oracle):
     sess, host = synthetic.build_session(SMALL, context=16, keep_host=True, ln_jitter=0.1)
     toks = sess.decode_greedy(5, 16, 24)
