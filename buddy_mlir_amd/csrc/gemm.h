@@ -51,8 +51,8 @@ int launch_rmsnorm_to_staging(const float *x, const float *w, int rows, int n, f
 int launch_silu_mul_to_staging(const float *g, const float *u, int rows, int n, int terms,
                                unsigned short *staged, hipStream_t stream);
 // the same producers for digit planes, and the plain conversion of A
-int launch_rmsnorm_to_digits(const float *x, const float *w, int rows, int n, float eps,
-                             int digits, void *staged, hipStream_t stream);
+int launch_rmsnorm_to_digits(const float *x, int64_t ldx, const float *w, int rows, int n,
+                             float eps, int digits, void *staged, hipStream_t stream);
 int launch_silu_mul_to_digits(const float *g, const float *u, int rows, int n, int digits,
                               void *staged, hipStream_t stream);
 int launch_activations_to_digits(const float *A, int64_t lda, int64_t M, int64_t K,

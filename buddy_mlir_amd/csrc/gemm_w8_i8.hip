@@ -173,13 +173,13 @@ activations_to_digits_kernel(const float *__restrict__ A, int64_t lda, int M, in
 }
 
 __global__ void __launch_bounds__(256)
-rmsnorm_to_digits_kernel(const float *__restrict__ x, const float *__restrict__ w, int n,
-                         float inv_n, float eps, int D, int Mp, int Kp,
-                         int8_t *__restrict__ planes) {
+rmsnorm_to_digits_kernel(const float *__restrict__ x, int64_t ldx,
+                         const float *__restrict__ w, int n, float inv_n, float eps, int D,
+                         int Mp, int Kp, int8_t *__restrict__ planes) {
   __shared__ float red[4];
   extern __shared__ __attribute__((aligned(16))) float row_cache[];
   const int row = blockIdx.x;
-  const float *xr = x + (size_t)row * n;
+  const float *xr = x + (int64_t)row * ldx;
   float s = 0.f;
   for (int i = threadIdx.x; i < n; i += 256)
     s = fmaf(xr[i], xr[i], s);
@@ -685,13 +685,13 @@ int launch_activations_to_digits(const float *A, int64_t lda, int64_t M, int64_t
   return BUDDY_HIP_OK;
 }
 
-int launch_rmsnorm_to_digits(const float *x, const float *w, int rows, int n, float eps,
-                             int digits, void *staged, hipStream_t stream) {
-  BH_REQUIRE(x && w && staged && rows > 0 && n > 0 && digits >= 2 && digits <= 3,
+int launch_rmsnorm_to_digits(const float *x, int64_t ldx, const float *w, int rows, int n,
+                             float eps, int digits, void *staged, hipStream_t stream) {
+  BH_REQUIRE(x && w && staged && rows > 0 && n > 0 && ldx >= n && digits >= 2 && digits <= 3,
              "rmsnorm_to_digits: bad argument");
   const GemmStagingLayout l = gemm_staging_layout(rows, n);
   hipLaunchKernelGGL(rmsnorm_to_digits_kernel, dim3(rows), dim3(256),
-                     row_cache_bytes(l.cols_padded), stream, x, w, n,
+                     row_cache_bytes(l.cols_padded), stream, x, ldx, w, n,
                      1.0f / (float)n, eps, digits, l.rows_padded, l.cols_padded,
                      static_cast<int8_t *>(staged));
   BH_CHECK_HIP(hipGetLastError());

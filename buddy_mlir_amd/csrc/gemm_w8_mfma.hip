@@ -462,8 +462,14 @@ __global__ void __launch_bounds__(kSlices *kWave) gemm_w8_bf16_wide_kernel(GemmA
       }
     }
   }
-  // loads of the repeated last chunk may still be in flight
+  // loads of the repeated last chunk may still be in flight: the ring registers
+  // stay allocated until they have landed (without these ties the compiler may
+  // put a temporary of the epilogue into one of them before the wait, and the
+  // late load would overwrite it)
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#pragma unroll
+  for (int u = 0; u < kRing; ++u)
+    wait_loads<0, TERMS>(ring[u]);
 
   // ---- epilogue: lane holds channels n..n+3 of row m for each row block ------
 #pragma unroll

@@ -40,7 +40,7 @@ struct GemvArgs {
 };
 
 int launch_gemv(const GemvArgs &a, hipStream_t stream);
-// Matrix-core variant for 2..16 rows (chosen by launch_gemv).
+// Matrix-core variant for 5..16 rows (chosen by launch_gemv).
 int launch_gemv_mfma(const GemvArgs &a, hipStream_t stream);
 
 } // namespace bh

@@ -293,7 +293,14 @@ __global__ void __launch_bounds__(kMaxWavesMfma *kWave)
       fetch_chunk<SPAN, DUAL, NORM>(a, w0, w1, gofs, xrow, kofs, min(c + R, clast), cur);
     }
   }
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // repeated last chunks
+  // repeated last chunks may still be in flight: the ring registers stay
+  // allocated until they have landed (without these ties the compiler may put
+  // a temporary of the code below into one of them before the wait, and the
+  // late load would overwrite it)
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#pragma unroll
+  for (int u = 0; u < R; ++u)
+    wait_fetch<0, SPAN, DUAL, NORM>(ring[u]);
   if (NORM) { // the four lanes that share a row hold different k
     ss += __shfl_xor(ss, 16, 64);
     ss += __shfl_xor(ss, 32, 64);
@@ -428,7 +435,10 @@ int launch_gemv_mfma(const GemvArgs &a, hipStream_t stream) {
   const bool dual = a.epilogue == kEpiSiluMul;
   // channel groups per wavefront (they share one conversion of the
   // activations): eight for wide single-matrix launches, else four, two when
-  // that leaves too few wavefronts to cover the chip even with 8 k-slices
+  // that leaves too few wavefronts to cover the chip even with 8 k-slices.
+  // (Measured: fewer, wider spans would cut the L2 -> CU traffic of the
+  // activations, but the launches get slower, not faster: 2.9 -> 3.9 ms for the
+  // Llama-3-8B sweep at 8 rows.)
   int span = 4;
   if (!dual && ceil_div(ka.groups, 8) >= 1024)
     span = 8;

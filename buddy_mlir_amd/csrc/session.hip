@@ -333,8 +333,8 @@ struct Session {
   int norm_to_staging(const float *x, const float *w, int rows, unsigned short *staged) {
     const auto &S = shape;
     if (gemm_digits)
-      return launch_rmsnorm_to_digits(x, w, rows, S.hidden, S.rms_eps, gemm_digits, staged,
-                                      stream);
+      return launch_rmsnorm_to_digits(x, S.hidden, w, rows, S.hidden, S.rms_eps, gemm_digits,
+                                      staged, stream);
     return launch_rmsnorm_to_staging(x, w, rows, S.hidden, S.rms_eps, gemm_terms, staged,
                                      stream);
   }
