@@ -181,6 +181,36 @@ def test_small_model_block_prefill_equals_token_by_token(oracle, precision):
     sess.close()
 
 
+def test_prefill_in_two_blocks_and_after_decode_steps(oracle):
+    """A prompt fed as two blocks (the second starts at position 24 and attends
+    to the cache rows of the first), then decode steps, then a third block: the
+    same logits and cache rows as 53 oracle decode steps."""
+    sess, host = synthetic.build_session(SMALL, context=0, keep_host=True, ln_jitter=0.1)
+    om = oracle_model(oracle, SMALL, host)
+    kv = [a.copy() for a in host["kv"]]
+    toks = synthetic.first_tokens(SMALL, 53, seed=11).tolist()
+    want = []
+    for pos, t in enumerate(toks):
+        otok, ologits = om.decode_step(t, pos, kv)
+        want.append((otok, ologits))
+    nxt, logits = sess.prefill(toks[:24], 0)
+    check_close(logits, want[23][1])
+    assert nxt == want[23][0]
+    nxt, logits = sess.prefill(toks[24:40], 24)
+    check_close(logits, want[39][1])
+    assert nxt == want[39][0]
+    for pos in range(40, 43):  # three tokens one by one
+        n2, lg = sess.decode(toks[pos], pos)
+        check_close(lg, want[pos][1])
+        assert n2 == want[pos][0]
+    nxt, logits = sess.prefill(toks[43:53], 43)  # a ragged block of 10
+    check_close(logits, want[52][1])
+    assert nxt == want[52][0]
+    for j in range(2 * SMALL.layers):
+        check_close(sess.get_kv(j)[:, :53, :], kv[j][:, :53, :])
+    sess.close()
+
+
 def test_session_prefill_refuses_overflow(bh):
     sess, _ = synthetic.build_session(SMALL, context=0)
     with pytest.raises(bma.BuddyHipError):
