@@ -25,7 +25,15 @@
  *   argmax_first ........... first-index tie rule
  *   w8a8_matmul ............ exact int64 brute force
  *   decode_step ............ composition; cross-checked against an independent
- *                            numpy float64 model in the tests
+ *                            numpy float64 model in the tests, and against the
+ *                            logits of the pip `transformers` Qwen2 model for a
+ *                            seeded tiny decoder (tests/golden fixture)
+ *   kv_discard, kv_adjust_rope  numpy slice assignment; rotation by -d against
+ *                            the pinned RoPE; refusals of the reference
+ *   f32_to_f16, pack_int4, w4a16_gemv  numpy.float16; closed form over all byte
+ *                            values; the reference example's inputs
+ * Parity unpinned: the order of parameters inside the reference's weight blobs
+ * (no blob written by the reference's importer exists to check it against).
  */
 #ifndef BUDDY_ORACLE_H
 #define BUDDY_ORACLE_H
