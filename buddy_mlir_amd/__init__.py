@@ -135,6 +135,11 @@ def _declare(lib):
         "buddy_hip_session_enqueue_steps": (c_int, [vp, c_int]),
         "buddy_hip_session_logits": (vp, [vp]),
         "buddy_hip_session_stream": (vp, [vp]),
+        "buddy_hip_session_vocab": (c_int, [vp]),
+        "buddy_hip_sampler_create": (vp, [vp]),
+        "buddy_hip_sampler_destroy": (None, [vp]),
+        "buddy_hip_sampler_sample": (c_int, [vp, vp, c_int, vp, c_int, vp, vp]),
+        "buddy_hip_session_decode_sample": (c_int, [vp, vp, c_int, c_int, vp, c_int, vp]),
         "buddy_hip_gemv_f32": (c_int, [vp, vp, vp, vp, i64, i64, c_uint, vp]),
         "buddy_hip_f32_tiles_bytes": (sz, [i64, i64]),
         "buddy_hip_tile_f32": (c_int, [vp, i64, i64, vp, vp]),

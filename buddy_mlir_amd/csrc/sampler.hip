@@ -1,0 +1,312 @@
+// sampler.hip -- the reference's token sampler with its vocabulary-sized part on
+// the device.
+//
+// runtime/include/buddy/runtime/llm/Sampler.h:62-206 copies the logits, applies
+// the repetition penalty (:112-129) and the temperature (:131-136), sorts the
+// whole vocabulary (:147-149), keeps the top K, and then works on those K
+// candidates only: softmax in f32, min-P, top-P, renormalisation and a draw from
+// std::discrete_distribution over std::mt19937 (:151-203).  In a decode loop
+// whose logits live on the device that would mean 608 KB over PCIe and a
+// 152k-element sort on the host per token.  Here the penalty, the temperature
+// and the top-K selection run on the device (two launches: per-block bitonic
+// sorts, then one sort of the block winners), K (value, index) pairs come back,
+// and the host does what the reference does with them, with the same standard
+// library generator and distribution, so the chosen token is the reference's.
+// Candidates of equal value are ordered by index (the reference's std::sort
+// leaves their order unspecified).  Without a top-K limit (or with one beyond
+// what the device selection holds) the logits are copied back and the whole of
+// the reference's algorithm runs on the host.
+#include "common.h"
+
+#include <algorithm>
+#include <cmath>
+#include <new>
+#include <random>
+#include <utility>
+#include <vector>
+
+struct buddy_hip_sampler {
+  buddy_hip_sampler_config cfg;
+  std::mt19937 rng;
+  int *d_recent = nullptr;
+  unsigned long long *d_partial = nullptr, *d_out = nullptr, *h_out = nullptr;
+  size_t partial_cap = 0; // keys
+  std::vector<float> h_logits;
+};
+
+namespace bh {
+namespace {
+
+typedef unsigned long long u64;
+
+constexpr int kBlockElems = 4096; // logits per workgroup of the first launch
+constexpr int kMergeElems = 8192; // keys the second launch sorts
+constexpr int kMaxWindow = 1024;  // repetition-penalty window held in LDS
+
+// (value, index) as one integer: larger value first, then the smaller index
+__device__ __forceinline__ u64 make_key(float v, int i) {
+  unsigned u = __float_as_uint(v);
+  u ^= (u >> 31) ? 0xffffffffu : 0x80000000u; // monotonic in v
+  return ((u64)u << 32) | (u64)(0xffffffffu - (unsigned)i);
+}
+inline void split_key(u64 k, float *v, int *i) {
+  unsigned u = (unsigned)(k >> 32);
+  u ^= (u >> 31) ? 0x80000000u : 0xffffffffu;
+  union {
+    unsigned u;
+    float f;
+  } c;
+  c.u = u;
+  *v = c.f;
+  *i = (int)(0xffffffffu - (unsigned)(k & 0xffffffffu));
+}
+
+// descending bitonic sort of N keys in LDS by T threads
+template <int N, int T> __device__ __forceinline__ void sort_desc(u64 *keys) {
+  for (int size = 2; size <= N; size <<= 1)
+    for (int stride = size >> 1; stride > 0; stride >>= 1) {
+      __syncthreads();
+      for (int t = threadIdx.x; t < N / 2; t += T) {
+        const int lo = 2 * t - (t & (stride - 1)), hi = lo + stride;
+        const bool desc = (lo & size) == 0;
+        const u64 a = keys[lo], b = keys[hi];
+        if ((a < b) == desc) {
+          keys[lo] = b;
+          keys[hi] = a;
+        }
+      }
+    }
+  __syncthreads();
+}
+
+// Workgroup b: penalty and temperature on logits [b*4096, +4096), its K largest
+// in order to partial[b*K ..].
+__global__ void __launch_bounds__(256)
+sampler_block_topk_kernel(const float *__restrict__ logits, int vocab,
+                          const int *__restrict__ recent, int n_recent, float penalty,
+                          float inv_temp, int K, u64 *__restrict__ partial) {
+  __shared__ u64 keys[kBlockElems];
+  __shared__ int win[kMaxWindow];
+  for (int i = threadIdx.x; i < n_recent; i += 256)
+    win[i] = recent[i];
+  __syncthreads();
+  const int base = blockIdx.x * kBlockElems;
+  for (int e = threadIdx.x; e < kBlockElems; e += 256) {
+    const int i = base + e;
+    u64 key = 0; // below every real key
+    if (i < vocab) {
+      float v = logits[i];
+      for (int r = 0; r < n_recent; ++r) // once per occurrence, like the reference
+        if (win[r] == i)
+          v = v > 0.0f ? v / penalty : v * penalty;
+      v *= inv_temp;
+      key = make_key(v, i);
+    }
+    keys[e] = key;
+  }
+  sort_desc<kBlockElems, 256>(keys);
+  for (int j = threadIdx.x; j < K; j += 256)
+    partial[(size_t)blockIdx.x * K + j] = keys[j];
+}
+
+// One workgroup: the K largest of the block winners, in order.
+__global__ void __launch_bounds__(1024)
+sampler_merge_kernel(const u64 *__restrict__ partial, int n, int K, u64 *__restrict__ out) {
+  __shared__ u64 keys[kMergeElems];
+  for (int i = threadIdx.x; i < kMergeElems; i += 1024)
+    keys[i] = i < n ? partial[i] : 0;
+  sort_desc<kMergeElems, 1024>(keys);
+  for (int j = threadIdx.x; j < K; j += 1024)
+    out[j] = keys[j];
+}
+
+// Sampler.h:151-203 on candidates sorted by value (all of them the top-K limit
+// lets through).  Returns the position of the chosen candidate.
+int draw(buddy_hip_sampler *s, const std::vector<std::pair<int, float>> &cand) {
+  size_t limit = cand.size();
+  const float max_logit = cand[0].second;
+  std::vector<float> probs(limit);
+  float sum_exp = 0.0f;
+  for (size_t i = 0; i < limit; ++i) {
+    probs[i] = std::exp(cand[i].second - max_logit);
+    sum_exp += probs[i];
+  }
+  for (size_t i = 0; i < limit; ++i)
+    probs[i] /= sum_exp;
+  if (s->cfg.min_p > 0.0f) {
+    const float threshold = s->cfg.min_p * probs[0];
+    size_t nl = limit;
+    for (size_t i = 0; i < limit; ++i)
+      if (probs[i] < threshold) {
+        nl = i;
+        break;
+      }
+    if (nl > 0)
+      limit = nl;
+  }
+  if (s->cfg.top_p < 1.0f) {
+    float cum = 0.0f;
+    size_t nl = limit;
+    for (size_t i = 0; i < limit; ++i) {
+      cum += probs[i];
+      if (cum >= s->cfg.top_p) {
+        nl = i + 1;
+        break;
+      }
+    }
+    limit = nl;
+  }
+  float final_sum = 0.0f;
+  for (size_t i = 0; i < limit; ++i)
+    final_sum += probs[i];
+  for (size_t i = 0; i < limit; ++i)
+    probs[i] /= final_sum;
+  std::discrete_distribution<int> dist(probs.begin(), probs.begin() + (long)limit);
+  return dist(s->rng);
+}
+
+} // namespace
+} // namespace bh
+
+extern "C" {
+
+buddy_hip_sampler *buddy_hip_sampler_create(const buddy_hip_sampler_config *cfg) {
+  if (!cfg || cfg->temperature < 0.0f || cfg->top_k < 0 || cfg->repeat_last_n < 0 ||
+      !(cfg->repeat_penalty > 0.0f)) {
+    bh::fail(BUDDY_HIP_ERR_ARG, "sampler_create: bad configuration");
+    return nullptr;
+  }
+  buddy_hip_sampler *s = new (std::nothrow) buddy_hip_sampler;
+  if (!s) {
+    bh::fail(BUDDY_HIP_ERR_ARG, "sampler_create: out of host memory");
+    return nullptr;
+  }
+  s->cfg = *cfg;
+  if (cfg->seed != 0) { // Sampler.h:51-56
+    s->rng.seed(cfg->seed);
+  } else {
+    std::random_device rd;
+    s->rng.seed(rd());
+  }
+  const int K = BUDDY_HIP_SAMPLER_MAX_TOP_K;
+  if (hipMalloc((void **)&s->d_recent, sizeof(int) * bh::kMaxWindow) != hipSuccess ||
+      hipMalloc((void **)&s->d_out, sizeof(bh::u64) * K) != hipSuccess ||
+      hipHostMalloc((void **)&s->h_out, sizeof(bh::u64) * K) != hipSuccess) {
+    bh::fail(BUDDY_HIP_ERR_HIP, "sampler_create: allocation failed");
+    buddy_hip_sampler_destroy(s);
+    return nullptr;
+  }
+  return s;
+}
+
+void buddy_hip_sampler_destroy(buddy_hip_sampler *s) {
+  if (!s)
+    return;
+  if (s->d_recent)
+    (void)hipFree(s->d_recent);
+  if (s->d_partial)
+    (void)hipFree(s->d_partial);
+  if (s->d_out)
+    (void)hipFree(s->d_out);
+  if (s->h_out)
+    (void)hipHostFree(s->h_out);
+  delete s;
+}
+
+int buddy_hip_sampler_sample(buddy_hip_sampler *s, const float *logits, int vocab,
+                             const int *recent, int n_recent, int *token_out,
+                             buddy_hip_stream hstream) {
+  BH_REQUIRE(s && logits && token_out && vocab > 0 && n_recent >= 0 && (recent || !n_recent),
+             "sampler_sample: bad argument");
+  hipStream_t stream = bh::as_stream(hstream);
+  const buddy_hip_sampler_config &c = s->cfg;
+  // the window the penalty looks at (Sampler.h:114-117)
+  int w0 = n_recent - c.repeat_last_n;
+  if (w0 < 0)
+    w0 = 0;
+  const bool penalty = c.repeat_penalty != 1.0f && n_recent > 0;
+  const int window = penalty ? n_recent - w0 : 0;
+  const bool greedy = c.temperature == 0.0f;
+  const float inv_temp = greedy ? 1.0f : 1.0f / c.temperature;
+  // greedy = the first maximum (Sampler.h:101-104): the top 1 with ties by index
+  const int K = greedy ? 1 : c.top_k;
+  const int blocks = (int)bh::ceil_div(vocab, bh::kBlockElems);
+  const bool on_device = K >= 1 && K <= BUDDY_HIP_SAMPLER_MAX_TOP_K && K <= vocab &&
+                         (int64_t)blocks * K <= bh::kMergeElems && window <= bh::kMaxWindow;
+  std::vector<std::pair<int, float>> cand;
+  if (on_device) {
+    if (s->partial_cap < (size_t)blocks * K) {
+      if (s->d_partial)
+        BH_CHECK_HIP(hipFree(s->d_partial));
+      s->d_partial = nullptr;
+      BH_CHECK_HIP(hipMalloc((void **)&s->d_partial, sizeof(bh::u64) * (size_t)blocks * K));
+      s->partial_cap = (size_t)blocks * K;
+    }
+    if (window)
+      BH_CHECK_HIP(hipMemcpyAsync(s->d_recent, recent + w0, sizeof(int) * window,
+                                  hipMemcpyHostToDevice, stream));
+    hipLaunchKernelGGL(bh::sampler_block_topk_kernel, dim3(blocks), dim3(256), 0, stream, logits,
+                       vocab, s->d_recent, window, c.repeat_penalty, inv_temp, K, s->d_partial);
+    BH_CHECK_HIP(hipGetLastError());
+    hipLaunchKernelGGL(bh::sampler_merge_kernel, dim3(1), dim3(1024), 0, stream, s->d_partial,
+                       blocks * K, K, s->d_out);
+    BH_CHECK_HIP(hipGetLastError());
+    BH_CHECK_HIP(hipMemcpyAsync(s->h_out, s->d_out, sizeof(bh::u64) * K, hipMemcpyDeviceToHost,
+                                stream));
+    BH_CHECK_HIP(hipStreamSynchronize(stream));
+    cand.resize((size_t)K);
+    for (int j = 0; j < K; ++j)
+      bh::split_key(s->h_out[j], &cand[(size_t)j].second, &cand[(size_t)j].first);
+  } else {
+    // the whole of the reference's algorithm on the host
+    s->h_logits.resize((size_t)vocab);
+    BH_CHECK_HIP(hipMemcpyAsync(s->h_logits.data(), logits, sizeof(float) * (size_t)vocab,
+                                hipMemcpyDefault, stream));
+    BH_CHECK_HIP(hipStreamSynchronize(stream));
+    std::vector<float> &work = s->h_logits;
+    for (int i = w0; penalty && i < n_recent; ++i) {
+      const int t = recent[i];
+      if (t < 0 || t >= vocab)
+        continue;
+      if (work[(size_t)t] > 0.0f)
+        work[(size_t)t] /= c.repeat_penalty;
+      else
+        work[(size_t)t] *= c.repeat_penalty;
+    }
+    if (greedy) {
+      *token_out = (int)std::distance(work.begin(), std::max_element(work.begin(), work.end()));
+      return BUDDY_HIP_OK;
+    }
+    for (float &v : work)
+      v *= inv_temp;
+    cand.resize((size_t)vocab);
+    for (int i = 0; i < vocab; ++i)
+      cand[(size_t)i] = {i, work[(size_t)i]};
+    std::sort(cand.begin(), cand.end(),
+              [](const std::pair<int, float> &a, const std::pair<int, float> &b) {
+                return a.second > b.second;
+              });
+    if (c.top_k > 0 && c.top_k < vocab)
+      cand.resize((size_t)c.top_k);
+  }
+  if (greedy) {
+    *token_out = cand[0].first;
+    return BUDDY_HIP_OK;
+  }
+  *token_out = cand[(size_t)bh::draw(s, cand)].first;
+  return BUDDY_HIP_OK;
+}
+
+int buddy_hip_session_decode_sample(buddy_hip_session *sess, buddy_hip_sampler *s, int token,
+                                    int pos, const int *recent, int n_recent,
+                                    int *next_token) {
+  BH_REQUIRE(sess && s && next_token, "session_decode_sample: null argument");
+  int rc = buddy_hip_session_set_state(sess, token, pos);
+  if (rc)
+    return rc;
+  if ((rc = buddy_hip_session_enqueue_steps(sess, 1)))
+    return rc;
+  return buddy_hip_sampler_sample(s, buddy_hip_session_logits(sess), buddy_hip_session_vocab(sess),
+                                  recent, n_recent, next_token, buddy_hip_session_stream(sess));
+}
+}

@@ -911,6 +911,11 @@ int buddy_hip_session_discard_kv(buddy_hip_session *hs, int keep, int discard,
   return BUDDY_HIP_OK;
 }
 
+int buddy_hip_session_vocab(buddy_hip_session *hs) {
+  Session *s = reinterpret_cast<Session *>(hs);
+  return s ? s->shape.vocab : 0;
+}
+
 buddy_hip_stream buddy_hip_session_stream(buddy_hip_session *hs) {
   Session *s = reinterpret_cast<Session *>(hs);
   return s ? reinterpret_cast<buddy_hip_stream>(s->stream) : nullptr;

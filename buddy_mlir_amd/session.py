@@ -153,6 +153,15 @@ class DecoderSession:
             "session_prefill")
         return nxt.value, logits
 
+    def decode_sample(self, sampler: "Sampler", token: int, pos: int, recent=()):
+        """One decode step, then the sampler's choice from its logits."""
+        rec = np.ascontiguousarray(recent, np.int32)
+        nxt = c_int(-1)
+        check(self._lib.buddy_hip_session_decode_sample(
+            self._h, sampler._h, token, pos, rec.ctypes.data if rec.size else None,
+            rec.size, ctypes.byref(nxt)), "session_decode_sample")
+        return nxt.value
+
     def set_state(self, token: int, pos: int):
         check(self._lib.buddy_hip_session_set_state(self._h, token, pos), "set_state")
 
@@ -167,3 +176,43 @@ class DecoderSession:
     @property
     def stream(self) -> int:
         return self._lib.buddy_hip_session_stream(self._h) or 0
+
+
+class SamplerConfig(Structure):
+    _fields_ = [("temperature", c_float), ("top_k", c_int), ("top_p", c_float),
+                ("min_p", c_float), ("repeat_penalty", c_float), ("repeat_last_n", c_int),
+                ("seed", ctypes.c_uint64)]
+
+
+class Sampler:
+    """buddy::runtime::Sampler (runtime/include/buddy/runtime/llm/Sampler.h:38-206)
+    with the same defaults; logits are a device tensor."""
+
+    def __init__(self, temperature=0.0, top_k=0, top_p=1.0, min_p=0.0, repeat_penalty=1.0,
+                 repeat_last_n=64, seed=0):
+        self._lib = lib()
+        cfg = SamplerConfig(temperature, top_k, top_p, min_p, repeat_penalty, repeat_last_n,
+                            seed)
+        self._h = self._lib.buddy_hip_sampler_create(ctypes.byref(cfg))
+        if not self._h:
+            raise BuddyHipError(self._lib.buddy_hip_last_error().decode())
+
+    def sample(self, logits: torch.Tensor, recent=(), stream: int = 0) -> int:
+        assert logits.dtype == torch.float32 and logits.is_contiguous()
+        rec = np.ascontiguousarray(recent, np.int32)
+        tok = c_int(-1)
+        check(self._lib.buddy_hip_sampler_sample(
+            self._h, logits.data_ptr(), logits.numel(), rec.ctypes.data if rec.size else None,
+            rec.size, ctypes.byref(tok), stream or None), "sampler_sample")
+        return tok.value
+
+    def close(self):
+        if getattr(self, "_h", None):
+            self._lib.buddy_hip_sampler_destroy(self._h)
+            self._h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass

@@ -299,6 +299,45 @@ int buddy_hip_session_set_state(buddy_hip_session *s, int token, int pos);
 int buddy_hip_session_enqueue_steps(buddy_hip_session *s, int steps);
 const float *buddy_hip_session_logits(buddy_hip_session *s); /* device */
 buddy_hip_stream buddy_hip_session_stream(buddy_hip_session *s);
+int buddy_hip_session_vocab(buddy_hip_session *s);
+
+/* ---- token sampler ----------------------------------------------------------
+ * buddy::runtime::Sampler (runtime/include/buddy/runtime/llm/Sampler.h:38-46
+ * the configuration, :62-206 sample()): repetition penalty over the last
+ * repeat_last_n ids, temperature, top-K, min-P, top-P, and a draw from
+ * std::discrete_distribution over std::mt19937 seeded with `seed` (0: from
+ * std::random_device, :51-56).  temperature 0 is greedy: the first maximum after
+ * the penalty (:101-104).  The logits stay on the device: penalty, temperature
+ * and the top-K selection run there and top_k (value, id) pairs come back; the
+ * rest runs on the host with the same standard-library generator, so a seeded
+ * sampler picks the reference's tokens.  Logits of equal value rank by id.
+ * top_k 0 (no limit), top_k above BUDDY_HIP_SAMPLER_MAX_TOP_K or a penalty
+ * window above 1024 ids copy the logits back and run everything on the host. */
+#define BUDDY_HIP_SAMPLER_MAX_TOP_K 128
+typedef struct buddy_hip_sampler_config {
+  float temperature;    /* Sampler.h:39; 0 = greedy */
+  int top_k;            /* :40; 0 = no limit */
+  float top_p;          /* :41; 1 = off */
+  float min_p;          /* :42; 0 = off */
+  float repeat_penalty; /* :43; 1 = off */
+  int repeat_last_n;    /* :44; the reference's default is 64 */
+  uint64_t seed;        /* :45; 0 = from std::random_device */
+} buddy_hip_sampler_config;
+typedef struct buddy_hip_sampler buddy_hip_sampler;
+buddy_hip_sampler *buddy_hip_sampler_create(const buddy_hip_sampler_config *cfg);
+void buddy_hip_sampler_destroy(buddy_hip_sampler *s);
+/* logits: device (or host-visible) f32[vocab]; recent: host array of the ids
+ * generated so far (Sampler.h:63 recentTokens), n_recent may be 0.  Synchronous
+ * on `stream`. */
+int buddy_hip_sampler_sample(buddy_hip_sampler *s, const float *logits, int vocab,
+                             const int *recent, int n_recent, int *token_out,
+                             buddy_hip_stream stream);
+/* One decode step of the session at (token, pos) followed by a sampled choice
+ * from its logits: the non-greedy branch of the generation loop
+ * (runtime/llm/TextGeneration.cpp:215-266 with a Sampler). */
+int buddy_hip_session_decode_sample(buddy_hip_session *sess, buddy_hip_sampler *s,
+                                    int token, int pos, const int *recent,
+                                    int n_recent, int *next_token);
 
 /* ---- KV-cache overflow ------------------------------------------------------
  * kvcache::discardKVCache followed by kvcache::adjustKeyCacheRope

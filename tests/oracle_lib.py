@@ -292,6 +292,34 @@ class Oracle:
         return int(self.lib.oracle_num_threads())
 
 
+class OracleSampler:
+    """The restated reference sampler (oracle/sampler.cpp)."""
+
+    def __init__(self, oracle, temperature=0.0, top_k=0, top_p=1.0, min_p=0.0,
+                 repeat_penalty=1.0, repeat_last_n=64, seed=1):
+        lib = oracle.lib
+        lib.oracle_sampler_create.restype = c_void_p
+        lib.oracle_sampler_sample.restype = c_int
+        self.lib = lib
+        self.h = c_void_p(lib.oracle_sampler_create(
+            c_float(temperature), c_int(top_k), c_float(top_p), c_float(min_p),
+            c_float(repeat_penalty), c_int(repeat_last_n), ctypes.c_uint64(seed)))
+
+    def sample(self, logits, recent=()):
+        logits = np.ascontiguousarray(logits, np.float32)
+        rec = np.ascontiguousarray(recent, np.int32)
+        kept = c_int64(0)
+        tok = self.lib.oracle_sampler_sample(self.h, _p(logits), c_int64(logits.size),
+                                             _p(rec) if rec.size else None, c_int64(rec.size),
+                                             ctypes.byref(kept))
+        return int(tok), int(kept.value)
+
+    def __del__(self):
+        if getattr(self, "h", None):
+            self.lib.oracle_sampler_destroy(self.h)
+            self.h = None
+
+
 class OracleModel:
     """Holds numpy weights and the ctypes structs that point at them."""
 
