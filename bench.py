@@ -3,7 +3,7 @@
 MI355X, next to the CPU oracle timed on the same host.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W]
-    python bench.py --workload gemv|mlp|prefill|llama8b|kvdiscard|w4a16|model_abi   (the other configurations)
+    python bench.py --workload gemv|mlp|prefill|llama8b|kvdiscard|w4a16|model_abi|sampler   (the other configurations)
 
 A step is one greedy decode step (one token) at batch 1 with the KV cache
 already holding 1024 positions; weights, KV cache and activations are resident
@@ -347,6 +347,65 @@ def bench_kvdiscard(bh, args):
     }
 
 
+def bench_sampler(bh, args):
+    """One sampled token from device logits of the Qwen2 vocabulary: penalty,
+    temperature and top-40 on the device, the rest on the host.  The CPU figure
+    is the restated reference sampler on logits copied back first, which is what
+    a host sampler behind device logits costs."""
+    import time
+
+    import numpy as np
+    import torch
+
+    from buddy_mlir_amd.session import Sampler
+
+    sys.path.insert(0, str(ROOT / "tests"))
+    import oracle_lib
+
+    vocab = 151936
+    cfg = dict(temperature=0.8, top_k=40, top_p=0.95, min_p=0.05, repeat_penalty=1.1,
+               repeat_last_n=64)
+    logits = [torch.randn(vocab, device="cuda") * 3 for _ in range(8)]
+    recent = list(np.random.default_rng(0).integers(0, vocab, 64))
+    sampler = Sampler(seed=1, **cfg)
+    iters = 200
+    for i in range(8):
+        sampler.sample(logits[i % 8], recent)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(iters):
+        sampler.sample(logits[i % 8], recent)
+    t = (time.perf_counter() - t0) / iters
+    cpu = oracle_lib.OracleSampler(oracle_lib.load(), seed=1, **cfg)
+    host = torch.empty(vocab, pin_memory=True)
+    n_cpu = 40
+    t0 = time.perf_counter()
+    for i in range(n_cpu):
+        host.copy_(logits[i % 8])
+        cpu.sample(host.numpy(), recent)
+    t_cpu = (time.perf_counter() - t0) / n_cpu
+    by = vocab * 4
+    return {
+        "metric": "sampled_tokens_per_sec", "value": 1.0 / t, "unit": "samples/s",
+        "n_gpus": 1, "steps": iters, "warmup": 8, "ms_per_step": t * 1e3,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": "sampler, vocabulary 151936, temperature 0.8 / top-K 40 / "
+                               "top-P 0.95 / min-P 0.05 / penalty 1.1 over 64 ids; each call "
+                               "synchronous (three launches, 328 B written to pinned host memory, host finish)"},
+        "roofline": {"kernel": "sampler_keys_kernel + sampler_candidates_kernel + sampler_pick_kernel",
+                     "bound": "hbm", "achieved": by / t / 1e9, "peak": HBM_PEAK_GBPS,
+                     "unit": "GB/s", "frac": by / t / 1e9 / HBM_PEAK_GBPS,
+                     "algorithmic_bytes_per_launch": by, "avg_launch_us": t * 1e6,
+                     "traffic": None,
+                     "note": "latency-bound: 608 KB of logits, three short launches and a host "
+                             "round trip; the call's wall time is used, not a kernel's"},
+        "cpu_baseline": {"value": 1.0 / t_cpu, "unit": "samples/s", "cores": 1, "kind": "port",
+                         "sample": f"{n_cpu} calls of the restated reference sampler, each after "
+                                   "copying the 151936 logits to pinned host memory"},
+    }
+
+
 def bench_w4a16(bh, args):
     """The reference's int4 weight-only decode GEMV (f16 activations and
     accumulator, k in order) at 1536 -> 8960 and 8960 -> 1536, 24 weight copies."""
@@ -526,7 +585,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=8)
     ap.add_argument("--workload", default="decode",
                     choices=["decode", "gemv", "mlp", "prefill", "llama8b", "kvdiscard", "w4a16",
-                             "model_abi"],
+                             "model_abi", "sampler"],
                     help="decode (default): the full decode step the headline metric "
                          "is quoted on; the others measure the remaining configurations")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -552,7 +611,7 @@ def main():
     if args.workload != "decode":
         fn = {"gemv": bench_gemv, "mlp": bench_mlp, "prefill": bench_prefill,
               "llama8b": bench_llama8b, "kvdiscard": bench_kvdiscard, "w4a16": bench_w4a16,
-              "model_abi": bench_model_abi}[args.workload]
+              "model_abi": bench_model_abi, "sampler": bench_sampler}[args.workload]
         print(json.dumps(fn(bh, args)))
         return
     K, W = args.steps, args.warmup

@@ -32,6 +32,10 @@
  *                            the pinned RoPE; refusals of the reference
  *   f32_to_f16, pack_int4, w4a16_gemv  numpy.float16; closed form over all byte
  *                            values; the reference example's inputs
+ *   sampler (sampler.cpp) .. numpy re-derivation of the whole pipeline and of the
+ *                            draw (MT19937 output sequence, libstdc++'s
+ *                            canonical double and discrete_distribution);
+ *                            closed-form frequencies
  * Parity unpinned: the order of parameters inside the reference's weight blobs
  * (no blob written by the reference's importer exists to check it against).
  */

@@ -75,7 +75,7 @@ def test_penalty_window_counts_each_occurrence(bh, oracle):
 
 
 def test_equal_logits_rank_by_id(bh):
-    logits = torch.zeros(10000, device="cuda")
+    logits = torch.ones(10000, device="cuda")
     assert Sampler(temperature=0.0, repeat_penalty=1.1).sample(logits, [0, 1]) == 2
     s = Sampler(temperature=1.0, top_k=4, seed=5)
     seen = {s.sample(logits) for _ in range(200)}
