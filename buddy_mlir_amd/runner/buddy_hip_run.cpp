@@ -13,6 +13,13 @@
 //                 --tokens 151646,8948,... [--max-new 64] [--max-len 1024]
 //                 [--eos 151643] [--layers 28 --hidden 1536 --heads 12
 //                 --kv-heads 2 --inter 8960 --vocab 151936]
+//                 [--temperature T --top-k K --top-p P --min-p P
+//                  --repeat-penalty R --repeat-last-n N --seed S]
+//
+// With a temperature above 0 or a repetition penalty other than 1 the next
+// token comes from the library's sampler
+// (runtime/include/buddy/runtime/llm/Sampler.h:38-46 names the options),
+// otherwise decoding is greedy on the device.
 //
 // Only the C interface of the library is used; nothing here touches the GPU
 // directly.
@@ -33,9 +40,12 @@ void usage(FILE *f) {
   fputs("usage: buddy_hip_run --f32 FILE --i8 FILE --tokens ID,ID,... [--max-new N]\n"
         "                     [--max-len N] [--eos ID] [--layers N --hidden N --heads N\n"
         "                     --kv-heads N --inter N --vocab N]\n"
+        "                     [--temperature T --top-k K --top-p P --min-p P\n"
+        "                      --repeat-penalty R --repeat-last-n N --seed S]\n"
         "Runs the reference's w8a32 parameter files (arg0-w8a32-f32.data,\n"
         "arg0-w8a32-i8.data) through libbuddy_hip: prefill of the prompt tokens, then\n"
-        "greedy decoding.  Defaults are the DeepSeek-R1-Distill-Qwen-1.5B shape.\n",
+        "greedy decoding, or sampling when a temperature or a repetition penalty is\n"
+        "given.  Defaults are the DeepSeek-R1-Distill-Qwen-1.5B shape.\n",
         f);
 }
 
@@ -92,6 +102,7 @@ int main(int argc, char **argv) {
   std::string f32_path, i8_path;
   std::vector<int> prompt;
   int max_new = 64, eos = 151643;
+  buddy_hip_sampler_config sampling = {0.0f, 0, 1.0f, 0.0f, 1.0f, 64, 0};
   for (int i = 1; i < argc; ++i) {
     const std::string a = argv[i];
     if (a == "--help" || a == "-h") {
@@ -119,6 +130,13 @@ int main(int argc, char **argv) {
     else if (a == "--kv-heads") shape.kv_heads = atoi(v);
     else if (a == "--inter") shape.inter = atoi(v);
     else if (a == "--vocab") shape.vocab = atoi(v);
+    else if (a == "--temperature") sampling.temperature = (float)atof(v);
+    else if (a == "--top-k") sampling.top_k = atoi(v);
+    else if (a == "--top-p") sampling.top_p = (float)atof(v);
+    else if (a == "--min-p") sampling.min_p = (float)atof(v);
+    else if (a == "--repeat-penalty") sampling.repeat_penalty = (float)atof(v);
+    else if (a == "--repeat-last-n") sampling.repeat_last_n = atoi(v);
+    else if (a == "--seed") sampling.seed = strtoull(v, nullptr, 10);
     else {
       usage(stderr);
       return 2;
@@ -158,10 +176,24 @@ int main(int argc, char **argv) {
   std::vector<int8_t>().swap(i8); // the session holds its own packed copy
   printf("[Log] Upload and packing: %.3fs\n", seconds_since(t0));
 
+  const bool sampled = sampling.temperature > 0.0f || sampling.repeat_penalty != 1.0f;
+  buddy_hip_sampler *sampler = nullptr;
+  if (sampled && !(sampler = buddy_hip_sampler_create(&sampling))) {
+    fprintf(stderr, "[Error] %s\n", buddy_hip_last_error());
+    return 1;
+  }
+
   // prefill: the prompt as one block; the token it predicts is the first output
   int next = -1;
   t0 = std::chrono::steady_clock::now();
   if (buddy_hip_session_prefill(s, prompt.data(), (int)prompt.size(), 0, nullptr, &next)) {
+    fprintf(stderr, "[Error] %s\n", buddy_hip_last_error());
+    return 1;
+  }
+  // the reference samples the first token from the prefill logits, with no
+  // recent ids yet (runtime/llm/TextGeneration.cpp:191-196)
+  if (sampled && buddy_hip_sampler_sample(sampler, buddy_hip_session_logits(s), shape.vocab,
+                                          nullptr, 0, &next, buddy_hip_session_stream(s))) {
     fprintf(stderr, "[Error] %s\n", buddy_hip_last_error());
     return 1;
   }
@@ -174,6 +206,18 @@ int main(int argc, char **argv) {
   int pos = (int)prompt.size();
   double decode_s = 0;
   int decoded = 0;
+  while (sampled && (int)out.size() < max_new && out.back() != eos) {
+    t0 = std::chrono::steady_clock::now();
+    if (buddy_hip_session_decode_sample(s, sampler, out.back(), pos, out.data(), (int)out.size(),
+                                        &next)) {
+      fprintf(stderr, "[Error] %s\n", buddy_hip_last_error());
+      return 1;
+    }
+    decode_s += seconds_since(t0);
+    ++decoded;
+    ++pos;
+    out.push_back(next);
+  }
   while ((int)out.size() < max_new && out.back() != eos) {
     const int run = std::min(16, max_new - (int)out.size());
     int buf[16];
@@ -191,6 +235,7 @@ int main(int argc, char **argv) {
         break;
     }
   }
+  buddy_hip_sampler_destroy(sampler);
   buddy_hip_session_destroy(s);
 
   printf("[Prefilling] %.1f tokens/s\n", (double)prompt.size() / prefill_s);

@@ -94,3 +94,29 @@ def test_runner_generates_what_the_session_and_the_oracle_generate(tmp_path, bh,
     out = [l for l in r.stdout.splitlines() if l.startswith("[Output ids]")][0]
     got = [int(t) for t in out.split("]")[1].split()]
     assert got == want[:want.index(want[3]) + 1]
+
+    # sampled generation: the same files, the reference's sampler options
+    opts = dict(temperature=0.9, top_k=20, top_p=0.95, min_p=0.02, repeat_penalty=1.15,
+                repeat_last_n=8)
+    r = run("--f32", str(tmp_path / "arg0-w8a32-f32.data"),
+            "--i8", str(tmp_path / "arg0-w8a32-i8.data"),
+            "--tokens", ",".join(map(str, prompt)), "--max-new", str(new), "--eos", "-1",
+            "--layers", str(SMALL.layers), "--hidden", str(SMALL.hidden),
+            "--heads", str(SMALL.heads), "--kv-heads", str(SMALL.kv_heads),
+            "--inter", str(SMALL.inter), "--vocab", str(SMALL.vocab),
+            "--max-len", str(SMALL.max_len), "--temperature", "0.9", "--top-k", "20",
+            "--top-p", "0.95", "--min-p", "0.02", "--repeat-penalty", "1.15",
+            "--repeat-last-n", "8", "--seed", "7")
+    assert r.returncode == 0, r.stderr
+    out = [l for l in r.stdout.splitlines() if l.startswith("[Output ids]")][0]
+    got = [int(t) for t in out.split("]")[1].split()]
+    sampler = oracle_lib.OracleSampler(oracle, seed=7, **opts)
+    kv = [np.zeros_like(k) for k in kv]
+    for pos, t in enumerate(prompt):
+        _, logits = om.decode_step(t, pos, kv)
+    want = [sampler.sample(logits, [])[0]]
+    for step in range(new - 1):
+        _, logits = om.decode_step(want[-1], len(prompt) + step, kv)
+        want.append(sampler.sample(logits, want)[0])
+    assert got == want
+    assert len(set(got)) > 1
