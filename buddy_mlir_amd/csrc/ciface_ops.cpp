@@ -7,6 +7,7 @@
 // fills the descriptor; strided inputs are compacted; errors go to stderr and
 // the function returns with the result left null.
 #include "common.h"
+#include "gemm.h"
 #include "gemv_w8a32.h"
 
 #include <cstdlib>
@@ -128,6 +129,29 @@ int to_device(OpContext &c, const T *src, bool src_on_device, int64_t rows,
   return BUDDY_HIP_OK;
 }
 
+// Packed copy of a dense device matrix and a dense copy of its scales.
+int fill_weight(OpContext &c, const int8_t *w_dev, const float *s, intptr_t sstride,
+                int64_t K, int64_t N, CachedWeight *cw) {
+  BH_CHECK_HIP(hipMalloc((void **)&cw->packed, buddy_hip_w8_packed_bytes(K, N)));
+  BH_CHECK_HIP(hipMalloc((void **)&cw->scale, sizeof(float) * (size_t)N));
+  int rc = buddy_hip_pack_w8(w_dev, K, N, cw->packed, c.stream);
+  if (rc)
+    return rc;
+  if (is_device_pointer(s)) {
+    BH_CHECK_HIP(hipMemcpy2DAsync(cw->scale, sizeof(float), s, sizeof(float) * sstride,
+                                  sizeof(float), N, hipMemcpyDeviceToDevice, c.stream));
+  } else {
+    std::vector<float> dense((size_t)N);
+    for (int64_t n = 0; n < N; ++n)
+      dense[(size_t)n] = s[n * sstride];
+    BH_CHECK_HIP(hipMemcpyAsync(cw->scale, dense.data(), sizeof(float) * N,
+                                hipMemcpyHostToDevice, c.stream));
+    BH_CHECK_HIP(hipStreamSynchronize(c.stream)); // `dense` dies with this scope
+  }
+  BH_CHECK_HIP(hipStreamSynchronize(c.stream));
+  return BUDDY_HIP_OK;
+}
+
 int get_weight(OpContext &c, buddy_memref_i8_2d *W, buddy_memref_f32_2d *scale,
                int64_t K, int64_t N, CachedWeight *out) {
   const int8_t *w = data_of(W->aligned, W->offset);
@@ -150,24 +174,14 @@ int get_weight(OpContext &c, buddy_memref_i8_2d *W, buddy_memref_f32_2d *scale,
                      W->strides[1], c.w_stage, &w_dev);
   if (rc)
     return rc;
-  BH_CHECK_HIP(hipMalloc((void **)&cw.packed, buddy_hip_w8_packed_bytes(K, N)));
-  BH_CHECK_HIP(hipMalloc((void **)&cw.scale, sizeof(float) * (size_t)N));
-  rc = buddy_hip_pack_w8(w_dev, K, N, cw.packed, c.stream);
-  if (rc)
+  rc = fill_weight(c, w_dev, s, sstride, K, N, &cw);
+  if (rc) { // nothing half-made stays behind
+    if (cw.packed)
+      (void)hipFree(cw.packed);
+    if (cw.scale)
+      (void)hipFree(cw.scale);
     return rc;
-  if (is_device_pointer(s)) {
-    BH_CHECK_HIP(hipMemcpy2DAsync(cw.scale, sizeof(float), s,
-                                  sizeof(float) * sstride, sizeof(float), N,
-                                  hipMemcpyDeviceToDevice, c.stream));
-  } else {
-    std::vector<float> dense((size_t)N);
-    for (int64_t n = 0; n < N; ++n)
-      dense[(size_t)n] = s[n * sstride];
-    BH_CHECK_HIP(hipMemcpyAsync(cw.scale, dense.data(), sizeof(float) * N,
-                                hipMemcpyHostToDevice, c.stream));
-    BH_CHECK_HIP(hipStreamSynchronize(c.stream));
   }
-  BH_CHECK_HIP(hipStreamSynchronize(c.stream));
   c.weights.emplace(key, cw);
   *out = cw;
   return BUDDY_HIP_OK;
@@ -211,7 +225,27 @@ int dequant_matmul(buddy_memref_f32_2d *A, buddy_memref_i8_2d *W,
                                     sizeof(float) * ldc, sizeof(float) * N, M,
                                     hipMemcpyHostToDevice, c.stream));
   }
-  for (int64_t m0 = 0; m0 < M; m0 += 16) {
+  if (M > 16) {
+    // a block of rows (the prefill shape): the matrix-core matmul, with every
+    // bit of the f32 activations carried (three bf16 terms), so that NaN and
+    // infinity propagate as they do in the reference's f32 arithmetic
+    GemmW8Args g;
+    g.A = a_dev;
+    g.lda = K;
+    g.W = cw.packed;
+    g.scale = cw.scale;
+    g.C = c_dev;
+    g.ldc = ldc_dev;
+    g.M = M;
+    g.K = K;
+    g.N = N;
+    g.accumulate = accumulate;
+    g.terms = 3;
+    rc = launch_gemm_w8(g, c.stream);
+    if (rc)
+      return rc;
+  }
+  for (int64_t m0 = 0; M <= 16 && m0 < M; m0 += 16) {
     GemvArgs g;
     g.A = a_dev + m0 * K;
     g.lda = K;

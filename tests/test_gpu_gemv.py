@@ -168,6 +168,47 @@ def test_memref_abi_strided_inputs_and_accumulate(bh, oracle):
     bh.buddy_hip_clear_weight_cache()
 
 
+def test_memref_abi_block_of_rows_takes_the_matrix_cores(bh, oracle):
+    # M above the GEMV's 16 rows: the prefill-shaped call through the operator
+    # symbol; all f32 bits of the activations are carried, NaN propagates
+    rng = np.random.default_rng(5)
+    M, K, N = 77, 300, 200
+    A = rng.normal(0, 1, (M, K)).astype(np.float32)
+    A[3] *= 1e20
+    A[5] *= 1e-20
+    W = rng.integers(-128, 128, (K, N)).astype(np.int8)
+    S = rng.uniform(1e-4, 1e-3, (1, N)).astype(np.float32)
+    res = bma.MemRefF32_2D()
+    a = bma.MemRef(A.ctypes.data, [M, K])
+    w = bma.MemRef(W.ctypes.data, [K, N], ctype=ctypes.c_int8)
+    s = bma.MemRef(S.ctypes.data, [1, N])
+    bh._mlir_ciface_buddy_dequant_matmul_i8_f32(ctypes.byref(res), ctypes.byref(a),
+                                                ctypes.byref(w), ctypes.byref(s))
+    assert res.aligned, bh.buddy_hip_last_error()
+    out = np.ctypeslib.as_array(res.aligned, shape=(M, N)).copy()
+    ctypes.CDLL(None).free(res.allocated)
+    want = oracle.blis_gemm_w8a32(A, W, S)
+    for m in range(M):  # rows differ by 40 orders of magnitude: compare row by row
+        check_close(out[m], want[m])
+    # accumulate into a strided host C
+    Cbig = rng.normal(0, 1, (M, N + 8)).astype(np.float32)
+    C0 = Cbig[:, :N].copy()
+    c = bma.MemRef(Cbig.ctypes.data, [M, N], strides=[N + 8, 1])
+    A[3] /= 1e20
+    A[5] /= 1e-20
+    bh._mlir_ciface_buddy_dequant_matmul_i8_f32_acc(ctypes.byref(c), ctypes.byref(a),
+                                                    ctypes.byref(w), ctypes.byref(s))
+    check_close(Cbig[:, :N], oracle.blis_gemm_w8a32(A, W, S, C0.copy()))
+    A[2, 7] = np.nan
+    res = bma.MemRefF32_2D()
+    bh._mlir_ciface_buddy_dequant_matmul_i8_f32(ctypes.byref(res), ctypes.byref(a),
+                                                ctypes.byref(w), ctypes.byref(s))
+    out = np.ctypeslib.as_array(res.aligned, shape=(M, N)).copy()
+    ctypes.CDLL(None).free(res.allocated)
+    assert np.isnan(out[2]).all() and not np.isnan(np.delete(out, 2, 0)).any()
+    bh.buddy_hip_clear_weight_cache()
+
+
 def test_bad_arguments_are_refused(bh):
     # null operands: message on stderr, result left null, nothing launched
     res = bma.MemRefF32_2D()
