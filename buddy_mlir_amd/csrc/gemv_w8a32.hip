@@ -56,16 +56,18 @@ int target_waves() {
   return v;
 }
 
-GemvPlan make_plan(int64_t M, int64_t K, int64_t N, bool dual, int tn) {
+GemvPlan make_plan(int64_t M, int64_t K, int64_t N, bool dual, int tn, bool fold = false) {
   (void)dual;
   GemvPlan p;
   p.chunks = ceil_div(K, 1024 / tn);
   p.groups = ceil_div(N, tn);
   // k-slices per channel group: enough wavefronts to cover 256 CUs several
-  // times, but at least two tiles per wavefront
+  // times, but at least two tiles per wavefront (one when the input is folded
+  // from attention partials: that prologue is a chain of dependent loads per
+  // tile, and more, shorter wavefronts shorten it)
   int ks = 1;
   while (ks < kMaxWaves && p.groups * ks < target_waves() &&
-         p.chunks / (ks * 2) >= 2)
+         p.chunks / (ks * 2) >= (fold ? 1 : 2))
     ks *= 2;
   // four staged tiles per wavefront must fit in LDS for every row
   auto red_bytes = [&](int waves) {
@@ -680,15 +682,16 @@ __global__ void __launch_bounds__(kMaxWaves *kWave)
     if (t0 + u < t1)
       fetch_tile<M, PRO, DUAL, true>(a, w0, w1, t0 + u, lane, slot[u]);
   if (PRO == kProAttn && t0 < t1) {
-    // four tiles per fold keep the partials of a batch in registers
-    float xf[(U + 3) / 4][4];
+    // at most four tiles per fold keep the partials of a batch in registers
+    constexpr int FB = U < 4 ? U : 4;
+    float xf[(U + FB - 1) / FB][FB];
 #pragma unroll
-    for (int q = 0; q < (U + 3) / 4; ++q)
-      if (t0 + 4 * q < t1)
-        attn_fold_tiles<4>(a, t0 + 4 * q, t1, lane, xf[q]);
+    for (int q = 0; q < (U + FB - 1) / FB; ++q)
+      if (t0 + FB * q < t1)
+        attn_fold_tiles<FB>(a, t0 + FB * q, t1, lane, xf[q]);
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      slot[u].x[0] = xf[u / 4][u % 4];
+      slot[u].x[0] = xf[u / FB][u % FB];
 #pragma unroll
       for (int m = 1; m < M; ++m)
         slot[u].x[m] = 0.f;
@@ -861,6 +864,12 @@ int launch_one(const KernelArgs &ka, const GemvPlan &p, hipStream_t stream) {
   if (M == 1) {
     // short runs: every tile of a wavefront is requested at once
     const int64_t tpw = ceil_div(p.chunks, p.KS); // tiles per wavefront
+    if constexpr (PRO == kProAttn) {
+      if (tpw <= 2)
+        return launch_bcast<1, EPI, PRO, 2, true>(ka, p, stream);
+      if (tpw <= 3) // the o_proj of the 1.5B shape: no fourth slot to fold for nothing
+        return launch_bcast<1, EPI, PRO, 3, true>(ka, p, stream);
+    }
     if (tpw <= 4)
       return launch_bcast<1, EPI, PRO, 4, true>(ka, p, stream);
     if (tpw <= 6)
@@ -937,7 +946,7 @@ int launch_gemv(const GemvArgs &a, hipStream_t stream) {
   const int mt = compiled_rows(a.M);
   BH_REQUIRE(a.tile_n == 16 || a.tile_n == 8 || a.tile_n == 4,
              "gemv: tile_n=%d (16, 8 or 4)", a.tile_n);
-  const GemvPlan p = make_plan(mt, a.K, a.N, dual, a.tile_n);
+  const GemvPlan p = make_plan(mt, a.K, a.N, dual, a.tile_n, a.attn_acc != nullptr);
   KernelArgs ka;
   ka.A = a.A;
   ka.W0 = reinterpret_cast<const int4 *>(a.W0);
