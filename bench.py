@@ -669,7 +669,7 @@ def main():
         "decode_step_hbm_gbps": step_b / step_s / 1e9,
         "decode_step_hbm_frac": step_b / step_s / 1e9 / HBM_PEAK_GBPS,
         "roofline": {
-            "kernel": "gemv_w8a32_bcast_kernel<1, 2, 1, 6, true> (RMSNorm + gate|up int8 GEMV "
+            "kernel": "gemv_w8a32_bcast_kernel<1, 2, 1, 4, true> (RMSNorm + gate|up int8 GEMV "
                       "+ SiLU*mul, 1536 -> 2 x 8960)",
             "bound": "hbm",
             "achieved": achieved,

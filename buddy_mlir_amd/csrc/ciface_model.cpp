@@ -42,6 +42,7 @@ struct ModelState {
   const void *f32_key = nullptr, *i8_key = nullptr;
   buddy_hip_model_shape shape{};
   float *dev_f32 = nullptr; // the f32 blob on the device (embedding is borrowed)
+  float *pinned_logits = nullptr; // [vocab]: the logits row lands here first
   bool kv_on_device = false;
 };
 
@@ -83,8 +84,11 @@ void destroy_locked(ModelState &m) {
     buddy_hip_session_destroy(m.sess);
   if (m.dev_f32)
     (void)hipFree(m.dev_f32);
+  if (m.pinned_logits)
+    (void)hipHostFree(m.pinned_logits);
   m.sess = nullptr;
   m.dev_f32 = nullptr;
+  m.pinned_logits = nullptr;
   m.f32_key = m.i8_key = nullptr;
   m.kv_on_device = false;
 }
@@ -257,12 +261,17 @@ int forward_decode(DecodeResult *res, buddy_memref_f32_1d *f32, buddy_memref_i8_
     m.kv_on_device = true;
   }
   const int64_t V = m.shape.vocab;
+  // the row crosses PCIe into pinned memory (a copy into pageable memory is
+  // staged by the runtime and several times slower) and is handed over in a
+  // malloc'd buffer, which is what the caller frees
+  if (!m.pinned_logits)
+    BH_CHECK_HIP(hipHostMalloc((void **)&m.pinned_logits, sizeof(float) * (size_t)V));
+  if ((rc = buddy_hip_session_decode(m.sess, (int)token, (int)position, m.pinned_logits,
+                                     nullptr)))
+    return rc;
   float *logits = static_cast<float *>(malloc(sizeof(float) * (size_t)V));
   BH_REQUIRE(logits, "forward_decode: out of host memory");
-  if ((rc = buddy_hip_session_decode(m.sess, (int)token, (int)position, logits, nullptr))) {
-    free(logits);
-    return rc;
-  }
+  memcpy(logits, m.pinned_logits, sizeof(float) * (size_t)V);
   // results: state tensors alias the caller's, logits are handed over
   res->pos_out = *pos;
   res->kv0 = *a.kv[0];

@@ -51,7 +51,7 @@ int target_waves() {
   static int v = [] {
     const char *e = getenv("BUDDY_HIP_GEMV_TARGET_WAVES");
     int t = e ? atoi(e) : 0;
-    return t > 0 ? t : 2048;
+    return t > 0 ? t : 4096;
   }();
   return v;
 }
@@ -65,8 +65,11 @@ GemvPlan make_plan(int64_t M, int64_t K, int64_t N, bool dual, int tn, bool fold
   // times, but at least two tiles per wavefront (one when the input is folded
   // from attention partials: that prologue is a chain of dependent loads per
   // tile, and more, shorter wavefronts shorten it)
+  // (one row: 16 wavefronts per CU's worth of them measured best; with more
+  // rows per wavefront, half as many)
+  const int target = M == 1 ? target_waves() : target_waves() / 2;
   int ks = 1;
-  while (ks < kMaxWaves && p.groups * ks < target_waves() &&
+  while (ks < kMaxWaves && p.groups * ks < target &&
          p.chunks / (ks * 2) >= (fold ? 1 : 2))
     ks *= 2;
   // four staged tiles per wavefront must fit in LDS for every row
