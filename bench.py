@@ -24,7 +24,7 @@ ROOT = Path(__file__).resolve().parent
 sys.path.insert(0, str(ROOT))
 sys.path.insert(0, str(ROOT / "tests"))
 
-GATE_UP_HBM_TRAFFIC_BYTES = 27916074
+GATE_UP_HBM_TRAFFIC_BYTES = 27893551
 HBM_PEAK_GBPS = 8000.0  # MI355X published HBM3E bandwidth
 CONTEXT = 1024
 
