@@ -45,15 +45,15 @@ struct GemmStagingLayout {
 GemmStagingLayout gemm_staging_layout(int64_t M, int64_t K);
 // Producers that write their result straight into a staging buffer:
 //   RMSNorm rows: y = w * (x * rsqrt(mean(x^2) + eps))
-//   SiLU(g) * u
+//   SiLU(g) * u   (g and u rows `ld` floats apart)
 int launch_rmsnorm_to_staging(const float *x, const float *w, int rows, int n, float eps,
                               int terms, unsigned short *staged, hipStream_t stream);
-int launch_silu_mul_to_staging(const float *g, const float *u, int rows, int n, int terms,
+int launch_silu_mul_to_staging(const float *g, const float *u, int64_t ld, int rows, int n, int terms,
                                unsigned short *staged, hipStream_t stream);
 // the same producers for digit planes, and the plain conversion of A
 int launch_rmsnorm_to_digits(const float *x, int64_t ldx, const float *w, int rows, int n,
                              float eps, int digits, void *staged, hipStream_t stream);
-int launch_silu_mul_to_digits(const float *g, const float *u, int rows, int n, int digits,
+int launch_silu_mul_to_digits(const float *g, const float *u, int64_t ld, int rows, int n, int digits,
                               void *staged, hipStream_t stream);
 int launch_activations_to_digits(const float *A, int64_t lda, int64_t M, int64_t K,
                                  int digits, void *staged, hipStream_t stream);

@@ -193,12 +193,12 @@ rmsnorm_to_digits_kernel(const float *__restrict__ x, int64_t ldx,
 }
 
 __global__ void __launch_bounds__(256)
-silu_mul_to_digits_kernel(const float *__restrict__ g, const float *__restrict__ u, int n,
-                          int D, int Mp, int Kp, int8_t *__restrict__ planes) {
+silu_mul_to_digits_kernel(const float *__restrict__ g, const float *__restrict__ u, int64_t ld,
+                          int n, int D, int Mp, int Kp, int8_t *__restrict__ planes) {
   __shared__ float red[4];
   extern __shared__ __attribute__((aligned(16))) float row_cache[];
   const int row = blockIdx.x;
-  row_to_digits(SiluMulRow{g + (size_t)row * n, u + (size_t)row * n, n}, n, row, D, Mp, Kp,
+  row_to_digits(SiluMulRow{g + (size_t)row * ld, u + (size_t)row * ld, n}, n, row, D, Mp, Kp,
                 planes, red, row_cache);
 }
 
@@ -698,13 +698,13 @@ int launch_rmsnorm_to_digits(const float *x, int64_t ldx, const float *w, int ro
   return BUDDY_HIP_OK;
 }
 
-int launch_silu_mul_to_digits(const float *g, const float *u, int rows, int n, int digits,
-                              void *staged, hipStream_t stream) {
-  BH_REQUIRE(g && u && staged && rows > 0 && n > 0 && digits >= 2 && digits <= 3,
+int launch_silu_mul_to_digits(const float *g, const float *u, int64_t ld, int rows, int n,
+                              int digits, void *staged, hipStream_t stream) {
+  BH_REQUIRE(g && u && staged && rows > 0 && n > 0 && ld >= n && digits >= 2 && digits <= 3,
              "silu_mul_to_digits: bad argument");
   const GemmStagingLayout l = gemm_staging_layout(rows, n);
   hipLaunchKernelGGL(silu_mul_to_digits_kernel, dim3(rows), dim3(256),
-                     row_cache_bytes(l.cols_padded), stream, g, u, n,
+                     row_cache_bytes(l.cols_padded), stream, g, u, ld, n,
                      digits, l.rows_padded, l.cols_padded, static_cast<int8_t *>(staged));
   BH_CHECK_HIP(hipGetLastError());
   return BUDDY_HIP_OK;

@@ -146,7 +146,7 @@ rmsnorm_to_staging_kernel(const float *__restrict__ x, const float *__restrict__
 
 __global__ void __launch_bounds__(256)
 silu_mul_to_staging_kernel(const float *__restrict__ g, const float *__restrict__ u,
-                           int rows, int n, int terms, int Mp, int Kp,
+                           int64_t ld, int rows, int n, int terms, int Mp, int Kp,
                            u16 *__restrict__ out) {
   const int kq = Kp / 8;
   const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
@@ -154,7 +154,7 @@ silu_mul_to_staging_kernel(const float *__restrict__ g, const float *__restrict_
     return;
   const int row = (int)(i / kq), k0 = (int)(i % kq) * 8;
   float r[8], gv[8], uv[8];
-  const float *gr = g + (size_t)row * n + k0, *ur = u + (size_t)row * n + k0;
+  const float *gr = g + (size_t)row * ld + k0, *ur = u + (size_t)row * ld + k0;
   if (k0 + 7 < n && ((reinterpret_cast<uintptr_t>(gr) | reinterpret_cast<uintptr_t>(ur)) & 15) == 0) {
     const float4 g0 = *reinterpret_cast<const float4 *>(gr), g1 = *reinterpret_cast<const float4 *>(gr + 4);
     const float4 u0 = *reinterpret_cast<const float4 *>(ur), u1 = *reinterpret_cast<const float4 *>(ur + 4);
@@ -603,14 +603,14 @@ int launch_rmsnorm_to_staging(const float *x, const float *w, int rows, int n, f
   return BUDDY_HIP_OK;
 }
 
-int launch_silu_mul_to_staging(const float *g, const float *u, int rows, int n, int terms,
+int launch_silu_mul_to_staging(const float *g, const float *u, int64_t ld, int rows, int n, int terms,
                                unsigned short *staged, hipStream_t stream) {
   BH_REQUIRE(g && u && staged && rows > 0 && n > 0 && terms >= 1 && terms <= 3,
              "silu_mul_to_staging: bad argument");
   const GemmStagingLayout l = gemm_staging_layout(rows, n);
   const int64_t threads = (int64_t)rows * (l.cols_padded / 8);
   hipLaunchKernelGGL(silu_mul_to_staging_kernel, dim3((unsigned)ceil_div(threads, 256)),
-                     dim3(256), 0, stream, g, u, rows, n, terms, l.rows_padded,
+                     dim3(256), 0, stream, g, u, ld, rows, n, terms, l.rows_padded,
                      l.cols_padded, staged);
   BH_CHECK_HIP(hipGetLastError());
   return BUDDY_HIP_OK;

@@ -58,6 +58,10 @@ struct PackedLinear {
 struct Layer {
   float *ln1 = nullptr, *ln2 = nullptr;
   PackedLinear qkv, o, gate, up, down;
+  // gate and up share one allocation (up right behind gate): when the
+  // intermediate size is a multiple of 16 the two are also one packed matrix of
+  // 2 * inter channels, which the prefill multiplies in one launch
+  bool gate_up_joint = false;
   // the reference's shipped w8a32 build keeps q/k/v in f32 with a bias
   // (they import as AddMMOp, which the quantizer does not touch):
   float *qkv_f32 = nullptr; // [hidden, q|k|v] dense, or null when int8
@@ -262,7 +266,7 @@ struct Session {
       return BUDDY_HIP_OK;
     const auto &S = shape;
     const size_t QN = (size_t)S.heads * S.head_dim, KVN = (size_t)S.kv_heads * S.head_dim;
-    for (float **p : {&pf_x, &pf_xn, &pf_qkv, &pf_att, &pf_g, &pf_u})
+    for (float **p : {&pf_x, &pf_xn, &pf_qkv, &pf_att, &pf_g})
       if (*p) {
         (void)hipFree(*p);
         *p = nullptr;
@@ -279,8 +283,9 @@ struct Session {
     BH_CHECK_HIP(hipMalloc((void **)&pf_xn, sizeof(float) * rows * S.hidden));
     BH_CHECK_HIP(hipMalloc((void **)&pf_qkv, sizeof(float) * rows * (QN + 2 * KVN)));
     BH_CHECK_HIP(hipMalloc((void **)&pf_att, sizeof(float) * rows * QN));
-    BH_CHECK_HIP(hipMalloc((void **)&pf_g, sizeof(float) * rows * S.inter));
-    BH_CHECK_HIP(hipMalloc((void **)&pf_u, sizeof(float) * rows * S.inter));
+    // gate | up side by side: rows of 2 * inter floats
+    BH_CHECK_HIP(hipMalloc((void **)&pf_g, sizeof(float) * rows * 2 * S.inter));
+    pf_u = pf_g + S.inter;
     BH_CHECK_HIP(hipMalloc((void **)&pf_tokens, sizeof(int) * rows));
     // bf16 staging of the matmul inputs that the norm and SiLU kernels write
     // directly (up to three terms)
@@ -313,14 +318,14 @@ struct Session {
   }
   // the same with the input already staged as bf16 terms
   int gemm_staged(const unsigned short *staged, const PackedLinear &W, float *C, int64_t M,
-                  bool accumulate) {
+                  bool accumulate, int64_t ldc = 0) {
     GemmW8Args g;
     g.staged = staged;
     g.W = W.w;
     g.scale = W.s;
     g.bias = accumulate ? nullptr : W.b;
     g.C = C;
-    g.ldc = W.N;
+    g.ldc = ldc ? ldc : W.N;
     g.M = M;
     g.K = W.K;
     g.N = W.N;
@@ -341,8 +346,10 @@ struct Session {
   int silu_mul_to_staging(const float *g, const float *u, int rows, unsigned short *staged) {
     const auto &S = shape;
     if (gemm_digits)
-      return launch_silu_mul_to_digits(g, u, rows, S.inter, gemm_digits, staged, stream);
-    return launch_silu_mul_to_staging(g, u, rows, S.inter, gemm_terms, staged, stream);
+      return launch_silu_mul_to_digits(g, u, 2 * (int64_t)S.inter, rows, S.inter, gemm_digits,
+                                       staged, stream);
+    return launch_silu_mul_to_staging(g, u, 2 * (int64_t)S.inter, rows, S.inter, gemm_terms,
+                                      staged, stream);
   }
 
   // Prompt processing for tokens already in pf_tokens: fills cache rows
@@ -399,10 +406,20 @@ struct Session {
         return rc;
       if ((rc = norm_to_staging(pf_x, L.ln2, n, pf_xn_bf)))
         return rc;
-      if ((rc = gemm_staged(pf_xn_bf, L.gate, pf_g, n, false)))
-        return rc;
-      if ((rc = gemm_staged(pf_xn_bf, L.up, pf_u, n, false)))
-        return rc;
+      const int64_t ld_gu = 2 * (int64_t)S.inter;
+      if (L.gate_up_joint) {
+        // gate | up as one matrix of 2 * inter channels: one launch, whose second
+        // round of tiles starts while the first one drains
+        PackedLinear both = L.gate;
+        both.N = 2 * L.gate.N;
+        if ((rc = gemm_staged(pf_xn_bf, both, pf_g, n, false, ld_gu)))
+          return rc;
+      } else {
+        if ((rc = gemm_staged(pf_xn_bf, L.gate, pf_g, n, false, ld_gu)))
+          return rc;
+        if ((rc = gemm_staged(pf_xn_bf, L.up, pf_u, n, false, ld_gu)))
+          return rc;
+      }
       if ((rc = silu_mul_to_staging(pf_g, pf_u, n, pf_g_bf)))
         return rc;
       if ((rc = gemm_staged(pf_g_bf, L.down, pf_x, n, true)))
@@ -544,7 +561,7 @@ void buddy_hip_session_destroy(buddy_hip_session *hs) {
   for (void *p : s->owned)
     (void)hipFree(p);
   for (void *p : {(void *)s->pf_x, (void *)s->pf_xn, (void *)s->pf_qkv, (void *)s->pf_att,
-                  (void *)s->pf_g, (void *)s->pf_u, (void *)s->pf_tokens,
+                  (void *)s->pf_g, (void *)s->pf_tokens,
                   (void *)s->pf_xn_bf, (void *)s->pf_g_bf})
     if (p)
       (void)hipFree(p);
@@ -626,9 +643,17 @@ int buddy_hip_session_set_layer(buddy_hip_session *hs, int index,
     L.gate.K = H; L.gate.N = I;
     L.up.K = H; L.up.N = I;
     L.down.K = I; L.down.N = H;
-    for (bh::PackedLinear *P : {&L.o, &L.gate, &L.up, &L.down}) {
+    for (bh::PackedLinear *P : {&L.o, &L.down}) {
       rc |= s->alloc(&P->w, buddy_hip_w8_packed_bytes(P->K, P->N));
       rc |= s->alloc(&P->s, (size_t)P->N);
+    }
+    const size_t gate_bytes = buddy_hip_w8_packed_bytes(H, I);
+    rc |= s->alloc(&L.gate.w, 2 * gate_bytes);
+    rc |= s->alloc(&L.gate.s, (size_t)(2 * I));
+    if (!rc) {
+      L.up.w = L.gate.w + gate_bytes;
+      L.up.s = L.gate.s + I;
+      L.gate_up_joint = I % bh::kTileN == 0; // no padding channels between the two
     }
     if (rc)
       return rc;
