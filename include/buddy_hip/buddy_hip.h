@@ -312,7 +312,9 @@ int buddy_hip_session_vocab(buddy_hip_session *s);
  * rest runs on the host with the same standard-library generator, so a seeded
  * sampler picks the reference's tokens.  Logits of equal value rank by id.
  * top_k 0 (no limit), top_k above BUDDY_HIP_SAMPLER_MAX_TOP_K or a penalty
- * window above 1024 ids copy the logits back and run everything on the host. */
+ * window above 1024 ids copy the logits back and run everything on the host.
+ * A sampler owns its generator state and device buffers: one call at a time
+ * per sampler. */
 #define BUDDY_HIP_SAMPLER_MAX_TOP_K 128
 typedef struct buddy_hip_sampler_config {
   float temperature;    /* Sampler.h:39; 0 = greedy */
