@@ -28,11 +28,14 @@
  *                            numpy float64 model in the tests, and against the
  *                            logits of the pip `transformers` Qwen2 model for a
  *                            seeded tiny decoder (tests/golden fixture)
- *   kv_discard, kv_adjust_rope  numpy slice assignment; rotation by -d against
- *                            the pinned RoPE; refusals of the reference
+ *   kv_discard, kv_adjust_rope  the reference's own KVCacheManager.h built as
+ *                            _ref/libref_llm.so (bit for bit); numpy slice
+ *                            assignment; rotation by -d against the pinned RoPE
  *   f32_to_f16, pack_int4, w4a16_gemv  numpy.float16; closed form over all byte
  *                            values; the reference example's inputs
- *   sampler (sampler.cpp) .. numpy re-derivation of the whole pipeline and of the
+ *   sampler (sampler.cpp) .. the reference's own Sampler.h built as
+ *                            _ref/libref_llm.so (token for token); numpy
+ *                            re-derivation of the whole pipeline and of the
  *                            draw (MT19937 output sequence, libstdc++'s
  *                            canonical double and discrete_distribution);
  *                            closed-form frequencies

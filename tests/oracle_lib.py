@@ -376,3 +376,64 @@ def load() -> Oracle:
             build()
         _cached = Oracle(ctypes.CDLL(str(SO)))
     return _cached
+
+
+REF_SO = ROOT / "oracle" / "_ref" / "libref_llm.so"
+
+
+class ReferenceRuntime:
+    """The reference's own header-only sampler and KV-cache manager, as built by
+    `make -C oracle ref` from the reference tree (oracle/ref_llm.cpp).  Only there
+    where that build exists; the tests that use it skip otherwise."""
+
+    def __init__(self):
+        lib = ctypes.CDLL(str(REF_SO))
+        lib.ref_sampler_create.restype = c_void_p
+        lib.ref_sampler_sample.restype = c_int
+        lib.ref_inverse_rope_freqs_count.restype = c_int
+        self.lib = lib
+
+    def sampler(self, temperature=0.0, top_k=0, top_p=1.0, min_p=0.0, repeat_penalty=1.0,
+                repeat_last_n=64, seed=1):
+        lib = self.lib
+        h = c_void_p(lib.ref_sampler_create(
+            c_float(temperature), c_int(top_k), c_float(top_p), c_float(min_p),
+            c_float(repeat_penalty), c_int(repeat_last_n), ctypes.c_uint64(seed)))
+
+        class _S:
+            def sample(_, logits, recent=()):
+                lg = np.ascontiguousarray(logits, np.float32)
+                rec = np.ascontiguousarray(recent, np.int32)
+                return int(lib.ref_sampler_sample(h, _p(lg), c_int64(lg.size),
+                                                  _p(rec) if rec.size else None,
+                                                  c_int64(rec.size)))
+
+            def __del__(_):
+                lib.ref_sampler_destroy(h)
+
+        return _S()
+
+    def _ptrs(self, tensors):
+        return (c_void_p * len(tensors))(*[t.ctypes.data for t in tensors])
+
+    def kv_discard(self, tensors, keep, discard, count):
+        """In place on a list of [heads, max_len, dim] f32 arrays."""
+        H, L, D = tensors[0].shape
+        self.lib.ref_kv_discard(self._ptrs(tensors), c_int(len(tensors)), c_int(H), c_int(L),
+                                c_int(D), c_int(keep), c_int(discard), c_int(count))
+
+    def kv_adjust_rope(self, tensors, keep, discard, count, inv_freq):
+        H, L, D = tensors[0].shape
+        f = np.ascontiguousarray(inv_freq, np.float32)
+        self.lib.ref_kv_adjust_rope(self._ptrs(tensors), c_int(len(tensors)), c_int(H), c_int(L),
+                                    c_int(D), c_int(keep), c_int(discard), c_int(count), _p(f))
+
+    def inverse_rope_freqs(self, theta, head_dim):
+        n = self.lib.ref_inverse_rope_freqs_count(c_float(theta), c_int(head_dim))
+        out = np.empty(n, np.float32)
+        self.lib.ref_inverse_rope_freqs(c_float(theta), c_int(head_dim), _p(out))
+        return out
+
+
+def load_reference_runtime():
+    return ReferenceRuntime() if REF_SO.exists() else None
