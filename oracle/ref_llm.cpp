@@ -6,7 +6,10 @@
  *   runtime/include/buddy/runtime/llm/KVCacheManager.h buddy::kvcache::discardKVCache,
  *                                                      adjustKeyCacheRope,
  *                                                      buildInverseRopeFreqs
- * Both need the C++ standard library only.  The result, oracle/_ref/libref_llm.so,
+ *   frontend/Interfaces/buddy/Core/Container.h         MemRef<T, N>, whose object
+ *                                                      layout is the descriptor the
+ *                                                      _mlir_ciface_* symbols receive
+ * All need the C++ standard library only.  The result, oracle/_ref/libref_llm.so,
  * is what the restated sampler and KV-cache functions of the oracle are checked
  * against.
  *
@@ -15,10 +18,45 @@
 #include <cstdint>
 #include <vector>
 
+#include <cstring>
+
+#include "buddy/Core/Container.h"
 #include "buddy/runtime/llm/KVCacheManager.h"
 #include "buddy/runtime/llm/Sampler.h"
 
+namespace {
+// Builds a MemRef<T, N> over `data` and copies the object's own bytes out: what
+// a callee that is handed `&memref` sees.  Returns sizeof(MemRef<T, N>).
+template <typename T, size_t N>
+int memref_bytes(const T *data, const int64_t *sizes, int64_t offset, void *out, int cap) {
+  intptr_t sz[N];
+  for (size_t i = 0; i < N; ++i)
+    sz[i] = (intptr_t)sizes[i];
+  MemRef<T, N> m(data, sz, (intptr_t)offset);
+  if ((int)sizeof(m) <= cap)
+    std::memcpy(out, static_cast<const void *>(&m), sizeof(m));
+  return (int)sizeof(m);
+}
+} // namespace
+
 extern "C" {
+
+// kind: 0 = float, 1 = int8, 2 = int64; the object's bytes of a MemRef built over
+// `data` with the given sizes and offset
+int ref_memref_object(int kind, int rank, const void *data, const int64_t *sizes, int64_t offset,
+                      void *out, int cap) {
+  switch (kind * 10 + rank) {
+  case 1: return memref_bytes<float, 1>((const float *)data, sizes, offset, out, cap);
+  case 2: return memref_bytes<float, 2>((const float *)data, sizes, offset, out, cap);
+  case 3: return memref_bytes<float, 3>((const float *)data, sizes, offset, out, cap);
+  case 4: return memref_bytes<float, 4>((const float *)data, sizes, offset, out, cap);
+  case 11: return memref_bytes<int8_t, 1>((const int8_t *)data, sizes, offset, out, cap);
+  case 12: return memref_bytes<int8_t, 2>((const int8_t *)data, sizes, offset, out, cap);
+  case 21: return memref_bytes<long long, 1>((const long long *)data, sizes, offset, out, cap);
+  case 22: return memref_bytes<long long, 2>((const long long *)data, sizes, offset, out, cap);
+  }
+  return -1;
+}
 
 void *ref_sampler_create(float temperature, int top_k, float top_p, float min_p,
                          float repeat_penalty, int repeat_last_n, uint64_t seed) {

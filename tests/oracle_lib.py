@@ -428,6 +428,15 @@ class ReferenceRuntime:
         self.lib.ref_kv_adjust_rope(self._ptrs(tensors), c_int(len(tensors)), c_int(H), c_int(L),
                                     c_int(D), c_int(keep), c_int(discard), c_int(count), _p(f))
 
+    def memref_object(self, kind, data, sizes, offset=0):
+        """Bytes of the reference's MemRef<T, N> object built over `data`
+        (kind 0 = f32, 1 = int8, 2 = int64)."""
+        sz = np.ascontiguousarray(sizes, np.int64)
+        buf = np.zeros(256, np.uint8)
+        n = self.lib.ref_memref_object(c_int(kind), c_int(sz.size), _p(data), _p(sz),
+                                       c_int64(offset), _p(buf), c_int(buf.size))
+        return n, buf
+
     def inverse_rope_freqs(self, theta, head_dim):
         n = self.lib.ref_inverse_rope_freqs_count(c_float(theta), c_int(head_dim))
         out = np.empty(n, np.float32)

@@ -1,5 +1,5 @@
-"""The restated sampler and KV-cache functions of the oracle against the
-reference's own code: runtime/include/buddy/runtime/llm/Sampler.h and
+"""The restated sampler and KV-cache functions of the oracle, and the memref
+descriptor of the C interface, against the reference's own code: runtime/include/buddy/runtime/llm/Sampler.h and
 KVCacheManager.h are header-only C++ that needs the standard library only, so
 `make -C oracle ref` compiles them from the reference tree into
 oracle/_ref/libref_llm.so (oracle/ref_llm.cpp is the C interface around them).
@@ -96,3 +96,32 @@ def test_inverse_frequencies_of_the_reference_are_the_models(oracle):
     i = np.arange(64, dtype=np.float64)
     np.testing.assert_allclose(f, 1.0 / 1e6 ** (2 * i / 128), rtol=3e-7)
     assert f[0] == 1.0 and f.dtype == np.float32
+
+
+@pytest.mark.parametrize("kind,ctype,dtype,rank", [
+    (0, "c_float", np.float32, 1), (0, "c_float", np.float32, 2), (0, "c_float", np.float32, 3),
+    (0, "c_float", np.float32, 4), (1, "c_int8", np.int8, 1), (1, "c_int8", np.int8, 2),
+    (2, "c_longlong", np.int64, 1), (2, "c_longlong", np.int64, 2)])
+def test_descriptor_structs_have_the_layout_of_the_reference_memref_object(kind, ctype, dtype,
+                                                                           rank):
+    """_mlir_ciface_* symbols are handed the address of a MemRef<T, N> object
+    (frontend/Interfaces/buddy/Core/Container.h:126-137): read through this
+    library's descriptor struct, the object of the reference's own class must
+    show its pointers, offset, sizes and row-major strides."""
+    import ctypes
+
+    import buddy_mlir_amd as bma
+
+    sizes = [3, 5, 2, 4][:rank]
+    data = np.arange(int(np.prod(sizes)), dtype=dtype)
+    n, raw = ref.memref_object(kind, data, sizes, offset=7)
+    T = bma.memref_type(getattr(ctypes, ctype), rank)
+    assert n == ctypes.sizeof(T) == 24 + 16 * rank
+    d = T.from_buffer_copy(raw[:n].tobytes())
+    alloc = ctypes.cast(d.allocated, ctypes.c_void_p).value
+    align = ctypes.cast(d.aligned, ctypes.c_void_p).value
+    assert alloc and alloc == align
+    assert d.offset == 7
+    assert list(d.sizes) == sizes
+    strides = [int(np.prod(sizes[i + 1:])) for i in range(rank)]
+    assert list(d.strides) == strides
