@@ -126,6 +126,7 @@ def _declare(lib):
         "buddy_hip_forward_invalidate_kv": (None, []),
         "buddy_hip_session_set_state": (c_int, [vp, c_int, c_int]),
         "buddy_hip_session_discard_kv": (c_int, [vp, c_int, c_int, c_int]),
+        "buddy_hip_session_discard_kv_freqs": (c_int, [vp, c_int, c_int, c_int, vp]),
         "buddy_hip_quantize_w4": (c_int, [vp, i64, i64, vp, vp, vp]),
         "buddy_hip_pack_int4": (c_int, [vp, i64, vp, vp]),
         "buddy_hip_gemv_w4a16": (c_int, [vp, vp, vp, vp, i64, i64, vp]),

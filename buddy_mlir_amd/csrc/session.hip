@@ -914,8 +914,8 @@ const float *buddy_hip_session_logits(buddy_hip_session *hs) {
   return s ? s->logits : nullptr;
 }
 
-int buddy_hip_session_discard_kv(buddy_hip_session *hs, int keep, int discard,
-                                 int count) {
+int buddy_hip_session_discard_kv_freqs(buddy_hip_session *hs, int keep, int discard,
+                                       int count, const float *inv_freq) {
   Session *s = reinterpret_cast<Session *>(hs);
   BH_REQUIRE(s, "session_discard_kv: null session");
   int rc = s->ready();
@@ -929,11 +929,16 @@ int buddy_hip_session_discard_kv(buddy_hip_session *hs, int keep, int discard,
   }
   rc = bh::launch_kv_discard(tensors.data(), (int)tensors.size(), S.kv_heads, S.max_len,
                              S.head_dim, keep, discard, count,
-                             s->inv_freq_host.data(), s->stream);
+                             inv_freq ? inv_freq : s->inv_freq_host.data(), s->stream);
   if (rc)
     return rc;
   BH_CHECK_HIP(hipStreamSynchronize(s->stream));
   return BUDDY_HIP_OK;
+}
+
+int buddy_hip_session_discard_kv(buddy_hip_session *hs, int keep, int discard,
+                                 int count) {
+  return buddy_hip_session_discard_kv_freqs(hs, keep, discard, count, nullptr);
 }
 
 int buddy_hip_session_vocab(buddy_hip_session *hs) {

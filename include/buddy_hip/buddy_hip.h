@@ -360,6 +360,12 @@ int buddy_hip_kv_discard(float *const *tensors, int num_tensors, int heads, int 
  * position count - discard. */
 int buddy_hip_session_discard_kv(buddy_hip_session *s, int keep, int discard,
                                  int count);
+/* The same with the caller's inverse frequencies (host, head_dim/2 floats): what
+ * ModelSession::handleKVCacheOverflow(keepTokenNum, ropeTheta) does with
+ * kvcache::buildInverseRopeFreqs(ropeTheta, head_dim)
+ * (tools/buddy-codegen/gen_session.py:1471-1511).  NULL: the session's own. */
+int buddy_hip_session_discard_kv_freqs(buddy_hip_session *s, int keep, int discard,
+                                       int count, const float *inv_freq);
 
 /* y[N] = bias[N] + x[K] . B[K,N] in f32 (bias may be NULL): the decode GEMV
  * of MatMulVectorizationDecode.cpp:142-175 followed by the q/k/v bias add. */
