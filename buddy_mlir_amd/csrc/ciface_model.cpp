@@ -230,6 +230,28 @@ struct DecodeResult {
 static_assert(sizeof(DecodeResult) == 40 + 2 * 88 + (kLayers - 1) * (40 + 2 * 88) + 72,
               "DecodeABI layout");
 
+// The result block of the hand-written example program for the same model
+// (examples/BuddyDeepSeekR1/buddy-deepseek-r1-w8a32-main.cpp:163-249) keeps the
+// 27 position copies together: [pos_out][kv0][kv1][dummy x 27][kv2 .. kv55]
+// [logits].  Same members, same size, another order; the caller says which one
+// it reads with BUDDY_HIP_DECODE_RESULT_LAYOUT=grouped in the environment.
+struct DecodeResultGrouped {
+  buddy_memref_i64_1d pos_out;
+  buddy_memref_f32_4d kv0, kv1;
+  buddy_memref_i64_1d dummy[kLayers - 1];
+  buddy_memref_f32_4d kv[2 * (kLayers - 1)];
+  buddy_memref_f32_3d logits;
+};
+static_assert(sizeof(DecodeResultGrouped) == sizeof(DecodeResult), "same members");
+
+bool grouped_result_layout() {
+  static const bool v = [] {
+    const char *e = getenv("BUDDY_HIP_DECODE_RESULT_LAYOUT");
+    return e && std::strcmp(e, "grouped") == 0;
+  }();
+  return v;
+}
+
 // PrefillABI (gen_session.py:908-911): [kv0 .. kv55][logits {1,max_len,V}]
 struct PrefillResult {
   buddy_memref_f32_4d kv[2 * kLayers];
@@ -272,24 +294,59 @@ int forward_decode(DecodeResult *res, buddy_memref_f32_1d *f32, buddy_memref_i8_
   float *logits = static_cast<float *>(malloc(sizeof(float) * (size_t)V));
   BH_REQUIRE(logits, "forward_decode: out of host memory");
   memcpy(logits, m.pinned_logits, sizeof(float) * (size_t)V);
-  // results: state tensors alias the caller's, logits are handed over
-  res->pos_out = *pos;
-  res->kv0 = *a.kv[0];
-  res->kv1 = *a.kv[1];
-  for (int i = 0; i < kLayers - 1; ++i) {
-    res->rest[i].dummy = *a.dummy[i];
-    res->rest[i].k = *a.kv[2 + 2 * i];
-    res->rest[i].v = *a.kv[3 + 2 * i];
+  // results: state tensors alias the caller's, logits are handed over.  The
+  // descriptors are read before any is written: the caller may pass members of
+  // the result block itself as arguments.
+  const buddy_memref_i64_1d pos_d = *pos;
+  buddy_memref_f32_4d kv_d[2 * kLayers];
+  buddy_memref_i64_1d dummy_d[kLayers - 1];
+  for (int i = 0; i < 2 * kLayers; ++i)
+    kv_d[i] = *a.kv[i];
+  for (int i = 0; i < kLayers - 1; ++i)
+    dummy_d[i] = *a.dummy[i];
+  buddy_memref_f32_3d *lg;
+  if (grouped_result_layout()) {
+    DecodeResultGrouped *g = reinterpret_cast<DecodeResultGrouped *>(res);
+    // that program owns every member of its result block and frees each at
+    // exit: the position comes back in a buffer of its own, not as an alias of
+    // the caller's cache_position tensor
+    long long *own = static_cast<long long *>(malloc(sizeof(long long)));
+    if (!own) {
+      free(logits);
+      return fail(BUDDY_HIP_ERR_ARG, "forward_decode: out of host memory");
+    }
+    *own = position;
+    g->pos_out = pos_d;
+    g->pos_out.allocated = own;
+    g->pos_out.aligned = own;
+    g->pos_out.offset = 0;
+    g->kv0 = kv_d[0];
+    g->kv1 = kv_d[1];
+    for (int i = 0; i < kLayers - 1; ++i)
+      g->dummy[i] = dummy_d[i];
+    for (int i = 0; i < 2 * (kLayers - 1); ++i)
+      g->kv[i] = kv_d[2 + i];
+    lg = &g->logits;
+  } else {
+    res->pos_out = pos_d;
+    res->kv0 = kv_d[0];
+    res->kv1 = kv_d[1];
+    for (int i = 0; i < kLayers - 1; ++i) {
+      res->rest[i].dummy = dummy_d[i];
+      res->rest[i].k = kv_d[2 + 2 * i];
+      res->rest[i].v = kv_d[3 + 2 * i];
+    }
+    lg = &res->logits;
   }
-  res->logits.allocated = logits;
-  res->logits.aligned = logits;
-  res->logits.offset = 0;
-  res->logits.sizes[0] = 1;
-  res->logits.sizes[1] = 1;
-  res->logits.sizes[2] = V;
-  res->logits.strides[0] = V;
-  res->logits.strides[1] = V;
-  res->logits.strides[2] = 1;
+  lg->allocated = logits;
+  lg->aligned = logits;
+  lg->offset = 0;
+  lg->sizes[0] = 1;
+  lg->sizes[1] = 1;
+  lg->sizes[2] = V;
+  lg->strides[0] = V;
+  lg->strides[1] = V;
+  lg->strides[2] = 1;
   return BUDDY_HIP_OK;
 }
 

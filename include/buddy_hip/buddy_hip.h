@@ -450,7 +450,14 @@ buddy_hip_session *buddy_hip_session_create_from_w8a32_blobs(
  * logits.  The device session is built on the first call and reused while the
  * blob addresses stay the same.  The KV cache is uploaded from the caller's
  * tensors on the first decode that no prefill preceded; call
- * buddy_hip_forward_invalidate_kv() after editing the host cache. */
+ * buddy_hip_forward_invalidate_kv() after editing the host cache.
+ * The hand-written program for the same model
+ * (examples/BuddyDeepSeekR1/buddy-deepseek-r1-w8a32-main.cpp:163-249) reads its
+ * decode results in another order -- position, kv0, kv1, the 27 position copies
+ * together, kv2..kv55, logits -- and frees every member at exit; with
+ * BUDDY_HIP_DECODE_RESULT_LAYOUT=grouped in the environment the block is written
+ * that way and the position comes back in a buffer of its own.  Arguments may
+ * be members of the result block itself (that program passes them so). */
 void _mlir_ciface_forward_prefill(void *result, buddy_memref_f32_1d *f32_params,
                                   buddy_memref_i8_1d *i8_params,
                                   buddy_memref_i64_2d *tokens);
