@@ -9,12 +9,12 @@
 //
 // The reference accumulates in f16, k in order: every step rounds to 11
 // significand bits, so a kernel that sums in another order (or in f32) does not
-// reproduce its results to 1e-3.  This kernel therefore keeps the reference's
-// order: a thread owns the two channels of one byte column and walks k, rounding
-// the f32 fused multiply-add to f16 after every step, which is exactly what f16
-// arithmetic is on the reference's x86 target.  The result equals the
-// reference's bit for bit; the price is that only N/2 threads stream the matrix
-// (its own layout is already coalesced for that: a row of bytes per k).
+// reproduce its results to 1e-3.  The kernels here therefore keep the reference's
+// order: one thread walks k for a channel, rounding the f32 fused multiply-add
+// to f16 after every step, which is exactly what f16 arithmetic is on the
+// reference's x86 target.  The result equals the reference's bit for bit; the
+// price is a chain of K dependent roundings per channel, so the launch time is
+// K times the time of one step, not the bytes it reads.
 #include "common.h"
 
 namespace bh {
@@ -88,71 +88,165 @@ w4a16_gemv_kernel(const u16 *__restrict__ a, const int8_t *__restrict__ packed,
   c[n + 1] = f32_to_f16_bits(f16_bits_to_f32(c[n + 1]) + s1);
 }
 
-// The same arithmetic for a full block of 64 byte columns whose rows can be read
-// as aligned 16-byte pieces.  One wavefront per block; the matrix strip
-// [K, 64 bytes] goes through LDS in blocks of kRows rows: the block after the one
-// being consumed is in flight in registers (kRows * 64 B = 32 KiB per
-// wavefront), which is what hides the memory latency when only N/128
-// wavefronts can work at all.
-constexpr int kRows = 512;                 // rows per block
-constexpr int kLoads = kRows * 64 / (64 * 16); // 16-byte loads per lane and block
+// The same arithmetic with the chain of dependent roundings as (nearly) the only
+// thing its wavefront does.  A workgroup owns 64 channels (32 byte columns).
+// Wavefront 0 walks k for them, one channel per lane: per step one LDS read of
+// its channel's weight (already f16) and one fused multiply-add that takes f16
+// operands and rounds its f32 result to f16 (v_fma_mixlo_f16: the reference's
+// step in one instruction); the activations come eight at a time.  Wavefronts
+// 1..3 prepare the block of rows after the one being consumed: a lane reads four
+// packed bytes of a row (a wavefront: eight whole rows of the block per load),
+// widens the eight nibbles to f16 and stores them as 16 contiguous bytes of the
+// row-major f16 block.  The bytes are requested a whole block ahead of their
+// decoding.  One barrier per block of rows.
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+constexpr int kChainRows = 256; // rows per block
+constexpr int kChainChannels = 64;
 
-__global__ void __launch_bounds__(kThreads)
-w4a16_gemv_block_kernel(const u16 *__restrict__ a, const int8_t *__restrict__ packed,
+__global__ void __launch_bounds__(256)
+w4a16_gemv_chain_kernel(const u16 *__restrict__ a, const int8_t *__restrict__ packed,
                         const u16 *__restrict__ scale, u16 *__restrict__ c, int K, int N) {
 #pragma clang fp contract(off)
-  __shared__ __attribute__((aligned(16))) unsigned char w_s[kRows * 64];
-  __shared__ float a_s[kRows];
+  __shared__ __attribute__((aligned(16))) _Float16 w_s[2][kChainRows * kChainChannels];
+  __shared__ __attribute__((aligned(16))) _Float16 x_s[2][kChainRows];
   const int cols = N / 2;
-  const int lane = threadIdx.x;
-  const int j = blockIdx.x * 64 + lane;
-  // lane L fetches 16 bytes of row (i * 16 + L / 4), columns (L % 4) * 16 ..
-  const int8_t *src = packed + (size_t)blockIdx.x * 64 + (lane & 3) * 16;
-  const int lrow = lane >> 2;
-  uint4 regs[kLoads];
-  auto fetch = [&](int k0) {
-#pragma unroll
-    for (int i = 0; i < kLoads; ++i) {
-      const int k = min(k0 + i * 16 + lrow, K - 1);
-      regs[i] = *reinterpret_cast<const uint4 *>(src + (size_t)k * cols);
-    }
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int col0 = blockIdx.x * (kChainChannels / 2);
+  const int nblocks = (K + kChainRows - 1) / kChainRows;
+
+  // producer lane: row (lane / 8) of a group of eight rows, bytes 4 (lane % 8) ..
+  // + 3 of the block's 32 byte columns = channels 8 (lane % 8) .. + 7.  Groups
+  // g = wave - 1, wave + 2, ... of the block's 32: at most 11 per wavefront.
+  constexpr int kTasks = (kChainRows / 8 + 2) / 3;
+  struct Raw {
+    int b[kTasks];
+    u16 x[kChainRows / 64];
   };
-  float acc0 = 0.f, acc1 = 0.f; // always exactly representable in f16
-  fetch(0);
-  for (int k0 = 0; k0 < K; k0 += kRows) {
-    const int kn = min(kRows, K - k0);
-    __syncthreads(); // the block before this one has been consumed
+  const int prow = lane >> 3, pcol = lane & 7;
+  // four bytes, read as bytes where the row is not 4-byte aligned
+  const bool aligned4 = ((reinterpret_cast<uintptr_t>(packed) | (unsigned)cols | (unsigned)col0) & 3) == 0;
+  auto request = [&](int blk, Raw &raw) {
+    const int k0 = blk * kChainRows;
 #pragma unroll
-    for (int i = 0; i < kLoads; ++i)
-      *reinterpret_cast<uint4 *>(w_s + (i * 16 + lrow) * 64 + (lane & 3) * 16) = regs[i];
-    for (int i = lane; i < kn; i += kThreads)
-      a_s[i] = f16_bits_to_f32(a[k0 + i]);
-    __syncthreads();
-    if (k0 + kRows < K)
-      fetch(k0 + kRows);
-    constexpr int U = 8;
-    for (int kk = 0; kk < kn; kk += U) {
-      int b[U];
-#pragma unroll
-      for (int u = 0; u < U; ++u)
-        b[u] = (signed char)w_s[min(kk + u, kn - 1) * 64 + lane];
-#pragma unroll
-      for (int u = 0; u < U; ++u) {
-        if (kk + u < kn) {
-          const float lo = (float)((int)((unsigned)b[u] << 28) >> 28);
-          const float hi = (float)((int)((unsigned)b[u] << 24) >> 28);
-          const float x = a_s[kk + u];
-          acc0 = round_to_f16(fmaf(x, lo, acc0));
-          acc1 = round_to_f16(fmaf(x, hi, acc1));
-        }
+    for (int t = 0; t < kTasks; ++t) {
+      const int g = min(wave - 1 + 3 * t, kChainRows / 8 - 1);
+      const int8_t *p = packed + (size_t)min(k0 + g * 8 + prow, K - 1) * cols + col0 + pcol * 4;
+      if (aligned4) {
+        raw.b[t] = *reinterpret_cast<const int *>(p);
+      } else {
+        raw.b[t] = (int)((unsigned)(unsigned char)p[0] | ((unsigned)(unsigned char)p[1] << 8) |
+                         ((unsigned)(unsigned char)p[2] << 16) |
+                         ((unsigned)(unsigned char)p[3] << 24));
       }
     }
+    if (wave == 1) {
+#pragma unroll
+      for (int i = 0; i < kChainRows / 64; ++i)
+        raw.x[i] = a[min(k0 + i * 64 + lane, K - 1)];
+    }
+  };
+  auto decode = [&](const Raw &raw, int buf) {
+#pragma unroll
+    for (int t = 0; t < kTasks; ++t) {
+      const int g = wave - 1 + 3 * t;
+      if (g < kChainRows / 8) {
+        half8 h;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) // nibble j: low nibble of a byte = the even channel
+          h[j] = (_Float16)(float)((int)((unsigned)raw.b[t] << (28 - 4 * j)) >> 28);
+        *reinterpret_cast<half8 *>(&w_s[buf][(g * 8 + prow) * kChainChannels + pcol * 8]) = h;
+      }
+    }
+    if (wave == 1) {
+#pragma unroll
+      for (int i = 0; i < kChainRows / 64; ++i) {
+        union {
+          u16 u;
+          _Float16 f;
+        } v;
+        v.u = raw.x[i];
+        x_s[buf][i * 64 + lane] = v.f;
+      }
+    }
+  };
+
+  _Float16 acc = (_Float16)0.0f;
+  Raw raw0, raw1; // block blk + 1 being decoded, block blk + 2 in flight (they swap)
+  if (wave != 0) {
+    request(0, raw0);
+    decode(raw0, 0);
+    request(1, raw0);
   }
-  const int n = 2 * j;
-  const float s0 = round_to_f16(acc0 * f16_bits_to_f32(scale[n]));
-  const float s1 = round_to_f16(acc1 * f16_bits_to_f32(scale[n + 1]));
-  c[n] = f32_to_f16_bits(f16_bits_to_f32(c[n]) + s0);
-  c[n + 1] = f32_to_f16_bits(f16_bits_to_f32(c[n + 1]) + s1);
+  __syncthreads();
+  for (int blk = 0; blk < nblocks; ++blk) {
+    const int buf = blk & 1;
+    if (wave != 0) {
+      // (a request past the last block rereads clamped rows: always the same
+      // number of loads, so that waiting for the older set leaves the newer in flight)
+      if (buf == 0) {
+        request(blk + 2, raw1);
+        if (blk + 1 < nblocks)
+          decode(raw0, 1);
+      } else {
+        request(blk + 2, raw0);
+        if (blk + 1 < nblocks)
+          decode(raw1, 0);
+      }
+    } else {
+      const int kn = min(kChainRows, K - blk * kChainRows);
+      const _Float16 *wcol = &w_s[buf][lane];
+      int kk = 0;
+      // 16 steps per batch; the operands of the next batch are read from LDS
+      // while the chain of this one runs (the read latency is several steps long)
+      if (kn >= 16) {
+        half8 x0 = *reinterpret_cast<const half8 *>(&x_s[buf][0]);
+        half8 x1 = *reinterpret_cast<const half8 *>(&x_s[buf][8]);
+        _Float16 w[16];
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+          w[r] = wcol[r * kChainChannels];
+        for (; kk + 16 <= kn; kk += 16) {
+          const int nk = kk + 32 <= kn ? kk + 16 : kk; // after the last batch: reread it
+          const half8 y0 = *reinterpret_cast<const half8 *>(&x_s[buf][nk]);
+          const half8 y1 = *reinterpret_cast<const half8 *>(&x_s[buf][nk + 8]);
+          _Float16 v[16];
+#pragma unroll
+          for (int r = 0; r < 16; ++r)
+            v[r] = wcol[(nk + r) * kChainChannels];
+#pragma unroll
+          for (int r = 0; r < 8; ++r)
+            acc = (_Float16)fmaf((float)x0[r], (float)w[r], (float)acc);
+#pragma unroll
+          for (int r = 0; r < 8; ++r)
+            acc = (_Float16)fmaf((float)x1[r], (float)w[8 + r], (float)acc);
+          x0 = y0;
+          x1 = y1;
+#pragma unroll
+          for (int r = 0; r < 16; ++r)
+            w[r] = v[r];
+        }
+      }
+      for (; kk + 8 <= kn; kk += 8) {
+        const half8 x = *reinterpret_cast<const half8 *>(&x_s[buf][kk]);
+        _Float16 w[8];
+#pragma unroll
+        for (int r = 0; r < 8; ++r)
+          w[r] = wcol[(kk + r) * kChainChannels];
+#pragma unroll
+        for (int r = 0; r < 8; ++r)
+          acc = (_Float16)fmaf((float)x[r], (float)w[r], (float)acc);
+      }
+      for (; kk < kn; ++kk)
+        acc = (_Float16)fmaf((float)x_s[buf][kk], (float)wcol[kk * kChainChannels], (float)acc);
+    }
+    __syncthreads();
+  }
+  if (wave != 0)
+    return;
+  const int n = 2 * col0 + lane;
+  const float s = round_to_f16((float)acc * f16_bits_to_f32(scale[n]));
+  c[n] = f32_to_f16_bits(f16_bits_to_f32(c[n]) + s);
 }
 
 // two int4 (stored as int8 in [-8, 7]) per byte, element 2i low, 2i+1 high
@@ -190,13 +284,12 @@ int buddy_hip_gemv_w4a16(const uint16_t *A, const int8_t *packed, const uint16_t
   // full blocks of 64 byte columns with 16-byte readable rows take the blocked
   // kernel, the ragged rest (or everything, if rows are not aligned) the plain one
   const int64_t cols = N / 2;
-  int64_t blocked = 0;
-  if (cols % 16 == 0 && (reinterpret_cast<uintptr_t>(packed) & 15) == 0)
-    blocked = cols / 64 * 64;
+  // whole blocks of 32 byte columns take the kernel whose chain wavefront does
+  // nothing but the chain; the ragged rest the plain one
+  const int64_t blocked = cols / 32 * 32;
   if (blocked) {
-    hipLaunchKernelGGL(bh::w4a16_gemv_block_kernel, dim3((unsigned)(blocked / 64)),
-                       dim3(bh::kThreads), 0, bh::as_stream(stream), A, packed, scale, C,
-                       (int)K, (int)N);
+    hipLaunchKernelGGL(bh::w4a16_gemv_chain_kernel, dim3((unsigned)(blocked / 32)), dim3(256), 0,
+                       bh::as_stream(stream), A, packed, scale, C, (int)K, (int)N);
   }
   if (blocked < cols) {
     hipLaunchKernelGGL(bh::w4a16_gemv_kernel,

@@ -15,7 +15,8 @@ def dev(a):
     return torch.from_numpy(np.ascontiguousarray(a)).cuda()
 
 
-@pytest.mark.parametrize("K,N", [(64, 16), (1536, 8960), (8960, 1536), (100, 70), (1, 2), (3000, 130)])
+@pytest.mark.parametrize("K,N", [(64, 16), (1536, 8960), (8960, 1536), (100, 70), (1, 2), (3000, 130),
+                                 (17, 64), (263, 128), (511, 192), (256, 64), (272, 66)])
 def test_quantize_pack_gemv_bit_exact(bh, oracle, K, N):
     g = torch.Generator(device="cuda").manual_seed(K * 7 + N)
     W = torch.randn((K, N), generator=g, device="cuda") * 0.02
