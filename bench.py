@@ -332,7 +332,35 @@ def bench_kvdiscard(bh, args):
     t = _time_launches(fn, 50, warm=3)
     tail = count - keep - discard
     by = n * heads * D * 4 * (2 * tail + (L - keep - tail))  # read + write tail, clear rest
-    return {
+    # the same on the host: the reference's own discardKVCache + adjustKeyCacheRope
+    # (KVCacheManager.h compiled as oracle/_ref) where that build exists, else the
+    # restatement
+    cpu = None
+    if not args.no_cpu_baseline:
+        import time
+
+        sys.path.insert(0, str(ROOT / "tests"))
+        import oracle_lib
+
+        host = [x.cpu().numpy() for x in tensors]
+        ref = oracle_lib.load_reference_runtime()
+        reps = 5
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            if ref is not None:
+                ref.kv_discard(host, keep, discard, count)
+                ref.kv_adjust_rope(host, keep, discard, count, f)
+            else:
+                o = oracle_lib.load()
+                for j in range(n):
+                    _, host[j] = o.kv_discard(host[j], keep, discard, count)
+                    if j % 2 == 0:
+                        host[j] = o.kv_adjust_rope(host[j], keep, discard, count, f)
+        t_cpu = (time.perf_counter() - t0) / reps
+        cpu = {"value": by / t_cpu / 1e9, "unit": "GB/s", "cores": 1,
+               "kind": "reference" if ref is not None else "port",
+               "sample": f"{reps} calls on 56 host tensors [2,1088,128], {t_cpu * 1e3:.2f} ms each"}
+    out = {
         "metric": "kv_discard_hbm_gbps", "value": by / t / 1e9, "unit": "GB/s",
         "n_gpus": 1, "steps": 50, "warmup": 3, "ms_per_step": t * 1e3,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
@@ -345,6 +373,9 @@ def bench_kvdiscard(bh, args):
                      "algorithmic_bytes_per_launch": by, "avg_launch_us": t * 1e6,
                      "traffic": None},
     }
+    if cpu:
+        out["cpu_baseline"] = cpu
+    return out
 
 
 def bench_sampler(bh, args):
