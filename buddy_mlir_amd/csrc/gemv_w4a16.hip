@@ -90,15 +90,20 @@ w4a16_gemv_kernel(const u16 *__restrict__ a, const int8_t *__restrict__ packed,
 
 // The same arithmetic with the chain of dependent roundings as (nearly) the only
 // thing its wavefront does.  A workgroup owns 64 channels (32 byte columns).
-// Wavefront 0 walks k for them, one channel per lane: per step one LDS read of
-// its channel's weight (already f16) and one fused multiply-add that takes f16
-// operands and rounds its f32 result to f16 (v_fma_mixlo_f16: the reference's
-// step in one instruction); the activations come eight at a time.  Wavefronts
-// 1..3 prepare the block of rows after the one being consumed: a lane reads four
-// packed bytes of a row (a wavefront: eight whole rows of the block per load),
-// widens the eight nibbles to f16 and stores them as 16 contiguous bytes of the
-// row-major f16 block.  The bytes are requested a whole block ahead of their
-// decoding.  One barrier per block of rows.
+// Wavefront 0 walks k for them, one channel per lane.  A step is one
+// v_fma_mixlo_f16: f16 operands taken from either half of a register, f32
+// multiply-add, one rounding to f16 -- the reference's step as one instruction.
+// Its operands: the activations of a whole block of 256 rows sit in registers
+// (read from LDS once per block, the same for every lane), and one LDS read
+// brings the lane's weights of two consecutive rows, already widened to f16;
+// the reads for the next 16 steps are issued before the chain of these 16.
+// Wavefronts 1..3 prepare the block of rows after the one being consumed: a lane
+// reads four packed bytes of each of two consecutive rows (a wavefront: 16 whole
+// rows of the block per pair of loads), widens the 16 nibbles to f16 and stores
+// them as 32 contiguous bytes of the block, laid out [row pair][channel][2].  The
+// bytes are requested a whole block ahead of their decoding.  One barrier per
+// block of rows.
+typedef _Float16 half2v __attribute__((ext_vector_type(2)));
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 constexpr int kChainRows = 256; // rows per block
 constexpr int kChainChannels = 64;
@@ -107,7 +112,8 @@ __global__ void __launch_bounds__(256)
 w4a16_gemv_chain_kernel(const u16 *__restrict__ a, const int8_t *__restrict__ packed,
                         const u16 *__restrict__ scale, u16 *__restrict__ c, int K, int N) {
 #pragma clang fp contract(off)
-  __shared__ __attribute__((aligned(16))) _Float16 w_s[2][kChainRows * kChainChannels];
+  // [row pair][channel] of (even row, odd row)
+  __shared__ __attribute__((aligned(16))) half2v w_s[2][kChainRows / 2 * kChainChannels];
   __shared__ __attribute__((aligned(16))) _Float16 x_s[2][kChainRows];
   const int cols = N / 2;
   const int tid = threadIdx.x, lane = tid & 63;
@@ -115,29 +121,35 @@ w4a16_gemv_chain_kernel(const u16 *__restrict__ a, const int8_t *__restrict__ pa
   const int col0 = blockIdx.x * (kChainChannels / 2);
   const int nblocks = (K + kChainRows - 1) / kChainRows;
 
-  // producer lane: row (lane / 8) of a group of eight rows, bytes 4 (lane % 8) ..
+  // producer lane: row pair (lane / 8) of a group of 16 rows, bytes 4 (lane % 8) ..
   // + 3 of the block's 32 byte columns = channels 8 (lane % 8) .. + 7.  Groups
-  // g = wave - 1, wave + 2, ... of the block's 32: at most 11 per wavefront.
-  constexpr int kTasks = (kChainRows / 8 + 2) / 3;
+  // g = wave - 1, wave + 2, ... of the block's 16: at most 6 per wavefront.
+  constexpr int kGroups = kChainRows / 16;
+  constexpr int kTasks = (kGroups + 2) / 3;
   struct Raw {
-    int b[kTasks];
+    int b[kTasks][2];
     u16 x[kChainRows / 64];
   };
-  const int prow = lane >> 3, pcol = lane & 7;
-  // four bytes, read as bytes where the row is not 4-byte aligned
-  const bool aligned4 = ((reinterpret_cast<uintptr_t>(packed) | (unsigned)cols | (unsigned)col0) & 3) == 0;
+  const int ppair = lane >> 3, pcol = lane & 7;
+  // four bytes at once where rows are 4-byte aligned, byte by byte otherwise
+  const bool aligned4 =
+      ((reinterpret_cast<uintptr_t>(packed) | (unsigned)cols | (unsigned)col0) & 3) == 0;
   auto request = [&](int blk, Raw &raw) {
     const int k0 = blk * kChainRows;
 #pragma unroll
     for (int t = 0; t < kTasks; ++t) {
-      const int g = min(wave - 1 + 3 * t, kChainRows / 8 - 1);
-      const int8_t *p = packed + (size_t)min(k0 + g * 8 + prow, K - 1) * cols + col0 + pcol * 4;
-      if (aligned4) {
-        raw.b[t] = *reinterpret_cast<const int *>(p);
-      } else {
-        raw.b[t] = (int)((unsigned)(unsigned char)p[0] | ((unsigned)(unsigned char)p[1] << 8) |
-                         ((unsigned)(unsigned char)p[2] << 16) |
-                         ((unsigned)(unsigned char)p[3] << 24));
+      const int g = min(wave - 1 + 3 * t, kGroups - 1);
+#pragma unroll
+      for (int e = 0; e < 2; ++e) {
+        const int8_t *p =
+            packed + (size_t)min(k0 + g * 16 + ppair * 2 + e, K - 1) * cols + col0 + pcol * 4;
+        if (aligned4) {
+          raw.b[t][e] = *reinterpret_cast<const int *>(p);
+        } else {
+          raw.b[t][e] =
+              (int)((unsigned)(unsigned char)p[0] | ((unsigned)(unsigned char)p[1] << 8) |
+                    ((unsigned)(unsigned char)p[2] << 16) | ((unsigned)(unsigned char)p[3] << 24));
+        }
       }
     }
     if (wave == 1) {
@@ -150,12 +162,19 @@ w4a16_gemv_chain_kernel(const u16 *__restrict__ a, const int8_t *__restrict__ pa
 #pragma unroll
     for (int t = 0; t < kTasks; ++t) {
       const int g = wave - 1 + 3 * t;
-      if (g < kChainRows / 8) {
-        half8 h;
+      if (g < kGroups) {
+        half8 h[2]; // channels 8 pcol .. + 3 and + 4 .. + 7, (even row, odd row) each
 #pragma unroll
-        for (int j = 0; j < 8; ++j) // nibble j: low nibble of a byte = the even channel
-          h[j] = (_Float16)(float)((int)((unsigned)raw.b[t] << (28 - 4 * j)) >> 28);
-        *reinterpret_cast<half8 *>(&w_s[buf][(g * 8 + prow) * kChainChannels + pcol * 8]) = h;
+        for (int j = 0; j < 8; ++j) { // nibble j: low nibble of a byte = the even channel
+          h[j / 4][2 * (j % 4)] =
+              (_Float16)(short)((int)((unsigned)raw.b[t][0] << (28 - 4 * j)) >> 28);
+          h[j / 4][2 * (j % 4) + 1] =
+              (_Float16)(short)((int)((unsigned)raw.b[t][1] << (28 - 4 * j)) >> 28);
+        }
+        half8 *dst = reinterpret_cast<half8 *>(
+            &w_s[buf][(g * 8 + ppair) * kChainChannels + pcol * 8]);
+        dst[0] = h[0];
+        dst[1] = h[1];
       }
     }
     if (wave == 1) {
@@ -195,50 +214,45 @@ w4a16_gemv_chain_kernel(const u16 *__restrict__ a, const int8_t *__restrict__ pa
       }
     } else {
       const int kn = min(kChainRows, K - blk * kChainRows);
-      const _Float16 *wcol = &w_s[buf][lane];
-      int kk = 0;
-      // 16 steps per batch; the operands of the next batch are read from LDS
-      // while the chain of this one runs (the read latency is several steps long)
-      if (kn >= 16) {
-        half8 x0 = *reinterpret_cast<const half8 *>(&x_s[buf][0]);
-        half8 x1 = *reinterpret_cast<const half8 *>(&x_s[buf][8]);
-        _Float16 w[16];
+      const half2v *wcol = &w_s[buf][lane];
+      // the block's activations: 32 reads, the same address in every lane
+      half8 x[kChainRows / 8];
 #pragma unroll
-        for (int r = 0; r < 16; ++r)
+      for (int q = 0; q < kChainRows / 8; ++q)
+        x[q] = *reinterpret_cast<const half8 *>(&x_s[buf][q * 8]);
+      // keep them in registers: left alone, the compiler reads each one again
+      // from LDS right before its use and the chain waits for that read
+#pragma unroll
+      for (int q = 0; q < kChainRows / 8; ++q)
+        asm volatile("" : "+v"(x[q]));
+      if (kn == kChainRows) {
+        half2v w[8];
+#pragma unroll
+        for (int r = 0; r < 8; ++r)
           w[r] = wcol[r * kChainChannels];
-        for (; kk + 16 <= kn; kk += 16) {
-          const int nk = kk + 32 <= kn ? kk + 16 : kk; // after the last batch: reread it
-          const half8 y0 = *reinterpret_cast<const half8 *>(&x_s[buf][nk]);
-          const half8 y1 = *reinterpret_cast<const half8 *>(&x_s[buf][nk + 8]);
-          _Float16 v[16];
 #pragma unroll
-          for (int r = 0; r < 16; ++r)
-            v[r] = wcol[(nk + r) * kChainChannels];
+        for (int q = 0; q < kChainRows / 16; ++q) { // 16 steps
+          half2v v[8];
+          const int nq = q + 1 < kChainRows / 16 ? q + 1 : q; // after the last: reread it
 #pragma unroll
           for (int r = 0; r < 8; ++r)
-            acc = (_Float16)fmaf((float)x0[r], (float)w[r], (float)acc);
+            v[r] = wcol[(nq * 8 + r) * kChainChannels];
+#pragma unroll
+          for (int r = 0; r < 8; ++r) {
+            acc = (_Float16)fmaf((float)x[2 * q + r / 4][2 * (r % 4)], (float)w[r][0], (float)acc);
+            acc = (_Float16)fmaf((float)x[2 * q + r / 4][2 * (r % 4) + 1], (float)w[r][1],
+                                 (float)acc);
+          }
 #pragma unroll
           for (int r = 0; r < 8; ++r)
-            acc = (_Float16)fmaf((float)x1[r], (float)w[8 + r], (float)acc);
-          x0 = y0;
-          x1 = y1;
-#pragma unroll
-          for (int r = 0; r < 16; ++r)
             w[r] = v[r];
         }
+      } else { // the ragged last block
+        for (int kk = 0; kk < kn; ++kk) {
+          const half2v w = wcol[(kk >> 1) * kChainChannels];
+          acc = (_Float16)fmaf((float)x_s[buf][kk], (float)w[kk & 1], (float)acc);
+        }
       }
-      for (; kk + 8 <= kn; kk += 8) {
-        const half8 x = *reinterpret_cast<const half8 *>(&x_s[buf][kk]);
-        _Float16 w[8];
-#pragma unroll
-        for (int r = 0; r < 8; ++r)
-          w[r] = wcol[(kk + r) * kChainChannels];
-#pragma unroll
-        for (int r = 0; r < 8; ++r)
-          acc = (_Float16)fmaf((float)x[r], (float)w[r], (float)acc);
-      }
-      for (; kk < kn; ++kk)
-        acc = (_Float16)fmaf((float)x_s[buf][kk], (float)wcol[kk * kChainChannels], (float)acc);
     }
     __syncthreads();
   }
