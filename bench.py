@@ -3,7 +3,7 @@
 MI355X, next to the CPU oracle timed on the same host.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W]
-    python bench.py --workload gemv|mlp|prefill|llama8b|kvdiscard|w4a16|model_abi|sampler   (the other configurations)
+    python bench.py --workload gemv|mlp|prefill|llama8b|kvdiscard|w4a16|model_abi|sampler|quantize   (the other configurations)
 
 A step is one greedy decode step (one token) at batch 1 with the KV cache
 already holding 1024 positions; weights, KV cache and activations are resident
@@ -378,6 +378,72 @@ def bench_kvdiscard(bh, args):
     return out
 
 
+def bench_quantize(bh, args):
+    """The import-time pair: per-output-channel int8 quantisation of an f32
+    matrix (amax pass + quantise pass) and the repacking of the int8 matrix into
+    wave tiles, at the gate/up shape.  CPU figure: the restated quantiser."""
+    import time
+
+    import torch
+
+    from buddy_mlir_amd import ops
+
+    K, N = 1536, 8960
+    ws = [torch.randn((K, N), device="cuda") * 0.02 for _ in range(8)]
+    qs = [ops.quantize_w8(w)[0] for w in ws]
+    # outputs allocated once: the loop times the kernels, not the allocator
+    q_out = torch.empty((K, N), dtype=torch.int8, device="cuda")
+    s_out = torch.empty((N,), dtype=torch.float32, device="cuda")
+    p_out = torch.empty_like(ops.pack_w8(qs[0]))
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def quantize(i):
+        if bh.buddy_hip_quantize_w8(ws[i % 8].data_ptr(), K, N, q_out.data_ptr(),
+                                    s_out.data_ptr(), stream):
+            raise RuntimeError("quantize_w8 failed")
+
+    def pack(i):
+        if bh.buddy_hip_pack_w8(qs[i % 8].data_ptr(), K, N, p_out.data_ptr(), stream):
+            raise RuntimeError("pack_w8 failed")
+
+    tq = _time_launches(quantize, 40, warm=3)
+    tp = _time_launches(pack, 40, warm=3)
+    by_q, by_p = 9 * K * N, 2 * K * N  # f32 read twice + int8 write; int8 read + write
+    out = {
+        "metric": "quantize_hbm_gbps", "value": by_q / tq / 1e9, "unit": "GB/s",
+        "n_gpus": 1, "steps": 40, "warmup": 3, "ms_per_step": tq * 1e3,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32->int8",
+        "data": "synthetic",
+        "config": {"workload": "per-channel int8 quantisation of f32 W[1536,8960], and its "
+                               "wave-tile packing"},
+        "detail": {"quantize": {"us": tq * 1e6, "gbps": by_q / tq / 1e9,
+                                "frac": by_q / tq / 1e9 / HBM_PEAK_GBPS},
+                   "pack": {"us": tp * 1e6, "gbps": by_p / tp / 1e9,
+                            "frac": by_p / tp / 1e9 / HBM_PEAK_GBPS}},
+        "roofline": {"kernel": "colwise_absmax + finalize_scale + quantize", "bound": "hbm",
+                     "achieved": by_q / tq / 1e9, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": by_q / tq / 1e9 / HBM_PEAK_GBPS,
+                     "algorithmic_bytes_per_launch": by_q, "avg_launch_us": tq * 1e6,
+                     "traffic": None},
+    }
+    if not args.no_cpu_baseline:
+        sys.path.insert(0, str(ROOT / "tests"))
+        import oracle_lib
+
+        o = oracle_lib.load()
+        wh = ws[0].cpu().numpy()
+        t0 = time.perf_counter()
+        reps = 5
+        for _ in range(reps):
+            o.quantize_w8(wh)
+        t_cpu = (time.perf_counter() - t0) / reps
+        out["cpu_baseline"] = {"value": by_q / t_cpu / 1e9, "unit": "GB/s",
+                               "cores": o.num_threads(), "kind": "port",
+                               "sample": f"{reps} calls of the restated quantiser on the same "
+                                         f"matrix, {t_cpu * 1e3:.1f} ms each"}
+    return out
+
+
 def bench_sampler(bh, args):
     """One sampled token from device logits of the Qwen2 vocabulary: penalty,
     temperature and top-40 on the device, the rest on the host.  The CPU figure
@@ -622,7 +688,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=8)
     ap.add_argument("--workload", default="decode",
                     choices=["decode", "gemv", "mlp", "prefill", "llama8b", "kvdiscard", "w4a16",
-                             "model_abi", "sampler"],
+                             "model_abi", "sampler", "quantize"],
                     help="decode (default): the full decode step the headline metric "
                          "is quoted on; the others measure the remaining configurations")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -648,7 +714,8 @@ def main():
     if args.workload != "decode":
         fn = {"gemv": bench_gemv, "mlp": bench_mlp, "prefill": bench_prefill,
               "llama8b": bench_llama8b, "kvdiscard": bench_kvdiscard, "w4a16": bench_w4a16,
-              "model_abi": bench_model_abi, "sampler": bench_sampler}[args.workload]
+              "model_abi": bench_model_abi, "sampler": bench_sampler,
+              "quantize": bench_quantize}[args.workload]
         print(json.dumps(fn(bh, args)))
         return
     K, W = args.steps, args.warmup

@@ -25,6 +25,42 @@ colwise_absmax_kernel(const float *__restrict__ W, int64_t K, int64_t N,
   atomicMax(&amax_bits[n], __float_as_uint(m));
 }
 
+// The same for four adjacent columns per thread (N a multiple of 4, W 16-byte
+// aligned): 16-byte loads, four times the bytes in flight.
+__global__ void __launch_bounds__(256)
+colwise_absmax4_kernel(const float *__restrict__ W, int64_t K, int64_t N,
+                       int64_t rows_per_block, unsigned *__restrict__ amax_bits) {
+  const int64_t n = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * 4;
+  if (n >= N)
+    return;
+  const int64_t k0 = (int64_t)blockIdx.y * rows_per_block;
+  const int64_t k1 = k0 + rows_per_block < K ? k0 + rows_per_block : K;
+  float m0 = 0.f, m1 = 0.f, m2 = 0.f, m3 = 0.f;
+  const float *p = W + k0 * N + n;
+  int64_t k = k0;
+  for (; k + 4 <= k1; k += 4, p += 4 * N) { // four rows requested together
+    const float4 a = *reinterpret_cast<const float4 *>(p);
+    const float4 b = *reinterpret_cast<const float4 *>(p + N);
+    const float4 c = *reinterpret_cast<const float4 *>(p + 2 * N);
+    const float4 d = *reinterpret_cast<const float4 *>(p + 3 * N);
+    m0 = fmaxf(fmaxf(m0, fabsf(a.x)), fmaxf(fabsf(b.x), fmaxf(fabsf(c.x), fabsf(d.x))));
+    m1 = fmaxf(fmaxf(m1, fabsf(a.y)), fmaxf(fabsf(b.y), fmaxf(fabsf(c.y), fabsf(d.y))));
+    m2 = fmaxf(fmaxf(m2, fabsf(a.z)), fmaxf(fabsf(b.z), fmaxf(fabsf(c.z), fabsf(d.z))));
+    m3 = fmaxf(fmaxf(m3, fabsf(a.w)), fmaxf(fabsf(b.w), fmaxf(fabsf(c.w), fabsf(d.w))));
+  }
+  for (; k < k1; ++k, p += N) {
+    const float4 a = *reinterpret_cast<const float4 *>(p);
+    m0 = fmaxf(m0, fabsf(a.x));
+    m1 = fmaxf(m1, fabsf(a.y));
+    m2 = fmaxf(m2, fabsf(a.z));
+    m3 = fmaxf(m3, fabsf(a.w));
+  }
+  atomicMax(&amax_bits[n], __float_as_uint(m0));
+  atomicMax(&amax_bits[n + 1], __float_as_uint(m1));
+  atomicMax(&amax_bits[n + 2], __float_as_uint(m2));
+  atomicMax(&amax_bits[n + 3], __float_as_uint(m3));
+}
+
 // scale = (amax / 127).clamp(min=1e-10)      (import_model.py:838,875)
 __global__ void __launch_bounds__(256)
 finalize_scale_kernel(float *__restrict__ scale, int64_t N, float qmax) {
@@ -49,6 +85,29 @@ quantize_kernel(const float *__restrict__ W, const float *__restrict__ scale,
   float r = rintf(W[i] / scale[n]);
   r = fminf(fmaxf(r, lo), hi);
   q[i] = (int8_t)r;
+}
+
+// The same for four adjacent elements of a row per thread (N a multiple of 4, W
+// 16-byte and q 4-byte aligned); blockIdx.y is the row.
+__global__ void __launch_bounds__(256)
+quantize4_kernel(const float *__restrict__ W, const float *__restrict__ scale, int64_t N,
+                 int8_t *__restrict__ q, float lo, float hi) {
+  const int64_t n = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * 4;
+  if (n >= N)
+    return;
+  const int64_t row = blockIdx.y;
+  const float4 w = *reinterpret_cast<const float4 *>(W + row * N + n);
+  const float4 s = *reinterpret_cast<const float4 *>(scale + n);
+  const float r0 = fminf(fmaxf(rintf(w.x / s.x), lo), hi);
+  const float r1 = fminf(fmaxf(rintf(w.y / s.y), lo), hi);
+  const float r2 = fminf(fmaxf(rintf(w.z / s.z), lo), hi);
+  const float r3 = fminf(fmaxf(rintf(w.w / s.w), lo), hi);
+  char4 out;
+  out.x = (signed char)r0;
+  out.y = (signed char)r1;
+  out.z = (signed char)r2;
+  out.w = (signed char)r3;
+  *reinterpret_cast<char4 *>(q + row * N + n) = out;
 }
 
 // One thread writes one lane's 16 bytes of one tile.
@@ -155,17 +214,31 @@ static int quantize_per_channel(const float *W, int64_t K, int64_t N, int8_t *q,
   hipStream_t st = bh::as_stream(stream);
   BH_CHECK_HIP(hipMemsetAsync(scale, 0, sizeof(float) * (size_t)N, st));
   const int64_t rows = 64;
-  hipLaunchKernelGGL(bh::colwise_absmax_kernel,
-                     dim3((unsigned)bh::ceil_div(N, 256),
-                          (unsigned)bh::ceil_div(K, rows)),
-                     dim3(256), 0, st, W, K, N, rows,
-                     reinterpret_cast<unsigned *>(scale));
+  // four columns per thread where rows can be read as aligned 16-byte pieces
+  const bool vec = N % 4 == 0 && K <= 65535 &&
+                   ((reinterpret_cast<uintptr_t>(W) | reinterpret_cast<uintptr_t>(scale)) & 15) == 0 &&
+                   (reinterpret_cast<uintptr_t>(q) & 3) == 0;
+  if (vec) {
+    hipLaunchKernelGGL(bh::colwise_absmax4_kernel,
+                       dim3((unsigned)bh::ceil_div(N / 4, 256), (unsigned)bh::ceil_div(K, rows)),
+                       dim3(256), 0, st, W, K, N, rows, reinterpret_cast<unsigned *>(scale));
+  } else {
+    hipLaunchKernelGGL(bh::colwise_absmax_kernel,
+                       dim3((unsigned)bh::ceil_div(N, 256), (unsigned)bh::ceil_div(K, rows)),
+                       dim3(256), 0, st, W, K, N, rows, reinterpret_cast<unsigned *>(scale));
+  }
   hipLaunchKernelGGL(bh::finalize_scale_kernel,
                      dim3((unsigned)bh::ceil_div(N, 256)), dim3(256), 0, st,
                      scale, N, qmax);
-  hipLaunchKernelGGL(bh::quantize_kernel,
-                     dim3((unsigned)bh::ceil_div(K * N, 256)), dim3(256), 0, st,
-                     W, scale, K, N, q, lo, hi);
+  if (vec) {
+    hipLaunchKernelGGL(bh::quantize4_kernel,
+                       dim3((unsigned)bh::ceil_div(N / 4, 256), (unsigned)K), dim3(256), 0, st, W,
+                       scale, N, q, lo, hi);
+  } else {
+    hipLaunchKernelGGL(bh::quantize_kernel,
+                       dim3((unsigned)bh::ceil_div(K * N, 256)), dim3(256), 0, st,
+                       W, scale, K, N, q, lo, hi);
+  }
   BH_CHECK_HIP(hipGetLastError());
   return BUDDY_HIP_OK;
 }

@@ -21,7 +21,8 @@ def make_weight(K, N, seed):
     return torch.randn((K, N), generator=g, device="cuda") * 0.02
 
 
-@pytest.mark.parametrize("K,N", [(64, 16), (1536, 8960), (8960, 1536), (100, 70), (1, 1)])
+@pytest.mark.parametrize("K,N", [(64, 16), (1536, 8960), (8960, 1536), (100, 70), (1, 1),
+                                 (131, 68), (3, 4), (70000, 8)])
 def test_quantizer_bit_exact(oracle, K, N):
     W = make_weight(K, N, K * 7 + N)
     if K > 3 and N > 2:
