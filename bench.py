@@ -195,6 +195,49 @@ def bench_gemv(bh, args):
         t = _time_launches(fn, 960)
         res[name] = {"us": t * 1e6, "gbps": by / t / 1e9, "frac": by / t / 1e9 / HBM_PEAK_GBPS}
         del sets
+    # the same shape through the other GEMV kernels of the path, weights rotated
+    # over HBM-cold copies: int8 activations with exact int32 sums (w8a8), and the
+    # f32 GEMV in row-major and in the reference's packed-panel layout
+    packed = _random_packed(K, N, 24)
+    wscale = torch.full((N,), 1e-3, device="cuda")
+    ws_bytes = bh.buddy_hip_w8a8_workspace_bytes(1, K)
+    ws = torch.empty((ws_bytes,), dtype=torch.int8, device="cuda")
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def w8a8(i):
+        if bh.buddy_hip_w8a8_matmul(x.data_ptr(), packed[i % 24].data_ptr(), wscale.data_ptr(),
+                                    y.data_ptr(), None, 1, K, N, ws.data_ptr(), ws_bytes, stream):
+            raise RuntimeError("w8a8_matmul failed")
+    t8 = _time_launches(w8a8, 240)
+    by8 = K * N + 4 * N + 4 * (K + N)
+    res["w8a8_int32_sums"] = {"us": t8 * 1e6, "gbps": by8 / t8 / 1e9,
+                              "frac": by8 / t8 / 1e9 / HBM_PEAK_GBPS,
+                              "note": "two launches: activation quantisation, then the GEMV"}
+    del packed
+    Bf = [torch.randn((K, N), device="cuda") for _ in range(12)]  # 660 MB of f32
+    byf = 4 * K * N + 4 * (K + N)
+
+    def f32_plain(i):
+        if bh.buddy_hip_gemv_f32(x.data_ptr(), Bf[i % 12].data_ptr(), None, y.data_ptr(), K, N,
+                                 0, stream):
+            raise RuntimeError("gemv_f32 failed")
+    tf = _time_launches(f32_plain, 240)
+    res["f32_row_major"] = {"us": tf * 1e6, "gbps": byf / tf / 1e9,
+                            "frac": byf / tf / 1e9 / HBM_PEAK_GBPS}
+    Pf = [torch.empty_like(b) for b in Bf]
+    for b_, p_ in zip(Bf, Pf):
+        if bh.buddy_hip_pack_panels_f32(b_.data_ptr(), K, N, 32, p_.data_ptr(), stream):
+            raise RuntimeError("pack_panels_f32 failed")
+    del Bf
+
+    def f32_panels(i):
+        if bh.buddy_hip_gemv_f32_panels(x.data_ptr(), Pf[i % 12].data_ptr(), y.data_ptr(), K, N,
+                                        0, stream):
+            raise RuntimeError("gemv_f32_panels failed")
+    tp = _time_launches(f32_panels, 240)
+    res["f32_reference_panels"] = {"us": tp * 1e6, "gbps": byf / tp / 1e9,
+                                   "frac": byf / tp / 1e9 / HBM_PEAK_GBPS}
+    del Pf
     t = res["hbm_cold"]["us"] * 1e-6
     return {
         "metric": "int8_gemv_hbm_gbps", "value": res["hbm_cold"]["gbps"], "unit": "GB/s",
