@@ -8,13 +8,16 @@
 // build the q/k/v projections are this kernel followed by a bias add
 // (examples/BuddyDeepSeekR1/subgraph0_decode_simplify.mlir:73-85).
 //
-// B is row-major with N contiguous.  The matrix is narrow for this chip (2048
-// columns at the q|k|v shape) and a sum over k must stay inside a workgroup (no
-// cross-workgroup reduction: it would cost an L2 write-back), so a workgroup
-// owns only 16 columns -- one 64-byte piece of every row -- and all of K: 128
-// workgroups at N = 2048.  A wavefront load reads 16 rows x 64 bytes (4 lanes of
-// float4 per row); the 8 wavefronts take interleaved 16-row blocks, all their
-// loads in flight at once, and meet in LDS in a fixed order.
+// B is row-major with N contiguous.  A sum over k must stay inside a workgroup
+// (no cross-workgroup reduction: it would cost an L2 write-back), so a workgroup
+// owns a strip of columns and all of K.  The q|k|v shape is narrow for this chip
+// (2048 columns): there a strip is 16 columns -- one 64-byte piece of every row,
+// 128 workgroups -- and a wavefront load reads 16 rows x 64 bytes (4 lanes of
+// float4 per row).  From 4096 columns on the strip is 32 columns, from 8192 on 64
+// (256-byte pieces, 4 rows per load): longer pieces of a row per request are worth
+// more than more workgroups once there are 128 of them (29.9 -> 15.5 us at
+// 1536 x 8960).  The 8 wavefronts take interleaved row blocks, all their loads in
+// flight at once, and meet in LDS in a fixed order.
 // RMSNorm can be fused in like in the int8 kernel: the norm weight multiplies x
 // as it is used, the sum of squares is gathered on the way (by the lanes of
 // column group 0 only, so every k counts once) and the rsqrt factor multiplies
@@ -25,25 +28,33 @@ namespace bh {
 namespace {
 
 constexpr int kWaves = 8;
-constexpr int kCols = 16;          // columns per workgroup
-constexpr int kRowsPerLoad = 16;   // rows per wavefront load
 constexpr int kUnroll = 6;         // loads in flight per lane
 
+// kCols = columns per workgroup: 16 (64-byte pieces of a row, the most workgroups)
+// for narrow matrices, 32 or 64 (longer pieces, fewer and larger requests per row)
+// once that still gives every compute unit a workgroup.
+template <int kCols>
 __global__ void __launch_bounds__(kWaves * 64)
 gemv_f32_kernel(const float *__restrict__ x, const float *__restrict__ B,
                 const float *__restrict__ bias, const float *__restrict__ norm_w,
                 float norm_eps, float norm_inv_k, float *__restrict__ y, int K, int N,
-                int64_t ldb, int accumulate) {
+                int64_t ldb, int64_t block_stride, int accumulate) {
+  // block_stride != 0: the columns of workgroup b are a matrix of their own, kCols
+  // wide, at B + b * block_stride (the reference's panel-packed layout)
   __shared__ float red[kWaves][kCols + 1];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int c4 = lane & 3, rsub = lane >> 2; // float4 column group, row in a load
+  constexpr int kLanesPerRow = kCols / 4;        // float4 lanes across a row piece
+  constexpr int kRowsPerLoad = 64 / kLanesPerRow; // rows per wavefront load
+  const int c4 = lane % kLanesPerRow, rsub = lane / kLanesPerRow;
   const int col = blockIdx.x * kCols + c4 * 4;
+  const int bcol = block_stride ? c4 * 4 : col;
+  B += (int64_t)blockIdx.x * block_stride;
   const bool full = blockIdx.x * kCols + kCols <= N && ((ldb & 3) == 0) &&
                     ((reinterpret_cast<uintptr_t>(B) & 15) == 0);
   float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
   float ss = 0.f;
-  // row blocks wave, wave + kWaves, ... of 16 rows each, kUnroll at a time
+  // row blocks wave, wave + kWaves, ... of kRowsPerLoad rows each, kUnroll at a time
   for (int kb = wave * kRowsPerLoad; kb < K; kb += kWaves * kRowsPerLoad * kUnroll) {
     float4 b[kUnroll];
     float xv[kUnroll], nw[kUnroll];
@@ -51,7 +62,7 @@ gemv_f32_kernel(const float *__restrict__ x, const float *__restrict__ B,
     for (int u = 0; u < kUnroll; ++u) {
       const int k = kb + u * kWaves * kRowsPerLoad + rsub;
       const int kc = min(k, K - 1); // rows past the end repeat the last, times zero
-      const float *row = B + (int64_t)kc * ldb + col;
+      const float *row = B + (int64_t)kc * ldb + bcol;
       if (full)
         b[u] = *reinterpret_cast<const float4 *>(row);
       else
@@ -71,16 +82,16 @@ gemv_f32_kernel(const float *__restrict__ x, const float *__restrict__ B,
       acc.w = fmaf(xs, b[u].w, acc.w);
     }
   }
-  // the 16 row lanes of a column group hold different k: lanes 4 apart ... 32 apart
+  // the row lanes of a column group hold different k: lanes kLanesPerRow apart ... 32 apart
 #pragma unroll
-  for (int o = 4; o < 64; o <<= 1) {
+  for (int o = kLanesPerRow; o < 64; o <<= 1) {
     acc.x += __shfl_xor(acc.x, o, 64);
     acc.y += __shfl_xor(acc.y, o, 64);
     acc.z += __shfl_xor(acc.z, o, 64);
     acc.w += __shfl_xor(acc.w, o, 64);
     ss += __shfl_xor(ss, o, 64);
   }
-  if (lane < 4) {
+  if (lane < kLanesPerRow) {
     red[wave][lane * 4 + 0] = acc.x;
     red[wave][lane * 4 + 1] = acc.y;
     red[wave][lane * 4 + 2] = acc.z;
@@ -220,9 +231,32 @@ int launch_gemv_f32_norm(const float *x, const float *B, const float *bias,
   BH_REQUIRE(K > 0 && N > 0 && K < (1 << 30) && N < (1 << 30) && ldb >= N,
              "gemv_f32: bad shape K=%lld N=%lld ldb=%lld", (long long)K,
              (long long)N, (long long)ldb);
-  hipLaunchKernelGGL(gemv_f32_kernel, dim3((unsigned)ceil_div(N, kCols)),
-                     dim3(kWaves * 64), 0, stream, x, B, bias, norm_w, norm_eps,
-                     1.0f / (float)K, y, (int)K, (int)N, ldb, accumulate ? 1 : 0);
+  const int cols = N >= 64 * 128 ? 64 : N >= 32 * 128 ? 32 : 16;
+#define BH_LAUNCH_F32(C)                                                                  \
+  hipLaunchKernelGGL(gemv_f32_kernel<C>, dim3((unsigned)ceil_div(N, C)), dim3(kWaves * 64), \
+                     0, stream, x, B, bias, norm_w, norm_eps, 1.0f / (float)K, y, (int)K,  \
+                     (int)N, ldb, (int64_t)0, accumulate ? 1 : 0)
+  if (cols == 64)
+    BH_LAUNCH_F32(64);
+  else if (cols == 32)
+    BH_LAUNCH_F32(32);
+  else
+    BH_LAUNCH_F32(16);
+#undef BH_LAUNCH_F32
+  BH_CHECK_HIP(hipGetLastError());
+  return BUDDY_HIP_OK;
+}
+
+int launch_gemv_f32_panels32(const float *x, const float *packed, float *y, int64_t K,
+                             int64_t N, bool accumulate, hipStream_t stream) {
+  BH_REQUIRE(x && packed && y, "gemv_f32_panels: null pointer");
+  BH_REQUIRE(K > 0 && N > 0 && K < (1 << 30) && N < (1 << 30) && N % 32 == 0,
+             "gemv_f32_panels: K=%lld N=%lld (N must be a multiple of 32)", (long long)K,
+             (long long)N);
+  hipLaunchKernelGGL(gemv_f32_kernel<32>, dim3((unsigned)(N / 32)), dim3(kWaves * 64), 0,
+                     stream, x, packed, (const float *)nullptr, (const float *)nullptr, 0.f,
+                     1.0f / (float)K, y, (int)K, (int)N, (int64_t)32, K * 32,
+                     accumulate ? 1 : 0);
   BH_CHECK_HIP(hipGetLastError());
   return BUDDY_HIP_OK;
 }

@@ -7,11 +7,14 @@
 // and MatMulVectorizationDecodePackedPattern (midend/lib/Conversion/
 // MatMulOptimization/MatMulVectorizationDecodePacked.cpp:207-248) walks one
 // panel per task with linear offset n0*K + k*V.  A weight file written in that
-// order can be consumed as is: one workgroup per panel, 32 lanes across v
-// (128 contiguous bytes per row), 8 rows in flight per load, rows met in LDS.
+// order can be consumed as is: a panel is a row-major [K, 32] matrix of its own,
+// so one workgroup per panel runs the row-major f32 GEMV kernel on it (8 float4
+// lanes across v, a wavefront load = 8 rows = 1 KiB of contiguous panel).
 #include "common.h"
 
 namespace bh {
+int launch_gemv_f32_panels32(const float *x, const float *packed, float *y, int64_t K,
+                             int64_t N, bool accumulate, hipStream_t stream);
 namespace {
 
 __global__ void __launch_bounds__(256)
@@ -26,28 +29,6 @@ pack_panels_kernel(const float *__restrict__ B, float *__restrict__ P, int64_t K
     P[i] = B[packed]; // B holds the panels, P the plain matrix
   else
     P[packed] = B[i];
-}
-
-__global__ void __launch_bounds__(256)
-gemv_panels_kernel(const float *__restrict__ x, const float *__restrict__ flatB,
-                   float *__restrict__ y, int K, int N, int zero_init) {
-  constexpr int V = 32;
-  __shared__ float red[8][V];
-  const int v = threadIdx.x & 31, kg = threadIdx.x >> 5;
-  const int64_t n0 = (int64_t)blockIdx.x * V;
-  const float *panel = flatB + n0 * K;
-  float acc = 0.f;
-  for (int k = kg; k < K; k += 8)
-    acc = fmaf(x[k], panel[(int64_t)k * V + v], acc);
-  red[kg][v] = acc;
-  __syncthreads();
-  if (kg == 0) {
-    float s = zero_init ? 0.f : y[n0 + v];
-#pragma unroll
-    for (int g = 0; g < 8; ++g)
-      s += red[g][v];
-    y[n0 + v] = s;
-  }
 }
 
 } // namespace
@@ -79,14 +60,8 @@ int buddy_hip_unpack_panels_f32(const float *packed, int64_t K, int64_t N, int V
 int buddy_hip_gemv_f32_panels(const float *x, const float *packed, float *y,
                               int64_t K, int64_t N, unsigned flags,
                               buddy_hip_stream stream) {
-  BH_REQUIRE(x && packed && y, "gemv_f32_panels: null pointer");
-  BH_REQUIRE(K > 0 && N > 0 && K < (1 << 30) && N < (1 << 30) && N % 32 == 0,
-             "gemv_f32_panels: K=%lld N=%lld (N must be a multiple of 32)",
-             (long long)K, (long long)N);
-  hipLaunchKernelGGL(bh::gemv_panels_kernel, dim3((unsigned)(N / 32)), dim3(256), 0,
-                     bh::as_stream(stream), x, packed, y, (int)K, (int)N,
-                     (flags & BUDDY_HIP_GEMV_ACCUMULATE) ? 0 : 1);
-  BH_CHECK_HIP(hipGetLastError());
-  return BUDDY_HIP_OK;
+  return bh::launch_gemv_f32_panels32(x, packed, y, K, N,
+                                      (flags & BUDDY_HIP_GEMV_ACCUMULATE) != 0,
+                                      bh::as_stream(stream));
 }
 }
