@@ -19,7 +19,10 @@ def sync_check(rc):
     torch.cuda.synchronize()
 
 
-@pytest.mark.parametrize("K,N", [(1536, 1536), (1536, 256), (128, 64), (100, 70), (8960, 1536)])
+# 4096 columns and more take 32-column strips, 8192 and more 64-column strips;
+# 4099 and 8197 leave a ragged last strip and rows that are not 16-byte aligned
+@pytest.mark.parametrize("K,N", [(1536, 1536), (1536, 256), (128, 64), (100, 70), (8960, 1536),
+                                 (1536, 4096), (300, 4099), (1536, 8960), (77, 8197)])
 def test_f32_gemv_with_bias(bh, oracle, K, N):
     g = torch.Generator(device="cuda").manual_seed(K + N)
     x = torch.randn(K, generator=g, device="cuda")
