@@ -38,7 +38,7 @@ COMMON = [
 # load is issued: if it spilled one of those registers it would store garbage
 # and hand the register to something else while the load is still in flight.
 # Their kernels must therefore use no scratch at all; the build checks it.
-NO_SCRATCH = {"gemm_w8_mfma.hip", "gemv_w8a32_mfma.hip", "gemm_w8_i8.hip",
+NO_SCRATCH = {"gemm_w8_mfma.hip", "gemv_w8a32_mfma.hip", "gemv_w8a32_i8.hip", "gemm_w8_i8.hip",
               "attn_prefill.hip"}
 
 

@@ -40,7 +40,10 @@ struct GemvArgs {
 };
 
 int launch_gemv(const GemvArgs &a, hipStream_t stream);
-// Matrix-core variant for 5..16 rows (chosen by launch_gemv).
+// Matrix-core variants for 5..16 rows (chosen by launch_gemv): int8 matrix
+// instructions over fixed-point activations (the default), or bf16 ones over
+// three bf16 terms of every activation (every f32 bit; BUDDY_HIP_GEMV_BATCH=bf16).
+int launch_gemv_i8(const GemvArgs &a, hipStream_t stream);
 int launch_gemv_mfma(const GemvArgs &a, hipStream_t stream);
 
 } // namespace bh

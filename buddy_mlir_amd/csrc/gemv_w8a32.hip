@@ -29,6 +29,7 @@
 #include "gemv_w8a32.h"
 
 #include <cstdlib>
+#include <cstring>
 
 namespace bh {
 namespace {
@@ -907,6 +908,13 @@ int launch_m(const GemvArgs &a, const KernelArgs &ka, const GemvPlan &p,
   return fail(BUDDY_HIP_ERR_ARG, "gemv: unknown epilogue %d", a.epilogue);
 }
 
+// BUDDY_HIP_GEMV_BATCH=bf16 sends batches of 5..16 rows to the bf16 matrix-core
+// kernel (three bf16 terms per activation: every f32 bit) instead of the int8
+// one.  Read at every call, so a host can switch between calls.
+bool batch_bf16() {
+  const char *e = getenv("BUDDY_HIP_GEMV_BATCH");
+  return e && strcmp(e, "bf16") == 0;
+}
 bool force_valu() {
   static bool v = getenv("BUDDY_HIP_GEMV_FORCE_VALU") != nullptr;
   return v;
@@ -936,14 +944,15 @@ int launch_gemv(const GemvArgs &a, hipStream_t stream) {
              "gemv: packed weights must be 16-byte aligned");
   BH_REQUIRE(!a.norm_w || (reinterpret_cast<uintptr_t>(a.norm_w) & 15) == 0,
              "gemv: norm weight must be 16-byte aligned");
-  // batches of 5..16 rows go to the matrix cores when the activations can be
-  // read as aligned 16-byte pieces; up to four rows the f32 FMA kernel (1 + M
-  // instructions per weight) is quicker, and it takes whatever is unaligned
+  // batches of 5..16 rows go to the matrix cores (int8 ones by default) when the
+  // activations can be read as aligned 16-byte pieces; up to four rows the f32
+  // FMA kernel (1 + M instructions per weight) is quicker, and it takes whatever
+  // is unaligned
   if (a.M >= 5 && !a.attn_acc && !force_valu() && a.tile_n == 16 && a.K >= 4 &&
       (a.K & 3) == 0 && (a.lda & 3) == 0 &&
       (reinterpret_cast<uintptr_t>(a.A) & 15) == 0 &&
       (!a.norm_w || (reinterpret_cast<uintptr_t>(a.norm_w) & 15) == 0))
-    return launch_gemv_mfma(a, stream);
+    return batch_bf16() ? launch_gemv_mfma(a, stream) : launch_gemv_i8(a, stream);
   // the kernel is compiled for 1, 2, 4, 8 and 16 rows; extra rows are zero-
   // filled in LDS and never stored
   const int mt = compiled_rows(a.M);

@@ -1,0 +1,485 @@
+// gemv_w8a32_i8.hip -- the int8 dequant matmul for small batches (5..16 rows) on
+// the int8 matrix cores.
+//
+// The reference has no kernel of its own for 1 < M <= 16 (its decode patterns
+// fire for m == 1 only, DequantMatMulVectorizationDecode.cpp:212-217; the BLIS
+// kernel of MatMulBlisVectorization.cpp:398-986 is the one vectorised kernel for
+// M > 1).  Here the weights stream exactly as in the one-row kernel, from the same
+// packed copy, and go into v_mfma_i32_16x16x64_i8 as they lie: a lane's 16 bytes
+// of a 16-channel x 64-k tile are that instruction's operand, so the loop spends
+// no instruction on a weight.  The f32 activations become fixed point for it, 64
+// k at a time:
+//   * a wavefront reads its 16 rows x 64 k of activations from L2 as whole
+//     256-byte row pieces (four rows per load instruction) and turns them through
+//     a private 4 KiB of LDS into operand order: lane l holds x[row l % 16][16
+//     consecutive k].  (Reading them in operand order directly makes every load
+//     instruction touch 64 cache lines; that, not the weight stream, then bounds
+//     the kernel.)
+//   * the four lanes of a row find the largest magnitude of the row's 64 values
+//     and from it a power-of-two step s with |x| / s < 2^22;
+//   * X = rint(x / s) is cut into three balanced int8 digits, X = d0 + 256 d1 +
+//     65536 d2 (the bytes of X + 0x8080, the lower two with their top bit
+//     flipped), and a byte transpose puts each digit plane into operand order;
+//   * three matrix instructions per tile give exact int32 sums r0, r1, r2, and
+//     acc += s * (r0 + 256 r1 + 65536 r2) in f32.
+// The only rounding of a product is that of X: at most 2^-23 of the largest of
+// the 64 activations it is summed with -- what an f32 sum of the same terms does
+// when it adds the largest one.  A row whose chunk holds a NaN or an infinity
+// gets a NaN step and with it NaN results, so non-finite activations still show.
+//   * A wavefront converts a chunk once and uses it for SPAN channel groups.
+//   * k-slices of a workgroup meet in LDS in slice order.
+//   * RMSNorm can be fused in: the norm weight multiplies the activation before
+//     it is converted, each lane gathers the squares of what it loads, and the
+//     row's rsqrt factor multiplies the finished sums.
+#include "gemv_w8a32.h"
+
+namespace bh {
+namespace {
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef int v4i __attribute__((ext_vector_type(4)));
+
+constexpr int kMaxWavesI8 = 8; // 512 threads: up to 256 registers per lane
+
+struct I8Args {
+  const float *A;
+  const int4 *W0, *W1;
+  const float *s0, *s1, *bias, *norm_w;
+  float *C;
+  int64_t lda, ldc;
+  float norm_eps, norm_inv_k;
+  int K, N, groups, chunks, spans; // spans = ceil(groups / SPAN)
+  int GS, KS;                      // spans x k-slices of wavefronts per workgroup
+  int rows;
+};
+
+__device__ __forceinline__ float silu(float g) {
+  const float sig = 1.0f / (1.0f + expf(-g));
+  return g * sig;
+}
+
+// Largest magnitude of 16 values as a bit pattern (sign dropped).  Integer
+// comparisons, so that a NaN (the largest patterns of all) is not lost: the
+// signed maximum finds the largest positive value, the unsigned one the
+// largest-magnitude negative value if there is any.
+__device__ __forceinline__ unsigned max_magnitude_bits(const float (&v)[16]) {
+  int hi = __float_as_int(v[0]);
+  unsigned lo = __float_as_uint(v[0]);
+#pragma unroll
+  for (int e = 1; e < 16; ++e) {
+    hi = max(hi, __float_as_int(v[e]));
+    lo = max(lo, __float_as_uint(v[e]));
+  }
+  const unsigned pos = hi < 0 ? 0u : (unsigned)hi;
+  const unsigned neg = (lo & 0x80000000u) ? (lo & 0x7fffffffu) : 0u;
+  return max(pos, neg);
+}
+
+// 16 values of one row -> this lane's operand of each of the three digit planes.
+__device__ __forceinline__ void to_digits(const float (&x)[16], float inv, v4i (&d)[3]) {
+  // x * inv + 1.5 * 2^23 is rounded to an integer by the addition itself and
+  // leaves 0x4B400000 + X in the word
+  constexpr float kMagic = 12582912.0f;
+  constexpr int kBias = 0x8080 - 0x4B400000;
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    unsigned y[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+      y[e] = (unsigned)(__float_as_int(fmaf(x[4 * q + e], inv, kMagic)) + kBias);
+    // 4 x 4 byte transpose, three rows of it
+    const unsigned ta = __builtin_amdgcn_perm(y[1], y[0], 0x05010400u);
+    const unsigned tb = __builtin_amdgcn_perm(y[3], y[2], 0x05010400u);
+    const unsigned tc = __builtin_amdgcn_perm(y[1], y[0], 0x00000602u);
+    const unsigned td = __builtin_amdgcn_perm(y[3], y[2], 0x00000602u);
+    d[0][q] = (int)(__builtin_amdgcn_perm(tb, ta, 0x05040100u) ^ 0x80808080u);
+    d[1][q] = (int)(__builtin_amdgcn_perm(tb, ta, 0x07060302u) ^ 0x80808080u);
+    d[2][q] = (int)__builtin_amdgcn_perm(td, tc, 0x05040100u);
+  }
+}
+
+// acc += step * (r0 + 256 r1 + 65536 r2); step65536 = 65536 * step
+__device__ __forceinline__ void combine(f32x4 &acc, const v4i &r0, const v4i &r1,
+                                        const v4i &r2, float step, float step65536) {
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int u = r0[i] + (r1[i] << 8); // |r0| <= 2^20, |r1| <= 2^20: exact
+    acc[i] = fmaf((float)r2[i], step65536, fmaf((float)u, step, acc[i]));
+  }
+}
+
+// The loads of the main loop are issued and waited for by hand: the compiler
+// sinks ordinary prefetch loads down to their first use and then waits for them
+// there.  A fetch is a fixed number of loads in a fixed order, vmcnt counts them
+// in order, and each wait names the registers it releases so that nothing reads
+// them earlier.
+__device__ __forceinline__ void issue_load(v4i &dst, const void *p) {
+  asm volatile("global_load_dwordx4 %0, %1, off nt" : "=v"(dst) : "v"(p) : "memory");
+}
+__device__ __forceinline__ void issue_load(f32x4 &dst, const void *p) {
+  asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(dst) : "v"(p) : "memory");
+}
+
+template <int SPAN, bool DUAL, bool NORM> struct FetchRegs {
+  v4i w0[SPAN];
+  v4i w1[DUAL ? SPAN : 1];
+  f32x4 x[4]; // k kcol .. kcol+3 of rows lane/16, 4 + lane/16, 8 + lane/16, 12 + lane/16
+  f32x4 nw[NORM ? 4 : 1];
+};
+template <int SPAN, bool DUAL, bool NORM> constexpr int fetch_loads() {
+  return SPAN * (DUAL ? 2 : 1) + 4 * (NORM ? 2 : 1);
+}
+// Fetches kept in flight: as many as fit in about 64 registers (the kernel stays
+// within 128, so that a compute unit holds 16 wavefronts), two at least.
+template <int SPAN, bool DUAL, bool NORM> constexpr int ring_depth() {
+  constexpr int regs = 4 * SPAN * (DUAL ? 2 : 1) + 16 * (NORM ? 2 : 1);
+  return 64 / regs < 2 ? 2 : 64 / regs;
+}
+
+template <int SPAN, bool DUAL, bool NORM>
+__device__ __forceinline__ void fetch_chunk(const I8Args &a, const int4 *w0, const int4 *w1,
+                                            const size_t (&gofs)[SPAN],
+                                            const float *const (&xrow)[4], int kcol,
+                                            int kofs, int c, bool real,
+                                            FetchRegs<SPAN, DUAL, NORM> &o) {
+  // a fetch past the end of the slice (issued only to keep the load counts
+  // fixed, never used) reads the first tile of the matrix, which stays in cache:
+  // a streaming load of a tile of its own would go to HBM again
+#pragma unroll
+  for (int s = 0; s < SPAN; ++s) {
+    const size_t ofs = real ? gofs[s] + (size_t)c * 64 : (size_t)0;
+    issue_load(o.w0[s], w0 + ofs);
+    if (DUAL)
+      issue_load(o.w1[DUAL ? s : 0], w1 + ofs);
+  }
+  // activations: load q takes 256 bytes of each of rows 4q .. 4q+3 (this lane:
+  // four k of one of them); clamped inside the row, what lies past the end of a
+  // ragged row is zeroed when it is consumed (K is a multiple of four)
+  const int kx = min(c * kTileK + kcol, a.K - 4);
+#pragma unroll
+  for (int q = 0; q < 4; ++q)
+    issue_load(o.x[q], xrow[q] + kx);
+  if (NORM) { // norm weights in operand order: 16 consecutive k, the same for all rows
+    const int k = c * kTileK + kofs;
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+      issue_load(o.nw[NORM ? q : 0], a.norm_w + min(k + 4 * q, a.K - 4));
+  }
+}
+
+// Waits until at most N loads are in flight; the registers of `f` are valid only
+// after it.
+template <int N, int SPAN, bool DUAL, bool NORM>
+__device__ __forceinline__ void wait_fetch(FetchRegs<SPAN, DUAL, NORM> &f) {
+  asm volatile("s_waitcnt vmcnt(%4)"
+               : "+v"(f.x[0]), "+v"(f.x[1]), "+v"(f.x[2]), "+v"(f.x[3])
+               : "n"(N)
+               : "memory");
+#pragma unroll
+  for (int s = 0; s < SPAN; ++s) {
+    asm volatile("" : "+v"(f.w0[s])::"memory");
+    if (DUAL)
+      asm volatile("" : "+v"(f.w1[DUAL ? s : 0])::"memory");
+  }
+  if (NORM) {
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+      asm volatile("" : "+v"(f.nw[NORM ? q : 0])::"memory");
+  }
+}
+
+constexpr int kTurnStride = 68;               // floats between rows of the turning area
+constexpr int kTurnFloats = 16 * kTurnStride; // per wavefront
+
+template <int EPI, int SPAN, bool NORM>
+__global__ void __launch_bounds__(kMaxWavesI8 *kWave, 2)
+    gemv_w8a32_i8_kernel(I8Args a) {
+  constexpr bool DUAL = (EPI == kEpiSiluMul);
+  constexpr int NA = DUAL ? 2 * SPAN : SPAN; // accumulators per lane
+  extern __shared__ __attribute__((aligned(16))) float red[];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int sl = wave / a.KS, ks = wave % a.KS;
+  const int span = blockIdx.x * a.GS + sl;
+  const bool live = span < a.spans;
+  const int g0 = (live ? span : 0) * SPAN;
+  const int per = (a.chunks + a.KS - 1) / a.KS;
+  const int c0 = min(ks * per, a.chunks), c1 = min(c0 + per, a.chunks);
+  const int m = lane & 15, kg = lane >> 4;
+
+  f32x4 acc0[SPAN], acc1[DUAL ? SPAN : 1];
+#pragma unroll
+  for (int s = 0; s < SPAN; ++s) {
+    acc0[s] = f32x4{0.f, 0.f, 0.f, 0.f};
+    if (DUAL)
+      acc1[DUAL ? s : 0] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+  float ss = 0.f;
+  // groups past the end of the matrix repeat the last one (never stored)
+  size_t gofs[SPAN];
+#pragma unroll
+  for (int s = 0; s < SPAN; ++s)
+    gofs[s] = (size_t)min(g0 + s, a.groups - 1) * a.chunks * 64;
+  const int4 *w0 = a.W0 + lane;
+  const int4 *w1 = (DUAL ? a.W1 : a.W0) + lane;
+  const float *xrow[4]; // rows past the batch repeat its last row (never stored)
+#pragma unroll
+  for (int q = 0; q < 4; ++q)
+    xrow[q] = a.A + (int64_t)min(4 * q + kg, a.rows - 1) * a.lda;
+  const int kcol = (lane & 15) * 4, kofs = kg * 16;
+  // this wavefront's 16 x 64 activations on their way into operand order; rows
+  // are 68 floats apart so that the 16 lanes of an operand read hit 64 banks
+  float *xt = red + (size_t)wave * kTurnFloats;
+  float *meet = red + (size_t)(a.GS * a.KS) * kTurnFloats;
+
+  constexpr int L = fetch_loads<SPAN, DUAL, NORM>();
+  constexpr int R = ring_depth<SPAN, DUAL, NORM>(); // fetches in flight
+  FetchRegs<SPAN, DUAL, NORM> ring[R];
+  // every fetch is exactly L loads, also one past the end of the slice, which
+  // keeps the counts exact
+  const int clast = max(c1 - 1, 0);
+#pragma unroll
+  for (int u = 0; u < R; ++u)
+    fetch_chunk<SPAN, DUAL, NORM>(a, w0, w1, gofs, xrow, kcol, kofs, min(c0 + u, clast),
+                                  c0 + u < c1, ring[u]);
+  const bool ragged = (a.K & (kTileK - 1)) != 0;
+  const v4i zero = v4i{0, 0, 0, 0};
+  for (int cb = c0; cb < c1; cb += R) {
+#pragma unroll
+    for (int u = 0; u < R; ++u) {
+      const int c = cb + u;
+      if (c >= c1)
+        continue;
+      FetchRegs<SPAN, DUAL, NORM> &cur = ring[u];
+      wait_fetch<(R - 1) * L, SPAN, DUAL, NORM>(cur); // chunk c has arrived
+      // rows 4q + kg, k kcol..kcol+3  ->  row m, k kofs..kofs+15
+      if (ragged && c == a.chunks - 1) { // only the last chunk of a ragged row has a tail
+        const bool past = c * kTileK + kcol >= a.K;
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+          *reinterpret_cast<f32x4 *>(xt + (4 * q + kg) * kTurnStride + kcol) =
+              past ? f32x4{0.f, 0.f, 0.f, 0.f} : cur.x[q];
+      } else {
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+          *reinterpret_cast<f32x4 *>(xt + (4 * q + kg) * kTurnStride + kcol) = cur.x[q];
+      }
+      float xv[16];
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const f32x4 t = *reinterpret_cast<const f32x4 *>(xt + m * kTurnStride + kofs + 4 * q);
+        xv[4 * q] = t.x;
+        xv[4 * q + 1] = t.y;
+        xv[4 * q + 2] = t.z;
+        xv[4 * q + 3] = t.w;
+      }
+      if (NORM) {
+        float nv[16] = {cur.nw[0].x, cur.nw[0].y, cur.nw[0].z, cur.nw[0].w,
+                        cur.nw[NORM ? 1 : 0].x, cur.nw[NORM ? 1 : 0].y, cur.nw[NORM ? 1 : 0].z, cur.nw[NORM ? 1 : 0].w,
+                        cur.nw[NORM ? 2 : 0].x, cur.nw[NORM ? 2 : 0].y, cur.nw[NORM ? 2 : 0].z, cur.nw[NORM ? 2 : 0].w,
+                        cur.nw[NORM ? 3 : 0].x, cur.nw[NORM ? 3 : 0].y, cur.nw[NORM ? 3 : 0].z, cur.nw[NORM ? 3 : 0].w};
+#pragma unroll
+        for (int e = 0; e < 16; ++e) { // past the end of a ragged row x is zero
+          ss = fmaf(xv[e], xv[e], ss);
+          xv[e] *= nv[e];
+        }
+      }
+      // the row's step for these 64 k: the smallest power of two s (not below
+      // 2^-126) with |x| / s < 2^22
+      unsigned mb = max_magnitude_bits(xv);
+      mb = max(mb, (unsigned)__shfl_xor((int)mb, 16, 64));
+      mb = max(mb, (unsigned)__shfl_xor((int)mb, 32, 64));
+      const int ex = (int)(mb >> 23) - 127; // floor(log2 max), -127 for zero and subnormals
+      const int e2 = max(ex + 1 - 22, -126);
+      const bool finite = mb < 0x7f800000u;
+      const float step = finite ? __uint_as_float((unsigned)(e2 + 127) << 23)
+                                : __uint_as_float(0x7fc00000u);
+      const float inv = __uint_as_float((unsigned)(127 - e2) << 23);
+      const float step65536 = step * 65536.0f;
+      v4i d[3];
+      to_digits(xv, inv, d);
+#pragma unroll
+      for (int s = 0; s < SPAN; ++s) {
+        {
+          const v4i r0 = __builtin_amdgcn_mfma_i32_16x16x64_i8(cur.w0[s], d[0], zero, 0, 0, 0);
+          const v4i r1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(cur.w0[s], d[1], zero, 0, 0, 0);
+          const v4i r2 = __builtin_amdgcn_mfma_i32_16x16x64_i8(cur.w0[s], d[2], zero, 0, 0, 0);
+          combine(acc0[s], r0, r1, r2, step, step65536);
+        }
+        if (DUAL) {
+          const v4i &w = cur.w1[DUAL ? s : 0];
+          const v4i r0 = __builtin_amdgcn_mfma_i32_16x16x64_i8(w, d[0], zero, 0, 0, 0);
+          const v4i r1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(w, d[1], zero, 0, 0, 0);
+          const v4i r2 = __builtin_amdgcn_mfma_i32_16x16x64_i8(w, d[2], zero, 0, 0, 0);
+          combine(acc1[DUAL ? s : 0], r0, r1, r2, step, step65536);
+        }
+      }
+      // the registers of chunk c are free: fetch the chunk R further on
+      fetch_chunk<SPAN, DUAL, NORM>(a, w0, w1, gofs, xrow, kcol, kofs, min(c + R, clast),
+                                    c + R < c1, cur);
+    }
+  }
+  // repeated last chunks may still be in flight: the ring registers stay
+  // allocated until they have landed (without these ties the compiler may put a
+  // temporary of the code below into one of them before the wait, and the late
+  // load would overwrite it)
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#pragma unroll
+  for (int u = 0; u < R; ++u)
+    wait_fetch<0, SPAN, DUAL, NORM>(ring[u]);
+  if (NORM) { // the four lanes that share a row hold different k
+    ss += __shfl_xor(ss, 16, 64);
+    ss += __shfl_xor(ss, 32, 64);
+  }
+
+  // ---- k-slices meet in LDS, in slice order --------------------------------
+  constexpr int kPerWave = (NA * 4 + 1) * kWave; // floats per wavefront
+  if (a.KS > 1) {
+    float *mine = meet + (size_t)wave * kPerWave;
+#pragma unroll
+    for (int s = 0; s < SPAN; ++s)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        mine[(s * 4 + i) * kWave + lane] = acc0[s][i];
+        if (DUAL)
+          mine[((SPAN + s) * 4 + i) * kWave + lane] = acc1[DUAL ? s : 0][i];
+      }
+    if (NORM)
+      mine[NA * 4 * kWave + lane] = ss;
+    __syncthreads();
+    if (ks != 0)
+      return;
+#pragma unroll
+    for (int s = 0; s < SPAN; ++s)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        float r0 = 0.f, r1 = 0.f;
+        for (int q = 0; q < a.KS; ++q) {
+          const float *o = meet + (size_t)(wave + q) * kPerWave;
+          r0 += o[(s * 4 + i) * kWave + lane];
+          if (DUAL)
+            r1 += o[((SPAN + s) * 4 + i) * kWave + lane];
+        }
+        acc0[s][i] = r0;
+        if (DUAL)
+          acc1[DUAL ? s : 0][i] = r1;
+      }
+    if (NORM) {
+      float r = 0.f;
+      for (int q = 0; q < a.KS; ++q)
+        r += meet[(size_t)(wave + q) * kPerWave + NA * 4 * kWave + lane];
+      ss = r;
+    }
+  }
+  // lane holds batch row m and channels kg*4 .. kg*4+3 of each group
+  if (!live || m >= a.rows)
+    return;
+  const float rn = NORM ? 1.0f / sqrtf(ss * a.norm_inv_k + a.norm_eps) : 1.0f;
+#pragma unroll
+  for (int s = 0; s < SPAN; ++s) {
+    const int g = g0 + s;
+    if (g >= a.groups)
+      continue;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int n = g * kTileN + kg * 4 + i;
+      if (n < a.N) {
+        float *c = a.C + (int64_t)m * a.ldc + n;
+        const float v = acc0[s][i] * rn * a.s0[n];
+        if (EPI == kEpiSiluMul)
+          *c = silu(v) * (acc1[DUAL ? s : 0][i] * rn * a.s1[n]);
+        else if (EPI == kEpiAccum)
+          *c = *c + v;
+        else
+          *c = a.bias ? a.bias[n] + v : v;
+      }
+    }
+  }
+}
+
+template <int EPI, int SPAN, bool NORM>
+int launch_kernel(const I8Args &ka, int blocks, hipStream_t stream) {
+  constexpr int NA = (EPI == kEpiSiluMul) ? 2 * SPAN : SPAN;
+  const int waves = ka.GS * ka.KS;
+  const size_t lds = sizeof(float) * waves *
+                     ((size_t)kTurnFloats + (ka.KS > 1 ? (size_t)(NA * 4 + 1) * kWave : 0));
+  auto kernel = gemv_w8a32_i8_kernel<EPI, SPAN, NORM>;
+  static bool attr_set = false;
+  if (!attr_set) {
+    BH_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                     hipFuncAttributeMaxDynamicSharedMemorySize,
+                                     144 * 1024));
+    attr_set = true;
+  }
+  hipLaunchKernelGGL(kernel, dim3(blocks), dim3(waves * kWave), lds, stream, ka);
+  BH_CHECK_HIP(hipGetLastError());
+  return BUDDY_HIP_OK;
+}
+
+template <int EPI, int SPAN>
+int launch_norm(const I8Args &ka, int blocks, hipStream_t stream) {
+  return ka.norm_w ? launch_kernel<EPI, SPAN, true>(ka, blocks, stream)
+                   : launch_kernel<EPI, SPAN, false>(ka, blocks, stream);
+}
+
+template <int SPAN>
+int launch_span(const I8Args &ka, int epilogue, int blocks, hipStream_t stream) {
+  switch (epilogue) {
+  case kEpiStore: return launch_norm<kEpiStore, SPAN>(ka, blocks, stream);
+  case kEpiAccum: return launch_norm<kEpiAccum, SPAN>(ka, blocks, stream);
+  case kEpiSiluMul:
+    if (SPAN > 2)
+      return fail(BUDDY_HIP_ERR_ARG, "gemv: SiLU*mul with %d groups per wavefront", SPAN);
+    return launch_norm<kEpiSiluMul, (SPAN > 2 ? 2 : SPAN)>(ka, blocks, stream);
+  }
+  return fail(BUDDY_HIP_ERR_ARG, "gemv: unknown epilogue %d", epilogue);
+}
+
+} // namespace
+
+// Small-batch path of launch_gemv (5 <= M <= 16) on the int8 matrix cores.
+int launch_gemv_i8(const GemvArgs &a, hipStream_t stream) {
+  I8Args ka;
+  ka.A = a.A;
+  ka.W0 = reinterpret_cast<const int4 *>(a.W0);
+  ka.W1 = reinterpret_cast<const int4 *>(a.W1);
+  ka.s0 = a.s0;
+  ka.s1 = a.s1;
+  ka.bias = a.bias;
+  ka.norm_w = a.norm_w;
+  ka.norm_eps = a.norm_eps;
+  ka.norm_inv_k = a.norm_inv_k;
+  ka.C = a.C;
+  ka.lda = a.lda;
+  ka.ldc = a.ldc;
+  ka.K = (int)a.K;
+  ka.N = (int)a.N;
+  ka.groups = (int)ceil_div(a.N, kTileN);
+  ka.chunks = (int)ceil_div(a.K, kTileK);
+  ka.rows = a.M;
+  const bool dual = a.epilogue == kEpiSiluMul;
+  // Channel groups per wavefront (they share one conversion of the activations
+  // and one read of them from L2): as many as still leave the chip a workgroup
+  // per compute unit.
+  int span = 1;
+  if (!dual && ka.groups >= 4 * 512)
+    span = 4;
+  else if (ka.groups >= 2 * 256)
+    span = 2;
+  ka.spans = (int)ceil_div(ka.groups, span);
+  // k-slices: as many wavefronts as the chip holds at once at these kernels'
+  // register count (16 per compute unit) and no more -- a second round of
+  // workgroups costs more than longer slices do --, at least two chunks each
+  int ks = 1;
+  while (ks < kMaxWavesI8 && (int64_t)ka.spans * ks * 2 <= 4096 && ka.chunks / (ks * 2) >= 2)
+    ks *= 2;
+  ka.KS = ks;
+  ka.GS = ks < 4 ? 4 / ks : 1;
+  const int blocks = (int)ceil_div(ka.spans, ka.GS);
+  if (span == 4)
+    return launch_span<4>(ka, a.epilogue, blocks, stream);
+  return span == 2 ? launch_span<2>(ka, a.epilogue, blocks, stream)
+                   : launch_span<1>(ka, a.epilogue, blocks, stream);
+}
+
+} // namespace bh

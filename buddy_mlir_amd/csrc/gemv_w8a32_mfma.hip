@@ -1,5 +1,8 @@
-// gemv_w8a32_mfma.hip -- the int8 dequant matmul for small batches (2..16 rows)
-// on the matrix cores.
+// gemv_w8a32_mfma.hip -- the int8 dequant matmul for small batches (5..16 rows)
+// on the bf16 matrix cores: the variant that keeps every bit of the f32
+// activations (BUDDY_HIP_GEMV_BATCH=bf16; the default is the int8 matrix-core
+// kernel of gemv_w8a32_i8.hip, which rounds them to 2^-23 of the largest of each
+// 64 and is quicker).
 //
 // The reference has no kernel of its own for 1 < M <= 16: its decode patterns
 // fire for m == 1 only (DequantMatMulVectorizationDecode.cpp:212-217) and the

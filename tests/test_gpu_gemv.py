@@ -109,6 +109,75 @@ def test_gemv_matches_oracle(oracle, K, N, M):
     check_close(y.cpu().numpy(), want)
 
 
+@pytest.fixture
+def bf16_batch_kernel(monkeypatch):
+    """Batches of 5..16 rows through the bf16 matrix-core kernel (every f32 bit of
+    the activations) instead of the default int8 matrix-core kernel."""
+    monkeypatch.setenv("BUDDY_HIP_GEMV_BATCH", "bf16")
+
+
+@pytest.mark.parametrize("K,N", [(1536, 8960), (8960, 1536), (100, 70), (1100, 40)])
+@pytest.mark.parametrize("M", [5, 16])
+def test_gemv_bf16_batch_kernel_matches_oracle(oracle, bf16_batch_kernel, K, N, M):
+    q, s = ops.quantize_w8(make_weight(K, N, K + N))
+    packed = ops.pack_w8(q)
+    g = torch.Generator(device="cuda").manual_seed(M)
+    x = torch.randn((M, K), generator=g, device="cuda")
+    y = ops.gemv_w8a32(x, packed, s, K, N)
+    torch.cuda.synchronize()
+    qh, sh, xh = q.cpu().numpy(), s.cpu().numpy(), x.cpu().numpy()
+    want = np.stack([oracle.dequant_gemv(xh[m], qh, sh) for m in range(M)])
+    check_close(y.cpu().numpy(), want)
+
+
+def test_int8_batch_kernel_scales_every_64_activations_on_their_own(oracle):
+    """The int8 matrix-core kernel turns the activations into fixed point 64 at a
+    time, each row and each run of 64 with a step of its own: rows 40 orders of
+    magnitude apart, and runs of one row 12 orders apart, must each keep f32
+    accuracy (compared row by row, and against a float64 sum)."""
+    K, N, M = 1536, 256, 8
+    q, s = ops.quantize_w8(make_weight(K, N, 77))
+    packed = ops.pack_w8(q)
+    rng = np.random.default_rng(5)
+    xh = rng.standard_normal((M, K)).astype(np.float32)
+    xh[1] *= 1e20
+    xh[2] *= 1e-20
+    xh[3, 64:128] *= 1e6      # one loud run of 64 in a quiet row
+    xh[4, :] *= 1e-6
+    xh[4, 640:704] *= 1e12
+    xh[5, 130] = 3e4          # a single outlier inside a run
+    xh[6] = 0.0               # a zero row stays zero
+    x = torch.from_numpy(xh).cuda()
+    y = ops.gemv_w8a32(x, packed, s, K, N).cpu().numpy()
+    qh, sh = q.cpu().numpy(), s.cpu().numpy()
+    want = (xh.astype(np.float64) @ qh.astype(np.float64)) * sh.astype(np.float64)
+    for m in range(M):
+        check_close(y[m], want[m])
+    assert not y[6].any()
+    # the quiet runs of row 3 are not drowned by its loud one: leave the loud run
+    # out on both sides and the rest still agrees to f32 accuracy
+    xq = xh.copy()
+    xq[3, 64:128] = 0.0
+    yq = ops.gemv_w8a32(torch.from_numpy(xq).cuda(), packed, s, K, N).cpu().numpy()
+    wq = (xq[3].astype(np.float64) @ qh.astype(np.float64)) * sh.astype(np.float64)
+    check_close(yq[3], wq)
+
+
+def test_int8_batch_kernel_shows_non_finite_activations():
+    """A NaN or an infinity in a row gives that row NaN results (the f32 product
+    would give NaN or infinity there) and leaves the other rows alone."""
+    K, N, M = 1536, 256, 8
+    q, s = ops.quantize_w8(make_weight(K, N, 78))
+    packed = ops.pack_w8(q)
+    rng = np.random.default_rng(6)
+    xh = rng.standard_normal((M, K)).astype(np.float32)
+    xh[2, 7] = np.nan
+    xh[5, 1000] = -np.inf
+    y = ops.gemv_w8a32(torch.from_numpy(xh).cuda(), packed, s, K, N).cpu().numpy()
+    assert np.isnan(y[2]).all() and np.isnan(y[5]).all()
+    assert np.isfinite(np.delete(y, [2, 5], 0)).all()
+
+
 def test_gemv_accumulates_into_c(oracle):
     K, N, M = 1536, 1536, 2
     q, s = ops.quantize_w8(make_weight(K, N, 5))
