@@ -129,8 +129,9 @@ template <int SPAN, bool DUAL, bool NORM> struct FetchRegs {
 template <int SPAN, bool DUAL, bool NORM> constexpr int fetch_loads() {
   return SPAN * (DUAL ? 2 : 1) + 4 * (NORM ? 2 : 1);
 }
-// Fetches kept in flight: as many as fit in about 64 registers (the kernel stays
-// within 128, so that a compute unit holds 16 wavefronts), two at least.
+// Fetches kept in flight: as many as fit in about 64 registers, two at least.
+// Without the fused norm the kernels then stay within 128 registers (a compute
+// unit holds 16 of their wavefronts); with it they take up to 147 (12).
 template <int SPAN, bool DUAL, bool NORM> constexpr int ring_depth() {
   constexpr int regs = 4 * SPAN * (DUAL ? 2 : 1) + 16 * (NORM ? 2 : 1);
   return 64 / regs < 2 ? 2 : 64 / regs;
@@ -192,7 +193,7 @@ constexpr int kTurnStride = 68;               // floats between rows of the turn
 constexpr int kTurnFloats = 16 * kTurnStride; // per wavefront
 
 template <int EPI, int SPAN, bool NORM>
-__global__ void __launch_bounds__(kMaxWavesI8 *kWave, 2)
+__global__ void __launch_bounds__(kMaxWavesI8 *kWave, 3) // 3 wavefronts per SIMD at least
     gemv_w8a32_i8_kernel(I8Args a) {
   constexpr bool DUAL = (EPI == kEpiSiluMul);
   constexpr int NA = DUAL ? 2 * SPAN : SPAN; // accumulators per lane
@@ -468,10 +469,12 @@ int launch_gemv_i8(const GemvArgs &a, hipStream_t stream) {
     span = 2;
   ka.spans = (int)ceil_div(ka.groups, span);
   // k-slices: as many wavefronts as the chip holds at once at these kernels'
-  // register count (16 per compute unit) and no more -- a second round of
-  // workgroups costs more than longer slices do --, at least two chunks each
+  // register count (16 per compute unit; with the fused norm one workgroup of 8)
+  // and no more -- a second round of workgroups costs more than longer slices
+  // do --, at least two chunks each
+  const int64_t resident = a.norm_w ? 2048 : 4096;
   int ks = 1;
-  while (ks < kMaxWavesI8 && (int64_t)ka.spans * ks * 2 <= 4096 && ka.chunks / (ks * 2) >= 2)
+  while (ks < kMaxWavesI8 && (int64_t)ka.spans * ks * 2 <= resident && ka.chunks / (ks * 2) >= 2)
     ks *= 2;
   ka.KS = ks;
   ka.GS = ks < 4 ? 4 / ks : 1;
