@@ -100,7 +100,14 @@ int buddy_hip_gemv_w4a16(const uint16_t *A, const int8_t *packed, const uint16_t
  * midend/lib/Conversion/MatMulOptimization/DequantMatMulVectorizationDecode.cpp
  * :250-321 generates:  C[m,n] (+)= (sum_k A[m,k] * W[k,n]) * scale[n].
  * M is 1..16 (the reference pattern is m == 1 only; M > 1 streams the weights
- * once for all rows).  A: f32 [M,K] row-major (lda = K), C: f32 [M,N]. */
+ * once for all rows).  A: f32 [M,K] row-major (lda = K), C: f32 [M,N].
+ * Up to 4 rows every product is an f32 multiply-add.  From 5 rows (with K a
+ * multiple of 4 and A 16-byte aligned) the int8 matrix cores are used: the
+ * activations of a row are rounded, 64 at a time, to 2^-23 of the largest of
+ * the 64, the sums are exact; a NaN or an infinity in a row turns that row of C
+ * into NaN.  With the environment variable BUDDY_HIP_GEMV_BATCH=bf16 (read at
+ * every call) those batches keep every bit of the activations instead, on the
+ * bf16 matrix cores, at about two thirds of the speed. */
 enum {
   BUDDY_HIP_GEMV_ACCUMULATE = 1 /* C += ...  (linalg.matmul semantics);
                                    without it C = ... and C need not be
