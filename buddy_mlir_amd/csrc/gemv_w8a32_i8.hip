@@ -58,21 +58,14 @@ __device__ __forceinline__ float silu(float g) {
   return g * sig;
 }
 
-// Largest magnitude of 16 values as a bit pattern (sign dropped).  Integer
-// comparisons, so that a NaN (the largest patterns of all) is not lost: the
-// signed maximum finds the largest positive value, the unsigned one the
-// largest-magnitude negative value if there is any.
-__device__ __forceinline__ unsigned max_magnitude_bits(const float (&v)[16]) {
-  int hi = __float_as_int(v[0]);
-  unsigned lo = __float_as_uint(v[0]);
+// Largest magnitude of 16 values; a NaN among them gives NaN (v_maximum3_f32, the
+// IEEE-754-2019 maximum, which does not drop NaNs the way fmaxf does).
+__device__ __forceinline__ float max_magnitude(const float (&v)[16]) {
+  float m = __builtin_fabsf(v[0]);
 #pragma unroll
-  for (int e = 1; e < 16; ++e) {
-    hi = max(hi, __float_as_int(v[e]));
-    lo = max(lo, __float_as_uint(v[e]));
-  }
-  const unsigned pos = hi < 0 ? 0u : (unsigned)hi;
-  const unsigned neg = (lo & 0x80000000u) ? (lo & 0x7fffffffu) : 0u;
-  return max(pos, neg);
+  for (int e = 1; e < 16; ++e)
+    m = __builtin_elementwise_maximum(m, __builtin_fabsf(v[e]));
+  return m;
 }
 
 // 16 values of one row -> this lane's operand of each of the three digit planes.
@@ -287,9 +280,10 @@ __global__ void __launch_bounds__(kMaxWavesI8 *kWave, 3) // 3 wavefronts per SIM
       }
       // the row's step for these 64 k: the smallest power of two s (not below
       // 2^-126) with |x| / s < 2^22
-      unsigned mb = max_magnitude_bits(xv);
-      mb = max(mb, (unsigned)__shfl_xor((int)mb, 16, 64));
-      mb = max(mb, (unsigned)__shfl_xor((int)mb, 32, 64));
+      float mx = max_magnitude(xv);
+      mx = __builtin_elementwise_maximum(mx, __shfl_xor(mx, 16, 64));
+      mx = __builtin_elementwise_maximum(mx, __shfl_xor(mx, 32, 64));
+      const unsigned mb = __float_as_uint(mx) & 0x7fffffffu;
       const int ex = (int)(mb >> 23) - 127; // floor(log2 max), -127 for zero and subnormals
       const int e2 = max(ex + 1 - 22, -126);
       const bool finite = mb < 0x7f800000u;
