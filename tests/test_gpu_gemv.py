@@ -95,8 +95,6 @@ SHAPES = [(1536, 8960), (8960, 1536), (1536, 1536), (1536, 256), (64, 16), (100,
 @pytest.mark.parametrize("K,N", SHAPES)
 @pytest.mark.parametrize("M", [1, 2, 4, 5, 8, 13, 16])
 def test_gemv_matches_oracle(oracle, K, N, M):
-    if M > 1 and K * N > 1536 * 8960:
-        pytest.skip("large shapes at M=1 only (CPU oracle time)")
     W = make_weight(K, N, K + 3 * N)
     q, s = ops.quantize_w8(W)
     packed = ops.pack_w8(q)
@@ -107,6 +105,88 @@ def test_gemv_matches_oracle(oracle, K, N, M):
     qh, sh, xh = q.cpu().numpy(), s.cpu().numpy(), x.cpu().numpy()
     want = np.stack([oracle.dequant_gemv(xh[m], qh, sh) for m in range(M)])
     check_close(y.cpu().numpy(), want)
+
+
+# The decode GEMV set of a Llama-3-8B-shaped step: q_proj, kv_proj, gate/up, down
+# and lm_head, each alone at one row and at eight.
+LLAMA3_8B = [(4096, 4096), (4096, 1024), (4096, 14336), (14336, 4096), (4096, 128256)]
+
+
+@pytest.mark.parametrize("K,N", LLAMA3_8B)
+@pytest.mark.parametrize("M", [1, 8])
+def test_llama3_8b_gemv_set_matches_oracle(oracle, K, N, M):
+    q, s = ops.quantize_w8(make_weight(K, N, K + 5 * N))
+    packed = ops.pack_w8(q)
+    g = torch.Generator(device="cuda").manual_seed(10 + M)
+    x = torch.randn((M, K), generator=g, device="cuda")
+    y = ops.gemv_w8a32(x, packed, s, K, N)
+    torch.cuda.synchronize()
+    qh, sh, xh = q.cpu().numpy(), s.cpu().numpy(), x.cpu().numpy()
+    want = np.stack([oracle.dequant_gemv(xh[m], qh, sh) for m in range(M)])
+    check_close(y.cpu().numpy(), want)
+
+
+@pytest.mark.parametrize("M", [1, 8])
+def test_llama3_8b_fused_launches_match_oracle(oracle, M):
+    """The launches a Llama-3-8B-shaped decode step makes: RMSNorm + q|k|v as one
+    matrix (4096 -> 6144), o_proj accumulating into the residual row, RMSNorm +
+    gate|up + SiLU*mul (4096 -> 2 x 14336), down accumulating (14336 -> 4096),
+    RMSNorm + lm_head (4096 -> 128256)."""
+    H, I, QKV, V = 4096, 14336, 4096 + 2 * 1024, 128256
+    eps = np.float32(1e-5)
+    g = torch.Generator(device="cuda").manual_seed(40 + M)
+    x = torch.randn((M, H), generator=g, device="cuda") * 2
+    w = 1 + 0.1 * torch.randn(H, generator=g, device="cuda")
+    xh, wh = x.cpu().numpy(), w.cpu().numpy()
+    xn = np.stack([oracle.rmsnorm(xh[m], wh, eps, np.float32(1.0) / np.float32(H))
+                   for m in range(M)])
+
+    def launch(**kw):
+        torch.cuda.synchronize()
+        ops.linear_w8a32(**kw)
+        torch.cuda.synchronize()
+
+    # RMSNorm + q|k|v
+    q, s = ops.quantize_w8(make_weight(H, QKV, 1))
+    out = torch.empty((M, QKV), device="cuda")
+    launch(A=x, lda=H, W0=ops.pack_w8(q), scale0=s, norm_w=w, norm_eps=float(eps), C=out,
+           ldc=QKV, M=M, K=H, N=QKV, epilogue=0)
+    qh, sh = q.cpu().numpy(), s.cpu().numpy()
+    check_close(out.cpu().numpy(), np.stack([oracle.dequant_gemv(xn[m], qh, sh) for m in range(M)]))
+    # o_proj, C += ...
+    q, s = ops.quantize_w8(make_weight(H, H, 2))
+    c0 = torch.randn((M, H), generator=g, device="cuda")
+    c = c0.clone()
+    launch(A=x, lda=H, W0=ops.pack_w8(q), scale0=s, C=c, ldc=H, M=M, K=H, N=H, epilogue=1)
+    qh, sh, c0h = q.cpu().numpy(), s.cpu().numpy(), c0.cpu().numpy()
+    check_close(c.cpu().numpy(),
+                np.stack([oracle.dequant_gemv(xh[m], qh, sh, c0h[m]) for m in range(M)]))
+    # RMSNorm + gate|up + SiLU*mul
+    qg, sg = ops.quantize_w8(make_weight(H, I, 3))
+    qu, su = ops.quantize_w8(make_weight(H, I, 4))
+    h = torch.empty((M, I), device="cuda")
+    launch(A=x, lda=H, W0=ops.pack_w8(qg), scale0=sg, W1=ops.pack_w8(qu), scale1=su, norm_w=w,
+           norm_eps=float(eps), C=h, ldc=I, M=M, K=H, N=I, epilogue=2)
+    qgh, sgh, quh, suh = (t.cpu().numpy() for t in (qg, sg, qu, su))
+    hh = np.stack([oracle.silu_mul(oracle.dequant_gemv(xn[m], qgh, sgh),
+                                   oracle.dequant_gemv(xn[m], quh, suh)) for m in range(M)])
+    check_close(h.cpu().numpy(), hh)
+    del qg, qu
+    # down, C += ...
+    q, s = ops.quantize_w8(make_weight(I, H, 5))
+    c = c0.clone()
+    hin = torch.from_numpy(hh).cuda()
+    launch(A=hin, lda=I, W0=ops.pack_w8(q), scale0=s, C=c, ldc=H, M=M, K=I, N=H, epilogue=1)
+    qh, sh = q.cpu().numpy(), s.cpu().numpy()
+    check_close(c.cpu().numpy(),
+                np.stack([oracle.dequant_gemv(hh[m], qh, sh, c0h[m]) for m in range(M)]))
+    # RMSNorm + lm_head
+    q, s = ops.quantize_w8(make_weight(H, V, 6))
+    out = torch.empty((M, V), device="cuda")
+    launch(A=x, lda=H, W0=ops.pack_w8(q), scale0=s, norm_w=w, norm_eps=float(eps), C=out,
+           ldc=V, M=M, K=H, N=V, epilogue=0)
+    qh, sh = q.cpu().numpy(), s.cpu().numpy()
+    check_close(out.cpu().numpy(), np.stack([oracle.dequant_gemv(xn[m], qh, sh) for m in range(M)]))
 
 
 @pytest.fixture

@@ -211,6 +211,32 @@ def test_prefill_in_two_blocks_and_after_decode_steps(oracle):
     sess.close()
 
 
+@pytest.mark.timeout(900)
+def test_qwen2_1p5b_shape_512_token_prefill(oracle):
+    """The full 28-layer shape, a prompt of 512 tokens as one block (digit-plane
+    matmuls, the default) against 512 oracle decode steps: last-row logits, the
+    greedy token, and the cache rows of the first and the last layer."""
+    shape = Shape()
+    sess, host = synthetic.build_session(shape, context=0, keep_host=True)
+    om = oracle_model(oracle, shape, host)
+    kv = host["kv"]
+    toks = synthetic.first_tokens(shape, 512, seed=21).tolist()
+    for pos, t in enumerate(toks):
+        otok, ologits = om.decode_step(t, pos, kv)
+    nxt, logits = sess.prefill(toks, 0)
+    check_close(logits, ologits)
+    top2 = np.partition(ologits, -2)[-2:]
+    assert nxt == otok, f"top-2 logit margin {float(top2[1] - top2[0]):.3e}"
+    for j in (0, 1, 2 * shape.layers - 2, 2 * shape.layers - 1):
+        check_close(sess.get_kv(j)[:, :512, :], kv[j][:, :512, :])
+    # one decode step on from the prefilled cache
+    n2, lg = sess.decode(otok, 512)
+    t2, olg = om.decode_step(otok, 512, kv)
+    check_close(lg, olg)
+    assert n2 == t2
+    sess.close()
+
+
 def test_session_prefill_refuses_overflow(bh):
     sess, _ = synthetic.build_session(SMALL, context=0)
     with pytest.raises(bma.BuddyHipError):
