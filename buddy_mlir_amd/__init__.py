@@ -100,7 +100,7 @@ def _declare(lib):
         "buddy_hip_argmax_workspace_bytes": (sz, []),
         "buddy_hip_argmax": (c_int, [vp, c_int, vp, vp, vp]),
         "buddy_hip_attn_decode_workspace_bytes": (sz, [c_int, c_int]),
-        "buddy_hip_gqa_decode_attention": (c_int, [vp, vp, vp, vp, vp, vp, c_int,
+        "buddy_hip_gqa_decode_attention": (c_int, [vp, vp, vp, vp, vp, vp, vp, c_int,
                                                    c_int, c_int, c_int, c_float,
                                                    vp, sz, vp]),
         "buddy_hip_prefill_attention": (c_int, [vp, vp, vp, vp, vp, c_int, c_int, c_int,
@@ -111,6 +111,8 @@ def _declare(lib):
         "buddy_hip_session_set_layer": (c_int, [vp, c_int, vp]),
         "buddy_hip_session_set_kv": (c_int, [vp, c_int, vp]),
         "buddy_hip_session_get_kv": (c_int, [vp, c_int, vp]),
+        "buddy_hip_session_get_kv_rows": (c_int, [vp, c_int, c_int, vp]),
+        "buddy_hip_session_decode_mirror": (c_int, [vp, c_int, c_int, vp, vp, vp]),
         "buddy_hip_session_use_graph": (c_int, [vp, c_int]),
         "buddy_hip_session_decode": (c_int, [vp, c_int, c_int, vp, vp]),
         "buddy_hip_session_decode_greedy": (c_int, [vp, c_int, c_int, c_int, vp]),

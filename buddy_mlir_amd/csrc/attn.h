@@ -17,6 +17,7 @@ struct AttnDecodeArgs {
   float *kcache = nullptr;         // [kv_heads, max_len, D]
   float *vcache = nullptr;
   float *out = nullptr;            // [heads*D]
+  float *lse = nullptr;            // optional [heads]: log-sum-exp of the scores
   int heads = 0, kv_heads = 0, head_dim = 0, max_len = 0;
   float scale = 0.f;
   void *workspace = nullptr; // flash-decoding partials

@@ -43,6 +43,7 @@ struct AttnArgs {
   float *part_acc;       // [heads, nchunks, D]
   float *part_ml;        // [heads, nchunks, 2]
   float *out;            // [heads*D]
+  float *lse;            // [heads] or null: m + log l of the whole softmax
   int heads, kv_heads, group, max_len, nchunks;
   float scale;
   int pairs_padded; // (chunk, kv head) pairs rounded up to the XCD count
@@ -112,7 +113,11 @@ __global__ void __launch_bounds__(kThreads) attn_decode_partial(AttnArgs a) {
   } else {
     inv_f = a.inv_freq[jj];
   }
-  const int pos = *a.pos_ptr;
+  // a position outside the cache (a caller's mistake the host cannot see: the
+  // position lives on the device) is clamped for the scan and writes nothing
+  const int pos_raw = *a.pos_ptr;
+  const bool pos_ok = pos_raw >= 0 && pos_raw < a.max_len;
+  const int pos = min(max(pos_raw, 0), a.max_len - 1);
 
   if (p0 > pos) { // nothing visible in this chunk: an empty partial
     if (qh < nh)
@@ -136,7 +141,7 @@ __global__ void __launch_bounds__(kThreads) attn_decode_partial(AttnArgs a) {
     const float kn = kraw * cs + kpair * sn;
     knew_s[j] = kn;
     vnew_s[j] = vraw;
-    if (hb == 0) { // one writer per cache row
+    if (hb == 0 && pos_ok) { // one writer per cache row
       a.kcache[((size_t)kvh * a.max_len + pos) * kD + j] = kn;
       a.vcache[((size_t)kvh * a.max_len + pos) * kD + j] = vraw;
     }
@@ -249,7 +254,7 @@ __global__ void __launch_bounds__(kThreads) attn_decode_partial(AttnArgs a) {
 // b = exp(m_s - m_new); l = l*a + l_s*b; acc = acc_s*b + acc*a; out = acc / l.
 __global__ void __launch_bounds__(kD) attn_decode_combine(AttnArgs a) {
   const int h = blockIdx.x, d = threadIdx.x;
-  const int pos = *a.pos_ptr;
+  const int pos = min(max(*a.pos_ptr, 0), a.max_len - 1);
   const int used = min(a.nchunks, pos / kChunk + 1);
   float m_run = kSeedM, l_run = 0.f, acc = 0.f;
   for (int s = 0; s < used; ++s) {
@@ -264,6 +269,8 @@ __global__ void __launch_bounds__(kD) attn_decode_combine(AttnArgs a) {
     m_run = m_new;
   }
   a.out[(size_t)h * kD + d] = acc / l_run;
+  if (a.lse && d == 0) // tosa.py:14576-14580
+    a.lse[h] = m_run + logf(l_run);
 }
 
 } // namespace
@@ -292,6 +299,7 @@ int launch_attn_decode(const AttnDecodeArgs &in, hipStream_t stream) {
              "attn_decode: heads=%d kv_heads=%d unsupported", in.heads,
              in.kv_heads);
   BH_REQUIRE(in.max_len > 0, "attn_decode: max_len=%d", in.max_len);
+  BH_REQUIRE(!in.lse || in.combine, "attn_decode: lse needs the combine pass");
   BH_REQUIRE(in.workspace_bytes >=
                  attn_decode_workspace_bytes(in.heads, in.max_len),
              "attn_decode: workspace of %zu bytes needed, %zu given",
@@ -314,6 +322,7 @@ int launch_attn_decode(const AttnDecodeArgs &in, hipStream_t stream) {
   a.part_acc = parts.acc;
   a.part_ml = parts.ml;
   a.out = in.out;
+  a.lse = in.lse;
   a.pairs_padded = (int)round_up((int64_t)a.nchunks * in.kv_heads, 8);
   const int head_blocks = (a.group + kHPB - 1) / kHPB;
   hipLaunchKernelGGL(attn_decode_partial, dim3(a.pairs_padded * head_blocks),
@@ -334,10 +343,11 @@ size_t buddy_hip_attn_decode_workspace_bytes(int heads, int max_len) {
 
 int buddy_hip_gqa_decode_attention(const float *qkv, const float *inv_freq,
                                    const int *pos, float *kcache, float *vcache,
-                                   float *out, int heads, int kv_heads,
-                                   int head_dim, int max_len, float scale,
-                                   void *workspace, size_t workspace_bytes,
-                                   buddy_hip_stream stream) {
+                                   float *out, float *lse, int heads,
+                                   int kv_heads, int head_dim, int max_len,
+                                   float scale, void *workspace,
+                                   size_t workspace_bytes,
+                                   buddy_hip_stream stream) try {
   bh::AttnDecodeArgs a;
   a.qkv = qkv;
   a.inv_freq = inv_freq;
@@ -345,6 +355,7 @@ int buddy_hip_gqa_decode_attention(const float *qkv, const float *inv_freq,
   a.kcache = kcache;
   a.vcache = vcache;
   a.out = out;
+  a.lse = lse;
   a.heads = heads;
   a.kv_heads = kv_heads;
   a.head_dim = head_dim;
@@ -353,5 +364,5 @@ int buddy_hip_gqa_decode_attention(const float *qkv, const float *inv_freq,
   a.workspace = workspace;
   a.workspace_bytes = workspace_bytes;
   return bh::launch_attn_decode(a, bh::as_stream(stream));
-}
+} BH_CATCH_INT("buddy_hip_gqa_decode_attention")
 }

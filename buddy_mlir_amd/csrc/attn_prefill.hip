@@ -345,7 +345,7 @@ extern "C" {
 int buddy_hip_prefill_attention(const float *q, const float *k, const float *v,
                                 const float *mask, float *out, int heads,
                                 int kv_heads, int head_dim, int q_len, int k_len,
-                                float scale, buddy_hip_stream stream) {
+                                float scale, buddy_hip_stream stream) try {
   // the reference operator's layout: [heads, len, head_dim] for q/out,
   // [kv_heads, len, head_dim] for k/v
   bh::AttnPrefillArgs a;
@@ -366,5 +366,5 @@ int buddy_hip_prefill_attention(const float *q, const float *k, const float *v,
   a.o_stride = head_dim;
   a.o_hstride = (int64_t)q_len * head_dim;
   return bh::launch_attn_prefill(a, bh::as_stream(stream));
-}
+} BH_CATCH_INT("buddy_hip_prefill_attention")
 }

@@ -28,6 +28,7 @@
 
 #include <cstdlib>
 #include <cstring>
+#include <memory>
 #include <mutex>
 #include <vector>
 
@@ -43,7 +44,31 @@ struct ModelState {
   buddy_hip_model_shape shape{};
   float *dev_f32 = nullptr; // the f32 blob on the device (embedding is borrowed)
   float *pinned_logits = nullptr; // [vocab]: the logits row lands here first
+  float *pinned_rows = nullptr;   // [2 * layers, kv_heads, head_dim]: a step's new cache rows
   bool kv_on_device = false;
+  // The position the next decode call is expected to carry when the caller just
+  // goes on generating; -1: any (after a prefill, whose prompt length only the
+  // caller knows, and after a device-side discard).  A call with another
+  // position means the caller edited its host tensors (the generated
+  // ModelSession::handleKVCacheOverflow shifts and re-rotates them and lowers
+  // its position, gen_session.py:1471-1511): the device cache is then reloaded
+  // from them.
+  long long expected_pos = -1;
+};
+
+// malloc'd host memory that is freed unless handed over
+struct HostBuf {
+  void *p = nullptr;
+  explicit HostBuf(size_t bytes) : p(malloc(bytes)) {}
+  HostBuf(const HostBuf &) = delete;
+  HostBuf &operator=(const HostBuf &) = delete;
+  ~HostBuf() { free(p); }
+  template <typename T> T *as() const { return static_cast<T *>(p); }
+  template <typename T> T *release() {
+    T *q = static_cast<T *>(p);
+    p = nullptr;
+    return q;
+  }
 };
 
 ModelState &state() {
@@ -86,6 +111,10 @@ void destroy_locked(ModelState &m) {
     (void)hipFree(m.dev_f32);
   if (m.pinned_logits)
     (void)hipHostFree(m.pinned_logits);
+  if (m.pinned_rows)
+    (void)hipHostFree(m.pinned_rows);
+  m.pinned_rows = nullptr;
+  m.expected_pos = -1;
   m.sess = nullptr;
   m.dev_f32 = nullptr;
   m.pinned_logits = nullptr;
@@ -276,24 +305,44 @@ int forward_decode(DecodeResult *res, buddy_memref_f32_1d *f32, buddy_memref_i8_
   BH_REQUIRE(token >= 0 && token < m.shape.vocab && position >= 0 &&
                  position < m.shape.max_len,
              "forward_decode: token %lld / position %lld out of range", token, position);
-  if (!m.kv_on_device) { // the caller's cache is the truth until we have run
+  // The caller's host tensors and the device cache are kept equal: every step
+  // writes its new rows through to the caller's tensors (below), so the caller
+  // may edit them between calls.  It has done so when the position is not the
+  // one that follows the last step; the device copy is then loaded again.
+  if (m.kv_on_device && m.expected_pos >= 0 && position != m.expected_pos)
+    m.kv_on_device = false;
+  if (!m.kv_on_device) { // the caller's cache is the truth
     for (int i = 0; i < 2 * kLayers; ++i)
       if ((rc = buddy_hip_session_set_kv(m.sess, i, a.kv[i]->aligned + a.kv[i]->offset)))
         return rc;
     m.kv_on_device = true;
   }
   const int64_t V = m.shape.vocab;
+  const size_t row_elems = (size_t)m.shape.kv_heads * m.shape.head_dim;
   // the row crosses PCIe into pinned memory (a copy into pageable memory is
   // staged by the runtime and several times slower) and is handed over in a
   // malloc'd buffer, which is what the caller frees
   if (!m.pinned_logits)
     BH_CHECK_HIP(hipHostMalloc((void **)&m.pinned_logits, sizeof(float) * (size_t)V));
-  if ((rc = buddy_hip_session_decode(m.sess, (int)token, (int)position, m.pinned_logits,
-                                     nullptr)))
+  if (!m.pinned_rows)
+    BH_CHECK_HIP(hipHostMalloc((void **)&m.pinned_rows,
+                               sizeof(float) * 2 * kLayers * row_elems));
+  if ((rc = buddy_hip_session_decode_mirror(m.sess, (int)token, (int)position,
+                                            m.pinned_logits, m.pinned_rows, nullptr)))
     return rc;
-  float *logits = static_cast<float *>(malloc(sizeof(float) * (size_t)V));
-  BH_REQUIRE(logits, "forward_decode: out of host memory");
-  memcpy(logits, m.pinned_logits, sizeof(float) * (size_t)V);
+  m.expected_pos = position + 1;
+  // write-through: row `position` of every cache, as the compiled model leaves
+  // it in the caller's tensors (index_put, subgraph0_decode_simplify.mlir:108-142)
+  for (int i = 0; i < 2 * kLayers; ++i) {
+    float *host = a.kv[i]->aligned + a.kv[i]->offset;
+    for (int h = 0; h < m.shape.kv_heads; ++h)
+      memcpy(host + ((size_t)h * m.shape.max_len + (size_t)position) * m.shape.head_dim,
+             m.pinned_rows + ((size_t)i * m.shape.kv_heads + h) * m.shape.head_dim,
+             sizeof(float) * m.shape.head_dim);
+  }
+  HostBuf logits_buf(sizeof(float) * (size_t)V);
+  BH_REQUIRE(logits_buf.p, "forward_decode: out of host memory");
+  memcpy(logits_buf.p, m.pinned_logits, sizeof(float) * (size_t)V);
   // results: state tensors alias the caller's, logits are handed over.  The
   // descriptors are read before any is written: the caller may pass members of
   // the result block itself as arguments.
@@ -311,10 +360,8 @@ int forward_decode(DecodeResult *res, buddy_memref_f32_1d *f32, buddy_memref_i8_
     // exit: the position comes back in a buffer of its own, not as an alias of
     // the caller's cache_position tensor
     long long *own = static_cast<long long *>(malloc(sizeof(long long)));
-    if (!own) {
-      free(logits);
-      return fail(BUDDY_HIP_ERR_ARG, "forward_decode: out of host memory");
-    }
+    if (!own)
+      return fail(BUDDY_HIP_ERR_HOST, "forward_decode: out of host memory");
     *own = position;
     g->pos_out = pos_d;
     g->pos_out.allocated = own;
@@ -338,6 +385,7 @@ int forward_decode(DecodeResult *res, buddy_memref_f32_1d *f32, buddy_memref_i8_
     }
     lg = &res->logits;
   }
+  float *logits = logits_buf.release<float>();
   lg->allocated = logits;
   lg->aligned = logits;
   lg->offset = 0;
@@ -371,28 +419,26 @@ int forward_prefill(PrefillResult *res, buddy_memref_f32_1d *f32,
   // (rows past the prompt are padding; causality keeps them from mattering)
   const size_t kv_elems = (size_t)S.kv_heads * S.max_len * S.head_dim;
   const size_t logit_elems = (size_t)S.max_len * S.vocab;
-  float *logits = static_cast<float *>(malloc(sizeof(float) * logit_elems));
-  BH_REQUIRE(logits, "forward_prefill: out of host memory");
-  std::vector<float *> kvbuf(2 * kLayers, nullptr);
-  auto fail_free = [&](int code) {
-    free(logits);
-    for (float *p : kvbuf)
-      free(p);
-    return code;
-  };
-  if ((rc = buddy_hip_session_prefill_all_logits(m.sess, toks.data(), max_len, 0, logits)))
-    return fail_free(rc);
+  HostBuf logits_buf(sizeof(float) * logit_elems);
+  BH_REQUIRE(logits_buf.p, "forward_prefill: out of host memory");
+  std::vector<std::unique_ptr<HostBuf>> kvbuf;
+  kvbuf.reserve(2 * kLayers);
+  if ((rc = buddy_hip_session_prefill_all_logits(m.sess, toks.data(), max_len, 0,
+                                                 logits_buf.as<float>())))
+    return rc;
   for (int i = 0; i < 2 * kLayers; ++i) {
-    kvbuf[(size_t)i] = static_cast<float *>(malloc(sizeof(float) * kv_elems));
-    if (!kvbuf[(size_t)i])
-      return fail_free(fail(BUDDY_HIP_ERR_ARG, "forward_prefill: out of host memory"));
-    if ((rc = buddy_hip_session_get_kv(m.sess, i, kvbuf[(size_t)i])))
-      return fail_free(rc);
+    kvbuf.emplace_back(new HostBuf(sizeof(float) * kv_elems));
+    BH_REQUIRE(kvbuf.back()->p, "forward_prefill: out of host memory");
+    if ((rc = buddy_hip_session_get_kv(m.sess, i, kvbuf.back()->as<float>())))
+      return rc;
   }
+  // nothing below can fail: the buffers now belong to the caller
+  float *logits = logits_buf.release<float>();
+  m.expected_pos = -1; // the prompt length is the caller's knowledge
   m.kv_on_device = true;
   for (int i = 0; i < 2 * kLayers; ++i) {
     buddy_memref_f32_4d &d = res->kv[i];
-    d.allocated = d.aligned = kvbuf[(size_t)i];
+    d.allocated = d.aligned = kvbuf[(size_t)i]->release<float>();
     d.offset = 0;
     d.sizes[0] = 1;
     d.sizes[1] = S.kv_heads;
@@ -434,7 +480,7 @@ void _mlir_ciface_forward_decode(
     BH_DKV(1) BH_DKV(2) BH_DKV(3) BH_DKV(4) BH_DKV(5) BH_DKV(6) BH_DKV(7) BH_DKV(8)
     BH_DKV(9) BH_DKV(10) BH_DKV(11) BH_DKV(12) BH_DKV(13) BH_DKV(14) BH_DKV(15)
     BH_DKV(16) BH_DKV(17) BH_DKV(18) BH_DKV(19) BH_DKV(20) BH_DKV(21) BH_DKV(22)
-    BH_DKV(23) BH_DKV(24) BH_DKV(25) BH_DKV(26) BH_DKV(27)) {
+    BH_DKV(23) BH_DKV(24) BH_DKV(25) BH_DKV(26) BH_DKV(27)) try {
   bh::KVArgs a;
   BH_PUT(0)
   BH_PUTD(1) BH_PUTD(2) BH_PUTD(3) BH_PUTD(4) BH_PUTD(5) BH_PUTD(6) BH_PUTD(7)
@@ -448,18 +494,18 @@ void _mlir_ciface_forward_decode(
     }
   (void)bh::forward_decode(static_cast<bh::DecodeResult *>(result), f32_params,
                            i8_params, token, cache_position, a);
-}
+} BH_CATCH_VOID("_mlir_ciface_forward_decode")
 
 void _mlir_ciface_forward_prefill(void *result, buddy_memref_f32_1d *f32_params,
                                   buddy_memref_i8_1d *i8_params,
-                                  buddy_memref_i64_2d *tokens) {
+                                  buddy_memref_i64_2d *tokens) try {
   (void)bh::forward_prefill(static_cast<bh::PrefillResult *>(result), f32_params,
                             i8_params, tokens);
-}
+} BH_CATCH_VOID("_mlir_ciface_forward_prefill")
 
 buddy_hip_session *buddy_hip_session_create_from_w8a32_blobs(
     const buddy_hip_model_shape *shape, const float *f32_params, int64_t n_f32,
-    const int8_t *i8_params, int64_t n_i8) {
+    const int8_t *i8_params, int64_t n_i8) try {
   if (!shape) {
     bh::fail(BUDDY_HIP_ERR_ARG, "create_from_w8a32_blobs: null shape");
     return nullptr;
@@ -470,10 +516,10 @@ buddy_hip_session *buddy_hip_session_create_from_w8a32_blobs(
     return nullptr;
   buddy_hip_session_adopt(sess, dev_f32); // freed with the session
   return sess;
-}
+} BH_CATCH_NULL("buddy_hip_session_create_from_w8a32_blobs")
 
 void buddy_hip_w8a32_blob_sizes(const buddy_hip_model_shape *shape, int64_t *n_f32,
-                                int64_t *n_i8) {
+                                int64_t *n_i8) try {
   if (!shape)
     return;
   const bh::BlobSizes b = bh::blob_sizes(*shape);
@@ -481,26 +527,30 @@ void buddy_hip_w8a32_blob_sizes(const buddy_hip_model_shape *shape, int64_t *n_f
     *n_f32 = b.f32;
   if (n_i8)
     *n_i8 = b.i8;
-}
+} BH_CATCH_VOID("buddy_hip_w8a32_blob_sizes")
 
-void buddy_hip_forward_reset(void) {
+void buddy_hip_forward_reset(void) try {
   bh::ModelState &m = bh::state();
   std::lock_guard<std::mutex> lock(m.mu);
   bh::destroy_locked(m);
-}
+} BH_CATCH_VOID("buddy_hip_forward_reset")
 
-int buddy_hip_forward_discard_kv(int keep, int discard, int count) {
+int buddy_hip_forward_discard_kv(int keep, int discard, int count) try {
   bh::ModelState &m = bh::state();
   std::lock_guard<std::mutex> lock(m.mu);
   if (!m.sess || !m.kv_on_device)
     return bh::fail(BUDDY_HIP_ERR_ARG,
                     "forward_discard_kv: no device-resident KV cache yet");
-  return buddy_hip_session_discard_kv(m.sess, keep, discard, count);
-}
+  int rc = buddy_hip_session_discard_kv(m.sess, keep, discard, count);
+  if (!rc) // the device cache is now ahead of the caller's tensors: never reload
+    m.expected_pos = -1;
+  return rc;
+} BH_CATCH_INT("buddy_hip_forward_discard_kv")
 
-void buddy_hip_forward_invalidate_kv(void) {
+void buddy_hip_forward_invalidate_kv(void) try {
   bh::ModelState &m = bh::state();
   std::lock_guard<std::mutex> lock(m.mu);
   m.kv_on_device = false;
-}
+  m.expected_pos = -1;
+} BH_CATCH_VOID("buddy_hip_forward_invalidate_kv")
 }

@@ -13,6 +13,7 @@
 #include <cstdlib>
 #include <cstring>
 #include <map>
+#include <memory>
 #include <mutex>
 #include <tuple>
 #include <vector>
@@ -287,7 +288,7 @@ extern "C" {
 void _mlir_ciface_buddy_dequant_matmul_i8_f32(buddy_memref_f32_2d *result,
                                               buddy_memref_f32_2d *A,
                                               buddy_memref_i8_2d *W,
-                                              buddy_memref_f32_2d *scale) {
+                                              buddy_memref_f32_2d *scale) try {
   if (!result)
     return;
   result->allocated = nullptr;
@@ -301,22 +302,22 @@ void _mlir_ciface_buddy_dequant_matmul_i8_f32(buddy_memref_f32_2d *result,
     bh::fail(BUDDY_HIP_ERR_ARG, "dequant_matmul: empty operand");
     return;
   }
-  float *out = static_cast<float *>(malloc(sizeof(float) * (size_t)(M * N)));
+  // freed again unless the product succeeds (also when an exception passes by)
+  std::unique_ptr<float, decltype(&free)> out(
+      static_cast<float *>(malloc(sizeof(float) * (size_t)(M * N))), &free);
   if (!out) {
-    bh::fail(BUDDY_HIP_ERR_ARG, "dequant_matmul: out of host memory");
+    bh::fail(BUDDY_HIP_ERR_HOST, "dequant_matmul: out of host memory");
     return;
   }
-  if (bh::dequant_matmul(A, W, scale, out, false, N, false) != BUDDY_HIP_OK) {
-    free(out);
+  if (bh::dequant_matmul(A, W, scale, out.get(), false, N, false) != BUDDY_HIP_OK)
     return;
-  }
-  bh::fill_result(result, out, M, N);
-}
+  bh::fill_result(result, out.release(), M, N);
+} BH_CATCH_VOID("_mlir_ciface_buddy_dequant_matmul_i8_f32")
 
 void _mlir_ciface_buddy_dequant_matmul_i8_f32_acc(buddy_memref_f32_2d *C,
                                                   buddy_memref_f32_2d *A,
                                                   buddy_memref_i8_2d *W,
-                                                  buddy_memref_f32_2d *scale) {
+                                                  buddy_memref_f32_2d *scale) try {
   if (!C || !C->aligned || !A || !W) {
     bh::fail(BUDDY_HIP_ERR_ARG, "dequant_matmul_acc: null descriptor");
     return;
@@ -330,9 +331,9 @@ void _mlir_ciface_buddy_dequant_matmul_i8_f32_acc(buddy_memref_f32_2d *C,
   float *c = C->aligned + C->offset;
   (void)bh::dequant_matmul(A, W, scale, c, bh::is_device_pointer(c),
                            C->strides[0], true);
-}
+} BH_CATCH_VOID("_mlir_ciface_buddy_dequant_matmul_i8_f32_acc")
 
-void buddy_hip_clear_weight_cache(void) {
+void buddy_hip_clear_weight_cache(void) try {
   bh::OpContext &c = bh::ctx();
   std::lock_guard<std::mutex> lock(c.mu);
   if (c.stream)
@@ -342,5 +343,5 @@ void buddy_hip_clear_weight_cache(void) {
     (void)hipFree(kv.second.scale);
   }
   c.weights.clear();
-}
+} BH_CATCH_VOID("buddy_hip_clear_weight_cache")
 }

@@ -2,6 +2,8 @@
 #include "common.h"
 
 #include <cstring>
+#include <exception>
+#include <new>
 
 namespace bh {
 namespace {
@@ -15,6 +17,18 @@ int fail(int code, const char *fmt, ...) {
   va_end(ap);
   fprintf(stderr, "[buddy_hip] %s\n", g_last_error);
   return code;
+}
+
+int caught(const char *where) noexcept {
+  try {
+    throw; // the exception being handled by the caller's catch (...)
+  } catch (const std::bad_alloc &) {
+    return fail(BUDDY_HIP_ERR_HOST, "%s: out of host memory", where);
+  } catch (const std::exception &e) {
+    return fail(BUDDY_HIP_ERR_HOST, "%s: %s", where, e.what());
+  } catch (...) {
+    return fail(BUDDY_HIP_ERR_HOST, "%s: unknown C++ exception", where);
+  }
 }
 } // namespace bh
 

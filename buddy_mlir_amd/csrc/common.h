@@ -30,6 +30,24 @@ int fail(int code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
       return ::bh::fail(BUDDY_HIP_ERR_ARG, __VA_ARGS__);                       \
   } while (0)
 
+// What an exported function does when a C++ exception reaches its outermost
+// scope (a std::vector that cannot grow, a standard-library error): message on
+// stderr and in buddy_hip_last_error(), then an ordinary error return, like the
+// reference's external kernels (examples/BuddyOneDNN/onednn_ops.cpp:229-241).
+// Every extern "C" definition is a function-try-block ending in one of the
+// BH_CATCH_* handlers, so nothing unwinds through the C ABI.
+int caught(const char *where) noexcept;
+
+#define BH_CATCH_INT(name)                                                     \
+  catch (...) { return ::bh::caught(name); }
+#define BH_CATCH_VOID(name)                                                    \
+  catch (...) { (void)::bh::caught(name); }
+#define BH_CATCH_NULL(name)                                                    \
+  catch (...) {                                                                \
+    (void)::bh::caught(name);                                                  \
+    return nullptr;                                                            \
+  }
+
 inline hipStream_t as_stream(buddy_hip_stream s) {
   return reinterpret_cast<hipStream_t>(s);
 }

@@ -29,6 +29,6 @@ int launch_argmax_partial(const float *x, int n, void *workspace, int *nparts_ou
 int launch_finish_step(void *amax_workspace, int nparts, int *state, int *token_log,
                        const float *table, int64_t hidden, int64_t vocab, float *x,
                        const float *inv_freq, int head_dim, float *rope, bool advance,
-                       hipStream_t stream);
+                       int token_log_cap, hipStream_t stream);
 
 } // namespace bh

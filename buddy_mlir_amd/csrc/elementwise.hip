@@ -143,7 +143,7 @@ finish_step_kernel(const float *__restrict__ pv, const int *__restrict__ pi,
                    int nparts, int *__restrict__ state, int *__restrict__ token_log,
                    const float *__restrict__ table, int64_t hidden, int64_t vocab,
                    float *__restrict__ x, const float *__restrict__ inv_freq,
-                   int half, float *__restrict__ rope, int advance) {
+                   int half, float *__restrict__ rope, int advance, int log_cap) {
   __shared__ float sv[4];
   __shared__ int si[4];
   __shared__ int s_tok, s_pos;
@@ -165,7 +165,9 @@ finish_step_kernel(const float *__restrict__ pv, const int *__restrict__ pi,
         amax_merge(v, idx, sv[w], si[w]);
       if (idx == 0x7fffffff)
         idx = 0;
-      token_log[state[2]] = idx;
+      // the host bounds the step count; a counter outside the log writes nothing
+      if ((unsigned)state[2] < (unsigned)log_cap)
+        token_log[state[2]] = idx;
       state[0] = idx;
     }
   }
@@ -197,7 +199,7 @@ finish_step_kernel(const float *__restrict__ pv, const int *__restrict__ pi,
 int launch_finish_step(void *amax_workspace, int nparts, int *state, int *token_log,
                        const float *table, int64_t hidden, int64_t vocab, float *x,
                        const float *inv_freq, int head_dim, float *rope, bool advance,
-                       hipStream_t stream) {
+                       int token_log_cap, hipStream_t stream) {
   BH_REQUIRE(state && table && x && inv_freq && rope && head_dim > 0 &&
                  head_dim / 2 <= 256 && (nparts == 0 || (amax_workspace && token_log)),
              "finish_step: bad argument");
@@ -205,7 +207,7 @@ int launch_finish_step(void *amax_workspace, int nparts, int *state, int *token_
   const int *pi = reinterpret_cast<const int *>(pv + kArgmaxParts);
   hipLaunchKernelGGL(finish_step_kernel, dim3(1), dim3(256), 0, stream, pv, pi, nparts,
                      state, token_log, table, hidden, vocab, x, inv_freq, head_dim / 2,
-                     rope, advance ? 1 : 0);
+                     rope, advance ? 1 : 0, token_log_cap);
   BH_CHECK_HIP(hipGetLastError());
   return BUDDY_HIP_OK;
 }
@@ -290,28 +292,28 @@ int launch_argmax(const float *x, int n, void *workspace, int *out_token,
 extern "C" {
 
 int buddy_hip_rmsnorm(const float *x, const float *w, float *y, int rows, int n,
-                      float eps, buddy_hip_stream stream) {
+                      float eps, buddy_hip_stream stream) try {
   return bh::launch_rmsnorm(x, w, y, rows, n, eps, bh::as_stream(stream));
-}
+} BH_CATCH_INT("buddy_hip_rmsnorm")
 
 int buddy_hip_rope(float *x, const float *inv_freq, const int *pos, int n_heads,
-                   int head_dim, buddy_hip_stream stream) {
+                   int head_dim, buddy_hip_stream stream) try {
   return bh::launch_rope(x, inv_freq, pos, n_heads, head_dim,
                          bh::as_stream(stream));
-}
+} BH_CATCH_INT("buddy_hip_rope")
 
 int buddy_hip_silu_mul(const float *g, const float *u, float *h, int64_t n,
-                       buddy_hip_stream stream) {
+                       buddy_hip_stream stream) try {
   return bh::launch_silu_mul(g, u, h, n, bh::as_stream(stream));
-}
+} BH_CATCH_INT("buddy_hip_silu_mul")
 
 size_t buddy_hip_argmax_workspace_bytes(void) {
   return bh::argmax_workspace_bytes();
 }
 
 int buddy_hip_argmax(const float *x, int n, void *workspace, int *out_index,
-                     buddy_hip_stream stream) {
+                     buddy_hip_stream stream) try {
   return bh::launch_argmax(x, n, workspace, out_index, nullptr, nullptr,
                            bh::as_stream(stream));
-}
+} BH_CATCH_INT("buddy_hip_argmax")
 }

@@ -722,7 +722,7 @@ extern "C" {
 
 int buddy_hip_gemm_w8a32(const float *A, const int8_t *packed, const float *scale,
                          float *C, int64_t M, int64_t K, int64_t N,
-                         unsigned flags, buddy_hip_stream stream) {
+                         unsigned flags, buddy_hip_stream stream) try {
   bh::GemmW8Args a;
   a.A = A;
   a.lda = K;
@@ -737,5 +737,5 @@ int buddy_hip_gemm_w8a32(const float *A, const int8_t *packed, const float *scal
   a.terms = (flags & BUDDY_HIP_GEMM_A_F32_EXACT) ? 3 : 1;
   a.digits = (flags & BUDDY_HIP_GEMM_A_I8_DIGITS) ? 3 : 0;
   return bh::launch_gemm_w8(a, bh::as_stream(stream));
-}
+} BH_CATCH_INT("buddy_hip_gemm_w8a32")
 }

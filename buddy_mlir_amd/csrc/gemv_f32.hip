@@ -314,11 +314,11 @@ extern "C" {
 
 int buddy_hip_gemv_f32(const float *x, const float *B, const float *bias,
                        float *y, int64_t K, int64_t N, unsigned flags,
-                       buddy_hip_stream stream) {
+                       buddy_hip_stream stream) try {
   return bh::launch_gemv_f32(x, B, bias, y, K, N, N,
                              (flags & BUDDY_HIP_GEMV_ACCUMULATE) != 0,
                              bh::as_stream(stream));
-}
+} BH_CATCH_INT("buddy_hip_gemv_f32")
 }
 
 extern "C" {
@@ -329,15 +329,15 @@ size_t buddy_hip_f32_tiles_bytes(int64_t K, int64_t N) {
 }
 
 int buddy_hip_tile_f32(const float *B, int64_t K, int64_t N, float *tiles,
-                       buddy_hip_stream stream) {
+                       buddy_hip_stream stream) try {
   return bh::launch_tile_f32(B, K, N, N, tiles, bh::as_stream(stream));
-}
+} BH_CATCH_INT("buddy_hip_tile_f32")
 
 int buddy_hip_gemv_f32_tiles(const float *x, const float *tiles, const float *bias,
                              const float *norm_w, float norm_eps, float *y, int64_t K,
-                             int64_t N, unsigned flags, buddy_hip_stream stream) {
+                             int64_t N, unsigned flags, buddy_hip_stream stream) try {
   return bh::launch_gemv_f32_tiles(x, tiles, bias, norm_w, norm_eps, y, K, N,
                                    (flags & BUDDY_HIP_GEMV_ACCUMULATE) != 0,
                                    bh::as_stream(stream));
-}
+} BH_CATCH_INT("buddy_hip_gemv_f32_tiles")
 }

@@ -37,7 +37,7 @@ pack_panels_kernel(const float *__restrict__ B, float *__restrict__ P, int64_t K
 extern "C" {
 
 int buddy_hip_pack_panels_f32(const float *B, int64_t K, int64_t N, int V,
-                              float *packed, buddy_hip_stream stream) {
+                              float *packed, buddy_hip_stream stream) try {
   BH_REQUIRE(B && packed && K > 0 && N > 0 && V > 0, "pack_panels: bad argument");
   // pack_decode_weights.py:95-99 refuses a ragged last panel
   BH_REQUIRE(N % V == 0, "pack_panels: N=%lld not divisible by V=%d", (long long)N, V);
@@ -45,23 +45,23 @@ int buddy_hip_pack_panels_f32(const float *B, int64_t K, int64_t N, int V,
                      dim3(256), 0, bh::as_stream(stream), B, packed, K, N, V, 0);
   BH_CHECK_HIP(hipGetLastError());
   return BUDDY_HIP_OK;
-}
+} BH_CATCH_INT("buddy_hip_pack_panels_f32")
 
 int buddy_hip_unpack_panels_f32(const float *packed, int64_t K, int64_t N, int V,
-                                float *B, buddy_hip_stream stream) {
+                                float *B, buddy_hip_stream stream) try {
   BH_REQUIRE(B && packed && K > 0 && N > 0 && V > 0, "unpack_panels: bad argument");
   BH_REQUIRE(N % V == 0, "unpack_panels: N=%lld not divisible by V=%d", (long long)N, V);
   hipLaunchKernelGGL(bh::pack_panels_kernel, dim3((unsigned)bh::ceil_div(K * N, 256)),
                      dim3(256), 0, bh::as_stream(stream), packed, B, K, N, V, 1);
   BH_CHECK_HIP(hipGetLastError());
   return BUDDY_HIP_OK;
-}
+} BH_CATCH_INT("buddy_hip_unpack_panels_f32")
 
 int buddy_hip_gemv_f32_panels(const float *x, const float *packed, float *y,
                               int64_t K, int64_t N, unsigned flags,
-                              buddy_hip_stream stream) {
+                              buddy_hip_stream stream) try {
   return bh::launch_gemv_f32_panels32(x, packed, y, K, N,
                                       (flags & BUDDY_HIP_GEMV_ACCUMULATE) != 0,
                                       bh::as_stream(stream));
-}
+} BH_CATCH_INT("buddy_hip_gemv_f32_panels")
 }

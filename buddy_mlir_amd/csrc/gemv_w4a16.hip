@@ -279,17 +279,17 @@ pack_int4_kernel(const int8_t *__restrict__ q, int64_t pairs, int8_t *__restrict
 extern "C" {
 
 int buddy_hip_pack_int4(const int8_t *q, int64_t count, int8_t *packed,
-                        buddy_hip_stream stream) {
+                        buddy_hip_stream stream) try {
   BH_REQUIRE(q && packed && count > 0, "pack_int4: bad argument");
   BH_REQUIRE(count % 2 == 0, "pack_int4: odd element count %lld", (long long)count);
   hipLaunchKernelGGL(bh::pack_int4_kernel, dim3((unsigned)bh::ceil_div(count / 2, 256)),
                      dim3(256), 0, bh::as_stream(stream), q, count / 2, packed);
   BH_CHECK_HIP(hipGetLastError());
   return BUDDY_HIP_OK;
-}
+} BH_CATCH_INT("buddy_hip_pack_int4")
 
 int buddy_hip_gemv_w4a16(const uint16_t *A, const int8_t *packed, const uint16_t *scale,
-                         uint16_t *C, int64_t K, int64_t N, buddy_hip_stream stream) {
+                         uint16_t *C, int64_t K, int64_t N, buddy_hip_stream stream) try {
   BH_REQUIRE(A && packed && scale && C, "gemv_w4a16: null pointer");
   BH_REQUIRE(K > 0 && N > 0 && K < (1 << 30) && N < (1 << 30),
              "gemv_w4a16: bad shape K=%lld N=%lld", (long long)K, (long long)N);
@@ -313,5 +313,5 @@ int buddy_hip_gemv_w4a16(const uint16_t *A, const int8_t *packed, const uint16_t
   }
   BH_CHECK_HIP(hipGetLastError());
   return BUDDY_HIP_OK;
-}
+} BH_CATCH_INT("buddy_hip_gemv_w4a16")
 }

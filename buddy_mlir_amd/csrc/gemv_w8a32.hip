@@ -1001,7 +1001,7 @@ int launch_gemv(const GemvArgs &a, hipStream_t stream) {
 extern "C" {
 
 int buddy_hip_linear_w8a32(const buddy_hip_linear_desc *d,
-                           buddy_hip_stream stream) {
+                           buddy_hip_stream stream) try {
   BH_REQUIRE(d, "linear_w8a32: null descriptor");
   bh::GemvArgs a;
   a.A = d->A;
@@ -1026,11 +1026,11 @@ int buddy_hip_linear_w8a32(const buddy_hip_linear_desc *d,
   BH_REQUIRE(!(d->bias && d->epilogue != BUDDY_HIP_EPI_STORE),
              "linear_w8a32: bias only with the STORE epilogue");
   return bh::launch_gemv(a, bh::as_stream(stream));
-}
+} BH_CATCH_INT("buddy_hip_linear_w8a32")
 
 int buddy_hip_gemv_w8a32(const float *A, const int8_t *packed,
                          const float *scale, float *C, int64_t M, int64_t K,
-                         int64_t N, unsigned flags, buddy_hip_stream stream) {
+                         int64_t N, unsigned flags, buddy_hip_stream stream) try {
   BH_REQUIRE(M >= 1, "gemv_w8a32: M=%lld", (long long)M);
   // rows beyond 16 go in slabs; each slab streams the weights once
   for (int64_t m0 = 0; m0 < M; m0 += 16) {
@@ -1051,5 +1051,5 @@ int buddy_hip_gemv_w8a32(const float *A, const int8_t *packed,
       return rc;
   }
   return BUDDY_HIP_OK;
-}
+} BH_CATCH_INT("buddy_hip_gemv_w8a32")
 }

@@ -129,7 +129,7 @@ size_t buddy_hip_w8a8_workspace_bytes(int64_t M, int64_t K) {
 int buddy_hip_w8a8_matmul(const float *A, const int8_t *packed, const float *wscale,
                           float *C, int32_t *acc_out, int64_t M, int64_t K,
                           int64_t N, void *workspace, size_t workspace_bytes,
-                          buddy_hip_stream stream) {
+                          buddy_hip_stream stream) try {
   BH_REQUIRE(A && packed && wscale && C && workspace, "w8a8_matmul: null pointer");
   BH_REQUIRE(M >= 1 && M <= 16, "w8a8_matmul: M=%lld outside 1..16", (long long)M);
   BH_REQUIRE(K > 0 && N > 0 && K < (1 << 30) && N < (1 << 30), "w8a8_matmul: bad shape");
@@ -161,5 +161,5 @@ int buddy_hip_w8a8_matmul(const float *A, const int8_t *packed, const float *wsc
 #undef BH_W8A8
   BH_CHECK_HIP(hipGetLastError());
   return BUDDY_HIP_OK;
-}
+} BH_CATCH_INT("buddy_hip_w8a8_matmul")
 }

@@ -73,7 +73,55 @@ __global__ void __launch_bounds__(256) kv_discard_kernel(DiscardArgs a) {
   }
 }
 
+struct GatherArgs {
+  const float *tensor[kMaxTensors];
+  int tensors, heads, max_len, dim, row0, rows;
+};
+
+// dst[((tensor * heads + head) * rows + r) * dim + d] = cache row row0 + r
+__global__ void __launch_bounds__(256)
+kv_gather_rows_kernel(GatherArgs a, float *__restrict__ dst) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const int64_t per_tensor = (int64_t)a.heads * a.rows * a.dim;
+  if (i >= a.tensors * per_tensor)
+    return;
+  const int tn = (int)(i / per_tensor);
+  const int64_t rem = i % per_tensor;
+  const int h = (int)(rem / ((int64_t)a.rows * a.dim));
+  const int r = (int)(rem / a.dim % a.rows), d = (int)(rem % a.dim);
+  dst[i] = a.tensor[tn][((size_t)h * a.max_len + a.row0 + r) * a.dim + d];
+}
+
 } // namespace
+
+int launch_kv_gather_rows(const float *const *tensors, int num_tensors, int heads,
+                          int max_len, int head_dim, int row0, int rows, float *dst,
+                          hipStream_t stream) {
+  BH_REQUIRE(tensors && dst && num_tensors > 0 && heads > 0 && head_dim > 0,
+             "kv_gather_rows: bad argument");
+  BH_REQUIRE(row0 >= 0 && rows > 0 && (int64_t)row0 + rows <= max_len,
+             "kv_gather_rows: rows %d..%d outside the cache (max_len %d)", row0,
+             row0 + rows - 1, max_len);
+  for (int t0 = 0; t0 < num_tensors; t0 += kMaxTensors) {
+    GatherArgs a;
+    a.tensors = num_tensors - t0 < kMaxTensors ? num_tensors - t0 : kMaxTensors;
+    for (int i = 0; i < kMaxTensors; ++i) {
+      a.tensor[i] = i < a.tensors ? tensors[t0 + i] : nullptr;
+      BH_REQUIRE(i >= a.tensors || a.tensor[i], "kv_gather_rows: tensor %d is null", t0 + i);
+    }
+    a.heads = heads;
+    a.max_len = max_len;
+    a.dim = head_dim;
+    a.row0 = row0;
+    a.rows = rows;
+    const int64_t per_tensor = (int64_t)heads * rows * head_dim;
+    hipLaunchKernelGGL(kv_gather_rows_kernel,
+                       dim3((unsigned)ceil_div(a.tensors * per_tensor, 256)), dim3(256), 0,
+                       stream, a, dst + (size_t)t0 * per_tensor);
+    BH_CHECK_HIP(hipGetLastError());
+  }
+  return BUDDY_HIP_OK;
+}
 
 int launch_kv_discard(float *const *tensors, int num_tensors, int heads, int max_len,
                       int head_dim, int keep, int discard, int count,
@@ -139,8 +187,8 @@ extern "C" {
 
 int buddy_hip_kv_discard(float *const *tensors, int num_tensors, int heads, int max_len,
                          int head_dim, int keep, int discard, int count,
-                         const float *inv_freq, buddy_hip_stream stream) {
+                         const float *inv_freq, buddy_hip_stream stream) try {
   return bh::launch_kv_discard(tensors, num_tensors, heads, max_len, head_dim, keep,
                                discard, count, inv_freq, bh::as_stream(stream));
-}
+} BH_CATCH_INT("buddy_hip_kv_discard")
 }

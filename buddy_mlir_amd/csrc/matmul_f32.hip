@@ -104,15 +104,15 @@ extern "C" {
 
 int buddy_hip_matmul_f32(const float *A, const float *B, float *C, int64_t M,
                          int64_t N, int64_t K, unsigned flags,
-                         buddy_hip_stream stream) {
+                         buddy_hip_stream stream) try {
   return bh::launch_matmul_f32(A, B, C, M, N, K, K, N, N,
                                (flags & BUDDY_HIP_GEMV_ACCUMULATE) != 0,
                                bh::as_stream(stream));
-}
+} BH_CATCH_INT("buddy_hip_matmul_f32")
 
 void _mlir_ciface_buddy_matmul_f32(buddy_memref_f32_2d *result,
                                    buddy_memref_f32_2d *A,
-                                   buddy_memref_f32_2d *B) {
+                                   buddy_memref_f32_2d *B) try {
   if (!result)
     return;
   result->allocated = nullptr;
@@ -164,5 +164,5 @@ void _mlir_ciface_buddy_matmul_f32(buddy_memref_f32_2d *result,
   result->sizes[1] = N;
   result->strides[0] = N;
   result->strides[1] = 1;
-}
+} BH_CATCH_VOID("_mlir_ciface_buddy_matmul_f32")
 }

@@ -166,7 +166,7 @@ size_t buddy_hip_w8_packed_bytes(int64_t K, int64_t N) {
 }
 
 int buddy_hip_pack_w8_tiles(const int8_t *W, int64_t K, int64_t N, int tile_n,
-                            int8_t *packed, buddy_hip_stream stream) {
+                            int8_t *packed, buddy_hip_stream stream) try {
   BH_REQUIRE(W && packed, "pack_w8: null pointer");
   BH_REQUIRE(K > 0 && N > 0, "pack_w8: bad shape K=%lld N=%lld", (long long)K,
              (long long)N);
@@ -179,15 +179,15 @@ int buddy_hip_pack_w8_tiles(const int8_t *W, int64_t K, int64_t N, int tile_n,
                      lanes, tile_n, packed);
   BH_CHECK_HIP(hipGetLastError());
   return BUDDY_HIP_OK;
-}
+} BH_CATCH_INT("buddy_hip_pack_w8_tiles")
 
 int buddy_hip_pack_w8(const int8_t *W, int64_t K, int64_t N, int8_t *packed,
-                      buddy_hip_stream stream) {
+                      buddy_hip_stream stream) try {
   return buddy_hip_pack_w8_tiles(W, K, N, bh::kTileN, packed, stream);
-}
+} BH_CATCH_INT("buddy_hip_pack_w8")
 
 int buddy_hip_unpack_w8_tiles(const int8_t *packed, int64_t K, int64_t N,
-                              int tile_n, int8_t *W, buddy_hip_stream stream) {
+                              int tile_n, int8_t *W, buddy_hip_stream stream) try {
   BH_REQUIRE(W && packed, "unpack_w8: null pointer");
   BH_REQUIRE(K > 0 && N > 0, "unpack_w8: bad shape K=%lld N=%lld", (long long)K,
              (long long)N);
@@ -198,12 +198,12 @@ int buddy_hip_unpack_w8_tiles(const int8_t *packed, int64_t K, int64_t N,
                      bh::as_stream(stream), packed, K, N, chunks, tile_n, W);
   BH_CHECK_HIP(hipGetLastError());
   return BUDDY_HIP_OK;
-}
+} BH_CATCH_INT("buddy_hip_unpack_w8_tiles")
 
 int buddy_hip_unpack_w8(const int8_t *packed, int64_t K, int64_t N, int8_t *W,
-                        buddy_hip_stream stream) {
+                        buddy_hip_stream stream) try {
   return buddy_hip_unpack_w8_tiles(packed, K, N, bh::kTileN, W, stream);
-}
+} BH_CATCH_INT("buddy_hip_unpack_w8")
 
 static int quantize_per_channel(const float *W, int64_t K, int64_t N, int8_t *q,
                                 float *scale, float qmax, float lo, float hi,
@@ -244,12 +244,12 @@ static int quantize_per_channel(const float *W, int64_t K, int64_t N, int8_t *q,
 }
 
 int buddy_hip_quantize_w8(const float *W, int64_t K, int64_t N, int8_t *q,
-                          float *scale, buddy_hip_stream stream) {
+                          float *scale, buddy_hip_stream stream) try {
   return quantize_per_channel(W, K, N, q, scale, 127.0f, -128.0f, 127.0f, stream);
-}
+} BH_CATCH_INT("buddy_hip_quantize_w8")
 
 int buddy_hip_quantize_w4(const float *W, int64_t K, int64_t N, int8_t *q,
-                          float *scale, buddy_hip_stream stream) {
+                          float *scale, buddy_hip_stream stream) try {
   return quantize_per_channel(W, K, N, q, scale, 7.0f, -8.0f, 7.0f, stream);
-}
+} BH_CATCH_INT("buddy_hip_quantize_w4")
 }

@@ -344,7 +344,7 @@ int draw(buddy_hip_sampler *s, const std::vector<std::pair<int, float>> &cand) {
 
 extern "C" {
 
-buddy_hip_sampler *buddy_hip_sampler_create(const buddy_hip_sampler_config *cfg) {
+buddy_hip_sampler *buddy_hip_sampler_create(const buddy_hip_sampler_config *cfg) try {
   if (!cfg || cfg->temperature < 0.0f || cfg->top_k < 0 || cfg->repeat_last_n < 0 ||
       !(cfg->repeat_penalty > 0.0f)) {
     bh::fail(BUDDY_HIP_ERR_ARG, "sampler_create: bad configuration");
@@ -374,9 +374,9 @@ buddy_hip_sampler *buddy_hip_sampler_create(const buddy_hip_sampler_config *cfg)
     return nullptr;
   }
   return s;
-}
+} BH_CATCH_NULL("buddy_hip_sampler_create")
 
-void buddy_hip_sampler_destroy(buddy_hip_sampler *s) {
+void buddy_hip_sampler_destroy(buddy_hip_sampler *s) try {
   if (!s)
     return;
   for (void *p : {(void *)s->d_hist, (void *)s->d_keys, (void *)s->d_cand, (void *)s->d_partial,
@@ -387,11 +387,11 @@ void buddy_hip_sampler_destroy(buddy_hip_sampler *s) {
     if (p)
       (void)hipHostFree(p);
   delete s;
-}
+} BH_CATCH_VOID("buddy_hip_sampler_destroy")
 
 int buddy_hip_sampler_sample(buddy_hip_sampler *s, const float *logits, int vocab,
                              const int *recent, int n_recent, int *token_out,
-                             buddy_hip_stream hstream) {
+                             buddy_hip_stream hstream) try {
   BH_REQUIRE(s && logits && token_out && vocab > 0 && n_recent >= 0 && (recent || !n_recent),
              "sampler_sample: bad argument");
   hipStream_t stream = bh::as_stream(hstream);
@@ -501,11 +501,11 @@ int buddy_hip_sampler_sample(buddy_hip_sampler *s, const float *logits, int voca
   }
   *token_out = cand[(size_t)bh::draw(s, cand)].first;
   return BUDDY_HIP_OK;
-}
+} BH_CATCH_INT("buddy_hip_sampler_sample")
 
 int buddy_hip_session_decode_sample(buddy_hip_session *sess, buddy_hip_sampler *s, int token,
                                     int pos, const int *recent, int n_recent,
-                                    int *next_token) {
+                                    int *next_token) try {
   BH_REQUIRE(sess && s && next_token, "session_decode_sample: null argument");
   int rc = buddy_hip_session_set_state(sess, token, pos);
   if (rc)
@@ -514,5 +514,5 @@ int buddy_hip_session_decode_sample(buddy_hip_session *sess, buddy_hip_sampler *
     return rc;
   return buddy_hip_sampler_sample(s, buddy_hip_session_logits(sess), buddy_hip_session_vocab(sess),
                                   recent, n_recent, next_token, buddy_hip_session_stream(sess));
-}
+} BH_CATCH_INT("buddy_hip_session_decode_sample")
 }

@@ -104,6 +104,10 @@ struct Session {
   int *token_log = nullptr; // device: greedy tokens by step
   int token_log_cap = 0;
   int *host_state = nullptr; // pinned staging for token/pos/step
+  // Host-side mirror of the device's (position, step): what the next enqueued
+  // step will use.  -1 until set_state; every step advances both on the device,
+  // so the host can refuse steps that would leave the cache or the token log.
+  int next_pos = -1, next_step = 0;
   hipGraph_t graph = nullptr;
   hipGraphExec_t graph_exec = nullptr;
   bool use_graph = true;
@@ -113,6 +117,8 @@ struct Session {
   float *pf_x = nullptr, *pf_xn = nullptr, *pf_qkv = nullptr, *pf_att = nullptr,
         *pf_g = nullptr, *pf_u = nullptr;
   int *pf_tokens = nullptr;
+  float *kv_rows = nullptr; // staging of get_kv_rows, grown on demand
+  size_t kv_rows_cap = 0;
   unsigned short *pf_xn_bf = nullptr, *pf_g_bf = nullptr; // bf16 matmul inputs
   int gemm_terms = 3; // bf16 terms per activation in the prefill matmuls (3 = exact)
   int gemm_digits = 3; // int8 digit planes instead of bf16 terms when not 0
@@ -251,14 +257,16 @@ struct Session {
     if ((rc = launch_argmax_partial(logits, S.vocab, amax_ws, &nparts, stream)))
       return rc;
     return launch_finish_step(amax_ws, nparts, state, token_log, embed, S.hidden,
-                              S.vocab, x, inv_freq, S.head_dim, rope, true, stream);
+                              S.vocab, x, inv_freq, S.head_dim, rope, true,
+                              token_log_cap, stream);
   }
 
   // After the host wrote token/position: embedding row and RoPE table of the step.
   int prepare_step() {
     const auto &S = shape;
     return launch_finish_step(amax_ws, 0, state, token_log, embed, S.hidden, S.vocab,
-                              x, inv_freq, S.head_dim, rope, false, stream);
+                              x, inv_freq, S.head_dim, rope, false, token_log_cap,
+                              stream);
   }
 
   int ensure_prefill_buffers(int rows) {
@@ -271,8 +279,10 @@ struct Session {
         (void)hipFree(*p);
         *p = nullptr;
       }
-    if (pf_tokens)
+    if (pf_tokens) {
       (void)hipFree(pf_tokens);
+      pf_tokens = nullptr;
+    }
     for (unsigned short **p : {&pf_xn_bf, &pf_g_bf})
       if (*p) {
         (void)hipFree(*p);
@@ -437,25 +447,63 @@ struct Session {
     return BUDDY_HIP_OK;
   }
 
+  // The position and step the device holds must stay inside the cache and the
+  // token log for every one of `steps` further steps.
+  int check_steps(int steps, const char *who) const {
+    BH_REQUIRE(next_pos >= 0, "%s: no token / position set (set_state first)", who);
+    BH_REQUIRE(steps > 0 && (int64_t)next_pos + steps <= shape.max_len,
+               "%s: %d step(s) from position %d leave the cache (max_len %d)", who, steps,
+               next_pos, shape.max_len);
+    BH_REQUIRE((int64_t)next_step + steps <= token_log_cap,
+               "%s: %d step(s) from step %d overflow the token log (%d entries)", who,
+               steps, next_step, token_log_cap);
+    return BUDDY_HIP_OK;
+  }
+
   int run_step() {
-    if (!use_graph)
-      return enqueue_step();
-    if (!graph_exec) {
-      BH_CHECK_HIP(hipStreamBeginCapture(stream, hipStreamCaptureModeThreadLocal));
-      int rc = enqueue_step();
-      hipError_t e = hipStreamEndCapture(stream, &graph);
-      if (rc)
-        return rc;
-      if (e != hipSuccess)
-        return fail(BUDDY_HIP_ERR_HIP, "hipStreamEndCapture: %s",
-                    hipGetErrorString(e));
-      BH_CHECK_HIP(hipGraphInstantiate(&graph_exec, graph, nullptr, nullptr, 0));
+    int rc = check_steps(1, "decode step");
+    if (rc)
+      return rc;
+    if (!use_graph) {
+      rc = enqueue_step();
+    } else {
+      if (!graph_exec) {
+        BH_CHECK_HIP(hipStreamBeginCapture(stream, hipStreamCaptureModeThreadLocal));
+        rc = enqueue_step();
+        hipError_t e = hipStreamEndCapture(stream, &graph);
+        if (!rc && e != hipSuccess)
+          rc = fail(BUDDY_HIP_ERR_HIP, "hipStreamEndCapture: %s", hipGetErrorString(e));
+        if (!rc && (e = hipGraphInstantiate(&graph_exec, graph, nullptr, nullptr, 0)) !=
+                       hipSuccess)
+          rc = fail(BUDDY_HIP_ERR_HIP, "hipGraphInstantiate: %s", hipGetErrorString(e));
+        if (rc) {
+          drop_graph(); // a half-built graph is not kept
+          return rc;
+        }
+      }
+      BH_CHECK_HIP(hipGraphLaunch(graph_exec, stream));
     }
-    BH_CHECK_HIP(hipGraphLaunch(graph_exec, stream));
+    if (!rc) {
+      ++next_pos;
+      ++next_step;
+    }
+    return rc;
+  }
+
+  // The captured step has kernel arguments baked in (weight, cache and embedding
+  // pointers): whoever may change one of them drops the graph first, and the
+  // next step captures a new one.
+  int invalidate_graph() {
+    if (graph_exec || graph) {
+      BH_CHECK_HIP(hipStreamSynchronize(stream));
+      drop_graph();
+    }
     return BUDDY_HIP_OK;
   }
 
   int set_state(int token, int pos, int step) {
+    next_pos = pos;
+    next_step = step;
     host_state[0] = token;
     host_state[1] = pos;
     host_state[2] = step;
@@ -477,7 +525,7 @@ using bh::Session;
 extern "C" {
 
 buddy_hip_session *buddy_hip_session_create(const buddy_hip_model_shape *shape,
-                                            buddy_hip_stream stream) {
+                                            buddy_hip_stream stream) try {
   if (!shape) {
     bh::fail(BUDDY_HIP_ERR_ARG, "session_create: null shape");
     return nullptr;
@@ -549,9 +597,9 @@ buddy_hip_session *buddy_hip_session_create(const buddy_hip_model_shape *shape,
     return nullptr;
   }
   return reinterpret_cast<buddy_hip_session *>(s);
-}
+} BH_CATCH_NULL("buddy_hip_session_create")
 
-void buddy_hip_session_destroy(buddy_hip_session *hs) {
+void buddy_hip_session_destroy(buddy_hip_session *hs) try {
   Session *s = reinterpret_cast<Session *>(hs);
   if (!s)
     return;
@@ -561,7 +609,7 @@ void buddy_hip_session_destroy(buddy_hip_session *hs) {
   for (void *p : s->owned)
     (void)hipFree(p);
   for (void *p : {(void *)s->pf_x, (void *)s->pf_xn, (void *)s->pf_qkv, (void *)s->pf_att,
-                  (void *)s->pf_g, (void *)s->pf_tokens,
+                  (void *)s->pf_g, (void *)s->pf_tokens, (void *)s->kv_rows,
                   (void *)s->pf_xn_bf, (void *)s->pf_g_bf})
     if (p)
       (void)hipFree(p);
@@ -571,15 +619,18 @@ void buddy_hip_session_destroy(buddy_hip_session *hs) {
   if (s->own_stream)
     (void)hipStreamDestroy(s->stream);
   delete s;
-}
+} BH_CATCH_VOID("buddy_hip_session_destroy")
 
 int buddy_hip_session_set_globals(buddy_hip_session *hs, const float *embed,
                                   const float *inv_freq, const float *ln_f,
-                                  const int8_t *w_lm, const float *s_lm) {
+                                  const int8_t *w_lm, const float *s_lm) try {
   Session *s = reinterpret_cast<Session *>(hs);
   BH_REQUIRE(s && embed && inv_freq && ln_f && w_lm && s_lm,
              "session_set_globals: null argument");
   const auto &S = s->shape;
+  int rc0 = s->invalidate_graph(); // the embedding pointer is baked into it
+  if (rc0)
+    return rc0;
   s->embed = embed;
   BH_CHECK_HIP(hipMemcpyAsync(s->inv_freq, inv_freq, sizeof(float) * S.head_dim / 2,
                               hipMemcpyDefault, s->stream));
@@ -601,10 +652,10 @@ int buddy_hip_session_set_globals(buddy_hip_session *hs, const float *embed,
   }
   BH_CHECK_HIP(hipStreamSynchronize(s->stream));
   return BUDDY_HIP_OK;
-}
+} BH_CATCH_INT("buddy_hip_session_set_globals")
 
 int buddy_hip_session_set_layer(buddy_hip_session *hs, int index,
-                                const buddy_hip_layer_weights *w) {
+                                const buddy_hip_layer_weights *w) try {
   Session *s = reinterpret_cast<Session *>(hs);
   BH_REQUIRE(s && w, "session_set_layer: null argument");
   const auto &S = s->shape;
@@ -624,7 +675,9 @@ int buddy_hip_session_set_layer(buddy_hip_session *hs, int index,
   bh::Layer &L = s->layers[(size_t)index];
   const int64_t H = S.hidden, QN = (int64_t)S.heads * S.head_dim,
                 KVN = (int64_t)S.kv_heads * S.head_dim, I = S.inter;
-  int rc = 0;
+  int rc = s->invalidate_graph();
+  if (rc)
+    return rc;
   if (!L.set) {
     // q|k|v share one packed matrix: channel groups are independent, so the
     // three packed blocks simply follow each other
@@ -694,10 +747,10 @@ int buddy_hip_session_set_layer(buddy_hip_session *hs, int index,
   BH_CHECK_HIP(hipStreamSynchronize(s->stream));
   L.set = true;
   return BUDDY_HIP_OK;
-}
+} BH_CATCH_INT("buddy_hip_session_set_layer")
 
 int buddy_hip_session_set_kv(buddy_hip_session *hs, int kv_index,
-                             const float *src) {
+                             const float *src) try {
   Session *s = reinterpret_cast<Session *>(hs);
   BH_REQUIRE(s && src, "session_set_kv: null argument");
   const auto &S = s->shape;
@@ -710,9 +763,9 @@ int buddy_hip_session_set_kv(buddy_hip_session *hs, int kv_index,
                               hipMemcpyDefault, s->stream));
   BH_CHECK_HIP(hipStreamSynchronize(s->stream));
   return BUDDY_HIP_OK;
-}
+} BH_CATCH_INT("buddy_hip_session_set_kv")
 
-int buddy_hip_session_get_kv(buddy_hip_session *hs, int kv_index, float *dst) {
+int buddy_hip_session_get_kv(buddy_hip_session *hs, int kv_index, float *dst) try {
   Session *s = reinterpret_cast<Session *>(hs);
   BH_REQUIRE(s && dst, "session_get_kv: null argument");
   const auto &S = s->shape;
@@ -725,17 +778,52 @@ int buddy_hip_session_get_kv(buddy_hip_session *hs, int kv_index, float *dst) {
                               hipMemcpyDefault, s->stream));
   BH_CHECK_HIP(hipStreamSynchronize(s->stream));
   return BUDDY_HIP_OK;
-}
+} BH_CATCH_INT("buddy_hip_session_get_kv")
 
-int buddy_hip_session_use_graph(buddy_hip_session *hs, int enable) {
+int buddy_hip_session_get_kv_rows(buddy_hip_session *hs, int row0, int rows,
+                                  float *dst) try {
+  Session *s = reinterpret_cast<Session *>(hs);
+  BH_REQUIRE(s && dst, "session_get_kv_rows: null argument");
+  const auto &S = s->shape;
+  BH_REQUIRE(row0 >= 0 && rows > 0 && (int64_t)row0 + rows <= S.max_len,
+             "session_get_kv_rows: rows %d..%d outside the cache (max_len %d)", row0,
+             row0 + rows - 1, S.max_len);
+  const size_t n = (size_t)2 * S.layers * S.kv_heads * rows * S.head_dim;
+  if (n > s->kv_rows_cap) {
+    BH_CHECK_HIP(hipStreamSynchronize(s->stream));
+    if (s->kv_rows)
+      (void)hipFree(s->kv_rows);
+    s->kv_rows = nullptr;
+    s->kv_rows_cap = 0;
+    BH_CHECK_HIP(hipMalloc((void **)&s->kv_rows, sizeof(float) * n));
+    s->kv_rows_cap = n;
+  }
+  std::vector<const float *> tensors;
+  for (auto &L : s->layers) {
+    tensors.push_back(L.kc);
+    tensors.push_back(L.vc);
+  }
+  int rc = bh::launch_kv_gather_rows(tensors.data(), (int)tensors.size(), S.kv_heads,
+                                     S.max_len, S.head_dim, row0, rows, s->kv_rows,
+                                     s->stream);
+  if (rc)
+    return rc;
+  BH_CHECK_HIP(hipMemcpyAsync(dst, s->kv_rows, sizeof(float) * n, hipMemcpyDefault,
+                              s->stream));
+  BH_CHECK_HIP(hipStreamSynchronize(s->stream));
+  return BUDDY_HIP_OK;
+} BH_CATCH_INT("buddy_hip_session_get_kv_rows")
+
+int buddy_hip_session_use_graph(buddy_hip_session *hs, int enable) try {
   Session *s = reinterpret_cast<Session *>(hs);
   BH_REQUIRE(s, "session_use_graph: null session");
   s->use_graph = enable != 0;
   return BUDDY_HIP_OK;
-}
+} BH_CATCH_INT("buddy_hip_session_use_graph")
 
-int buddy_hip_session_decode(buddy_hip_session *hs, int token, int pos,
-                             float *logits_out, int *next_token) {
+int buddy_hip_session_decode_mirror(buddy_hip_session *hs, int token, int pos,
+                                    float *logits_out, float *kv_rows_out,
+                                    int *next_token) try {
   Session *s = reinterpret_cast<Session *>(hs);
   BH_REQUIRE(s, "session_decode: null session");
   int rc = s->ready();
@@ -755,14 +843,23 @@ int buddy_hip_session_decode(buddy_hip_session *hs, int token, int pos,
                                 s->stream));
   BH_CHECK_HIP(hipMemcpyAsync(s->host_state, s->state, 3 * sizeof(int),
                               hipMemcpyDeviceToHost, s->stream));
+  if (kv_rows_out) { // the cache rows this step wrote, all layers
+    if ((rc = buddy_hip_session_get_kv_rows(hs, pos, 1, kv_rows_out)))
+      return rc;
+  }
   BH_CHECK_HIP(hipStreamSynchronize(s->stream));
   if (next_token)
     *next_token = s->host_state[0];
   return BUDDY_HIP_OK;
+} BH_CATCH_INT("buddy_hip_session_decode_mirror")
+
+int buddy_hip_session_decode(buddy_hip_session *hs, int token, int pos,
+                             float *logits_out, int *next_token) {
+  return buddy_hip_session_decode_mirror(hs, token, pos, logits_out, nullptr, next_token);
 }
 
 int buddy_hip_session_decode_greedy(buddy_hip_session *hs, int first_token,
-                                    int start_pos, int steps, int *tokens_out) {
+                                    int start_pos, int steps, int *tokens_out) try {
   Session *s = reinterpret_cast<Session *>(hs);
   BH_REQUIRE(s && tokens_out, "session_decode_greedy: null argument");
   int rc = s->ready();
@@ -784,11 +881,11 @@ int buddy_hip_session_decode_greedy(buddy_hip_session *hs, int first_token,
                               hipMemcpyDefault, s->stream));
   BH_CHECK_HIP(hipStreamSynchronize(s->stream));
   return BUDDY_HIP_OK;
-}
+} BH_CATCH_INT("buddy_hip_session_decode_greedy")
 
 int buddy_hip_session_prefill(buddy_hip_session *hs, const int *tokens,
                               int n_tokens, int start_pos, float *logits_out,
-                              int *next_token) {
+                              int *next_token) try {
   Session *s = reinterpret_cast<Session *>(hs);
   BH_REQUIRE(s && tokens, "session_prefill: null argument");
   int rc = s->ready();
@@ -835,11 +932,11 @@ int buddy_hip_session_prefill(buddy_hip_session *hs, const int *tokens,
   if (next_token)
     *next_token = s->host_state[0];
   return BUDDY_HIP_OK;
-}
+} BH_CATCH_INT("buddy_hip_session_prefill")
 
 int buddy_hip_session_prefill_all_logits(buddy_hip_session *hs, const int *tokens,
                                          int n_tokens, int start_pos,
-                                         float *logits_out) {
+                                         float *logits_out) try {
   Session *s = reinterpret_cast<Session *>(hs);
   BH_REQUIRE(s && tokens && logits_out, "session_prefill_all_logits: null argument");
   int rc = s->ready();
@@ -867,15 +964,15 @@ int buddy_hip_session_prefill_all_logits(buddy_hip_session *hs, const int *token
   (void)hipStreamSynchronize(s->stream);
   (void)hipFree(dev_logits);
   return rc;
-}
+} BH_CATCH_INT("buddy_hip_session_prefill_all_logits")
 
-void buddy_hip_session_adopt(buddy_hip_session *hs, void *device_ptr) {
+void buddy_hip_session_adopt(buddy_hip_session *hs, void *device_ptr) try {
   Session *s = reinterpret_cast<Session *>(hs);
   if (s && device_ptr)
     s->owned.push_back(device_ptr);
-}
+} BH_CATCH_VOID("buddy_hip_session_adopt")
 
-int buddy_hip_session_set_prefill_precision(buddy_hip_session *hs, int mode) {
+int buddy_hip_session_set_prefill_precision(buddy_hip_session *hs, int mode) try {
   Session *s = reinterpret_cast<Session *>(hs);
   BH_REQUIRE(s, "session_set_prefill_precision: null session");
   BH_REQUIRE(mode >= 0 && mode <= 2, "session_set_prefill_precision: mode %d outside 0..2",
@@ -883,21 +980,24 @@ int buddy_hip_session_set_prefill_precision(buddy_hip_session *hs, int mode) {
   s->gemm_terms = mode == 1 ? 3 : 1;
   s->gemm_digits = mode == 2 ? 3 : 0;
   return BUDDY_HIP_OK;
-}
+} BH_CATCH_INT("buddy_hip_session_set_prefill_precision")
 
-int buddy_hip_session_enqueue_steps(buddy_hip_session *hs, int steps) {
+int buddy_hip_session_enqueue_steps(buddy_hip_session *hs, int steps) try {
   Session *s = reinterpret_cast<Session *>(hs);
   BH_REQUIRE(s && steps > 0, "session_enqueue_steps: bad argument");
   int rc = s->ready();
   if (rc)
     return rc;
+  // refused as a whole: no step is enqueued when the last one would not fit
+  if ((rc = s->check_steps(steps, "session_enqueue_steps")))
+    return rc;
   for (int i = 0; i < steps; ++i)
     if ((rc = s->run_step()))
       return rc;
   return BUDDY_HIP_OK;
-}
+} BH_CATCH_INT("buddy_hip_session_enqueue_steps")
 
-int buddy_hip_session_set_state(buddy_hip_session *hs, int token, int pos) {
+int buddy_hip_session_set_state(buddy_hip_session *hs, int token, int pos) try {
   Session *s = reinterpret_cast<Session *>(hs);
   BH_REQUIRE(s, "session_set_state: null session");
   BH_REQUIRE(token >= 0 && token < s->shape.vocab && pos >= 0 &&
@@ -907,7 +1007,7 @@ int buddy_hip_session_set_state(buddy_hip_session *hs, int token, int pos) {
   if (rc)
     return rc;
   return s->set_state(token, pos, 0);
-}
+} BH_CATCH_INT("buddy_hip_session_set_state")
 
 const float *buddy_hip_session_logits(buddy_hip_session *hs) {
   Session *s = reinterpret_cast<Session *>(hs);
@@ -915,7 +1015,7 @@ const float *buddy_hip_session_logits(buddy_hip_session *hs) {
 }
 
 int buddy_hip_session_discard_kv_freqs(buddy_hip_session *hs, int keep, int discard,
-                                       int count, const float *inv_freq) {
+                                       int count, const float *inv_freq) try {
   Session *s = reinterpret_cast<Session *>(hs);
   BH_REQUIRE(s, "session_discard_kv: null session");
   int rc = s->ready();
@@ -934,17 +1034,17 @@ int buddy_hip_session_discard_kv_freqs(buddy_hip_session *hs, int keep, int disc
     return rc;
   BH_CHECK_HIP(hipStreamSynchronize(s->stream));
   return BUDDY_HIP_OK;
-}
+} BH_CATCH_INT("buddy_hip_session_discard_kv_freqs")
 
 int buddy_hip_session_discard_kv(buddy_hip_session *hs, int keep, int discard,
-                                 int count) {
+                                 int count) try {
   return buddy_hip_session_discard_kv_freqs(hs, keep, discard, count, nullptr);
-}
+} BH_CATCH_INT("buddy_hip_session_discard_kv")
 
-int buddy_hip_session_vocab(buddy_hip_session *hs) {
+int buddy_hip_session_vocab(buddy_hip_session *hs) try {
   Session *s = reinterpret_cast<Session *>(hs);
   return s ? s->shape.vocab : 0;
-}
+} BH_CATCH_INT("buddy_hip_session_vocab")
 
 buddy_hip_stream buddy_hip_session_stream(buddy_hip_session *hs) {
   Session *s = reinterpret_cast<Session *>(hs);

@@ -37,7 +37,9 @@ enum {
   BUDDY_HIP_OK = 0,
   BUDDY_HIP_ERR_ARG = 1,     /* shape / pointer / size check failed */
   BUDDY_HIP_ERR_HIP = 2,     /* a HIP runtime call failed */
-  BUDDY_HIP_ERR_NO_DEVICE = 3
+  BUDDY_HIP_ERR_NO_DEVICE = 3,
+  BUDDY_HIP_ERR_HOST = 4     /* host side: out of memory or a C++ exception,
+                                caught at this boundary */
 };
 
 /* ---- library ---------------------------------------------------------- */
@@ -186,14 +188,17 @@ int buddy_hip_argmax(const float *x, int n, void *workspace, int *out_index,
  * (subgraph0_decode_simplify.mlir:88-142).  qkv = [q | k | v] as the
  * projections leave them (before RoPE); the kernel rotates q and k, writes k'
  * and v into row *pos of the caches ([kv_heads, max_len, head_dim] f32 each)
- * and attends over rows 0..*pos.  out: [heads*head_dim].  head_dim must be 128.
- */
+ * and attends over rows 0..*pos.  out: [heads*head_dim].  lse: [heads] or NULL,
+ * the op's second result, max + log(sum) of each head's scaled scores
+ * (tosa.py:14576-14594).  head_dim must be 128.  *pos must lie in
+ * 0..max_len-1; a position outside writes no cache row. */
 size_t buddy_hip_attn_decode_workspace_bytes(int heads, int max_len);
 int buddy_hip_gqa_decode_attention(const float *qkv, const float *inv_freq,
                                    const int *pos, float *kcache, float *vcache,
-                                   float *out, int heads, int kv_heads,
-                                   int head_dim, int max_len, float scale,
-                                   void *workspace, size_t workspace_bytes,
+                                   float *out, float *lse, int heads,
+                                   int kv_heads, int head_dim, int max_len,
+                                   float scale, void *workspace,
+                                   size_t workspace_bytes,
                                    buddy_hip_stream stream);
 
 /* ---- prefill attention ----------------------------------------------------
@@ -266,6 +271,11 @@ int buddy_hip_session_set_layer(buddy_hip_session *s, int index,
  * f32 [kv_heads, max_len, head_dim]; src/dst may be host or device memory. */
 int buddy_hip_session_set_kv(buddy_hip_session *s, int kv_index, const float *src);
 int buddy_hip_session_get_kv(buddy_hip_session *s, int kv_index, float *dst);
+/* Rows row0 .. row0 + rows - 1 of all 2 * layers caches at once, packed as
+ * dst[kv_index][kv_head][row][head_dim] (host or device): the rows a decode
+ * step or a prefill just wrote, for a caller that mirrors the caches on the
+ * host the way the generated ModelSession does (gen_session.py:1421-1430). */
+int buddy_hip_session_get_kv_rows(buddy_hip_session *s, int row0, int rows, float *dst);
 /* 1 (default): a decode step is replayed from a captured hipGraph; 0: launched
  * kernel by kernel. */
 int buddy_hip_session_use_graph(buddy_hip_session *s, int enable);
@@ -274,6 +284,12 @@ int buddy_hip_session_use_graph(buddy_hip_session *s, int enable);
  * next_token is the greedy choice (first maximum).  Synchronous. */
 int buddy_hip_session_decode(buddy_hip_session *s, int token, int pos,
                              float *logits_out, int *next_token);
+/* The same, and the cache rows the step wrote are handed back as well:
+ * kv_rows_out (host or device, may be NULL) receives row `pos` of all
+ * 2 * layers caches as [kv_index][kv_head][head_dim]. */
+int buddy_hip_session_decode_mirror(buddy_hip_session *s, int token, int pos,
+                                    float *logits_out, float *kv_rows_out,
+                                    int *next_token);
 /* `steps` greedy steps starting from first_token at start_pos; each step's
  * argmax feeds the next step on the device.  tokens_out[i] = token chosen by
  * step i.  Synchronous. */
@@ -455,9 +471,15 @@ buddy_hip_session *buddy_hip_session_create_from_w8a32_blobs(
  * the caller's KV and position buffers and hand over a malloc'd [1,1,vocab]
  * logits buffer; prefill hands over malloc'd KV tensors and [1,max_len,vocab]
  * logits.  The device session is built on the first call and reused while the
- * blob addresses stay the same.  The KV cache is uploaded from the caller's
- * tensors on the first decode that no prefill preceded; call
- * buddy_hip_forward_invalidate_kv() after editing the host cache.
+ * blob addresses stay the same.  The caller's KV tensors and the device cache
+ * are kept equal: the cache is uploaded from the caller's tensors on the first
+ * decode that no prefill preceded, and every decode writes the row it produced
+ * through to the caller's tensors, as the compiled model does.  A caller may
+ * therefore edit its tensors between calls the way the generated
+ * ModelSession::handleKVCacheOverflow does (gen_session.py:1471-1511: shift,
+ * re-rotate, lower the position): a decode whose cache_position is not the one
+ * that follows the previous call reloads the device cache from the caller's
+ * tensors.  buddy_hip_forward_invalidate_kv() forces that reload.
  * The hand-written program for the same model
  * (examples/BuddyDeepSeekR1/buddy-deepseek-r1-w8a32-main.cpp:163-249) reads its
  * decode results in another order -- position, kv0, kv1, the 27 position copies
@@ -483,8 +505,11 @@ void _mlir_ciface_forward_decode(
 void buddy_hip_forward_reset(void);         /* drops the cached device session */
 void buddy_hip_forward_invalidate_kv(void); /* next decode re-uploads the KV cache */
 /* discardKVCache + adjustKeyCacheRope on the device-resident cache of the
- * session behind _mlir_ciface_forward_*: what the decode loop calls instead of
- * editing its host tensors (TextGeneration.cpp:231-237). */
+ * session behind _mlir_ciface_forward_*: what a decode loop may call instead of
+ * editing its host tensors (TextGeneration.cpp:231-237); it saves the reload.
+ * From then on the device cache is the only complete copy: the caller's tensors
+ * keep receiving the new rows but are not shifted, and are never reloaded
+ * unless buddy_hip_forward_invalidate_kv() is called. */
 int buddy_hip_forward_discard_kv(int keep, int discard, int count);
 
 /* ---- operator-level memref entry points --------------------------------

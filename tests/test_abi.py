@@ -45,3 +45,21 @@ def test_packed_bytes_is_padded_to_tiles(bh):
     assert bh.buddy_hip_w8_packed_bytes(1, 1) == 64 * 16
     assert bh.buddy_hip_w8_packed_bytes(65, 17) == 128 * 32
     assert bh.buddy_hip_w8_packed_bytes(0, 5) == 0
+
+
+def test_exception_is_caught_at_the_boundary(bh):
+    """A request whose host staging cannot exist (2^62 floats: std::vector
+    refuses with std::length_error before anything is touched) must come back
+    as an ordinary failure: result left null, message in buddy_hip_last_error(),
+    the process alive -- nothing unwinds through the C ABI
+    (examples/BuddyOneDNN/onednn_ops.cpp:229-241: stderr + return)."""
+    import numpy as np
+    a = np.zeros(4, np.float32)
+    big = 1 << 31
+    A = bma.MemRef(a.ctypes.data, [big, big], strides=[0, 0])
+    B = bma.MemRef(a.ctypes.data, [big, 1], strides=[0, 0])
+    res = bma.MemRefF32_2D()
+    bh._mlir_ciface_buddy_matmul_f32(ctypes.byref(res), ctypes.byref(A), ctypes.byref(B))
+    assert not res.aligned and not res.allocated
+    msg = bh.buddy_hip_last_error()
+    assert b"_mlir_ciface_buddy_matmul_f32" in msg, msg

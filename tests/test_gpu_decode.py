@@ -185,6 +185,7 @@ def test_decode_attention_with_rope_and_kv_write(bh, oracle, pos):
     vc[:, pos:, :] = 1e30
     inv = synthetic.inv_freq(D)
     out = torch.empty(H * D, device="cuda")
+    lse = torch.empty(H, device="cuda")
     pos_t = torch.tensor([pos], dtype=torch.int32, device="cuda")
     nb = bh.buddy_hip_attn_decode_workspace_bytes(H, L)
     ws = torch.empty(nb, dtype=torch.uint8, device="cuda")
@@ -193,7 +194,7 @@ def test_decode_attention_with_rope_and_kv_write(bh, oracle, pos):
     torch.cuda.synchronize()
     bma.check(bh.buddy_hip_gqa_decode_attention(
         qkv.data_ptr(), inv.data_ptr(), pos_t.data_ptr(), kc.data_ptr(), vc.data_ptr(),
-        out.data_ptr(), H, HKV, D, L, float(scale), ws.data_ptr(), nb, None))
+        out.data_ptr(), lse.data_ptr(), H, HKV, D, L, float(scale), ws.data_ptr(), nb, None))
     torch.cuda.synchronize()
     # oracle: RoPE, cache write, then attention over the whole cache with the mask
     c, s = oracle.rope_cos_sin(inv.cpu().numpy(), pos)
@@ -205,8 +206,10 @@ def test_decode_attention_with_rope_and_kv_write(bh, oracle, pos):
     kch[:, pos + 1:, :] = 0  # the oracle multiplies masked rows by exactly 0
     vch[:, pos + 1:, :] = 0
     mask = np.where(np.arange(L) <= pos, 0.0, -np.inf).astype(np.float32)
-    want, _ = oracle.gqa_decode_attention(q, kch, vch, mask, scale, 4)
+    want, want_lse = oracle.gqa_decode_attention(q, kch, vch, mask, scale, 4)
     check_close(out.cpu().numpy().reshape(H, D), want)
+    # the op's second result: lse = m + log l per head (tosa.py:14576-14594)
+    check_close(lse.cpu().numpy(), want_lse)
     # the new K/V rows landed in the cache, nothing else moved
     check_close(kc[:, pos, :].cpu().numpy(), k)
     np.testing.assert_array_equal(vc[:, pos, :].cpu().numpy(), v)
@@ -264,7 +267,7 @@ def test_decode_attention_long_context(bh, oracle, pos):
     torch.cuda.synchronize()
     bma.check(bh.buddy_hip_gqa_decode_attention(
         qkv.data_ptr(), inv.data_ptr(), pos_t.data_ptr(), kc.data_ptr(), vc.data_ptr(),
-        out.data_ptr(), H, HKV, D, L, float(scale), ws.data_ptr(), nb, None))
+        out.data_ptr(), None, H, HKV, D, L, float(scale), ws.data_ptr(), nb, None))
     torch.cuda.synchronize()
     c, s = oracle.rope_cos_sin(inv.cpu().numpy(), pos)
     q = oracle.rope_apply(qh[:H * D].reshape(H, D), c, s)
@@ -316,6 +319,22 @@ def test_session_refuses_bad_arguments(bh):
         sess.decode(SMALL.vocab, 0)  # token id out of range
     with pytest.raises(bma.BuddyHipError):
         sess.decode_greedy(1, SMALL.max_len - 3, 8)  # would run off the cache
+    # asynchronous steps are bounded on the host as well: the device advances
+    # its own position and step counter, and nothing may run off the cache or
+    # the token log
+    with pytest.raises(bma.BuddyHipError):
+        sess.enqueue_steps(1)  # no token / position set yet
+    sess.set_state(5, SMALL.max_len - 4)
+    with pytest.raises(bma.BuddyHipError):
+        sess.enqueue_steps(5)  # the fifth step would write row max_len
+    assert b"leave the cache" in bh.buddy_hip_last_error()
+    sess.enqueue_steps(3)
+    with pytest.raises(bma.BuddyHipError):
+        sess.enqueue_steps(2)  # refused as a whole: one row is left
+    sess.enqueue_steps(1)
+    with pytest.raises(bma.BuddyHipError):
+        sess.enqueue_steps(1)
+    torch.cuda.synchronize()
     sess.close()
     bad = Shape(head_dim=64)
     with pytest.raises(bma.BuddyHipError):

@@ -200,6 +200,82 @@ def test_model_level_entry_points_full_shape(bh, oracle):
     bh.buddy_hip_forward_reset()
 
 
+def decode_args(res, mf, mi, mtok, mpos, kvm, mdum):
+    args = [ctypes.byref(res), ctypes.byref(mf), ctypes.byref(mi), ctypes.byref(mtok),
+            ctypes.byref(mpos), ctypes.byref(kvm[0]), ctypes.byref(kvm[1])]
+    for i in range(27):
+        args += [ctypes.byref(mdum[i]), ctypes.byref(kvm[2 + 2 * i]),
+                 ctypes.byref(kvm[3 + 2 * i])]
+    assert len(args) == 88
+    return args
+
+
+@pytest.mark.timeout(900)
+def test_forward_decode_survives_the_callers_own_overflow_handling(bh, oracle):
+    """The generated ModelSession handles a full cache on its HOST tensors
+    (gen_session.py:1471-1511: discardKVCache, adjustKeyCacheRope, position
+    lowered) and goes on calling forward_decode.  forward_decode writes every new
+    row through to the caller's tensors and reloads the device cache when the
+    position is not the one that follows, so such a caller needs no change: a
+    64-row cache decoded from empty, overflowed, edited on the host with the
+    restated KVCacheManager, and decoded on, yields the oracle's tokens."""
+    L = 64
+    shape = Shape(max_len=L)
+    f32, i8, host = make_blobs(bh, shape, seed=2)
+    om = oracle_lib.model_from_host(oracle, shape, host)
+    okv = [np.zeros((2, L, 128), np.float32) for _ in range(56)]
+    state_kv = [np.zeros((2, L, 128), np.float32) for _ in range(56)]
+    free = ctypes.CDLL(None).free
+    free.argtypes = [ctypes.c_void_p]
+    mf = bma.MemRef(f32.ctypes.data, [f32.size])
+    mi = bma.MemRef(i8.ctypes.data, [i8.size], ctype=ctypes.c_int8)
+    kvm = [bma.MemRef(a.ctypes.data, [1, 2, L, 128]) for a in state_kv]
+    posbuf = np.zeros(1, np.int64)
+    tokbuf = np.zeros((1, 1), np.int64)
+    dummies = [np.zeros(1, np.int64) for _ in range(27)]
+    mpos = bma.MemRef(posbuf.ctypes.data, [1], ctype=ctypes.c_longlong)
+    mtok = bma.MemRef(tokbuf.ctypes.data, [1, 1], ctype=ctypes.c_longlong)
+    mdum = [bma.MemRef(d.ctypes.data, [1], ctype=ctypes.c_longlong) for d in dummies]
+    inv_freq = host["globals"]["inv_freq"]
+    keep = L // 4                       # TextGeneration.cpp:164
+    discard = max(1, (L - keep) // 2)   # gen_session.py:1477-1479
+
+    def step(tok, pos):
+        tokbuf[0, 0], posbuf[0] = tok, pos
+        for d in dummies:
+            d[0] = pos
+        res = DecodeResult()
+        bh._mlir_ciface_forward_decode(*decode_args(res, mf, mi, mtok, mpos, kvm, mdum))
+        assert res.logits.aligned, bh.buddy_hip_last_error()
+        lg = np.ctypeslib.as_array(res.logits.aligned, shape=(shape.vocab,)).copy()
+        free(ctypes.cast(res.logits.allocated, ctypes.c_void_p))
+        return lg
+
+    bh.buddy_hip_forward_reset()
+    tok, pos, got, want = 11, 0, [], []
+    for n in range(L + 12):
+        if pos >= L:  # the caller edits ITS tensors; the oracle edits its own
+            for kvset in (state_kv, okv):
+                for j in range(56):
+                    _, new = oracle.kv_discard(kvset[j], keep, discard, L)
+                    if j % 2 == 0:
+                        new = oracle.kv_adjust_rope(new, keep, discard, L, inv_freq)
+                    kvset[j][...] = new
+            pos = L - discard
+        lg = step(tok, pos)
+        otok, olg = om.decode_step(tok, pos, okv)
+        if n in (0, L - 1, L, L + 11):
+            check_close(lg, olg)
+            # the row the step wrote is in the caller's tensors
+            for j in (0, 1, 54, 55):
+                check_close(state_kv[j][:, pos, :], okv[j][:, pos, :])
+        got.append(int(lg.argmax()))
+        want.append(otok)
+        tok, pos = otok, pos + 1
+    assert got == want
+    bh.buddy_hip_forward_reset()
+
+
 def test_model_level_entry_points_refuse_bad_blobs(bh):
     f32 = np.zeros(10, np.float32)
     i8 = np.zeros(10, np.int8)
