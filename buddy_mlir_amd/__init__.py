@@ -103,6 +103,9 @@ def _declare(lib):
         "buddy_hip_gqa_decode_attention": (c_int, [vp, vp, vp, vp, vp, vp, vp, c_int,
                                                    c_int, c_int, c_int, c_float,
                                                    vp, sz, vp]),
+        "buddy_hip_gqa_decode_attention_static": (c_int, [vp, vp, vp, vp, vp, vp, vp, c_int,
+                                                          c_int, c_int, c_int, c_float,
+                                                          vp]),
         "buddy_hip_prefill_attention": (c_int, [vp, vp, vp, vp, vp, c_int, c_int, c_int,
                                                 c_int, c_int, c_float, vp]),
         "buddy_hip_session_create": (vp, [vp, vp]),

@@ -6,6 +6,7 @@
 namespace bh {
 
 constexpr int kAttnChunk = 64; // cache positions per flash-decoding partial
+constexpr int kAttnHeadDim = 128; // the head size the decode kernel is written for
 
 struct AttnDecodeArgs {
   const float *qkv = nullptr;      // [heads*D | kv_heads*D | kv_heads*D], pre-RoPE

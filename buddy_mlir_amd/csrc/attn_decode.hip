@@ -24,6 +24,8 @@
 // folds them in chunk order with the reference's own combine rule.
 #include "attn.h"
 
+#include <mutex>
+
 namespace bh {
 namespace {
 
@@ -31,7 +33,7 @@ constexpr int kChunk = kAttnChunk; // cache positions per workgroup
 constexpr int kThreads = 256;
 constexpr int kMaxGroup = 8;     // query heads per KV head
 constexpr int kHPB = 1;          // query heads per workgroup
-constexpr int kD = 128;          // head_dim this kernel is written for
+constexpr int kD = kAttnHeadDim; // head_dim this kernel is written for
 constexpr float kSeedM = -1.0e30f; // tosa.py:13971
 
 struct AttnArgs {
@@ -273,6 +275,35 @@ __global__ void __launch_bounds__(kD) attn_decode_combine(AttnArgs a) {
     a.lse[h] = m_run + logf(l_run);
 }
 
+// ---- scratch of the entry point that allocates nothing --------------------
+// Flash-decoding partials for up to kStaticPartials (head, chunk) pairs, e.g.
+// 32 heads x 16384 cache positions: 8192 x (128 + 2) floats = 4.06 MiB of
+// device memory that every GPU the library runs on holds until the process
+// ends.  In host code the array's name is only a handle for
+// hipGetSymbolAddress: the address a kernel may use is looked up once per
+// device and kept in g_scratch_ptr.
+constexpr int kStaticPartials = 8192;
+constexpr int kMaxDevices = 64;
+static __device__ __align__(256) float g_attn_scratch[(size_t)kStaticPartials * (kD + 2)];
+std::mutex g_scratch_mu;
+float *g_scratch_ptr[kMaxDevices] = {};
+
+// Device address of the current device's copy of g_attn_scratch.
+int static_scratch(float **out) {
+  int dev = -1;
+  BH_CHECK_HIP(hipGetDevice(&dev));
+  BH_REQUIRE(dev >= 0 && dev < kMaxDevices, "attn_decode: device index %d", dev);
+  std::lock_guard<std::mutex> lock(g_scratch_mu);
+  if (!g_scratch_ptr[dev]) {
+    void *p = nullptr;
+    BH_CHECK_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(g_attn_scratch)));
+    BH_REQUIRE(p, "attn_decode: no device address for the static scratch");
+    g_scratch_ptr[dev] = static_cast<float *>(p);
+  }
+  *out = g_scratch_ptr[dev];
+  return BUDDY_HIP_OK;
+}
+
 } // namespace
 
 size_t attn_decode_workspace_bytes(int heads, int max_len) {
@@ -365,4 +396,39 @@ int buddy_hip_gqa_decode_attention(const float *qkv, const float *inv_freq,
   a.workspace_bytes = workspace_bytes;
   return bh::launch_attn_decode(a, bh::as_stream(stream));
 } BH_CATCH_INT("buddy_hip_gqa_decode_attention")
+
+int buddy_hip_gqa_decode_attention_static(const float *qkv, const float *inv_freq,
+                                          const int *pos, float *kcache,
+                                          float *vcache, float *out, float *lse,
+                                          int heads, int kv_heads, int head_dim,
+                                          int max_len, float scale,
+                                          buddy_hip_stream stream) try {
+  BH_REQUIRE(heads > 0 && max_len > 0, "attn_decode_static: heads=%d max_len=%d", heads,
+             max_len);
+  const int64_t pairs = (int64_t)heads * bh::ceil_div(max_len, bh::kAttnChunk);
+  BH_REQUIRE(pairs <= bh::kStaticPartials,
+             "attn_decode_static: heads x ceil(max_len / %d) = %lld exceeds the built-in "
+             "scratch of %d partials; use buddy_hip_gqa_decode_attention with a workspace",
+             bh::kAttnChunk, (long long)pairs, bh::kStaticPartials);
+  float *scratch = nullptr;
+  int rc = bh::static_scratch(&scratch);
+  if (rc)
+    return rc;
+  bh::AttnDecodeArgs a;
+  a.qkv = qkv;
+  a.inv_freq = inv_freq;
+  a.pos_ptr = pos;
+  a.kcache = kcache;
+  a.vcache = vcache;
+  a.out = out;
+  a.lse = lse;
+  a.heads = heads;
+  a.kv_heads = kv_heads;
+  a.head_dim = head_dim;
+  a.max_len = max_len;
+  a.scale = scale;
+  a.workspace = scratch;
+  a.workspace_bytes = sizeof(float) * (size_t)bh::kStaticPartials * (bh::kAttnHeadDim + 2);
+  return bh::launch_attn_decode(a, bh::as_stream(stream));
+} BH_CATCH_INT("buddy_hip_gqa_decode_attention_static")
 }

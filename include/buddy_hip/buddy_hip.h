@@ -201,6 +201,25 @@ int buddy_hip_gqa_decode_attention(const float *qkv, const float *inv_freq,
                                    size_t workspace_bytes,
                                    buddy_hip_stream stream);
 
+/* The same call for callers that cannot allocate device memory or pass a
+ * workspace around (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc).  It has no counterpart in the reference.
+ * The flash-decoding partials go to a buffer built into the library (4.06 MiB
+ * of device memory per GPU, held until the process ends) instead of a
+ * caller's workspace, and the call allocates nothing.  Limit: heads x
+ * ceil(max_len / 64) <= 8192 (e.g. 32 heads x 16384 positions); larger shapes
+ * are refused with BUDDY_HIP_ERR_ARG.  Results are bit-identical to
+ * buddy_hip_gqa_decode_attention.  Every call on a GPU shares that GPU's
+ * buffer: calls that overlap on one GPU (two streams, two threads) race; calls
+ * on one stream are ordered.  The device that is current at the call must be
+ * the stream's device. */
+int buddy_hip_gqa_decode_attention_static(const float *qkv, const float *inv_freq,
+                                          const int *pos, float *kcache,
+                                          float *vcache, float *out, float *lse,
+                                          int heads, int kv_heads, int head_dim,
+                                          int max_len, float scale,
+                                          buddy_hip_stream stream);
+
 /* ---- prefill attention ----------------------------------------------------
  * Replaces flash_attention_for_cpu_prefill_op
  * (frontend/Python/ops/tosa.py:4326-4810).  q, out: [heads, q_len, head_dim];
