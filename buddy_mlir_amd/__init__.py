@@ -19,7 +19,9 @@ __all__ = [
 ]
 
 _PKG = Path(__file__).resolve().parent
-_LIB_PATH = _PKG / "lib" / "libbuddy_hip.so"
+# BUDDY_HIP_LIBRARY: another build of the library (a measurement build), for
+# the process that sets it
+_LIB_PATH = Path(os.environ.get("BUDDY_HIP_LIBRARY") or _PKG / "lib" / "libbuddy_hip.so")
 _lib = None
 
 

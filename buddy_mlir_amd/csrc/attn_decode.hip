@@ -29,6 +29,8 @@
 namespace bh {
 namespace {
 
+BH_TL_DECLARE(g_tl_attn)
+
 constexpr int kChunk = kAttnChunk; // cache positions per workgroup
 constexpr int kThreads = 256;
 constexpr int kMaxGroup = 8;     // query heads per KV head
@@ -64,6 +66,8 @@ __global__ void __launch_bounds__(kThreads) attn_decode_partial(AttnArgs a) {
 
   const int tid = threadIdx.x;
   const int hb = blockIdx.x / a.pairs_padded, ckv = blockIdx.x % a.pairs_padded;
+  [[maybe_unused]] const int tl_wave = blockIdx.x * (kThreads / 64) + (tid >> 6);
+  BH_TL(g_tl_attn, tl_wave, 0);
   if (ckv >= a.nchunks * a.kv_heads)
     return; // padding id
   const int chunk = ckv % a.nchunks, kvh = ckv / a.nchunks;
@@ -130,6 +134,7 @@ __global__ void __launch_bounds__(kThreads) attn_decode_partial(AttnArgs a) {
     }
     return;
   }
+  BH_TL(g_tl_attn, tl_wave, 1);
   const int p1 = min(p0 + kChunk, pos + 1);
   const int np = p1 - p0;
   const bool has_new = pos >= p0 && pos < p1;
@@ -149,6 +154,7 @@ __global__ void __launch_bounds__(kThreads) attn_decode_partial(AttnArgs a) {
     }
   }
   __syncthreads();
+  BH_TL(g_tl_attn, tl_wave, 2);
 
   // ---- scores: 4 threads per position, 32 dims each ----------------------
   {
@@ -187,6 +193,7 @@ __global__ void __launch_bounds__(kThreads) attn_decode_partial(AttnArgs a) {
     }
   }
   __syncthreads();
+  BH_TL(g_tl_attn, tl_wave, 3);
 
   // ---- per-head max, exp, sum over the chunk: one wavefront per head -------
   if ((tid >> 6) < nh) {
@@ -202,6 +209,7 @@ __global__ void __launch_bounds__(kThreads) attn_decode_partial(AttnArgs a) {
     }
   }
   __syncthreads();
+  BH_TL(g_tl_attn, tl_wave, 4);
 
   // ---- acc[h][d] = sum_p e[h][p] * V[p][d]: 32 threads across d, 8 rows of p
   {
@@ -238,6 +246,7 @@ __global__ void __launch_bounds__(kThreads) attn_decode_partial(AttnArgs a) {
             make_float4(acc[h][0], acc[h][1], acc[h][2], acc[h][3]);
   }
   __syncthreads();
+  BH_TL(g_tl_attn, tl_wave, 5);
   if (qh < nh) {
     float s = 0.f;
 #pragma unroll
@@ -249,6 +258,7 @@ __global__ void __launch_bounds__(kThreads) attn_decode_partial(AttnArgs a) {
     a.part_ml[((size_t)(h0 + tid) * a.nchunks + chunk) * 2 + 0] = m_s[tid];
     a.part_ml[((size_t)(h0 + tid) * a.nchunks + chunk) * 2 + 1] = l_s[tid];
   }
+  BH_TL(g_tl_attn, tl_wave, 6);
 }
 
 // Folds the partials of one head in chunk order with the reference's combine
@@ -364,6 +374,7 @@ int launch_attn_decode(const AttnDecodeArgs &in, hipStream_t stream) {
   return BUDDY_HIP_OK;
 }
 
+BH_TL_EXPORT(buddy_hip_debug_timeline_attn, g_tl_attn)
 } // namespace bh
 
 extern "C" {

@@ -57,6 +57,30 @@ constexpr int kTileN = 16;         // output channels per packed tile
 constexpr int kTileK = 64;         // k values per packed tile
 constexpr int kTileBytes = 1024;   // one wavefront-wide 128-bit load
 
+// Phase timestamps inside a kernel, for builds made with BUDDY_HIP_TIMELINE=1 in
+// the environment (never the shipped build): lane 0 of a wavefront records the
+// constant-rate 100 MHz clock into slot `slot` of its row of a per-file device
+// array, which a debug export copies out.  Empty otherwise.
+#if defined(BH_TIMELINE) && defined(__HIPCC__)
+#define BH_TL_DECLARE(name) static __device__ unsigned long long name[1 << 18];
+#define BH_TL(name, wave_id, slot)                                             \
+  do {                                                                         \
+    if ((threadIdx.x & 63) == 0)                                               \
+      name[(((size_t)(wave_id)) * 8 + (slot)) & ((1u << 18) - 1)] = wall_clock64(); \
+  } while (0)
+#define BH_TL_EXPORT(fn, name)                                                 \
+  extern "C" int fn(unsigned long long *dst, size_t count) {                   \
+    return (int)hipMemcpyFromSymbol(dst, HIP_SYMBOL(name),                     \
+                                    sizeof(unsigned long long) * count);       \
+  }
+#else
+#define BH_TL_DECLARE(name)
+#define BH_TL(name, wave_id, slot)                                             \
+  do {                                                                         \
+  } while (0)
+#define BH_TL_EXPORT(fn, name)
+#endif
+
 inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 inline int64_t round_up(int64_t a, int64_t b) { return ceil_div(a, b) * b; }
 

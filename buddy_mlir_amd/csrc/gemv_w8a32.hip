@@ -34,6 +34,8 @@
 namespace bh {
 namespace {
 
+BH_TL_DECLARE(g_tl_gemv)
+
 constexpr int kMaxWaves = 16;            // wavefronts per workgroup
 constexpr int kXStride = 20;             // floats per (tile, k-group) in LDS:
                                          // 16 used + 4 pad, conflict-free b128
@@ -45,6 +47,10 @@ constexpr size_t kLdsBudget = 40 * 1024;    // preferred, keeps ~4 workgroups pe
 struct GemvPlan {
   int64_t chunks, groups;
   int G, KS, waves, tiles_per_round, blocks;
+  // 1: two workgroups per channel group, each streaming the bytes of 8 of its 16
+  // channels (narrow, long matrices: 96 channel groups would otherwise keep
+  // only 96 of the 256 compute units streaming)
+  int half_split = 0;
   size_t lds_bytes;
 };
 
@@ -57,8 +63,12 @@ int target_waves() {
   return v;
 }
 
+bool no_half_split() {
+  static bool v = getenv("BUDDY_HIP_GEMV_NO_HALF_SPLIT") != nullptr;
+  return v;
+}
+
 GemvPlan make_plan(int64_t M, int64_t K, int64_t N, bool dual, int tn, bool fold = false) {
-  (void)dual;
   GemvPlan p;
   p.chunks = ceil_div(K, 1024 / tn);
   p.groups = ceil_div(N, tn);
@@ -96,6 +106,12 @@ GemvPlan make_plan(int64_t M, int64_t K, int64_t N, bool dual, int tn, bool fold
     cap = 4;
   p.tiles_per_round = (int)(tiles < cap ? round_up(tiles, 4) : cap);
   p.lds_bytes = round_bytes(p.waves, p.tiles_per_round) + red_bytes(p.waves);
+  // One row, 16-channel tiles, at most half of the compute units busy and enough
+  // bytes per channel group (>= 64 KiB) for the stream, not latency, to decide
+  // the launch: measured 6.6 -> 5.x us for 8960 -> 1536.
+  if (M == 1 && tn == 16 && !dual && !fold && p.G == 1 && p.blocks <= 128 &&
+      p.chunks >= 64 && !no_half_split())
+    p.half_split = 1;
   return p;
 }
 
@@ -580,6 +596,33 @@ __device__ __forceinline__ void attn_fold_tiles(const KernelArgs &a, int t0, int
     m[u] = -1.0e30f;
     l[u] = 0.f;
   }
+  if (used <= B) {
+    // The usual case (a cache of up to 18 chunks = 1152 positions): one batch,
+    // and nothing in it depends on anything loaded -- the (max, sum) pair of
+    // every chunk and the partial sums of every tile are requested together, so
+    // the fold costs one trip to memory, not two.  Slots past the last chunk
+    // repeat it (a valid, finite partial) and get weight 0.
+    float2 mine[U];
+    float v[U][B];
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+      mine[u] = ml[u][min(lane, used - 1)];
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int j = 0; j < B; ++j)
+        v[u][j] = acc[u][(size_t)min(j, used - 1) * a.head_dim];
+    const bool valid = lane < used;
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const float mb = wave_max(valid ? mine[u].x : -1.0e30f);
+      const float w = valid ? expf(mine[u].x - mb) : 0.f;
+      l[u] = wave_sum(mine[u].y * w);
+#pragma unroll
+      for (int j = 0; j < B; ++j)
+        r[u] = fmaf(v[u][j], lane_f(w, j), r[u]);
+    }
+  } else {
   for (int c0 = 0; c0 < used; c0 += kWave) { // 64 chunks per pass
     const int cnt = min(kWave, used - c0);
     float w[U];
@@ -609,6 +652,7 @@ __device__ __forceinline__ void attn_fold_tiles(const KernelArgs &a, int t0, int
             r[u] = fmaf(v[u][j], lane_f(w[u], s0 + j), r[u]);
     }
   }
+  } // longer caches
 #pragma unroll
   for (int u = 0; u < U; ++u)
     x[u] = r[u] * (1.0f / l[u]);
@@ -645,28 +689,56 @@ __device__ __forceinline__ void fetch_tile(const KernelArgs &a, const int4 *w0,
         o.x[m] = x1[0];
       }
     } else {
-      const int mc = m < a.rows ? m : a.rows - 1;
-      o.x[m] = a.A[(int64_t)mc * a.lda + kc];
+      if (M == 1) {
+        o.x[m] = a.A[kc];
+      } else {
+        const int mc = m < a.rows ? m : a.rows - 1;
+        o.x[m] = a.A[(int64_t)mc * a.lda + kc];
+      }
     }
   }
 }
 
 // ONE: every wavefront's run of tiles fits in U, so all its loads go out at
 // once and nothing is double-buffered.
+//
+// Everything a wavefront needs before it can request its tiles -- four
+// pointers and six integers, 14 argument words -- are separate leading
+// parameters: this file is built with -amdgpu-kernarg-preload-count=14, so the
+// command processor hands them to every wavefront in SGPRs and the first loads
+// do not wait for a scalar load of the argument block.  The remaining fields
+// travel in `rest` and are loaded as usual, behind the stream.
 template <int M, int EPI, int PRO, int U, bool ONE>
 __global__ void __launch_bounds__(kMaxWaves *kWave)
-    gemv_w8a32_bcast_kernel(KernelArgs a) {
+    gemv_w8a32_bcast_kernel(const int4 *pW0, const int4 *pW1, const float *pA,
+                            const float *pnorm_w, int p_chunks, int p_KS, int p_G,
+                            int p_groups, int p_K, int p_rows, KernelArgs rest) {
+  KernelArgs a = rest;
+  a.W0 = pW0;
+  a.W1 = pW1;
+  a.A = pA;
+  a.norm_w = pnorm_w;
+  a.chunks = p_chunks;
+  a.KS = p_KS;
+  a.G = p_G & 0xffff;
+  const int hs = p_G >> 16; // 1: this workgroup takes 8 of its group's 16 channels
+  a.groups = p_groups;
+  a.K = p_K;
+  a.rows = p_rows;
   constexpr bool DUAL = (EPI == kEpiSiluMul);
   constexpr bool NORM = (PRO == kProNorm);
   extern __shared__ float lds[]; // only the meeting place of the k-slices
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
   const int gl = wave / a.KS, ks = wave % a.KS;
-  const int g = blockIdx.x * a.G + gl;
+  const int gi = blockIdx.x * a.G + gl;
+  const int g = gi >> hs, half = gi & hs;
   const bool live = g < a.groups;
   const int per = (a.chunks + a.KS - 1) / a.KS;
   const int t0 = min(ks * per, a.chunks);
   const int t1 = min(t0 + per, a.chunks);
+  [[maybe_unused]] const int tl_wave = blockIdx.x * (a.G * a.KS) + wave;
+  BH_TL(g_tl_gemv, tl_wave, 0);
 
   float acc0[M], acc1[M], ss[M];
 #pragma unroll
@@ -675,7 +747,12 @@ __global__ void __launch_bounds__(kMaxWaves *kWave)
     acc1[m] = 0.f;
     ss[m] = 0.f;
   }
-  const size_t wbase = ((size_t)(live ? g : 0) * a.chunks) * 64 + lane;
+  // With the channel group split over two workgroups, the lanes of the other
+  // half read their partner's 16 bytes (lane ^ 8: the same cache line, no extra
+  // traffic) and compute a copy of its sums that nobody stores: every load
+  // instruction then moves four whole 128-byte lines, half a tile.
+  const int wlane = hs ? ((lane & ~8) | (half << 3)) : lane;
+  const size_t wbase = ((size_t)(live ? g : 0) * a.chunks) * 64 + wlane;
   const int4 *w0 = a.W0 + wbase;
   const int4 *w1 = DUAL ? a.W1 + wbase : a.W0 + wbase;
 
@@ -703,7 +780,8 @@ __global__ void __launch_bounds__(kMaxWaves *kWave)
   }
 
   const int n = g * kTileN + lane;
-  const bool writer = ks == 0 && lane < kTileN && live && n < a.N;
+  const bool writer = ks == 0 && lane < kTileN && live && n < a.N &&
+                      (!hs || (lane >> 3) == half);
   EpilogueOperands<M> epi;
   if (writer) {
     epi.s0 = a.s0[n];
@@ -719,6 +797,7 @@ __global__ void __launch_bounds__(kMaxWaves *kWave)
     }
   }
 
+  BH_TL(g_tl_gemv, tl_wave, 1);
   for (int t = t0; t < (ONE ? min(t1, t0 + 1) : t1); t += U) {
 #pragma unroll
     for (int u = 0; u < U; ++u) {
@@ -753,9 +832,12 @@ __global__ void __launch_bounds__(kMaxWaves *kWave)
         }
         if (!ONE && t + U + u < t1)
           fetch_tile<M, PRO, DUAL>(a, w0, w1, t + U + u, lane, slot[u]);
+        if (u == 0 && t == t0)
+          BH_TL(g_tl_gemv, tl_wave, 2);
       }
     }
   }
+  BH_TL(g_tl_gemv, tl_wave, 3);
 
   // the four rows of a wavefront hold different k sub-ranges of the same channels
 #pragma unroll
@@ -787,6 +869,7 @@ __global__ void __launch_bounds__(kMaxWaves *kWave)
         mine[m * 33 + 32] = ss[m];
     }
     __syncthreads();
+    BH_TL(g_tl_gemv, tl_wave, 4);
     if (ks != 0)
       return;
     if (lane < kTileN) {
@@ -824,13 +907,16 @@ __global__ void __launch_bounds__(kMaxWaves *kWave)
       }
     }
   }
+  BH_TL(g_tl_gemv, tl_wave, 5);
 }
 
 template <int M, int EPI, int PRO, int U, bool ONE>
 int launch_bcast(const KernelArgs &ka, const GemvPlan &p, hipStream_t stream) {
   auto kernel = gemv_w8a32_bcast_kernel<M, EPI, PRO, U, ONE>;
-  hipLaunchKernelGGL(kernel, dim3(p.blocks), dim3(p.waves * kWave),
-                     sizeof(float) * p.waves * (size_t)M * 33, stream, ka);
+  hipLaunchKernelGGL(kernel, dim3(p.blocks << p.half_split), dim3(p.waves * kWave),
+                     sizeof(float) * p.waves * (size_t)M * 33, stream, ka.W0, ka.W1, ka.A,
+                     ka.norm_w, ka.chunks, ka.KS, ka.G | (p.half_split << 16), ka.groups,
+                     ka.K, ka.rows, ka);
   BH_CHECK_HIP(hipGetLastError());
   return BUDDY_HIP_OK;
 }
@@ -996,6 +1082,7 @@ int launch_gemv(const GemvArgs &a, hipStream_t stream) {
   }
 }
 
+BH_TL_EXPORT(buddy_hip_debug_timeline_gemv, g_tl_gemv)
 } // namespace bh
 
 extern "C" {
