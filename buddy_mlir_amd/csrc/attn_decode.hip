@@ -34,7 +34,6 @@ BH_TL_DECLARE(g_tl_attn)
 constexpr int kChunk = kAttnChunk; // cache positions per workgroup
 constexpr int kThreads = 256;
 constexpr int kMaxGroup = 8;     // query heads per KV head
-constexpr int kHPB = 1;          // query heads per workgroup
 constexpr int kD = kAttnHeadDim; // head_dim this kernel is written for
 constexpr float kSeedM = -1.0e30f; // tosa.py:13971
 
@@ -53,71 +52,79 @@ struct AttnArgs {
   int pairs_padded; // (chunk, kv head) pairs rounded up to the XCD count
 };
 
-// One workgroup: 64 cache positions x kHPB query heads (one) of one KV head.  The
-// workgroups that share a chunk (different query heads, same K/V rows) get
-// linear ids that are equal modulo 8, so they run on the same XCD and the rows
-// come out of that XCD's L2 after the first of them has fetched them.
+// One workgroup: 64 cache positions x one query head.  The workgroups that
+// share a chunk (the query heads of one KV head: same K/V rows) get linear ids
+// that are equal modulo 8, so they run on the same XCD and the rows come out of
+// that XCD's L2 after the first of them has fetched them.
+//
+// The step is latency bound, so the kernel is built to have almost nothing
+// behind the arrival of its K/V rows: the small operands (q, the token's own
+// k and v, the RoPE table) are requested first, the K/V rows right behind
+// them, and q is rotated into LDS while the rows are still on their way -- the
+// one barrier before the merge.  Each of the four wavefronts then handles 16
+// positions entirely on its own (scores, its own max / exp / sum, its share of
+// P.V) in registers and cross-lane operations, and the four meet once in LDS.
 __global__ void __launch_bounds__(kThreads) attn_decode_partial(AttnArgs a) {
-  __shared__ float q_s[kHPB][kD];
-  __shared__ float knew_s[kD], vnew_s[kD];
-  __shared__ float sc_s[kHPB][kChunk];
-  __shared__ float red_s[kThreads / 32][kHPB][kD];
-  __shared__ float m_s[kHPB], l_s[kHPB];
+  constexpr int kWaves = kThreads / 64;
+  constexpr int kPW = kChunk / kWaves; // positions per wavefront: 16
+  constexpr int kR = kPW / 2;          // rows per lane: 8
+  __shared__ __attribute__((aligned(16))) float q_s[kD], knew_s[kD], vnew_s[kD];
+  __shared__ __attribute__((aligned(16))) float accw_s[kWaves][kD];
+  __shared__ float mw_s[kWaves], lw_s[kWaves];
 
   const int tid = threadIdx.x;
+  const int wave = tid >> 6, lane = tid & 63;
   const int hb = blockIdx.x / a.pairs_padded, ckv = blockIdx.x % a.pairs_padded;
-  [[maybe_unused]] const int tl_wave = blockIdx.x * (kThreads / 64) + (tid >> 6);
+  [[maybe_unused]] const int tl_wave = blockIdx.x * kWaves + wave;
   BH_TL(g_tl_attn, tl_wave, 0);
   if (ckv >= a.nchunks * a.kv_heads)
     return; // padding id
   const int chunk = ckv % a.nchunks, kvh = ckv / a.nchunks;
   const int p0 = chunk * kChunk;
-  const int G = a.group;
-  const int nh = min(kHPB, G - hb * kHPB); // query heads of this workgroup
-  const int h0 = kvh * G + hb * kHPB;
+  const int h = kvh * a.group + hb; // this workgroup's query head
 
-  // ---- every load that does not need the position goes out first ----------
-  // The cache rows of the chunk exist whatever the position is (rows beyond it
-  // hold zeros or stale data and are masked by select, never multiplied in), so
-  // nothing below waits for the position to arrive.
-  const int sp = tid >> 2, spart = tid & 3; // scores: 4 threads per position
-  const int vq = tid & 31, vg = tid >> 5;   // P.V: 32 threads over d, 8 rows
-  float4 kreg[8], vreg[kChunk / 8];
-  {
-    const int prow = min(p0 + sp, a.max_len - 1);
-    const float *krow = a.kcache + ((size_t)kvh * a.max_len + prow) * kD + spart * 32;
-#pragma unroll
-    for (int c = 0; c < 8; ++c)
-      kreg[c] = *reinterpret_cast<const float4 *>(krow + c * 4);
-#pragma unroll
-    for (int i = 0; i < kChunk / 8; ++i) {
-      const int vrow = min(p0 + vg + 8 * i, a.max_len - 1);
-      vreg[i] = *reinterpret_cast<const float4 *>(
-          a.vcache + ((size_t)kvh * a.max_len + vrow) * kD + vq * 4);
-    }
-  }
-  // raw q of the workgroup's heads (one value per thread), raw k and v of the
-  // token; every thread rotates with the angle of its own j mod 64
-  const int qh = tid / kD, j = tid % kD, jj = j & (kD / 2 - 1);
-  float qraw = 0.f, qpair = 0.f;
-  if (qh < nh) {
-    const float *q = a.qkv + (size_t)(h0 + qh) * kD;
+  // ---- small operands first: they are what the barrier below waits for ----
+  // thread j < 128 rotates element j of q and of the token's k, with the angle
+  // of j mod 64
+  const int j = tid & (kD - 1), jj = j & (kD / 2 - 1);
+  float qraw = 0.f, qpair = 0.f, kraw = 0.f, kpair = 0.f, vraw = 0.f;
+  float inv_f = 0.f, cs = 0.f, sn = 0.f;
+  if (tid < kD) {
+    const float *q = a.qkv + (size_t)h * kD;
     qraw = q[j];
     qpair = j < kD / 2 ? -q[j + kD / 2] : q[j - kD / 2];
-  }
-  float kraw = 0.f, kpair = 0.f, vraw = 0.f;
-  if (tid < kD) {
     const float *k = a.qkv + (size_t)a.heads * kD + (size_t)kvh * kD;
     kraw = k[j];
     kpair = j < kD / 2 ? -k[j + kD / 2] : k[j - kD / 2];
     vraw = k[(size_t)a.kv_heads * kD + j];
+    if (a.rope_table) {
+      cs = a.rope_table[jj];
+      sn = a.rope_table[kD / 2 + jj];
+    } else {
+      inv_f = a.inv_freq[jj];
+    }
   }
-  float inv_f = 0.f, cs = 0.f, sn = 0.f;
-  if (a.rope_table) {
-    cs = a.rope_table[jj];
-    sn = a.rope_table[kD / 2 + jj];
-  } else {
-    inv_f = a.inv_freq[jj];
+  // ---- then this wavefront's 16 K rows and 16 V rows -----------------------
+  // One lane mapping for both: lane = (float4 column c4 of the 128 dims, row
+  // parity par), rows par, par + 2, ..., so that every load instruction reads
+  // two whole 512-byte rows (eight cache lines, nothing else).  The rows exist
+  // whatever the position is (rows beyond it hold zeros or stale data and are
+  // masked by select, never multiplied in), so nothing here waits for the
+  // position to arrive.
+  const int c4 = lane & 31, par = lane >> 5;
+  const int pw0 = p0 + wave * kPW; // first position of this wavefront
+  float4 kreg[kR], vreg[kR];
+#pragma unroll
+  for (int i = 0; i < kR; ++i) {
+    const int row = min(pw0 + par + 2 * i, a.max_len - 1);
+    kreg[i] = *reinterpret_cast<const float4 *>(
+        a.kcache + ((size_t)kvh * a.max_len + row) * kD + c4 * 4);
+  }
+#pragma unroll
+  for (int i = 0; i < kR; ++i) {
+    const int row = min(pw0 + par + 2 * i, a.max_len - 1);
+    vreg[i] = *reinterpret_cast<const float4 *>(
+        a.vcache + ((size_t)kvh * a.max_len + row) * kD + c4 * 4);
   }
   // a position outside the cache (a caller's mistake the host cannot see: the
   // position lives on the device) is clamped for the scan and writes nothing
@@ -126,139 +133,113 @@ __global__ void __launch_bounds__(kThreads) attn_decode_partial(AttnArgs a) {
   const int pos = min(max(pos_raw, 0), a.max_len - 1);
 
   if (p0 > pos) { // nothing visible in this chunk: an empty partial
-    if (qh < nh)
-      a.part_acc[((size_t)(h0 + qh) * a.nchunks + chunk) * kD + j] = 0.f;
-    if (tid < nh) {
-      a.part_ml[((size_t)(h0 + tid) * a.nchunks + chunk) * 2 + 0] = kSeedM;
-      a.part_ml[((size_t)(h0 + tid) * a.nchunks + chunk) * 2 + 1] = 0.f;
+    if (tid < kD)
+      a.part_acc[((size_t)h * a.nchunks + chunk) * kD + j] = 0.f;
+    if (tid == 0) {
+      a.part_ml[((size_t)h * a.nchunks + chunk) * 2 + 0] = kSeedM;
+      a.part_ml[((size_t)h * a.nchunks + chunk) * 2 + 1] = 0.f;
     }
     return;
   }
   BH_TL(g_tl_attn, tl_wave, 1);
-  const int p1 = min(p0 + kChunk, pos + 1);
-  const int np = p1 - p0;
-  const bool has_new = pos >= p0 && pos < p1;
+  const bool has_new = pos < p0 + kChunk; // the token's own row lies in this chunk
 
   // ---- RoPE: q' = q*cos + cat(-q[64:], q[:64])*sin, same for the new k ------
-  if (!a.rope_table)
-    sincosf(inv_f * (float)pos, &sn, &cs);
-  if (qh < nh)
-    q_s[qh][j] = qraw * cs + qpair * sn;
-  if (has_new && tid < kD) {
-    const float kn = kraw * cs + kpair * sn;
-    knew_s[j] = kn;
-    vnew_s[j] = vraw;
-    if (hb == 0 && pos_ok) { // one writer per cache row
-      a.kcache[((size_t)kvh * a.max_len + pos) * kD + j] = kn;
-      a.vcache[((size_t)kvh * a.max_len + pos) * kD + j] = vraw;
+  if (tid < kD) {
+    if (!a.rope_table)
+      sincosf(inv_f * (float)pos, &sn, &cs);
+    q_s[j] = qraw * cs + qpair * sn;
+    if (has_new) {
+      const float kn = kraw * cs + kpair * sn;
+      knew_s[j] = kn;
+      vnew_s[j] = vraw;
+      if (hb == 0 && pos_ok) { // one writer per cache row
+        a.kcache[((size_t)kvh * a.max_len + pos) * kD + j] = kn;
+        a.vcache[((size_t)kvh * a.max_len + pos) * kD + j] = vraw;
+      }
     }
   }
   __syncthreads();
   BH_TL(g_tl_attn, tl_wave, 2);
 
-  // ---- scores: 4 threads per position, 32 dims each ----------------------
-  {
-    const int p = sp, part = spart;
-    float dot[kHPB];
+  // ---- scores of this wavefront's 16 positions ------------------------------
+  // every lane of a half ends up with the 8 scores of its half's rows
+  const float4 q4 = *reinterpret_cast<const float4 *>(q_s + c4 * 4);
+  float sc[kR];
 #pragma unroll
-    for (int h = 0; h < kHPB; ++h)
-      dot[h] = 0.f;
-    if (p < np) {
-      const bool is_new = (p0 + p == pos);
-#pragma unroll
-      for (int c = 0; c < 8; ++c) {
-        const int d = part * 32 + c * 4;
-        const float4 kv =
-            is_new ? *reinterpret_cast<const float4 *>(knew_s + d) : kreg[c];
-#pragma unroll
-        for (int h = 0; h < kHPB; ++h) {
-          if (h < nh) {
-            const float4 qv = *reinterpret_cast<const float4 *>(&q_s[h][d]);
-            dot[h] = fmaf(qv.x, kv.x, dot[h]);
-            dot[h] = fmaf(qv.y, kv.y, dot[h]);
-            dot[h] = fmaf(qv.z, kv.z, dot[h]);
-            dot[h] = fmaf(qv.w, kv.w, dot[h]);
-          }
-        }
-      }
-    }
-#pragma unroll
-    for (int h = 0; h < kHPB; ++h)
-      dot[h] = quad_sum(dot[h]);
-    if (part == 0) {
-#pragma unroll
-      for (int h = 0; h < kHPB; ++h)
-        if (h < nh)
-          sc_s[h][p] = p < np ? dot[h] * a.scale : -INFINITY;
-    }
+  for (int i = 0; i < kR; ++i) {
+    const int p = pw0 + par + 2 * i;
+    float4 k4 = kreg[i];
+    if (p == pos) // the token's own key is not in the cache yet
+      k4 = *reinterpret_cast<const float4 *>(knew_s + c4 * 4);
+    float d = fmaf(q4.x, k4.x, fmaf(q4.y, k4.y, fmaf(q4.z, k4.z, q4.w * k4.w)));
+    d = row16_sum(d);               // the 16 lanes of a row
+    d += __shfl_xor(d, 16, 64);     // the two rows of a half: all 128 dims
+    sc[i] = p <= pos ? d * a.scale : -INFINITY;
   }
-  __syncthreads();
+  // ---- this wavefront's own max, exp and sum --------------------------------
+  float m_w = kSeedM; // stays there when no position is visible
+#pragma unroll
+  for (int i = 0; i < kR; ++i)
+    m_w = fmaxf(m_w, sc[i]);
+  m_w = fmaxf(m_w, __shfl_xor(m_w, 32, 64));
+  float l_w = 0.f;
+#pragma unroll
+  for (int i = 0; i < kR; ++i) {
+    sc[i] = expf(sc[i] - m_w); // -inf -> 0 beyond the position
+    l_w += sc[i];
+  }
+  l_w += __shfl_xor(l_w, 32, 64);
   BH_TL(g_tl_attn, tl_wave, 3);
 
-  // ---- per-head max, exp, sum over the chunk: one wavefront per head -------
-  if ((tid >> 6) < nh) {
-    const int h = tid >> 6, p = tid & 63;
-    const float s = sc_s[h][p];
-    const float m = wave_max(s);
-    const float e = expf(s - m); // -inf -> 0 for the positions beyond pos
-    const float l = wave_sum(e);
-    sc_s[h][p] = e;
-    if (p == 0) {
-      m_s[h] = m;
-      l_s[h] = l;
+  // ---- acc[d] = sum_p e[p] * V[p][d]: this lane's 8 rows x 4 dims -----------
+  float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+  for (int i = 0; i < kR; ++i) {
+    const int p = pw0 + par + 2 * i;
+    float4 v = vreg[i];
+    if (p == pos) // the token's own value row
+      v = *reinterpret_cast<const float4 *>(vnew_s + c4 * 4);
+    if (p <= pos) { // rows beyond the position may hold anything
+      acc.x = fmaf(v.x, sc[i], acc.x);
+      acc.y = fmaf(v.y, sc[i], acc.y);
+      acc.z = fmaf(v.z, sc[i], acc.z);
+      acc.w = fmaf(v.w, sc[i], acc.w);
     }
+  }
+  acc.x += __shfl_xor(acc.x, 32, 64);
+  acc.y += __shfl_xor(acc.y, 32, 64);
+  acc.z += __shfl_xor(acc.z, 32, 64);
+  acc.w += __shfl_xor(acc.w, 32, 64);
+  if (lane < 32)
+    *reinterpret_cast<float4 *>(&accw_s[wave][c4 * 4]) = acc;
+  if (lane == 0) {
+    mw_s[wave] = m_w;
+    lw_s[wave] = l_w;
   }
   __syncthreads();
   BH_TL(g_tl_attn, tl_wave, 4);
 
-  // ---- acc[h][d] = sum_p e[h][p] * V[p][d]: 32 threads across d, 8 rows of p
-  {
-    const int dq = vq, pg = vg;
-    float acc[kHPB][4];
+  // ---- the four wavefronts meet: one partial per (head, chunk) --------------
+  if (tid < kD) {
+    float m = mw_s[0];
 #pragma unroll
-    for (int h = 0; h < kHPB; ++h)
+    for (int w = 1; w < kWaves; ++w)
+      m = fmaxf(m, mw_s[w]);
+    float o = 0.f, l = 0.f;
 #pragma unroll
-      for (int c = 0; c < 4; ++c)
-        acc[h][c] = 0.f;
-#pragma unroll
-    for (int i = 0; i < kChunk / 8; ++i) {
-      const int p = pg + 8 * i;
-      if (p < np) {
-        const bool is_new = (p0 + p == pos);
-        const float4 v =
-            is_new ? *reinterpret_cast<const float4 *>(vnew_s + dq * 4) : vreg[i];
-#pragma unroll
-        for (int h = 0; h < kHPB; ++h) {
-          if (h < nh) {
-            const float e = sc_s[h][p];
-            acc[h][0] = fmaf(v.x, e, acc[h][0]);
-            acc[h][1] = fmaf(v.y, e, acc[h][1]);
-            acc[h][2] = fmaf(v.z, e, acc[h][2]);
-            acc[h][3] = fmaf(v.w, e, acc[h][3]);
-          }
-        }
-      }
+    for (int w = 0; w < kWaves; ++w) {
+      const float f = expf(mw_s[w] - m);
+      o = fmaf(accw_s[w][tid], f, o);
+      l = fmaf(lw_s[w], f, l);
     }
-#pragma unroll
-    for (int h = 0; h < kHPB; ++h)
-      if (h < nh)
-        *reinterpret_cast<float4 *>(&red_s[pg][h][dq * 4]) =
-            make_float4(acc[h][0], acc[h][1], acc[h][2], acc[h][3]);
+    a.part_acc[((size_t)h * a.nchunks + chunk) * kD + tid] = o;
+    if (tid == 0) {
+      a.part_ml[((size_t)h * a.nchunks + chunk) * 2 + 0] = m;
+      a.part_ml[((size_t)h * a.nchunks + chunk) * 2 + 1] = l;
+    }
   }
-  __syncthreads();
   BH_TL(g_tl_attn, tl_wave, 5);
-  if (qh < nh) {
-    float s = 0.f;
-#pragma unroll
-    for (int g = 0; g < kThreads / 32; ++g)
-      s += red_s[g][qh][j];
-    a.part_acc[((size_t)(h0 + qh) * a.nchunks + chunk) * kD + j] = s;
-  }
-  if (tid < nh) {
-    a.part_ml[((size_t)(h0 + tid) * a.nchunks + chunk) * 2 + 0] = m_s[tid];
-    a.part_ml[((size_t)(h0 + tid) * a.nchunks + chunk) * 2 + 1] = l_s[tid];
-  }
-  BH_TL(g_tl_attn, tl_wave, 6);
 }
 
 // Folds the partials of one head in chunk order with the reference's combine
@@ -365,8 +346,7 @@ int launch_attn_decode(const AttnDecodeArgs &in, hipStream_t stream) {
   a.out = in.out;
   a.lse = in.lse;
   a.pairs_padded = (int)round_up((int64_t)a.nchunks * in.kv_heads, 8);
-  const int head_blocks = (a.group + kHPB - 1) / kHPB;
-  hipLaunchKernelGGL(attn_decode_partial, dim3(a.pairs_padded * head_blocks),
+  hipLaunchKernelGGL(attn_decode_partial, dim3(a.pairs_padded * a.group),
                      dim3(kThreads), 0, stream, a);
   if (in.combine)
     hipLaunchKernelGGL(attn_decode_combine, dim3(in.heads), dim3(kD), 0, stream, a);
