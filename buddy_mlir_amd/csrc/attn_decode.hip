@@ -164,6 +164,7 @@ __global__ void __launch_bounds__(kThreads) attn_decode_partial(AttnArgs a) {
 
   // ---- scores of this wavefront's 16 positions ------------------------------
   // every lane of a half ends up with the 8 scores of its half's rows
+  BH_TL_AFTER(g_tl_attn, tl_wave, 6, kreg[kR - 1].x);
   const float4 q4 = *reinterpret_cast<const float4 *>(q_s + c4 * 4);
   float sc[kR];
 #pragma unroll
@@ -191,6 +192,7 @@ __global__ void __launch_bounds__(kThreads) attn_decode_partial(AttnArgs a) {
   }
   l_w += __shfl_xor(l_w, 32, 64);
   BH_TL(g_tl_attn, tl_wave, 3);
+  BH_TL_AFTER(g_tl_attn, tl_wave, 7, vreg[kR - 1].x);
 
   // ---- acc[d] = sum_p e[p] * V[p][d]: this lane's 8 rows x 4 dims -----------
   float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);

@@ -68,6 +68,12 @@ constexpr int kTileBytes = 1024;   // one wavefront-wide 128-bit load
     if ((threadIdx.x & 63) == 0)                                               \
       name[(((size_t)(wave_id)) * 8 + (slot)) & ((1u << 18) - 1)] = wall_clock64(); \
   } while (0)
+// the same once `value` (the result of a load) has arrived
+#define BH_TL_AFTER(name, wave_id, slot, value)                                \
+  do {                                                                         \
+    asm volatile("" ::"v"(value));                                             \
+    BH_TL(name, wave_id, slot);                                                \
+  } while (0)
 #define BH_TL_EXPORT(fn, name)                                                 \
   extern "C" int fn(unsigned long long *dst, size_t count) {                   \
     return (int)hipMemcpyFromSymbol(dst, HIP_SYMBOL(name),                     \
@@ -76,6 +82,9 @@ constexpr int kTileBytes = 1024;   // one wavefront-wide 128-bit load
 #else
 #define BH_TL_DECLARE(name)
 #define BH_TL(name, wave_id, slot)                                             \
+  do {                                                                         \
+  } while (0)
+#define BH_TL_AFTER(name, wave_id, slot, value)                                \
   do {                                                                         \
   } while (0)
 #define BH_TL_EXPORT(fn, name)
