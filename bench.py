@@ -24,9 +24,37 @@ ROOT = Path(__file__).resolve().parent
 sys.path.insert(0, str(ROOT))
 sys.path.insert(0, str(ROOT / "tests"))
 
-GATE_UP_HBM_TRAFFIC_BYTES = 27893551
+# The CPU baseline runs OpenMP loops: pin its threads to neighbouring cores like
+# the reference's own runs do (docs/Runtime.md:192 leaves the thread count to
+# OMP_NUM_THREADS).  Must be in the environment before any OpenMP runtime loads.
+OMP_BINDING = {"OMP_PROC_BIND": "close", "OMP_PLACES": "cores"}
+for _k, _v in OMP_BINDING.items():
+    os.environ.setdefault(_k, _v)
+
 HBM_PEAK_GBPS = 8000.0  # MI355X published HBM3E bandwidth
 CONTEXT = 1024
+GATE_UP_KERNEL = "gemv_w8a32_bcast_kernel<1, 2, 1, 4, true>"
+TRAFFIC_PROFILE = "profiles/decode_kernels_hbm_traffic.md"
+
+
+def gate_up_traffic():
+    """HBM bytes per launch of the dominant kernel as the counter summary under
+    profiles/ records them (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by a
+    copy of known size): a counter reading, not something this script can
+    measure live.  Refuses a summary that was taken for another kernel."""
+    import re
+
+    path = ROOT / TRAFFIC_PROFILE
+    if not path.exists():
+        return None, f"{TRAFFIC_PROFILE} not found"
+    m = re.search(r"gate\|up GEMV \(`([^`]+)`\) per launch:.*?=\s*([0-9,]+) B against",
+                  path.read_text(), re.S)
+    if not m:
+        raise SystemExit(f"bench.py: no per-launch traffic line in {TRAFFIC_PROFILE}")
+    if m.group(1) != GATE_UP_KERNEL:
+        raise SystemExit(f"bench.py: {TRAFFIC_PROFILE} holds the traffic of `{m.group(1)}`, "
+                         f"but the dominant kernel is `{GATE_UP_KERNEL}`: take the counters again")
+    return int(m.group(2).replace(",", "")), TRAFFIC_PROFILE
 
 
 def gate_up_bytes(hidden: int, inter: int) -> int:
@@ -50,7 +78,8 @@ def decode_step_bytes(shape, ctx: int) -> int:
 def time_gate_up(bh, shape, sess_stream, layers, iters):
     """Average duration of the dominant kernel (fused gate|up GEMV), launched
     back to back over `layers` distinct weight sets (more than the 256 MB
-    last-level cache holds), timed with HIP events on the launch stream."""
+    last-level cache holds) from a replayed hipGraph, as the decode step
+    launches it, timed with HIP events on the launch stream."""
     import torch
     from buddy_mlir_amd import check, ops, synthetic
 
@@ -77,12 +106,24 @@ def time_gate_up(bh, shape, sess_stream, layers, iters):
     stream = torch.cuda.ExternalStream(sess_stream)
     for d in descs:
         check(bh.buddy_hip_linear_w8a32(ctypes.byref(d), sess_stream))
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     stream.synchronize()
-    e0.record(stream)
-    for i in range(iters):
-        bh.buddy_hip_linear_w8a32(ctypes.byref(descs[i % layers]), sess_stream)
-    e1.record(stream)
+
+    def enqueue():
+        for i in range(iters):
+            bh.buddy_hip_linear_w8a32(ctypes.byref(descs[i % layers]), sess_stream)
+
+    # the decode step launches this kernel from a replayed hipGraph: time it the
+    # same way, `iters` launches per replay
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=stream):
+        enqueue()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    with torch.cuda.stream(stream):
+        graph.replay()
+        stream.synchronize()
+        e0.record(stream)
+        graph.replay()
+        e1.record(stream)
     e1.synchronize()
     return e0.elapsed_time(e1) * 1e-3 / iters
 
@@ -110,7 +151,8 @@ def cpu_baseline(shape, host, first_token, budget_s=12.0, max_steps=4096):
     return {"value": n / dt, "unit": "tokens/s", "cores": oracle.num_threads(),
             "kind": "port",
             "sample": f"{n} decode steps at context {CONTEXT}, same weights, "
-                      f"{dt:.1f} s of CPU time"}
+                      f"{dt:.1f} s of CPU time",
+            "omp": {k: os.environ.get(k) for k in OMP_BINDING}}
 
 
 # ---------------------------------------------------------------------------
@@ -179,6 +221,43 @@ def _linear_bytes(K, N, M, dual, norm):
     return (2 if dual else 1) * (K * N + 4 * N) + 4 * M * (K + N) + (4 * K if norm else 0)
 
 
+def cpu_baseline_gemv(K, N, budget_s=6.0, copies=8):
+    """The CPU oracle's int8 GEMV on this shape, weights rotated over `copies`
+    matrices (110 MB: beyond the host's last-level cache), ~budget_s each for the
+    reference's plain row-major layout (stride-N inner loop,
+    DequantMatMulVectorizationDecode.cpp:259-283) and for the same loop over the
+    reference's packed-panel order applied to int8, so that the GPU is not
+    compared with the slower layout only."""
+    import numpy as np
+
+    import oracle_lib
+
+    oracle = oracle_lib.load()
+    rng = np.random.default_rng(1)
+    x = rng.standard_normal(K).astype(np.float32)
+    scale = np.full(N, 1e-3, np.float32)
+    plain = [rng.integers(-127, 128, (K, N), dtype=np.int8) for _ in range(copies)]
+    panels = [np.ascontiguousarray(w.reshape(K, N // 32, 32).transpose(1, 0, 2)) for w in plain]
+    by = K * N + 4 * N + 4 * (K + N)
+    out = {}
+    for name, fn in (("plain_row_major", lambda i: oracle.dequant_gemv(x, plain[i], scale)),
+                     ("packed_panels", lambda i: oracle.dequant_gemv_panels(x, panels[i], scale, K, N))):
+        fn(0)
+        t0 = time.perf_counter()
+        n = 0
+        while time.perf_counter() - t0 < budget_s:
+            fn(n % copies)
+            n += 1
+        dt = (time.perf_counter() - t0) / n
+        out[name] = {"us": dt * 1e6, "gbps": by / dt / 1e9, "calls": n}
+    return {"value": out["plain_row_major"]["gbps"], "unit": "GB/s",
+            "cores": oracle.num_threads(), "kind": "port",
+            "sample": f"{out['plain_row_major']['calls']} + {out['packed_panels']['calls']} "
+                      f"GEMVs {K} -> {N} over {copies} rotating matrices, {budget_s:.0f} s each",
+            "plain_row_major": out["plain_row_major"], "packed_panels": out["packed_panels"],
+            "omp": {k: os.environ.get(k) for k in OMP_BINDING}}
+
+
 def bench_gemv(bh, args):
     """configs[0]: one int8 GEMV 1536 -> 8960 at M = 1, weights rotated over 48
     copies (HBM-cold, 660 MB) and over one copy (cache-warm)."""
@@ -239,7 +318,9 @@ def bench_gemv(bh, args):
                                    "frac": byf / tp / 1e9 / HBM_PEAK_GBPS}
     del Pf
     t = res["hbm_cold"]["us"] * 1e-6
+    cpu = None if args.no_cpu_baseline else cpu_baseline_gemv(K, N)
     return {
+        **({"cpu_baseline": cpu} if cpu else {}),
         "metric": "int8_gemv_hbm_gbps", "value": res["hbm_cold"]["gbps"], "unit": "GB/s",
         "n_gpus": 1, "steps": 960, "warmup": 8, "ms_per_step": t * 1e3,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
@@ -790,6 +871,7 @@ def main():
     gu_b = gate_up_bytes(shape.hidden, shape.inter)
     achieved = gu_b / gu_s / 1e9
     step_b = decode_step_bytes(shape, CONTEXT + W + K // 2)
+    traffic, traffic_source = gate_up_traffic()
 
     out = {
         "metric": "decode_tokens_per_s",
@@ -816,7 +898,7 @@ def main():
         "decode_step_hbm_gbps": step_b / step_s / 1e9,
         "decode_step_hbm_frac": step_b / step_s / 1e9 / HBM_PEAK_GBPS,
         "roofline": {
-            "kernel": "gemv_w8a32_bcast_kernel<1, 2, 1, 4, true> (RMSNorm + gate|up int8 GEMV "
+            "kernel": GATE_UP_KERNEL + " (RMSNorm + gate|up int8 GEMV "
                       "+ SiLU*mul, 1536 -> 2 x 8960)",
             "bound": "hbm",
             "achieved": achieved,
@@ -825,10 +907,8 @@ def main():
             "frac": achieved / HBM_PEAK_GBPS,
             "algorithmic_bytes_per_launch": gu_b,
             "avg_launch_us": gu_s * 1e6,
-            # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-            # (13614.6 KiB x 1.99982 + 35 KiB x 1.0, factors from a 256 MiB copy);
-            # a counter reading, not something this script can measure live
-            "traffic": GATE_UP_HBM_TRAFFIC_BYTES,
+            "traffic": traffic,
+            "traffic_source": traffic_source,
         },
     }
     if args.calibrate_copy:

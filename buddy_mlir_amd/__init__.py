@@ -85,6 +85,8 @@ def _declare(lib):
         "buddy_hip_version": (c_char_p, []),
         "buddy_hip_last_error": (c_char_p, []),
         "buddy_hip_device_count": (c_int, []),
+        "buddy_hip_variant_report": (i64, [vp, i64]),
+        "buddy_hip_variant_reset": (None, []),
         "buddy_hip_w8_packed_bytes": (sz, [i64, i64]),
         "buddy_hip_pack_w8": (c_int, [vp, i64, i64, vp, vp]),
         "buddy_hip_unpack_w8": (c_int, [vp, i64, i64, vp, vp]),
@@ -126,6 +128,8 @@ def _declare(lib):
         "buddy_hip_session_prefill_all_logits": (c_int, [vp, vp, c_int, c_int, vp]),
         "buddy_hip_session_adopt": (None, [vp, vp]),
         "buddy_hip_w8a32_blob_sizes": (None, [vp, vp, vp]),
+        "buddy_hip_w8a32_blob_layout": (i64, [vp, vp, i64]),
+        "buddy_hip_set_gemv_batch_kernel": (c_int, [c_int]),
         "buddy_hip_session_create_from_w8a32_blobs": (vp, [vp, vp, i64, vp, i64]),
         "_mlir_ciface_forward_prefill": (None, [vp, vp, vp, vp]),
         "_mlir_ciface_forward_decode": (None, [vp] * 88),

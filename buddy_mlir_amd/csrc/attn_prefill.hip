@@ -285,6 +285,8 @@ rope_kv_write_kernel(float *qkv, int64_t row_stride, const float *inv_freq,
 
 } // namespace
 
+BH_VARIANT_FAMILY(AttnPrefillFamily, "attn_prefill_kernel");
+
 int launch_attn_prefill(const AttnPrefillArgs &in, hipStream_t stream) {
   BH_REQUIRE(in.q && in.k && in.v && in.out, "attn_prefill: null pointer");
   BH_REQUIRE(in.head_dim == kD, "attn_prefill: head_dim %d (only %d is built)",
@@ -316,6 +318,7 @@ int launch_attn_prefill(const AttnPrefillArgs &in, hipStream_t stream) {
   a.q_offset = in.k_len - in.q_len; // the last query sees every key
   a.scale = in.scale;
   BH_REQUIRE(ceil_div(in.q_len, kQB) <= 65535, "attn_prefill: q_len %d too long", in.q_len);
+  BH_NOTE_VARIANT(AttnPrefillFamily);
   hipLaunchKernelGGL(attn_prefill_kernel, dim3(in.heads, (unsigned)ceil_div(in.q_len, kQB)),
                      dim3(kAttnWaves * kWave), 0, stream, a);
   BH_CHECK_HIP(hipGetLastError());

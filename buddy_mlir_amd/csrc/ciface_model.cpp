@@ -90,17 +90,74 @@ buddy_hip_model_shape default_shape(int kv_heads, int max_len, int head_dim) {
   return s;
 }
 
+// The parameters of the reference's w8a32 package in the order they lie in the
+// two blobs, with running element offsets per dtype.
+//  * Parameters keep their trace order = the order of the function arguments of
+//    examples/BuddyDeepSeekR1/subgraph0_decode_simplify.mlir:4 with the run-time
+//    inputs (token, positions, KV caches) left out; packing walks them in that
+//    order and advances one running offset per dtype
+//    (frontend/Python/graph/graph.py:848-863, 1001-1018).
+//  * The weights of plain matmuls (o_proj, gate, up, down, lm_head) are int8,
+//    the q/k/v weights, which feed a matmul + bias add, stay f32
+//    (frontend/Python/graph/transform/quantization/weight_only_channel_wise.py
+//    :366-461).
+//  * One f32 scaler vector per int8 weight follows all original parameters, in
+//    the order of the weights
+//    (frontend/Python/graph/transform/quantization/quantize.py:561-590).
+std::vector<buddy_hip_blob_entry> blob_layout(const buddy_hip_model_shape &S) {
+  const int64_t H = S.hidden, QN = (int64_t)S.heads * S.head_dim,
+                KVN = (int64_t)S.kv_heads * S.head_dim, I = S.inter, V = S.vocab;
+  std::vector<buddy_hip_blob_entry> t;
+  int64_t off[2] = {0, 0};
+  auto add = [&](int param, int layer, int dtype, int64_t rows, int64_t cols) {
+    buddy_hip_blob_entry e;
+    e.param = param;
+    e.layer = layer;
+    e.dtype = dtype;
+    e.reserved = 0;
+    e.rows = rows;
+    e.cols = cols;
+    e.offset = off[dtype];
+    e.count = rows * cols;
+    off[dtype] += e.count;
+    t.push_back(e);
+  };
+  constexpr int F = BUDDY_HIP_BLOB_F32, Q = BUDDY_HIP_BLOB_I8;
+  add(BUDDY_HIP_PARAM_EMBED, -1, F, V, H);
+  add(BUDDY_HIP_PARAM_INV_FREQ, -1, F, 1, S.head_dim / 2);
+  for (int l = 0; l < S.layers; ++l) {
+    add(BUDDY_HIP_PARAM_LN1, l, F, 1, H);
+    add(BUDDY_HIP_PARAM_Q_BIAS, l, F, 1, QN);
+    add(BUDDY_HIP_PARAM_Q_W, l, F, H, QN);
+    add(BUDDY_HIP_PARAM_K_BIAS, l, F, 1, KVN);
+    add(BUDDY_HIP_PARAM_K_W, l, F, H, KVN);
+    add(BUDDY_HIP_PARAM_V_BIAS, l, F, 1, KVN);
+    add(BUDDY_HIP_PARAM_V_W, l, F, H, KVN);
+    add(BUDDY_HIP_PARAM_O_W, l, Q, QN, H);
+    add(BUDDY_HIP_PARAM_LN2, l, F, 1, H);
+    add(BUDDY_HIP_PARAM_GATE_W, l, Q, H, I);
+    add(BUDDY_HIP_PARAM_UP_W, l, Q, H, I);
+    add(BUDDY_HIP_PARAM_DOWN_W, l, Q, I, H);
+  }
+  add(BUDDY_HIP_PARAM_LN_F, -1, F, 1, H);
+  add(BUDDY_HIP_PARAM_LM_HEAD_W, -1, Q, H, V);
+  for (int l = 0; l < S.layers; ++l) { // scalers, in weight order
+    add(BUDDY_HIP_PARAM_O_SCALE, l, F, 1, H);
+    add(BUDDY_HIP_PARAM_GATE_SCALE, l, F, 1, I);
+    add(BUDDY_HIP_PARAM_UP_SCALE, l, F, 1, I);
+    add(BUDDY_HIP_PARAM_DOWN_SCALE, l, F, 1, H);
+  }
+  add(BUDDY_HIP_PARAM_LM_HEAD_SCALE, -1, F, 1, V);
+  return t;
+}
+
 struct BlobSizes {
   int64_t f32, i8;
 };
 BlobSizes blob_sizes(const buddy_hip_model_shape &S) {
-  const int64_t H = S.hidden, QN = (int64_t)S.heads * S.head_dim,
-                KVN = (int64_t)S.kv_heads * S.head_dim, I = S.inter, V = S.vocab;
-  BlobSizes b;
-  b.f32 = V * H + S.head_dim / 2 +
-          S.layers * (H + QN + H * QN + KVN + H * KVN + KVN + H * KVN + H) + H +
-          S.layers * (H + I + I + H) + V;
-  b.i8 = S.layers * (QN * H + 3 * H * I) + H * V;
+  BlobSizes b{0, 0};
+  for (const buddy_hip_blob_entry &e : blob_layout(S))
+    (e.dtype == BUDDY_HIP_BLOB_F32 ? b.f32 : b.i8) += e.count;
   return b;
 }
 
@@ -154,39 +211,43 @@ int session_from_blobs(const float *f32, int64_t n_f32, const int8_t *i8,
     return cleanup(fail(BUDDY_HIP_ERR_HIP, "w8a32 blobs: upload failed: %s",
                         hipGetErrorString(hipGetLastError())));
 
-  const int64_t H = S.hidden, QN = (int64_t)S.heads * S.head_dim,
-                KVN = (int64_t)S.kv_heads * S.head_dim, I = S.inter, V = S.vocab;
-  const float *p = dev_f32;
-  const float *embed = p;            p += V * H;
-  const float *inv_freq = p;         p += S.head_dim / 2;
+  // cut the blobs into tensors by the one layout table
+  const std::vector<buddy_hip_blob_entry> table = blob_layout(S);
+  const float *embed = nullptr, *inv_freq = nullptr, *ln_f = nullptr, *s_lm = nullptr;
+  const int8_t *w_lm = nullptr;
   std::vector<buddy_hip_layer_weights> lw((size_t)S.layers);
-  for (auto &w : lw) {
+  for (auto &w : lw)
     std::memset(&w, 0, sizeof(w));
-    w.ln1 = p; p += H;
-    w.bq = p;  p += QN;
-    w.fq = p;  p += H * QN;
-    w.bk = p;  p += KVN;
-    w.fk = p;  p += H * KVN;
-    w.bv = p;  p += KVN;
-    w.fv = p;  p += H * KVN;
-    w.ln2 = p; p += H;
+  for (const buddy_hip_blob_entry &e : table) {
+    const float *pf = dev_f32 + e.offset;
+    const int8_t *pi = dev_i8 + e.offset;
+    buddy_hip_layer_weights *w = e.layer >= 0 ? &lw[(size_t)e.layer] : nullptr;
+    switch (e.param) {
+    case BUDDY_HIP_PARAM_EMBED:    embed = pf; break;
+    case BUDDY_HIP_PARAM_INV_FREQ: inv_freq = pf; break;
+    case BUDDY_HIP_PARAM_LN1:      w->ln1 = pf; break;
+    case BUDDY_HIP_PARAM_Q_BIAS:   w->bq = pf; break;
+    case BUDDY_HIP_PARAM_Q_W:      w->fq = pf; break;
+    case BUDDY_HIP_PARAM_K_BIAS:   w->bk = pf; break;
+    case BUDDY_HIP_PARAM_K_W:      w->fk = pf; break;
+    case BUDDY_HIP_PARAM_V_BIAS:   w->bv = pf; break;
+    case BUDDY_HIP_PARAM_V_W:      w->fv = pf; break;
+    case BUDDY_HIP_PARAM_O_W:      w->wo = pi; break;
+    case BUDDY_HIP_PARAM_LN2:      w->ln2 = pf; break;
+    case BUDDY_HIP_PARAM_GATE_W:   w->wg = pi; break;
+    case BUDDY_HIP_PARAM_UP_W:     w->wu = pi; break;
+    case BUDDY_HIP_PARAM_DOWN_W:   w->wd = pi; break;
+    case BUDDY_HIP_PARAM_LN_F:     ln_f = pf; break;
+    case BUDDY_HIP_PARAM_LM_HEAD_W: w_lm = pi; break;
+    case BUDDY_HIP_PARAM_O_SCALE:    w->so = pf; break;
+    case BUDDY_HIP_PARAM_GATE_SCALE: w->sg = pf; break;
+    case BUDDY_HIP_PARAM_UP_SCALE:   w->su = pf; break;
+    case BUDDY_HIP_PARAM_DOWN_SCALE: w->sd = pf; break;
+    case BUDDY_HIP_PARAM_LM_HEAD_SCALE: s_lm = pf; break;
+    default:
+      return cleanup(fail(BUDDY_HIP_ERR_ARG, "w8a32 blobs: unknown parameter %d", e.param));
+    }
   }
-  const float *ln_f = p;             p += H;
-  for (auto &w : lw) {               // scalers, in weight order
-    w.so = p; p += H;
-    w.sg = p; p += I;
-    w.su = p; p += I;
-    w.sd = p; p += H;
-  }
-  const float *s_lm = p;             p += V;
-  const int8_t *q = dev_i8;
-  for (auto &w : lw) {
-    w.wo = q; q += QN * H;
-    w.wg = q; q += H * I;
-    w.wu = q; q += H * I;
-    w.wd = q; q += I * H;
-  }
-  const int8_t *w_lm = q;
   int rc = buddy_hip_session_set_globals(sess, embed, inv_freq, ln_f, w_lm, s_lm);
   for (int i = 0; !rc && i < S.layers; ++i)
     rc = buddy_hip_session_set_layer(sess, i, &lw[(size_t)i]);
@@ -517,6 +578,18 @@ buddy_hip_session *buddy_hip_session_create_from_w8a32_blobs(
   buddy_hip_session_adopt(sess, dev_f32); // freed with the session
   return sess;
 } BH_CATCH_NULL("buddy_hip_session_create_from_w8a32_blobs")
+
+int64_t buddy_hip_w8a32_blob_layout(const buddy_hip_model_shape *shape,
+                                    buddy_hip_blob_entry *entries, int64_t capacity) try {
+  if (!shape)
+    return 0;
+  const std::vector<buddy_hip_blob_entry> t = bh::blob_layout(*shape);
+  for (int64_t i = 0; entries && i < capacity && i < (int64_t)t.size(); ++i)
+    entries[i] = t[(size_t)i];
+  return (int64_t)t.size();
+} catch (...) {
+  return 0;
+}
 
 void buddy_hip_w8a32_blob_sizes(const buddy_hip_model_shape *shape, int64_t *n_f32,
                                 int64_t *n_i8) try {

@@ -5,6 +5,7 @@
 
 #include <cstdarg>
 #include <cstdint>
+#include <initializer_list>
 #include <cstdio>
 
 #include "buddy_hip/buddy_hip.h"
@@ -89,6 +90,23 @@ constexpr int kTileBytes = 1024;   // one wavefront-wide 128-bit load
   } while (0)
 #define BH_TL_EXPORT(fn, name)
 #endif
+
+// ---- which template instantiations of the hand-scheduled kernels were launched
+// Every instantiation a launch site can reach registers itself when the library
+// is loaded (a static member of Variant<Family, params...>, instantiated where
+// the launch site names it) and counts its launches, so that a test can ask
+// whether every compiled variant of such a kernel has met the oracle
+// (buddy_hip_variant_report).
+int register_variant(const char *family, std::initializer_list<int> params);
+void note_variant_launch(int id);
+template <typename Family, int... P> struct Variant {
+  static inline const int id = register_variant(Family::name, {P...});
+};
+#define BH_VARIANT_FAMILY(tag, text)                                           \
+  struct tag {                                                                 \
+    static constexpr const char *name = text;                                  \
+  }
+#define BH_NOTE_VARIANT(...) ::bh::note_variant_launch(::bh::Variant<__VA_ARGS__>::id)
 
 inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 inline int64_t round_up(int64_t a, int64_t b) { return ceil_div(a, b) * b; }

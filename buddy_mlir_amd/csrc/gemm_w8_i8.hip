@@ -654,11 +654,15 @@ reduce_slices_kernel(GemmI8Args a, int rb_per_tile, int gpw) {
     }
 }
 
+BH_VARIANT_FAMILY(WideFamily, "gemm_w8_i8_wide_kernel");
+BH_VARIANT_FAMILY(SplitFamily, "gemm_w8_i8_kernel");
+
 template <int D, int RB, int GPW>
 int launch_wide(const GemmI8Args &a, unsigned blocks, hipStream_t stream) {
   // three fragment buffers in the loop, four output tiles in the epilogue
   constexpr size_t lds = std::max(sizeof(v4i32) * 3 * D * RB * kWave,
                                   sizeof(float) * kSlices * 16 * (GPW * 16 + 4));
+  BH_NOTE_VARIANT(WideFamily, D, RB, GPW);
   hipLaunchKernelGGL((gemm_w8_i8_wide_kernel<D, RB, GPW>), dim3(blocks),
                      dim3(kSlices * kWave), lds, stream, a);
   BH_CHECK_HIP(hipGetLastError());
@@ -747,6 +751,7 @@ template <int D> int launch_split(const GemmI8Args &a, unsigned blocks, hipStrea
                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
     attr_set = true;
   }
+  BH_NOTE_VARIANT(SplitFamily, D);
   hipLaunchKernelGGL(kernel, dim3(blocks), dim3(kSlices * kWave), lds, stream, a);
   BH_CHECK_HIP(hipGetLastError());
   return BUDDY_HIP_OK;
@@ -839,8 +844,6 @@ int launch_gemm_w8_digits(const GemmW8Args &in, const void *planes, hipStream_t 
     a.ncols = (int)ceil_div(a.groups, kSplitGroups);
     a.cols_padded = (int)round_up(a.ncols, 8);
     const unsigned blocks = (unsigned)(a.cols_padded * (a.Mp / 64));
-    if (in.digits == 2)
-      return launch_split<2>(a, blocks, stream);
     return launch_split<3>(a, blocks, stream);
   }
   a.ncols = (int)ceil_div(a.groups, best_gpw * kSlices);
@@ -857,8 +860,7 @@ int launch_gemm_w8_digits(const GemmW8Args &in, const void *planes, hipStream_t 
     a.partial = reinterpret_cast<float *>(ws);
   }
   const unsigned blocks = (unsigned)(a.cols_padded * row_tiles);
-  int rc = in.digits == 2 ? launch_shape<2>(best_rb, best_gpw, a, blocks, stream)
-                          : launch_shape<3>(best_rb, best_gpw, a, blocks, stream);
+  int rc = launch_shape<3>(best_rb, best_gpw, a, blocks, stream);
   if (rc || best_s == 1)
     return rc;
   const int64_t threads = (int64_t)a.M * ((a.N + 3) / 4);

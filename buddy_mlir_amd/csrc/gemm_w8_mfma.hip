@@ -557,9 +557,13 @@ int staging_for(hipStream_t stream, size_t bytes, const GemmW8Args &in, u16 **ou
   return BUDDY_HIP_OK;
 }
 
+BH_VARIANT_FAMILY(WideFamily, "gemm_w8_bf16_wide_kernel");
+BH_VARIANT_FAMILY(SplitFamily, "gemm_w8_bf16_kernel");
+
 template <int TERMS, int RB>
 int launch_wide(const GemmArgs &a, unsigned blocks, hipStream_t stream) {
   constexpr size_t lds = sizeof(v4i32) * 2 * TERMS * 2 * RB * kWave;
+  BH_NOTE_VARIANT(WideFamily, TERMS, RB);
   hipLaunchKernelGGL((gemm_w8_bf16_wide_kernel<TERMS, RB>), dim3(blocks),
                      dim3(kSlices * kWave), lds, stream, a);
   BH_CHECK_HIP(hipGetLastError());
@@ -577,6 +581,7 @@ int launch_terms(const GemmArgs &a, unsigned blocks, hipStream_t stream) {
                                      (int)lds));
     attr_set = true;
   }
+  BH_NOTE_VARIANT(SplitFamily, TERMS);
   hipLaunchKernelGGL(kernel, dim3(blocks), dim3(kSlices * kWave), lds, stream, a);
   BH_CHECK_HIP(hipGetLastError());
   return BUDDY_HIP_OK;
@@ -624,9 +629,11 @@ int launch_gemm_w8(const GemmW8Args &in, hipStream_t stream) {
              (long long)in.K, (long long)in.N);
   BH_REQUIRE((in.staged || in.lda >= in.K) && in.ldc >= in.N,
              "gemm_w8: row stride below row length");
-  BH_REQUIRE(in.terms >= 1 && in.terms <= 3, "gemm_w8: terms=%d outside 1..3", in.terms);
-  BH_REQUIRE(in.digits == 0 || (in.digits >= 2 && in.digits <= 3),
-             "gemm_w8: digits=%d outside 2..3", in.digits);
+  // one bf16 term (activations cast to bf16) or three (every f32 bit); digit
+  // planes always three: the variants in between were never reachable from an
+  // entry point and are not built
+  BH_REQUIRE(in.terms == 1 || in.terms == 3, "gemm_w8: terms=%d (1 or 3)", in.terms);
+  BH_REQUIRE(in.digits == 0 || in.digits == 3, "gemm_w8: digits=%d (0 or 3)", in.digits);
   BH_REQUIRE(in.digits == 0 || in.K <= (1 << 17),
              "gemm_w8: K=%lld beyond 2^17 would overflow the int32 sums of the digit planes",
              (long long)in.K);
@@ -682,25 +689,12 @@ int launch_gemm_w8(const GemmW8Args &in, hipStream_t stream) {
     a.ncols = wide_cols;
     a.cols_padded = (int)round_up(wide_cols, 8);
     const unsigned wb = (unsigned)(a.cols_padded * ceil_div(in.M, rows));
-    if (three) {
-      switch (in.terms) {
-      case 1: return launch_wide<1, 3>(a, wb, stream);
-      case 2: return launch_wide<2, 3>(a, wb, stream);
-      default: return launch_wide<3, 3>(a, wb, stream);
-      }
-    }
-    switch (in.terms) {
-    case 1: return launch_wide<1, 4>(a, wb, stream);
-    case 2: return launch_wide<2, 4>(a, wb, stream);
-    default: return launch_wide<3, 4>(a, wb, stream);
-    }
+    if (three)
+      return in.terms == 1 ? launch_wide<1, 3>(a, wb, stream) : launch_wide<3, 3>(a, wb, stream);
+    return in.terms == 1 ? launch_wide<1, 4>(a, wb, stream) : launch_wide<3, 4>(a, wb, stream);
   }
   const unsigned blocks = (unsigned)(a.cols_padded * (a.Mp / kRowsPerWave));
-  switch (in.terms) {
-  case 1: return launch_terms<1>(a, blocks, stream);
-  case 2: return launch_terms<2>(a, blocks, stream);
-  default: return launch_terms<3>(a, blocks, stream);
-  }
+  return in.terms == 1 ? launch_terms<1>(a, blocks, stream) : launch_terms<3>(a, blocks, stream);
 }
 
 void release_gemm_staging(hipStream_t stream) {

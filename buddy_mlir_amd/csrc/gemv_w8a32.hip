@@ -28,6 +28,7 @@
 // No MFMA: at M = 1 the arithmetic is far below the bandwidth ridge.
 #include "gemv_w8a32.h"
 
+#include <atomic>
 #include <cstdlib>
 #include <cstring>
 
@@ -994,12 +995,21 @@ int launch_m(const GemvArgs &a, const KernelArgs &ka, const GemvPlan &p,
   return fail(BUDDY_HIP_ERR_ARG, "gemv: unknown epilogue %d", a.epilogue);
 }
 
-// BUDDY_HIP_GEMV_BATCH=bf16 sends batches of 5..16 rows to the bf16 matrix-core
-// kernel (three bf16 terms per activation: every f32 bit) instead of the int8
-// one.  Read at every call, so a host can switch between calls.
+// Which matrix-core kernel takes batches of 5..16 rows: 0 = int8 (default),
+// 1 = bf16 (three bf16 terms per activation: every f32 bit).  The environment
+// variable BUDDY_HIP_GEMV_BATCH=bf16 sets the default, read once per process;
+// buddy_hip_set_gemv_batch_kernel changes it between calls.
+std::atomic<int> g_batch_kernel{-1};
 bool batch_bf16() {
-  const char *e = getenv("BUDDY_HIP_GEMV_BATCH");
-  return e && strcmp(e, "bf16") == 0;
+  int k = g_batch_kernel.load(std::memory_order_relaxed);
+  if (k < 0) {
+    const char *e = getenv("BUDDY_HIP_GEMV_BATCH");
+    k = e && strcmp(e, "bf16") == 0;
+    int expected = -1; // a setter that ran meanwhile wins
+    if (!g_batch_kernel.compare_exchange_strong(expected, k))
+      k = expected;
+  }
+  return k == 1;
 }
 bool force_valu() {
   static bool v = getenv("BUDDY_HIP_GEMV_FORCE_VALU") != nullptr;
@@ -1086,6 +1096,13 @@ BH_TL_EXPORT(buddy_hip_debug_timeline_gemv, g_tl_gemv)
 } // namespace bh
 
 extern "C" {
+
+int buddy_hip_set_gemv_batch_kernel(int kernel) try {
+  BH_REQUIRE(kernel == BUDDY_HIP_GEMV_BATCH_INT8 || kernel == BUDDY_HIP_GEMV_BATCH_BF16,
+             "set_gemv_batch_kernel: %d (0 = int8, 1 = bf16)", kernel);
+  bh::g_batch_kernel.store(kernel, std::memory_order_relaxed);
+  return BUDDY_HIP_OK;
+} BH_CATCH_INT("buddy_hip_set_gemv_batch_kernel")
 
 int buddy_hip_linear_w8a32(const buddy_hip_linear_desc *d,
                            buddy_hip_stream stream) try {

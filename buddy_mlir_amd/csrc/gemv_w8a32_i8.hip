@@ -392,6 +392,8 @@ __global__ void __launch_bounds__(kMaxWavesI8 *kWave, 3) // 3 wavefronts per SIM
   }
 }
 
+BH_VARIANT_FAMILY(I8Family, "gemv_w8a32_i8_kernel");
+
 template <int EPI, int SPAN, bool NORM>
 int launch_kernel(const I8Args &ka, int blocks, hipStream_t stream) {
   constexpr int NA = (EPI == kEpiSiluMul) ? 2 * SPAN : SPAN;
@@ -406,6 +408,7 @@ int launch_kernel(const I8Args &ka, int blocks, hipStream_t stream) {
                                      144 * 1024));
     attr_set = true;
   }
+  BH_NOTE_VARIANT(I8Family, EPI, SPAN, NORM);
   hipLaunchKernelGGL(kernel, dim3(blocks), dim3(waves * kWave), lds, stream, ka);
   BH_CHECK_HIP(hipGetLastError());
   return BUDDY_HIP_OK;

@@ -374,6 +374,8 @@ __global__ void __launch_bounds__(kMaxWavesMfma *kWave)
   }
 }
 
+BH_VARIANT_FAMILY(MfmaFamily, "gemv_w8a32_mfma_kernel");
+
 template <int EPI, int SPAN, bool NORM>
 int launch_kernel(const MfmaArgs &ka, int blocks, hipStream_t stream) {
   constexpr int NA = (EPI == kEpiSiluMul) ? 2 * SPAN : SPAN;
@@ -387,6 +389,7 @@ int launch_kernel(const MfmaArgs &ka, int blocks, hipStream_t stream) {
                                      144 * 1024));
     attr_set = true;
   }
+  BH_NOTE_VARIANT(MfmaFamily, EPI, SPAN, NORM);
   hipLaunchKernelGGL(kernel, dim3(blocks), dim3(waves * kWave), lds, stream, ka);
   BH_CHECK_HIP(hipGetLastError());
   return BUDDY_HIP_OK;

@@ -18,7 +18,7 @@
 // Run it under `rocprofv3 --kernel-trace --stats` to see the same chains as
 // per-kernel durations.
 //
-//   launch_floor_probe [--chain 128] [--replays 20] [--no-graph]
+//   launch_floor_probe [--chain 128] [--replays 20] [--no-graph] [--layer]
 #include <hip/hip_runtime.h>
 
 #include <cstdint>
@@ -46,6 +46,7 @@ namespace {
 
 int g_chain = 128, g_replays = 20;
 bool g_graph = true;
+bool g_layer_only = false; // --layer: only the GEMV ladder and the fused launches
 hipStream_t g_stream;
 
 // Captures `chain` launches made by `enqueue(i)` into a graph, replays it and
@@ -107,6 +108,8 @@ int main(int argc, char **argv) {
       g_replays = atoi(argv[++i]);
     else if (!strcmp(argv[i], "--no-graph"))
       g_graph = false;
+    else if (!strcmp(argv[i], "--layer"))
+      g_layer_only = true;
   }
   CK(hipStreamCreateWithFlags(&g_stream, hipStreamNonBlocking));
   int *sink; // 16 ints per wavefront of the largest grid
@@ -132,6 +135,8 @@ int main(int argc, char **argv) {
          "codeloop");
   const unsigned window = 16u << 20; // a fresh 16 MiB per launch: tiles come from HBM
   for (const Grid &g : grids) {
+    if (g_layer_only)
+      break;
     auto run = [&](bool pre, int which) {
       return time_chain([&](int i) {
         const int8_t *w = pool + ((size_t)i * window) % (pool_bytes - window);
@@ -149,7 +154,7 @@ int main(int argc, char **argv) {
   }
 
   // ---- how long the dispatcher takes to start every wavefront of a grid -----
-  {
+  if (!g_layer_only) {
     printf("\ndispatch spread: first to last wavefront start of one launch, us "
            "(median of 20 launches)\n");
     printf("%-12s %8s %10s %12s %14s\n", "grid", "waves", "no LDS", "1 KiB LDS", "14 args in SGPRs");
@@ -200,7 +205,7 @@ int main(int argc, char **argv) {
          (long long)K, pool_bytes >> 20);
   printf("%10s %10s %10s %10s\n", "MB", "N", "us", "GB/s");
   std::vector<double> xs, ys;
-  for (int mb = 1; mb <= 256; mb *= 2) {
+  for (int mb = 1; mb <= (g_layer_only ? 32 : 256); mb *= 2) {
     const int64_t N = ((int64_t)mb << 20) / K / 16 * 16;
     const size_t bytes = (size_t)K * N;
     const size_t slots = pool_bytes / bytes;

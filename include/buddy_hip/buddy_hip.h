@@ -47,6 +47,17 @@ const char *buddy_hip_version(void);
 const char *buddy_hip_last_error(void);
 int buddy_hip_device_count(void);
 
+/* Which compiled variants of the hand-scheduled kernels (the ones that issue
+ * their global loads by hand) this process has launched.  Writes one line per
+ * variant, "name<template arguments>\tlaunch count\n", into `text` (at most
+ * capacity - 1 characters and a terminating 0) and returns the size the whole
+ * report needs.  A variant is listed from the moment the library is loaded,
+ * launched or not, so a test can tell which ones its cases did not reach.
+ * buddy_hip_variant_reset sets every count back to 0.  Host only; no
+ * counterpart in the reference. */
+int64_t buddy_hip_variant_report(char *text, int64_t capacity);
+void buddy_hip_variant_reset(void);
+
 /* ---- packed int8 weight layout ("wave tiles") --------------------------
  * Replaces frontend/Python/graph/transform/pack_decode_weights.py:102-108
  * (panels [N/V][K][V], refused for int8 by tools/buddy-codegen/gen_config.py:
@@ -107,9 +118,14 @@ int buddy_hip_gemv_w4a16(const uint16_t *A, const int8_t *packed, const uint16_t
  * multiple of 4 and A 16-byte aligned) the int8 matrix cores are used: the
  * activations of a row are rounded, 64 at a time, to 2^-23 of the largest of
  * the 64, the sums are exact; a NaN or an infinity in a row turns that row of C
- * into NaN.  With the environment variable BUDDY_HIP_GEMV_BATCH=bf16 (read at
- * every call) those batches keep every bit of the activations instead, on the
- * bf16 matrix cores, at about two thirds of the speed. */
+ * into NaN.  buddy_hip_set_gemv_batch_kernel(BUDDY_HIP_GEMV_BATCH_BF16) makes
+ * those batches keep every bit of the activations instead, on the bf16 matrix
+ * cores, at about two thirds of the speed; the environment variable
+ * BUDDY_HIP_GEMV_BATCH=bf16, read once per process, sets that as the default.
+ * The choice is process-wide.  (No counterpart in the reference, whose decode
+ * pattern is m == 1 only.) */
+enum { BUDDY_HIP_GEMV_BATCH_INT8 = 0, BUDDY_HIP_GEMV_BATCH_BF16 = 1 };
+int buddy_hip_set_gemv_batch_kernel(int kernel);
 enum {
   BUDDY_HIP_GEMV_ACCUMULATE = 1 /* C += ...  (linalg.matmul semantics);
                                    without it C = ... and C need not be
@@ -475,6 +491,33 @@ int buddy_hip_w8a8_matmul(const float *A, const int8_t *packed, const float *wsc
  * Blobs may be host or device memory and are not referenced after the call. */
 void buddy_hip_w8a32_blob_sizes(const buddy_hip_model_shape *shape, int64_t *n_f32,
                                 int64_t *n_i8);
+/* The same layout as a table, one entry per parameter in blob order: which
+ * parameter, its layer (-1: none), which blob, its shape and its element
+ * offset inside that blob (the running offsets of
+ * frontend/Python/graph/graph.py:848-863,1001-1018).  The blob reader below
+ * cuts the blobs by this table and nothing else.  Writes at most `capacity`
+ * entries and returns how many the layout has (0: null shape).  Host only. */
+enum { BUDDY_HIP_BLOB_F32 = 0, BUDDY_HIP_BLOB_I8 = 1 };
+enum {
+  BUDDY_HIP_PARAM_EMBED = 0, BUDDY_HIP_PARAM_INV_FREQ, BUDDY_HIP_PARAM_LN1,
+  BUDDY_HIP_PARAM_Q_BIAS, BUDDY_HIP_PARAM_Q_W, BUDDY_HIP_PARAM_K_BIAS,
+  BUDDY_HIP_PARAM_K_W, BUDDY_HIP_PARAM_V_BIAS, BUDDY_HIP_PARAM_V_W,
+  BUDDY_HIP_PARAM_O_W, BUDDY_HIP_PARAM_LN2, BUDDY_HIP_PARAM_GATE_W,
+  BUDDY_HIP_PARAM_UP_W, BUDDY_HIP_PARAM_DOWN_W, BUDDY_HIP_PARAM_LN_F,
+  BUDDY_HIP_PARAM_LM_HEAD_W, BUDDY_HIP_PARAM_O_SCALE, BUDDY_HIP_PARAM_GATE_SCALE,
+  BUDDY_HIP_PARAM_UP_SCALE, BUDDY_HIP_PARAM_DOWN_SCALE, BUDDY_HIP_PARAM_LM_HEAD_SCALE
+};
+typedef struct buddy_hip_blob_entry {
+  int32_t param;    /* BUDDY_HIP_PARAM_* */
+  int32_t layer;    /* 0.., or -1 */
+  int32_t dtype;    /* BUDDY_HIP_BLOB_F32 / BUDDY_HIP_BLOB_I8 */
+  int32_t reserved;
+  int64_t rows, cols; /* [rows, cols]; vectors have rows = 1 */
+  int64_t offset;   /* elements from the start of its blob */
+  int64_t count;    /* rows * cols */
+} buddy_hip_blob_entry;
+int64_t buddy_hip_w8a32_blob_layout(const buddy_hip_model_shape *shape,
+                                    buddy_hip_blob_entry *entries, int64_t capacity);
 buddy_hip_session *buddy_hip_session_create_from_w8a32_blobs(
     const buddy_hip_model_shape *shape, const float *f32_params, int64_t n_f32,
     const int8_t *i8_params, int64_t n_i8);

@@ -190,10 +190,12 @@ def test_llama3_8b_fused_launches_match_oracle(oracle, M):
 
 
 @pytest.fixture
-def bf16_batch_kernel(monkeypatch):
+def bf16_batch_kernel(bh):
     """Batches of 5..16 rows through the bf16 matrix-core kernel (every f32 bit of
     the activations) instead of the default int8 matrix-core kernel."""
-    monkeypatch.setenv("BUDDY_HIP_GEMV_BATCH", "bf16")
+    assert bh.buddy_hip_set_gemv_batch_kernel(1) == 0
+    yield
+    assert bh.buddy_hip_set_gemv_batch_kernel(0) == 0
 
 
 @pytest.mark.parametrize("K,N", [(1536, 8960), (8960, 1536), (100, 70), (1100, 40)])

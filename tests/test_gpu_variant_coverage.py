@@ -1,0 +1,164 @@
+"""Every compiled variant of the kernels that issue their global loads by hand
+meets the oracle.
+
+Those kernels (the int8 and bf16 matrix-core kernels of the small-batch GEMV
+and of the prefill matmul, and the prefill attention) wait for their loads by
+counting; a mistake in one template variant shows only in that variant.  The
+library lists every variant it was built with (buddy_hip_variant_report); this
+test drives one parity case through each plan that selects one, and fails when
+a variant is left that none of its cases launched -- so a variant added to the
+source without a case here fails the suite."""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+import buddy_mlir_amd as bma
+from buddy_mlir_amd import ops, synthetic
+from parity import check_close
+from test_gpu_prefill import SCALE, bf16_round, run_attn
+
+pytestmark = pytest.mark.gpu
+
+
+def report(bh):
+    n = bh.buddy_hip_variant_report(None, 0)
+    buf = ctypes.create_string_buffer(n)
+    bh.buddy_hip_variant_report(buf, n)
+    out = {}
+    for line in buf.value.decode().splitlines():
+        name, hits = line.split("\t")
+        out[name] = int(hits)
+    return out
+
+
+def launched(bh, family):
+    return {k for k, v in report(bh).items() if k.startswith(family + "<") and v > 0}
+
+
+def compiled(bh, family):
+    return {k for k in report(bh) if k.startswith(family + "<")}
+
+
+# ---- small-batch GEMV: <epilogue, channel groups per wavefront, fused norm> ----
+# N picks the channel groups per wavefront (see launch_gemv_i8 / launch_gemv_mfma)
+def gemv_case(bh, oracle, M, K, N, epilogue, norm, seed):
+    dual = epilogue == 2
+    q0, s0 = synthetic.quantized_linear(K, N, seed)
+    q1, s1 = synthetic.quantized_linear(K, N, seed + 1) if dual else (None, None)
+    g = torch.Generator(device="cuda").manual_seed(seed)
+    x = torch.randn((M, K), generator=g, device="cuda")
+    w = torch.rand((K,), generator=g, device="cuda") + 0.5
+    c0 = torch.randn((M, N), generator=g, device="cuda")
+    c = c0.clone()
+    kw = dict(A=x, lda=K, W0=ops.pack_w8(q0), scale0=s0, C=c, ldc=N, M=M, K=K, N=N,
+              epilogue=epilogue)
+    if dual:
+        kw.update(W1=ops.pack_w8(q1), scale1=s1)
+    if norm:
+        kw.update(norm_w=w, norm_eps=1e-6)
+    torch.cuda.synchronize()
+    ops.linear_w8a32(stream=None, **kw)
+    torch.cuda.synchronize()
+    xh = x.cpu().numpy()
+    if norm:
+        xh = np.stack([oracle.rmsnorm(r, w.cpu().numpy(), eps=np.float32(1e-6)) for r in xh])
+    y0 = np.stack([oracle.dequant_gemv(r, q0.cpu().numpy(), s0.cpu().numpy()) for r in xh])
+    if dual:
+        y1 = np.stack([oracle.dequant_gemv(r, q1.cpu().numpy(), s1.cpu().numpy()) for r in xh])
+        want = np.stack([oracle.silu_mul(a, b) for a, b in zip(y0, y1)])
+    elif epilogue == 1:
+        want = c0.cpu().numpy() + y0
+    else:
+        want = y0
+    got = c.cpu().numpy()
+    for m in range(M):
+        check_close(got[m], want[m])
+
+
+GEMV_I8_N = [320, 8192, 32768]        # 1, 2, 4 channel groups per wavefront
+GEMV_BF16_N = [320, 8192, 131072]     # 2, 4, 8
+
+
+def test_every_int8_batch_gemv_variant(bh, oracle):
+    bh.buddy_hip_variant_reset()
+    for i, N in enumerate(GEMV_I8_N):
+        for epilogue in (0, 1, 2):
+            for norm in (False, True):
+                gemv_case(bh, oracle, 5 + 3 * i, 192, N, epilogue, norm, 100 + i)
+    fam = "gemv_w8a32_i8_kernel"
+    assert launched(bh, fam) == compiled(bh, fam), compiled(bh, fam) - launched(bh, fam)
+
+
+def test_every_bf16_batch_gemv_variant(bh, oracle):
+    bh.buddy_hip_variant_reset()
+    assert bh.buddy_hip_set_gemv_batch_kernel(1) == 0
+    try:
+        for i, N in enumerate(GEMV_BF16_N):
+            for epilogue in (0, 1, 2):
+                for norm in (False, True):
+                    gemv_case(bh, oracle, 6 + 5 * i, 128, N, epilogue, norm, 200 + i)
+    finally:
+        assert bh.buddy_hip_set_gemv_batch_kernel(0) == 0
+    fam = "gemv_w8a32_mfma_kernel"
+    assert launched(bh, fam) == compiled(bh, fam), compiled(bh, fam) - launched(bh, fam)
+
+
+# ---- prefill matmul: the tile shape comes out of the launch's cost model -------
+GEMM_I8_SHAPES = [(144, 256, 16384), (300, 256, 10240), (200, 192, 16384), (512, 192, 8960),
+                  (17, 64, 64)]
+GEMM_BF16_SHAPES = [(512, 64, 8960), (300, 64, 10240), (17, 64, 64)]
+
+
+def gemm_case(oracle, M, K, N, mode):
+    q, s = synthetic.quantized_linear(K, N, M + K + N)
+    g = torch.Generator(device="cuda").manual_seed(M)
+    x = torch.randn((M, K), generator=g, device="cuda")
+    y = ops.gemm_w8a32(x, ops.pack_w8(q), s, K, N, exact=mode == "exact", digits=mode == "digits")
+    torch.cuda.synchronize()
+    xh = x.cpu().numpy()
+    a_in = bf16_round(xh) if mode == "bf16" else xh
+    want = oracle.blis_gemm_w8a32(a_in, q.cpu().numpy(), s.cpu().numpy())
+    got = y.cpu().numpy()
+    for m in range(M):
+        check_close(got[m], want[m])
+
+
+def test_every_int8_prefill_matmul_variant(bh, oracle):
+    bh.buddy_hip_variant_reset()
+    for M, K, N in GEMM_I8_SHAPES:
+        gemm_case(oracle, M, K, N, "digits")
+    for fam in ("gemm_w8_i8_wide_kernel", "gemm_w8_i8_kernel"):
+        assert launched(bh, fam) == compiled(bh, fam), compiled(bh, fam) - launched(bh, fam)
+
+
+def test_every_bf16_prefill_matmul_variant(bh, oracle):
+    bh.buddy_hip_variant_reset()
+    for M, K, N in GEMM_BF16_SHAPES:
+        for mode in ("bf16", "exact"):
+            gemm_case(oracle, M, K, N, mode)
+    for fam in ("gemm_w8_bf16_wide_kernel", "gemm_w8_bf16_kernel"):
+        assert launched(bh, fam) == compiled(bh, fam), compiled(bh, fam) - launched(bh, fam)
+
+
+def test_prefill_attention_and_no_unlisted_family(bh, oracle):
+    bh.buddy_hip_variant_reset()
+    heads, kv_heads, L, D = 4, 2, 40, 128
+    g = torch.Generator(device="cuda").manual_seed(3)
+    q = torch.randn((heads, L, D), generator=g, device="cuda")
+    k = torch.randn((kv_heads, L, D), generator=g, device="cuda")
+    v = torch.randn((kv_heads, L, D), generator=g, device="cuda")
+    got = run_attn(bh, q, k, v, None, heads, kv_heads, L, L)
+    rep = heads // kv_heads
+    kk = np.repeat(k.cpu().numpy(), rep, axis=0)
+    vv = np.repeat(v.cpu().numpy(), rep, axis=0)
+    mask = np.triu(np.full((L, L), -np.inf, np.float32), 1)
+    want = oracle.prefill_flash_attention(q.cpu().numpy(), kk, vv, mask, SCALE)
+    check_close(got, want)
+    assert launched(bh, "attn_prefill_kernel") == compiled(bh, "attn_prefill_kernel")
+    # every family the library lists is one of those this file drives
+    known = ("gemv_w8a32_i8_kernel", "gemv_w8a32_mfma_kernel", "gemm_w8_i8_wide_kernel",
+             "gemm_w8_i8_kernel", "gemm_w8_bf16_wide_kernel", "gemm_w8_bf16_kernel",
+             "attn_prefill_kernel")
+    assert {name.split("<")[0] for name in report(bh)} == set(known)
