@@ -33,6 +33,9 @@
 //     row's rsqrt factor multiplies the finished sums.
 #include "gemv_w8a32.h"
 
+#include <cstdio>
+#include <cstdlib>
+
 namespace bh {
 namespace {
 
@@ -226,6 +229,33 @@ __global__ void __launch_bounds__(kMaxWavesI8 *kWave, 3) // 3 wavefronts per SIM
   float *xt = red + (size_t)wave * kTurnFloats;
   float *meet = red + (size_t)(a.GS * a.KS) * kTurnFloats;
 
+  // Per-channel operands of the epilogue, requested before the stream starts so
+  // that their latency hides behind it (they are older than every fetch, so the
+  // counted waits cover them).
+  // With four groups per wavefront the registers are worth more than the
+  // latency, and they are loaded after the stream.
+  constexpr bool EARLY = SPAN <= 2;
+  const bool writer = live && ks == 0 && m < a.rows;
+  float e_s0[SPAN][4], e_s1[SPAN][4], e_c[SPAN][4];
+  auto load_epilogue = [&]() {
+#pragma unroll
+    for (int s = 0; s < SPAN; ++s)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int n = (g0 + s) * kTileN + kg * 4 + i;
+        const bool in = writer && g0 + s < a.groups && n < a.N;
+        e_s0[s][i] = in ? a.s0[n] : 0.f;
+        e_s1[s][i] = (DUAL && in) ? a.s1[n] : 0.f;
+        e_c[s][i] = 0.f;
+        if (in && EPI == kEpiAccum)
+          e_c[s][i] = a.C[(int64_t)m * a.ldc + n];
+        if (in && EPI == kEpiStore && a.bias)
+          e_c[s][i] = a.bias[n];
+      }
+  };
+  if (EARLY)
+    load_epilogue();
+
   constexpr int L = fetch_loads<SPAN, DUAL, NORM>();
   constexpr int R = ring_depth<SPAN, DUAL, NORM>(); // fetches in flight
   FetchRegs<SPAN, DUAL, NORM> ring[R];
@@ -322,6 +352,21 @@ __global__ void __launch_bounds__(kMaxWavesI8 *kWave, 3) // 3 wavefronts per SIM
 #pragma unroll
   for (int u = 0; u < R; ++u)
     wait_fetch<0, SPAN, DUAL, NORM>(ring[u]);
+  if (EARLY) {
+    // nothing that depends on the epilogue operands moves above this point
+#pragma unroll
+    for (int s = 0; s < SPAN; ++s)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        asm volatile("" : "+v"(e_s0[s][i]));
+        if (DUAL)
+          asm volatile("" : "+v"(e_s1[s][i]));
+        else
+          asm volatile("" : "+v"(e_c[s][i]));
+      }
+  } else {
+    load_epilogue();
+  }
   if (NORM) { // the four lanes that share a row hold different k
     ss += __shfl_xor(ss, 16, 64);
     ss += __shfl_xor(ss, 32, 64);
@@ -344,30 +389,50 @@ __global__ void __launch_bounds__(kMaxWavesI8 *kWave, 3) // 3 wavefronts per SIM
     __syncthreads();
     if (ks != 0)
       return;
+    // four slices at a time, all their reads in flight together (KS is a power
+    // of two; with two slices the reads past them repeat the last and are dropped)
+    float r[NA][4], rs = 0.f;
+#pragma unroll
+    for (int t = 0; t < NA; ++t)
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        r[t][i] = 0.f;
+    for (int q0 = 0; q0 < a.KS; q0 += 4) {
+      float v[4][NA][4], vs[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const float *o = meet + (size_t)(wave + min(q0 + j, a.KS - 1)) * kPerWave + lane;
+#pragma unroll
+        for (int t = 0; t < NA; ++t)
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            v[j][t][i] = o[(t * 4 + i) * kWave];
+        vs[j] = NORM ? o[NA * 4 * kWave] : 0.f;
+      }
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const bool has = q0 + j < a.KS;
+#pragma unroll
+        for (int t = 0; t < NA; ++t)
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            r[t][i] += has ? v[j][t][i] : 0.f;
+        rs += has ? vs[j] : 0.f;
+      }
+    }
 #pragma unroll
     for (int s = 0; s < SPAN; ++s)
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        float r0 = 0.f, r1 = 0.f;
-        for (int q = 0; q < a.KS; ++q) {
-          const float *o = meet + (size_t)(wave + q) * kPerWave;
-          r0 += o[(s * 4 + i) * kWave + lane];
-          if (DUAL)
-            r1 += o[((SPAN + s) * 4 + i) * kWave + lane];
-        }
-        acc0[s][i] = r0;
+        acc0[s][i] = r[s][i];
         if (DUAL)
-          acc1[DUAL ? s : 0][i] = r1;
+          acc1[DUAL ? s : 0][i] = r[DUAL ? SPAN + s : 0][i];
       }
-    if (NORM) {
-      float r = 0.f;
-      for (int q = 0; q < a.KS; ++q)
-        r += meet[(size_t)(wave + q) * kPerWave + NA * 4 * kWave + lane];
-      ss = r;
-    }
+    if (NORM)
+      ss = rs;
   }
   // lane holds batch row m and channels kg*4 .. kg*4+3 of each group
-  if (!live || m >= a.rows)
+  if (!writer)
     return;
   const float rn = NORM ? 1.0f / sqrtf(ss * a.norm_inv_k + a.norm_eps) : 1.0f;
 #pragma unroll
@@ -380,13 +445,11 @@ __global__ void __launch_bounds__(kMaxWavesI8 *kWave, 3) // 3 wavefronts per SIM
       const int n = g * kTileN + kg * 4 + i;
       if (n < a.N) {
         float *c = a.C + (int64_t)m * a.ldc + n;
-        const float v = acc0[s][i] * rn * a.s0[n];
+        const float v = acc0[s][i] * rn * e_s0[s][i];
         if (EPI == kEpiSiluMul)
-          *c = silu(v) * (acc1[DUAL ? s : 0][i] * rn * a.s1[n]);
-        else if (EPI == kEpiAccum)
-          *c = *c + v;
-        else
-          *c = a.bias ? a.bias[n] + v : v;
+          *c = silu(v) * (acc1[DUAL ? s : 0][i] * rn * e_s1[s][i]);
+        else // the residual row (accumulate) or the bias (or 0)
+          *c = e_c[s][i] + v;
       }
     }
   }
@@ -394,12 +457,26 @@ __global__ void __launch_bounds__(kMaxWavesI8 *kWave, 3) // 3 wavefronts per SIM
 
 BH_VARIANT_FAMILY(I8Family, "gemv_w8a32_i8_kernel");
 
+// Workgroups of `waves` wavefronts of this variant that one compute unit holds
+// (asked of the runtime once per variant and size: it knows the registers the
+// compiler used).
+template <int EPI, int SPAN, bool NORM> int workgroups_per_cu(int waves, size_t lds) {
+  static int cached[kMaxWavesI8 + 1] = {};
+  if (!cached[waves]) {
+    int n = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(
+            &n, reinterpret_cast<const void *>(gemv_w8a32_i8_kernel<EPI, SPAN, NORM>),
+            waves * kWave, lds) != hipSuccess ||
+        n < 1)
+      n = 1;
+    cached[waves] = n;
+  }
+  return cached[waves];
+}
+
 template <int EPI, int SPAN, bool NORM>
-int launch_kernel(const I8Args &ka, int blocks, hipStream_t stream) {
+int launch_kernel(I8Args ka, int ks_forced, hipStream_t stream) {
   constexpr int NA = (EPI == kEpiSiluMul) ? 2 * SPAN : SPAN;
-  const int waves = ka.GS * ka.KS;
-  const size_t lds = sizeof(float) * waves *
-                     ((size_t)kTurnFloats + (ka.KS > 1 ? (size_t)(NA * 4 + 1) * kWave : 0));
   auto kernel = gemv_w8a32_i8_kernel<EPI, SPAN, NORM>;
   static bool attr_set = false;
   if (!attr_set) {
@@ -408,27 +485,51 @@ int launch_kernel(const I8Args &ka, int blocks, hipStream_t stream) {
                                      144 * 1024));
     attr_set = true;
   }
+  auto lds_bytes = [&](int ks, int waves) {
+    return sizeof(float) * waves *
+           ((size_t)kTurnFloats + (ks > 1 ? (size_t)(NA * 4 + 1) * kWave : 0));
+  };
+  // k-slices per workgroup: as many as give every wavefront two chunks at least
+  // and still let every workgroup of the launch run at once (the chip has 256
+  // compute units) -- a second round of workgroups costs far more than longer
+  // slices do (1536 -> 2 x 8960 at 16 rows: 16.2 us with 280 workgroups of 8
+  // wavefronts, of which 256 fit, 12.8 us with 280 of 4)
+  int ks = kMaxWavesI8;
+  for (; ks > 1; ks /= 2) {
+    if (ka.chunks / ks < 2)
+      continue;
+    const int gs = ks < 4 ? 4 / ks : 1, waves = gs * ks;
+    const int64_t blocks = ceil_div(ka.spans, gs);
+    if (blocks <= 256 * (int64_t)workgroups_per_cu<EPI, SPAN, NORM>(waves, lds_bytes(ks, waves)))
+      break;
+  }
+  if (ks_forced)
+    ks = ks_forced;
+  ka.KS = ks;
+  ka.GS = ks < 4 ? 4 / ks : 1;
+  const int waves = ka.GS * ka.KS;
+  const int blocks = (int)ceil_div(ka.spans, ka.GS);
   BH_NOTE_VARIANT(I8Family, EPI, SPAN, NORM);
-  hipLaunchKernelGGL(kernel, dim3(blocks), dim3(waves * kWave), lds, stream, ka);
+  hipLaunchKernelGGL(kernel, dim3(blocks), dim3(waves * kWave), lds_bytes(ks, waves), stream, ka);
   BH_CHECK_HIP(hipGetLastError());
   return BUDDY_HIP_OK;
 }
 
 template <int EPI, int SPAN>
-int launch_norm(const I8Args &ka, int blocks, hipStream_t stream) {
-  return ka.norm_w ? launch_kernel<EPI, SPAN, true>(ka, blocks, stream)
-                   : launch_kernel<EPI, SPAN, false>(ka, blocks, stream);
+int launch_norm(const I8Args &ka, int ks_forced, hipStream_t stream) {
+  return ka.norm_w ? launch_kernel<EPI, SPAN, true>(ka, ks_forced, stream)
+                   : launch_kernel<EPI, SPAN, false>(ka, ks_forced, stream);
 }
 
 template <int SPAN>
-int launch_span(const I8Args &ka, int epilogue, int blocks, hipStream_t stream) {
+int launch_span(const I8Args &ka, int epilogue, int ks_forced, hipStream_t stream) {
   switch (epilogue) {
-  case kEpiStore: return launch_norm<kEpiStore, SPAN>(ka, blocks, stream);
-  case kEpiAccum: return launch_norm<kEpiAccum, SPAN>(ka, blocks, stream);
+  case kEpiStore: return launch_norm<kEpiStore, SPAN>(ka, ks_forced, stream);
+  case kEpiAccum: return launch_norm<kEpiAccum, SPAN>(ka, ks_forced, stream);
   case kEpiSiluMul:
     if (SPAN > 2)
       return fail(BUDDY_HIP_ERR_ARG, "gemv: SiLU*mul with %d groups per wavefront", SPAN);
-    return launch_norm<kEpiSiluMul, (SPAN > 2 ? 2 : SPAN)>(ka, blocks, stream);
+    return launch_norm<kEpiSiluMul, (SPAN > 2 ? 2 : SPAN)>(ka, ks_forced, stream);
   }
   return fail(BUDDY_HIP_ERR_ARG, "gemv: unknown epilogue %d", epilogue);
 }
@@ -465,21 +566,20 @@ int launch_gemv_i8(const GemvArgs &a, hipStream_t stream) {
   else if (ka.groups >= 2 * 256)
     span = 2;
   ka.spans = (int)ceil_div(ka.groups, span);
-  // k-slices: as many wavefronts as the chip holds at once at these kernels'
-  // register count (16 per compute unit; with the fused norm one workgroup of 8)
-  // and no more -- a second round of workgroups costs more than longer slices
-  // do --, at least two chunks each
-  const int64_t resident = a.norm_w ? 2048 : 4096;
-  int ks = 1;
-  while (ks < kMaxWavesI8 && (int64_t)ka.spans * ks * 2 <= resident && ka.chunks / (ks * 2) >= 2)
-    ks *= 2;
-  ka.KS = ks;
-  ka.GS = ks < 4 ? 4 / ks : 1;
-  const int blocks = (int)ceil_div(ka.spans, ka.GS);
+  int ks_forced = 0;
+  if (const char *e = getenv("BUDDY_HIP_I8_PLAN")) { // measurement only: "span,ks"
+    int s_ = 0, k_ = 0;
+    if (sscanf(e, "%d,%d", &s_, &k_) == 2 && (s_ == 1 || s_ == 2 || (s_ == 4 && !dual)) &&
+        (k_ == 1 || k_ == 2 || k_ == 4 || k_ == kMaxWavesI8)) {
+      span = s_;
+      ks_forced = k_;
+      ka.spans = (int)ceil_div(ka.groups, span);
+    }
+  }
   if (span == 4)
-    return launch_span<4>(ka, a.epilogue, blocks, stream);
-  return span == 2 ? launch_span<2>(ka, a.epilogue, blocks, stream)
-                   : launch_span<1>(ka, a.epilogue, blocks, stream);
+    return launch_span<4>(ka, a.epilogue, ks_forced, stream);
+  return span == 2 ? launch_span<2>(ka, a.epilogue, ks_forced, stream)
+                   : launch_span<1>(ka, a.epilogue, ks_forced, stream);
 }
 
 } // namespace bh
