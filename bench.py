@@ -75,7 +75,7 @@ def decode_step_bytes(shape, ctx: int) -> int:
     return w + scales + kv + norms + 4 * H + 4 * V
 
 
-def time_gate_up(bh, shape, sess_stream, layers, iters):
+def time_gate_up(bh, shape, sess_stream, layers, iters, use_graph=True):
     """Average duration of the dominant kernel (fused gate|up GEMV), launched
     back to back over `layers` distinct weight sets (more than the 256 MB
     last-level cache holds) from a replayed hipGraph, as the decode step
@@ -112,12 +112,18 @@ def time_gate_up(bh, shape, sess_stream, layers, iters):
         for i in range(iters):
             bh.buddy_hip_linear_w8a32(ctypes.byref(descs[i % layers]), sess_stream)
 
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    if not use_graph:  # plain stream launches (what a per-dispatch counter run needs)
+        e0.record(stream)
+        enqueue()
+        e1.record(stream)
+        e1.synchronize()
+        return e0.elapsed_time(e1) * 1e-3 / iters
     # the decode step launches this kernel from a replayed hipGraph: time it the
     # same way, `iters` launches per replay
     graph = torch.cuda.CUDAGraph()
     with torch.cuda.graph(graph, stream=stream):
         enqueue()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     with torch.cuda.stream(stream):
         graph.replay()
         stream.synchronize()
@@ -867,7 +873,7 @@ def main():
     step_s = max(dev_s, wall) / K  # the slower of the two clocks
 
     # dominant kernel, measured live on its launch stream
-    gu_s = time_gate_up(bh, shape, sess.stream, layers=16, iters=160)
+    gu_s = time_gate_up(bh, shape, sess.stream, layers=16, iters=160, use_graph=not args.no_graph)
     gu_b = gate_up_bytes(shape.hidden, shape.inter)
     achieved = gu_b / gu_s / 1e9
     step_b = decode_step_bytes(shape, CONTEXT + W + K // 2)

@@ -187,7 +187,7 @@ __global__ void __launch_bounds__(kThreads) attn_decode_partial(AttnArgs a) {
   float l_w = 0.f;
 #pragma unroll
   for (int i = 0; i < kR; ++i) {
-    sc[i] = expf(sc[i] - m_w); // -inf -> 0 beyond the position
+    sc[i] = fast_exp(sc[i] - m_w); // -inf -> 0 beyond the position
     l_w += sc[i];
   }
   l_w += __shfl_xor(l_w, 32, 64);
@@ -231,7 +231,7 @@ __global__ void __launch_bounds__(kThreads) attn_decode_partial(AttnArgs a) {
     float o = 0.f, l = 0.f;
 #pragma unroll
     for (int w = 0; w < kWaves; ++w) {
-      const float f = expf(mw_s[w] - m);
+      const float f = fast_exp(mw_s[w] - m);
       o = fmaf(accw_s[w][tid], f, o);
       l = fmaf(lw_s[w], f, l);
     }

@@ -112,6 +112,16 @@ inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 inline int64_t round_up(int64_t a, int64_t b) { return ceil_div(a, b) * b; }
 
 #if defined(__HIPCC__)
+// One-instruction transcendental forms (v_exp_f32, v_rcp_f32, v_rsq_f32: 1 ulp)
+// for the epilogues of the decode kernels, where a single wavefront finishes a
+// tile alone and the library routines' twenty-odd dependent instructions each
+// would sit on the critical path of the launch.
+__device__ __forceinline__ float fast_exp(float x) {
+  return __builtin_amdgcn_exp2f(x * 1.44269504088896341f);
+}
+__device__ __forceinline__ float fast_rcp(float x) { return __builtin_amdgcn_rcpf(x); }
+__device__ __forceinline__ float fast_rsqrt(float x) { return __builtin_amdgcn_rsqf(x); }
+
 // Cross-lane reductions on DPP (data-parallel primitives: a VALU operand read
 // from another lane of the same row of 16, a few cycles) instead of
 // ds_bpermute round trips through the LDS crossbar.

@@ -173,7 +173,7 @@ __device__ __forceinline__ void fma_tile(const int4 &w, const float *xl,
 __device__ __forceinline__ float silu(float g) {
   // (g * sigmoid(g)), sigmoid = 1/(1+exp(-g))
   // examples/BuddyDeepSeekR1/subgraph0_decode_simplify.mlir:225-227
-  const float sig = 1.0f / (1.0f + expf(-g));
+  const float sig = fast_rcp(1.0f + fast_exp(-g));
   return g * sig;
 }
 
@@ -232,7 +232,7 @@ __device__ __forceinline__ float4 attn_combined(const KernelArgs &a, int k) {
     for (int j = 0; j < B; ++j)
       if (s0 + j < used)
         mb = fmaxf(mb, mlv[j].x);
-    const float al = expf(m - mb); // rescale what was gathered so far
+    const float al = fast_exp(m - mb); // rescale what was gathered so far
     r.x *= al;
     r.y *= al;
     r.z *= al;
@@ -242,7 +242,7 @@ __device__ __forceinline__ float4 attn_combined(const KernelArgs &a, int k) {
 #pragma unroll
     for (int j = 0; j < B; ++j) {
       if (s0 + j < used) {
-        const float w = expf(mlv[j].x - m);
+        const float w = fast_exp(mlv[j].x - m);
         l = fmaf(mlv[j].y, w, l);
         r.x = fmaf(v[j].x, w, r.x);
         r.y = fmaf(v[j].y, w, r.y);
@@ -251,7 +251,7 @@ __device__ __forceinline__ float4 attn_combined(const KernelArgs &a, int k) {
       }
     }
   }
-  const float inv = 1.0f / l;
+  const float inv = fast_rcp(l);
   return make_float4(r.x * inv, r.y * inv, r.z * inv, r.w * inv);
 }
 
@@ -467,7 +467,7 @@ __global__ void __launch_bounds__(kMaxWaves *kWave)
           // x' = w (.) (x * r) with r = rsqrt(mean(x^2) + eps): r is common to
           // the whole row, so it multiplies the finished sum
           // (subgraph0_decode_simplify.mlir:60-72)
-          const float r = 1.0f / sqrtf(ss[m] * a.norm_inv_k + a.norm_eps);
+          const float r = fast_rsqrt(ss[m] * a.norm_inv_k + a.norm_eps);
           v0 *= r;
           v1 *= r;
         }
@@ -617,7 +617,7 @@ __device__ __forceinline__ void attn_fold_tiles(const KernelArgs &a, int t0, int
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const float mb = wave_max(valid ? mine[u].x : -1.0e30f);
-      const float w = valid ? expf(mine[u].x - mb) : 0.f;
+      const float w = valid ? fast_exp(mine[u].x - mb) : 0.f;
       l[u] = wave_sum(mine[u].y * w);
 #pragma unroll
       for (int j = 0; j < B; ++j)
@@ -632,8 +632,8 @@ __device__ __forceinline__ void attn_fold_tiles(const KernelArgs &a, int t0, int
       const float2 mine = ml[u][c0 + min(lane, cnt - 1)];
       const bool valid = lane < cnt;
       const float mb = fmaxf(m[u], wave_max(valid ? mine.x : -1.0e30f));
-      const float al = expf(m[u] - mb); // rescale what earlier passes gathered
-      w[u] = valid ? expf(mine.x - mb) : 0.f;
+      const float al = fast_exp(m[u] - mb); // rescale what earlier passes gathered
+      w[u] = valid ? fast_exp(mine.x - mb) : 0.f;
       l[u] = fmaf(l[u], al, wave_sum(mine.y * w[u]));
       r[u] *= al;
       m[u] = mb;
@@ -656,7 +656,7 @@ __device__ __forceinline__ void attn_fold_tiles(const KernelArgs &a, int t0, int
   } // longer caches
 #pragma unroll
   for (int u = 0; u < U; ++u)
-    x[u] = r[u] * (1.0f / l[u]);
+    x[u] = r[u] * fast_rcp(l[u]);
 }
 
 // One tile's worth of operands of one wavefront.
@@ -900,7 +900,7 @@ __global__ void __launch_bounds__(kMaxWaves *kWave)
           // x' = w (.) (x * r) with r = rsqrt(mean(x^2) + eps): r is common to
           // the whole row, so it multiplies the finished sum
           // (subgraph0_decode_simplify.mlir:60-72)
-          const float r = 1.0f / sqrtf(ss[m] * a.norm_inv_k + a.norm_eps);
+          const float r = fast_rsqrt(ss[m] * a.norm_inv_k + a.norm_eps);
           v0 *= r;
           v1 *= r;
         }
