@@ -259,42 +259,56 @@ int main(int argc, char **argv) {
   CK(hipMalloc(&nw, sizeof(float) * 8960));
   CK(hipMemset(xin, 0, sizeof(float) * 8960));
   CK(hipMemset(nw, 0, sizeof(float) * 8960));
-  printf("\nfused launches of a decoder layer, same rotation\n");
+  // The small operands (activation row, norm weight, scales, output row) either
+  // stay where they are from launch to launch (they sit in every L2) or rotate
+  // through their own 512 MiB like the weights: in a decoder every layer has its
+  // own, read once per step.
+  const size_t small_bytes = (size_t)512 << 20;
+  char *small_pool;
+  CK(hipMalloc(&small_pool, small_bytes));
+  CK(hipMemset(small_pool, 0, small_bytes));
+  const size_t small_slot = (size_t)256 << 10; // 4 vectors of up to 64 KiB
   std::vector<std::pair<double, double>> fused_res;
-  for (const Fused &f : fused) {
-    const size_t bytes = (size_t)f.K * f.N;
-    const size_t per = bytes * (f.dual ? 2 : 1);
-    const size_t slots = pool_bytes / per;
-    const double us = time_chain([&](int i) {
-      buddy_hip_linear_desc d;
-      memset(&d, 0, sizeof d);
-      d.A = xin;
-      d.lda = f.K;
-      d.W0 = pool + (size_t)(i % slots) * per;
-      d.scale0 = scale;
-      if (f.dual) {
-        d.W1 = d.W0 + bytes;
-        d.scale1 = scale + f.N;
-      }
-      if (f.norm) {
-        d.norm_w = nw;
-        d.norm_eps = 1e-6f;
-      }
-      d.C = y;
-      d.ldc = f.N;
-      d.M = 1;
-      d.K = f.K;
-      d.N = f.N;
-      d.epilogue = f.epi;
-      if (buddy_hip_linear_w8a32(&d, g_stream)) {
-        fprintf(stderr, "gemv failed: %s\n", buddy_hip_last_error());
-        exit(1);
-      }
-    });
-    const double b = (double)per + 4.0 * (f.K * (f.norm ? 2 : 1) + f.N * (f.dual ? 3 : 2) +
-                                          (f.epi == BUDDY_HIP_EPI_ACCUM ? f.N : 0));
-    fused_res.push_back({b, us});
-    printf("  %-50s %8.2f MB %7.2f us %6.0f GB/s\n", f.name, b / 1e6, us, b / us / 1e3);
+  for (int cold = 0; cold < 2; ++cold) {
+    printf("\nfused launches of a decoder layer, same rotation of the weights; small operands %s\n",
+           cold ? "rotated too (cold)" : "in place (cache-warm)");
+    for (const Fused &f : fused) {
+      const size_t bytes = (size_t)f.K * f.N;
+      const size_t per = bytes * (f.dual ? 2 : 1);
+      const size_t slots = pool_bytes / per;
+      const double us = time_chain([&](int i) {
+        buddy_hip_linear_desc d;
+        memset(&d, 0, sizeof d);
+        float *sm = reinterpret_cast<float *>(
+            small_pool + ((size_t)i * 7919 % (small_bytes / small_slot)) * small_slot);
+        d.A = cold ? sm : xin;
+        d.lda = f.K;
+        d.W0 = pool + (size_t)(i % slots) * per;
+        d.scale0 = cold ? sm + 16384 : scale;
+        if (f.dual) {
+          d.W1 = d.W0 + bytes;
+          d.scale1 = d.scale0 + f.N;
+        }
+        if (f.norm) {
+          d.norm_w = cold ? sm + 49152 : nw;
+          d.norm_eps = 1e-6f;
+        }
+        d.C = cold ? sm + 32768 : y;
+        d.ldc = f.N;
+        d.M = 1;
+        d.K = f.K;
+        d.N = f.N;
+        d.epilogue = f.epi;
+        if (buddy_hip_linear_w8a32(&d, g_stream)) {
+          fprintf(stderr, "gemv failed: %s\n", buddy_hip_last_error());
+          exit(1);
+        }
+      });
+      const double b = (double)per + 4.0 * (f.K * (f.norm ? 2 : 1) + f.N * (f.dual ? 3 : 2) +
+                                            (f.epi == BUDDY_HIP_EPI_ACCUM ? f.N : 0));
+      fused_res.push_back({b, us});
+      printf("  %-50s %8.2f MB %7.2f us %6.0f GB/s\n", f.name, b / 1e6, us, b / us / 1e3);
+    }
   }
 
   // least squares  us = a + bytes / b
