@@ -27,9 +27,12 @@ sys.path.insert(0, str(ROOT / "tests"))
 # The CPU baseline runs OpenMP loops: pin its threads to neighbouring cores like
 # the reference's own runs do (docs/Runtime.md:192 leaves the thread count to
 # OMP_NUM_THREADS).  Must be in the environment before any OpenMP runtime loads.
+# Only when the baseline will run: the binding also pins the process's first
+# thread, and every helper thread a profiler starts inherits that.
 OMP_BINDING = {"OMP_PROC_BIND": "close", "OMP_PLACES": "cores"}
-for _k, _v in OMP_BINDING.items():
-    os.environ.setdefault(_k, _v)
+if "--no-cpu-baseline" not in sys.argv:
+    for _k, _v in OMP_BINDING.items():
+        os.environ.setdefault(_k, _v)
 
 HBM_PEAK_GBPS = 8000.0  # MI355X published HBM3E bandwidth
 CONTEXT = 1024
