@@ -156,6 +156,30 @@ __device__ __forceinline__ float wave_max(float v) {
   v = row16_max(v);
   return fmaxf(fmaxf(lane_f(v, 0), lane_f(v, 16)), fmaxf(lane_f(v, 32), lane_f(v, 48)));
 }
+// v of this lane and v of lane ^ 32 (W = 32) or lane ^ 16 (W = 16), in an order
+// that depends on the lane: for commutative merges.  One VALU instruction
+// (v_permlane32_swap / v_permlane16_swap) instead of a trip through the LDS
+// crossbar (ds_bpermute).
+template <int W> __device__ __forceinline__ void lane_pair(float v, float &a, float &b) {
+  static_assert(W == 16 || W == 32, "rows (16) or halves (32) of a wavefront");
+  const unsigned u = __float_as_uint(v);
+  if constexpr (W == 32) {
+    const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    a = __uint_as_float(r[0]);
+    b = __uint_as_float(r[1]);
+  } else {
+    const auto r = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+    a = __uint_as_float(r[0]);
+    b = __uint_as_float(r[1]);
+  }
+}
+template <int W> __device__ __forceinline__ float sum_xor(float v) {
+  float a, b;
+  lane_pair<W>(v, a, b);
+  return a + b;
+}
+// every lane gets the sum over the lanes l, l ^ 16, l ^ 32, l ^ 48
+__device__ __forceinline__ float sum_rows(float v) { return sum_xor<32>(sum_xor<16>(v)); }
 // sum over the 4 lanes of a quad / the 8 lanes of two adjacent quads
 __device__ __forceinline__ float quad_sum(float v) {
   v += dpp_f<0xB1>(v);

@@ -15,22 +15,28 @@
 //    wavefronts streaming.  The k-slices meet in LDS, in slice order, so the
 //    sum is deterministic and no workgroup ever waits for another one (cross-
 //    XCD traffic inside a kernel costs an L2 write-back on this part);
-//  * activations never pass through LDS: a lane loads the one activation whose
-//    k equals its position in the tile and the multiply-add reads its
-//    neighbours' values through DPP row broadcasts (gemv_w8a32_bcast_kernel).
-//    RMSNorm is fused in (weight multiplied while consuming, the row's sum of
+//  * one row (gemv_w8a32_dot4_kernel): a wavefront turns the activations of its
+//    run of tiles into three int8 digit planes of a 23-bit fixed-point value,
+//    leaves them in a private corner of LDS and multiplies four weights per
+//    instruction (v_dot4_i32_i8) into exact int32 sums;
+//  * two to four rows, and runs too long for one batch of loads
+//    (gemv_w8a32_bcast_kernel): activations never pass through LDS, a lane
+//    loads the one activation whose k equals its position in the tile and the
+//    f32 multiply-add reads its neighbours' values through DPP row broadcasts;
+//  * RMSNorm is fused in (weight multiplied while consuming, the row's sum of
 //    squares gathered on the way, the common rsqrt factor applied to the
 //    finished sums), as is folding the attention partials (o_proj);
 //  * scale, bias, residual add and SiLU*up are applied to the finished sums in
 //    the same kernel; their operands are requested before the stream starts.
 // The 8- and 4-channel tile layouts keep the older kernel that stages the
 // activations in LDS (gemv_w8a32_kernel).
-// No MFMA: at M = 1 the arithmetic is far below the bandwidth ridge.
+// No MFMA: with one row 15 of a matrix instruction's 16 columns would be empty.
 #include "gemv_w8a32.h"
 
 #include <atomic>
 #include <cstdlib>
 #include <cstring>
+#include <utility>
 
 namespace bh {
 namespace {
@@ -700,16 +706,13 @@ __device__ __forceinline__ void fetch_tile(const KernelArgs &a, const int4 *w0,
   }
 }
 
-// ONE: every wavefront's run of tiles fits in U, so all its loads go out at
-// once and nothing is double-buffered.
-//
 // Everything a wavefront needs before it can request its tiles -- four
 // pointers and six integers, 14 argument words -- are separate leading
 // parameters: this file is built with -amdgpu-kernarg-preload-count=14, so the
 // command processor hands them to every wavefront in SGPRs and the first loads
 // do not wait for a scalar load of the argument block.  The remaining fields
 // travel in `rest` and are loaded as usual, behind the stream.
-template <int M, int EPI, int PRO, int U, bool ONE>
+template <int M, int EPI, int PRO, int U>
 __global__ void __launch_bounds__(kMaxWaves *kWave)
     gemv_w8a32_bcast_kernel(const int4 *pW0, const int4 *pW1, const float *pA,
                             const float *pnorm_w, int p_chunks, int p_KS, int p_G,
@@ -799,7 +802,7 @@ __global__ void __launch_bounds__(kMaxWaves *kWave)
   }
 
   BH_TL(g_tl_gemv, tl_wave, 1);
-  for (int t = t0; t < (ONE ? min(t1, t0 + 1) : t1); t += U) {
+  for (int t = t0; t < t1; t += U) {
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       if (t + u < t1) {
@@ -831,7 +834,7 @@ __global__ void __launch_bounds__(kMaxWaves *kWave)
               fma16_row_bcast(acc1[m], x, wf1);
           }
         }
-        if (!ONE && t + U + u < t1)
+        if (t + U + u < t1)
           fetch_tile<M, PRO, DUAL>(a, w0, w1, t + U + u, lane, slot[u]);
         if (u == 0 && t == t0)
           BH_TL(g_tl_gemv, tl_wave, 2);
@@ -843,12 +846,9 @@ __global__ void __launch_bounds__(kMaxWaves *kWave)
   // the four rows of a wavefront hold different k sub-ranges of the same channels
 #pragma unroll
   for (int m = 0; m < M; ++m) {
-    acc0[m] += __shfl_xor(acc0[m], 16, 64);
-    acc0[m] += __shfl_xor(acc0[m], 32, 64);
-    if (DUAL) {
-      acc1[m] += __shfl_xor(acc1[m], 16, 64);
-      acc1[m] += __shfl_xor(acc1[m], 32, 64);
-    }
+    acc0[m] = sum_rows(acc0[m]);
+    if (DUAL)
+      acc1[m] = sum_rows(acc1[m]);
     if (NORM)
       ss[m] = wave_sum(ss[m]);
   }
@@ -911,9 +911,287 @@ __global__ void __launch_bounds__(kMaxWaves *kWave)
   BH_TL(g_tl_gemv, tl_wave, 5);
 }
 
-template <int M, int EPI, int PRO, int U, bool ONE>
+// ---------------------------------------------------------------------------
+// One row on the integer dot product (v_dot4_i32_i8), 0.75 instructions per
+// weight instead of two.
+//
+// A wavefront turns the activations of its own run of tiles into fixed point,
+// X = rint(x / s) with s the smallest power of two that keeps |X| < 2^22 over
+// the run, cuts X into three balanced int8 digits (X = d0 + 256 d1 + 65536 d2)
+// and leaves each digit plane in its own corner of LDS in k order.  A lane then
+// reads the 16 digits that go with its 16 weights as one 128-bit word per plane
+// (the 16 lanes of a row read the same word: a broadcast) and multiplies four
+// weights at a time.  The int32 sums are exact; the only rounding is that of X,
+// 2^-23 of the largest activation of the run.  Nothing waits for another
+// wavefront before the stream: the planes are private to the wavefront that
+// wrote them.
+// ---------------------------------------------------------------------------
+__device__ __forceinline__ unsigned wave_max_u32(unsigned v) {
+  auto dpp = [](unsigned x, auto ctrl) {
+    return (unsigned)__builtin_amdgcn_update_dpp(0, (int)x, decltype(ctrl)::value, 0xf, 0xf,
+                                                 true);
+  };
+  v = max(v, dpp(v, std::integral_constant<int, 0xB1>{}));
+  v = max(v, dpp(v, std::integral_constant<int, 0x4E>{}));
+  v = max(v, dpp(v, std::integral_constant<int, 0x141>{}));
+  v = max(v, dpp(v, std::integral_constant<int, 0x140>{}));
+  const unsigned a = __builtin_amdgcn_readlane((int)v, 0), b = __builtin_amdgcn_readlane((int)v, 16);
+  const unsigned c = __builtin_amdgcn_readlane((int)v, 32), d = __builtin_amdgcn_readlane((int)v, 48);
+  return max(max(a, b), max(c, d));
+}
+
+constexpr int kDigitBytesPerTile = 3 * kTileK; // three planes of 64 digits
+
+//
+// HS (a channel group split over two workgroups): a load instruction covers the
+// workgroup's 8 channels of two consecutive tiles -- the lanes that would hold
+// the other workgroup's channels take the second tile instead -- so it moves
+// 1 KiB of weights that nobody else reads, in whole 128-byte lines.
+template <int EPI, int PRO, int U, bool HS>
+__global__ void __launch_bounds__(kMaxWaves *kWave)
+    gemv_w8a32_dot4_kernel(const int4 *pW0, const int4 *pW1, const float *pA,
+                           const float *pnorm_w, int p_chunks, int p_KS, int p_G,
+                           int p_groups, int p_K, int p_rows, KernelArgs rest) {
+  KernelArgs a = rest;
+  a.W0 = pW0;
+  a.W1 = pW1;
+  a.A = pA;
+  a.norm_w = pnorm_w;
+  a.chunks = p_chunks;
+  a.KS = p_KS;
+  a.G = p_G & 0xffff;
+  const int hs = p_G >> 16; // 1: this workgroup takes 8 of its group's 16 channels
+  a.groups = p_groups;
+  a.K = p_K;
+  a.rows = p_rows;
+  constexpr bool DUAL = (EPI == kEpiSiluMul);
+  constexpr bool NORM = (PRO == kProNorm);
+  extern __shared__ float lds[];
+  const int tid = threadIdx.x;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+  const int nwaves = a.G * a.KS;
+  const int gl = wave / a.KS, ks = wave % a.KS;
+  const int gi = blockIdx.x * a.G + gl;
+  const int g = gi >> hs, half = gi & hs;
+  const bool live = g < a.groups;
+  const int per = (a.chunks + a.KS - 1) / a.KS;
+  const int t0 = min(ks * per, a.chunks);
+  const int t1 = min(t0 + per, a.chunks);
+
+  // ---- activations first: their use must not wait for the weights ----------
+  float x[U], nw[U];
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    const int k = (t0 + u) * kTileK + lane;
+    const int kc = min(k, a.K - 1);
+    x[u] = 0.f;
+    nw[u] = 0.f;
+    if (PRO != kProAttn)
+      x[u] = a.A[kc];
+    if (NORM)
+      nw[u] = a.norm_w[kc];
+  }
+  static_assert(!HS || (!DUAL && U % 2 == 0), "split groups: one matrix, tiles in pairs");
+  constexpr int P = HS ? U / 2 : U; // weight loads per matrix
+  const int wlane = HS ? ((lane & ~8) | (half << 3)) : lane;
+  const int second = HS ? (((lane >> 3) & 1) ^ half) : 0; // this lane takes the pair's second tile
+  const size_t wbase = ((size_t)(live ? g : 0) * a.chunks) * 64 + wlane;
+  const int4 *w0 = a.W0 + wbase;
+  const int4 *w1 = DUAL ? a.W1 + wbase : a.W0 + wbase;
+  int4 wa[P], wb[P];
+#pragma unroll
+  for (int u = 0; u < P; ++u) {
+    // Every load is issued whatever the run's length, so that the wait for the
+    // activations can name the exact number of weight loads behind them.  A
+    // slot past the run repeats the run's last tile (lines this wavefront has
+    // just asked for) and meets zero digits (the second tile of a last pair) or
+    // is not used; the slot counts are dense so that few runs have such a slot.
+    const int t = min(t0 + (HS ? 2 * u + second : u), max(t1 - 1, 0));
+    wa[u] = load_stream(w0 + (size_t)t * 64);
+    if (DUAL)
+      wb[u] = load_stream(w1 + (size_t)t * 64);
+  }
+  if (PRO == kProAttn && t0 < t1) {
+    constexpr int FB = U < 4 ? U : 4;
+    float xf[(U + FB - 1) / FB][FB];
+#pragma unroll
+    for (int q = 0; q < (U + FB - 1) / FB; ++q)
+      if (t0 + FB * q < t1)
+        attn_fold_tiles<FB>(a, t0 + FB * q, t1, lane, xf[q]);
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+      x[u] = xf[u / FB][u % FB];
+  }
+
+  const int n = g * kTileN + lane;
+  const bool writer = ks == 0 && lane < kTileN && live && n < a.N &&
+                      (!hs || (lane >> 3) == half);
+  EpilogueOperands<1> epi;
+  if (writer) {
+    epi.s0 = a.s0[n];
+    if (DUAL)
+      epi.s1 = a.s1[n];
+    if (EPI == kEpiStore && a.bias)
+      epi.bias = a.bias[n];
+    if (EPI == kEpiAccum)
+      epi.c[0] = a.C[n];
+  }
+
+  // ---- this wavefront's activations -> digit planes in LDS -----------------
+  unsigned char *planes =
+      reinterpret_cast<unsigned char *>(lds + (size_t)nwaves * 33) +
+      (size_t)wave * (U * kDigitBytesPerTile);
+  float ss = 0.f;
+  unsigned mb = 0;
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    const bool in = t0 + u < t1 && (t0 + u) * kTileK + lane < a.K;
+    float v = in ? x[u] : 0.f;
+    if (NORM) {
+      ss = fmaf(v, v, ss);
+      v *= nw[u];
+    }
+    x[u] = v;
+    mb = max(mb, __float_as_uint(v) & 0x7fffffffu);
+  }
+  mb = wave_max_u32(mb); // a NaN or infinity is the largest pattern
+  const int ex = (int)(mb >> 23) - 127; // floor(log2 max), -127 for zero and subnormals
+  const int e2 = max(ex + 1 - 22, -126);
+  const bool finite = mb < 0x7f800000u;
+  const float step = finite ? __uint_as_float((unsigned)(e2 + 127) << 23)
+                            : __uint_as_float(0x7fc00000u);
+  const float inv = __uint_as_float((unsigned)(127 - e2) << 23);
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    // x * inv + 1.5 * 2^23 is rounded to an integer by the addition itself and
+    // leaves 0x4B400000 + X in the word; adding 0x8080 makes the low two bytes
+    // the balanced digits with their sign bits flipped
+    constexpr float kMagic = 12582912.0f;
+    constexpr int kBias = 0x8080 - 0x4B400000;
+    const unsigned z =
+        (unsigned)(__float_as_int(fmaf(x[u], inv, kMagic)) + kBias) ^ 0x8080u;
+    unsigned char *p = planes + u * kDigitBytesPerTile + lane;
+    p[0] = (unsigned char)z;
+    p[kTileK] = (unsigned char)(z >> 8);
+    p[2 * kTileK] = (unsigned char)(z >> 16);
+  }
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+
+  int s0[3] = {0, 0, 0}, s1[3] = {0, 0, 0};
+  const unsigned char *mine_d = planes + 16 * (lane >> 4) + second * kDigitBytesPerTile;
+#pragma unroll
+  for (int u = 0; u < P; ++u) {
+    if (t0 + (HS ? 2 : 1) * u < t1) {
+#pragma unroll
+      for (int d = 0; d < 3; ++d) {
+        const int4 xd = *reinterpret_cast<const int4 *>(
+            mine_d + (HS ? 2 : 1) * u * kDigitBytesPerTile + d * kTileK);
+        s0[d] = __builtin_amdgcn_sdot4(wa[u].x, xd.x, s0[d], false);
+        s0[d] = __builtin_amdgcn_sdot4(wa[u].y, xd.y, s0[d], false);
+        s0[d] = __builtin_amdgcn_sdot4(wa[u].z, xd.z, s0[d], false);
+        s0[d] = __builtin_amdgcn_sdot4(wa[u].w, xd.w, s0[d], false);
+        if (DUAL) {
+          s1[d] = __builtin_amdgcn_sdot4(wb[u].x, xd.x, s1[d], false);
+          s1[d] = __builtin_amdgcn_sdot4(wb[u].y, xd.y, s1[d], false);
+          s1[d] = __builtin_amdgcn_sdot4(wb[u].z, xd.z, s1[d], false);
+          s1[d] = __builtin_amdgcn_sdot4(wb[u].w, xd.w, s1[d], false);
+        }
+      }
+    }
+  }
+  // |s0[0]|, |s0[1]| < 2^22 per lane (at most 10 x 16 products of 2^14): exact
+  const float step65536 = step * 65536.0f;
+  float acc0 = fmaf((float)s0[2], step65536, (float)(s0[0] + (s0[1] << 8)) * step);
+  float acc1 = DUAL ? fmaf((float)s1[2], step65536, (float)(s1[0] + (s1[1] << 8)) * step) : 0.f;
+
+  // the four rows of a wavefront hold different k sub-ranges of the same channels
+  // (and so do the two halves of a row when tiles go in pairs)
+  if (HS)
+    acc0 += dpp_f<0x128>(acc0); // row_ror:8, lane ^ 8
+  acc0 = sum_rows(acc0);
+  if (DUAL)
+    acc1 = sum_rows(acc1);
+  if (NORM)
+    ss = wave_sum(ss);
+
+  // ---- k-slices of one channel group meet in LDS, in slice order ----------
+  if (a.KS > 1) {
+    float *mine = lds + (size_t)wave * 33;
+    if (lane < kTileN) {
+      mine[lane] = acc0;
+      if (DUAL)
+        mine[16 + lane] = acc1;
+    }
+    if (NORM && lane == 0)
+      mine[32] = ss;
+    __syncthreads();
+    if (ks != 0)
+      return;
+    if (lane < kTileN) {
+      float r0 = 0.f, r1 = 0.f, rs = 0.f;
+      for (int s = 0; s < a.KS; ++s) {
+        const float *o = lds + (size_t)(wave + s) * 33;
+        r0 += o[lane];
+        if (DUAL)
+          r1 += o[16 + lane];
+        if (NORM)
+          rs += o[32];
+      }
+      acc0 = r0;
+      acc1 = r1;
+      ss = rs;
+    }
+  }
+  if (writer) {
+    if (NORM) {
+      const float r = fast_rsqrt(ss * a.norm_inv_k + a.norm_eps);
+      acc0 *= r;
+      acc1 *= r;
+    }
+    finish<1, EPI>(a, 0, n, acc0, acc1, epi);
+  }
+}
+
+BH_VARIANT_FAMILY(RowDot4Family, "gemv_w8a32_dot4_kernel");
+
+template <int EPI, int PRO, int U, bool HS = false>
+int launch_dot4(const KernelArgs &ka, const GemvPlan &p, hipStream_t stream) {
+  BH_NOTE_VARIANT(RowDot4Family, EPI, PRO, U, HS ? 1 : 0);
+  auto kernel = gemv_w8a32_dot4_kernel<EPI, PRO, U, HS>;
+  const size_t lds = sizeof(float) * p.waves * 33 + (size_t)p.waves * U * kDigitBytesPerTile;
+  hipLaunchKernelGGL(kernel, dim3(p.blocks << p.half_split), dim3(p.waves * kWave), lds,
+                     stream, ka.W0, ka.W1, ka.A, ka.norm_w, ka.chunks, ka.KS,
+                     ka.G | (p.half_split << 16), ka.groups, ka.K, ka.rows, ka);
+  BH_CHECK_HIP(hipGetLastError());
+  return BUDDY_HIP_OK;
+}
+
+constexpr int kNoFit = -1000; // no compiled slot count holds the run
+
+// the smallest compiled slot count that holds `tpw` tiles per wavefront
+template <int EPI, int PRO, bool HS, int... Us>
+int launch_dot4_fit(std::integer_sequence<int, Us...>, int64_t tpw, const KernelArgs &ka,
+                    const GemvPlan &p, hipStream_t stream) {
+  int rc = kNoFit;
+  bool done = false;
+  ((done || tpw > Us ? 0 : (done = true, rc = launch_dot4<EPI, PRO, Us, HS>(ka, p, stream))),
+   ...);
+  return rc;
+}
+
+bool row_dot4() {
+  static bool v = [] {
+    const char *e = getenv("BUDDY_HIP_GEMV_ROW");
+    return !(e && strcmp(e, "f32") == 0);
+  }();
+  return v;
+}
+
+template <int M, int EPI, int PRO, int U>
 int launch_bcast(const KernelArgs &ka, const GemvPlan &p, hipStream_t stream) {
-  auto kernel = gemv_w8a32_bcast_kernel<M, EPI, PRO, U, ONE>;
+  auto kernel = gemv_w8a32_bcast_kernel<M, EPI, PRO, U>;
   hipLaunchKernelGGL(kernel, dim3(p.blocks << p.half_split), dim3(p.waves * kWave),
                      sizeof(float) * p.waves * (size_t)M * 33, stream, ka.W0, ka.W1, ka.A,
                      ka.norm_w, ka.chunks, ka.KS, ka.G | (p.half_split << 16), ka.groups,
@@ -952,24 +1230,32 @@ int launch_one(const KernelArgs &ka, const GemvPlan &p, hipStream_t stream) {
       return launch_tn<kNarrowOk ? 1 : M, kNarrowOk ? EPI : kEpiStore, PRO, 4, kNarrowOk ? 8 : 16>(ka, p, stream);
     return launch_tn<kNarrowOk ? 1 : M, kNarrowOk ? EPI : kEpiStore, PRO, 4, kNarrowOk ? 4 : 16>(ka, p, stream);
   }
-  if (M == 1) {
-    // short runs: every tile of a wavefront is requested at once
+  if (M == 1 && row_dot4()) {
+    // short runs (every tile of a wavefront requested at once) go to the integer
+    // dot product; the slot counts are dense where a spare slot is a large part
+    // of the run
     const int64_t tpw = ceil_div(p.chunks, p.KS); // tiles per wavefront
-    if constexpr (PRO == kProAttn) {
-      if (tpw <= 2)
-        return launch_bcast<1, EPI, PRO, 2, true>(ka, p, stream);
-      if (tpw <= 3) // the o_proj of the 1.5B shape: no fourth slot to fold for nothing
-        return launch_bcast<1, EPI, PRO, 3, true>(ka, p, stream);
+    int rc = kNoFit;
+    if (p.half_split) {
+      if constexpr (!kDual && PRO != kProAttn)
+        rc = launch_dot4_fit<EPI, PRO, true>(std::integer_sequence<int, 4, 6, 8, 10>{}, tpw,
+                                             ka, p, stream);
+    } else if constexpr (PRO == kProAttn) { // the fold keeps 18 partials per tile in registers
+      rc = launch_dot4_fit<EPI, PRO, false>(std::integer_sequence<int, 2, 3, 4>{}, tpw, ka, p,
+                                            stream);
+    } else if constexpr (kDual) {
+      rc = launch_dot4_fit<EPI, PRO, false>(
+          std::integer_sequence<int, 2, 3, 4, 5, 6, 7, 8, 9>{}, tpw, ka, p, stream);
+    } else {
+      rc = launch_dot4_fit<EPI, PRO, false>(
+          std::integer_sequence<int, 2, 3, 4, 5, 6, 7, 8, 9, 10, 12, 14, 16>{}, tpw, ka, p,
+          stream);
     }
-    if (tpw <= 4)
-      return launch_bcast<1, EPI, PRO, 4, true>(ka, p, stream);
-    if (tpw <= 6)
-      return launch_bcast<1, EPI, PRO, 6, true>(ka, p, stream);
-    if (!kDual && tpw <= 9)
-      return launch_bcast<1, EPI, PRO, kDual ? 6 : 9, true>(ka, p, stream);
+    if (rc != kNoFit)
+      return rc;
   }
   constexpr int kRing = M == 1 ? (kDual ? 6 : 8) : M <= 4 ? 4 : M == 8 ? 2 : 1;
-  return launch_bcast<M, EPI, PRO, kRing, false>(ka, p, stream);
+  return launch_bcast<M, EPI, PRO, kRing>(ka, p, stream);
 }
 
 template <int M>

@@ -368,8 +368,7 @@ __global__ void __launch_bounds__(kMaxWavesI8 *kWave, 3) // 3 wavefronts per SIM
     load_epilogue();
   }
   if (NORM) { // the four lanes that share a row hold different k
-    ss += __shfl_xor(ss, 16, 64);
-    ss += __shfl_xor(ss, 32, 64);
+    ss = sum_rows(ss);
   }
 
   // ---- k-slices meet in LDS, in slice order --------------------------------

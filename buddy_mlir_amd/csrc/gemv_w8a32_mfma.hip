@@ -305,8 +305,7 @@ __global__ void __launch_bounds__(kMaxWavesMfma *kWave)
   for (int u = 0; u < R; ++u)
     wait_fetch<0, SPAN, DUAL, NORM>(ring[u]);
   if (NORM) { // the four lanes that share a row hold different k
-    ss += __shfl_xor(ss, 16, 64);
-    ss += __shfl_xor(ss, 32, 64);
+    ss = sum_rows(ss);
   }
 
   // ---- k-slices meet in LDS, in slice order --------------------------------

@@ -212,6 +212,61 @@ def test_gemv_bf16_batch_kernel_matches_oracle(oracle, bf16_batch_kernel, K, N, 
     check_close(y.cpu().numpy(), want)
 
 
+def test_row_kernel_fixed_point_keeps_f32_accuracy():
+    """One row goes through the integer dot product: every wavefront turns its
+    own run of the row (here 1536 / 8 = 192 values) into 23-bit fixed point with
+    a step of its own.  Rows of any magnitude, a loud run next to quiet ones and
+    a zero row each agree with a float64 sum to f32 accuracy; inside a run, a
+    value 2^-23 of the run's largest and below is rounded away, which the
+    comparison allows for through the run's largest value."""
+    K, N = 1536, 4096
+    q, s = ops.quantize_w8(make_weight(K, N, 79))
+    packed = ops.pack_w8(q)
+    qh, sh = q.cpu().numpy().astype(np.float64), s.cpu().numpy().astype(np.float64)
+    rng = np.random.default_rng(7)
+    base = rng.standard_normal(K).astype(np.float32)
+    rows = {"plain": base, "huge": base * np.float32(1e20), "tiny": base * np.float32(1e-20),
+            "zero": np.zeros(K, np.float32)}
+    loud = base.copy()
+    loud[192:384] *= np.float32(1e6)          # one wavefront's run, 10^6 louder
+    rows["loud run"] = loud
+    for name, xh in rows.items():
+        y = ops.gemv_w8a32(torch.from_numpy(xh[None]).cuda(), packed, s, K, N).cpu().numpy()[0]
+        want = (xh.astype(np.float64) @ qh) * sh
+        if name == "zero":
+            assert not y.any()
+            continue
+        check_close(y, want)
+    # the quiet runs are not drowned by the loud one: without it the rest still
+    # agrees to f32 accuracy
+    quiet = loud.copy()
+    quiet[192:384] = 0.0
+    y = ops.gemv_w8a32(torch.from_numpy(quiet[None]).cuda(), packed, s, K, N).cpu().numpy()[0]
+    check_close(y, (quiet.astype(np.float64) @ qh) * sh)
+    # an outlier inside a run costs that run's other values its resolution and
+    # nothing more: the error stays below 2^-22 of the outlier times sum |w|
+    out = base.copy()
+    out[200] = np.float32(3e4)
+    y = ops.gemv_w8a32(torch.from_numpy(out[None]).cuda(), packed, s, K, N).cpu().numpy()[0]
+    want = (out.astype(np.float64) @ qh) * sh
+    bound = 2.0 ** -22 * 3e4 * np.abs(qh[192:384]).sum(0) * sh + 1e-6 * np.abs(want).max()
+    assert (np.abs(y - want) <= bound).all()
+
+
+def test_row_kernel_shows_non_finite_activations():
+    """A NaN or an infinity in the row gives NaN results (the f32 product would
+    give NaN or infinity there)."""
+    K, N = 1536, 256
+    q, s = ops.quantize_w8(make_weight(K, N, 80))
+    packed = ops.pack_w8(q)
+    rng = np.random.default_rng(8)
+    for bad in (np.nan, np.inf, -np.inf):
+        xh = rng.standard_normal((1, K)).astype(np.float32)
+        xh[0, 777] = bad
+        y = ops.gemv_w8a32(torch.from_numpy(xh).cuda(), packed, s, K, N).cpu().numpy()
+        assert np.isnan(y).all()
+
+
 def test_int8_batch_kernel_scales_every_64_activations_on_their_own(oracle):
     """The int8 matrix-core kernel turns the activations into fixed point 64 at a
     time, each row and each run of 64 with a step of its own: rows 40 orders of

@@ -1,8 +1,8 @@
-"""Every compiled variant of the kernels that issue their global loads by hand
-meets the oracle.
+"""Every compiled variant of the kernels that issue their global loads by hand,
+and of the one-row GEMV with its many slot counts, meets the oracle.
 
-Those kernels (the int8 and bf16 matrix-core kernels of the small-batch GEMV
-and of the prefill matmul, and the prefill attention) wait for their loads by
+The first (the int8 and bf16 matrix-core kernels of the small-batch GEMV and of
+the prefill matmul, and the prefill attention) wait for their loads by
 counting; a mistake in one template variant shows only in that variant.  The
 library lists every variant it was built with (buddy_hip_variant_report); this
 test drives one parity case through each plan that selects one, and fails when
@@ -15,7 +15,9 @@ import pytest
 import torch
 
 import buddy_mlir_amd as bma
+import oracle_lib
 from buddy_mlir_amd import ops, synthetic
+from buddy_mlir_amd.session import Shape
 from parity import check_close
 from test_gpu_prefill import SCALE, bf16_round, run_attn
 
@@ -105,6 +107,50 @@ def test_every_bf16_batch_gemv_variant(bh, oracle):
     assert launched(bh, fam) == compiled(bh, fam), compiled(bh, fam) - launched(bh, fam)
 
 
+# ---- one-row GEMV on the integer dot product: <epilogue, input, tile slots per
+# wavefront, channel group split over two workgroups> -----------------------------
+# With more than 128 channel groups a wavefront gets ceil(K / 64 / 16) tiles (16
+# k-slices) once K >= 4096, and K = 128, 192 give runs of 2 and 3; with 4 channel
+# groups and K >= 4096 the groups are split and the tiles go in pairs.  The rows
+# end inside a tile (K % 64 != 0) wherever that keeps the run's length.
+ROW_K = {2: 123, 3: 187, **{t: 1024 * t - 7 for t in range(4, 17)}}
+ROW_SINGLE = [2, 3, 4, 5, 6, 7, 8, 9, 10, 12, 14, 16]
+ROW_DUAL = [2, 3, 4, 5, 6, 7, 8, 9]
+ROW_SPLIT = [4, 6, 8, 10]
+FOLD_HEADS = {2: (12, 2), 3: (24, 4), 4: (32, 4)}  # o_proj of heads x 128 inputs: 2, 3, 4 tiles
+
+
+def test_every_row_gemv_variant(bh, oracle):
+    bh.buddy_hip_variant_reset()
+    for t in ROW_SINGLE:
+        for epilogue in (0, 1):
+            for norm in (False, True):
+                gemv_case(bh, oracle, 1, ROW_K[t], 2064, epilogue, norm, 300 + t)
+    for t in ROW_DUAL:
+        for norm in (False, True):
+            gemv_case(bh, oracle, 1, ROW_K[t], 2064, 2, norm, 330 + t)
+    for t in ROW_SPLIT:
+        for epilogue in (0, 1):
+            for norm in (False, True):
+                gemv_case(bh, oracle, 1, ROW_K[t] - 1024 * (t == 10), 64, epilogue, norm, 360 + t)
+    # input folded from the attention partials: the o_proj of a decode step
+    for tiles, (heads, kv_heads) in FOLD_HEADS.items():
+        shape = Shape(layers=1, hidden=256, heads=heads, kv_heads=kv_heads, head_dim=128, inter=512,
+                      vocab=1024, max_len=128, rms_eps=1e-6)
+        sess, host = synthetic.build_session(shape, context=70, keep_host=True, ln_jitter=0.1)
+        om = oracle_lib.model_from_host(oracle, shape, host)
+        kv = [a.copy() for a in host["kv"]]
+        tok = 3
+        for step in range(3):
+            nxt, logits = sess.decode(tok, 70 + step)
+            tok, ologits = om.decode_step(tok, 70 + step, kv)
+            check_close(logits, ologits)
+            assert nxt == tok
+        sess.close()
+    fam = "gemv_w8a32_dot4_kernel"
+    assert launched(bh, fam) == compiled(bh, fam), compiled(bh, fam) - launched(bh, fam)
+
+
 # ---- prefill matmul: the tile shape comes out of the launch's cost model -------
 GEMM_I8_SHAPES = [(144, 256, 16384), (300, 256, 10240), (200, 192, 16384), (512, 192, 8960),
                   (17, 64, 64)]
@@ -160,5 +206,5 @@ def test_prefill_attention_and_no_unlisted_family(bh, oracle):
     # every family the library lists is one of those this file drives
     known = ("gemv_w8a32_i8_kernel", "gemv_w8a32_mfma_kernel", "gemm_w8_i8_wide_kernel",
              "gemm_w8_i8_kernel", "gemm_w8_bf16_wide_kernel", "gemm_w8_bf16_kernel",
-             "attn_prefill_kernel")
+             "attn_prefill_kernel", "gemv_w8a32_dot4_kernel")
     assert {name.split("<")[0] for name in report(bh)} == set(known)
