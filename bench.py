@@ -36,7 +36,7 @@ if "--no-cpu-baseline" not in sys.argv:
 
 HBM_PEAK_GBPS = 8000.0  # MI355X published HBM3E bandwidth
 CONTEXT = 1024
-GATE_UP_KERNEL = "gemv_w8a32_dot4_kernel<2, 1, 3, false>"
+GATE_UP_KERNEL = "gemv_w8a32_dot4_kernel<1, 2, 1, 3, false>"
 TRAFFIC_PROFILE = "profiles/decode_kernels_hbm_traffic.md"
 
 
@@ -337,7 +337,7 @@ def bench_gemv(bh, args):
         "config": {"workload": "single int8 weight-only GEMV x[1,1536] . W[1536,8960] "
                                "(BASELINE configs[0]), 48 rotating weight copies"},
         "detail": res,
-        "roofline": {"kernel": "gemv_w8a32_dot4_kernel<0, 0, 3, false>", "bound": "hbm",
+        "roofline": {"kernel": "gemv_w8a32_dot4_kernel<1, 0, 0, 3, false>", "bound": "hbm",
                      "achieved": res["hbm_cold"]["gbps"], "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": res["hbm_cold"]["frac"],
                      "algorithmic_bytes_per_launch": by, "avg_launch_us": t * 1e6,

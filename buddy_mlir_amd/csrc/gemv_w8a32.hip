@@ -58,6 +58,8 @@ struct GemvPlan {
   // channels (narrow, long matrices: 96 channel groups would otherwise keep
   // only 96 of the 256 compute units streaming)
   int half_split = 0;
+  // planned for (and checked against the variants of) the dot-product kernel
+  bool row_dot4 = false;
   size_t lds_bytes;
 };
 
@@ -947,7 +949,9 @@ constexpr int kDigitBytesPerTile = 3 * kTileK; // three planes of 64 digits
 // workgroup's 8 channels of two consecutive tiles -- the lanes that would hold
 // the other workgroup's channels take the second tile instead -- so it moves
 // 1 KiB of weights that nobody else reads, in whole 128-byte lines.
-template <int EPI, int PRO, int U, bool HS>
+// M rows (1, 2 or 4) share the weight registers: each row has its own digit
+// planes and sums, 0.75 M instructions per weight.
+template <int M, int EPI, int PRO, int U, bool HS>
 __global__ void __launch_bounds__(kMaxWaves *kWave)
     gemv_w8a32_dot4_kernel(const int4 *pW0, const int4 *pW1, const float *pA,
                            const float *pnorm_w, int p_chunks, int p_KS, int p_G,
@@ -966,6 +970,7 @@ __global__ void __launch_bounds__(kMaxWaves *kWave)
   a.rows = p_rows;
   constexpr bool DUAL = (EPI == kEpiSiluMul);
   constexpr bool NORM = (PRO == kProNorm);
+  static_assert(M == 1 || PRO != kProAttn, "the attention fold feeds one row");
   extern __shared__ float lds[];
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
@@ -979,17 +984,31 @@ __global__ void __launch_bounds__(kMaxWaves *kWave)
   const int t1 = min(t0 + per, a.chunks);
 
   // ---- activations first: their use must not wait for the weights ----------
-  float x[U], nw[U];
+  // A lane takes four consecutive k of the run per load (64 lanes: four tiles),
+  // so that it can cut their digits and write whole dwords of the planes.  The
+  // 16 bytes start inside the row and are aligned, so they never leave the page
+  // the row ends in; values past the row or the run are dropped below.  When
+  // the input is folded from attention partials a lane holds one k per tile.
+  constexpr bool VEC = PRO != kProAttn;
+  constexpr int XV = VEC ? (U + 3) / 4 : U; // activation slots per row
+  constexpr int XE = VEC ? 4 : 1;           // values per slot
+  float x[M][XV][XE], nw[XV][XE];
+  if constexpr (VEC) {
+    const int klast = ((a.K + 3) & ~3) - 4;
 #pragma unroll
-  for (int u = 0; u < U; ++u) {
-    const int k = (t0 + u) * kTileK + lane;
-    const int kc = min(k, a.K - 1);
-    x[u] = 0.f;
-    nw[u] = 0.f;
-    if (PRO != kProAttn)
-      x[u] = a.A[kc];
-    if (NORM)
-      nw[u] = a.norm_w[kc];
+    for (int q = 0; q < XV; ++q) {
+      const int kc = min(t0 * kTileK + q * 256 + 4 * lane, klast);
+      if (NORM) {
+        const float4 v = *reinterpret_cast<const float4 *>(a.norm_w + kc);
+        nw[q][0] = v.x, nw[q][1] = v.y, nw[q][2] = v.z, nw[q][3] = v.w;
+      }
+#pragma unroll
+      for (int m = 0; m < M; ++m) { // rows past the batch repeat its last row; never stored
+        const float4 v = *reinterpret_cast<const float4 *>(
+            a.A + (int64_t)(M == 1 ? 0 : min(m, a.rows - 1)) * a.lda + kc);
+        x[m][q][0] = v.x, x[m][q][1] = v.y, x[m][q][2] = v.z, x[m][q][3] = v.w;
+      }
+    }
   }
   static_assert(!HS || (!DUAL && U % 2 == 0), "split groups: one matrix, tiles in pairs");
   constexpr int P = HS ? U / 2 : U; // weight loads per matrix
@@ -1011,156 +1030,244 @@ __global__ void __launch_bounds__(kMaxWaves *kWave)
     if (DUAL)
       wb[u] = load_stream(w1 + (size_t)t * 64);
   }
-  if (PRO == kProAttn && t0 < t1) {
-    constexpr int FB = U < 4 ? U : 4;
-    float xf[(U + FB - 1) / FB][FB];
+  if constexpr (PRO == kProAttn) {
+    if (t0 < t1) {
+      constexpr int FB = U < 4 ? U : 4;
+      float xf[(U + FB - 1) / FB][FB];
 #pragma unroll
-    for (int q = 0; q < (U + FB - 1) / FB; ++q)
-      if (t0 + FB * q < t1)
-        attn_fold_tiles<FB>(a, t0 + FB * q, t1, lane, xf[q]);
+      for (int q = 0; q < (U + FB - 1) / FB; ++q)
+        if (t0 + FB * q < t1)
+          attn_fold_tiles<FB>(a, t0 + FB * q, t1, lane, xf[q]);
 #pragma unroll
-    for (int u = 0; u < U; ++u)
-      x[u] = xf[u / FB][u % FB];
+      for (int u = 0; u < U; ++u)
+        x[0][u][0] = xf[u / FB][u % FB];
+    } else {
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+        x[0][u][0] = 0.f;
+    }
   }
 
   const int n = g * kTileN + lane;
   const bool writer = ks == 0 && lane < kTileN && live && n < a.N &&
                       (!hs || (lane >> 3) == half);
-  EpilogueOperands<1> epi;
+  EpilogueOperands<M> epi;
   if (writer) {
     epi.s0 = a.s0[n];
     if (DUAL)
       epi.s1 = a.s1[n];
     if (EPI == kEpiStore && a.bias)
       epi.bias = a.bias[n];
-    if (EPI == kEpiAccum)
-      epi.c[0] = a.C[n];
+    if (EPI == kEpiAccum) {
+#pragma unroll
+      for (int m = 0; m < M; ++m)
+        if (m < a.rows)
+          epi.c[m] = a.C[(int64_t)m * a.ldc + n];
+    }
   }
 
   // ---- this wavefront's activations -> digit planes in LDS -----------------
+  // [tile][row][digit][64 k] bytes, after the meeting place of the k-slices
   unsigned char *planes =
-      reinterpret_cast<unsigned char *>(lds + (size_t)nwaves * 33) +
-      (size_t)wave * (U * kDigitBytesPerTile);
-  float ss = 0.f;
-  unsigned mb = 0;
+      reinterpret_cast<unsigned char *>(lds + (size_t)nwaves * M * 33) +
+      (size_t)wave * (U * M * kDigitBytesPerTile);
+  float ss[M], step[M];
 #pragma unroll
-  for (int u = 0; u < U; ++u) {
-    const bool in = t0 + u < t1 && (t0 + u) * kTileK + lane < a.K;
-    float v = in ? x[u] : 0.f;
-    if (NORM) {
-      ss = fmaf(v, v, ss);
-      v *= nw[u];
+  for (int m = 0; m < M; ++m) {
+    ss[m] = 0.f;
+    unsigned mb = 0;
+#pragma unroll
+    for (int q = 0; q < XV; ++q) {
+#pragma unroll
+      for (int e = 0; e < XE; ++e) {
+        // VEC: k = 64 t0 + 256 q + 4 lane + e; otherwise k = 64 (t0 + q) + lane
+        const int k = VEC ? t0 * kTileK + q * 256 + 4 * lane + e : (t0 + q) * kTileK + lane;
+        const bool in = k < t1 * kTileK && k < a.K;
+        float v = in ? x[m][q][e] : 0.f;
+        if (NORM) {
+          ss[m] = fmaf(v, v, ss[m]);
+          v *= nw[q][e];
+        }
+        x[m][q][e] = v;
+        mb = max(mb, __float_as_uint(v) & 0x7fffffffu);
+      }
     }
-    x[u] = v;
-    mb = max(mb, __float_as_uint(v) & 0x7fffffffu);
-  }
-  mb = wave_max_u32(mb); // a NaN or infinity is the largest pattern
-  const int ex = (int)(mb >> 23) - 127; // floor(log2 max), -127 for zero and subnormals
-  const int e2 = max(ex + 1 - 22, -126);
-  const bool finite = mb < 0x7f800000u;
-  const float step = finite ? __uint_as_float((unsigned)(e2 + 127) << 23)
-                            : __uint_as_float(0x7fc00000u);
-  const float inv = __uint_as_float((unsigned)(127 - e2) << 23);
-#pragma unroll
-  for (int u = 0; u < U; ++u) {
+    mb = wave_max_u32(mb); // a NaN or infinity is the largest pattern
+    const int ex = (int)(mb >> 23) - 127; // floor(log2 max), -127 for zero and subnormals
+    const int e2 = max(ex + 1 - 22, -126);
+    const bool finite = mb < 0x7f800000u;
+    step[m] = finite ? __uint_as_float((unsigned)(e2 + 127) << 23)
+                     : __uint_as_float(0x7fc00000u);
+    const float inv = __uint_as_float((unsigned)(127 - e2) << 23);
     // x * inv + 1.5 * 2^23 is rounded to an integer by the addition itself and
     // leaves 0x4B400000 + X in the word; adding 0x8080 makes the low two bytes
     // the balanced digits with their sign bits flipped
     constexpr float kMagic = 12582912.0f;
     constexpr int kBias = 0x8080 - 0x4B400000;
-    const unsigned z =
-        (unsigned)(__float_as_int(fmaf(x[u], inv, kMagic)) + kBias) ^ 0x8080u;
-    unsigned char *p = planes + u * kDigitBytesPerTile + lane;
-    p[0] = (unsigned char)z;
-    p[kTileK] = (unsigned char)(z >> 8);
-    p[2 * kTileK] = (unsigned char)(z >> 16);
+#pragma unroll
+    for (int q = 0; q < XV; ++q) {
+      if constexpr (VEC) {
+        unsigned y[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          y[e] = (unsigned)(__float_as_int(fmaf(x[m][q][e], inv, kMagic)) + kBias);
+        // 4 x 4 byte transpose, three rows of it: a dword per plane
+        const unsigned ta = __builtin_amdgcn_perm(y[1], y[0], 0x05010400u);
+        const unsigned tb = __builtin_amdgcn_perm(y[3], y[2], 0x05010400u);
+        const unsigned tc = __builtin_amdgcn_perm(y[1], y[0], 0x00000602u);
+        const unsigned td = __builtin_amdgcn_perm(y[3], y[2], 0x00000602u);
+        const unsigned d0 = __builtin_amdgcn_perm(tb, ta, 0x05040100u) ^ 0x80808080u;
+        const unsigned d1 = __builtin_amdgcn_perm(tb, ta, 0x07060302u) ^ 0x80808080u;
+        const unsigned d2 = __builtin_amdgcn_perm(td, tc, 0x05040100u);
+        // tile 4 q + lane / 16 of the run, bytes 4 (lane % 16) .. + 3 of its planes
+        const int u = 4 * q + (lane >> 4);
+        if (u < U) {
+          unsigned *p = reinterpret_cast<unsigned *>(planes + (u * M + m) * kDigitBytesPerTile) +
+                        (lane & 15);
+          p[0] = d0;
+          p[kTileK / 4] = d1;
+          p[2 * kTileK / 4] = d2;
+        }
+      } else {
+        const unsigned z =
+            (unsigned)(__float_as_int(fmaf(x[m][q][0], inv, kMagic)) + kBias) ^ 0x8080u;
+        unsigned char *p = planes + (q * M + m) * kDigitBytesPerTile + lane;
+        p[0] = (unsigned char)z;
+        p[kTileK] = (unsigned char)(z >> 8);
+        p[2 * kTileK] = (unsigned char)(z >> 16);
+      }
+    }
   }
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
   __builtin_amdgcn_wave_barrier();
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 
-  int s0[3] = {0, 0, 0}, s1[3] = {0, 0, 0};
-  const unsigned char *mine_d = planes + 16 * (lane >> 4) + second * kDigitBytesPerTile;
+  int s0[M][3], s1[M][3];
+#pragma unroll
+  for (int m = 0; m < M; ++m)
+#pragma unroll
+    for (int d = 0; d < 3; ++d) {
+      s0[m][d] = 0;
+      s1[m][d] = 0;
+    }
+  const unsigned char *mine_d =
+      planes + 16 * (lane >> 4) + second * (M * kDigitBytesPerTile);
 #pragma unroll
   for (int u = 0; u < P; ++u) {
     if (t0 + (HS ? 2 : 1) * u < t1) {
 #pragma unroll
-      for (int d = 0; d < 3; ++d) {
-        const int4 xd = *reinterpret_cast<const int4 *>(
-            mine_d + (HS ? 2 : 1) * u * kDigitBytesPerTile + d * kTileK);
-        s0[d] = __builtin_amdgcn_sdot4(wa[u].x, xd.x, s0[d], false);
-        s0[d] = __builtin_amdgcn_sdot4(wa[u].y, xd.y, s0[d], false);
-        s0[d] = __builtin_amdgcn_sdot4(wa[u].z, xd.z, s0[d], false);
-        s0[d] = __builtin_amdgcn_sdot4(wa[u].w, xd.w, s0[d], false);
-        if (DUAL) {
-          s1[d] = __builtin_amdgcn_sdot4(wb[u].x, xd.x, s1[d], false);
-          s1[d] = __builtin_amdgcn_sdot4(wb[u].y, xd.y, s1[d], false);
-          s1[d] = __builtin_amdgcn_sdot4(wb[u].z, xd.z, s1[d], false);
-          s1[d] = __builtin_amdgcn_sdot4(wb[u].w, xd.w, s1[d], false);
+      for (int m = 0; m < M; ++m) {
+#pragma unroll
+        for (int d = 0; d < 3; ++d) {
+          const int4 xd = *reinterpret_cast<const int4 *>(
+              mine_d + ((HS ? 2 : 1) * u * M + m) * kDigitBytesPerTile + d * kTileK);
+          s0[m][d] = __builtin_amdgcn_sdot4(wa[u].x, xd.x, s0[m][d], false);
+          s0[m][d] = __builtin_amdgcn_sdot4(wa[u].y, xd.y, s0[m][d], false);
+          s0[m][d] = __builtin_amdgcn_sdot4(wa[u].z, xd.z, s0[m][d], false);
+          s0[m][d] = __builtin_amdgcn_sdot4(wa[u].w, xd.w, s0[m][d], false);
+          if (DUAL) {
+            s1[m][d] = __builtin_amdgcn_sdot4(wb[u].x, xd.x, s1[m][d], false);
+            s1[m][d] = __builtin_amdgcn_sdot4(wb[u].y, xd.y, s1[m][d], false);
+            s1[m][d] = __builtin_amdgcn_sdot4(wb[u].z, xd.z, s1[m][d], false);
+            s1[m][d] = __builtin_amdgcn_sdot4(wb[u].w, xd.w, s1[m][d], false);
+          }
         }
       }
     }
   }
-  // |s0[0]|, |s0[1]| < 2^22 per lane (at most 10 x 16 products of 2^14): exact
-  const float step65536 = step * 65536.0f;
-  float acc0 = fmaf((float)s0[2], step65536, (float)(s0[0] + (s0[1] << 8)) * step);
-  float acc1 = DUAL ? fmaf((float)s1[2], step65536, (float)(s1[0] + (s1[1] << 8)) * step) : 0.f;
-
-  // the four rows of a wavefront hold different k sub-ranges of the same channels
-  // (and so do the two halves of a row when tiles go in pairs)
-  if (HS)
-    acc0 += dpp_f<0x128>(acc0); // row_ror:8, lane ^ 8
-  acc0 = sum_rows(acc0);
-  if (DUAL)
-    acc1 = sum_rows(acc1);
-  if (NORM)
-    ss = wave_sum(ss);
+  float acc0[M], acc1[M];
+#pragma unroll
+  for (int m = 0; m < M; ++m) {
+    // |s[0]|, |s[1]| < 2^22 per lane (at most 16 x 16 products of 2^14): exact
+    const float step65536 = step[m] * 65536.0f;
+    acc0[m] = fmaf((float)s0[m][2], step65536, (float)(s0[m][0] + (s0[m][1] << 8)) * step[m]);
+    acc1[m] = DUAL ? fmaf((float)s1[m][2], step65536,
+                          (float)(s1[m][0] + (s1[m][1] << 8)) * step[m])
+                   : 0.f;
+    // the four rows of a wavefront hold different k sub-ranges of the same
+    // channels (and so do the two halves of a row when tiles go in pairs)
+    if (HS)
+      acc0[m] += dpp_f<0x128>(acc0[m]); // row_ror:8, lane ^ 8
+    acc0[m] = sum_rows(acc0[m]);
+    if (DUAL)
+      acc1[m] = sum_rows(acc1[m]);
+    if (NORM)
+      ss[m] = wave_sum(ss[m]);
+  }
 
   // ---- k-slices of one channel group meet in LDS, in slice order ----------
   if (a.KS > 1) {
-    float *mine = lds + (size_t)wave * 33;
+    float *mine = lds + (size_t)wave * M * 33;
     if (lane < kTileN) {
-      mine[lane] = acc0;
-      if (DUAL)
-        mine[16 + lane] = acc1;
+#pragma unroll
+      for (int m = 0; m < M; ++m) {
+        mine[m * 33 + lane] = acc0[m];
+        if (DUAL)
+          mine[m * 33 + 16 + lane] = acc1[m];
+      }
     }
-    if (NORM && lane == 0)
-      mine[32] = ss;
+    if (NORM && lane == 0) {
+#pragma unroll
+      for (int m = 0; m < M; ++m)
+        mine[m * 33 + 32] = ss[m];
+    }
     __syncthreads();
     if (ks != 0)
       return;
     if (lane < kTileN) {
-      float r0 = 0.f, r1 = 0.f, rs = 0.f;
-      for (int s = 0; s < a.KS; ++s) {
-        const float *o = lds + (size_t)(wave + s) * 33;
-        r0 += o[lane];
-        if (DUAL)
-          r1 += o[16 + lane];
-        if (NORM)
-          rs += o[32];
+#pragma unroll
+      for (int m = 0; m < M; ++m) {
+        float r0 = 0.f, r1 = 0.f, rs = 0.f;
+        for (int s = 0; s < a.KS; ++s) {
+          const float *o = lds + (size_t)(wave + s) * M * 33 + m * 33;
+          r0 += o[lane];
+          if (DUAL)
+            r1 += o[16 + lane];
+          if (NORM)
+            rs += o[32];
+        }
+        acc0[m] = r0;
+        acc1[m] = r1;
+        ss[m] = rs;
       }
-      acc0 = r0;
-      acc1 = r1;
-      ss = rs;
     }
   }
   if (writer) {
-    if (NORM) {
-      const float r = fast_rsqrt(ss * a.norm_inv_k + a.norm_eps);
-      acc0 *= r;
-      acc1 *= r;
+#pragma unroll
+    for (int m = 0; m < M; ++m) {
+      if (m < a.rows) {
+        float v0 = acc0[m], v1 = acc1[m];
+        if (NORM) {
+          const float r = fast_rsqrt(ss[m] * a.norm_inv_k + a.norm_eps);
+          v0 *= r;
+          v1 *= r;
+        }
+        finish<M, EPI>(a, m, n, v0, v1, epi);
+      }
     }
-    finish<1, EPI>(a, 0, n, acc0, acc1, epi);
   }
 }
 
 BH_VARIANT_FAMILY(RowDot4Family, "gemv_w8a32_dot4_kernel");
 
-template <int EPI, int PRO, int U, bool HS = false>
+constexpr size_t dot4_lds_bytes(int waves, int M, int U) {
+  return sizeof(float) * waves * (size_t)M * 33 + (size_t)waves * U * M * kDigitBytesPerTile;
+}
+
+template <int M, int EPI, int PRO, int U, bool HS = false>
 int launch_dot4(const KernelArgs &ka, const GemvPlan &p, hipStream_t stream) {
-  BH_NOTE_VARIANT(RowDot4Family, EPI, PRO, U, HS ? 1 : 0);
-  auto kernel = gemv_w8a32_dot4_kernel<EPI, PRO, U, HS>;
-  const size_t lds = sizeof(float) * p.waves * 33 + (size_t)p.waves * U * kDigitBytesPerTile;
+  BH_NOTE_VARIANT(RowDot4Family, M, EPI, PRO, U, HS ? 1 : 0);
+  auto kernel = gemv_w8a32_dot4_kernel<M, EPI, PRO, U, HS>;
+  const size_t lds = dot4_lds_bytes(p.waves, M, U);
+  if constexpr (dot4_lds_bytes(kMaxWaves, M, U) > 48 * 1024) {
+    static bool attr_set = false;
+    if (!attr_set) {
+      BH_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize,
+                                       (int)dot4_lds_bytes(kMaxWaves, M, U)));
+      attr_set = true;
+    }
+  }
   hipLaunchKernelGGL(kernel, dim3(p.blocks << p.half_split), dim3(p.waves * kWave), lds,
                      stream, ka.W0, ka.W1, ka.A, ka.norm_w, ka.chunks, ka.KS,
                      ka.G | (p.half_split << 16), ka.groups, ka.K, ka.rows, ka);
@@ -1171,14 +1278,59 @@ int launch_dot4(const KernelArgs &ka, const GemvPlan &p, hipStream_t stream) {
 constexpr int kNoFit = -1000; // no compiled slot count holds the run
 
 // the smallest compiled slot count that holds `tpw` tiles per wavefront
-template <int EPI, int PRO, bool HS, int... Us>
+template <int M, int EPI, int PRO, bool HS, int... Us>
 int launch_dot4_fit(std::integer_sequence<int, Us...>, int64_t tpw, const KernelArgs &ka,
                     const GemvPlan &p, hipStream_t stream) {
   int rc = kNoFit;
   bool done = false;
-  ((done || tpw > Us ? 0 : (done = true, rc = launch_dot4<EPI, PRO, Us, HS>(ka, p, stream))),
+  ((done || tpw > Us ? 0
+                     : (done = true, rc = launch_dot4<M, EPI, PRO, Us, HS>(ka, p, stream))),
    ...);
   return rc;
+}
+
+// Slot counts compiled per form: dense for one row, where a spare slot is a
+// large part of a short run; coarser for 2 and 4 rows, and only as far as the
+// activations (M per slot) and the weights fit in 128 registers.
+template <int M> struct Dot4Slots { // M = 4
+  using Single = std::integer_sequence<int, 2, 3, 4, 6, 8>;
+  using Dual = std::integer_sequence<int, 2, 3, 4, 6>;
+};
+template <> struct Dot4Slots<2> {
+  using Single = std::integer_sequence<int, 2, 3, 4, 6, 8, 10, 12>;
+  using Dual = std::integer_sequence<int, 2, 3, 4, 6, 8>;
+};
+template <> struct Dot4Slots<1> {
+  using Single = std::integer_sequence<int, 2, 3, 4, 5, 6, 7, 8, 9, 10, 12, 14, 16>;
+  using Dual = std::integer_sequence<int, 2, 3, 4, 5, 6, 7, 8, 9>;
+};
+using Dot4SlotsSplit = std::integer_sequence<int, 4, 6, 8, 10>;
+using Dot4SlotsFold = std::integer_sequence<int, 2, 3, 4>; // 18 partials per tile in registers
+
+// the slot count a run of `tpw` tiles gets from a list, 0 if none holds it
+template <int... Us> int slots_for(std::integer_sequence<int, Us...>, int64_t tpw) {
+  int v = 0;
+  ((v = (v == 0 && tpw <= Us) ? Us : v), ...);
+  return v;
+}
+
+// Does a plan made for the dot-product kernel have a compiled variant?
+bool dot4_fits(int M, const GemvPlan &p, bool dual, bool fold) {
+  const int64_t tpw = ceil_div(p.chunks, p.KS);
+  int u = 0;
+  if (p.half_split)
+    u = (dual || fold) ? 0 : slots_for(Dot4SlotsSplit{}, tpw);
+  else if (fold)
+    u = M == 1 ? slots_for(Dot4SlotsFold{}, tpw) : 0;
+  else if (dual)
+    u = M == 1   ? slots_for(Dot4Slots<1>::Dual{}, tpw)
+        : M == 2 ? slots_for(Dot4Slots<2>::Dual{}, tpw)
+                 : slots_for(Dot4Slots<4>::Dual{}, tpw);
+  else
+    u = M == 1   ? slots_for(Dot4Slots<1>::Single{}, tpw)
+        : M == 2 ? slots_for(Dot4Slots<2>::Single{}, tpw)
+                 : slots_for(Dot4Slots<4>::Single{}, tpw);
+  return u != 0 && dot4_lds_bytes(p.waves, M, u) <= kMaxLdsBytes;
 }
 
 bool row_dot4() {
@@ -1230,29 +1382,29 @@ int launch_one(const KernelArgs &ka, const GemvPlan &p, hipStream_t stream) {
       return launch_tn<kNarrowOk ? 1 : M, kNarrowOk ? EPI : kEpiStore, PRO, 4, kNarrowOk ? 8 : 16>(ka, p, stream);
     return launch_tn<kNarrowOk ? 1 : M, kNarrowOk ? EPI : kEpiStore, PRO, 4, kNarrowOk ? 4 : 16>(ka, p, stream);
   }
-  if (M == 1 && row_dot4()) {
-    // short runs (every tile of a wavefront requested at once) go to the integer
-    // dot product; the slot counts are dense where a spare slot is a large part
-    // of the run
-    const int64_t tpw = ceil_div(p.chunks, p.KS); // tiles per wavefront
-    int rc = kNoFit;
-    if (p.half_split) {
-      if constexpr (!kDual && PRO != kProAttn)
-        rc = launch_dot4_fit<EPI, PRO, true>(std::integer_sequence<int, 4, 6, 8, 10>{}, tpw,
-                                             ka, p, stream);
-    } else if constexpr (PRO == kProAttn) { // the fold keeps 18 partials per tile in registers
-      rc = launch_dot4_fit<EPI, PRO, false>(std::integer_sequence<int, 2, 3, 4>{}, tpw, ka, p,
-                                            stream);
-    } else if constexpr (kDual) {
-      rc = launch_dot4_fit<EPI, PRO, false>(
-          std::integer_sequence<int, 2, 3, 4, 5, 6, 7, 8, 9>{}, tpw, ka, p, stream);
-    } else {
-      rc = launch_dot4_fit<EPI, PRO, false>(
-          std::integer_sequence<int, 2, 3, 4, 5, 6, 7, 8, 9, 10, 12, 14, 16>{}, tpw, ka, p,
-          stream);
+  if constexpr (M <= 4) {
+    if (p.row_dot4) {
+      // every tile of a wavefront's run is requested at once
+      const int64_t tpw = ceil_div(p.chunks, p.KS); // tiles per wavefront
+      int rc = kNoFit;
+      if (p.half_split) {
+        if constexpr (!kDual && PRO != kProAttn)
+          rc = launch_dot4_fit<M, EPI, PRO, true>(Dot4SlotsSplit{}, tpw, ka, p, stream);
+      } else if constexpr (PRO == kProAttn) {
+        if constexpr (M == 1)
+          rc = launch_dot4_fit<1, EPI, PRO, false>(Dot4SlotsFold{}, tpw, ka, p, stream);
+      } else if constexpr (kDual) {
+        rc = launch_dot4_fit<M, EPI, PRO, false>(typename Dot4Slots<M>::Dual{}, tpw, ka, p,
+                                                 stream);
+      } else {
+        rc = launch_dot4_fit<M, EPI, PRO, false>(typename Dot4Slots<M>::Single{}, tpw, ka, p,
+                                                 stream);
+      }
+      if (rc != kNoFit)
+        return rc;
+      return fail(BUDDY_HIP_ERR_ARG, "gemv: no dot-product variant for %lld tiles per wavefront",
+                  (long long)tpw);
     }
-    if (rc != kNoFit)
-      return rc;
   }
   constexpr int kRing = M == 1 ? (kDual ? 6 : 8) : M <= 4 ? 4 : M == 8 ? 2 : 1;
   return launch_bcast<M, EPI, PRO, kRing>(ka, p, stream);
@@ -1340,7 +1492,21 @@ int launch_gemv(const GemvArgs &a, hipStream_t stream) {
   const int mt = compiled_rows(a.M);
   BH_REQUIRE(a.tile_n == 16 || a.tile_n == 8 || a.tile_n == 4,
              "gemv: tile_n=%d (16, 8 or 4)", a.tile_n);
-  const GemvPlan p = make_plan(mt, a.K, a.N, dual, a.tile_n, a.attn_acc != nullptr);
+  // Up to four rows go to the dot-product kernel, cut as for one row, when it
+  // has a variant for the run a wavefront gets; otherwise the f32 kernel with
+  // its own cut.
+  const bool fold = a.attn_acc != nullptr;
+  GemvPlan p = make_plan(mt, a.K, a.N, dual, a.tile_n, fold);
+  // (its activation rows are read as aligned 16-byte pieces)
+  const bool rows_aligned =
+      fold || ((reinterpret_cast<uintptr_t>(a.A) & 15) == 0 && (a.M == 1 || (a.lda & 3) == 0));
+  if (mt <= 4 && a.tile_n == 16 && rows_aligned && row_dot4()) {
+    GemvPlan q = make_plan(1, a.K, a.N, dual, a.tile_n, fold);
+    if (dot4_fits(mt, q, dual, fold)) {
+      q.row_dot4 = true;
+      p = q;
+    }
+  }
   KernelArgs ka;
   ka.A = a.A;
   ka.W0 = reinterpret_cast<const int4 *>(a.W0);

@@ -107,32 +107,37 @@ def test_every_bf16_batch_gemv_variant(bh, oracle):
     assert launched(bh, fam) == compiled(bh, fam), compiled(bh, fam) - launched(bh, fam)
 
 
-# ---- one-row GEMV on the integer dot product: <epilogue, input, tile slots per
-# wavefront, channel group split over two workgroups> -----------------------------
+# ---- GEMV of up to four rows on the integer dot product: <rows, epilogue, input,
+# tile slots per wavefront, channel group split over two workgroups> ---------------
 # With more than 128 channel groups a wavefront gets ceil(K / 64 / 16) tiles (16
 # k-slices) once K >= 4096, and K = 128, 192 give runs of 2 and 3; with 4 channel
 # groups and K >= 4096 the groups are split and the tiles go in pairs.  The rows
-# end inside a tile (K % 64 != 0) wherever that keeps the run's length.
-ROW_K = {2: 123, 3: 187, **{t: 1024 * t - 7 for t in range(4, 17)}}
-ROW_SINGLE = [2, 3, 4, 5, 6, 7, 8, 9, 10, 12, 14, 16]
-ROW_DUAL = [2, 3, 4, 5, 6, 7, 8, 9]
+# end inside a tile (K % 64 != 0) wherever that keeps the run's length; K stays a
+# multiple of 4 so that batches of rows keep 16-byte aligned rows (one row with
+# K % 4 != 0 is covered by the shapes of test_gpu_gemv.py).
+ROW_K = {2: 124, 3: 188, **{t: 1024 * t - 8 for t in range(4, 17)}}
+ROW_SINGLE = {1: [2, 3, 4, 5, 6, 7, 8, 9, 10, 12, 14, 16], 2: [2, 3, 4, 6, 8, 10, 12],
+              3: [2, 3, 4, 6, 8]}
+ROW_DUAL = {1: [2, 3, 4, 5, 6, 7, 8, 9], 2: [2, 3, 4, 6, 8], 3: [2, 3, 4, 6]}
 ROW_SPLIT = [4, 6, 8, 10]
 FOLD_HEADS = {2: (12, 2), 3: (24, 4), 4: (32, 4)}  # o_proj of heads x 128 inputs: 2, 3, 4 tiles
 
 
 def test_every_row_gemv_variant(bh, oracle):
     bh.buddy_hip_variant_reset()
-    for t in ROW_SINGLE:
-        for epilogue in (0, 1):
+    for rows in (1, 2, 3):  # three rows run the kernel compiled for four
+        for t in ROW_SINGLE[rows]:
+            for epilogue in (0, 1):
+                for norm in (False, True):
+                    gemv_case(bh, oracle, rows, ROW_K[t], 2064, epilogue, norm, 300 + t)
+        for t in ROW_DUAL[rows]:
             for norm in (False, True):
-                gemv_case(bh, oracle, 1, ROW_K[t], 2064, epilogue, norm, 300 + t)
-    for t in ROW_DUAL:
-        for norm in (False, True):
-            gemv_case(bh, oracle, 1, ROW_K[t], 2064, 2, norm, 330 + t)
-    for t in ROW_SPLIT:
-        for epilogue in (0, 1):
-            for norm in (False, True):
-                gemv_case(bh, oracle, 1, ROW_K[t] - 1024 * (t == 10), 64, epilogue, norm, 360 + t)
+                gemv_case(bh, oracle, rows, ROW_K[t], 2064, 2, norm, 330 + t)
+        for t in ROW_SPLIT:
+            for epilogue in (0, 1):
+                for norm in (False, True):
+                    gemv_case(bh, oracle, rows, ROW_K[t] - 1024 * (t == 10), 64, epilogue, norm,
+                              360 + t)
     # input folded from the attention partials: the o_proj of a decode step
     for tiles, (heads, kv_heads) in FOLD_HEADS.items():
         shape = Shape(layers=1, hidden=256, heads=heads, kv_heads=kv_heads, head_dim=128, inter=512,
