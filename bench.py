@@ -36,7 +36,7 @@ if "--no-cpu-baseline" not in sys.argv:
 
 HBM_PEAK_GBPS = 8000.0  # MI355X published HBM3E bandwidth
 CONTEXT = 1024
-GATE_UP_KERNEL = "gemv_w8a32_dot4_kernel<1, 2, 1, 3, false>"
+GATE_UP_KERNEL = "gemv_w8a32_digits_kernel<1, 2, 1, 3, false>"
 TRAFFIC_PROFILE = "profiles/decode_kernels_hbm_traffic.md"
 
 
@@ -337,7 +337,7 @@ def bench_gemv(bh, args):
         "config": {"workload": "single int8 weight-only GEMV x[1,1536] . W[1536,8960] "
                                "(BASELINE configs[0]), 48 rotating weight copies"},
         "detail": res,
-        "roofline": {"kernel": "gemv_w8a32_dot4_kernel<1, 0, 0, 3, false>", "bound": "hbm",
+        "roofline": {"kernel": "gemv_w8a32_digits_kernel<1, 0, 0, 3, false>", "bound": "hbm",
                      "achieved": res["hbm_cold"]["gbps"], "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": res["hbm_cold"]["frac"],
                      "algorithmic_bytes_per_launch": by, "avg_launch_us": t * 1e6,
@@ -739,7 +739,7 @@ def bench_llama8b(bh, args):
         "config": {"workload": "Llama-3-8B-shaped decode GEMV sweep, 32 layers + lm_head, "
                                "161 dependent launches (BASELINE configs[4]); value is M=1"},
         "detail": res,
-        "roofline": {"kernel": "gemv_w8a32_dot4_kernel, gemv_w8a32_bcast_kernel for lm_head (all shapes of the sweep)",
+        "roofline": {"kernel": "gemv_w8a32_digits_kernel, gemv_w8a32_bcast_kernel for lm_head (all shapes of the sweep)",
                      "bound": "hbm", "achieved": r1["gbps"], "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": r1["frac"], "traffic": None},
     }
@@ -896,9 +896,10 @@ def main():
         "dtype": "int8",
         "data": "synthetic",
         "config": {
-            "arithmetic": "per-layer GEMVs: int8 weights x f32 activations cut into three int8 "
-                          "digit planes (23-bit fixed point per wavefront's run), exact int32 "
-                          "sums; attention, norms, lm_head and every kernel boundary: f32",
+            "arithmetic": "per-layer GEMVs: int8 weights x f32 activations cut into four int8 "
+                          "digit planes (31-bit fixed point per wavefront's run) on the int8 "
+                          "matrix cores, exact int32 sums; attention, norms, lm_head and every "
+                          "kernel boundary: f32",
             "workload": "Qwen2-1.5B-shaped int8 weight-only (w8a32) decoder, one "
                         "greedy decode step, batch 1, KV cache prefilled to 1024 "
                         "positions (BASELINE configs[2])",

@@ -15,11 +15,11 @@
 //    wavefronts streaming.  The k-slices meet in LDS, in slice order, so the
 //    sum is deterministic and no workgroup ever waits for another one (cross-
 //    XCD traffic inside a kernel costs an L2 write-back on this part);
-//  * one row (gemv_w8a32_dot4_kernel): a wavefront turns the activations of its
-//    run of tiles into three int8 digit planes of a 23-bit fixed-point value,
-//    leaves them in a private corner of LDS and multiplies four weights per
-//    instruction (v_dot4_i32_i8) into exact int32 sums;
-//  * two to four rows, and runs too long for one batch of loads
+//  * one to four rows (gemv_w8a32_digits_kernel): a wavefront turns the
+//    activations of its run of tiles into four int8 digit planes of a 31-bit
+//    fixed-point value per row, leaves them in a private corner of LDS and
+//    feeds weight tiles and planes to the int8 matrix cores (exact int32 sums);
+//  * runs too long for one batch of loads, or rows that are not 16-byte aligned
 //    (gemv_w8a32_bcast_kernel): activations never pass through LDS, a lane
 //    loads the one activation whose k equals its position in the tile and the
 //    f32 multiply-add reads its neighbours' values through DPP row broadcasts;
@@ -30,7 +30,6 @@
 //    the same kernel; their operands are requested before the stream starts.
 // The 8- and 4-channel tile layouts keep the older kernel that stages the
 // activations in LDS (gemv_w8a32_kernel).
-// No MFMA: with one row 15 of a matrix instruction's 16 columns would be empty.
 #include "gemv_w8a32.h"
 
 #include <atomic>
@@ -58,8 +57,8 @@ struct GemvPlan {
   // channels (narrow, long matrices: 96 channel groups would otherwise keep
   // only 96 of the 256 compute units streaming)
   int half_split = 0;
-  // planned for (and checked against the variants of) the dot-product kernel
-  bool row_dot4 = false;
+  // planned for (and checked against the variants of) the digit-plane kernel
+  bool on_digits = false;
   size_t lds_bytes;
 };
 
@@ -914,19 +913,21 @@ __global__ void __launch_bounds__(kMaxWaves *kWave)
 }
 
 // ---------------------------------------------------------------------------
-// One row on the integer dot product (v_dot4_i32_i8), 0.75 instructions per
-// weight instead of two.
+// One to four rows on the int8 matrix cores, no VALU instruction per weight.
 //
 // A wavefront turns the activations of its own run of tiles into fixed point,
-// X = rint(x / s) with s the smallest power of two that keeps |X| < 2^22 over
-// the run, cuts X into three balanced int8 digits (X = d0 + 256 d1 + 65536 d2)
-// and leaves each digit plane in its own corner of LDS in k order.  A lane then
-// reads the 16 digits that go with its 16 weights as one 128-bit word per plane
-// (the 16 lanes of a row read the same word: a broadcast) and multiplies four
-// weights at a time.  The int32 sums are exact; the only rounding is that of X,
-// 2^-23 of the largest activation of the run.  Nothing waits for another
-// wavefront before the stream: the planes are private to the wavefront that
-// wrote them.
+// X = rint(x / s) with s the smallest power of two that keeps |X| < 2^30 over
+// the run (one s per row), cuts X into four balanced int8 digits
+// (X = d0 + 256 d1 + 65536 d2 + 2^24 d3) and leaves each digit plane in its own
+// corner of LDS in k order.  A weight tile as it lies in its registers is the A
+// operand of v_mfma_i32_16x16x64_i8 (16 channels x 64 k); the 4 M digit planes
+// of the tile are columns of B, of which lane (k / 16, column) reads its 16
+// bytes with one ds_read_b128.  One matrix instruction per tile and matrix
+// multiplies every row and digit.  The int32 sums are exact; the only rounding
+// is that of X, 2^-31 of the row's largest activation in the run, so that an
+// activation within 2^7 of that largest one enters with all its 24 bits.
+// Nothing waits for another wavefront before the stream: the planes are private
+// to the wavefront that wrote them.
 // ---------------------------------------------------------------------------
 __device__ __forceinline__ unsigned wave_max_u32(unsigned v) {
   auto dpp = [](unsigned x, auto ctrl) {
@@ -942,18 +943,18 @@ __device__ __forceinline__ unsigned wave_max_u32(unsigned v) {
   return max(max(a, b), max(c, d));
 }
 
-constexpr int kDigitBytesPerTile = 3 * kTileK; // three planes of 64 digits
+constexpr int kDigits = 4;                            // int8 digits per activation
+constexpr int kDigitBytesPerTile = kDigits * kTileK;  // the planes of one tile and row
 
-//
 // HS (a channel group split over two workgroups): a load instruction covers the
 // workgroup's 8 channels of two consecutive tiles -- the lanes that would hold
 // the other workgroup's channels take the second tile instead -- so it moves
-// 1 KiB of weights that nobody else reads, in whole 128-byte lines.
-// M rows (1, 2 or 4) share the weight registers: each row has its own digit
-// planes and sums, 0.75 M instructions per weight.
+// 1 KiB of weights that nobody else reads, in whole 128-byte lines.  The rows
+// of such an A operand belong to two tiles: it is multiplied once with each
+// tile's planes and every row keeps the product that is its own.
 template <int M, int EPI, int PRO, int U, bool HS>
 __global__ void __launch_bounds__(kMaxWaves *kWave)
-    gemv_w8a32_dot4_kernel(const int4 *pW0, const int4 *pW1, const float *pA,
+    gemv_w8a32_digits_kernel(const int4 *pW0, const int4 *pW1, const float *pA,
                            const float *pnorm_w, int p_chunks, int p_KS, int p_G,
                            int p_groups, int p_K, int p_rows, KernelArgs rest) {
   KernelArgs a = rest;
@@ -1067,11 +1068,11 @@ __global__ void __launch_bounds__(kMaxWaves *kWave)
   }
 
   // ---- this wavefront's activations -> digit planes in LDS -----------------
-  // [tile][row][digit][64 k] bytes, after the meeting place of the k-slices
-  unsigned char *planes =
-      reinterpret_cast<unsigned char *>(lds + (size_t)nwaves * M * 33) +
-      (size_t)wave * (U * M * kDigitBytesPerTile);
-  float ss[M], step[M];
+  // Four digits: X = rint(x / s) with |X| < 2^30, so that an activation within
+  // 2^7 of the row's largest in the run keeps every one of its 24 bits.
+  // Per row the run's largest magnitude first (a NaN or infinity is the
+  // largest bit pattern), then the step.
+  float ss[M], step[M], inv[M];
 #pragma unroll
   for (int m = 0; m < M; ++m) {
     ss[m] = 0.f;
@@ -1092,118 +1093,176 @@ __global__ void __launch_bounds__(kMaxWaves *kWave)
         mb = max(mb, __float_as_uint(v) & 0x7fffffffu);
       }
     }
-    mb = wave_max_u32(mb); // a NaN or infinity is the largest pattern
+    mb = wave_max_u32(mb);
     const int ex = (int)(mb >> 23) - 127; // floor(log2 max), -127 for zero and subnormals
-    const int e2 = max(ex + 1 - 22, -126);
+    const int e2 = max(ex + 1 - 30, -126);
     const bool finite = mb < 0x7f800000u;
     step[m] = finite ? __uint_as_float((unsigned)(e2 + 127) << 23)
                      : __uint_as_float(0x7fc00000u);
-    const float inv = __uint_as_float((unsigned)(127 - e2) << 23);
-    // x * inv + 1.5 * 2^23 is rounded to an integer by the addition itself and
-    // leaves 0x4B400000 + X in the word; adding 0x8080 makes the low two bytes
-    // the balanced digits with their sign bits flipped
-    constexpr float kMagic = 12582912.0f;
-    constexpr int kBias = 0x8080 - 0x4B400000;
+    inv[m] = __uint_as_float((unsigned)(127 - e2) << 23);
+  }
+  // The planes of four tiles at a time, [tile][row][digit][64 k] bytes, in a
+  // corner of LDS private to the wavefront (after the meeting place of the
+  // k-slices): group q + 1 is cut and written once the reads of group q have
+  // been issued (LDS serves a wavefront's requests in order).
+  constexpr int NG = VEC ? XV : 1;      // groups of tiles
+  constexpr int TG = VEC ? 4 : U;       // tiles per group
+  static_assert(TG <= 4, "a group of planes holds four tiles");
+  unsigned char *planes =
+      reinterpret_cast<unsigned char *>(lds + (size_t)nwaves * M * 33) +
+      (size_t)wave * (4 * M * kDigitBytesPerTile);
+  auto cut_group = [&](int q) {
 #pragma unroll
-    for (int q = 0; q < XV; ++q) {
+    for (int m = 0; m < M; ++m) {
       if constexpr (VEC) {
+        // X + 0x00808080: the low three bytes are the balanced digits with their
+        // sign bits flipped, the top byte is the fourth digit as it is
         unsigned y[4];
 #pragma unroll
-        for (int e = 0; e < 4; ++e)
-          y[e] = (unsigned)(__float_as_int(fmaf(x[m][q][e], inv, kMagic)) + kBias);
-        // 4 x 4 byte transpose, three rows of it: a dword per plane
+        for (int e = 0; e < 4; ++e) {
+          const int r = (int)__builtin_rintf(x[m][q][e] * inv[m]); // exact: |.| < 2^30
+          y[e] = (unsigned)r + 0x00808080u;
+        }
+        // 4 x 4 byte transpose: a dword per plane
         const unsigned ta = __builtin_amdgcn_perm(y[1], y[0], 0x05010400u);
         const unsigned tb = __builtin_amdgcn_perm(y[3], y[2], 0x05010400u);
-        const unsigned tc = __builtin_amdgcn_perm(y[1], y[0], 0x00000602u);
-        const unsigned td = __builtin_amdgcn_perm(y[3], y[2], 0x00000602u);
+        const unsigned tc = __builtin_amdgcn_perm(y[1], y[0], 0x07030602u);
+        const unsigned td = __builtin_amdgcn_perm(y[3], y[2], 0x07030602u);
         const unsigned d0 = __builtin_amdgcn_perm(tb, ta, 0x05040100u) ^ 0x80808080u;
         const unsigned d1 = __builtin_amdgcn_perm(tb, ta, 0x07060302u) ^ 0x80808080u;
-        const unsigned d2 = __builtin_amdgcn_perm(td, tc, 0x05040100u);
-        // tile 4 q + lane / 16 of the run, bytes 4 (lane % 16) .. + 3 of its planes
-        const int u = 4 * q + (lane >> 4);
-        if (u < U) {
-          unsigned *p = reinterpret_cast<unsigned *>(planes + (u * M + m) * kDigitBytesPerTile) +
-                        (lane & 15);
-          p[0] = d0;
-          p[kTileK / 4] = d1;
-          p[2 * kTileK / 4] = d2;
-        }
+        const unsigned d2 = __builtin_amdgcn_perm(td, tc, 0x05040100u) ^ 0x80808080u;
+        const unsigned d3 = __builtin_amdgcn_perm(td, tc, 0x07060302u);
+        // tile lane / 16 of the group, bytes 4 (lane % 16) .. + 3 of its planes
+        unsigned *p = reinterpret_cast<unsigned *>(planes +
+                                                   ((lane >> 4) * M + m) * kDigitBytesPerTile) +
+                      (lane & 15);
+        p[0] = d0;
+        p[kTileK / 4] = d1;
+        p[2 * kTileK / 4] = d2;
+        p[3 * kTileK / 4] = d3;
       } else {
-        const unsigned z =
-            (unsigned)(__float_as_int(fmaf(x[m][q][0], inv, kMagic)) + kBias) ^ 0x8080u;
-        unsigned char *p = planes + (q * M + m) * kDigitBytesPerTile + lane;
-        p[0] = (unsigned char)z;
-        p[kTileK] = (unsigned char)(z >> 8);
-        p[2 * kTileK] = (unsigned char)(z >> 16);
+#pragma unroll
+        for (int t = 0; t < U; ++t) { // one k per tile and lane
+          const int r = (int)__builtin_rintf(x[m][t][0] * inv[m]);
+          const unsigned z = ((unsigned)r + 0x00808080u) ^ 0x00808080u;
+          unsigned char *p = planes + (t * M + m) * kDigitBytesPerTile + lane;
+          p[0] = (unsigned char)z;
+          p[kTileK] = (unsigned char)(z >> 8);
+          p[2 * kTileK] = (unsigned char)(z >> 16);
+          p[3 * kTileK] = (unsigned char)(z >> 24);
+        }
       }
     }
-  }
-  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-  __builtin_amdgcn_wave_barrier();
-  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  };
+  auto lds_turn = [] { // this wavefront's LDS writes before its LDS reads that follow
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  };
 
-  int s0[M][3], s1[M][3];
+  // ---- the matrix cores: a weight tile as it lies is the A operand (16
+  // channels x 64 k), the 4 M digit planes of the tile are columns of B: column
+  // 4 m + d, lane (k / 16, column) reading 16 bytes.  One instruction per tile
+  // and matrix multiplies every row and digit; the int32 sums stay exact over
+  // the run (at most 16 x 64 products of 2^14).
+  typedef int v4i32 __attribute__((ext_vector_type(4)));
+  constexpr int COLS = kDigits * M;
+  static_assert(COLS <= 16, "the digit planes of all rows are the 16 columns of one B operand");
+  const int col = lane & 15, kq = lane >> 4;
+  const unsigned char *my_b = planes + min(col, COLS - 1) * kTileK + 16 * kq;
+  v4i32 c0 = {0, 0, 0, 0}, c1 = {0, 0, 0, 0}; // HS: c1 collects the pairs' second tiles
+  cut_group(0);
 #pragma unroll
-  for (int m = 0; m < M; ++m)
+  for (int q = 0; q < NG; ++q) {
+    lds_turn();
+    v4i32 b[TG];
 #pragma unroll
-    for (int d = 0; d < 3; ++d) {
-      s0[m][d] = 0;
-      s1[m][d] = 0;
+    for (int t = 0; t < TG; ++t)
+      b[t] = *reinterpret_cast<const v4i32 *>(my_b + t * (M * kDigitBytesPerTile));
+    if (q + 1 < NG) {
+      lds_turn();
+      cut_group(q + 1);
     }
-  const unsigned char *mine_d =
-      planes + 16 * (lane >> 4) + second * (M * kDigitBytesPerTile);
+    if constexpr (HS) {
 #pragma unroll
-  for (int u = 0; u < P; ++u) {
-    if (t0 + (HS ? 2 : 1) * u < t1) {
+      for (int jp = 0; jp < 2; ++jp) { // the pairs 2 q and 2 q + 1
+        const int u = 2 * q + jp;
+        if (u < P) {
+          if (t0 + 2 * u < t1) {
+            const v4i32 wv = {wa[u < P ? u : 0].x, wa[u < P ? u : 0].y, wa[u < P ? u : 0].z,
+                              wa[u < P ? u : 0].w};
+            // rows of the other half of the lanes belong to the pair's second tile
+            c0 = __builtin_amdgcn_mfma_i32_16x16x64_i8(wv, b[2 * jp], c0, 0, 0, 0);
+            c1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(wv, b[2 * jp + 1], c1, 0, 0, 0);
+          }
+        }
+      }
+    } else {
 #pragma unroll
-      for (int m = 0; m < M; ++m) {
-#pragma unroll
-        for (int d = 0; d < 3; ++d) {
-          const int4 xd = *reinterpret_cast<const int4 *>(
-              mine_d + ((HS ? 2 : 1) * u * M + m) * kDigitBytesPerTile + d * kTileK);
-          s0[m][d] = __builtin_amdgcn_sdot4(wa[u].x, xd.x, s0[m][d], false);
-          s0[m][d] = __builtin_amdgcn_sdot4(wa[u].y, xd.y, s0[m][d], false);
-          s0[m][d] = __builtin_amdgcn_sdot4(wa[u].z, xd.z, s0[m][d], false);
-          s0[m][d] = __builtin_amdgcn_sdot4(wa[u].w, xd.w, s0[m][d], false);
-          if (DUAL) {
-            s1[m][d] = __builtin_amdgcn_sdot4(wb[u].x, xd.x, s1[m][d], false);
-            s1[m][d] = __builtin_amdgcn_sdot4(wb[u].y, xd.y, s1[m][d], false);
-            s1[m][d] = __builtin_amdgcn_sdot4(wb[u].z, xd.z, s1[m][d], false);
-            s1[m][d] = __builtin_amdgcn_sdot4(wb[u].w, xd.w, s1[m][d], false);
+      for (int t = 0; t < TG; ++t) {
+        const int u = TG * q + t;
+        if (u < U) {
+          if (t0 + u < t1) {
+            const v4i32 wv = {wa[u < U ? u : 0].x, wa[u < U ? u : 0].y, wa[u < U ? u : 0].z,
+                              wa[u < U ? u : 0].w};
+            c0 = __builtin_amdgcn_mfma_i32_16x16x64_i8(wv, b[t], c0, 0, 0, 0);
+            if (DUAL) {
+              const int ud = DUAL && u < U ? u : 0;
+              const v4i32 wu = {wb[ud].x, wb[ud].y, wb[ud].z, wb[ud].w};
+              c1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(wu, b[t], c1, 0, 0, 0);
+            }
           }
         }
       }
     }
   }
-  float acc0[M], acc1[M];
+  // Lane (kq, col) holds the sums of channels 4 kq + i for its column.  Scale
+  // by the column's step (step of row col / 4 times 256^(col % 4)), then the
+  // four digits of a row, which sit in neighbouring lanes, are added up in the
+  // lane of digit 0.
+  float colscale = 0.f;
 #pragma unroll
   for (int m = 0; m < M; ++m) {
-    // |s[0]|, |s[1]| < 2^22 per lane (at most 16 x 16 products of 2^14): exact
-    const float step65536 = step[m] * 65536.0f;
-    acc0[m] = fmaf((float)s0[m][2], step65536, (float)(s0[m][0] + (s0[m][1] << 8)) * step[m]);
-    acc1[m] = DUAL ? fmaf((float)s1[m][2], step65536,
-                          (float)(s1[m][0] + (s1[m][1] << 8)) * step[m])
-                   : 0.f;
-    // the four rows of a wavefront hold different k sub-ranges of the same
-    // channels (and so do the two halves of a row when tiles go in pairs)
-    if (HS)
-      acc0[m] += dpp_f<0x128>(acc0[m]); // row_ror:8, lane ^ 8
-    acc0[m] = sum_rows(acc0[m]);
-    if (DUAL)
-      acc1[m] = sum_rows(acc1[m]);
+    colscale = col == 4 * m ? step[m] : colscale;
+    colscale = col == 4 * m + 1 ? step[m] * 256.0f : colscale;
+    colscale = col == 4 * m + 2 ? step[m] * 65536.0f : colscale;
+    colscale = col == 4 * m + 3 ? step[m] * 16777216.0f : colscale;
+  }
+  auto digits_sum = [](float v) { // row_shl:1..3: lanes col + 1, col + 2, col + 3
+    return (v + dpp_f<0x101>(v)) + (dpp_f<0x102>(v) + dpp_f<0x103>(v));
+  };
+  float f0[4], f1[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    if (HS) {
+      // channels 8 half + j: row j of the first tiles' product and row 8 + j of
+      // the second tiles' (or the other way round for the other half)
+      const bool first = (kq >> 1) == half;
+      f0[i] = sum_xor<32>(digits_sum((float)(first ? c0[i] : c1[i]) * colscale));
+      f1[i] = 0.f;
+    } else {
+      f0[i] = digits_sum((float)c0[i] * colscale);
+      f1[i] = DUAL ? digits_sum((float)c1[i] * colscale) : 0.f;
+    }
+  }
+#pragma unroll
+  for (int m = 0; m < M; ++m)
     if (NORM)
       ss[m] = wave_sum(ss[m]);
-  }
 
-  // ---- k-slices of one channel group meet in LDS, in slice order ----------
-  if (a.KS > 1) {
+  // ---- hand the sums over in LDS: [row][channel], the layout the k-slices
+  // meet in; lane (kq, 4 m) has row m of channels 4 kq .. 4 kq + 3 -------------
+  float acc0[M], acc1[M];
+  {
     float *mine = lds + (size_t)wave * M * 33;
-    if (lane < kTileN) {
+    const int mrow = col >> 2;
+    if (col < COLS && (col & 3) == 0 && (!HS || kq < 2)) {
+      const int ch = HS ? 8 * half + 4 * kq : 4 * kq;
 #pragma unroll
-      for (int m = 0; m < M; ++m) {
-        mine[m * 33 + lane] = acc0[m];
+      for (int i = 0; i < 4; ++i) {
+        mine[mrow * 33 + ch + i] = f0[i];
         if (DUAL)
-          mine[m * 33 + 16 + lane] = acc1[m];
+          mine[mrow * 33 + 16 + ch + i] = f1[i];
       }
     }
     if (NORM && lane == 0) {
@@ -1211,25 +1270,31 @@ __global__ void __launch_bounds__(kMaxWaves *kWave)
       for (int m = 0; m < M; ++m)
         mine[m * 33 + 32] = ss[m];
     }
+  }
+  if (a.KS > 1) {
     __syncthreads();
     if (ks != 0)
       return;
-    if (lane < kTileN) {
+  } else {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  }
+  if (lane < kTileN) {
 #pragma unroll
-      for (int m = 0; m < M; ++m) {
-        float r0 = 0.f, r1 = 0.f, rs = 0.f;
-        for (int s = 0; s < a.KS; ++s) {
-          const float *o = lds + (size_t)(wave + s) * M * 33 + m * 33;
-          r0 += o[lane];
-          if (DUAL)
-            r1 += o[16 + lane];
-          if (NORM)
-            rs += o[32];
-        }
-        acc0[m] = r0;
-        acc1[m] = r1;
-        ss[m] = rs;
+    for (int m = 0; m < M; ++m) {
+      float r0 = 0.f, r1 = 0.f, rs = 0.f;
+      for (int s = 0; s < a.KS; ++s) {
+        const float *o = lds + (size_t)(wave + s) * M * 33 + m * 33;
+        r0 += o[lane];
+        if (DUAL)
+          r1 += o[16 + lane];
+        if (NORM)
+          rs += o[32];
       }
+      acc0[m] = r0;
+      acc1[m] = r1;
+      ss[m] = rs;
     }
   }
   if (writer) {
@@ -1248,23 +1313,24 @@ __global__ void __launch_bounds__(kMaxWaves *kWave)
   }
 }
 
-BH_VARIANT_FAMILY(RowDot4Family, "gemv_w8a32_dot4_kernel");
+BH_VARIANT_FAMILY(DigitsFamily, "gemv_w8a32_digits_kernel");
 
-constexpr size_t dot4_lds_bytes(int waves, int M, int U) {
-  return sizeof(float) * waves * (size_t)M * 33 + (size_t)waves * U * M * kDigitBytesPerTile;
+// the meeting place of the k-slices and, per wavefront, the planes of four tiles
+constexpr size_t digits_lds_bytes(int waves, int M) {
+  return sizeof(float) * waves * (size_t)M * 33 + (size_t)waves * 4 * M * kDigitBytesPerTile;
 }
 
 template <int M, int EPI, int PRO, int U, bool HS = false>
-int launch_dot4(const KernelArgs &ka, const GemvPlan &p, hipStream_t stream) {
-  BH_NOTE_VARIANT(RowDot4Family, M, EPI, PRO, U, HS ? 1 : 0);
-  auto kernel = gemv_w8a32_dot4_kernel<M, EPI, PRO, U, HS>;
-  const size_t lds = dot4_lds_bytes(p.waves, M, U);
-  if constexpr (dot4_lds_bytes(kMaxWaves, M, U) > 48 * 1024) {
+int launch_digits(const KernelArgs &ka, const GemvPlan &p, hipStream_t stream) {
+  BH_NOTE_VARIANT(DigitsFamily, M, EPI, PRO, U, HS ? 1 : 0);
+  auto kernel = gemv_w8a32_digits_kernel<M, EPI, PRO, U, HS>;
+  const size_t lds = digits_lds_bytes(p.waves, M);
+  if constexpr (digits_lds_bytes(kMaxWaves, M) > 48 * 1024) {
     static bool attr_set = false;
     if (!attr_set) {
       BH_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
                                        hipFuncAttributeMaxDynamicSharedMemorySize,
-                                       (int)dot4_lds_bytes(kMaxWaves, M, U)));
+                                       (int)digits_lds_bytes(kMaxWaves, M)));
       attr_set = true;
     }
   }
@@ -1279,12 +1345,12 @@ constexpr int kNoFit = -1000; // no compiled slot count holds the run
 
 // the smallest compiled slot count that holds `tpw` tiles per wavefront
 template <int M, int EPI, int PRO, bool HS, int... Us>
-int launch_dot4_fit(std::integer_sequence<int, Us...>, int64_t tpw, const KernelArgs &ka,
+int launch_digits_fit(std::integer_sequence<int, Us...>, int64_t tpw, const KernelArgs &ka,
                     const GemvPlan &p, hipStream_t stream) {
   int rc = kNoFit;
   bool done = false;
   ((done || tpw > Us ? 0
-                     : (done = true, rc = launch_dot4<M, EPI, PRO, Us, HS>(ka, p, stream))),
+                     : (done = true, rc = launch_digits<M, EPI, PRO, Us, HS>(ka, p, stream))),
    ...);
   return rc;
 }
@@ -1292,20 +1358,20 @@ int launch_dot4_fit(std::integer_sequence<int, Us...>, int64_t tpw, const Kernel
 // Slot counts compiled per form: dense for one row, where a spare slot is a
 // large part of a short run; coarser for 2 and 4 rows, and only as far as the
 // activations (M per slot) and the weights fit in 128 registers.
-template <int M> struct Dot4Slots { // M = 4
+template <int M> struct DigitSlots { // M = 4
   using Single = std::integer_sequence<int, 2, 3, 4, 6, 8>;
   using Dual = std::integer_sequence<int, 2, 3, 4, 6>;
 };
-template <> struct Dot4Slots<2> {
+template <> struct DigitSlots<2> {
   using Single = std::integer_sequence<int, 2, 3, 4, 6, 8, 10, 12>;
   using Dual = std::integer_sequence<int, 2, 3, 4, 6, 8>;
 };
-template <> struct Dot4Slots<1> {
+template <> struct DigitSlots<1> {
   using Single = std::integer_sequence<int, 2, 3, 4, 5, 6, 7, 8, 9, 10, 12, 14, 16>;
   using Dual = std::integer_sequence<int, 2, 3, 4, 5, 6, 7, 8, 9>;
 };
-using Dot4SlotsSplit = std::integer_sequence<int, 4, 6, 8, 10>;
-using Dot4SlotsFold = std::integer_sequence<int, 2, 3, 4>; // 18 partials per tile in registers
+using DigitSlotsSplit = std::integer_sequence<int, 4, 6, 8, 10>;
+using DigitSlotsFold = std::integer_sequence<int, 2, 3, 4>; // 18 partials per tile in registers
 
 // the slot count a run of `tpw` tiles gets from a list, 0 if none holds it
 template <int... Us> int slots_for(std::integer_sequence<int, Us...>, int64_t tpw) {
@@ -1314,26 +1380,26 @@ template <int... Us> int slots_for(std::integer_sequence<int, Us...>, int64_t tp
   return v;
 }
 
-// Does a plan made for the dot-product kernel have a compiled variant?
-bool dot4_fits(int M, const GemvPlan &p, bool dual, bool fold) {
+// Does a plan made for the digit-plane kernel have a compiled variant?
+bool digits_fit(int M, const GemvPlan &p, bool dual, bool fold) {
   const int64_t tpw = ceil_div(p.chunks, p.KS);
   int u = 0;
   if (p.half_split)
-    u = (dual || fold) ? 0 : slots_for(Dot4SlotsSplit{}, tpw);
+    u = (dual || fold) ? 0 : slots_for(DigitSlotsSplit{}, tpw);
   else if (fold)
-    u = M == 1 ? slots_for(Dot4SlotsFold{}, tpw) : 0;
+    u = M == 1 ? slots_for(DigitSlotsFold{}, tpw) : 0;
   else if (dual)
-    u = M == 1   ? slots_for(Dot4Slots<1>::Dual{}, tpw)
-        : M == 2 ? slots_for(Dot4Slots<2>::Dual{}, tpw)
-                 : slots_for(Dot4Slots<4>::Dual{}, tpw);
+    u = M == 1   ? slots_for(DigitSlots<1>::Dual{}, tpw)
+        : M == 2 ? slots_for(DigitSlots<2>::Dual{}, tpw)
+                 : slots_for(DigitSlots<4>::Dual{}, tpw);
   else
-    u = M == 1   ? slots_for(Dot4Slots<1>::Single{}, tpw)
-        : M == 2 ? slots_for(Dot4Slots<2>::Single{}, tpw)
-                 : slots_for(Dot4Slots<4>::Single{}, tpw);
-  return u != 0 && dot4_lds_bytes(p.waves, M, u) <= kMaxLdsBytes;
+    u = M == 1   ? slots_for(DigitSlots<1>::Single{}, tpw)
+        : M == 2 ? slots_for(DigitSlots<2>::Single{}, tpw)
+                 : slots_for(DigitSlots<4>::Single{}, tpw);
+  return u != 0;
 }
 
-bool row_dot4() {
+bool rows_on_digits() {
   static bool v = [] {
     const char *e = getenv("BUDDY_HIP_GEMV_ROW");
     return !(e && strcmp(e, "f32") == 0);
@@ -1383,26 +1449,26 @@ int launch_one(const KernelArgs &ka, const GemvPlan &p, hipStream_t stream) {
     return launch_tn<kNarrowOk ? 1 : M, kNarrowOk ? EPI : kEpiStore, PRO, 4, kNarrowOk ? 4 : 16>(ka, p, stream);
   }
   if constexpr (M <= 4) {
-    if (p.row_dot4) {
+    if (p.on_digits) {
       // every tile of a wavefront's run is requested at once
       const int64_t tpw = ceil_div(p.chunks, p.KS); // tiles per wavefront
       int rc = kNoFit;
       if (p.half_split) {
         if constexpr (!kDual && PRO != kProAttn)
-          rc = launch_dot4_fit<M, EPI, PRO, true>(Dot4SlotsSplit{}, tpw, ka, p, stream);
+          rc = launch_digits_fit<M, EPI, PRO, true>(DigitSlotsSplit{}, tpw, ka, p, stream);
       } else if constexpr (PRO == kProAttn) {
         if constexpr (M == 1)
-          rc = launch_dot4_fit<1, EPI, PRO, false>(Dot4SlotsFold{}, tpw, ka, p, stream);
+          rc = launch_digits_fit<1, EPI, PRO, false>(DigitSlotsFold{}, tpw, ka, p, stream);
       } else if constexpr (kDual) {
-        rc = launch_dot4_fit<M, EPI, PRO, false>(typename Dot4Slots<M>::Dual{}, tpw, ka, p,
+        rc = launch_digits_fit<M, EPI, PRO, false>(typename DigitSlots<M>::Dual{}, tpw, ka, p,
                                                  stream);
       } else {
-        rc = launch_dot4_fit<M, EPI, PRO, false>(typename Dot4Slots<M>::Single{}, tpw, ka, p,
+        rc = launch_digits_fit<M, EPI, PRO, false>(typename DigitSlots<M>::Single{}, tpw, ka, p,
                                                  stream);
       }
       if (rc != kNoFit)
         return rc;
-      return fail(BUDDY_HIP_ERR_ARG, "gemv: no dot-product variant for %lld tiles per wavefront",
+      return fail(BUDDY_HIP_ERR_ARG, "gemv: no digit-plane variant for %lld tiles per wavefront",
                   (long long)tpw);
     }
   }
@@ -1492,7 +1558,7 @@ int launch_gemv(const GemvArgs &a, hipStream_t stream) {
   const int mt = compiled_rows(a.M);
   BH_REQUIRE(a.tile_n == 16 || a.tile_n == 8 || a.tile_n == 4,
              "gemv: tile_n=%d (16, 8 or 4)", a.tile_n);
-  // Up to four rows go to the dot-product kernel, cut as for one row, when it
+  // Up to four rows go to the digit-plane kernel, cut as for one row, when it
   // has a variant for the run a wavefront gets; otherwise the f32 kernel with
   // its own cut.
   const bool fold = a.attn_acc != nullptr;
@@ -1500,10 +1566,10 @@ int launch_gemv(const GemvArgs &a, hipStream_t stream) {
   // (its activation rows are read as aligned 16-byte pieces)
   const bool rows_aligned =
       fold || ((reinterpret_cast<uintptr_t>(a.A) & 15) == 0 && (a.M == 1 || (a.lda & 3) == 0));
-  if (mt <= 4 && a.tile_n == 16 && rows_aligned && row_dot4()) {
+  if (mt <= 4 && a.tile_n == 16 && rows_aligned && rows_on_digits()) {
     GemvPlan q = make_plan(1, a.K, a.N, dual, a.tile_n, fold);
-    if (dot4_fits(mt, q, dual, fold)) {
-      q.row_dot4 = true;
+    if (digits_fit(mt, q, dual, fold)) {
+      q.on_digits = true;
       p = q;
     }
   }

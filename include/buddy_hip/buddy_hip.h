@@ -114,12 +114,14 @@ int buddy_hip_gemv_w4a16(const uint16_t *A, const int8_t *packed, const uint16_t
  * :250-321 generates:  C[m,n] (+)= (sum_k A[m,k] * W[k,n]) * scale[n].
  * M is 1..16 (the reference pattern is m == 1 only; M > 1 streams the weights
  * once for all rows).  A: f32 [M,K] row-major (lda = K), C: f32 [M,N].
- * One row, with at most 16 tiles of 64 k per wavefront (every matrix of a
- * decoder layer), runs on the integer dot product: a wavefront rounds the
- * 64..1024 activations it multiplies to 2^-23 of the largest of them, the
- * sums are exact, and a NaN or an infinity turns C into NaN; the environment
- * variable BUDDY_HIP_GEMV_ROW=f32, read once per process, keeps the f32
- * multiply-add kernel instead.  Longer runs and 2 to 4 rows: every product is
+ * Up to 4 rows, with at most 16 tiles of 64 k per wavefront (every matrix of a
+ * decoder layer) and 16-byte aligned rows, run on the int8 matrix cores: a
+ * wavefront rounds the 64..1024 activations of a row it multiplies to 2^-31 of
+ * the largest of them (one within 2^7 of it keeps all 24 bits), the products
+ * and sums are exact, and a NaN or an infinity turns the
+ * row of C into NaN; the environment variable BUDDY_HIP_GEMV_ROW=f32, read once
+ * per process, keeps the f32 multiply-add kernel instead.  Longer runs and
+ * unaligned rows: every product is
  * an f32 multiply-add.  From 5 rows (with K a
  * multiple of 4 and A 16-byte aligned) the int8 matrix cores are used: the
  * activations of a row are rounded, 64 at a time, to 2^-23 of the largest of

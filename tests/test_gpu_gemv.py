@@ -213,12 +213,13 @@ def test_gemv_bf16_batch_kernel_matches_oracle(oracle, bf16_batch_kernel, K, N, 
 
 
 def test_row_kernel_fixed_point_keeps_f32_accuracy():
-    """One row goes through the integer dot product: every wavefront turns its
-    own run of the row (here 1536 / 8 = 192 values) into 23-bit fixed point with
+    """One row goes through the int8 matrix cores: every wavefront turns its
+    own run of the row (here 1536 / 8 = 192 values) into 31-bit fixed point with
     a step of its own.  Rows of any magnitude, a loud run next to quiet ones and
     a zero row each agree with a float64 sum to f32 accuracy; inside a run, a
-    value 2^-23 of the run's largest and below is rounded away, which the
-    comparison allows for through the run's largest value."""
+    value keeps all its bits down to 2^-7 of the run's largest and is rounded
+    to 2^-31 of that largest below, which the comparison allows for through the
+    run's largest value."""
     K, N = 1536, 4096
     q, s = ops.quantize_w8(make_weight(K, N, 79))
     packed = ops.pack_w8(q)
@@ -243,14 +244,41 @@ def test_row_kernel_fixed_point_keeps_f32_accuracy():
     quiet[192:384] = 0.0
     y = ops.gemv_w8a32(torch.from_numpy(quiet[None]).cuda(), packed, s, K, N).cpu().numpy()[0]
     check_close(y, (quiet.astype(np.float64) @ qh) * sh)
-    # an outlier inside a run costs that run's other values its resolution and
-    # nothing more: the error stays below 2^-22 of the outlier times sum |w|
+    # an outlier inside a run costs that run's other values resolution below
+    # 2^-31 of the outlier and nothing more: the error stays below 2^-30 of the
+    # outlier times sum |w| (plus the rounding of the f32 results)
     out = base.copy()
     out[200] = np.float32(3e4)
     y = ops.gemv_w8a32(torch.from_numpy(out[None]).cuda(), packed, s, K, N).cpu().numpy()[0]
     want = (out.astype(np.float64) @ qh) * sh
-    bound = 2.0 ** -22 * 3e4 * np.abs(qh[192:384]).sum(0) * sh + 1e-6 * np.abs(want).max()
+    bound = 2.0 ** -30 * 3e4 * np.abs(qh[192:384]).sum(0) * sh + 1e-6 * np.abs(want).max()
     assert (np.abs(y - want) <= bound).all()
+
+
+def test_row_kernel_steps_are_per_row():
+    """Four rows in one launch, 40 orders of magnitude apart and one of them
+    zero: every row has its own fixed-point step, so each keeps f32 accuracy;
+    a NaN in one row leaves the others alone."""
+    K, N = 1536, 4096
+    q, s = ops.quantize_w8(make_weight(K, N, 81))
+    packed = ops.pack_w8(q)
+    qh, sh = q.cpu().numpy().astype(np.float64), s.cpu().numpy().astype(np.float64)
+    rng = np.random.default_rng(9)
+    xh = rng.standard_normal((4, K)).astype(np.float32)
+    xh[1] *= np.float32(1e20)
+    xh[2] *= np.float32(1e-20)
+    xh[3] = 0.0
+    y = ops.gemv_w8a32(torch.from_numpy(xh).cuda(), packed, s, K, N).cpu().numpy()
+    want = (xh.astype(np.float64) @ qh) * sh
+    for m in range(3):
+        check_close(y[m], want[m])
+    assert not y[3].any()
+    xh[1, 5] = np.nan
+    y = ops.gemv_w8a32(torch.from_numpy(xh).cuda(), packed, s, K, N).cpu().numpy()
+    assert np.isnan(y[1]).all()
+    check_close(y[0], want[0])
+    check_close(y[2], want[2])
+    assert not y[3].any()
 
 
 def test_row_kernel_shows_non_finite_activations():

@@ -1,5 +1,5 @@
 """Every compiled variant of the kernels that issue their global loads by hand,
-and of the one-row GEMV with its many slot counts, meets the oracle.
+and of the one-to-four-row GEMV with its many slot counts, meets the oracle.
 
 The first (the int8 and bf16 matrix-core kernels of the small-batch GEMV and of
 the prefill matmul, and the prefill attention) wait for their loads by
@@ -107,7 +107,7 @@ def test_every_bf16_batch_gemv_variant(bh, oracle):
     assert launched(bh, fam) == compiled(bh, fam), compiled(bh, fam) - launched(bh, fam)
 
 
-# ---- GEMV of up to four rows on the integer dot product: <rows, epilogue, input,
+# ---- GEMV of up to four rows over digit planes on the matrix cores: <rows, epilogue, input,
 # tile slots per wavefront, channel group split over two workgroups> ---------------
 # With more than 128 channel groups a wavefront gets ceil(K / 64 / 16) tiles (16
 # k-slices) once K >= 4096, and K = 128, 192 give runs of 2 and 3; with 4 channel
@@ -152,7 +152,7 @@ def test_every_row_gemv_variant(bh, oracle):
             check_close(logits, ologits)
             assert nxt == tok
         sess.close()
-    fam = "gemv_w8a32_dot4_kernel"
+    fam = "gemv_w8a32_digits_kernel"
     assert launched(bh, fam) == compiled(bh, fam), compiled(bh, fam) - launched(bh, fam)
 
 
@@ -211,5 +211,5 @@ def test_prefill_attention_and_no_unlisted_family(bh, oracle):
     # every family the library lists is one of those this file drives
     known = ("gemv_w8a32_i8_kernel", "gemv_w8a32_mfma_kernel", "gemm_w8_i8_wide_kernel",
              "gemm_w8_i8_kernel", "gemm_w8_bf16_wide_kernel", "gemm_w8_bf16_kernel",
-             "attn_prefill_kernel", "gemv_w8a32_dot4_kernel")
+             "attn_prefill_kernel", "gemv_w8a32_digits_kernel")
     assert {name.split("<")[0] for name in report(bh)} == set(known)
