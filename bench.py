@@ -40,11 +40,13 @@ GATE_UP_KERNEL = "gemv_w8a32_digits_kernel<1, 2, 1, 3, false>"
 TRAFFIC_PROFILE = "profiles/decode_kernels_hbm_traffic.md"
 
 
-def gate_up_traffic():
+def gate_up_traffic(collecting: bool = False):
     """HBM bytes per launch of the dominant kernel as the counter summary under
     profiles/ records them (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by a
     copy of known size): a counter reading, not something this script can
-    measure live.  A summary that was taken for another kernel gives no figure."""
+    measure live.  A summary that was taken for another kernel is refused --
+    except in the run that collects the counters for a new one (`collecting`,
+    the --calibrate-copy form), which reports no figure instead."""
     import re
 
     path = ROOT / TRAFFIC_PROFILE
@@ -54,9 +56,12 @@ def gate_up_traffic():
                   path.read_text(), re.S)
     if not m:
         raise SystemExit(f"bench.py: no per-launch traffic line in {TRAFFIC_PROFILE}")
-    if m.group(1) != GATE_UP_KERNEL:  # counters of another kernel are not this one's traffic
-        return None, (f"{TRAFFIC_PROFILE} holds the counters of `{m.group(1)}`, not of the "
-                      f"dominant kernel: take them again")
+    if m.group(1) != GATE_UP_KERNEL:
+        why = (f"{TRAFFIC_PROFILE} holds the counters of `{m.group(1)}`, but the dominant "
+               f"kernel is `{GATE_UP_KERNEL}`: take the counters again")
+        if not collecting:
+            raise SystemExit("bench.py: " + why)
+        return None, why
     return int(m.group(2).replace(",", "")), TRAFFIC_PROFILE
 
 
@@ -880,7 +885,7 @@ def main():
     gu_b = gate_up_bytes(shape.hidden, shape.inter)
     achieved = gu_b / gu_s / 1e9
     step_b = decode_step_bytes(shape, CONTEXT + W + K // 2)
-    traffic, traffic_source = gate_up_traffic()
+    traffic, traffic_source = gate_up_traffic(collecting=args.calibrate_copy)
 
     out = {
         "metric": "decode_tokens_per_s",
