@@ -995,7 +995,9 @@ __global__ void __launch_bounds__(kMaxWaves *kWave)
   constexpr int XE = VEC ? 4 : 1;           // values per slot
   float x[M][XV][XE], nw[XV][XE];
   if constexpr (VEC) {
-    const int klast = ((a.K + 3) & ~3) - 4;
+    // lanes past the run repeat its last 16 bytes (a line this wavefront reads
+    // anyway, not one that every wavefront of the launch would share)
+    const int klast = max(min(((a.K + 3) & ~3), t1 * kTileK) - 4, 0);
 #pragma unroll
     for (int q = 0; q < XV; ++q) {
       const int kc = min(t0 * kTileK + q * 256 + 4 * lane, klast);
