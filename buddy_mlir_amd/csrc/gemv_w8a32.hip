@@ -1382,23 +1382,11 @@ template <int... Us> int slots_for(std::integer_sequence<int, Us...>, int64_t tp
   return v;
 }
 
+int digit_slots(int M, const GemvPlan &p, bool dual, bool fold);
+
 // Does a plan made for the digit-plane kernel have a compiled variant?
 bool digits_fit(int M, const GemvPlan &p, bool dual, bool fold) {
-  const int64_t tpw = ceil_div(p.chunks, p.KS);
-  int u = 0;
-  if (p.half_split)
-    u = (dual || fold) ? 0 : slots_for(DigitSlotsSplit{}, tpw);
-  else if (fold)
-    u = M == 1 ? slots_for(DigitSlotsFold{}, tpw) : 0;
-  else if (dual)
-    u = M == 1   ? slots_for(DigitSlots<1>::Dual{}, tpw)
-        : M == 2 ? slots_for(DigitSlots<2>::Dual{}, tpw)
-                 : slots_for(DigitSlots<4>::Dual{}, tpw);
-  else
-    u = M == 1   ? slots_for(DigitSlots<1>::Single{}, tpw)
-        : M == 2 ? slots_for(DigitSlots<2>::Single{}, tpw)
-                 : slots_for(DigitSlots<4>::Single{}, tpw);
-  return u != 0;
+  return digit_slots(M, p, dual, fold) != 0;
 }
 
 bool rows_on_digits() {
@@ -1517,6 +1505,38 @@ bool batch_bf16() {
   }
   return k == 1;
 }
+// The cut of a launch of up to four rows (or of the f32 kernel for more): the
+// digit-plane kernel, cut as for one row, when it has a variant for the run a
+// wavefront gets; otherwise the f32 kernel with its own cut.
+GemvPlan choose_plan(int mt, int64_t K, int64_t N, bool dual, int tile_n, bool fold,
+                     bool rows_aligned) {
+  GemvPlan p = make_plan(mt, K, N, dual, tile_n, fold);
+  if (mt <= 4 && tile_n == 16 && rows_aligned && rows_on_digits()) {
+    GemvPlan q = make_plan(1, K, N, dual, tile_n, fold);
+    if (digits_fit(mt, q, dual, fold)) {
+      q.on_digits = true;
+      p = q;
+    }
+  }
+  return p;
+}
+
+// the slot count the digit-plane kernel is launched with for a plan, 0 if none
+int digit_slots(int M, const GemvPlan &p, bool dual, bool fold) {
+  const int64_t tpw = ceil_div(p.chunks, p.KS);
+  if (p.half_split)
+    return (dual || fold) ? 0 : slots_for(DigitSlotsSplit{}, tpw);
+  if (fold)
+    return M == 1 ? slots_for(DigitSlotsFold{}, tpw) : 0;
+  if (dual)
+    return M == 1   ? slots_for(DigitSlots<1>::Dual{}, tpw)
+           : M == 2 ? slots_for(DigitSlots<2>::Dual{}, tpw)
+                    : slots_for(DigitSlots<4>::Dual{}, tpw);
+  return M == 1   ? slots_for(DigitSlots<1>::Single{}, tpw)
+         : M == 2 ? slots_for(DigitSlots<2>::Single{}, tpw)
+                  : slots_for(DigitSlots<4>::Single{}, tpw);
+}
+
 bool force_valu() {
   static bool v = getenv("BUDDY_HIP_GEMV_FORCE_VALU") != nullptr;
   return v;
@@ -1560,21 +1580,11 @@ int launch_gemv(const GemvArgs &a, hipStream_t stream) {
   const int mt = compiled_rows(a.M);
   BH_REQUIRE(a.tile_n == 16 || a.tile_n == 8 || a.tile_n == 4,
              "gemv: tile_n=%d (16, 8 or 4)", a.tile_n);
-  // Up to four rows go to the digit-plane kernel, cut as for one row, when it
-  // has a variant for the run a wavefront gets; otherwise the f32 kernel with
-  // its own cut.
   const bool fold = a.attn_acc != nullptr;
-  GemvPlan p = make_plan(mt, a.K, a.N, dual, a.tile_n, fold);
   // (its activation rows are read as aligned 16-byte pieces)
   const bool rows_aligned =
       fold || ((reinterpret_cast<uintptr_t>(a.A) & 15) == 0 && (a.M == 1 || (a.lda & 3) == 0));
-  if (mt <= 4 && a.tile_n == 16 && rows_aligned && rows_on_digits()) {
-    GemvPlan q = make_plan(1, a.K, a.N, dual, a.tile_n, fold);
-    if (digits_fit(mt, q, dual, fold)) {
-      q.on_digits = true;
-      p = q;
-    }
-  }
+  const GemvPlan p = choose_plan(mt, a.K, a.N, dual, a.tile_n, fold, rows_aligned);
   KernelArgs ka;
   ka.A = a.A;
   ka.W0 = reinterpret_cast<const int4 *>(a.W0);
@@ -1623,6 +1633,39 @@ int buddy_hip_set_gemv_batch_kernel(int kernel) try {
   bh::g_batch_kernel.store(kernel, std::memory_order_relaxed);
   return BUDDY_HIP_OK;
 } BH_CATCH_INT("buddy_hip_set_gemv_batch_kernel")
+
+int buddy_hip_gemv_w8a32_plan(int64_t M, int64_t K, int64_t N, unsigned flags,
+                              buddy_hip_gemv_plan *out) try {
+  BH_REQUIRE(out, "gemv_w8a32_plan: null result");
+  BH_REQUIRE(M >= 1 && M <= 16, "gemv_w8a32_plan: M=%lld outside 1..16", (long long)M);
+  BH_REQUIRE(K > 0 && N > 0 && K < (1 << 30) && N < (1 << 30),
+             "gemv_w8a32_plan: bad shape K=%lld N=%lld", (long long)K, (long long)N);
+  const bool dual = flags & BUDDY_HIP_PLAN_TWO_MATRICES, fold = flags & BUDDY_HIP_PLAN_FOLD_INPUT;
+  BH_REQUIRE(!(fold && (M != 1 || dual)), "gemv_w8a32_plan: folded input is one row, one matrix");
+  *out = buddy_hip_gemv_plan{};
+  const bool aligned = !(flags & BUDDY_HIP_PLAN_UNALIGNED_ROWS);
+  if (M >= 5 && !fold && !bh::force_valu() && (K & 3) == 0 && aligned) {
+    out->kernel = bh::batch_bf16() ? BUDDY_HIP_PLAN_BATCH_BF16 : BUDDY_HIP_PLAN_BATCH_INT8;
+    out->rows_compiled = 16;
+    return BUDDY_HIP_OK; // those kernels cut their launch by what the device holds
+  }
+  const int mt = bh::compiled_rows(M);
+  const bh::GemvPlan p = bh::choose_plan(mt, K, N, dual, 16, fold, aligned);
+  out->kernel = p.on_digits ? BUDDY_HIP_PLAN_DIGITS : BUDDY_HIP_PLAN_F32;
+  out->rows_compiled = mt;
+  out->channel_groups = (int32_t)p.groups;
+  out->tiles = (int32_t)p.chunks;
+  out->groups_per_workgroup = p.G;
+  out->k_slices = p.KS;
+  out->wavefronts = p.waves;
+  out->workgroups = p.blocks << p.half_split;
+  out->split = p.half_split;
+  out->tiles_per_wavefront = (int32_t)bh::ceil_div(p.chunks, p.KS);
+  out->slots = p.on_digits ? bh::digit_slots(mt, p, dual, fold) : 0;
+  out->lds_bytes = p.on_digits ? (int64_t)bh::digits_lds_bytes(p.waves, mt)
+                               : (int64_t)(sizeof(float) * p.waves * (size_t)mt * 33);
+  return BUDDY_HIP_OK;
+} BH_CATCH_INT("buddy_hip_gemv_w8a32_plan")
 
 int buddy_hip_linear_w8a32(const buddy_hip_linear_desc *d,
                            buddy_hip_stream stream) try {

@@ -139,6 +139,40 @@ enum {
                                    without it C = ... and C need not be
                                    initialised */
 };
+/* How a launch of buddy_hip_gemv_w8a32 / buddy_hip_linear_w8a32 would be cut:
+ * host arithmetic only, nothing is launched and no device is touched.  For
+ * tests of the launch shapes, and for callers that want to know which kernel a
+ * shape gets.  (No counterpart in the reference, whose loop nest is fixed at
+ * compile time.) */
+enum {
+  BUDDY_HIP_PLAN_TWO_MATRICES = 1,   /* the SiLU(gate) * up form */
+  BUDDY_HIP_PLAN_FOLD_INPUT = 2,     /* input folded from attention partials */
+  BUDDY_HIP_PLAN_UNALIGNED_ROWS = 4  /* A or lda not a multiple of 16 bytes */
+};
+enum {
+  BUDDY_HIP_PLAN_DIGITS = 0,     /* digit planes on the int8 matrix cores, 1..4 rows */
+  BUDDY_HIP_PLAN_F32 = 1,        /* f32 multiply-add kernel */
+  BUDDY_HIP_PLAN_BATCH_INT8 = 2, /* 5..16 rows, int8 matrix cores */
+  BUDDY_HIP_PLAN_BATCH_BF16 = 3  /* 5..16 rows, bf16 matrix cores */
+};
+typedef struct {
+  int32_t kernel;               /* BUDDY_HIP_PLAN_* */
+  int32_t rows_compiled;        /* rows the kernel variant is compiled for */
+  int32_t channel_groups;       /* ceil(N / 16) */
+  int32_t tiles;                /* ceil(K / 64): 1 KiB tiles per channel group */
+  int32_t groups_per_workgroup; /* channel groups a workgroup covers */
+  int32_t k_slices;             /* wavefronts that share one channel group */
+  int32_t wavefronts;           /* per workgroup */
+  int32_t workgroups;
+  int32_t split;                /* 1: two workgroups per channel group */
+  int32_t tiles_per_wavefront;
+  int32_t slots;                /* tile slots of the digit-plane variant, else 0 */
+  int32_t reserved;
+  int64_t lds_bytes;            /* dynamic LDS of one workgroup */
+} buddy_hip_gemv_plan;
+int buddy_hip_gemv_w8a32_plan(int64_t M, int64_t K, int64_t N, unsigned flags,
+                              buddy_hip_gemv_plan *out);
+
 int buddy_hip_gemv_w8a32(const float *A, const int8_t *packed,
                          const float *scale, float *C, int64_t M, int64_t K,
                          int64_t N, unsigned flags, buddy_hip_stream stream);
