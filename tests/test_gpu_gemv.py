@@ -89,7 +89,7 @@ def test_narrow_tile_layouts(oracle, K, N, tn):
 # (102, 70): K % 4 != 0 keeps every batch size on the f32 FMA kernel; (100, 70)
 # and (1100, 40) end a row inside a 16-k run of the matrix-core kernel
 SHAPES = [(1536, 8960), (8960, 1536), (1536, 1536), (1536, 256), (64, 16), (100, 70),
-          (102, 70), (1100, 40), (1536, 151936), (4096, 4096)]
+          (102, 70), (1100, 40), (1536, 151936), (4096, 4096), (1, 1), (3, 17), (5, 33)]
 
 
 @pytest.mark.parametrize("K,N", SHAPES)
