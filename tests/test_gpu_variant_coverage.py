@@ -156,6 +156,20 @@ def test_every_row_gemv_variant(bh, oracle):
     assert launched(bh, fam) == compiled(bh, fam), compiled(bh, fam) - launched(bh, fam)
 
 
+def test_row_gemv_random_shapes(bh, oracle):
+    """120 seeded random shapes, row counts and fused forms through whatever
+    kernel the launch's cut picks (ragged K and N, rows whose length is not a
+    multiple of four, narrow long matrices that are split over two workgroups)."""
+    rng = np.random.default_rng(2024)
+    for case in range(120):
+        K = int(rng.choice([rng.integers(1, 300), rng.integers(300, 12000)]))
+        N = int(rng.choice([rng.integers(1, 200), rng.integers(200, 3000)]))
+        M = int(rng.integers(1, 5))
+        epilogue = int(rng.integers(0, 3))
+        norm = bool(rng.integers(0, 2))
+        gemv_case(bh, oracle, M, K, N, epilogue, norm, 1000 + case)
+
+
 # ---- prefill matmul: the tile shape comes out of the launch's cost model -------
 GEMM_I8_SHAPES = [(144, 256, 16384), (300, 256, 10240), (200, 192, 16384), (512, 192, 8960),
                   (17, 64, 64)]
