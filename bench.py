@@ -370,7 +370,8 @@ def bench_mlp(bh, args):
             f1(i)
             f2(i)
         t = _time_launches(fn, 480)
-        by = 3 * H * I + 4 * (2 * I + H) + 4 * M * 2 * H  # the survey's formula
+        # three int8 matrices, their scales, M rows in and M rows out
+        by = 3 * H * I + 4 * (2 * I + H) + 4 * M * 2 * H
         res[f"M={M}"] = {"us": t * 1e6, "gbps": by / t / 1e9,
                          "frac": by / t / 1e9 / HBM_PEAK_GBPS}
     t = res["M=1"]["us"] * 1e-6
