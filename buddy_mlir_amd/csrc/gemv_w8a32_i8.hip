@@ -564,6 +564,16 @@ int launch_gemv_i8(const GemvArgs &a, hipStream_t stream) {
     span = 4;
   else if (ka.groups >= 2 * 256)
     span = 2;
+  // Between 257 and 1024 channel groups: the fewest groups per wavefront that
+  // bring the launch down to one workgroup of 8 k-slices per compute unit (all
+  // of them resident at once) beat more, shorter workgroups (4096 -> 6144 at 8
+  // rows: 13.5 us as 384 workgroups of 4 wavefronts, 10.3 us as 192 of 8).
+  if (ka.groups > 256 && ka.chunks >= 2 * kMaxWavesI8) {
+    if (ka.groups <= 2 * 256)
+      span = 2;
+    else if (!dual && ka.groups <= 4 * 256)
+      span = 4;
+  }
   ka.spans = (int)ceil_div(ka.groups, span);
   int ks_forced = 0;
   if (const char *e = getenv("BUDDY_HIP_I8_PLAN")) { // measurement only: "span,ks"
