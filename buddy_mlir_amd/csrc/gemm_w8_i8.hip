@@ -89,8 +89,8 @@ struct SiluMulRow { // silu(g) * u
     load4(g, k0, n, gv);
     load4(u, k0, n, uv);
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      const float sig = 1.0f / (1.0f + expf(-gv[e]));
+    for (int e = 0; e < 4; ++e) { // one-instruction exp and reciprocal (1 ulp each)
+      const float sig = fast_rcp(1.0f + fast_exp(-gv[e]));
       v[e] = (gv[e] * sig) * uv[e];
     }
   }
@@ -100,7 +100,9 @@ struct SiluMulRow { // silu(g) * u
 // row maximum and the pass that writes the digits; longer rows are computed twice.
 constexpr int kRowCache = 12288;
 
-// One workgroup of 256 threads writes row `row` of every plane and its step.
+constexpr int kRowThreads = 512; // threads of a producer workgroup (one row)
+
+// One workgroup of kRowThreads threads writes row `row` of every plane and its step.
 // A thread owns the same groups of four values in both passes.
 template <class F>
 __device__ __forceinline__ void row_to_digits(const F &f, int n, int row, int D, int Mp,
@@ -108,7 +110,8 @@ __device__ __forceinline__ void row_to_digits(const F &f, int n, int row, int D,
                                               float *cache) {
   const bool cached = Kp <= kRowCache;
   float mx = 0.f;
-  for (int k0 = threadIdx.x * 4; k0 < Kp; k0 += 256 * 4) {
+#pragma unroll 3
+  for (int k0 = threadIdx.x * 4; k0 < Kp; k0 += kRowThreads * 4) {
     float v[4];
     f(k0, v);
     mx = fmaxf(fmaxf(mx, fmaxf(fabsf(v[0]), fabsf(v[1]))), fmaxf(fabsf(v[2]), fabsf(v[3])));
@@ -120,14 +123,20 @@ __device__ __forceinline__ void row_to_digits(const F &f, int n, int row, int D,
   if ((threadIdx.x & 63) == 0)
     red[threadIdx.x >> 6] = mx;
   __syncthreads();
-  mx = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+  {
+    float m2 = red[0];
+#pragma unroll
+    for (int w = 1; w < kRowThreads / 64; ++w)
+      m2 = fmaxf(m2, red[w]);
+    mx = m2;
+  }
   const float step = digit_step(mx, D);
   const float inv = 1.0f / step; // a power of two as well
   float *steps = reinterpret_cast<float *>(planes + (size_t)D * Mp * Kp);
   if (threadIdx.x == 0)
     steps[row] = step;
   const size_t plane = (size_t)Mp * Kp;
-  for (int k0 = threadIdx.x * 4; k0 < Kp; k0 += 256 * 4) {
+  for (int k0 = threadIdx.x * 4; k0 < Kp; k0 += kRowThreads * 4) {
     float v[4];
     if (cached) {
       const float4 q = *reinterpret_cast<const float4 *>(cache + k0);
@@ -154,15 +163,15 @@ __device__ __forceinline__ void row_to_digits(const F &f, int n, int row, int D,
   }
 }
 
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(kRowThreads)
 activations_to_digits_kernel(const float *__restrict__ A, int64_t lda, int M, int K, int D,
                              int Mp, int Kp, int8_t *__restrict__ planes) {
-  __shared__ float red[4];
+  __shared__ float red[kRowThreads / 64];
   extern __shared__ __attribute__((aligned(16))) float row_cache[];
   const int row = blockIdx.x;
   if (row >= M) { // padding rows: zero digits, step 1
     for (int j = 0; j < D; ++j)
-      for (int k0 = threadIdx.x * 4; k0 < Kp; k0 += 256 * 4)
+      for (int k0 = threadIdx.x * 4; k0 < Kp; k0 += kRowThreads * 4)
         *reinterpret_cast<unsigned *>(planes + ((size_t)j * Mp + row) * Kp + k0) = 0u;
     if (threadIdx.x == 0)
       reinterpret_cast<float *>(planes + (size_t)D * Mp * Kp)[row] = 1.0f;
@@ -172,30 +181,33 @@ activations_to_digits_kernel(const float *__restrict__ A, int64_t lda, int M, in
                 row_cache);
 }
 
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(kRowThreads)
 rmsnorm_to_digits_kernel(const float *__restrict__ x, int64_t ldx,
                          const float *__restrict__ w, int n, float inv_n, float eps, int D,
                          int Mp, int Kp, int8_t *__restrict__ planes) {
-  __shared__ float red[4];
+  __shared__ float red[kRowThreads / 64];
   extern __shared__ __attribute__((aligned(16))) float row_cache[];
   const int row = blockIdx.x;
   const float *xr = x + (int64_t)row * ldx;
   float s = 0.f;
-  for (int i = threadIdx.x; i < n; i += 256)
+  for (int i = threadIdx.x; i < n; i += kRowThreads)
     s = fmaf(xr[i], xr[i], s);
   s = wave_sum(s);
   if ((threadIdx.x & 63) == 0)
     red[threadIdx.x >> 6] = s;
   __syncthreads();
-  const float tot = (red[0] + red[1]) + (red[2] + red[3]);
+  float tot = 0.f;
+#pragma unroll
+  for (int w = 0; w < kRowThreads / 64; w += 2) // pairs first, as four wavefronts did
+    tot += red[w] + red[w + 1];
   const float rs = 1.0f / sqrtf(tot * inv_n + eps);
   row_to_digits(NormRow{xr, w, rs, n}, n, row, D, Mp, Kp, planes, red, row_cache);
 }
 
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(kRowThreads)
 silu_mul_to_digits_kernel(const float *__restrict__ g, const float *__restrict__ u, int64_t ld,
                           int n, int D, int Mp, int Kp, int8_t *__restrict__ planes) {
-  __shared__ float red[4];
+  __shared__ float red[kRowThreads / 64];
   extern __shared__ __attribute__((aligned(16))) float row_cache[];
   const int row = blockIdx.x;
   row_to_digits(SiluMulRow{g + (size_t)row * ld, u + (size_t)row * ld, n}, n, row, D, Mp, Kp,
@@ -682,7 +694,7 @@ int launch_activations_to_digits(const float *A, int64_t lda, int64_t M, int64_t
   BH_REQUIRE(A && staged && M > 0 && K > 0 && digits >= 2 && digits <= 3 && lda >= K,
              "activations_to_digits: bad argument");
   const GemmStagingLayout l = gemm_staging_layout(M, K);
-  hipLaunchKernelGGL(activations_to_digits_kernel, dim3((unsigned)l.rows_padded), dim3(256),
+  hipLaunchKernelGGL(activations_to_digits_kernel, dim3((unsigned)l.rows_padded), dim3(kRowThreads),
                      row_cache_bytes(l.cols_padded), stream, A, lda, (int)M, (int)K, digits, l.rows_padded,
                      l.cols_padded, static_cast<int8_t *>(staged));
   BH_CHECK_HIP(hipGetLastError());
@@ -694,7 +706,7 @@ int launch_rmsnorm_to_digits(const float *x, int64_t ldx, const float *w, int ro
   BH_REQUIRE(x && w && staged && rows > 0 && n > 0 && ldx >= n && digits >= 2 && digits <= 3,
              "rmsnorm_to_digits: bad argument");
   const GemmStagingLayout l = gemm_staging_layout(rows, n);
-  hipLaunchKernelGGL(rmsnorm_to_digits_kernel, dim3(rows), dim3(256),
+  hipLaunchKernelGGL(rmsnorm_to_digits_kernel, dim3(rows), dim3(kRowThreads),
                      row_cache_bytes(l.cols_padded), stream, x, ldx, w, n,
                      1.0f / (float)n, eps, digits, l.rows_padded, l.cols_padded,
                      static_cast<int8_t *>(staged));
@@ -707,7 +719,7 @@ int launch_silu_mul_to_digits(const float *g, const float *u, int64_t ld, int ro
   BH_REQUIRE(g && u && staged && rows > 0 && n > 0 && ld >= n && digits >= 2 && digits <= 3,
              "silu_mul_to_digits: bad argument");
   const GemmStagingLayout l = gemm_staging_layout(rows, n);
-  hipLaunchKernelGGL(silu_mul_to_digits_kernel, dim3(rows), dim3(256),
+  hipLaunchKernelGGL(silu_mul_to_digits_kernel, dim3(rows), dim3(kRowThreads),
                      row_cache_bytes(l.cols_padded), stream, g, u, ld, n,
                      digits, l.rows_padded, l.cols_padded, static_cast<int8_t *>(staged));
   BH_CHECK_HIP(hipGetLastError());
