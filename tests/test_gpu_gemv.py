@@ -281,6 +281,33 @@ def test_row_kernel_steps_are_per_row():
     assert not y[3].any()
 
 
+@pytest.mark.parametrize("M", [1, 3, 4])
+@pytest.mark.parametrize("shift", [0, 1])
+def test_row_kernel_strided_and_unaligned_rows(oracle, M, shift):
+    """Rows with a stride beyond their length and an output with a stride of its
+    own; with `shift` the first row starts 4 bytes off a 16-byte boundary, which
+    sends the launch to the f32 kernel (the matrix-core kernel reads 16-byte
+    pieces of the rows)."""
+    K, N, lda, ldc = 1536, 272, 1536 + 12, 272 + 5
+    q, s = ops.quantize_w8(make_weight(K, N, 82))
+    packed = ops.pack_w8(q)
+    g = torch.Generator(device="cuda").manual_seed(83 + M)
+    buf = torch.randn((M * lda + 4,), generator=g, device="cuda")
+    out = torch.full((M * ldc,), 7.0, device="cuda")
+    a = buf[shift:]
+    torch.cuda.synchronize()
+    ops.linear_w8a32(A=a.data_ptr(), lda=lda, W0=packed, scale0=s, C=out, ldc=ldc, M=M, K=K, N=N,
+                     epilogue=0)
+    torch.cuda.synchronize()
+    ah = a.cpu().numpy()
+    oh = out.cpu().numpy()
+    qh, sh = q.cpu().numpy(), s.cpu().numpy()
+    for m in range(M):
+        check_close(oh[m * ldc:m * ldc + N], oracle.dequant_gemv(ah[m * lda:m * lda + K], qh, sh))
+        if m + 1 < M:  # the gap between output rows is left alone
+            assert (oh[m * ldc + N:(m + 1) * ldc] == 7.0).all()
+
+
 def test_row_kernel_shows_non_finite_activations():
     """A NaN or an infinity in the row gives NaN results (the f32 product would
     give NaN or infinity there)."""
