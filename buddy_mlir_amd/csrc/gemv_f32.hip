@@ -27,8 +27,28 @@
 namespace bh {
 namespace {
 
+typedef float v4f __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ float4 load_stream4(const float *p) {
+  const v4f v = __builtin_nontemporal_load(reinterpret_cast<const v4f *>(p));
+  return make_float4(v.x, v.y, v.z, v.w);
+}
+
+// Sum over the lanes S, 2 S, ... 32 apart (S a power of two: lanes that are equal
+// modulo S stay apart): DPP inside a row of 16 lanes, lane swaps across rows, no
+// trip through LDS.
+template <int S> __device__ __forceinline__ float sum_lanes_apart(float v) {
+  static_assert(S == 2 || S == 4 || S == 8 || S == 16, "2, 4, 8 or 16 lanes apart");
+  if (S <= 2)
+    v += dpp_f<0x4E>(v);  // quad_perm [2,3,0,1]: lane ^ 2
+  if (S <= 4)
+    v += dpp_f<0x124>(v); // row_ror:4: lanes 4, 8, 12 further on ...
+  if (S <= 8)
+    v += dpp_f<0x128>(v); // ... with row_ror:8
+  return sum_rows(v);
+}
+
 constexpr int kWaves = 8;
-constexpr int kUnroll = 6;         // loads in flight per lane
+constexpr int kUnroll = 12;        // loads in flight per lane         // loads in flight per lane
 
 // kCols = columns per workgroup: 16 (64-byte pieces of a row, the most workgroups)
 // for narrow matrices, 32 or 64 (longer pieces, fewer and larger requests per row)
@@ -64,7 +84,7 @@ gemv_f32_kernel(const float *__restrict__ x, const float *__restrict__ B,
       const int kc = min(k, K - 1); // rows past the end repeat the last, times zero
       const float *row = B + (int64_t)kc * ldb + bcol;
       if (full)
-        b[u] = *reinterpret_cast<const float4 *>(row);
+        b[u] = load_stream4(row); // read once per launch: past the caches
       else
         b[u] = make_float4(col < N ? row[0] : 0.f, col + 1 < N ? row[1] : 0.f,
                            col + 2 < N ? row[2] : 0.f, col + 3 < N ? row[3] : 0.f);
@@ -83,14 +103,11 @@ gemv_f32_kernel(const float *__restrict__ x, const float *__restrict__ B,
     }
   }
   // the row lanes of a column group hold different k: lanes kLanesPerRow apart ... 32 apart
-#pragma unroll
-  for (int o = kLanesPerRow; o < 64; o <<= 1) {
-    acc.x += __shfl_xor(acc.x, o, 64);
-    acc.y += __shfl_xor(acc.y, o, 64);
-    acc.z += __shfl_xor(acc.z, o, 64);
-    acc.w += __shfl_xor(acc.w, o, 64);
-    ss += __shfl_xor(ss, o, 64);
-  }
+  acc.x = sum_lanes_apart<kLanesPerRow>(acc.x);
+  acc.y = sum_lanes_apart<kLanesPerRow>(acc.y);
+  acc.z = sum_lanes_apart<kLanesPerRow>(acc.z);
+  acc.w = sum_lanes_apart<kLanesPerRow>(acc.w);
+  ss = sum_lanes_apart<kLanesPerRow>(ss);
   if (lane < kLanesPerRow) {
     red[wave][lane * 4 + 0] = acc.x;
     red[wave][lane * 4 + 1] = acc.y;
@@ -162,7 +179,7 @@ gemv_f32_tiles_kernel(const float *__restrict__ x, const float *__restrict__ T,
     for (int u = 0; u < kTileUnroll; ++u) {
       const int blk = b0 + u * kWaves;
       const int bc = min(blk, blocks - 1); // past the end: the last tile again, x = 0
-      b[u] = strip[(int64_t)bc * 64];
+      b[u] = load_stream4(reinterpret_cast<const float *>(strip + (int64_t)bc * 64));
       const int k = blk * kTileRows + row;
       const int kc = min(k, K - 1);
       xv[u] = (blk < blocks && k < K) ? x[kc] : 0.f;
@@ -179,14 +196,11 @@ gemv_f32_tiles_kernel(const float *__restrict__ x, const float *__restrict__ T,
       acc.w = fmaf(xs, b[u].w, acc.w);
     }
   }
-#pragma unroll
-  for (int o = 2; o < 64; o <<= 1) {
-    acc.x += __shfl_xor(acc.x, o, 64);
-    acc.y += __shfl_xor(acc.y, o, 64);
-    acc.z += __shfl_xor(acc.z, o, 64);
-    acc.w += __shfl_xor(acc.w, o, 64);
-    ss += __shfl_xor(ss, o, 64);
-  }
+  acc.x = sum_lanes_apart<2>(acc.x);
+  acc.y = sum_lanes_apart<2>(acc.y);
+  acc.z = sum_lanes_apart<2>(acc.z);
+  acc.w = sum_lanes_apart<2>(acc.w);
+  ss = sum_lanes_apart<2>(ss);
   if (lane < 2) {
     red[wave][lane * 4 + 0] = acc.x;
     red[wave][lane * 4 + 1] = acc.y;
