@@ -427,6 +427,25 @@ def bench_prefill(bh, args):
                      "gemm_tflops": gemm_flop / t / 1e12,
                      "mfma_frac": gemm_flop / t / 1e12 / peak}
     sess.close()
+    # the w8a8 matmul (int8 activations, exact int32 sums) at 512 rows of the two
+    # MLP shapes: quantisation (two launches) + one int8 plane through the same
+    # matrix-core kernel
+    for K, N in ((H, I), (I, H)):
+        x = torch.randn((M, K), device="cuda")
+        packed = _random_packed(K, N, 4)
+        wscale = torch.full((N,), 1e-3, device="cuda")
+        y = torch.empty((M, N), device="cuda")
+        nb = bh.buddy_hip_w8a8_workspace_bytes(M, K)
+        ws = torch.empty((nb,), dtype=torch.int8, device="cuda")
+        stream = torch.cuda.current_stream().cuda_stream
+
+        def w8a8(i):
+            if bh.buddy_hip_w8a8_matmul(x.data_ptr(), packed[i % 4].data_ptr(), wscale.data_ptr(),
+                                        y.data_ptr(), None, M, K, N, ws.data_ptr(), nb, stream):
+                raise RuntimeError("w8a8_matmul failed")
+        t8 = _time_launches(w8a8, 80)
+        res[f"w8a8_512x{K}x{N}"] = {"us": t8 * 1e6, "tops": 2 * M * K * N / t8 / 1e12,
+                                    "mfma_frac": 2 * M * K * N / t8 / 1e12 / MFMA_I8_PEAK_TOPS}
     t = res["i8_3digit"]["ms"] * 1e-3
     return {
         "metric": "prefill_tokens_per_s", "value": M / t, "unit": "tokens/s",

@@ -62,6 +62,14 @@ int launch_gemm_w8_digits(const GemmW8Args &a, const void *planes, hipStream_t s
 
 int launch_gemm_w8(const GemmW8Args &a, hipStream_t stream);
 
+// w8a8 for more than 16 rows: one int8 plane of activations (layout of
+// gemm_staging_layout(M, K) with one digit, every row step = the activation
+// scale) times the packed int8 weights; C = f32(sum) * (step * wscale[n]) and,
+// when `sums` is not null, the int32 sums themselves (dense [M, N]).
+int launch_gemm_w8a8_plane(const void *plane, const int8_t *W, const float *wscale, float *C,
+                           int32_t *sums, int64_t M, int64_t K, int64_t N,
+                           hipStream_t stream);
+
 // split-K workspace of the int8 matmul (dropped together with the staging)
 void release_gemm_i8_workspace(hipStream_t stream);
 

@@ -232,6 +232,7 @@ struct GemmI8Args {
   int slices, chunks_per_slice;
   float *partial;     // [tile][slice][wavefront][row block][16][16 GPW]
   int accumulate;
+  int32_t *sums;      // one plane only: the int32 sums themselves, dense [M, N], or null
 };
 
 // sum_j 256^j acc_j as f32 (each int32 sum is exact; the conversions round to 24
@@ -242,6 +243,12 @@ template <int D> __device__ __forceinline__ float combine(const v4i32 (&acc)[D],
   for (int j = D - 2; j >= 0; --j)
     v = fmaf(v, 256.0f, (float)acc[j][r]);
   return v;
+}
+
+// The finished value of one output.  One plane is the w8a8 matmul, whose result
+// is f32(sum) * (s_a * s_w[n]) in exactly that order (linalg.py:12833-12845).
+template <int D> __device__ __forceinline__ float scaled(float v, float step, float s) {
+  return D == 1 ? v * (step * s) : (v * step) * s;
 }
 
 constexpr int kSplitGroups = 4; // channel groups of 16 per workgroup of the split kernel
@@ -603,10 +610,10 @@ __global__ void __launch_bounds__(kSlices *kWave) gemm_w8_i8_wide_kernel(GemmI8A
 #pragma unroll
     for (int g = 0; g < GPW; ++g) {
       float4 o;
-      o.x = b[g][0] + (combine<D>(acc[g][rb], 0) * step) * s[g][0];
-      o.y = b[g][1] + (combine<D>(acc[g][rb], 1) * step) * s[g][1];
-      o.z = b[g][2] + (combine<D>(acc[g][rb], 2) * step) * s[g][2];
-      o.w = b[g][3] + (combine<D>(acc[g][rb], 3) * step) * s[g][3];
+      o.x = b[g][0] + scaled<D>(combine<D>(acc[g][rb], 0), step, s[g][0]);
+      o.y = b[g][1] + scaled<D>(combine<D>(acc[g][rb], 1), step, s[g][1]);
+      o.z = b[g][2] + scaled<D>(combine<D>(acc[g][rb], 2), step, s[g][2]);
+      o.w = b[g][3] + scaled<D>(combine<D>(acc[g][rb], 3), step, s[g][3]);
       *reinterpret_cast<float4 *>(tile + (lane & 15) * kPad + g * 16 + (lane >> 4) * 4) = o;
     }
 #pragma unroll
@@ -631,6 +638,36 @@ __global__ void __launch_bounds__(kSlices *kWave) gemm_w8_i8_wide_kernel(GemmI8A
         for (int r = 0; r < 4; ++r)
           if (n + r < a.N)
             c[r] = a.accumulate ? c[r] + v[r] : v[r];
+      }
+    }
+    if constexpr (D == 1) {
+      if (a.sums) { // the same turn for the integer sums, carried as float bit patterns
+#pragma unroll
+        for (int g = 0; g < GPW; ++g)
+          *reinterpret_cast<float4 *>(tile + (lane & 15) * kPad + g * 16 + (lane >> 4) * 4) =
+              make_float4(__int_as_float(acc[g][rb][0][0]), __int_as_float(acc[g][rb][0][1]),
+                          __int_as_float(acc[g][rb][0][2]), __int_as_float(acc[g][rb][0][3]));
+        const bool ivec = (a.N & 3) == 0 && (reinterpret_cast<uintptr_t>(a.sums) & 15) == 0;
+#pragma unroll
+        for (int i = 0; i < GPW; ++i) {
+          const int idx = lane + 64 * i;
+          const int row = idx / (GPW * 4), c4 = idx % (GPW * 4);
+          const float4 q = *reinterpret_cast<const float4 *>(tile + row * kPad + c4 * 4);
+          const v4i32 o = {__float_as_int(q.x), __float_as_int(q.y), __float_as_int(q.z),
+                           __float_as_int(q.w)};
+          const int m = m0 + rb * 16 + row, n = n0 + c4 * 4;
+          if (m >= a.M || n >= a.N)
+            continue;
+          int32_t *c = a.sums + (int64_t)m * a.N + n;
+          if (ivec) {
+            *reinterpret_cast<v4i32 *>(c) = o;
+          } else {
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+              if (n + r < a.N)
+                c[r] = o[r];
+          }
+        }
       }
     }
   }
@@ -813,6 +850,7 @@ int launch_gemm_w8_digits(const GemmW8Args &in, const void *planes, hipStream_t 
   a.chunks = (int)ceil_div(in.K, kTileK);
   a.accumulate = in.accumulate ? 1 : 0;
   a.partial = nullptr;
+  a.sums = nullptr;
   a.slices = 1;
   // Three schemes, chosen by a model of their cost in microseconds (fitted to
   // measurements at the Qwen2-1.5B shapes and M = 512):
@@ -880,6 +918,56 @@ int launch_gemm_w8_digits(const GemmW8Args &in, const void *planes, hipStream_t 
                      stream, a, best_rb, best_gpw);
   BH_CHECK_HIP(hipGetLastError());
   return BUDDY_HIP_OK;
+}
+
+// The w8a8 matmul for more than 16 rows: `plane` holds the int8 activations as
+// one plane ([rows_padded][cols_padded], zero padded) followed by the row steps,
+// every one of them the per-tensor activation scale.  K stays within one
+// workgroup, so the int32 sums are whole and exact (K <= 2^17: 2^17 * 127 * 128
+// is below 2^31).
+int launch_gemm_w8a8_plane(const void *plane, const int8_t *W, const float *wscale, float *C,
+                           int32_t *sums, int64_t M, int64_t K, int64_t N,
+                           hipStream_t stream) {
+  BH_REQUIRE(K <= (1 << 17), "w8a8 matmul: K=%lld above 131072", (long long)K);
+  GemmI8Args a;
+  const GemmStagingLayout layout = gemm_staging_layout(M, K);
+  a.Mp = layout.rows_padded;
+  a.Kp = layout.cols_padded;
+  a.planes = static_cast<const int8_t *>(plane);
+  a.steps = reinterpret_cast<const float *>(a.planes + (size_t)a.Mp * a.Kp);
+  a.W = reinterpret_cast<const int4 *>(W);
+  a.scale = wscale;
+  a.bias = nullptr;
+  a.C = C;
+  a.ldc = N;
+  a.M = (int)M;
+  a.N = (int)N;
+  a.groups = (int)ceil_div(N, kTileN);
+  a.chunks = (int)ceil_div(K, kTileK);
+  a.accumulate = 0;
+  a.partial = nullptr;
+  a.sums = sums;
+  a.slices = 1;
+  a.chunks_per_slice = a.chunks;
+  // the same cost model as above, whole K per workgroup only
+  int best_gpw = 0, best_rb = 0;
+  double best_cost = 0;
+  for (int gpw : {5, 4})
+    for (int rb : {4, 3}) {
+      const int64_t ncols = ceil_div(a.groups, gpw * kSlices), rows = ceil_div(M, 16 * rb);
+      const int64_t per_xcd = ceil_div(ncols, 8) * rows;
+      const double wg = 0.0125 * (double)(a.chunks * gpw * rb) + 7.0;
+      const double cost = (double)ceil_div(per_xcd, 32) * wg;
+      if (!best_gpw || cost < best_cost - 1e-9) {
+        best_gpw = gpw;
+        best_rb = rb;
+        best_cost = cost;
+      }
+    }
+  a.ncols = (int)ceil_div(a.groups, best_gpw * kSlices);
+  a.cols_padded = (int)round_up((int64_t)a.ncols, 8);
+  const int row_tiles = (int)ceil_div(M, 16 * best_rb);
+  return launch_shape<1>(best_rb, best_gpw, a, (unsigned)(a.cols_padded * row_tiles), stream);
 }
 
 } // namespace bh

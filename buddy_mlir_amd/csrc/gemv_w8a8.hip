@@ -11,7 +11,17 @@
 // The int8 weights are the same wave-tile packed copy the w8a32 kernels read;
 // the dot products run on v_dot4_i32_i8 (four multiply-adds per lane per
 // instruction), so the partial sums are exact integers whatever the order.
+//
+// Above 16 rows the product runs on the int8 matrix cores (the i8 x i8 -> i32
+// branch of the reference's BLIS kernel,
+// midend/lib/Conversion/MatMulOptimization/MatMulBlisVectorization.cpp:668-724):
+// the quantised activations are written as one plane in the layout the prefill
+// matmul reads, by two launches (partial maxima over the tensor, then one
+// workgroup per row), and the prefill kernel multiplies it with whole K per
+// workgroup, so that the int32 sums stay whole.
 #include "common.h"
+#include <algorithm>
+#include "gemm.h"
 
 namespace bh {
 namespace {
@@ -50,6 +60,67 @@ w8a8_quantize_kernel(const float *__restrict__ x, int64_t n, int M, int K, int K
       r = fminf(fmaxf(r, -128.0f), 127.0f);
     }
     xq[i] = (int8_t)r;
+  }
+}
+
+constexpr int kMaxParts = 256; // workgroups of the partial-maximum launch
+
+// stage 1 of the quantisation of many rows: workgroup g leaves the largest
+// magnitude of its share of the tensor in part[g]
+__global__ void __launch_bounds__(256)
+w8a8_absmax_parts_kernel(const float *__restrict__ x, int64_t n, float *__restrict__ part) {
+  __shared__ float red[4];
+  float m = 0.f;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256)
+    m = fmaxf(m, fabsf(x[i]));
+  m = wave_max(m);
+  if ((threadIdx.x & 63) == 0)
+    red[threadIdx.x >> 6] = m;
+  __syncthreads();
+  if (threadIdx.x == 0)
+    part[blockIdx.x] = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+}
+
+// stage 2: workgroup `row` writes row `row` of the plane ([Mp][Kp], zeros past M
+// and K) and its step, the activation scale (1 for padding rows)
+__global__ void __launch_bounds__(256)
+w8a8_rows_to_plane_kernel(const float *__restrict__ x, int M, int K, int Kp,
+                          const float *__restrict__ part, int parts,
+                          int8_t *__restrict__ plane, float *__restrict__ steps,
+                          float *__restrict__ scale_out) {
+  __shared__ float red[4];
+  const int row = blockIdx.x;
+  float m = 0.f;
+  for (int i = threadIdx.x; i < parts; i += 256)
+    m = fmaxf(m, part[i]);
+  m = wave_max(m);
+  if ((threadIdx.x & 63) == 0)
+    red[threadIdx.x >> 6] = m;
+  __syncthreads();
+  m = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+  const float r127 = 1.0f / 127.0f;
+  const float s = fmaxf(m * r127, 1e-10f);
+  const float inv = 1.0f / s;
+  if (threadIdx.x == 0) {
+    steps[row] = row < M ? s : 1.0f;
+    if (row == 0)
+      *scale_out = s;
+  }
+  const float *xr = x + (int64_t)row * K;
+  for (int k0 = threadIdx.x * 4; k0 < Kp; k0 += 256 * 4) {
+    unsigned word = 0;
+    if (row < M) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        float r = 0.f;
+        if (k0 + e < K) {
+          r = rintf(xr[k0 + e] * inv);
+          r = fminf(fmaxf(r, -128.0f), 127.0f);
+        }
+        word |= ((unsigned)(int)r & 0xffu) << (8 * e);
+      }
+    }
+    *reinterpret_cast<unsigned *>(plane + (size_t)row * Kp + k0) = word;
   }
 }
 
@@ -123,7 +194,11 @@ extern "C" {
 size_t buddy_hip_w8a8_workspace_bytes(int64_t M, int64_t K) {
   if (M <= 0 || K <= 0)
     return 0;
-  return (size_t)(M * bh::round_up(K, 64)) + 64;
+  if (M <= 16)
+    return (size_t)(M * bh::round_up(K, 64)) + 64;
+  // the plane with its row steps, the partial maxima, the scale
+  const bh::GemmStagingLayout l = bh::gemm_staging_layout(M, K);
+  return l.bytes_digits(1) + sizeof(float) * (bh::kMaxParts + 16);
 }
 
 int buddy_hip_w8a8_matmul(const float *A, const int8_t *packed, const float *wscale,
@@ -131,7 +206,7 @@ int buddy_hip_w8a8_matmul(const float *A, const int8_t *packed, const float *wsc
                           int64_t N, void *workspace, size_t workspace_bytes,
                           buddy_hip_stream stream) try {
   BH_REQUIRE(A && packed && wscale && C && workspace, "w8a8_matmul: null pointer");
-  BH_REQUIRE(M >= 1 && M <= 16, "w8a8_matmul: M=%lld outside 1..16", (long long)M);
+  BH_REQUIRE(M >= 1 && M < (1 << 24), "w8a8_matmul: M=%lld outside 1..2^24", (long long)M);
   BH_REQUIRE(K > 0 && N > 0 && K < (1 << 30) && N < (1 << 30), "w8a8_matmul: bad shape");
   BH_REQUIRE(workspace_bytes >= buddy_hip_w8a8_workspace_bytes(M, K),
              "w8a8_matmul: workspace of %zu bytes needed, %zu given",
@@ -140,6 +215,21 @@ int buddy_hip_w8a8_matmul(const float *A, const int8_t *packed, const float *wsc
                  (reinterpret_cast<uintptr_t>(packed) & 15) == 0,
              "w8a8_matmul: workspace and weights must be 16-byte aligned");
   hipStream_t st = bh::as_stream(stream);
+  if (M > 16) {
+    BH_REQUIRE(K <= (1 << 17), "w8a8_matmul: K=%lld above 131072 with more than 16 rows",
+               (long long)K);
+    const bh::GemmStagingLayout l = bh::gemm_staging_layout(M, K);
+    int8_t *plane = static_cast<int8_t *>(workspace);
+    float *steps = reinterpret_cast<float *>(plane + (size_t)l.rows_padded * l.cols_padded);
+    float *part = steps + l.rows_padded, *scale = part + bh::kMaxParts;
+    const int parts = (int)std::min<int64_t>(bh::kMaxParts, bh::ceil_div(M * K, 4096));
+    hipLaunchKernelGGL(bh::w8a8_absmax_parts_kernel, dim3(parts), dim3(256), 0, st, A, M * K,
+                       part);
+    hipLaunchKernelGGL(bh::w8a8_rows_to_plane_kernel, dim3(l.rows_padded), dim3(256), 0, st, A,
+                       (int)M, (int)K, l.cols_padded, part, parts, plane, steps, scale);
+    BH_CHECK_HIP(hipGetLastError());
+    return bh::launch_gemm_w8a8_plane(plane, packed, wscale, C, acc_out, M, K, N, st);
+  }
   const int Kp = (int)bh::round_up(K, 64);
   int8_t *xq = static_cast<int8_t *>(workspace);
   float *scale = reinterpret_cast<float *>(xq + (size_t)M * Kp);

@@ -508,8 +508,12 @@ int buddy_hip_gemv_f32_panels(const float *x, const float *packed, float *y,
  * quantized_matmul_op (frontend/Python/ops/linalg.py:12728-12847): per-tensor
  * dynamic activation scale s_a = max(absmax(A)/127, 1e-10), A_q = clamp(rint(
  * A/s_a)), acc = A_q . W in int32 (exact), C = f32(acc) * (s_a * wscale[n]).
- * `packed` is the wave-tile copy of W; acc_out (int32 [M,N]) may be NULL;
- * M in 1..16.  workspace: buddy_hip_w8a8_workspace_bytes, 16-byte aligned. */
+ * `packed` is the wave-tile copy of W; acc_out (int32 [M,N], dense) may be
+ * NULL.  Up to 16 rows run as a GEMV; more rows run on the int8 matrix cores
+ * (the i8 x i8 -> i32 branch of the BLIS kernel,
+ * midend/lib/Conversion/MatMulOptimization/MatMulBlisVectorization.cpp:668-724)
+ * and need K <= 131072.  A and C are dense ([M,K], [M,N]).
+ * workspace: buddy_hip_w8a8_workspace_bytes, 16-byte aligned. */
 size_t buddy_hip_w8a8_workspace_bytes(int64_t M, int64_t K);
 int buddy_hip_w8a8_matmul(const float *A, const int8_t *packed, const float *wscale,
                           float *C, int32_t *acc_out, int64_t M, int64_t K,

@@ -102,7 +102,12 @@ def test_panel_pack_and_packed_gemv(bh, oracle, K, N):
     assert bh.buddy_hip_pack_panels_f32(B.data_ptr(), K, N - 1, 32, P.data_ptr(), None) != 0
 
 
-@pytest.mark.parametrize("M,K,N", [(1, 1536, 8960), (3, 200, 40), (16, 1536, 256), (1, 8960, 1536)])
+# up to 16 rows: the dot-product GEMV; above: one int8 plane through the prefill
+# matmul (ragged M, K and N, the four tile shapes, the full MLP shapes)
+@pytest.mark.parametrize("M,K,N", [(1, 1536, 8960), (3, 200, 40), (16, 1536, 256), (1, 8960, 1536),
+                                   (17, 64, 64), (50, 100, 30), (144, 256, 16384),
+                                   (300, 256, 10240), (200, 192, 16384), (512, 1536, 8960),
+                                   (512, 8960, 1536)])
 def test_w8a8_int32_partial_sums_bit_exact(bh, oracle, M, K, N):
     q, s = synthetic.quantized_linear(K, N, M + K)
     packed = ops.pack_w8(q)
@@ -119,6 +124,34 @@ def test_w8a8_int32_partial_sums_bit_exact(bh, oracle, M, K, N):
     wC, wacc = oracle.w8a8_matmul(A.cpu().numpy(), q.cpu().numpy(), s.cpu().numpy())
     np.testing.assert_array_equal(acc.cpu().numpy(), wacc)  # integers: exact
     np.testing.assert_array_equal(C.cpu().numpy(), wC)      # same f32 ops on them
+    # the integer sums are optional
+    C2 = torch.empty((M, N), device="cuda")
+    sync_check(bh.buddy_hip_w8a8_matmul(A.data_ptr(), packed.data_ptr(), s.data_ptr(),
+                                        C2.data_ptr(), None, M, K, N, ws.data_ptr(), nb, None))
+    np.testing.assert_array_equal(C2.cpu().numpy(), wC)
+
+
+def test_w8a8_many_rows_extremes(bh, oracle):
+    """All-zero activations (the 1e-10 floor of the scale), and +-127 everywhere
+    with weights of +-128: the largest sums the int32 accumulators meet."""
+    M, K, N = 40, 1024, 48
+    q = torch.full((K, N), -128, dtype=torch.int8, device="cuda")
+    q[:, 1::2] = 127
+    s = torch.full((N,), 0.01, device="cuda")
+    packed = ops.pack_w8(q)
+    nb = bh.buddy_hip_w8a8_workspace_bytes(M, K)
+    ws = torch.empty(nb, dtype=torch.uint8, device="cuda")
+    for A in (torch.zeros((M, K), device="cuda"), torch.full((M, K), -3.0, device="cuda")):
+        C = torch.empty((M, N), device="cuda")
+        acc = torch.empty((M, N), dtype=torch.int32, device="cuda")
+        torch.cuda.synchronize()
+        sync_check(bh.buddy_hip_w8a8_matmul(A.data_ptr(), packed.data_ptr(), s.data_ptr(),
+                                            C.data_ptr(), acc.data_ptr(), M, K, N,
+                                            ws.data_ptr(), nb, None))
+        wC, wacc = oracle.w8a8_matmul(A.cpu().numpy(), q.cpu().numpy(), s.cpu().numpy())
+        np.testing.assert_array_equal(acc.cpu().numpy(), wacc)
+        np.testing.assert_array_equal(C.cpu().numpy(), wC)
+    assert abs(int(wacc[0, 0])) == K * 127 * 128
 
 
 def test_buddy_matmul_f32_entry_point(bh):

@@ -190,10 +190,29 @@ def gemm_case(oracle, M, K, N, mode):
         check_close(got[m], want[m])
 
 
+def w8a8_case(bh, oracle, M, K, N):
+    q, s = synthetic.quantized_linear(K, N, M + K + N)
+    g = torch.Generator(device="cuda").manual_seed(M)
+    x = torch.randn((M, K), generator=g, device="cuda")
+    C = torch.empty((M, N), device="cuda")
+    acc = torch.empty((M, N), dtype=torch.int32, device="cuda")
+    nb = bh.buddy_hip_w8a8_workspace_bytes(M, K)
+    ws = torch.empty(nb, dtype=torch.uint8, device="cuda")
+    packed = ops.pack_w8(q)
+    torch.cuda.synchronize()
+    assert bh.buddy_hip_w8a8_matmul(x.data_ptr(), packed.data_ptr(), s.data_ptr(), C.data_ptr(),
+                                    acc.data_ptr(), M, K, N, ws.data_ptr(), nb, None) == 0
+    torch.cuda.synchronize()
+    wC, wacc = oracle.w8a8_matmul(x.cpu().numpy(), q.cpu().numpy(), s.cpu().numpy())
+    np.testing.assert_array_equal(acc.cpu().numpy(), wacc)
+    np.testing.assert_array_equal(C.cpu().numpy(), wC)
+
+
 def test_every_int8_prefill_matmul_variant(bh, oracle):
     bh.buddy_hip_variant_reset()
     for M, K, N in GEMM_I8_SHAPES:
         gemm_case(oracle, M, K, N, "digits")
+        w8a8_case(bh, oracle, M, K, N)  # the one-plane variants of the same tile shapes
     for fam in ("gemm_w8_i8_wide_kernel", "gemm_w8_i8_kernel"):
         assert launched(bh, fam) == compiled(bh, fam), compiled(bh, fam) - launched(bh, fam)
 
