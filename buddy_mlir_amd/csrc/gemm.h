@@ -20,6 +20,9 @@ struct GemmW8Args {
   // relative to each row's maximum) and multiply on the int8 matrix cores;
   // 0: bf16 terms as above
   int digits = 0;
+  // digits only: W holds two matrices of N / 2 channels one behind the other
+  // (scales likewise), and C [M, N / 2] = SiLU(A . first) * (A . second)
+  bool silu_pair = false;
   // A (same pointer, shape, terms, contents) was the input of the previous
   // matmul on this stream: its bf16 copy is still staged, skip the conversion
   bool reuse_staged_a = false;

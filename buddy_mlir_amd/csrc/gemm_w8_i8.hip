@@ -81,6 +81,11 @@ struct NormRow { // w * (x * rs)
       v[e] = wv[e] * (xv[e] * rs);
   }
 };
+// SiLU(g) * u with the one-instruction exp and reciprocal (1 ulp each)
+__device__ __forceinline__ float silu_times(float g, float u) {
+  const float sig = fast_rcp(1.0f + fast_exp(-g));
+  return (g * sig) * u;
+}
 struct SiluMulRow { // silu(g) * u
   const float *g, *u;
   int n;
@@ -89,10 +94,8 @@ struct SiluMulRow { // silu(g) * u
     load4(g, k0, n, gv);
     load4(u, k0, n, uv);
 #pragma unroll
-    for (int e = 0; e < 4; ++e) { // one-instruction exp and reciprocal (1 ulp each)
-      const float sig = fast_rcp(1.0f + fast_exp(-gv[e]));
-      v[e] = (gv[e] * sig) * uv[e];
-    }
+    for (int e = 0; e < 4; ++e)
+      v[e] = silu_times(gv[e], uv[e]);
   }
 };
 
@@ -438,7 +441,13 @@ __device__ __forceinline__ void wait_loads(FetchRegs<D, GPW> &f) {
     asm volatile("" : "+v"(f.a[j])::"memory");
 }
 
-template <int D, int RB, int GPW>
+// PAIR: W holds two matrices of a.groups / 2 channel groups each, one behind the
+// other; wavefronts 0 and 1 of a workgroup take 32 GPW channels of the first,
+// wavefronts 2 and 3 the same channels of the second, and the result is
+// SiLU(first) * second ([M, N / 2]): the two exchange halves of their tiles
+// through LDS in the epilogue, so only half as much is stored and no launch
+// reads both results again.
+template <int D, int RB, int GPW, bool PAIR>
 __global__ void __launch_bounds__(kSlices *kWave) gemm_w8_i8_wide_kernel(GemmI8Args a) {
   constexpr int kRing = RingDepth<GPW>::value;
   constexpr int L = GPW + D; // loads per fetch
@@ -455,7 +464,11 @@ __global__ void __launch_bounds__(kSlices *kWave) gemm_w8_i8_wide_kernel(GemmI8A
     return; // padding id
   const int col = unit % a.ncols, slice = unit / a.ncols;
   const int m0 = rbk * RB * 16;
-  const int g0 = (col * kSlices + wave) * GPW;
+  const int half_groups = a.groups / 2; // PAIR only
+  // first channel group of this wavefront; with PAIR, within its matrix
+  const int g0 = PAIR ? (col * 2 + (wave & 1)) * GPW : (col * kSlices + wave) * GPW;
+  const int gbase = PAIR ? (wave >> 1) * half_groups : 0;
+  const int glast = PAIR ? half_groups - 1 : a.groups - 1;
   const int cb = slice * a.chunks_per_slice;
   const int nch = min(a.chunks_per_slice, a.chunks - cb); // chunks of this slice, >= 1
 
@@ -472,7 +485,7 @@ __global__ void __launch_bounds__(kSlices *kWave) gemm_w8_i8_wide_kernel(GemmI8A
 #pragma unroll
   for (int g = 0; g < GPW; ++g) // groups past the end repeat the last one
     wp[g] = reinterpret_cast<const v4i32 *>(a.W) +
-            ((size_t)min(g0 + g, a.groups - 1) * a.chunks + cb) * 64 + lane;
+            ((size_t)(gbase + min(g0 + g, glast)) * a.chunks + cb) * 64 + lane;
   const size_t plane = (size_t)a.Mp * a.Kp;
   // this wavefront fetches row block `wave` of the activation tile (with three
   // row blocks the fourth wavefront repeats the third's loads and stages nothing)
@@ -593,27 +606,79 @@ __global__ void __launch_bounds__(kSlices *kWave) gemm_w8_i8_wide_kernel(GemmI8A
     }
     return;
   }
-  float s[GPW][4], b[GPW][4];
-#pragma unroll
-  for (int g = 0; g < GPW; ++g) {
-    const int n = (g0 + g) * kTileN + (lane >> 4) * 4;
-#pragma unroll
-    for (int r = 0; r < 4; ++r) {
-      s[g][r] = n + r < a.N ? a.scale[n + r] : 0.f;
-      b[g][r] = (a.bias && n + r < a.N) ? a.bias[n + r] : 0.f;
-    }
-  }
-#pragma unroll
-  for (int rb = 0; rb < RB; ++rb) {
-    const int mr = m0 + rb * 16 + (lane & 15);
-    const float step = mr < a.M ? a.steps[mr] : 0.f;
+  // without PAIR the scales and the bias stay in registers over the row blocks;
+  // with it there is no register left for them, and each use loads them again
+  float s[PAIR ? 1 : GPW][4], b[PAIR ? 1 : GPW][4];
+  if constexpr (!PAIR) {
 #pragma unroll
     for (int g = 0; g < GPW; ++g) {
-      float4 o;
+      const int n = (g0 + g) * kTileN + (lane >> 4) * 4;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        s[g][r] = n + r < a.N ? a.scale[n + r] : 0.f;
+        b[g][r] = (a.bias && n + r < a.N) ? a.bias[n + r] : 0.f;
+      }
+    }
+  }
+  // finished values of channel group g, row block rb (PAIR: the scales of the
+  // second matrix follow those of the first; a.N is a multiple of 16)
+  auto finished = [&](int g, int rb, float step) {
+    float4 o;
+    if constexpr (PAIR) {
+      const int n = (g0 + g) * kTileN + (lane >> 4) * 4;
+      float4 sc = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (n < a.N)
+        sc = *reinterpret_cast<const float4 *>(a.scale + (wave >> 1) * a.N + n);
+      o.x = scaled<D>(combine<D>(acc[g][rb], 0), step, sc.x);
+      o.y = scaled<D>(combine<D>(acc[g][rb], 1), step, sc.y);
+      o.z = scaled<D>(combine<D>(acc[g][rb], 2), step, sc.z);
+      o.w = scaled<D>(combine<D>(acc[g][rb], 3), step, sc.w);
+    } else {
       o.x = b[g][0] + scaled<D>(combine<D>(acc[g][rb], 0), step, s[g][0]);
       o.y = b[g][1] + scaled<D>(combine<D>(acc[g][rb], 1), step, s[g][1]);
       o.z = b[g][2] + scaled<D>(combine<D>(acc[g][rb], 2), step, s[g][2]);
       o.w = b[g][3] + scaled<D>(combine<D>(acc[g][rb], 3), step, s[g][3]);
+    }
+    return o;
+  };
+  // PAIR: the wavefronts of the first matrix finish the upper row blocks of the
+  // tile, those of the second the lower ones (each stores half as much as an
+  // unpaired wavefront): what a wavefront computed of the other's row blocks
+  // crosses over through LDS, same lane, same registers
+  constexpr int kUpper = (RB + 1) / 2;
+  const bool second = PAIR && wave >= 2;
+  float4 *cross = reinterpret_cast<float4 *>(reinterpret_cast<float *>(frag_s) +
+                                             kSlices * 16 * kPad);
+  if constexpr (PAIR) {
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb) {
+      if (second ? rb >= kUpper : rb < kUpper)
+        continue; // stays here
+      const int mr = m0 + rb * 16 + (lane & 15);
+      const float step = mr < a.M ? a.steps[mr] : 0.f;
+      const int slot = rb < kUpper ? rb : rb - kUpper;
+#pragma unroll
+      for (int g = 0; g < GPW; ++g)
+        cross[((wave * kUpper + slot) * GPW + g) * kWave + lane] = finished(g, rb, step);
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb) {
+    if (PAIR && (second ? rb < kUpper : rb >= kUpper))
+      continue; // the partner wavefront finishes this row block
+    const int mr = m0 + rb * 16 + (lane & 15);
+    const float step = mr < a.M ? a.steps[mr] : 0.f;
+#pragma unroll
+    for (int g = 0; g < GPW; ++g) {
+      float4 o = finished(g, rb, step);
+      if constexpr (PAIR) {
+        const int slot = rb < kUpper ? rb : rb - kUpper;
+        const float4 p = cross[(((wave ^ 2) * kUpper + slot) * GPW + g) * kWave + lane];
+        const float4 gate = second ? p : o, up = second ? o : p;
+        o = make_float4(silu_times(gate.x, up.x), silu_times(gate.y, up.y),
+                        silu_times(gate.z, up.z), silu_times(gate.w, up.w));
+      }
       *reinterpret_cast<float4 *>(tile + (lane & 15) * kPad + g * 16 + (lane >> 4) * 4) = o;
     }
 #pragma unroll
@@ -706,14 +771,25 @@ reduce_slices_kernel(GemmI8Args a, int rb_per_tile, int gpw) {
 BH_VARIANT_FAMILY(WideFamily, "gemm_w8_i8_wide_kernel");
 BH_VARIANT_FAMILY(SplitFamily, "gemm_w8_i8_kernel");
 
-template <int D, int RB, int GPW>
+template <int D, int RB, int GPW, bool PAIR = false>
 int launch_wide(const GemmI8Args &a, unsigned blocks, hipStream_t stream) {
-  // three fragment buffers in the loop, four output tiles in the epilogue
-  constexpr size_t lds = std::max(sizeof(v4i32) * 3 * D * RB * kWave,
-                                  sizeof(float) * kSlices * 16 * (GPW * 16 + 4));
-  BH_NOTE_VARIANT(WideFamily, D, RB, GPW);
-  hipLaunchKernelGGL((gemm_w8_i8_wide_kernel<D, RB, GPW>), dim3(blocks),
-                     dim3(kSlices * kWave), lds, stream, a);
+  // three fragment buffers in the loop, four output tiles in the epilogue (and
+  // with PAIR the values that cross from wavefronts 2 and 3 to 0 and 1)
+  constexpr size_t lds =
+      std::max(sizeof(v4i32) * 3 * D * RB * kWave,
+               sizeof(float) * kSlices * 16 * (GPW * 16 + 4) +
+                   (PAIR ? sizeof(float4) * kSlices * ((RB + 1) / 2) * GPW * kWave : 0));
+  auto kernel = gemm_w8_i8_wide_kernel<D, RB, GPW, PAIR>;
+  if (lds > 48 * 1024) {
+    static bool attr_set = false;
+    if (!attr_set) {
+      BH_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+      attr_set = true;
+    }
+  }
+  BH_NOTE_VARIANT(WideFamily, D, RB, GPW, (int)PAIR);
+  hipLaunchKernelGGL(kernel, dim3(blocks), dim3(kSlices * kWave), lds, stream, a);
   BH_CHECK_HIP(hipGetLastError());
   return BUDDY_HIP_OK;
 }
@@ -806,13 +882,13 @@ template <int D> int launch_split(const GemmI8Args &a, unsigned blocks, hipStrea
   return BUDDY_HIP_OK;
 }
 
-template <int D> int launch_shape(int rb, int gpw, const GemmI8Args &a, unsigned blocks,
-                                  hipStream_t stream) {
+template <int D, bool PAIR = false>
+int launch_shape(int rb, int gpw, const GemmI8Args &a, unsigned blocks, hipStream_t stream) {
   switch (rb * 10 + gpw) {
-  case 34: return launch_wide<D, 3, 4>(a, blocks, stream);
-  case 35: return launch_wide<D, 3, 5>(a, blocks, stream);
-  case 44: return launch_wide<D, 4, 4>(a, blocks, stream);
-  default: return launch_wide<D, 4, 5>(a, blocks, stream);
+  case 34: return launch_wide<D, 3, 4, PAIR>(a, blocks, stream);
+  case 35: return launch_wide<D, 3, 5, PAIR>(a, blocks, stream);
+  case 44: return launch_wide<D, 4, 4, PAIR>(a, blocks, stream);
+  default: return launch_wide<D, 4, 5, PAIR>(a, blocks, stream);
   }
 }
 
@@ -852,6 +928,35 @@ int launch_gemm_w8_digits(const GemmW8Args &in, const void *planes, hipStream_t 
   a.partial = nullptr;
   a.sums = nullptr;
   a.slices = 1;
+  if (in.silu_pair) {
+    // two matrices of N / 2 channels, result SiLU(first) * second: wide tiles of
+    // 32 GPW channels of both, whole K per workgroup
+    BH_REQUIRE(in.N % (2 * kTileN) == 0 && !in.accumulate && !in.bias,
+               "gemm_w8: the SiLU pair needs two matrices of a multiple of 16 channels, no "
+               "bias, no accumulation");
+    a.N = (int)(in.N / 2);
+    a.chunks_per_slice = a.chunks;
+    const int half_groups = a.groups / 2;
+    int best_gpw = 0, best_rb = 0;
+    double best_cost = 0;
+    for (int gpw : {5, 4})
+      for (int rb : {4, 3}) {
+        const int64_t ncols = ceil_div(half_groups, 2 * gpw), rows = ceil_div(in.M, 16 * rb);
+        const int64_t per_xcd = ceil_div(ncols, 8) * rows;
+        const double wg = 0.0125 * (double)(a.chunks * gpw * rb * in.digits) + 7.0;
+        const double cost = (double)ceil_div(per_xcd, 32) * wg;
+        if (!best_gpw || cost < best_cost - 1e-9) {
+          best_gpw = gpw;
+          best_rb = rb;
+          best_cost = cost;
+        }
+      }
+    a.ncols = (int)ceil_div(half_groups, 2 * best_gpw);
+    a.cols_padded = (int)round_up((int64_t)a.ncols, 8);
+    const int row_tiles = (int)ceil_div(in.M, 16 * best_rb);
+    return launch_shape<3, true>(best_rb, best_gpw, a, (unsigned)(a.cols_padded * row_tiles),
+                                 stream);
+  }
   // Three schemes, chosen by a model of their cost in microseconds (fitted to
   // measurements at the Qwen2-1.5B shapes and M = 512):
   //  * wide tiles, whole K per workgroup: the chip runs 256 workgroups at a time

@@ -627,8 +627,9 @@ int launch_gemm_w8(const GemmW8Args &in, hipStream_t stream) {
                  in.K < (1 << 24) && in.N < (1 << 24),
              "gemm_w8: bad shape M=%lld K=%lld N=%lld", (long long)in.M,
              (long long)in.K, (long long)in.N);
-  BH_REQUIRE((in.staged || in.lda >= in.K) && in.ldc >= in.N,
+  BH_REQUIRE((in.staged || in.lda >= in.K) && in.ldc >= (in.silu_pair ? in.N / 2 : in.N),
              "gemm_w8: row stride below row length");
+  BH_REQUIRE(!in.silu_pair || in.digits, "gemm_w8: the SiLU pair runs on digit planes only");
   // one bf16 term (activations cast to bf16) or three (every f32 bit); digit
   // planes always three: the variants in between were never reachable from an
   // entry point and are not built
@@ -730,6 +731,11 @@ int buddy_hip_gemm_w8a32(const float *A, const int8_t *packed, const float *scal
   a.accumulate = (flags & BUDDY_HIP_GEMV_ACCUMULATE) != 0;
   a.terms = (flags & BUDDY_HIP_GEMM_A_F32_EXACT) ? 3 : 1;
   a.digits = (flags & BUDDY_HIP_GEMM_A_I8_DIGITS) ? 3 : 0;
+  if (flags & BUDDY_HIP_GEMM_SILU_PAIR) {
+    BH_REQUIRE(a.digits, "gemm_w8a32: BUDDY_HIP_GEMM_SILU_PAIR needs BUDDY_HIP_GEMM_A_I8_DIGITS");
+    a.silu_pair = true;
+    a.N = 2 * N; // both matrices; the result has N channels
+  }
   return bh::launch_gemm_w8(a, bh::as_stream(stream));
 } BH_CATCH_INT("buddy_hip_gemm_w8a32")
 }

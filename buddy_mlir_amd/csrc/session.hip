@@ -417,6 +417,30 @@ struct Session {
       if ((rc = norm_to_staging(pf_x, L.ln2, n, pf_xn_bf)))
         return rc;
       const int64_t ld_gu = 2 * (int64_t)S.inter;
+      if (L.gate_up_joint && gemm_digits) {
+        // gate and up in one launch whose workgroups hold matching tiles of
+        // both: SiLU(gate) * up leaves the matmul, and one pass turns it into
+        // the digit planes of down's input
+        GemmW8Args g;
+        g.staged = pf_xn_bf;
+        g.W = L.gate.w;
+        g.scale = L.gate.s;
+        g.C = pf_g;
+        g.ldc = S.inter;
+        g.M = n;
+        g.K = L.gate.K;
+        g.N = 2 * L.gate.N;
+        g.digits = gemm_digits;
+        g.silu_pair = true;
+        if ((rc = launch_gemm_w8(g, stream)))
+          return rc;
+        if ((rc = launch_activations_to_digits(pf_g, S.inter, n, S.inter, gemm_digits, pf_g_bf,
+                                               stream)))
+          return rc;
+        if ((rc = gemm_staged(pf_g_bf, L.down, pf_x, n, true)))
+          return rc;
+        continue;
+      }
       if (L.gate_up_joint) {
         // gate | up as one matrix of 2 * inter channels: one launch, whose second
         // round of tiles starts while the first one drains

@@ -218,8 +218,17 @@ int buddy_hip_linear_w8a32(const buddy_hip_linear_desc *desc,
  * the int8 weights are multiplied as they are on the int8 matrix cores, with
  * exact int32 sums: the only rounding is that of a, at most 2^-23 of the row's
  * largest magnitude (NaN and infinity do not survive it; K <= 2^17).
- * BUDDY_HIP_GEMV_ACCUMULATE as above. */
-enum { BUDDY_HIP_GEMM_A_F32_EXACT = 2, BUDDY_HIP_GEMM_A_I8_DIGITS = 4 };
+ * BUDDY_HIP_GEMV_ACCUMULATE as above.
+ * BUDDY_HIP_GEMM_SILU_PAIR (with BUDDY_HIP_GEMM_A_I8_DIGITS; N % 16 == 0; no
+ * accumulation): `packed` holds two [K,N] matrices one behind the other, each
+ * packed on its own, `scale` 2 N values, and C[M,N] = SiLU(A . W0) * (A . W1),
+ * the prefill form of BUDDY_HIP_EPI_SILU_MUL
+ * (subgraph0_decode_simplify.mlir:225-232 over M rows). */
+enum {
+  BUDDY_HIP_GEMM_A_F32_EXACT = 2,
+  BUDDY_HIP_GEMM_A_I8_DIGITS = 4,
+  BUDDY_HIP_GEMM_SILU_PAIR = 8
+};
 int buddy_hip_gemm_w8a32(const float *A, const int8_t *packed, const float *scale,
                          float *C, int64_t M, int64_t K, int64_t N,
                          unsigned flags, buddy_hip_stream stream);

@@ -92,6 +92,52 @@ def test_digit_planes_are_the_rounded_fixed_point(M, K):
     assert (np.abs(got - xh) <= 0.5 * step + 2e-7 * np.abs(xh)).all()
 
 
+# gate and up in one launch with SiLU(gate) * up in its epilogue: the model's
+# shape, one shape for each of the four workgroup tiles, single-tile and ragged rows
+SILU_PAIR_SHAPES = [(512, 1536, 8960), (144, 256, 8192), (300, 256, 5120), (200, 192, 8192),
+                    (512, 192, 4480), (17, 64, 16), (100, 100, 160)]
+
+
+def silu_pair_case(oracle, M, K, N):
+    q0, s0 = synthetic.quantized_linear(K, N, M + K + N)
+    q1, s1 = synthetic.quantized_linear(K, N, M + K + N + 1)
+    packed = torch.cat([ops.pack_w8(q0), ops.pack_w8(q1)])
+    scale = torch.cat([s0, s1])
+    g = torch.Generator(device="cuda").manual_seed(M)
+    x = torch.randn((M, K), generator=g, device="cuda")
+    y = ops.gemm_w8a32(x, packed, scale, K, N, digits=True, silu_pair=True)
+    torch.cuda.synchronize()
+    xh = x.cpu().numpy()
+    gate = oracle.blis_gemm_w8a32(xh, q0.cpu().numpy(), s0.cpu().numpy())
+    up = oracle.blis_gemm_w8a32(xh, q1.cpu().numpy(), s1.cpu().numpy())
+    got = y.cpu().numpy()
+    assert got.shape == (M, N)
+    for m in range(M):
+        check_close(got[m], oracle.silu_mul(gate[m], up[m]))
+
+
+@pytest.mark.parametrize("M,K,N", SILU_PAIR_SHAPES)
+def test_prefill_gemm_silu_pair(oracle, M, K, N):
+    silu_pair_case(oracle, M, K, N)
+
+
+def test_prefill_gemm_silu_pair_refusals(bh):
+    x = torch.zeros((32, 64), device="cuda")
+    w = torch.zeros((2 * 64 * 64,), dtype=torch.int8, device="cuda")
+    s = torch.ones((128,), device="cuda")
+    c = torch.zeros((32, 64), device="cuda")
+    # not without the digit planes, not with accumulation, not with a ragged N
+    assert bh.buddy_hip_gemm_w8a32(x.data_ptr(), w.data_ptr(), s.data_ptr(), c.data_ptr(),
+                                   32, 64, 64, ops.GEMM_SILU_PAIR, None) != 0
+    assert bh.buddy_hip_gemm_w8a32(x.data_ptr(), w.data_ptr(), s.data_ptr(), c.data_ptr(),
+                                   32, 64, 64, ops.GEMM_SILU_PAIR | ops.GEMM_A_I8_DIGITS |
+                                   ops.GEMV_ACCUMULATE, None) != 0
+    assert bh.buddy_hip_gemm_w8a32(x.data_ptr(), w.data_ptr(), s.data_ptr(), c.data_ptr(),
+                                   32, 64, 40, ops.GEMM_SILU_PAIR | ops.GEMM_A_I8_DIGITS,
+                                   None) != 0
+    torch.cuda.synchronize()
+
+
 @pytest.mark.parametrize("exact", [True, False])
 @pytest.mark.parametrize("M,K,N", [(100, 256, 96), (490, 136, 6600)])
 def test_prefill_gemm_accumulates(oracle, M, K, N, exact):

@@ -19,7 +19,7 @@ import oracle_lib
 from buddy_mlir_amd import ops, synthetic
 from buddy_mlir_amd.session import Shape
 from parity import check_close
-from test_gpu_prefill import SCALE, bf16_round, run_attn
+from test_gpu_prefill import SCALE, SILU_PAIR_SHAPES, bf16_round, run_attn, silu_pair_case
 
 pytestmark = pytest.mark.gpu
 
@@ -213,6 +213,8 @@ def test_every_int8_prefill_matmul_variant(bh, oracle):
     for M, K, N in GEMM_I8_SHAPES:
         gemm_case(oracle, M, K, N, "digits")
         w8a8_case(bh, oracle, M, K, N)  # the one-plane variants of the same tile shapes
+    for M, K, N in SILU_PAIR_SHAPES[1:5]:  # the paired variants
+        silu_pair_case(oracle, M, K, N)
     for fam in ("gemm_w8_i8_wide_kernel", "gemm_w8_i8_kernel"):
         assert launched(bh, fam) == compiled(bh, fam), compiled(bh, fam) - launched(bh, fam)
 
