@@ -23,6 +23,13 @@ struct GemmW8Args {
   // digits only: W holds two matrices of N / 2 channels one behind the other
   // (scales likewise), and C [M, N / 2] = SiLU(A . first) * (A . second)
   bool silu_pair = false;
+  // digits only: the finished rows of C also leave as RMSNorm(row) * then_norm_w
+  // in digit planes (then_norm_staged: layout of gemm_staging_layout(M, N)), the
+  // input of the matmul that follows -- written by the kernel that adds the K
+  // slices where there is one, by a launch of its own otherwise
+  const float *then_norm_w = nullptr;
+  float then_norm_eps = 0.f;
+  void *then_norm_staged = nullptr;
   // A (same pointer, shape, terms, contents) was the input of the previous
   // matmul on this stream: its bf16 copy is still staged, skip the conversion
   bool reuse_staged_a = false;

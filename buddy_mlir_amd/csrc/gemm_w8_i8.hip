@@ -738,6 +738,24 @@ __global__ void __launch_bounds__(kSlices *kWave) gemm_w8_i8_wide_kernel(GemmI8A
   }
 }
 
+// Sum of a float4 over the K slices, in slice order, four loads in flight at a
+// time (slices past the end repeat the last one and are not added).
+__device__ __forceinline__ void sum_slices(const float *p, size_t slice_stride, int slices,
+                                           float (&v)[4]) {
+  v[0] = v[1] = v[2] = v[3] = 0.f;
+  for (int sl = 0; sl < slices; sl += 4) {
+    float4 q[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+      q[u] = *reinterpret_cast<const float4 *>(p + (size_t)min(sl + u, slices - 1) * slice_stride);
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+      if (sl + u < slices) {
+        v[0] += q[u].x; v[1] += q[u].y; v[2] += q[u].z; v[3] += q[u].w;
+      }
+  }
+}
+
 // C (+)= step[m] * scale[n] * sum over slices of the unscaled sums, slice order.
 __global__ void __launch_bounds__(256)
 reduce_slices_kernel(GemmI8Args a, int rb_per_tile, int gpw) {
@@ -753,11 +771,8 @@ reduce_slices_kernel(GemmI8Args a, int rb_per_tile, int gpw) {
   const size_t slice_stride = (size_t)kSlices * rb_per_tile * sub;
   const float *p = a.partial + ((size_t)(rbk * a.ncols + col) * a.slices) * slice_stride +
                    ((size_t)wave * rb_per_tile + rb) * sub + row * span + ch;
-  float v[4] = {0.f, 0.f, 0.f, 0.f};
-  for (int sl = 0; sl < a.slices; ++sl) {
-    const float4 q = *reinterpret_cast<const float4 *>(p + sl * slice_stride);
-    v[0] += q.x; v[1] += q.y; v[2] += q.z; v[3] += q.w;
-  }
+  float v[4];
+  sum_slices(p, slice_stride, a.slices, v);
   const float step = a.steps[m];
   float *c = a.C + (int64_t)m * a.ldc + n;
 #pragma unroll
@@ -766,6 +781,58 @@ reduce_slices_kernel(GemmI8Args a, int rb_per_tile, int gpw) {
       const float o = (a.bias ? a.bias[n + r] : 0.f) + (v[r] * step) * a.scale[n + r];
       c[r] = a.accumulate ? c[r] + o : o;
     }
+}
+
+// The same, one workgroup per row, which then holds the finished row and goes on
+// to write RMSNorm(row) * w as the digit planes of the next matmul's input (what
+// rmsnorm_to_digits_kernel would read back from C): lds = [Kp2] cache of
+// row_to_digits, then [Kp2] the row.
+__global__ void __launch_bounds__(kRowThreads)
+reduce_slices_norm_kernel(GemmI8Args a, int rb_per_tile, int gpw,
+                          const float *__restrict__ norm_w, float inv_n, float eps, int D,
+                          int Mp2, int Kp2, int8_t *__restrict__ planes) {
+  __shared__ float red[kRowThreads / 64];
+  extern __shared__ __attribute__((aligned(16))) float row_lds[];
+  float *xrow = row_lds + Kp2;
+  const int m = blockIdx.x;
+  const int n4 = (a.N + 3) / 4;
+  const int span = 16 * gpw;
+  const int rbk = m / (16 * rb_per_tile), rb = (m / 16) % rb_per_tile, row = m % 16;
+  const int sub = 16 * span;
+  const size_t slice_stride = (size_t)kSlices * rb_per_tile * sub;
+  const float step = a.steps[m];
+  for (int q4 = threadIdx.x; q4 < n4; q4 += kRowThreads) {
+    const int n = q4 * 4;
+    const int col = n / (kSlices * span), wave = (n / span) % kSlices, ch = n % span;
+    const float *p = a.partial + ((size_t)(rbk * a.ncols + col) * a.slices) * slice_stride +
+                     ((size_t)wave * rb_per_tile + rb) * sub + row * span + ch;
+    float v[4];
+    sum_slices(p, slice_stride, a.slices, v);
+    float *c = a.C + (int64_t)m * a.ldc + n;
+#pragma unroll
+    for (int r = 0; r < 4; ++r)
+      if (n + r < a.N) {
+        float o = (a.bias ? a.bias[n + r] : 0.f) + (v[r] * step) * a.scale[n + r];
+        if (a.accumulate)
+          o += c[r];
+        c[r] = o;
+        xrow[n + r] = o;
+      }
+  }
+  __syncthreads();
+  float s = 0.f;
+  for (int i = threadIdx.x; i < a.N; i += kRowThreads)
+    s = fmaf(xrow[i], xrow[i], s);
+  s = wave_sum(s);
+  if ((threadIdx.x & 63) == 0)
+    red[threadIdx.x >> 6] = s;
+  __syncthreads();
+  float tot = 0.f;
+#pragma unroll
+  for (int w = 0; w < kRowThreads / 64; w += 2)
+    tot += red[w] + red[w + 1];
+  const float rs = 1.0f / sqrtf(tot * inv_n + eps);
+  row_to_digits(NormRow{xrow, norm_w, rs, a.N}, a.N, m, D, Mp2, Kp2, planes, red, row_lds);
 }
 
 BH_VARIANT_FAMILY(WideFamily, "gemm_w8_i8_wide_kernel");
@@ -931,6 +998,7 @@ int launch_gemm_w8_digits(const GemmW8Args &in, const void *planes, hipStream_t 
   if (in.silu_pair) {
     // two matrices of N / 2 channels, result SiLU(first) * second: wide tiles of
     // 32 GPW channels of both, whole K per workgroup
+    BH_REQUIRE(!in.then_norm_w, "gemm_w8: no norm after the SiLU pair");
     BH_REQUIRE(in.N % (2 * kTileN) == 0 && !in.accumulate && !in.bias,
                "gemm_w8: the SiLU pair needs two matrices of a multiple of 16 channels, no "
                "bias, no accumulation");
@@ -993,13 +1061,23 @@ int launch_gemm_w8_digits(const GemmW8Args &in, const void *planes, hipStream_t 
         }
       }
     }
+  // the RMSNorm of the finished rows into digit planes, where the caller asked
+  // for it and no kernel of the matmul holds whole rows
+  auto then_norm = [&]() -> int {
+    if (!in.then_norm_w)
+      return BUDDY_HIP_OK;
+    return launch_rmsnorm_to_digits(in.C, in.ldc, in.then_norm_w, (int)in.M, (int)in.N,
+                                    in.then_norm_eps, in.digits, in.then_norm_staged, stream);
+  };
   const int64_t split_wgs = ceil_div(a.groups, kSplitGroups) * (a.Mp / 64);
   const double split_cost = 1.0 + (double)split_wgs * a.chunks * 16384.0 / 6e6;
   if (split_cost < best_cost) {
     a.ncols = (int)ceil_div(a.groups, kSplitGroups);
     a.cols_padded = (int)round_up(a.ncols, 8);
     const unsigned blocks = (unsigned)(a.cols_padded * (a.Mp / 64));
-    return launch_split<3>(a, blocks, stream);
+    if (int rc = launch_split<3>(a, blocks, stream))
+      return rc;
+    return then_norm();
   }
   a.ncols = (int)ceil_div(a.groups, best_gpw * kSlices);
   a.cols_padded = (int)round_up((int64_t)a.ncols * best_s, 8);
@@ -1016,13 +1094,26 @@ int launch_gemm_w8_digits(const GemmW8Args &in, const void *planes, hipStream_t 
   }
   const unsigned blocks = (unsigned)(a.cols_padded * row_tiles);
   int rc = launch_shape<3>(best_rb, best_gpw, a, blocks, stream);
-  if (rc || best_s == 1)
+  if (rc)
     return rc;
+  if (best_s == 1)
+    return then_norm();
+  const GemmStagingLayout next = gemm_staging_layout(in.M, in.N);
+  if (in.then_norm_w && next.cols_padded <= kRowCache) {
+    // the kernel that adds the slices holds whole rows: it writes the planes too
+    hipLaunchKernelGGL(reduce_slices_norm_kernel, dim3((unsigned)a.M), dim3(kRowThreads),
+                       2 * sizeof(float) * (size_t)next.cols_padded, stream, a, best_rb,
+                       best_gpw, in.then_norm_w, 1.0f / (float)in.N, in.then_norm_eps,
+                       in.digits, next.rows_padded, next.cols_padded,
+                       static_cast<int8_t *>(in.then_norm_staged));
+    BH_CHECK_HIP(hipGetLastError());
+    return BUDDY_HIP_OK;
+  }
   const int64_t threads = (int64_t)a.M * ((a.N + 3) / 4);
   hipLaunchKernelGGL(reduce_slices_kernel, dim3((unsigned)ceil_div(threads, 256)), dim3(256), 0,
                      stream, a, best_rb, best_gpw);
   BH_CHECK_HIP(hipGetLastError());
-  return BUDDY_HIP_OK;
+  return then_norm();
 }
 
 // The w8a8 matmul for more than 16 rows: `plane` holds the int8 activations as

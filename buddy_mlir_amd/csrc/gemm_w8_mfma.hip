@@ -630,6 +630,8 @@ int launch_gemm_w8(const GemmW8Args &in, hipStream_t stream) {
   BH_REQUIRE((in.staged || in.lda >= in.K) && in.ldc >= (in.silu_pair ? in.N / 2 : in.N),
              "gemm_w8: row stride below row length");
   BH_REQUIRE(!in.silu_pair || in.digits, "gemm_w8: the SiLU pair runs on digit planes only");
+  BH_REQUIRE(!in.then_norm_w || (in.digits && in.then_norm_staged),
+             "gemm_w8: a following norm needs digit planes and a buffer for them");
   // one bf16 term (activations cast to bf16) or three (every f32 bit); digit
   // planes always three: the variants in between were never reachable from an
   // entry point and are not built

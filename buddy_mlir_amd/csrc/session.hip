@@ -328,8 +328,12 @@ struct Session {
   }
   // the same with the input already staged as bf16 terms
   int gemm_staged(const unsigned short *staged, const PackedLinear &W, float *C, int64_t M,
-                  bool accumulate, int64_t ldc = 0) {
+                  bool accumulate, int64_t ldc = 0, const float *then_norm_w = nullptr,
+                  void *then_norm_staged = nullptr) {
     GemmW8Args g;
+    g.then_norm_w = then_norm_w;
+    g.then_norm_eps = shape.rms_eps;
+    g.then_norm_staged = then_norm_staged;
     g.staged = staged;
     g.W = W.w;
     g.scale = W.s;
@@ -373,6 +377,7 @@ struct Session {
                        pf_tokens, (int64_t)S.hidden, (int64_t)S.vocab, pf_x);
     BH_CHECK_HIP(hipGetLastError());
     int rc;
+    bool normed_ahead = false; // pf_xn_bf already holds this layer's normed input
     for (int i = 0; i < S.layers; ++i) {
       Layer &L = layers[(size_t)i];
       if (L.qkv_f32) {
@@ -384,9 +389,11 @@ struct Session {
                                     L.qkv.K, L.qkv.N, L.qkv.N, true, stream)))
           return rc;
       } else {
-        // the norm writes the matmul's bf16 input directly
-        if ((rc = norm_to_staging(pf_x, L.ln1, n, pf_xn_bf)))
+        // the norm writes the matmul's input format directly (digit planes: the
+        // previous layer's down matmul already has)
+        if (!normed_ahead && (rc = norm_to_staging(pf_x, L.ln1, n, pf_xn_bf)))
           return rc;
+        normed_ahead = false;
         if ((rc = gemm_staged(pf_xn_bf, L.qkv, pf_qkv, n, false)))
           return rc;
       }
@@ -437,8 +444,13 @@ struct Session {
         if ((rc = launch_activations_to_digits(pf_g, S.inter, n, S.inter, gemm_digits, pf_g_bf,
                                                stream)))
           return rc;
-        if ((rc = gemm_staged(pf_g_bf, L.down, pf_x, n, true)))
+        // down's finished rows go on as the next layer's normed q|k|v input
+        const Layer *nx = i + 1 < S.layers ? &layers[(size_t)i + 1] : nullptr;
+        const bool ahead = nx && !nx->qkv_f32;
+        if ((rc = gemm_staged(pf_g_bf, L.down, pf_x, n, true, 0, ahead ? nx->ln1 : nullptr,
+                              ahead ? pf_xn_bf : nullptr)))
           return rc;
+        normed_ahead = ahead;
         continue;
       }
       if (L.gate_up_joint) {
