@@ -63,7 +63,7 @@ w8a8_quantize_kernel(const float *__restrict__ x, int64_t n, int M, int K, int K
   }
 }
 
-constexpr int kMaxParts = 256; // workgroups of the partial-maximum launch
+constexpr int kMaxParts = 1024; // workgroups of the partial-maximum launch
 
 // stage 1 of the quantisation of many rows: workgroup g leaves the largest
 // magnitude of its share of the tensor in part[g]
@@ -71,8 +71,19 @@ __global__ void __launch_bounds__(256)
 w8a8_absmax_parts_kernel(const float *__restrict__ x, int64_t n, float *__restrict__ part) {
   __shared__ float red[4];
   float m = 0.f;
-  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256)
-    m = fmaxf(m, fabsf(x[i]));
+  const int64_t stride = (int64_t)gridDim.x * 256, first = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if ((reinterpret_cast<uintptr_t>(x) & 15) == 0) { // 16 bytes per load, the tail one by one
+    const int64_t n4 = n / 4;
+    for (int64_t i = first; i < n4; i += stride) {
+      const float4 v = reinterpret_cast<const float4 *>(x)[i];
+      m = fmaxf(fmaxf(m, fmaxf(fabsf(v.x), fabsf(v.y))), fmaxf(fabsf(v.z), fabsf(v.w)));
+    }
+    for (int64_t i = 4 * n4 + first; i < n; i += stride)
+      m = fmaxf(m, fabsf(x[i]));
+  } else {
+    for (int64_t i = first; i < n; i += stride)
+      m = fmaxf(m, fabsf(x[i]));
+  }
   m = wave_max(m);
   if ((threadIdx.x & 63) == 0)
     red[threadIdx.x >> 6] = m;
@@ -222,7 +233,7 @@ int buddy_hip_w8a8_matmul(const float *A, const int8_t *packed, const float *wsc
     int8_t *plane = static_cast<int8_t *>(workspace);
     float *steps = reinterpret_cast<float *>(plane + (size_t)l.rows_padded * l.cols_padded);
     float *part = steps + l.rows_padded, *scale = part + bh::kMaxParts;
-    const int parts = (int)std::min<int64_t>(bh::kMaxParts, bh::ceil_div(M * K, 4096));
+    const int parts = (int)std::min<int64_t>(bh::kMaxParts, bh::ceil_div(M * K, 4096)); // 16 values per thread at least
     hipLaunchKernelGGL(bh::w8a8_absmax_parts_kernel, dim3(parts), dim3(256), 0, st, A, M * K,
                        part);
     hipLaunchKernelGGL(bh::w8a8_rows_to_plane_kernel, dim3(l.rows_padded), dim3(256), 0, st, A,
