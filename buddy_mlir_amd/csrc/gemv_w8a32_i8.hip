@@ -27,12 +27,18 @@
 // when it adds the largest one.  A row whose chunk holds a NaN or an infinity
 // gets a NaN step and with it NaN results, so non-finite activations still show.
 //   * A wavefront converts a chunk once and uses it for SPAN channel groups.
+//   * Up to 8 rows (T2): the 16 columns of the activation operand are 8 rows of
+//     two consecutive tiles, so that one conversion serves two tiles; each tile's
+//     weights are multiplied with the whole operand and a lane keeps the product
+//     that belongs to its own tile (columns 0-7 the first, 8-15 the second); the
+//     two halves are added at the end.
 //   * k-slices of a workgroup meet in LDS in slice order.
 //   * RMSNorm can be fused in: the norm weight multiplies the activation before
 //     it is converted, each lane gathers the squares of what it loads, and the
 //     row's rsqrt factor multiplies the finished sums.
 #include "gemv_w8a32.h"
 
+#include <algorithm>
 #include <cstdio>
 #include <cstdlib>
 
@@ -54,6 +60,7 @@ struct I8Args {
   int K, N, groups, chunks, spans; // spans = ceil(groups / SPAN)
   int GS, KS;                      // spans x k-slices of wavefronts per workgroup
   int rows;
+  bool two_tiles; // up to 8 rows: the variant that converts two tiles at a time
 };
 
 __device__ __forceinline__ float silu(float g) {
@@ -116,48 +123,60 @@ __device__ __forceinline__ void issue_load(f32x4 &dst, const void *p) {
   asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(dst) : "v"(p) : "memory");
 }
 
-template <int SPAN, bool DUAL, bool NORM> struct FetchRegs {
-  v4i w0[SPAN];
-  v4i w1[DUAL ? SPAN : 1];
+template <int SPAN, bool DUAL, bool NORM, bool T2> struct FetchRegs {
+  static constexpr int W = SPAN * (T2 ? 2 : 1); // weight tiles per matrix: [group][tile of the pair]
+  v4i w0[W];
+  v4i w1[DUAL ? W : 1];
   f32x4 x[4]; // k kcol .. kcol+3 of rows lane/16, 4 + lane/16, 8 + lane/16, 12 + lane/16
+              // (T2: of rows lane/16, 4 + lane/16 of the first tile, then of the second)
   f32x4 nw[NORM ? 4 : 1];
 };
-template <int SPAN, bool DUAL, bool NORM> constexpr int fetch_loads() {
-  return SPAN * (DUAL ? 2 : 1) + 4 * (NORM ? 2 : 1);
+template <int SPAN, bool DUAL, bool NORM, bool T2> constexpr int fetch_loads() {
+  return SPAN * (T2 ? 2 : 1) * (DUAL ? 2 : 1) + 4 * (NORM ? 2 : 1);
 }
 // Fetches kept in flight: as many as fit in about 64 registers, two at least.
 // Without the fused norm the kernels then stay within 128 registers (a compute
 // unit holds 16 of their wavefronts); with it they take up to 147 (12).
-template <int SPAN, bool DUAL, bool NORM> constexpr int ring_depth() {
-  constexpr int regs = 4 * SPAN * (DUAL ? 2 : 1) + 16 * (NORM ? 2 : 1);
+template <int SPAN, bool DUAL, bool NORM, bool T2> constexpr int ring_depth() {
+  constexpr int regs = 4 * SPAN * (T2 ? 2 : 1) * (DUAL ? 2 : 1) + 16 * (NORM ? 2 : 1);
   return 64 / regs < 2 ? 2 : 64 / regs;
 }
 
-template <int SPAN, bool DUAL, bool NORM>
+// `c` counts chunks, or pairs of chunks with T2 (`upper`: this lane's operand
+// column belongs to the pair's second tile).
+template <int SPAN, bool DUAL, bool NORM, bool T2>
 __device__ __forceinline__ void fetch_chunk(const I8Args &a, const int4 *w0, const int4 *w1,
                                             const size_t (&gofs)[SPAN],
                                             const float *const (&xrow)[4], int kcol,
-                                            int kofs, int c, bool real,
-                                            FetchRegs<SPAN, DUAL, NORM> &o) {
+                                            int kofs, int c, bool real, int upper,
+                                            FetchRegs<SPAN, DUAL, NORM, T2> &o) {
   // a fetch past the end of the slice (issued only to keep the load counts
   // fixed, never used) reads the first tile of the matrix, which stays in cache:
   // a streaming load of a tile of its own would go to HBM again
+  constexpr int TP = T2 ? 2 : 1;
+  // the chunks of this fetch; a second tile past the end of the matrix repeats
+  // the last one and meets zero digits
+  const int ca = TP * c, cb = min(TP * c + 1, a.chunks - 1);
 #pragma unroll
-  for (int s = 0; s < SPAN; ++s) {
-    const size_t ofs = real ? gofs[s] + (size_t)c * 64 : (size_t)0;
-    issue_load(o.w0[s], w0 + ofs);
-    if (DUAL)
-      issue_load(o.w1[DUAL ? s : 0], w1 + ofs);
-  }
+  for (int s = 0; s < SPAN; ++s)
+#pragma unroll
+    for (int t = 0; t < TP; ++t) {
+      const size_t ofs = real ? gofs[s] + (size_t)(t ? cb : ca) * 64 : (size_t)0;
+      issue_load(o.w0[s * TP + t], w0 + ofs);
+      if (DUAL)
+        issue_load(o.w1[DUAL ? s * TP + t : 0], w1 + ofs);
+    }
   // activations: load q takes 256 bytes of each of rows 4q .. 4q+3 (this lane:
   // four k of one of them); clamped inside the row, what lies past the end of a
-  // ragged row is zeroed when it is consumed (K is a multiple of four)
-  const int kx = min(c * kTileK + kcol, a.K - 4);
+  // ragged row is zeroed when it is consumed (K is a multiple of four).  T2:
+  // loads 0 and 1 take rows 0..7 of the first tile, loads 2 and 3 of the second.
 #pragma unroll
-  for (int q = 0; q < 4; ++q)
-    issue_load(o.x[q], xrow[q] + kx);
+  for (int q = 0; q < 4; ++q) {
+    const int tile = T2 ? ca + (q >> 1) : ca;
+    issue_load(o.x[q], xrow[q] + min(tile * kTileK + kcol, a.K - 4));
+  }
   if (NORM) { // norm weights in operand order: 16 consecutive k, the same for all rows
-    const int k = c * kTileK + kofs;
+    const int k = (ca + (T2 ? upper : 0)) * kTileK + kofs;
 #pragma unroll
     for (int q = 0; q < 4; ++q)
       issue_load(o.nw[NORM ? q : 0], a.norm_w + min(k + 4 * q, a.K - 4));
@@ -166,14 +185,14 @@ __device__ __forceinline__ void fetch_chunk(const I8Args &a, const int4 *w0, con
 
 // Waits until at most N loads are in flight; the registers of `f` are valid only
 // after it.
-template <int N, int SPAN, bool DUAL, bool NORM>
-__device__ __forceinline__ void wait_fetch(FetchRegs<SPAN, DUAL, NORM> &f) {
+template <int N, int SPAN, bool DUAL, bool NORM, bool T2>
+__device__ __forceinline__ void wait_fetch(FetchRegs<SPAN, DUAL, NORM, T2> &f) {
   asm volatile("s_waitcnt vmcnt(%4)"
                : "+v"(f.x[0]), "+v"(f.x[1]), "+v"(f.x[2]), "+v"(f.x[3])
                : "n"(N)
                : "memory");
 #pragma unroll
-  for (int s = 0; s < SPAN; ++s) {
+  for (int s = 0; s < FetchRegs<SPAN, DUAL, NORM, T2>::W; ++s) {
     asm volatile("" : "+v"(f.w0[s])::"memory");
     if (DUAL)
       asm volatile("" : "+v"(f.w1[DUAL ? s : 0])::"memory");
@@ -188,7 +207,7 @@ __device__ __forceinline__ void wait_fetch(FetchRegs<SPAN, DUAL, NORM> &f) {
 constexpr int kTurnStride = 68;               // floats between rows of the turning area
 constexpr int kTurnFloats = 16 * kTurnStride; // per wavefront
 
-template <int EPI, int SPAN, bool NORM>
+template <int EPI, int SPAN, bool NORM, bool T2>
 __global__ void __launch_bounds__(kMaxWavesI8 *kWave, 3) // 3 wavefronts per SIMD at least
     gemv_w8a32_i8_kernel(I8Args a) {
   constexpr bool DUAL = (EPI == kEpiSiluMul);
@@ -200,9 +219,15 @@ __global__ void __launch_bounds__(kMaxWavesI8 *kWave, 3) // 3 wavefronts per SIM
   const int span = blockIdx.x * a.GS + sl;
   const bool live = span < a.spans;
   const int g0 = (live ? span : 0) * SPAN;
-  const int per = (a.chunks + a.KS - 1) / a.KS;
-  const int c0 = min(ks * per, a.chunks), c1 = min(c0 + per, a.chunks);
-  const int m = lane & 15, kg = lane >> 4;
+  // what a wavefront's slice is cut from and a fetch brings: chunks, or pairs of
+  // chunks with T2
+  const int units = T2 ? (a.chunks + 1) / 2 : a.chunks;
+  const int per = (units + a.KS - 1) / a.KS;
+  const int c0 = min(ks * per, units), c1 = min(c0 + per, units);
+  const int kg = lane >> 4;
+  const int col = lane & 15;          // column of the activation operand
+  const int m = T2 ? col & 7 : col;   // its batch row
+  const int upper = T2 ? col >> 3 : 0; // T2: the column belongs to the pair's second tile
 
   f32x4 acc0[SPAN], acc1[DUAL ? SPAN : 1];
 #pragma unroll
@@ -222,7 +247,7 @@ __global__ void __launch_bounds__(kMaxWavesI8 *kWave, 3) // 3 wavefronts per SIM
   const float *xrow[4]; // rows past the batch repeat its last row (never stored)
 #pragma unroll
   for (int q = 0; q < 4; ++q)
-    xrow[q] = a.A + (int64_t)min(4 * q + kg, a.rows - 1) * a.lda;
+    xrow[q] = a.A + (int64_t)min(T2 ? (4 * q + kg) & 7 : 4 * q + kg, a.rows - 1) * a.lda;
   const int kcol = (lane & 15) * 4, kofs = kg * 16;
   // this wavefront's 16 x 64 activations on their way into operand order; rows
   // are 68 floats apart so that the 16 lanes of an operand read hit 64 banks
@@ -235,7 +260,7 @@ __global__ void __launch_bounds__(kMaxWavesI8 *kWave, 3) // 3 wavefronts per SIM
   // With four groups per wavefront the registers are worth more than the
   // latency, and they are loaded after the stream.
   constexpr bool EARLY = SPAN <= 2;
-  const bool writer = live && ks == 0 && m < a.rows;
+  const bool writer = live && ks == 0 && col < a.rows; // (T2: rows <= 8, the lower columns)
   float e_s0[SPAN][4], e_s1[SPAN][4], e_c[SPAN][4];
   auto load_epilogue = [&]() {
 #pragma unroll
@@ -256,17 +281,18 @@ __global__ void __launch_bounds__(kMaxWavesI8 *kWave, 3) // 3 wavefronts per SIM
   if (EARLY)
     load_epilogue();
 
-  constexpr int L = fetch_loads<SPAN, DUAL, NORM>();
-  constexpr int R = ring_depth<SPAN, DUAL, NORM>(); // fetches in flight
-  FetchRegs<SPAN, DUAL, NORM> ring[R];
+  constexpr int L = fetch_loads<SPAN, DUAL, NORM, T2>();
+  constexpr int R = ring_depth<SPAN, DUAL, NORM, T2>(); // fetches in flight
+  FetchRegs<SPAN, DUAL, NORM, T2> ring[R];
   // every fetch is exactly L loads, also one past the end of the slice, which
   // keeps the counts exact
   const int clast = max(c1 - 1, 0);
 #pragma unroll
   for (int u = 0; u < R; ++u)
-    fetch_chunk<SPAN, DUAL, NORM>(a, w0, w1, gofs, xrow, kcol, kofs, min(c0 + u, clast),
-                                  c0 + u < c1, ring[u]);
-  const bool ragged = (a.K & (kTileK - 1)) != 0;
+    fetch_chunk<SPAN, DUAL, NORM, T2>(a, w0, w1, gofs, xrow, kcol, kofs, min(c0 + u, clast),
+                                      c0 + u < c1, upper, ring[u]);
+  // the last fetch of the matrix may bring a ragged tile or (T2) no second tile
+  const bool ragged = (a.K & (kTileK - 1)) != 0 || (T2 && (a.chunks & 1));
   const v4i zero = v4i{0, 0, 0, 0};
   for (int cb = c0; cb < c1; cb += R) {
 #pragma unroll
@@ -274,15 +300,17 @@ __global__ void __launch_bounds__(kMaxWavesI8 *kWave, 3) // 3 wavefronts per SIM
       const int c = cb + u;
       if (c >= c1)
         continue;
-      FetchRegs<SPAN, DUAL, NORM> &cur = ring[u];
-      wait_fetch<(R - 1) * L, SPAN, DUAL, NORM>(cur); // chunk c has arrived
-      // rows 4q + kg, k kcol..kcol+3  ->  row m, k kofs..kofs+15
-      if (ragged && c == a.chunks - 1) { // only the last chunk of a ragged row has a tail
-        const bool past = c * kTileK + kcol >= a.K;
+      FetchRegs<SPAN, DUAL, NORM, T2> &cur = ring[u];
+      wait_fetch<(R - 1) * L, SPAN, DUAL, NORM, T2>(cur); // chunk c has arrived
+      // rows 4q + kg, k kcol..kcol+3  ->  column col, k kofs..kofs+15
+      if (ragged && c == units - 1) { // only the last chunk of a ragged row has a tail
 #pragma unroll
-        for (int q = 0; q < 4; ++q)
+        for (int q = 0; q < 4; ++q) {
+          const int tile = T2 ? 2 * c + (q >> 1) : c;
+          const bool past = tile * kTileK + kcol >= a.K;
           *reinterpret_cast<f32x4 *>(xt + (4 * q + kg) * kTurnStride + kcol) =
               past ? f32x4{0.f, 0.f, 0.f, 0.f} : cur.x[q];
+        }
       } else {
 #pragma unroll
         for (int q = 0; q < 4; ++q)
@@ -291,7 +319,7 @@ __global__ void __launch_bounds__(kMaxWavesI8 *kWave, 3) // 3 wavefronts per SIM
       float xv[16];
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
-        const f32x4 t = *reinterpret_cast<const f32x4 *>(xt + m * kTurnStride + kofs + 4 * q);
+        const f32x4 t = *reinterpret_cast<const f32x4 *>(xt + col * kTurnStride + kofs + 4 * q);
         xv[4 * q] = t.x;
         xv[4 * q + 1] = t.y;
         xv[4 * q + 2] = t.z;
@@ -323,25 +351,38 @@ __global__ void __launch_bounds__(kMaxWavesI8 *kWave, 3) // 3 wavefronts per SIM
       const float step65536 = step * 65536.0f;
       v4i d[3];
       to_digits(xv, inv, d);
+      // the three exact sums of one weight tile with the operand; T2: of both
+      // tiles of the pair, each lane keeping those of its own tile
+      auto products = [&](const v4i *w, v4i &r0, v4i &r1, v4i &r2) {
+        r0 = __builtin_amdgcn_mfma_i32_16x16x64_i8(w[0], d[0], zero, 0, 0, 0);
+        r1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(w[0], d[1], zero, 0, 0, 0);
+        r2 = __builtin_amdgcn_mfma_i32_16x16x64_i8(w[0], d[2], zero, 0, 0, 0);
+        if constexpr (T2) {
+          const v4i u0 = __builtin_amdgcn_mfma_i32_16x16x64_i8(w[1], d[0], zero, 0, 0, 0);
+          const v4i u1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(w[1], d[1], zero, 0, 0, 0);
+          const v4i u2 = __builtin_amdgcn_mfma_i32_16x16x64_i8(w[1], d[2], zero, 0, 0, 0);
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            r0[i] = upper ? u0[i] : r0[i];
+            r1[i] = upper ? u1[i] : r1[i];
+            r2[i] = upper ? u2[i] : r2[i];
+          }
+        }
+      };
+      constexpr int TP = T2 ? 2 : 1;
 #pragma unroll
       for (int s = 0; s < SPAN; ++s) {
-        {
-          const v4i r0 = __builtin_amdgcn_mfma_i32_16x16x64_i8(cur.w0[s], d[0], zero, 0, 0, 0);
-          const v4i r1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(cur.w0[s], d[1], zero, 0, 0, 0);
-          const v4i r2 = __builtin_amdgcn_mfma_i32_16x16x64_i8(cur.w0[s], d[2], zero, 0, 0, 0);
-          combine(acc0[s], r0, r1, r2, step, step65536);
-        }
+        v4i r0, r1, r2;
+        products(&cur.w0[s * TP], r0, r1, r2);
+        combine(acc0[s], r0, r1, r2, step, step65536);
         if (DUAL) {
-          const v4i &w = cur.w1[DUAL ? s : 0];
-          const v4i r0 = __builtin_amdgcn_mfma_i32_16x16x64_i8(w, d[0], zero, 0, 0, 0);
-          const v4i r1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(w, d[1], zero, 0, 0, 0);
-          const v4i r2 = __builtin_amdgcn_mfma_i32_16x16x64_i8(w, d[2], zero, 0, 0, 0);
+          products(&cur.w1[DUAL ? s * TP : 0], r0, r1, r2);
           combine(acc1[DUAL ? s : 0], r0, r1, r2, step, step65536);
         }
       }
       // the registers of chunk c are free: fetch the chunk R further on
-      fetch_chunk<SPAN, DUAL, NORM>(a, w0, w1, gofs, xrow, kcol, kofs, min(c + R, clast),
-                                    c + R < c1, cur);
+      fetch_chunk<SPAN, DUAL, NORM, T2>(a, w0, w1, gofs, xrow, kcol, kofs, min(c + R, clast),
+                                        c + R < c1, upper, cur);
     }
   }
   // repeated last chunks may still be in flight: the ring registers stay
@@ -351,7 +392,7 @@ __global__ void __launch_bounds__(kMaxWavesI8 *kWave, 3) // 3 wavefronts per SIM
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 #pragma unroll
   for (int u = 0; u < R; ++u)
-    wait_fetch<0, SPAN, DUAL, NORM>(ring[u]);
+    wait_fetch<0, SPAN, DUAL, NORM, T2>(ring[u]);
   if (EARLY) {
     // nothing that depends on the epilogue operands moves above this point
 #pragma unroll
@@ -366,6 +407,18 @@ __global__ void __launch_bounds__(kMaxWavesI8 *kWave, 3) // 3 wavefronts per SIM
       }
   } else {
     load_epilogue();
+  }
+  if constexpr (T2) { // columns col and col + 8 hold the two tiles' shares of a row
+#pragma unroll
+    for (int s = 0; s < SPAN; ++s)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        acc0[s][i] += dpp_f<0x128>(acc0[s][i]); // row_ror:8
+        if (DUAL)
+          acc1[DUAL ? s : 0][i] += dpp_f<0x128>(acc1[DUAL ? s : 0][i]);
+      }
+    if (NORM)
+      ss += dpp_f<0x128>(ss);
   }
   if (NORM) { // the four lanes that share a row hold different k
     ss = sum_rows(ss);
@@ -459,12 +512,12 @@ BH_VARIANT_FAMILY(I8Family, "gemv_w8a32_i8_kernel");
 // Workgroups of `waves` wavefronts of this variant that one compute unit holds
 // (asked of the runtime once per variant and size: it knows the registers the
 // compiler used).
-template <int EPI, int SPAN, bool NORM> int workgroups_per_cu(int waves, size_t lds) {
+template <int EPI, int SPAN, bool NORM, bool T2> int workgroups_per_cu(int waves, size_t lds) {
   static int cached[kMaxWavesI8 + 1] = {};
   if (!cached[waves]) {
     int n = 0;
     if (hipOccupancyMaxActiveBlocksPerMultiprocessor(
-            &n, reinterpret_cast<const void *>(gemv_w8a32_i8_kernel<EPI, SPAN, NORM>),
+            &n, reinterpret_cast<const void *>(gemv_w8a32_i8_kernel<EPI, SPAN, NORM, T2>),
             waves * kWave, lds) != hipSuccess ||
         n < 1)
       n = 1;
@@ -473,10 +526,10 @@ template <int EPI, int SPAN, bool NORM> int workgroups_per_cu(int waves, size_t 
   return cached[waves];
 }
 
-template <int EPI, int SPAN, bool NORM>
+template <int EPI, int SPAN, bool NORM, bool T2>
 int launch_kernel(I8Args ka, int ks_forced, hipStream_t stream) {
   constexpr int NA = (EPI == kEpiSiluMul) ? 2 * SPAN : SPAN;
-  auto kernel = gemv_w8a32_i8_kernel<EPI, SPAN, NORM>;
+  auto kernel = gemv_w8a32_i8_kernel<EPI, SPAN, NORM, T2>;
   static bool attr_set = false;
   if (!attr_set) {
     BH_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
@@ -493,13 +546,16 @@ int launch_kernel(I8Args ka, int ks_forced, hipStream_t stream) {
   // compute units) -- a second round of workgroups costs far more than longer
   // slices do (1536 -> 2 x 8960 at 16 rows: 16.2 us with 280 workgroups of 8
   // wavefronts, of which 256 fit, 12.8 us with 280 of 4)
+  // (chunks, or with T2 the pairs of chunks a fetch brings)
+  const int units = T2 ? (ka.chunks + 1) / 2 : ka.chunks;
   int ks = kMaxWavesI8;
   for (; ks > 1; ks /= 2) {
-    if (ka.chunks / ks < 2)
+    if (units / ks < 2)
       continue;
     const int gs = ks < 4 ? 4 / ks : 1, waves = gs * ks;
     const int64_t blocks = ceil_div(ka.spans, gs);
-    if (blocks <= 256 * (int64_t)workgroups_per_cu<EPI, SPAN, NORM>(waves, lds_bytes(ks, waves)))
+    if (blocks <=
+        256 * (int64_t)workgroups_per_cu<EPI, SPAN, NORM, T2>(waves, lds_bytes(ks, waves)))
       break;
   }
   if (ks_forced)
@@ -508,7 +564,7 @@ int launch_kernel(I8Args ka, int ks_forced, hipStream_t stream) {
   ka.GS = ks < 4 ? 4 / ks : 1;
   const int waves = ka.GS * ka.KS;
   const int blocks = (int)ceil_div(ka.spans, ka.GS);
-  BH_NOTE_VARIANT(I8Family, EPI, SPAN, NORM);
+  BH_NOTE_VARIANT(I8Family, EPI, SPAN, NORM, T2);
   hipLaunchKernelGGL(kernel, dim3(blocks), dim3(waves * kWave), lds_bytes(ks, waves), stream, ka);
   BH_CHECK_HIP(hipGetLastError());
   return BUDDY_HIP_OK;
@@ -516,8 +572,18 @@ int launch_kernel(I8Args ka, int ks_forced, hipStream_t stream) {
 
 template <int EPI, int SPAN>
 int launch_norm(const I8Args &ka, int ks_forced, hipStream_t stream) {
-  return ka.norm_w ? launch_kernel<EPI, SPAN, true>(ka, ks_forced, stream)
-                   : launch_kernel<EPI, SPAN, false>(ka, ks_forced, stream);
+  // up to 8 rows: two tiles per conversion of the activations (built for the
+  // group counts whose two weight tiles per group fit the registers)
+  if (ka.two_tiles) {
+    if constexpr (EPI == kEpiSiluMul ? SPAN == 1 : SPAN <= 2)
+      return ka.norm_w ? launch_kernel<EPI, SPAN, true, true>(ka, ks_forced, stream)
+                       : launch_kernel<EPI, SPAN, false, true>(ka, ks_forced, stream);
+    else
+      return fail(BUDDY_HIP_ERR_ARG, "gemv: no two-tile variant for %d groups per wavefront",
+                  SPAN);
+  }
+  return ka.norm_w ? launch_kernel<EPI, SPAN, true, false>(ka, ks_forced, stream)
+                   : launch_kernel<EPI, SPAN, false, false>(ka, ks_forced, stream);
 }
 
 template <int SPAN>
@@ -574,11 +640,19 @@ int launch_gemv_i8(const GemvArgs &a, hipStream_t stream) {
     else if (!dual && ka.groups <= 4 * 256)
       span = 4;
   }
+  // Up to 8 rows: two tiles per conversion, with at most two groups per
+  // wavefront.  Two matrices with two groups each stay on the one-tile variant
+  // (the same four weight tiles per conversion; 4096 -> 2 x 14336 at 8 rows:
+  // 26.0 us against 29.0).
+  ka.two_tiles = a.M <= 8 && !(dual && span == 2);
+  if (ka.two_tiles && span == 4)
+    span = 2;
   ka.spans = (int)ceil_div(ka.groups, span);
   int ks_forced = 0;
   if (const char *e = getenv("BUDDY_HIP_I8_PLAN")) { // measurement only: "span,ks"
     int s_ = 0, k_ = 0;
-    if (sscanf(e, "%d,%d", &s_, &k_) == 2 && (s_ == 1 || s_ == 2 || (s_ == 4 && !dual)) &&
+    if (sscanf(e, "%d,%d", &s_, &k_) == 2 &&
+        (s_ == 1 || (ka.two_tiles ? s_ == 2 && !dual : s_ == 2 || (s_ == 4 && !dual))) &&
         (k_ == 1 || k_ == 2 || k_ == 4 || k_ == kMaxWavesI8)) {
       span = s_;
       ks_forced = k_;

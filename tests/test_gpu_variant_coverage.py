@@ -85,10 +85,15 @@ GEMV_BF16_N = [320, 8192, 131072]     # 2, 4, 8
 
 def test_every_int8_batch_gemv_variant(bh, oracle):
     bh.buddy_hip_variant_reset()
+    # up to 8 rows take the variants that convert two tiles at a time (K = 192:
+    # a pair and a last tile without a partner; K = 320 ends inside a pair's
+    # second tile), more rows the one-tile variants
     for i, N in enumerate(GEMV_I8_N):
         for epilogue in (0, 1, 2):
             for norm in (False, True):
-                gemv_case(bh, oracle, 5 + 3 * i, 192, N, epilogue, norm, 100 + i)
+                gemv_case(bh, oracle, 9 + 3 * i, 192, N, epilogue, norm, 100 + i)
+                if i < 2:
+                    gemv_case(bh, oracle, 5 + 3 * i, 192 + 108 * i, N, epilogue, norm, 150 + i)
     fam = "gemv_w8a32_i8_kernel"
     assert launched(bh, fam) == compiled(bh, fam), compiled(bh, fam) - launched(bh, fam)
 
