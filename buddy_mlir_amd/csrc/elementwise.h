@@ -26,9 +26,12 @@ int launch_argmax_partial(const float *x, int n, void *workspace, int *nparts_ou
 // Tail of a decode step (nparts > 0: pick + log the token; advance: pos/step += 1)
 // and head of the next one (x = embedding row of state[0], rope = [cos | sin] of
 // state[1]).  With nparts = 0 and advance = false it only prepares a step.
-int launch_finish_step(void *amax_workspace, int nparts, int *state, int *token_log,
-                       const float *table, int64_t hidden, int64_t vocab, float *x,
-                       const float *inv_freq, int head_dim, float *rope, bool advance,
-                       int token_log_cap, hipStream_t stream);
+// The candidates are (value, index) pairs in two arrays: the workspace of
+// launch_argmax_partial (values, then indices kArgmaxParts further on) or the
+// per-group maxima a GEMV left behind.
+int launch_finish_step(const float *cand_v, const int *cand_i, int nparts, int *state,
+                       int *token_log, const float *table, int64_t hidden, int64_t vocab,
+                       float *x, const float *inv_freq, int head_dim, float *rope,
+                       bool advance, int token_log_cap, hipStream_t stream);
 
 } // namespace bh

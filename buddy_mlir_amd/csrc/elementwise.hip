@@ -138,20 +138,33 @@ argmax_final_kernel(const float *__restrict__ pv, const int *__restrict__ pi,
 // candidates, logs it, advances position and step, then prepares the next step:
 // its embedding row and the cos/sin table of its position (shared by every
 // layer's attention kernel).  One workgroup.
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(1024)
 finish_step_kernel(const float *__restrict__ pv, const int *__restrict__ pi,
                    int nparts, int *__restrict__ state, int *__restrict__ token_log,
                    const float *__restrict__ table, int64_t hidden, int64_t vocab,
                    float *__restrict__ x, const float *__restrict__ inv_freq,
                    int half, float *__restrict__ rope, int advance, int log_cap) {
-  __shared__ float sv[4];
-  __shared__ int si[4];
+  __shared__ float sv[16];
+  __shared__ int si[16];
   __shared__ int s_tok, s_pos;
+  const int threads = blockDim.x; // 256, or 1024 for thousands of candidates
   if (nparts > 0) {
     float v = -INFINITY;
     int idx = 0x7fffffff;
-    for (int i = threadIdx.x; i < nparts; i += 256)
-      amax_merge(v, idx, pv[i], pi[i]);
+    for (int i0 = threadIdx.x; i0 < nparts; i0 += 4 * threads) { // four loads in flight
+      float cv[4];
+      int ci[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int i = min(i0 + j * threads, nparts - 1);
+        cv[j] = pv[i];
+        ci[j] = pi[i];
+      }
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        if (i0 + j * threads < nparts)
+          amax_merge(v, idx, cv[j], ci[j]);
+    }
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1)
       amax_merge(v, idx, __shfl_xor(v, o, 64), __shfl_xor(idx, o, 64));
@@ -161,7 +174,7 @@ finish_step_kernel(const float *__restrict__ pv, const int *__restrict__ pi,
     }
     __syncthreads();
     if (threadIdx.x == 0) {
-      for (int w = 1; w < 4; ++w)
+      for (int w = 1; w < threads / 64; ++w)
         amax_merge(v, idx, sv[w], si[w]);
       if (idx == 0x7fffffff)
         idx = 0;
@@ -184,7 +197,7 @@ finish_step_kernel(const float *__restrict__ pv, const int *__restrict__ pi,
   if (t < 0 || t >= vocab)
     t = 0;
   const float *row = table + t * hidden;
-  for (int64_t i = threadIdx.x; i < hidden; i += 256)
+  for (int64_t i = threadIdx.x; i < hidden; i += threads)
     x[i] = row[i];
   if (threadIdx.x < half) {
     float sn, cs;
@@ -196,18 +209,16 @@ finish_step_kernel(const float *__restrict__ pv, const int *__restrict__ pi,
 
 } // namespace
 
-int launch_finish_step(void *amax_workspace, int nparts, int *state, int *token_log,
-                       const float *table, int64_t hidden, int64_t vocab, float *x,
-                       const float *inv_freq, int head_dim, float *rope, bool advance,
-                       int token_log_cap, hipStream_t stream) {
+int launch_finish_step(const float *cand_v, const int *cand_i, int nparts, int *state,
+                       int *token_log, const float *table, int64_t hidden, int64_t vocab,
+                       float *x, const float *inv_freq, int head_dim, float *rope,
+                       bool advance, int token_log_cap, hipStream_t stream) {
   BH_REQUIRE(state && table && x && inv_freq && rope && head_dim > 0 &&
-                 head_dim / 2 <= 256 && (nparts == 0 || (amax_workspace && token_log)),
+                 head_dim / 2 <= 256 && (nparts == 0 || (cand_v && cand_i && token_log)),
              "finish_step: bad argument");
-  const float *pv = static_cast<const float *>(amax_workspace);
-  const int *pi = reinterpret_cast<const int *>(pv + kArgmaxParts);
-  hipLaunchKernelGGL(finish_step_kernel, dim3(1), dim3(256), 0, stream, pv, pi, nparts,
-                     state, token_log, table, hidden, vocab, x, inv_freq, head_dim / 2,
-                     rope, advance ? 1 : 0, token_log_cap);
+  hipLaunchKernelGGL(finish_step_kernel, dim3(1), dim3(nparts > 1024 ? 1024 : 256), 0, stream,
+                     cand_v, cand_i, nparts, state, token_log, table, hidden, vocab, x,
+                     inv_freq, head_dim / 2, rope, advance ? 1 : 0, token_log_cap);
   BH_CHECK_HIP(hipGetLastError());
   return BUDDY_HIP_OK;
 }

@@ -34,6 +34,15 @@ struct GemvArgs {
   const int *pos_ptr = nullptr;
   int attn_nchunks = 0, attn_chunk = 0, head_dim = 0;
   int tile_n = 16; // channels per packed tile: 16 (default), 8 or 4
+  // One row with the STORE epilogue, optional: the first maximum of every
+  // channel group's 16 results, (value, index) at [group] of these two arrays
+  // (NaNs are not candidates; a group without one holds (-inf, INT_MAX)), so
+  // that a greedy pick need not read the row again.  *argmax_groups receives
+  // the number of groups written, or 0 when the launch's kernel does not emit
+  // them (the caller then scans the row itself).
+  float *argmax_v = nullptr;
+  int *argmax_i = nullptr;
+  int *argmax_groups = nullptr;
   int M = 1;
   int64_t K = 0, N = 0;
   int epilogue = kEpiStore;

@@ -137,6 +137,9 @@ struct KernelArgs {
   const float *attn_acc, *attn_ml;
   const int *pos_ptr;
   int attn_nchunks, attn_chunk, head_dim;
+  // one row, STORE: per channel group the first maximum of its results, or null
+  float *cand_v;
+  int *cand_i;
 };
 
 typedef int v4i __attribute__((ext_vector_type(4)));
@@ -193,18 +196,49 @@ struct EpilogueOperands {
   float c[M];
 };
 
+// stores one result and returns it
 template <int M, int EPI>
-__device__ __forceinline__ void finish(const KernelArgs &a, int m, int n, float raw0,
-                                       float raw1, const EpilogueOperands<M> &e) {
+__device__ __forceinline__ float finish(const KernelArgs &a, int m, int n, float raw0,
+                                        float raw1, const EpilogueOperands<M> &e) {
   float *c = a.C + (int64_t)m * a.ldc + n;
   const float v = raw0 * e.s0;
+  float y;
   if (EPI == kEpiSiluMul) {
     const float u = raw1 * e.s1;
-    *c = silu(v) * u;
+    y = silu(v) * u;
   } else if (EPI == kEpiAccum) {
-    *c = e.c[m] + v;
+    y = e.c[m] + v;
   } else {
-    *c = a.bias ? e.bias + v : v;
+    y = a.bias ? e.bias + v : v;
+  }
+  *c = y;
+  return y;
+}
+
+// The first maximum of the 16 results of a channel group (lanes 0..15 of the
+// wavefront that finished it; `y` of a lane without a result is ignored):
+// larger value first, then smaller index, NaNs never -- the order of
+// std::max_element over the row.  Lane 0 writes (value, index) for the group.
+__device__ __forceinline__ void emit_group_maximum(const KernelArgs &a, int g, int lane,
+                                                   bool has, float y, int n) {
+  float v = -INFINITY;
+  int i = 0x7fffffff;
+  if (has && y == y) {
+    v = y;
+    i = n;
+  }
+#pragma unroll
+  for (int o = 8; o > 0; o >>= 1) {
+    const float ov = __shfl_xor(v, o, 16);
+    const int oi = __shfl_xor(i, o, 16);
+    if (ov > v || (ov == v && oi < i)) {
+      v = ov;
+      i = oi;
+    }
+  }
+  if (lane == 0) {
+    a.cand_v[g] = v;
+    a.cand_i[g] = i;
   }
 }
 
@@ -892,6 +926,7 @@ __global__ void __launch_bounds__(kMaxWaves *kWave)
       }
     }
   }
+  float y_row = 0.f; // one row: its result of this lane's channel
   if (writer) {
 #pragma unroll
     for (int m = 0; m < M; ++m) {
@@ -905,10 +940,14 @@ __global__ void __launch_bounds__(kMaxWaves *kWave)
           v0 *= r;
           v1 *= r;
         }
-        finish<M, EPI>(a, m, n, v0, v1, epi);
+        const float y = finish<M, EPI>(a, m, n, v0, v1, epi);
+        if (M == 1)
+          y_row = y;
       }
     }
   }
+  if (M == 1 && EPI == kEpiStore && a.cand_v && live)
+    emit_group_maximum(a, g, lane, writer, y_row, n);
   BH_TL(g_tl_gemv, tl_wave, 5);
 }
 
@@ -1574,7 +1613,11 @@ int launch_gemv(const GemvArgs &a, hipStream_t stream) {
       (a.K & 3) == 0 && (a.lda & 3) == 0 &&
       (reinterpret_cast<uintptr_t>(a.A) & 15) == 0 &&
       (!a.norm_w || (reinterpret_cast<uintptr_t>(a.norm_w) & 15) == 0))
+  {
+    if (a.argmax_groups)
+      *a.argmax_groups = 0;
     return batch_bf16() ? launch_gemv_mfma(a, stream) : launch_gemv_i8(a, stream);
+  }
   // the kernel is compiled for 1, 2, 4, 8 and 16 rows; extra rows are zero-
   // filled in LDS and never stored
   const int mt = compiled_rows(a.M);
@@ -1607,6 +1650,14 @@ int launch_gemv(const GemvArgs &a, hipStream_t stream) {
   ka.tiles_per_round = p.tiles_per_round;
   ka.tile_n = a.tile_n;
   ka.rows = a.M;
+  // the per-group maxima come from the f32 kernel of one row (whole groups per
+  // workgroup); other cuts leave the row to the caller
+  const bool emit = a.argmax_v && a.argmax_i && mt == 1 && a.tile_n == 16 && !p.on_digits &&
+                    !p.half_split && !fold && a.epilogue == kEpiStore;
+  ka.cand_v = emit ? a.argmax_v : nullptr;
+  ka.cand_i = emit ? a.argmax_i : nullptr;
+  if (a.argmax_groups)
+    *a.argmax_groups = emit ? (int)p.groups : 0;
   ka.attn_acc = a.attn_acc;
   ka.attn_ml = a.attn_ml;
   ka.pos_ptr = a.pos_ptr;

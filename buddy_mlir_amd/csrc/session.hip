@@ -99,6 +99,8 @@ struct Session {
   float *x = nullptr, *xn = nullptr, *qkv = nullptr, *att = nullptr,
         *h = nullptr, *logits = nullptr;
   void *attn_ws = nullptr, *amax_ws = nullptr;
+  float *group_max_v = nullptr; // first maxima of lm_head's channel groups: values,
+  int *group_max_i = nullptr;   // indices
   size_t attn_ws_bytes = 0;
   int *state = nullptr;     // device: token, pos, step
   int *token_log = nullptr; // device: greedy tokens by step
@@ -251,20 +253,47 @@ struct Session {
       if ((rc = gemv(h, L.down, nullptr, nullptr, x, kEpiAccum)))
         return rc;
     }
-    if ((rc = gemv(x, lm, nullptr, ln_f, logits, kEpiStore)))
-      return rc;
+    // lm_head leaves the first maximum of every 16 logits behind where its cut
+    // allows it; otherwise a launch of its own scans the row
     int nparts = 0;
+    {
+      GemvArgs g;
+      g.A = x;
+      g.lda = lm.K;
+      g.W0 = lm.w;
+      g.s0 = lm.s;
+      g.bias = lm.b;
+      g.norm_w = ln_f;
+      g.norm_eps = S.rms_eps;
+      g.norm_inv_k = 1.0f / (float)lm.K;
+      g.C = logits;
+      g.ldc = lm.N;
+      g.M = 1;
+      g.K = lm.K;
+      g.N = lm.N;
+      g.epilogue = kEpiStore;
+      g.argmax_v = group_max_v;
+      g.argmax_i = group_max_i;
+      g.argmax_groups = &nparts;
+      if ((rc = launch_gemv(g, stream)))
+        return rc;
+    }
+    if (nparts > 0)
+      return launch_finish_step(group_max_v, group_max_i, nparts, state, token_log, embed,
+                                S.hidden, S.vocab, x, inv_freq, S.head_dim, rope, true,
+                                token_log_cap, stream);
     if ((rc = launch_argmax_partial(logits, S.vocab, amax_ws, &nparts, stream)))
       return rc;
-    return launch_finish_step(amax_ws, nparts, state, token_log, embed, S.hidden,
-                              S.vocab, x, inv_freq, S.head_dim, rope, true,
-                              token_log_cap, stream);
+    const float *pv = static_cast<const float *>(amax_ws);
+    return launch_finish_step(pv, reinterpret_cast<const int *>(pv + kArgmaxParts), nparts,
+                              state, token_log, embed, S.hidden, S.vocab, x, inv_freq,
+                              S.head_dim, rope, true, token_log_cap, stream);
   }
 
   // After the host wrote token/position: embedding row and RoPE table of the step.
   int prepare_step() {
     const auto &S = shape;
-    return launch_finish_step(amax_ws, 0, state, token_log, embed, S.hidden, S.vocab,
+    return launch_finish_step(nullptr, nullptr, 0, state, token_log, embed, S.hidden, S.vocab,
                               x, inv_freq, S.head_dim, rope, false, token_log_cap,
                               stream);
   }
@@ -610,6 +639,11 @@ buddy_hip_session *buddy_hip_session_create(const buddy_hip_model_shape *shape,
   s->attn_ws_bytes = bh::attn_decode_workspace_bytes(S.heads, S.max_len);
   rc |= s->alloc((char **)&s->attn_ws, s->attn_ws_bytes);
   rc |= s->alloc((char **)&s->amax_ws, bh::argmax_workspace_bytes());
+  {
+    const size_t groups = (size_t)bh::ceil_div(S.vocab, bh::kTileN);
+    rc |= s->alloc(&s->group_max_v, groups);
+    rc |= s->alloc(&s->group_max_i, groups);
+  }
   for (auto &L : s->layers) {
     rc |= s->alloc(&L.kc, KVN * (size_t)S.max_len);
     rc |= s->alloc(&L.vc, KVN * (size_t)S.max_len);

@@ -369,3 +369,35 @@ def test_qwen2_1p5b_shape_64_greedy_steps(oracle):
     for j in (2 * shape.layers - 2, 2 * shape.layers - 1):
         check_close(sess.get_kv(j)[:, 1024:1088, :], kv[j][:, 1024:1088, :])
     sess.close()
+
+
+def test_greedy_pick_taken_from_the_lm_head_launch_keeps_the_first_maximum(bh, oracle):
+    """Where lm_head runs on the one-row f32 kernel (runs of more than 16 tiles:
+    the shipped shape and this one) its launch leaves the first maximum of every
+    16 logits behind and the step's last kernel picks among those.  Every
+    vocabulary column here is the same int8 vector, so that the logits are the
+    scales times one number and their maxima are ties: the token must be the
+    first of them, whatever the sign of that number."""
+    shape = Shape(layers=1, hidden=1152, heads=9, kv_heads=3, head_dim=128, inter=256,
+                  vocab=70000, max_len=64)
+    from test_gemv_plan import F32, plan as gemv_plan
+    cut = gemv_plan(bh, 1, shape.hidden, shape.vocab)
+    assert cut.kernel == F32 and cut.tiles_per_wavefront > 16 and not cut.split
+    sess, _ = synthetic.build_session(shape, context=0)
+    g = sess._globals
+    w = g["w_lm"]
+    w[:] = w[:, :1]
+    s = torch.ones(shape.vocab, device="cuda")
+    s[[123, 40000, 50001, 69999]] = 2.0  # the maxima when the common product is positive
+    s[[7, 60000]] = 0.5                  # ... and when it is negative
+    sess.set_globals(g["embed"], g["inv_freq"], g["ln_f"], w, s)
+    tok, seen = 11, set()
+    for pos in range(12):
+        nxt, logits = sess.decode(tok, pos)
+        assert (logits == logits.max()).sum() >= 2
+        assert nxt == oracle.argmax_first(logits) == int(np.argmax(logits))
+        assert nxt in (7, 123)
+        seen.add(nxt)
+        tok = (tok * 7919 + 13) % shape.vocab  # other rows of the embedding
+    sess.close()
+    assert len(seen) >= 1
