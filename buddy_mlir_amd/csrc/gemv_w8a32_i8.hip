@@ -61,6 +61,10 @@ struct I8Args {
   int GS, KS;                      // spans x k-slices of wavefronts per workgroup
   int rows;
   bool two_tiles; // up to 8 rows: the variant that converts two tiles at a time
+  // 9..16 rows of a narrow matrix: two workgroups per span, rows 0..7 and 8..15,
+  // each on the two-tile variant (neighbouring workgroup ids, so that the second
+  // reads the weights while the first's requests have them on their way)
+  bool row_split;
 };
 
 __device__ __forceinline__ float silu(float g) {
@@ -216,7 +220,13 @@ __global__ void __launch_bounds__(kMaxWavesI8 *kWave, 3) // 3 wavefronts per SIM
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int sl = wave / a.KS, ks = wave % a.KS;
-  const int span = blockIdx.x * a.GS + sl;
+  const int row_half = a.row_split ? blockIdx.x & 1 : 0;
+  if (a.row_split) { // this workgroup's rows: the first eight or the rest
+    a.A += (int64_t)row_half * 8 * a.lda;
+    a.C += (int64_t)row_half * 8 * a.ldc;
+    a.rows = row_half ? a.rows - 8 : 8;
+  }
+  const int span = (a.row_split ? blockIdx.x >> 1 : blockIdx.x) * a.GS + sl;
   const bool live = span < a.spans;
   const int g0 = (live ? span : 0) * SPAN;
   // what a wavefront's slice is cut from and a fetch brings: chunks, or pairs of
@@ -553,7 +563,7 @@ int launch_kernel(I8Args ka, int ks_forced, hipStream_t stream) {
     if (units / ks < 2)
       continue;
     const int gs = ks < 4 ? 4 / ks : 1, waves = gs * ks;
-    const int64_t blocks = ceil_div(ka.spans, gs);
+    const int64_t blocks = ceil_div(ka.spans, gs) * (ka.row_split ? 2 : 1);
     if (blocks <=
         256 * (int64_t)workgroups_per_cu<EPI, SPAN, NORM, T2>(waves, lds_bytes(ks, waves)))
       break;
@@ -563,7 +573,7 @@ int launch_kernel(I8Args ka, int ks_forced, hipStream_t stream) {
   ka.KS = ks;
   ka.GS = ks < 4 ? 4 / ks : 1;
   const int waves = ka.GS * ka.KS;
-  const int blocks = (int)ceil_div(ka.spans, ka.GS);
+  const int blocks = (int)ceil_div(ka.spans, ka.GS) * (ka.row_split ? 2 : 1);
   BH_NOTE_VARIANT(I8Family, EPI, SPAN, NORM, T2);
   hipLaunchKernelGGL(kernel, dim3(blocks), dim3(waves * kWave), lds_bytes(ks, waves), stream, ka);
   BH_CHECK_HIP(hipGetLastError());
@@ -597,6 +607,13 @@ int launch_span(const I8Args &ka, int epilogue, int ks_forced, hipStream_t strea
     return launch_norm<kEpiSiluMul, (SPAN > 2 ? 2 : SPAN)>(ka, ks_forced, stream);
   }
   return fail(BUDDY_HIP_ERR_ARG, "gemv: unknown epilogue %d", epilogue);
+}
+
+// measurement only: BUDDY_HIP_I8_NO_ROW_SPLIT (any value) keeps 9..16 rows in one
+// workgroup per span (read once per process)
+bool no_row_split() {
+  static bool v = getenv("BUDDY_HIP_I8_NO_ROW_SPLIT") != nullptr;
+  return v;
 }
 
 } // namespace
@@ -644,7 +661,12 @@ int launch_gemv_i8(const GemvArgs &a, hipStream_t stream) {
   // wavefront.  Two matrices with two groups each stay on the one-tile variant
   // (the same four weight tiles per conversion; 4096 -> 2 x 14336 at 8 rows:
   // 26.0 us against 29.0).
-  ka.two_tiles = a.M <= 8 && !(dual && span == 2);
+  // 9..16 rows of a matrix so narrow that at most half of the compute units
+  // would have a workgroup: the rows go to two workgroups of up to 8 rows (each
+  // converts half as much, two tiles at a time; the weights are read twice, the
+  // second time from cache)
+  ka.row_split = a.M > 8 && ka.groups <= 128 && !no_row_split();
+  ka.two_tiles = (a.M <= 8 || ka.row_split) && !(dual && span == 2);
   if (ka.two_tiles && span == 4)
     span = 2;
   ka.spans = (int)ceil_div(ka.groups, span);

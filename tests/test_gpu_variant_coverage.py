@@ -79,7 +79,7 @@ def gemv_case(bh, oracle, M, K, N, epilogue, norm, seed):
         check_close(got[m], want[m])
 
 
-GEMV_I8_N = [320, 8192, 32768]        # 1, 2, 4 channel groups per wavefront
+GEMV_I8_N = [2560, 8192, 32768]       # 1, 2, 4 channel groups per wavefront
 GEMV_BF16_N = [320, 8192, 131072]     # 2, 4, 8
 
 
@@ -88,12 +88,17 @@ def test_every_int8_batch_gemv_variant(bh, oracle):
     # up to 8 rows take the variants that convert two tiles at a time (K = 192:
     # a pair and a last tile without a partner; K = 320 ends inside a pair's
     # second tile), more rows the one-tile variants
+    # (more than 8 rows of a matrix of up to 128 channel groups go to two
+    # workgroups of up to 8 rows on the two-tile variants: the last case)
     for i, N in enumerate(GEMV_I8_N):
         for epilogue in (0, 1, 2):
             for norm in (False, True):
                 gemv_case(bh, oracle, 9 + 3 * i, 192, N, epilogue, norm, 100 + i)
                 if i < 2:
-                    gemv_case(bh, oracle, 5 + 3 * i, 192 + 108 * i, N, epilogue, norm, 150 + i)
+                    gemv_case(bh, oracle, 5 + 3 * i, 192 + 108 * i, (320, 8192)[i], epilogue,
+                              norm, 150 + i)
+                if i == 0:
+                    gemv_case(bh, oracle, 13, 192, 320, epilogue, norm, 170)
     fam = "gemv_w8a32_i8_kernel"
     assert launched(bh, fam) == compiled(bh, fam), compiled(bh, fam) - launched(bh, fam)
 
