@@ -351,7 +351,7 @@ def bench_gemv(bh, args):
 
 
 def bench_mlp(bh, args):
-    """configs[1]: h = SiLU(x G) * (x U), y = h D at M in {1, 4, 16}: two launches
+    """configs[1]: h = SiLU(x G) * (x U), y = h D at M in {1, 4, 16} (--mlp-rows): two launches
     (fused gate|up, then down), 12 rotating weight sets (496 MB)."""
     import torch
 
@@ -359,7 +359,10 @@ def bench_mlp(bh, args):
     gu = _random_packed(H, I, 24)
     dn = _random_packed(I, H, 12)
     res = {}
-    for M in (1, 4, 16):
+    rows = [int(v) for v in args.mlp_rows.split(",")]
+    if any(M < 1 or M > 16 for M in rows) or 1 not in rows:
+        raise SystemExit("--mlp-rows: row counts from 1 to 16, 1 among them")
+    for M in rows:
         x = torch.randn((M, H), device="cuda")
         h = torch.empty((M, I), device="cuda")
         y = torch.zeros((M, H), device="cuda")
@@ -373,7 +376,10 @@ def bench_mlp(bh, args):
         # three int8 matrices, their scales, M rows in and M rows out
         by = 3 * H * I + 4 * (2 * I + H) + 4 * M * 2 * H
         res[f"M={M}"] = {"us": t * 1e6, "gbps": by / t / 1e9,
-                         "frac": by / t / 1e9 / HBM_PEAK_GBPS}
+                         "frac": by / t / 1e9 / HBM_PEAK_GBPS,
+                         # each launch on its own, same rotation
+                         "gate_up_us": _time_launches(f1, 240) * 1e6,
+                         "down_us": _time_launches(f2, 240) * 1e6}
     t = res["M=1"]["us"] * 1e-6
     return {
         "metric": "int8_mlp_hbm_gbps", "value": res["M=1"]["gbps"], "unit": "GB/s",
@@ -849,6 +855,8 @@ def main():
                              "model_abi", "sampler", "quantize"],
                     help="decode (default): the full decode step the headline metric "
                          "is quoted on; the others measure the remaining configurations")
+    ap.add_argument("--mlp-rows", default="1,4,16",
+                    help="--workload mlp: the row counts to time (1..16, comma separated)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-graph", action="store_true")
     ap.add_argument("--calibrate-copy", action="store_true",
