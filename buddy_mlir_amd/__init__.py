@@ -110,6 +110,7 @@ def _declare(lib):
         "buddy_hip_gqa_decode_attention_static": (c_int, [vp, vp, vp, vp, vp, vp, vp, c_int,
                                                           c_int, c_int, c_int, c_float,
                                                           vp]),
+        "buddy_hip_static_scratch_init": (c_int, []),
         "buddy_hip_prefill_attention": (c_int, [vp, vp, vp, vp, vp, c_int, c_int, c_int,
                                                 c_int, c_int, c_float, vp]),
         "buddy_hip_session_create": (vp, [vp, vp]),
@@ -168,6 +169,8 @@ def _declare(lib):
         "_mlir_ciface_buddy_dequant_matmul_i8_f32": (None, [vp, vp, vp, vp]),
         "_mlir_ciface_buddy_dequant_matmul_i8_f32_acc": (None, [vp, vp, vp, vp]),
         "buddy_hip_clear_weight_cache": (None, []),
+        "buddy_hip_set_weight_cache_limit": (None, [sz]),
+        "buddy_hip_weight_cache_stats": (None, [vp]),
     }
     for name, (res, args) in sigs.items():
         if hasattr(lib, name):

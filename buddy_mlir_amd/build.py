@@ -17,16 +17,11 @@ from pathlib import Path
 PKG = Path(__file__).resolve().parent
 ROOT = PKG.parent
 CSRC = PKG / "csrc"
-# a measurement build (BUDDY_HIP_TIMELINE=1) never lands where the product is
-LIBDIR = PKG / ("lib_timeline" if os.environ.get("BUDDY_HIP_TIMELINE") else "lib")
+LIBDIR = PKG / "lib"
 OBJDIR = LIBDIR / "obj"
 LIB = LIBDIR / "libbuddy_hip.so"
 RUNNER_SRC = PKG / "runner" / "buddy_hip_run.cpp"
 RUNNER = LIBDIR / "buddy_hip_run"
-# measurement program: per-kernel cost of a dependent chain (see its header)
-PROBE_SRC = PKG / "runner" / "launch_floor_probe.hip"
-PROBE_KERNELS = PKG / "runner" / "launch_floor_kernels.hip"
-PROBE = LIBDIR / "launch_floor_probe"
 
 ARCH = "gfx950"
 # -packed-fp32-ops off: scalar float code must not be turned into v_pk_*_f32.
@@ -36,12 +31,6 @@ COMMON = [
     "-Wno-unused-command-line-argument", "-Wno-unknown-warning-option",
     f"-I{ROOT / 'include'}", f"-I{CSRC}",
 ]
-
-
-# BUDDY_HIP_TIMELINE=1: a measurement build whose kernels record phase timestamps
-# (see BH_TL in csrc/common.h).  Never the shipped build.
-if os.environ.get("BUDDY_HIP_TIMELINE"):
-    COMMON.append("-DBH_TIMELINE")
 
 
 # Kernels of these files issue global loads through inline asm and wait for them
@@ -129,22 +118,6 @@ def build(force: bool = False, jobs: int = 8, verbose: bool = True) -> Path:
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError(f"runner build failed:\n{r.stdout}\n{r.stderr}")
-    # the launch-floor probe: its kernels are built twice, plain and with the
-    # first 14 kernel-argument words preloaded into SGPRs
-    hip = [_hipcc(), *COMMON, f"-I{PKG / 'runner'}", "-x", "hip", "-c"]
-    pk_plain, pk_pre, pk_main = (OBJDIR / n for n in
-                                 ("probe_plain.o", "probe_preload.o", "probe_main.o"))
-    for cmd in (
-        [*hip, str(PROBE_KERNELS), "-DPROBE_NS=plain", "-o", str(pk_plain)],
-        [*hip, str(PROBE_KERNELS), "-DPROBE_NS=preload", "-mllvm",
-         "-amdgpu-kernarg-preload-count=14", "-o", str(pk_pre)],
-        [*hip, str(PROBE_SRC), "-o", str(pk_main)],
-        [_hipcc(), f"--offload-arch={ARCH}", str(pk_main), str(pk_plain), str(pk_pre),
-         f"-L{LIBDIR}", "-lbuddy_hip", "-Wl,-rpath,$ORIGIN", "-o", str(PROBE)],
-    ):
-        r = subprocess.run(cmd, capture_output=True, text=True)
-        if r.returncode != 0:
-            raise RuntimeError(f"probe build failed:\n{' '.join(cmd)}\n{r.stdout}\n{r.stderr}")
     if verbose:
         print(f"built {LIB} from {len(srcs)} sources, and {RUNNER.name}")
     return LIB

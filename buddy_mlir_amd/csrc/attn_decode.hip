@@ -24,12 +24,11 @@
 // folds them in chunk order with the reference's own combine rule.
 #include "attn.h"
 
-#include <mutex>
+#include <atomic>
 
 namespace bh {
 namespace {
 
-BH_TL_DECLARE(g_tl_attn)
 
 constexpr int kChunk = kAttnChunk; // cache positions per workgroup
 constexpr int kThreads = 256;
@@ -75,8 +74,6 @@ __global__ void __launch_bounds__(kThreads) attn_decode_partial(AttnArgs a) {
   const int tid = threadIdx.x;
   const int wave = tid >> 6, lane = tid & 63;
   const int hb = blockIdx.x / a.pairs_padded, ckv = blockIdx.x % a.pairs_padded;
-  [[maybe_unused]] const int tl_wave = blockIdx.x * kWaves + wave;
-  BH_TL(g_tl_attn, tl_wave, 0);
   if (ckv >= a.nchunks * a.kv_heads)
     return; // padding id
   const int chunk = ckv % a.nchunks, kvh = ckv / a.nchunks;
@@ -141,7 +138,6 @@ __global__ void __launch_bounds__(kThreads) attn_decode_partial(AttnArgs a) {
     }
     return;
   }
-  BH_TL(g_tl_attn, tl_wave, 1);
   const bool has_new = pos < p0 + kChunk; // the token's own row lies in this chunk
 
   // ---- RoPE: q' = q*cos + cat(-q[64:], q[:64])*sin, same for the new k ------
@@ -160,11 +156,9 @@ __global__ void __launch_bounds__(kThreads) attn_decode_partial(AttnArgs a) {
     }
   }
   __syncthreads();
-  BH_TL(g_tl_attn, tl_wave, 2);
 
   // ---- scores of this wavefront's 16 positions ------------------------------
   // every lane of a half ends up with the 8 scores of its half's rows
-  BH_TL_AFTER(g_tl_attn, tl_wave, 6, kreg[kR - 1].x);
   const float4 q4 = *reinterpret_cast<const float4 *>(q_s + c4 * 4);
   float sc[kR];
 #pragma unroll
@@ -191,8 +185,6 @@ __global__ void __launch_bounds__(kThreads) attn_decode_partial(AttnArgs a) {
     l_w += sc[i];
   }
   l_w += __shfl_xor(l_w, 32, 64);
-  BH_TL(g_tl_attn, tl_wave, 3);
-  BH_TL_AFTER(g_tl_attn, tl_wave, 7, vreg[kR - 1].x);
 
   // ---- acc[d] = sum_p e[p] * V[p][d]: this lane's 8 rows x 4 dims -----------
   float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
@@ -220,7 +212,6 @@ __global__ void __launch_bounds__(kThreads) attn_decode_partial(AttnArgs a) {
     lw_s[wave] = l_w;
   }
   __syncthreads();
-  BH_TL(g_tl_attn, tl_wave, 4);
 
   // ---- the four wavefronts meet: one partial per (head, chunk) --------------
   if (tid < kD) {
@@ -241,7 +232,6 @@ __global__ void __launch_bounds__(kThreads) attn_decode_partial(AttnArgs a) {
       a.part_ml[((size_t)h * a.nchunks + chunk) * 2 + 1] = l;
     }
   }
-  BH_TL(g_tl_attn, tl_wave, 5);
 }
 
 // Folds the partials of one head in chunk order with the reference's combine
@@ -278,22 +268,34 @@ __global__ void __launch_bounds__(kD) attn_decode_combine(AttnArgs a) {
 constexpr int kStaticPartials = 8192;
 constexpr int kMaxDevices = 64;
 static __device__ __align__(256) float g_attn_scratch[(size_t)kStaticPartials * (kD + 2)];
-std::mutex g_scratch_mu;
-float *g_scratch_ptr[kMaxDevices] = {};
+std::atomic<float *> g_scratch_ptr[kMaxDevices] = {};
 
-// Device address of the current device's copy of g_attn_scratch.
-int static_scratch(float **out) {
+// Device address of the current device's copy of g_attn_scratch.  The first
+// call on a device asks the runtime (hipGetSymbolAddress, which may load the
+// code object); that must not happen inside a stream capture, so a capturing
+// caller that has not made an eager call or buddy_hip_static_scratch_init() on
+// this device first is refused.  Later calls are one atomic load.
+int static_scratch(float **out, hipStream_t stream) {
   int dev = -1;
   BH_CHECK_HIP(hipGetDevice(&dev));
   BH_REQUIRE(dev >= 0 && dev < kMaxDevices, "attn_decode: device index %d", dev);
-  std::lock_guard<std::mutex> lock(g_scratch_mu);
-  if (!g_scratch_ptr[dev]) {
-    void *p = nullptr;
-    BH_CHECK_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(g_attn_scratch)));
-    BH_REQUIRE(p, "attn_decode: no device address for the static scratch");
-    g_scratch_ptr[dev] = static_cast<float *>(p);
+  float *p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+  if (!p) {
+    if (stream) {
+      hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+      BH_CHECK_HIP(hipStreamIsCapturing(stream, &st));
+      BH_REQUIRE(st == hipStreamCaptureStatusNone,
+                 "attn_decode_static: call buddy_hip_static_scratch_init() on this device "
+                 "before capturing");
+    }
+    void *q = nullptr;
+    BH_CHECK_HIP(hipGetSymbolAddress(&q, HIP_SYMBOL(g_attn_scratch)));
+    BH_REQUIRE(q, "attn_decode: no device address for the static scratch");
+    p = static_cast<float *>(q);
+    // two threads may both ask: they get the same address
+    g_scratch_ptr[dev].store(p, std::memory_order_release);
   }
-  *out = g_scratch_ptr[dev];
+  *out = p;
   return BUDDY_HIP_OK;
 }
 
@@ -356,7 +358,6 @@ int launch_attn_decode(const AttnDecodeArgs &in, hipStream_t stream) {
   return BUDDY_HIP_OK;
 }
 
-BH_TL_EXPORT(buddy_hip_debug_timeline_attn, g_tl_attn)
 } // namespace bh
 
 extern "C" {
@@ -404,7 +405,7 @@ int buddy_hip_gqa_decode_attention_static(const float *qkv, const float *inv_fre
              "scratch of %d partials; use buddy_hip_gqa_decode_attention with a workspace",
              bh::kAttnChunk, (long long)pairs, bh::kStaticPartials);
   float *scratch = nullptr;
-  int rc = bh::static_scratch(&scratch);
+  int rc = bh::static_scratch(&scratch, bh::as_stream(stream));
   if (rc)
     return rc;
   bh::AttnDecodeArgs a;
@@ -424,4 +425,9 @@ int buddy_hip_gqa_decode_attention_static(const float *qkv, const float *inv_fre
   a.workspace_bytes = sizeof(float) * (size_t)bh::kStaticPartials * (bh::kAttnHeadDim + 2);
   return bh::launch_attn_decode(a, bh::as_stream(stream));
 } BH_CATCH_INT("buddy_hip_gqa_decode_attention_static")
+
+int buddy_hip_static_scratch_init(void) try {
+  float *scratch = nullptr;
+  return bh::static_scratch(&scratch, nullptr);
+} BH_CATCH_INT("buddy_hip_static_scratch_init")
 }

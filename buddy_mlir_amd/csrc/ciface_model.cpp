@@ -54,6 +54,11 @@ struct ModelState {
   // its position, gen_session.py:1471-1511): the device cache is then reloaded
   // from them.
   long long expected_pos = -1;
+  // Set by a device-side discard (buddy_hip_forward_discard_kv): the caller's
+  // tensors were not shifted, so from then on only the device cache is whole
+  // and a decode at any position keeps it.  Cleared by invalidate_kv, reset
+  // and a prefill.
+  bool device_is_truth = false;
 };
 
 // malloc'd host memory that is freed unless handed over
@@ -172,6 +177,7 @@ void destroy_locked(ModelState &m) {
     (void)hipHostFree(m.pinned_rows);
   m.pinned_rows = nullptr;
   m.expected_pos = -1;
+  m.device_is_truth = false;
   m.sess = nullptr;
   m.dev_f32 = nullptr;
   m.pinned_logits = nullptr;
@@ -370,7 +376,8 @@ int forward_decode(DecodeResult *res, buddy_memref_f32_1d *f32, buddy_memref_i8_
   // writes its new rows through to the caller's tensors (below), so the caller
   // may edit them between calls.  It has done so when the position is not the
   // one that follows the last step; the device copy is then loaded again.
-  if (m.kv_on_device && m.expected_pos >= 0 && position != m.expected_pos)
+  if (m.kv_on_device && !m.device_is_truth && m.expected_pos >= 0 &&
+      position != m.expected_pos)
     m.kv_on_device = false;
   if (!m.kv_on_device) { // the caller's cache is the truth
     for (int i = 0; i < 2 * kLayers; ++i)
@@ -496,6 +503,7 @@ int forward_prefill(PrefillResult *res, buddy_memref_f32_1d *f32,
   // nothing below can fail: the buffers now belong to the caller
   float *logits = logits_buf.release<float>();
   m.expected_pos = -1; // the prompt length is the caller's knowledge
+  m.device_is_truth = false; // the caller receives the whole cache below
   m.kv_on_device = true;
   for (int i = 0; i < 2 * kLayers; ++i) {
     buddy_memref_f32_4d &d = res->kv[i];
@@ -615,8 +623,10 @@ int buddy_hip_forward_discard_kv(int keep, int discard, int count) try {
     return bh::fail(BUDDY_HIP_ERR_ARG,
                     "forward_discard_kv: no device-resident KV cache yet");
   int rc = buddy_hip_session_discard_kv(m.sess, keep, discard, count);
-  if (!rc) // the device cache is now ahead of the caller's tensors: never reload
+  if (!rc) { // the device cache is now ahead of the caller's tensors: never reload
     m.expected_pos = -1;
+    m.device_is_truth = true;
+  }
   return rc;
 } BH_CATCH_INT("buddy_hip_forward_discard_kv")
 
@@ -624,6 +634,7 @@ void buddy_hip_forward_invalidate_kv(void) try {
   bh::ModelState &m = bh::state();
   std::lock_guard<std::mutex> lock(m.mu);
   m.kv_on_device = false;
+  m.device_is_truth = false;
   m.expected_pos = -1;
 } BH_CATCH_VOID("buddy_hip_forward_invalidate_kv")
 }

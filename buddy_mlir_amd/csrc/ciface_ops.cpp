@@ -52,7 +52,20 @@ struct DeviceBuffer {
 struct CachedWeight {
   int8_t *packed = nullptr;
   float *scale = nullptr;
+  uint64_t fingerprint = 0; // of the caller's W and scale when it was packed
+  size_t bytes = 0;         // device bytes held
+  uint64_t last_use = 0;    // the context's call counter at the last hit
 };
+
+// What the weight cache compares on every hit: up to 64 leading elements of
+// four rows of W (first, 1/3, 2/3, last) and the first and last 16 scales,
+// folded with the shape.  A buffer that was freed and reused at the same
+// address with other contents almost surely differs in one of them; a change
+// confined to bytes that are not sampled is not seen (the documented remedy is
+// buddy_hip_clear_weight_cache).
+constexpr int kFpRowBytes = 64;
+constexpr int kFpRows = 4;
+constexpr int kFpScales = 16;
 
 struct OpContext {
   std::mutex mu;
@@ -61,6 +74,20 @@ struct OpContext {
   std::map<std::tuple<const void *, const void *, int64_t, int64_t>,
            CachedWeight>
       weights;
+  size_t cache_bytes = 0;            // sum of the entries' device bytes
+  size_t cache_limit = default_cache_limit();
+  uint64_t calls = 0, uploads = 0, evictions = 0;
+  unsigned char *fp_stage = nullptr; // pinned: samples of device-resident operands
+
+  static size_t default_cache_limit() {
+    if (const char *e = std::getenv("BUDDY_HIP_WEIGHT_CACHE_BYTES")) {
+      char *end = nullptr;
+      const unsigned long long v = std::strtoull(e, &end, 10);
+      if (end != e)
+        return (size_t)v;
+    }
+    return (size_t)16 << 30; // a Llama-3-8B-sized int8 model twice over
+  }
 
   int ensure_stream() {
     if (stream)
@@ -153,26 +180,122 @@ int fill_weight(OpContext &c, const int8_t *w_dev, const float *s, intptr_t sstr
   return BUDDY_HIP_OK;
 }
 
+uint64_t fold(uint64_t h, const void *data, size_t n) { // FNV-1a
+  const unsigned char *b = static_cast<const unsigned char *>(data);
+  for (size_t i = 0; i < n; ++i)
+    h = (h ^ b[i]) * 0x100000001b3ull;
+  return h;
+}
+
+// Fingerprint of the caller's operands as they are now (see kFpRowBytes).
+int fingerprint_of(OpContext &c, const int8_t *w, intptr_t ws0, intptr_t ws1, const float *s,
+                   intptr_t sstride, int64_t K, int64_t N, uint64_t *out) {
+  const int64_t rows[kFpRows] = {0, K / 3, (2 * K) / 3, K - 1};
+  const int64_t nb = N < kFpRowBytes ? N : kFpRowBytes;
+  const int64_t ns = N < kFpScales ? N : kFpScales;
+  int8_t wsample[kFpRows * kFpRowBytes] = {};
+  float ssample[2 * kFpScales] = {};
+  const bool w_dev = is_device_pointer(w), s_dev = is_device_pointer(s);
+  if (w_dev || s_dev) {
+    if (!c.fp_stage)
+      BH_CHECK_HIP(hipHostMalloc((void **)&c.fp_stage, sizeof(wsample) + sizeof(ssample)));
+  }
+  if (w_dev) {
+    BH_REQUIRE(ws1 == 1, "device operand with non-unit inner stride");
+    for (int r = 0; r < kFpRows; ++r)
+      BH_CHECK_HIP(hipMemcpyAsync(c.fp_stage + r * kFpRowBytes, w + rows[r] * ws0, (size_t)nb,
+                                  hipMemcpyDeviceToHost, c.stream));
+  } else {
+    for (int r = 0; r < kFpRows; ++r)
+      for (int64_t j = 0; j < nb; ++j)
+        wsample[r * kFpRowBytes + j] = w[rows[r] * ws0 + j * ws1];
+  }
+  if (s_dev) {
+    float *dst = reinterpret_cast<float *>(c.fp_stage + sizeof(wsample));
+    BH_CHECK_HIP(hipMemcpy2DAsync(dst, sizeof(float), s, sizeof(float) * sstride, sizeof(float),
+                                  (size_t)ns, hipMemcpyDeviceToHost, c.stream));
+    BH_CHECK_HIP(hipMemcpy2DAsync(dst + kFpScales, sizeof(float), s + (N - ns) * sstride,
+                                  sizeof(float) * sstride, sizeof(float), (size_t)ns,
+                                  hipMemcpyDeviceToHost, c.stream));
+  } else {
+    for (int64_t j = 0; j < ns; ++j) {
+      ssample[j] = s[j * sstride];
+      ssample[kFpScales + j] = s[(N - ns + j) * sstride];
+    }
+  }
+  if (w_dev || s_dev) {
+    BH_CHECK_HIP(hipStreamSynchronize(c.stream));
+    if (w_dev)
+      std::memcpy(wsample, c.fp_stage, (size_t)kFpRows * kFpRowBytes);
+    if (s_dev)
+      std::memcpy(ssample, c.fp_stage + sizeof(wsample), sizeof(ssample));
+  }
+  uint64_t h = 0xcbf29ce484222325ull;
+  h = fold(h, &K, sizeof(K));
+  h = fold(h, &N, sizeof(N));
+  h = fold(h, wsample, sizeof(wsample));
+  h = fold(h, ssample, sizeof(ssample));
+  *out = h;
+  return BUDDY_HIP_OK;
+}
+
+void drop_entry(OpContext &c, CachedWeight &cw) {
+  (void)hipFree(cw.packed);
+  (void)hipFree(cw.scale);
+  c.cache_bytes -= cw.bytes;
+}
+
+// Frees least recently used entries until `incoming` more bytes fit under the
+// limit (or nothing is left: an entry larger than the limit is still kept for
+// the call that needs it and goes first the next time).  The stream is idle:
+// every operator call ends with a synchronisation.
+void make_room(OpContext &c, size_t incoming) {
+  while (!c.weights.empty() && c.cache_bytes + incoming > c.cache_limit) {
+    auto oldest = c.weights.begin();
+    for (auto it = c.weights.begin(); it != c.weights.end(); ++it)
+      if (it->second.last_use < oldest->second.last_use)
+        oldest = it;
+    drop_entry(c, oldest->second);
+    c.weights.erase(oldest);
+    ++c.evictions;
+  }
+}
+
 int get_weight(OpContext &c, buddy_memref_i8_2d *W, buddy_memref_f32_2d *scale,
                int64_t K, int64_t N, CachedWeight *out) {
   const int8_t *w = data_of(W->aligned, W->offset);
   const float *s = data_of(scale->aligned, scale->offset);
-  auto key = std::make_tuple((const void *)w, (const void *)s, K, N);
-  auto it = c.weights.find(key);
-  if (it != c.weights.end()) {
-    *out = it->second;
-    return BUDDY_HIP_OK;
-  }
   // scale: N values along whichever axis is not 1
   const int64_t sn = (int64_t)scale->sizes[0] * (int64_t)scale->sizes[1];
   BH_REQUIRE(sn == N, "dequant_matmul: scale has %lld values, N=%lld",
              (long long)sn, (long long)N);
   const intptr_t sstride = scale->sizes[1] == N ? scale->strides[1]
                                                 : scale->strides[0];
+  uint64_t fp = 0;
+  int rc = fingerprint_of(c, w, W->strides[0], W->strides[1], s, sstride, K, N, &fp);
+  if (rc)
+    return rc;
+  ++c.calls;
+  auto key = std::make_tuple((const void *)w, (const void *)s, K, N);
+  auto it = c.weights.find(key);
+  if (it != c.weights.end()) {
+    if (it->second.fingerprint == fp) {
+      it->second.last_use = c.calls;
+      *out = it->second;
+      return BUDDY_HIP_OK;
+    }
+    // same addresses, other contents: the buffer was rewritten or reused
+    drop_entry(c, it->second);
+    c.weights.erase(it);
+  }
   CachedWeight cw;
+  cw.fingerprint = fp;
+  cw.last_use = c.calls;
+  cw.bytes = buddy_hip_w8_packed_bytes(K, N) + sizeof(float) * (size_t)N;
+  make_room(c, cw.bytes);
   const int8_t *w_dev = nullptr;
-  int rc = to_device(c, w, is_device_pointer(w), K, N, W->strides[0],
-                     W->strides[1], c.w_stage, &w_dev);
+  rc = to_device(c, w, is_device_pointer(w), K, N, W->strides[0],
+                 W->strides[1], c.w_stage, &w_dev);
   if (rc)
     return rc;
   rc = fill_weight(c, w_dev, s, sstride, K, N, &cw);
@@ -184,6 +307,8 @@ int get_weight(OpContext &c, buddy_memref_i8_2d *W, buddy_memref_f32_2d *scale,
     return rc;
   }
   c.weights.emplace(key, cw);
+  c.cache_bytes += cw.bytes;
+  ++c.uploads;
   *out = cw;
   return BUDDY_HIP_OK;
 }
@@ -338,10 +463,29 @@ void buddy_hip_clear_weight_cache(void) try {
   std::lock_guard<std::mutex> lock(c.mu);
   if (c.stream)
     (void)hipStreamSynchronize(c.stream);
-  for (auto &kv : c.weights) {
-    (void)hipFree(kv.second.packed);
-    (void)hipFree(kv.second.scale);
-  }
+  for (auto &kv : c.weights)
+    bh::drop_entry(c, kv.second);
   c.weights.clear();
 } BH_CATCH_VOID("buddy_hip_clear_weight_cache")
+
+void buddy_hip_set_weight_cache_limit(size_t bytes) try {
+  bh::OpContext &c = bh::ctx();
+  std::lock_guard<std::mutex> lock(c.mu);
+  if (c.stream)
+    (void)hipStreamSynchronize(c.stream);
+  c.cache_limit = bytes;
+  bh::make_room(c, 0);
+} BH_CATCH_VOID("buddy_hip_set_weight_cache_limit")
+
+void buddy_hip_weight_cache_stats(buddy_hip_weight_cache_info *info) try {
+  if (!info)
+    return;
+  bh::OpContext &c = bh::ctx();
+  std::lock_guard<std::mutex> lock(c.mu);
+  info->entries = (int64_t)c.weights.size();
+  info->bytes = (int64_t)c.cache_bytes;
+  info->limit_bytes = (int64_t)c.cache_limit;
+  info->uploads = (int64_t)c.uploads;
+  info->evictions = (int64_t)c.evictions;
+} BH_CATCH_VOID("buddy_hip_weight_cache_stats")
 }

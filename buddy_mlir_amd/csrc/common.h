@@ -3,6 +3,7 @@
 
 #include <hip/hip_runtime.h>
 
+#include <atomic>
 #include <cstdarg>
 #include <cstdint>
 #include <initializer_list>
@@ -49,6 +50,28 @@ int caught(const char *where) noexcept;
     return nullptr;                                                            \
   }
 
+// A kernel that asks for more dynamic LDS than the default limit needs
+// hipFuncAttributeMaxDynamicSharedMemorySize raised once per device.  One
+// DynLdsOnce per launch site (a function-local static) keeps a bit per device;
+// host threads that launch at the same time on separate streams may both make
+// the (idempotent) call, none skips it before it has succeeded.
+struct DynLdsOnce {
+  std::atomic<uint64_t> done{0};
+};
+inline hipError_t ensure_dyn_lds(DynLdsOnce &once, const void *kernel, int bytes) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess)
+    return e;
+  const uint64_t bit = 1ull << (dev & 63);
+  if (once.done.load(std::memory_order_acquire) & bit)
+    return hipSuccess;
+  e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+  if (e == hipSuccess)
+    once.done.fetch_or(bit, std::memory_order_release);
+  return e;
+}
+
 inline hipStream_t as_stream(buddy_hip_stream s) {
   return reinterpret_cast<hipStream_t>(s);
 }
@@ -57,39 +80,6 @@ constexpr int kWave = 64;          // gfx950 wavefront
 constexpr int kTileN = 16;         // output channels per packed tile
 constexpr int kTileK = 64;         // k values per packed tile
 constexpr int kTileBytes = 1024;   // one wavefront-wide 128-bit load
-
-// Phase timestamps inside a kernel, for builds made with BUDDY_HIP_TIMELINE=1 in
-// the environment (never the shipped build): lane 0 of a wavefront records the
-// constant-rate 100 MHz clock into slot `slot` of its row of a per-file device
-// array, which a debug export copies out.  Empty otherwise.
-#if defined(BH_TIMELINE) && defined(__HIPCC__)
-#define BH_TL_DECLARE(name) static __device__ unsigned long long name[1 << 18];
-#define BH_TL(name, wave_id, slot)                                             \
-  do {                                                                         \
-    if ((threadIdx.x & 63) == 0)                                               \
-      name[(((size_t)(wave_id)) * 8 + (slot)) & ((1u << 18) - 1)] = wall_clock64(); \
-  } while (0)
-// the same once `value` (the result of a load) has arrived
-#define BH_TL_AFTER(name, wave_id, slot, value)                                \
-  do {                                                                         \
-    asm volatile("" ::"v"(value));                                             \
-    BH_TL(name, wave_id, slot);                                                \
-  } while (0)
-#define BH_TL_EXPORT(fn, name)                                                 \
-  extern "C" int fn(unsigned long long *dst, size_t count) {                   \
-    return (int)hipMemcpyFromSymbol(dst, HIP_SYMBOL(name),                     \
-                                    sizeof(unsigned long long) * count);       \
-  }
-#else
-#define BH_TL_DECLARE(name)
-#define BH_TL(name, wave_id, slot)                                             \
-  do {                                                                         \
-  } while (0)
-#define BH_TL_AFTER(name, wave_id, slot, value)                                \
-  do {                                                                         \
-  } while (0)
-#define BH_TL_EXPORT(fn, name)
-#endif
 
 // ---- which template instantiations of the hand-scheduled kernels were launched
 // Every instantiation a launch site can reach registers itself when the library
@@ -155,6 +145,18 @@ __device__ __forceinline__ float wave_sum(float v) {
 __device__ __forceinline__ float wave_max(float v) {
   v = row16_max(v);
   return fmaxf(fmaxf(lane_f(v, 0), lane_f(v, 16)), fmaxf(lane_f(v, 32), lane_f(v, 48)));
+}
+// Maximum of an unsigned value over the 64 lanes.  With the bit pattern of |x|
+// (sign cleared) as the value this is a magnitude maximum in which a NaN or an
+// infinity wins over every finite number, where fmaxf would drop a NaN.
+__device__ __forceinline__ unsigned wave_max_u32(unsigned v) {
+  v = max(v, (unsigned)__builtin_amdgcn_update_dpp(0, (int)v, 0xB1, 0xf, 0xf, true));
+  v = max(v, (unsigned)__builtin_amdgcn_update_dpp(0, (int)v, 0x4E, 0xf, 0xf, true));
+  v = max(v, (unsigned)__builtin_amdgcn_update_dpp(0, (int)v, 0x141, 0xf, 0xf, true));
+  v = max(v, (unsigned)__builtin_amdgcn_update_dpp(0, (int)v, 0x140, 0xf, 0xf, true));
+  const unsigned a = __builtin_amdgcn_readlane((int)v, 0), b = __builtin_amdgcn_readlane((int)v, 16);
+  const unsigned c = __builtin_amdgcn_readlane((int)v, 32), d = __builtin_amdgcn_readlane((int)v, 48);
+  return max(max(a, b), max(c, d));
 }
 // v of this lane and v of lane ^ 32 (W = 32) or lane ^ 16 (W = 16), in an order
 // that depends on the lane: for commutative merges.  One VALU instruction

@@ -17,9 +17,11 @@
 // The only rounding of the whole product is that of X: at most s/2 per element,
 // i.e. 2^-(8D-1) of the row's largest magnitude (D = 3: 2^-23, the rounding an
 // f32 sum of the same row makes when it adds the largest term; D = 2: 2^-15).
-// The sums themselves are exact and do not depend on any order.  NaN and
-// infinity do not survive the conversion to integers: the bf16 modes are the
-// ones that propagate them.  |d q| <= 2^14, so K may not exceed 2^17.
+// The sums themselves are exact and do not depend on any order.  A row that
+// holds a NaN or an infinity gets a NaN step, so every result of that row is
+// NaN, as a NaN spreads through the reference's f32 multiply-add chain over the
+// row (an infinity gives the reference +-inf or NaN per column; here NaN).
+// |d q| <= 2^14, so K may not exceed 2^17.
 //
 // Digit planes lie like the bf16 terms do: [digit][row][k] int8, rows and k zero
 // padded, followed by the row steps (f32 [rows_padded]).  A lane's operand is 16
@@ -112,29 +114,37 @@ __device__ __forceinline__ void row_to_digits(const F &f, int n, int row, int D,
                                               int Kp, int8_t *planes, float *red,
                                               float *cache) {
   const bool cached = Kp <= kRowCache;
-  float mx = 0.f;
+  // the row's largest magnitude as the largest bit pattern of |v|: a NaN or an
+  // infinity is then the maximum (fmaxf would drop a NaN) and gives the row a
+  // NaN step, so that every result of the row is NaN -- what the reference's f32
+  // multiply-add chain makes of such a row (MatMulBlisVectorization.cpp:644-740)
+  unsigned mb = 0;
+  constexpr unsigned kAbs = 0x7fffffffu;
 #pragma unroll 3
   for (int k0 = threadIdx.x * 4; k0 < Kp; k0 += kRowThreads * 4) {
     float v[4];
     f(k0, v);
-    mx = fmaxf(fmaxf(mx, fmaxf(fabsf(v[0]), fabsf(v[1]))), fmaxf(fabsf(v[2]), fabsf(v[3])));
+    mb = max(max(mb, max(__float_as_uint(v[0]) & kAbs, __float_as_uint(v[1]) & kAbs)),
+             max(__float_as_uint(v[2]) & kAbs, __float_as_uint(v[3]) & kAbs));
     if (cached)
       *reinterpret_cast<float4 *>(cache + k0) = make_float4(v[0], v[1], v[2], v[3]);
   }
-  mx = wave_max(mx);
+  mb = wave_max_u32(mb);
   __syncthreads(); // red may still be read by the caller's own reduction
   if ((threadIdx.x & 63) == 0)
-    red[threadIdx.x >> 6] = mx;
+    red[threadIdx.x >> 6] = __uint_as_float(mb);
   __syncthreads();
   {
-    float m2 = red[0];
+    unsigned m2 = __float_as_uint(red[0]);
 #pragma unroll
     for (int w = 1; w < kRowThreads / 64; ++w)
-      m2 = fmaxf(m2, red[w]);
-    mx = m2;
+      m2 = max(m2, __float_as_uint(red[w]));
+    mb = m2;
   }
-  const float step = digit_step(mx, D);
-  const float inv = 1.0f / step; // a power of two as well
+  const bool finite = mb < 0x7f800000u;
+  const float step = finite ? digit_step(__uint_as_float(mb), D) : __uint_as_float(0x7fc00000u);
+  // a power of two as well; the digits of a non-finite row are left zero
+  const float inv = finite ? 1.0f / step : 0.f;
   float *steps = reinterpret_cast<float *>(planes + (size_t)D * Mp * Kp);
   if (threadIdx.x == 0)
     steps[row] = step;
@@ -150,7 +160,7 @@ __device__ __forceinline__ void row_to_digits(const F &f, int n, int row, int D,
     int X[4];
 #pragma unroll
     for (int e = 0; e < 4; ++e)
-      X[e] = (int)rintf(v[e] * inv);
+      X[e] = finite ? (int)rintf(v[e] * inv) : 0;
     int8_t *dst = planes + (size_t)row * Kp + k0;
     for (int j = 0; j < D; ++j) {
       unsigned word = 0;
@@ -848,12 +858,9 @@ int launch_wide(const GemmI8Args &a, unsigned blocks, hipStream_t stream) {
                    (PAIR ? sizeof(float4) * kSlices * ((RB + 1) / 2) * GPW * kWave : 0));
   auto kernel = gemm_w8_i8_wide_kernel<D, RB, GPW, PAIR>;
   if (lds > 48 * 1024) {
-    static bool attr_set = false;
-    if (!attr_set) {
-      BH_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-      attr_set = true;
-    }
+    static DynLdsOnce dyn_lds;
+    BH_CHECK_HIP(ensure_dyn_lds(dyn_lds, reinterpret_cast<const void *>(kernel),
+                                (int)lds));
   }
   BH_NOTE_VARIANT(WideFamily, D, RB, GPW, (int)PAIR);
   hipLaunchKernelGGL(kernel, dim3(blocks), dim3(kSlices * kWave), lds, stream, a);
@@ -937,12 +944,9 @@ int workspace_for(hipStream_t stream, size_t bytes, char **out) {
 template <int D> int launch_split(const GemmI8Args &a, unsigned blocks, hipStream_t stream) {
   constexpr size_t lds = sizeof(float) * kSlices * 64 * kWave;
   auto kernel = gemm_w8_i8_kernel<D>;
-  static bool attr_set = false;
-  if (!attr_set) {
-    BH_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
-                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-    attr_set = true;
-  }
+  static DynLdsOnce dyn_lds;
+  BH_CHECK_HIP(ensure_dyn_lds(dyn_lds, reinterpret_cast<const void *>(kernel),
+                              (int)lds));
   BH_NOTE_VARIANT(SplitFamily, D);
   hipLaunchKernelGGL(kernel, dim3(blocks), dim3(kSlices * kWave), lds, stream, a);
   BH_CHECK_HIP(hipGetLastError());
@@ -1101,8 +1105,15 @@ int launch_gemm_w8_digits(const GemmW8Args &in, const void *planes, hipStream_t 
   const GemmStagingLayout next = gemm_staging_layout(in.M, in.N);
   if (in.then_norm_w && next.cols_padded <= kRowCache) {
     // the kernel that adds the slices holds whole rows: it writes the planes too
+    const size_t row_lds = 2 * sizeof(float) * (size_t)next.cols_padded;
+    if (row_lds > 48 * 1024) { // up to 96 KiB at kRowCache columns
+      static DynLdsOnce dyn_lds;
+      BH_CHECK_HIP(ensure_dyn_lds(dyn_lds,
+                                  reinterpret_cast<const void *>(reduce_slices_norm_kernel),
+                                  (int)(2 * sizeof(float) * kRowCache)));
+    }
     hipLaunchKernelGGL(reduce_slices_norm_kernel, dim3((unsigned)a.M), dim3(kRowThreads),
-                       2 * sizeof(float) * (size_t)next.cols_padded, stream, a, best_rb,
+                       row_lds, stream, a, best_rb,
                        best_gpw, in.then_norm_w, 1.0f / (float)in.N, in.then_norm_eps,
                        in.digits, next.rows_padded, next.cols_padded,
                        static_cast<int8_t *>(in.then_norm_staged));

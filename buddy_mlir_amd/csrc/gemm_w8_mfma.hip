@@ -574,13 +574,9 @@ template <int TERMS>
 int launch_terms(const GemmArgs &a, unsigned blocks, hipStream_t stream) {
   constexpr size_t lds = sizeof(float) * kSlices * 64 * kWave;
   auto kernel = gemm_w8_bf16_kernel<TERMS>;
-  static bool attr_set = false;
-  if (!attr_set) {
-    BH_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
-                                     hipFuncAttributeMaxDynamicSharedMemorySize,
-                                     (int)lds));
-    attr_set = true;
-  }
+  static DynLdsOnce dyn_lds;
+  BH_CHECK_HIP(ensure_dyn_lds(dyn_lds, reinterpret_cast<const void *>(kernel),
+                              (int)lds));
   BH_NOTE_VARIANT(SplitFamily, TERMS);
   hipLaunchKernelGGL(kernel, dim3(blocks), dim3(kSlices * kWave), lds, stream, a);
   BH_CHECK_HIP(hipGetLastError());

@@ -40,7 +40,6 @@
 namespace bh {
 namespace {
 
-BH_TL_DECLARE(g_tl_gemv)
 
 constexpr int kMaxWaves = 16;            // wavefronts per workgroup
 constexpr int kXStride = 20;             // floats per (tile, k-group) in LDS:
@@ -776,8 +775,6 @@ __global__ void __launch_bounds__(kMaxWaves *kWave)
   const int per = (a.chunks + a.KS - 1) / a.KS;
   const int t0 = min(ks * per, a.chunks);
   const int t1 = min(t0 + per, a.chunks);
-  [[maybe_unused]] const int tl_wave = blockIdx.x * (a.G * a.KS) + wave;
-  BH_TL(g_tl_gemv, tl_wave, 0);
 
   float acc0[M], acc1[M], ss[M];
 #pragma unroll
@@ -836,7 +833,6 @@ __global__ void __launch_bounds__(kMaxWaves *kWave)
     }
   }
 
-  BH_TL(g_tl_gemv, tl_wave, 1);
   for (int t = t0; t < t1; t += U) {
 #pragma unroll
     for (int u = 0; u < U; ++u) {
@@ -871,12 +867,9 @@ __global__ void __launch_bounds__(kMaxWaves *kWave)
         }
         if (t + U + u < t1)
           fetch_tile<M, PRO, DUAL>(a, w0, w1, t + U + u, lane, slot[u]);
-        if (u == 0 && t == t0)
-          BH_TL(g_tl_gemv, tl_wave, 2);
       }
     }
   }
-  BH_TL(g_tl_gemv, tl_wave, 3);
 
   // the four rows of a wavefront hold different k sub-ranges of the same channels
 #pragma unroll
@@ -905,7 +898,6 @@ __global__ void __launch_bounds__(kMaxWaves *kWave)
         mine[m * 33 + 32] = ss[m];
     }
     __syncthreads();
-    BH_TL(g_tl_gemv, tl_wave, 4);
     if (ks != 0)
       return;
     if (lane < kTileN) {
@@ -948,7 +940,6 @@ __global__ void __launch_bounds__(kMaxWaves *kWave)
   }
   if (M == 1 && EPI == kEpiStore && a.cand_v && live)
     emit_group_maximum(a, g, lane, writer, y_row, n);
-  BH_TL(g_tl_gemv, tl_wave, 5);
 }
 
 // ---------------------------------------------------------------------------
@@ -968,20 +959,6 @@ __global__ void __launch_bounds__(kMaxWaves *kWave)
 // Nothing waits for another wavefront before the stream: the planes are private
 // to the wavefront that wrote them.
 // ---------------------------------------------------------------------------
-__device__ __forceinline__ unsigned wave_max_u32(unsigned v) {
-  auto dpp = [](unsigned x, auto ctrl) {
-    return (unsigned)__builtin_amdgcn_update_dpp(0, (int)x, decltype(ctrl)::value, 0xf, 0xf,
-                                                 true);
-  };
-  v = max(v, dpp(v, std::integral_constant<int, 0xB1>{}));
-  v = max(v, dpp(v, std::integral_constant<int, 0x4E>{}));
-  v = max(v, dpp(v, std::integral_constant<int, 0x141>{}));
-  v = max(v, dpp(v, std::integral_constant<int, 0x140>{}));
-  const unsigned a = __builtin_amdgcn_readlane((int)v, 0), b = __builtin_amdgcn_readlane((int)v, 16);
-  const unsigned c = __builtin_amdgcn_readlane((int)v, 32), d = __builtin_amdgcn_readlane((int)v, 48);
-  return max(max(a, b), max(c, d));
-}
-
 constexpr int kDigits = 4;                            // int8 digits per activation
 constexpr int kDigitBytesPerTile = kDigits * kTileK;  // the planes of one tile and row
 
@@ -1367,13 +1344,9 @@ int launch_digits(const KernelArgs &ka, const GemvPlan &p, hipStream_t stream) {
   auto kernel = gemv_w8a32_digits_kernel<M, EPI, PRO, U, HS>;
   const size_t lds = digits_lds_bytes(p.waves, M);
   if constexpr (digits_lds_bytes(kMaxWaves, M) > 48 * 1024) {
-    static bool attr_set = false;
-    if (!attr_set) {
-      BH_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize,
-                                       (int)digits_lds_bytes(kMaxWaves, M)));
-      attr_set = true;
-    }
+    static DynLdsOnce dyn_lds;
+    BH_CHECK_HIP(ensure_dyn_lds(dyn_lds, reinterpret_cast<const void *>(kernel),
+                                (int)digits_lds_bytes(kMaxWaves, M)));
   }
   hipLaunchKernelGGL(kernel, dim3(p.blocks << p.half_split), dim3(p.waves * kWave), lds,
                      stream, ka.W0, ka.W1, ka.A, ka.norm_w, ka.chunks, ka.KS,
@@ -1450,13 +1423,9 @@ int launch_bcast(const KernelArgs &ka, const GemvPlan &p, hipStream_t stream) {
 template <int M, int EPI, int PRO, int U, int TN>
 int launch_tn(const KernelArgs &ka, const GemvPlan &p, hipStream_t stream) {
   auto kernel = gemv_w8a32_kernel<M, EPI, PRO, U, TN>;
-  static bool attr_set = false;
-  if (!attr_set) {
-    BH_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
-                                     hipFuncAttributeMaxDynamicSharedMemorySize,
-                                     (int)(kMaxLdsBytes + 4096)));
-    attr_set = true;
-  }
+  static DynLdsOnce dyn_lds;
+  BH_CHECK_HIP(ensure_dyn_lds(dyn_lds, reinterpret_cast<const void *>(kernel),
+                              (int)(kMaxLdsBytes + 4096)));
   hipLaunchKernelGGL(kernel, dim3(p.blocks), dim3(p.waves * kWave), p.lds_bytes,
                      stream, ka);
   BH_CHECK_HIP(hipGetLastError());
@@ -1624,7 +1593,9 @@ int launch_gemv(const GemvArgs &a, hipStream_t stream) {
   BH_REQUIRE(a.tile_n == 16 || a.tile_n == 8 || a.tile_n == 4,
              "gemv: tile_n=%d (16, 8 or 4)", a.tile_n);
   const bool fold = a.attn_acc != nullptr;
-  // (its activation rows are read as aligned 16-byte pieces)
+  // (its activation rows are read as aligned 16-byte pieces; the norm weight,
+  // read the same way, was required to be 16-byte aligned above, so that a
+  // piece that starts inside the array ends inside its last 16-byte line)
   const bool rows_aligned =
       fold || ((reinterpret_cast<uintptr_t>(a.A) & 15) == 0 && (a.M == 1 || (a.lda & 3) == 0));
   const GemvPlan p = choose_plan(mt, a.K, a.N, dual, a.tile_n, fold, rows_aligned);
@@ -1673,7 +1644,6 @@ int launch_gemv(const GemvArgs &a, hipStream_t stream) {
   }
 }
 
-BH_TL_EXPORT(buddy_hip_debug_timeline_gemv, g_tl_gemv)
 } // namespace bh
 
 extern "C" {

@@ -540,13 +540,9 @@ template <int EPI, int SPAN, bool NORM, bool T2>
 int launch_kernel(I8Args ka, int ks_forced, hipStream_t stream) {
   constexpr int NA = (EPI == kEpiSiluMul) ? 2 * SPAN : SPAN;
   auto kernel = gemv_w8a32_i8_kernel<EPI, SPAN, NORM, T2>;
-  static bool attr_set = false;
-  if (!attr_set) {
-    BH_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
-                                     hipFuncAttributeMaxDynamicSharedMemorySize,
-                                     144 * 1024));
-    attr_set = true;
-  }
+  static DynLdsOnce dyn_lds;
+  BH_CHECK_HIP(ensure_dyn_lds(dyn_lds, reinterpret_cast<const void *>(kernel),
+                              144 * 1024));
   auto lds_bytes = [&](int ks, int waves) {
     return sizeof(float) * waves *
            ((size_t)kTurnFloats + (ks > 1 ? (size_t)(NA * 4 + 1) * kWave : 0));

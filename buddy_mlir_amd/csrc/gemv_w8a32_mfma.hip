@@ -381,13 +381,9 @@ int launch_kernel(const MfmaArgs &ka, int blocks, hipStream_t stream) {
   const int waves = ka.GS * ka.KS;
   const size_t lds = ka.KS > 1 ? sizeof(float) * waves * (size_t)(NA * 4 + 1) * kWave : 0;
   auto kernel = gemv_w8a32_mfma_kernel<EPI, SPAN, NORM>;
-  static bool attr_set = false;
-  if (!attr_set) {
-    BH_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
-                                     hipFuncAttributeMaxDynamicSharedMemorySize,
-                                     144 * 1024));
-    attr_set = true;
-  }
+  static DynLdsOnce dyn_lds;
+  BH_CHECK_HIP(ensure_dyn_lds(dyn_lds, reinterpret_cast<const void *>(kernel),
+                              144 * 1024));
   BH_NOTE_VARIANT(MfmaFamily, EPI, SPAN, NORM);
   hipLaunchKernelGGL(kernel, dim3(blocks), dim3(waves * kWave), lds, stream, ka);
   BH_CHECK_HIP(hipGetLastError());

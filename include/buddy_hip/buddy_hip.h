@@ -188,7 +188,8 @@ typedef struct buddy_hip_linear_desc {
   const float *scale1;
   const float *bias;    /* [N] or NULL: C = bias + acc*scale (epilogue STORE) */
   const float *norm_w;  /* [K] or NULL: RMSNorm applied to A first
-                           (subgraph0_decode_simplify.mlir:60-72) */
+                           (subgraph0_decode_simplify.mlir:60-72); 16-byte
+                           aligned, other addresses are refused */
   float norm_eps;
   float *C;             /* [M, N], row stride ldc (>= N) */
   int64_t ldc;
@@ -279,13 +280,19 @@ int buddy_hip_gqa_decode_attention(const float *qkv, const float *inv_freq,
  * buddy_hip_gqa_decode_attention.  Every call on a GPU shares that GPU's
  * buffer: calls that overlap on one GPU (two streams, two threads) race; calls
  * on one stream are ordered.  The device that is current at the call must be
- * the stream's device. */
+ * the stream's device.  The first call on a device looks the buffer's address
+ * up in the runtime; a caller that records the call into a HIP graph makes one
+ * eager call, or buddy_hip_static_scratch_init() with that device current,
+ * before the capture starts (a first call under capture is refused). */
 int buddy_hip_gqa_decode_attention_static(const float *qkv, const float *inv_freq,
                                           const int *pos, float *kcache,
                                           float *vcache, float *out, float *lse,
                                           int heads, int kv_heads, int head_dim,
                                           int max_len, float scale,
                                           buddy_hip_stream stream);
+/* Resolves the built-in buffer of the current device (no allocation, no
+ * launch); idempotent.  No counterpart in the reference. */
+int buddy_hip_static_scratch_init(void);
 
 /* ---- prefill attention ----------------------------------------------------
  * Replaces flash_attention_for_cpu_prefill_op
@@ -625,8 +632,10 @@ void buddy_hip_forward_invalidate_kv(void); /* next decode re-uploads the KV cac
  * session behind _mlir_ciface_forward_*: what a decode loop may call instead of
  * editing its host tensors (TextGeneration.cpp:231-237); it saves the reload.
  * From then on the device cache is the only complete copy: the caller's tensors
- * keep receiving the new rows but are not shifted, and are never reloaded
- * unless buddy_hip_forward_invalidate_kv() is called. */
+ * keep receiving the new rows but are not shifted, and are never reloaded,
+ * whatever position later decode calls carry (a rewind, a repeated position),
+ * until buddy_hip_forward_invalidate_kv(), buddy_hip_forward_reset() or a
+ * prefill. */
 int buddy_hip_forward_discard_kv(int keep, int discard, int count);
 
 /* ---- operator-level memref entry points --------------------------------
@@ -642,8 +651,16 @@ void _mlir_ciface_buddy_matmul_f32(buddy_memref_f32_2d *result,
  * int8 external kernel: runtime/external_kernels/CMakeLists.txt:5-9); it
  * stands for the sitofp -> mulf -> linalg.matmul chain that
  * DequantMatMulVectorizationDecode.cpp:93-189 matches.  The packed device copy
- * of W is cached by (W pointer, K, N) because weights are immutable after
- * loadWeights (tools/buddy-codegen/gen_session.py:1301-1331). */
+ * of W is cached by (W pointer, scale pointer, K, N) because weights are
+ * immutable after loadWeights (tools/buddy-codegen/gen_session.py:1301-1331).
+ * Every call compares a fingerprint of the operands as they are now (64
+ * leading bytes of four rows of W, the first and last 16 scales, the shape)
+ * with the one taken when the copy was made: a buffer that was freed and
+ * reused at the same address with other contents is packed again.  The cache
+ * holds at most a byte limit (16 GiB, or BUDDY_HIP_WEIGHT_CACHE_BYTES in the
+ * environment); the least recently used copies are freed first.  The
+ * reference's own external kernel caches nothing
+ * (runtime/external_kernels/matmul/MatmulTorq.cpp:116-166). */
 void _mlir_ciface_buddy_dequant_matmul_i8_f32(buddy_memref_f32_2d *result,
                                               buddy_memref_f32_2d *A,
                                               buddy_memref_i8_2d *W,
@@ -656,6 +673,17 @@ void _mlir_ciface_buddy_dequant_matmul_i8_f32_acc(buddy_memref_f32_2d *C,
                                                   buddy_memref_f32_2d *scale);
 /* Drops every cached device copy made by the entry points above. */
 void buddy_hip_clear_weight_cache(void);
+/* The byte limit of that cache (entries beyond it are freed at once, least
+ * recently used first) and its counters.  No counterpart in the reference. */
+typedef struct buddy_hip_weight_cache_info {
+  int64_t entries;     /* packed copies held */
+  int64_t bytes;       /* device bytes they take */
+  int64_t limit_bytes; /* the limit in force */
+  int64_t uploads;     /* copies made since the library was loaded */
+  int64_t evictions;   /* copies freed to stay under the limit */
+} buddy_hip_weight_cache_info;
+void buddy_hip_set_weight_cache_limit(size_t bytes);
+void buddy_hip_weight_cache_stats(buddy_hip_weight_cache_info *info);
 
 #ifdef __cplusplus
 }

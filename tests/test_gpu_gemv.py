@@ -190,6 +190,32 @@ def test_llama3_8b_fused_launches_match_oracle(oracle, M):
     check_close(out.cpu().numpy(), np.stack([oracle.dequant_gemv(xn[m], qh, sh) for m in range(M)]))
 
 
+@pytest.mark.parametrize("M", [1, 3])
+def test_norm_weight_alignment_and_ragged_k(bh, oracle, M):
+    """RMSNorm fused into the GEMV with K not a multiple of 4: the kernels read
+    the norm weight in 16-byte pieces, so one that is not 16-byte aligned (a
+    piece could run past its end) is refused; an aligned one gives the oracle's
+    result."""
+    K, N = 1001, 272
+    eps = np.float32(1e-6)
+    g = torch.Generator(device="cuda").manual_seed(70 + M)
+    x = torch.randn((M, K), generator=g, device="cuda")
+    wbuf = 1 + 0.1 * torch.randn(K + 1, generator=g, device="cuda")
+    q, s = ops.quantize_w8(make_weight(K, N, 7))
+    out = torch.empty((M, N), device="cuda")
+    assert wbuf[1:].data_ptr() % 16 == 4
+    with pytest.raises(bma.BuddyHipError, match="16-byte aligned"):
+        ops.linear_w8a32(A=x, lda=K, W0=ops.pack_w8(q), scale0=s, norm_w=wbuf[1:],
+                         norm_eps=float(eps), C=out, ldc=N, M=M, K=K, N=N, epilogue=0)
+    w = wbuf[:K].clone()
+    ops.linear_w8a32(A=x, lda=K, W0=ops.pack_w8(q), scale0=s, norm_w=w, norm_eps=float(eps),
+                     C=out, ldc=N, M=M, K=K, N=N, epilogue=0)
+    torch.cuda.synchronize()
+    xh, wh, qh, sh = x.cpu().numpy(), w.cpu().numpy(), q.cpu().numpy(), s.cpu().numpy()
+    xn = [oracle.rmsnorm(xh[m], wh, eps, np.float32(1.0) / np.float32(K)) for m in range(M)]
+    check_close(out.cpu().numpy(), np.stack([oracle.dequant_gemv(xn[m], qh, sh) for m in range(M)]))
+
+
 @pytest.fixture
 def bf16_batch_kernel(bh):
     """Batches of 5..16 rows through the bf16 matrix-core kernel (every f32 bit of
@@ -473,6 +499,110 @@ def test_memref_abi_block_of_rows_takes_the_matrix_cores(bh, oracle):
     ctypes.CDLL(None).free(res.allocated)
     assert np.isnan(out[2]).all() and not np.isnan(np.delete(out, 2, 0)).any()
     bh.buddy_hip_clear_weight_cache()
+
+
+class WeightCacheInfo(ctypes.Structure):
+    _fields_ = [(n, ctypes.c_int64) for n in ("entries", "bytes", "limit_bytes", "uploads",
+                                              "evictions")]
+
+
+def cache_info(bh):
+    info = WeightCacheInfo()
+    bh.buddy_hip_weight_cache_stats(ctypes.byref(info))
+    return info
+
+
+def dequant_matmul_host(bh, A, W, S):
+    res = bma.MemRefF32_2D()
+    a = bma.MemRef(A.ctypes.data, list(A.shape))
+    w = bma.MemRef(W.ctypes.data, list(W.shape), ctype=ctypes.c_int8)
+    s = bma.MemRef(S.ctypes.data, list(S.shape))
+    bh._mlir_ciface_buddy_dequant_matmul_i8_f32(ctypes.byref(res), ctypes.byref(a),
+                                                ctypes.byref(w), ctypes.byref(s))
+    assert res.aligned, bh.buddy_hip_last_error()
+    out = np.ctypeslib.as_array(res.aligned, shape=(A.shape[0], W.shape[1])).copy()
+    ctypes.CDLL(None).free(res.allocated)
+    return out
+
+
+def test_weight_cache_sees_new_contents_at_the_same_address(bh, oracle):
+    """The operator-level cache is keyed by the operands' addresses; a caller
+    that frees a weight buffer and gets the same address back with other
+    contents (or rewrites the buffer) must not be served the old packed copy."""
+    bh.buddy_hip_clear_weight_cache()
+    rng = np.random.default_rng(8)
+    K, N = 320, 96
+    A = rng.normal(0, 1, (2, K)).astype(np.float32)
+    W = rng.integers(-128, 128, (K, N)).astype(np.int8)
+    S = rng.uniform(1e-4, 1e-3, (1, N)).astype(np.float32)
+    u0 = cache_info(bh).uploads
+    out = dequant_matmul_host(bh, A, W, S)
+    check_close(out, np.stack([oracle.dequant_gemv(A[m], W, S) for m in range(2)]))
+    out = dequant_matmul_host(bh, A, W, S)          # a hit: no second upload
+    assert cache_info(bh).uploads == u0 + 1 and cache_info(bh).entries == 1
+    W[...] = rng.integers(-128, 128, (K, N)).astype(np.int8)   # same address, new weights
+    out = dequant_matmul_host(bh, A, W, S)
+    check_close(out, np.stack([oracle.dequant_gemv(A[m], W, S) for m in range(2)]))
+    assert cache_info(bh).uploads == u0 + 2 and cache_info(bh).entries == 1
+    S[...] = S[:, ::-1].copy()                      # new scales only
+    out = dequant_matmul_host(bh, A, W, S)
+    check_close(out, np.stack([oracle.dequant_gemv(A[m], W, S) for m in range(2)]))
+    assert cache_info(bh).uploads == u0 + 3 and cache_info(bh).entries == 1
+    # device-resident operands are fingerprinted too
+    Wd, Sd = torch.from_numpy(W).cuda(), torch.from_numpy(S).cuda()
+    w = bma.MemRef(Wd.data_ptr(), [K, N], ctype=ctypes.c_int8)
+    s = bma.MemRef(Sd.data_ptr(), [1, N])
+    a = bma.MemRef(A.ctypes.data, [2, K])
+
+    def run_dev():
+        res = bma.MemRefF32_2D()
+        bh._mlir_ciface_buddy_dequant_matmul_i8_f32(ctypes.byref(res), ctypes.byref(a),
+                                                    ctypes.byref(w), ctypes.byref(s))
+        assert res.aligned, bh.buddy_hip_last_error()
+        o = np.ctypeslib.as_array(res.aligned, shape=(2, N)).copy()
+        ctypes.CDLL(None).free(res.allocated)
+        return o
+
+    check_close(run_dev(), np.stack([oracle.dequant_gemv(A[m], W, S) for m in range(2)]))
+    W2 = rng.integers(-128, 128, (K, N)).astype(np.int8)
+    Wd.copy_(torch.from_numpy(W2))
+    torch.cuda.synchronize()
+    check_close(run_dev(), np.stack([oracle.dequant_gemv(A[m], W2, S) for m in range(2)]))
+    bh.buddy_hip_clear_weight_cache()
+    assert cache_info(bh).entries == 0 and cache_info(bh).bytes == 0
+
+
+def test_weight_cache_is_bounded_and_frees_the_least_recently_used(bh, oracle):
+    bh.buddy_hip_clear_weight_cache()
+    limit0 = cache_info(bh).limit_bytes
+    rng = np.random.default_rng(9)
+    K, N = 256, 64
+    per_entry = bh.buddy_hip_w8_packed_bytes(K, N) + 4 * N
+    bh.buddy_hip_set_weight_cache_limit(3 * per_entry)
+    try:
+        A = rng.normal(0, 1, (1, K)).astype(np.float32)
+        Ws = [rng.integers(-128, 128, (K, N)).astype(np.int8) for _ in range(5)]
+        S = rng.uniform(1e-4, 1e-3, (1, N)).astype(np.float32)
+        Ss = [S.copy() for _ in range(5)]
+        e0, u0 = cache_info(bh).evictions, cache_info(bh).uploads
+        for i in range(3):
+            dequant_matmul_host(bh, A, Ws[i], Ss[i])
+        assert cache_info(bh).entries == 3 and cache_info(bh).bytes == 3 * per_entry
+        dequant_matmul_host(bh, A, Ws[0], Ss[0])        # touch 0: 1 is now the oldest
+        dequant_matmul_host(bh, A, Ws[3], Ss[3])        # evicts 1
+        info = cache_info(bh)
+        assert (info.entries, info.evictions - e0, info.uploads - u0) == (3, 1, 4)
+        assert info.bytes <= info.limit_bytes
+        dequant_matmul_host(bh, A, Ws[0], Ss[0])        # still cached
+        assert cache_info(bh).uploads - u0 == 4
+        out = dequant_matmul_host(bh, A, Ws[1], Ss[1])  # was freed: packed again, right result
+        assert cache_info(bh).uploads - u0 == 5
+        check_close(out, oracle.dequant_gemv(A[0], Ws[1], Ss[1])[None])
+        bh.buddy_hip_set_weight_cache_limit(per_entry)   # shrinking frees at once
+        assert cache_info(bh).entries == 1
+    finally:
+        bh.buddy_hip_set_weight_cache_limit(limit0)
+        bh.buddy_hip_clear_weight_cache()
 
 
 def test_bad_arguments_are_refused(bh):

@@ -276,6 +276,80 @@ def test_forward_decode_survives_the_callers_own_overflow_handling(bh, oracle):
     bh.buddy_hip_forward_reset()
 
 
+@pytest.mark.timeout(900)
+def test_device_side_discard_keeps_the_device_cache_at_any_later_position(bh, oracle):
+    """After buddy_hip_forward_discard_kv the caller's tensors are stale (never
+    shifted), so no later decode may reload them, whatever its position: decode
+    16 tokens, discard on the device, decode the position that follows, then
+    decode that same position again with another token (a rewind).  Every step
+    must give the oracle's logits on the oracle's own shifted cache."""
+    L = 64
+    shape = Shape(max_len=L)
+    f32, i8, host = make_blobs(bh, shape, seed=4)
+    om = oracle_lib.model_from_host(oracle, shape, host)
+    okv = [np.zeros((2, L, 128), np.float32) for _ in range(56)]
+    state_kv = [np.zeros((2, L, 128), np.float32) for _ in range(56)]
+    free = ctypes.CDLL(None).free
+    free.argtypes = [ctypes.c_void_p]
+    mf = bma.MemRef(f32.ctypes.data, [f32.size])
+    mi = bma.MemRef(i8.ctypes.data, [i8.size], ctype=ctypes.c_int8)
+    kvm = [bma.MemRef(a.ctypes.data, [1, 2, L, 128]) for a in state_kv]
+    posbuf = np.zeros(1, np.int64)
+    tokbuf = np.zeros((1, 1), np.int64)
+    dummies = [np.zeros(1, np.int64) for _ in range(27)]
+    mpos = bma.MemRef(posbuf.ctypes.data, [1], ctype=ctypes.c_longlong)
+    mtok = bma.MemRef(tokbuf.ctypes.data, [1, 1], ctype=ctypes.c_longlong)
+    mdum = [bma.MemRef(d.ctypes.data, [1], ctype=ctypes.c_longlong) for d in dummies]
+    inv_freq = host["globals"]["inv_freq"]
+
+    def step(tok, pos):
+        tokbuf[0, 0], posbuf[0] = tok, pos
+        for d in dummies:
+            d[0] = pos
+        res = DecodeResult()
+        bh._mlir_ciface_forward_decode(*decode_args(res, mf, mi, mtok, mpos, kvm, mdum))
+        assert res.logits.aligned, bh.buddy_hip_last_error()
+        lg = np.ctypeslib.as_array(res.logits.aligned, shape=(shape.vocab,)).copy()
+        free(ctypes.cast(res.logits.allocated, ctypes.c_void_p))
+        return lg
+
+    bh.buddy_hip_forward_reset()
+    tok = 5
+    for pos in range(16):
+        lg = step(tok, pos)
+        otok, _ = om.decode_step(tok, pos, okv)
+        assert int(lg.argmax()) == otok
+        tok = otok
+    keep, discard, count = 4, 4, 16
+    assert bh.buddy_hip_forward_discard_kv(keep, discard, count) == 0, bh.buddy_hip_last_error()
+    for j in range(56):
+        _, new = oracle.kv_discard(okv[j], keep, discard, count)
+        if j % 2 == 0:
+            new = oracle.kv_adjust_rope(new, keep, discard, count, inv_freq)
+        okv[j][...] = new
+    pos = count - discard
+    lg = step(tok, pos)                      # the position that follows
+    otok, olg = om.decode_step(tok, pos, okv)
+    check_close(lg, olg)
+    assert int(lg.argmax()) == otok
+    other = (tok + 17) % shape.vocab
+    lg = step(other, pos)                    # the same position again: a rewind
+    otok, olg = om.decode_step(other, pos, okv)
+    check_close(lg, olg)
+    assert int(lg.argmax()) == otok
+    lg = step(otok, 3)                       # and far back, inside the kept prefix
+    otok2, olg = om.decode_step(otok, 3, okv)
+    check_close(lg, olg)
+    assert int(lg.argmax()) == otok2
+    # invalidate_kv hands the truth back to the caller's (stale, unshifted) tensors
+    bh.buddy_hip_forward_invalidate_kv()
+    stale = [a.copy() for a in state_kv]
+    lg = step(tok, pos)
+    otok3, olg = om.decode_step(tok, pos, stale)
+    check_close(lg, olg)
+    bh.buddy_hip_forward_reset()
+
+
 def test_model_level_entry_points_refuse_bad_blobs(bh):
     f32 = np.zeros(10, np.float32)
     i8 = np.zeros(10, np.int8)

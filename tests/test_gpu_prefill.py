@@ -70,6 +70,73 @@ def test_prefill_gemm_matches_blis_oracle(oracle, M, K, N, mode):
     check_close(y.cpu().numpy(), want)
 
 
+@pytest.mark.parametrize("M,K,N", [(512, 1536, 8960), (512, 8960, 1536), (70, 200, 48)])
+def test_non_finite_activation_rows_come_out_nan_in_the_digit_mode(M, K, N):
+    """The reference's prefill kernel is an f32 multiply-add chain
+    (MatMulBlisVectorization.cpp:644-740): a NaN in a row of A makes that row of
+    C NaN, an infinity makes it +-inf or NaN.  The digit-plane matmul gives such a
+    row a NaN step: every element of the row is NaN, every other row is what it
+    is without the poison, bit for bit."""
+    q, s = synthetic.quantized_linear(K, N, 5)
+    packed = ops.pack_w8(q)
+    g = torch.Generator(device="cuda").manual_seed(M + K)
+    x = torch.randn((M, K), generator=g, device="cuda")
+    clean = ops.gemm_w8a32(x, packed, s, K, N, digits=True).cpu().numpy()
+    x[3, K // 2] = float("nan")
+    x[M - 2, 0] = float("-inf")
+    x[5, K - 1] = float("inf")
+    got = ops.gemm_w8a32(x, packed, s, K, N, digits=True).cpu().numpy()
+    bad = [3, 5, M - 2]
+    assert np.isnan(got[bad]).all()
+    rest = np.delete(np.arange(M), bad)
+    assert np.isfinite(got[rest]).all()
+    np.testing.assert_array_equal(got[rest], clean[rest])
+    # the paired gate|up form with SiLU*mul in its epilogue
+    if N % 64 == 0:
+        both = torch.cat([packed, packed])
+        got = ops.gemm_w8a32(x, both, torch.cat([s, s]), K, N, digits=True,
+                             silu_pair=True).cpu().numpy()
+        assert np.isnan(got[bad]).all() and np.isfinite(got[rest]).all()
+
+
+def test_non_finite_token_through_session_prefill():
+    """A prompt whose last token's embedding row holds a NaN (then an infinity):
+    that row's logits are NaN; the logits of every earlier row are those of the
+    clean prompt bit for bit (causality), through every digit-plane producer of
+    the block (RMSNorm rows, SiLU*mul rows, the slice-adding kernel that writes
+    the next layer's rows).  The poisoned token is the first of a 16-row block of
+    the attention kernel: a masked key still meets the queries of its own block
+    in the P.V matrix product as 0 x NaN (in the reference the additive -inf
+    mask lets a NaN key reach every query of the prompt)."""
+    sess, _ = synthetic.build_session(SMALL, context=0, ln_jitter=0.1)
+    lib = bma.lib()
+    V = SMALL.vocab
+    toks = synthetic.first_tokens(SMALL, 33, seed=5).astype(np.int32)
+    poisoned = int(toks[-1])
+    toks[:-1][toks[:-1] == poisoned] = (poisoned + 1) % V
+
+    def all_logits():
+        out = np.empty((toks.size, V), np.float32)
+        bma.check(lib.buddy_hip_session_prefill_all_logits(
+            sess._h, toks.ctypes.data, toks.size, 0, out.ctypes.data), "prefill_all_logits")
+        return out
+
+    clean = all_logits()
+    assert np.isfinite(clean).all()
+    embed = sess._globals["embed"]
+    for poison in (float("nan"), float("-inf")):
+        keep = embed[poisoned].clone()
+        embed[poisoned, 7] = poison
+        torch.cuda.synchronize()
+        got = all_logits()
+        embed[poisoned] = keep
+        torch.cuda.synchronize()
+        assert np.isnan(got[-1]).all()
+        np.testing.assert_array_equal(got[:-1], clean[:-1])
+    np.testing.assert_array_equal(all_logits(), clean)
+    sess.close()
+
+
 @pytest.mark.parametrize("M,K", [(1, 64), (5, 100), (70, 1536), (48, 8960)])
 def test_digit_planes_are_the_rounded_fixed_point(M, K):
     """W = 127 I with scale 1/127 copies the activations: what comes out is

@@ -65,3 +65,46 @@ def test_static_scratch_entry_point_refuses_what_does_not_fit(bh):
                                                   SCALE, None)
     assert rc == 1
     assert b"exceeds the built-in scratch" in bh.buddy_hip_last_error()
+
+
+def test_static_scratch_entry_point_recorded_into_a_graph(bh):
+    """The use the entry point exists for: after buddy_hip_static_scratch_init()
+    the call is captured into a HIP graph (no allocation, no address lookup
+    under capture) and replayed with new inputs in the same buffers; every
+    replay, with eager work and synchronisations of the program's own between
+    them, equals the workspace entry point bit for bit."""
+    H, HKV, L, D = 12, 2, 1088, 128
+    bma.check(bh.buddy_hip_static_scratch_init())
+    g = torch.Generator(device="cuda").manual_seed(5)
+    qkv = torch.randn((H + 2 * HKV) * D, generator=g, device="cuda")
+    kc = torch.randn((HKV, L, D), generator=g, device="cuda")
+    vc = torch.randn((HKV, L, D), generator=g, device="cuda")
+    inv = synthetic.inv_freq(D)
+    pos_t = torch.tensor([900], dtype=torch.int32, device="cuda")
+    out = torch.zeros(H * D, device="cuda")
+    lse = torch.zeros(H, device="cuda")
+    nb = bh.buddy_hip_attn_decode_workspace_bytes(H, L)
+    ws = torch.empty(nb, dtype=torch.uint8, device="cuda")
+    k2, v2 = kc.clone(), vc.clone()
+    out2, lse2 = torch.zeros_like(out), torch.zeros_like(lse)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    with torch.cuda.graph(graph, stream=side):
+        bma.check(bh.buddy_hip_gqa_decode_attention_static(
+            qkv.data_ptr(), inv.data_ptr(), pos_t.data_ptr(), kc.data_ptr(), vc.data_ptr(),
+            out.data_ptr(), lse.data_ptr(), H, HKV, D, L, SCALE, side.cuda_stream))
+    torch.cuda.synchronize()
+    for replay, pos in enumerate((900, 17, 1087, 333)):
+        qkv.copy_(torch.randn(qkv.shape, generator=g, device="cuda"))
+        pos_t.fill_(pos)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        bma.check(bh.buddy_hip_gqa_decode_attention(
+            qkv.data_ptr(), inv.data_ptr(), pos_t.data_ptr(), k2.data_ptr(), v2.data_ptr(),
+            out2.data_ptr(), lse2.data_ptr(), H, HKV, D, L, SCALE, ws.data_ptr(), nb, None))
+        torch.cuda.synchronize()
+        assert torch.isfinite(out).all(), replay
+        assert torch.equal(out, out2) and torch.equal(lse, lse2), replay
+        assert torch.equal(kc, k2) and torch.equal(vc, v2), replay
