@@ -143,6 +143,9 @@ def _declare(lib):
         "buddy_hip_quantize_w4": (c_int, [vp, i64, i64, vp, vp, vp]),
         "buddy_hip_pack_int4": (c_int, [vp, i64, vp, vp]),
         "buddy_hip_gemv_w4a16": (c_int, [vp, vp, vp, vp, i64, i64, vp]),
+        "buddy_hip_w4_tiles_bytes": (sz, [i64, i64]),
+        "buddy_hip_pack_w4_tiles": (c_int, [vp, i64, i64, vp, vp]),
+        "buddy_hip_gemv_w4a16_fast": (c_int, [vp, vp, vp, vp, i64, i64, vp]),
         "buddy_hip_kv_discard": (c_int, [vp, c_int, c_int, c_int, c_int, c_int, c_int,
                                          c_int, vp, vp]),
         "buddy_hip_forward_discard_kv": (c_int, [c_int, c_int, c_int]),

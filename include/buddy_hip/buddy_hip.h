@@ -107,6 +107,27 @@ int buddy_hip_pack_int4(const int8_t *q, int64_t count, int8_t *packed,
                         buddy_hip_stream stream);
 int buddy_hip_gemv_w4a16(const uint16_t *A, const int8_t *packed, const uint16_t *scale,
                          uint16_t *C, int64_t K, int64_t N, buddy_hip_stream stream);
+/* The same operands with another summation, opt-in:
+ *   C[n] = f16(f32(C[n]) + (sum_k A[k] * w[k][n]) * f32(scale[n]))
+ * with exact products and a sum that is exact up to one rounding of every
+ * activation to 2^-31 of the largest of its run of 128..1024 values, rounded to
+ * f16 once at the end.  The reference's f16 chain
+ * (Int4DequantMatMulVectorizationDecode.cpp:438-446) rounds after every one of
+ * its K steps, so this result is at least as close to the real-number sum as
+ * the reference's own but is not the reference's bit for bit; in exchange the
+ * launch is bound by the half byte per weight it reads (the bit-exact kernel
+ * above by its chain of K dependent roundings).  A NaN or an infinity among
+ * the activations of a run turns C into NaN.  The weights come as "int4 wave
+ * tiles" (16 channels x 128 k per KiB, in the order the int8 matrix cores take
+ * them), made once from the reference's [K, N/2] bytes by
+ * buddy_hip_pack_w4_tiles into buddy_hip_w4_tiles_bytes(K, N) bytes (16-byte
+ * aligned; K and N are zero padded inside).  A: 8-byte aligned.  No counterpart
+ * in the reference. */
+size_t buddy_hip_w4_tiles_bytes(int64_t K, int64_t N);
+int buddy_hip_pack_w4_tiles(const int8_t *packed, int64_t K, int64_t N, int8_t *tiles,
+                            buddy_hip_stream stream);
+int buddy_hip_gemv_w4a16_fast(const uint16_t *A, const int8_t *tiles, const uint16_t *scale,
+                              uint16_t *C, int64_t K, int64_t N, buddy_hip_stream stream);
 
 /* ---- int8 dequant decode GEMV / small-batch matmul ---------------------
  * Replaces the kernel that
