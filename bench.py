@@ -446,6 +446,7 @@ def bench_prefill(bh, args):
     res = {}
     n = max(1, min(args.steps, 20))
     for name, precision, peak in (("i8_3digit", "digits", MFMA_I8_PEAK_TOPS),
+                                  ("i8_2digit", "digits2", MFMA_I8_PEAK_TOPS),
                                   ("bf16_1term", "bf16", MFMA_BF16_PEAK_TFLOPS),
                                   ("bf16_3term_exact", "exact", MFMA_BF16_PEAK_TFLOPS)):
         for _ in range(max(1, args.warmup)):

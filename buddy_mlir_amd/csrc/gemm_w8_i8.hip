@@ -979,7 +979,9 @@ void release_gemm_i8_workspace(hipStream_t stream) {
 
 // `planes` holds the digit planes and row steps of the activations (written by
 // one of the producers above for exactly this M, K and digit count).
-int launch_gemm_w8_digits(const GemmW8Args &in, const void *planes, hipStream_t stream) {
+namespace {
+template <int D>
+int launch_gemm_w8_digits_d(const GemmW8Args &in, const void *planes, hipStream_t stream) {
   GemmI8Args a;
   const GemmStagingLayout layout = gemm_staging_layout(in.M, in.K);
   a.Mp = layout.rows_padded;
@@ -1026,7 +1028,7 @@ int launch_gemm_w8_digits(const GemmW8Args &in, const void *planes, hipStream_t 
     a.ncols = (int)ceil_div(half_groups, 2 * best_gpw);
     a.cols_padded = (int)round_up((int64_t)a.ncols, 8);
     const int row_tiles = (int)ceil_div(in.M, 16 * best_rb);
-    return launch_shape<3, true>(best_rb, best_gpw, a, (unsigned)(a.cols_padded * row_tiles),
+    return launch_shape<D, true>(best_rb, best_gpw, a, (unsigned)(a.cols_padded * row_tiles),
                                  stream);
   }
   // Three schemes, chosen by a model of their cost in microseconds (fitted to
@@ -1079,7 +1081,7 @@ int launch_gemm_w8_digits(const GemmW8Args &in, const void *planes, hipStream_t 
     a.ncols = (int)ceil_div(a.groups, kSplitGroups);
     a.cols_padded = (int)round_up(a.ncols, 8);
     const unsigned blocks = (unsigned)(a.cols_padded * (a.Mp / 64));
-    if (int rc = launch_split<3>(a, blocks, stream))
+    if (int rc = launch_split<D>(a, blocks, stream))
       return rc;
     return then_norm();
   }
@@ -1097,7 +1099,7 @@ int launch_gemm_w8_digits(const GemmW8Args &in, const void *planes, hipStream_t 
     a.partial = reinterpret_cast<float *>(ws);
   }
   const unsigned blocks = (unsigned)(a.cols_padded * row_tiles);
-  int rc = launch_shape<3>(best_rb, best_gpw, a, blocks, stream);
+  int rc = launch_shape<D>(best_rb, best_gpw, a, blocks, stream);
   if (rc)
     return rc;
   if (best_s == 1)
@@ -1125,6 +1127,12 @@ int launch_gemm_w8_digits(const GemmW8Args &in, const void *planes, hipStream_t 
                      stream, a, best_rb, best_gpw);
   BH_CHECK_HIP(hipGetLastError());
   return then_norm();
+}
+} // namespace
+
+int launch_gemm_w8_digits(const GemmW8Args &in, const void *planes, hipStream_t stream) {
+  return in.digits == 2 ? launch_gemm_w8_digits_d<2>(in, planes, stream)
+                        : launch_gemm_w8_digits_d<3>(in, planes, stream);
 }
 
 // The w8a8 matmul for more than 16 rows: `plane` holds the int8 activations as

@@ -628,11 +628,12 @@ int launch_gemm_w8(const GemmW8Args &in, hipStream_t stream) {
   BH_REQUIRE(!in.silu_pair || in.digits, "gemm_w8: the SiLU pair runs on digit planes only");
   BH_REQUIRE(!in.then_norm_w || (in.digits && in.then_norm_staged),
              "gemm_w8: a following norm needs digit planes and a buffer for them");
-  // one bf16 term (activations cast to bf16) or three (every f32 bit); digit
-  // planes always three: the variants in between were never reachable from an
-  // entry point and are not built
+  // one bf16 term (activations cast to bf16) or three (every f32 bit); three
+  // digit planes (23 bits below the row's maximum) or two (15 bits: the fixed
+  // point counterpart of the bf16 cast, for the same third less matrix work)
   BH_REQUIRE(in.terms == 1 || in.terms == 3, "gemm_w8: terms=%d (1 or 3)", in.terms);
-  BH_REQUIRE(in.digits == 0 || in.digits == 3, "gemm_w8: digits=%d (0 or 3)", in.digits);
+  BH_REQUIRE(in.digits == 0 || in.digits == 2 || in.digits == 3,
+             "gemm_w8: digits=%d (0, 2 or 3)", in.digits);
   BH_REQUIRE(in.digits == 0 || in.K <= (1 << 17),
              "gemm_w8: K=%lld beyond 2^17 would overflow the int32 sums of the digit planes",
              (long long)in.K);
@@ -728,7 +729,9 @@ int buddy_hip_gemm_w8a32(const float *A, const int8_t *packed, const float *scal
   a.N = N;
   a.accumulate = (flags & BUDDY_HIP_GEMV_ACCUMULATE) != 0;
   a.terms = (flags & BUDDY_HIP_GEMM_A_F32_EXACT) ? 3 : 1;
-  a.digits = (flags & BUDDY_HIP_GEMM_A_I8_DIGITS) ? 3 : 0;
+  a.digits = (flags & BUDDY_HIP_GEMM_A_I8_DIGITS) ? ((flags & BUDDY_HIP_GEMM_TWO_DIGITS) ? 2 : 3) : 0;
+  BH_REQUIRE(a.digits || !(flags & BUDDY_HIP_GEMM_TWO_DIGITS),
+             "gemm_w8a32: BUDDY_HIP_GEMM_TWO_DIGITS needs BUDDY_HIP_GEMM_A_I8_DIGITS");
   if (flags & BUDDY_HIP_GEMM_SILU_PAIR) {
     BH_REQUIRE(a.digits, "gemm_w8a32: BUDDY_HIP_GEMM_SILU_PAIR needs BUDDY_HIP_GEMM_A_I8_DIGITS");
     a.silu_pair = true;

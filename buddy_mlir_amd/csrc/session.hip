@@ -1045,10 +1045,10 @@ void buddy_hip_session_adopt(buddy_hip_session *hs, void *device_ptr) try {
 int buddy_hip_session_set_prefill_precision(buddy_hip_session *hs, int mode) try {
   Session *s = reinterpret_cast<Session *>(hs);
   BH_REQUIRE(s, "session_set_prefill_precision: null session");
-  BH_REQUIRE(mode >= 0 && mode <= 2, "session_set_prefill_precision: mode %d outside 0..2",
+  BH_REQUIRE(mode >= 0 && mode <= 3, "session_set_prefill_precision: mode %d outside 0..3",
              mode);
   s->gemm_terms = mode == 1 ? 3 : 1;
-  s->gemm_digits = mode == 2 ? 3 : 0;
+  s->gemm_digits = mode == 2 ? 3 : mode == 3 ? 2 : 0;
   return BUDDY_HIP_OK;
 } BH_CATCH_INT("buddy_hip_session_set_prefill_precision")
 

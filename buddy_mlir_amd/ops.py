@@ -128,15 +128,16 @@ def gemv_w8a32(x: torch.Tensor, packed: torch.Tensor, scale: torch.Tensor,
 GEMM_A_F32_EXACT = 2
 GEMM_A_I8_DIGITS = 4
 GEMM_SILU_PAIR = 8
+GEMM_TWO_DIGITS = 16
 
 
 def gemm_w8a32(x: torch.Tensor, packed: torch.Tensor, scale: torch.Tensor,
                K: int, N: int, out: torch.Tensor | None = None,
-               accumulate: bool = False, exact: bool = False, digits: bool = False,
+               accumulate: bool = False, exact: bool = False, digits: bool | int = False,
                silu_pair: bool = False):
     """Prefill matmul on the matrix cores: out[M,N] (+)= x[M,K] . (W * scale).
     Activations: cast to bf16 (default), three bf16 terms (exact) or three int8
-    digit planes on the int8 matrix cores (digits).  silu_pair (with digits):
+    digit planes on the int8 matrix cores (digits; digits=2: two planes).  silu_pair (with digits):
     packed and scale hold two matrices of N channels one behind the other and
     out[M,N] = SiLU(x . W0) * (x . W1)."""
     _dev(x, torch.float32)
@@ -148,7 +149,8 @@ def gemm_w8a32(x: torch.Tensor, packed: torch.Tensor, scale: torch.Tensor,
             raise ValueError("accumulate needs an output tensor")
         out = torch.empty((M, N), dtype=torch.float32, device=x.device)
     flags = ((GEMV_ACCUMULATE if accumulate else 0) | (GEMM_A_F32_EXACT if exact else 0) |
-             (GEMM_A_I8_DIGITS if digits else 0) | (GEMM_SILU_PAIR if silu_pair else 0))
+             (GEMM_A_I8_DIGITS if digits else 0) | (GEMM_SILU_PAIR if silu_pair else 0) |
+             (GEMM_TWO_DIGITS if digits == 2 and digits is not True else 0))
     check(lib().buddy_hip_gemm_w8a32(x.data_ptr(), packed.data_ptr(), scale.data_ptr(),
                                      out.data_ptr(), M, K, N, flags, _stream()),
           "gemm_w8a32")

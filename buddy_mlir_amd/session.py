@@ -134,14 +134,15 @@ class DecoderSession:
             self._h, first_token, start_pos, steps, out.ctypes.data), "decode_greedy")
         return out
 
-    PREFILL_PRECISION = {"bf16": 0, "exact": 1, "digits": 2}
+    PREFILL_PRECISION = {"bf16": 0, "exact": 1, "digits": 2, "digits2": 3}
 
     def prefill(self, tokens, start_pos: int = 0, want_logits: bool = True,
                 precision: str = "digits"):
         """ModelSession::prefill: the prompt as one block.  Returns (greedy next
         token, logits of the last prompt token).  precision: how the matmuls
         carry their f32 activations -- "digits" (three int8 digit planes on the
-        int8 matrix cores), "exact" (three bf16 terms) or "bf16" (cast)."""
+        int8 matrix cores), "digits2" (two planes), "exact" (three bf16 terms)
+        or "bf16" (cast)."""
         toks = np.ascontiguousarray(tokens, np.int32)
         check(self._lib.buddy_hip_session_set_prefill_precision(
             self._h, self.PREFILL_PRECISION[precision]), "set_prefill_precision")

@@ -239,7 +239,11 @@ int buddy_hip_linear_w8a32(const buddy_hip_linear_desc *desc,
  * |a| / s < 2^22, rint(a / s) written as three balanced base-256 digits -- and
  * the int8 weights are multiplied as they are on the int8 matrix cores, with
  * exact int32 sums: the only rounding is that of a, at most 2^-23 of the row's
- * largest magnitude (NaN and infinity do not survive it; K <= 2^17).
+ * largest magnitude (a NaN or an infinity in a row turns that row of C into
+ * NaN; K <= 2^17).  BUDDY_HIP_GEMM_TWO_DIGITS (with BUDDY_HIP_GEMM_A_I8_DIGITS)
+ * keeps two digits, |a| / s < 2^14: the rounding is 2^-15 of the row's largest
+ * magnitude -- the fixed-point counterpart of casting the activations to bf16
+ * (2^-9 of each value), for two thirds of the matrix instructions.
  * BUDDY_HIP_GEMV_ACCUMULATE as above.
  * BUDDY_HIP_GEMM_SILU_PAIR (with BUDDY_HIP_GEMM_A_I8_DIGITS; N % 16 == 0; no
  * accumulation): `packed` holds two [K,N] matrices one behind the other, each
@@ -249,7 +253,8 @@ int buddy_hip_linear_w8a32(const buddy_hip_linear_desc *desc,
 enum {
   BUDDY_HIP_GEMM_A_F32_EXACT = 2,
   BUDDY_HIP_GEMM_A_I8_DIGITS = 4,
-  BUDDY_HIP_GEMM_SILU_PAIR = 8
+  BUDDY_HIP_GEMM_SILU_PAIR = 8,
+  BUDDY_HIP_GEMM_TWO_DIGITS = 16
 };
 int buddy_hip_gemm_w8a32(const float *A, const int8_t *packed, const float *scale,
                          float *C, int64_t M, int64_t K, int64_t N,
@@ -428,7 +433,9 @@ void buddy_hip_session_adopt(buddy_hip_session *s, void *device_ptr);
 /* How the prefill matmuls carry their f32 activations:
  * 1: all f32 bits (three bf16 terms); 0: cast to bf16, one MFMA pass instead of
  * three; 2 (default): three int8 digit planes on the int8 matrix cores, 23 bits
- * below each row's largest magnitude (BUDDY_HIP_GEMM_A_I8_DIGITS). */
+ * below each row's largest magnitude (BUDDY_HIP_GEMM_A_I8_DIGITS); 3: two digit
+ * planes, 15 bits below it (BUDDY_HIP_GEMM_TWO_DIGITS), the int8 counterpart of
+ * mode 0. */
 int buddy_hip_session_set_prefill_precision(buddy_hip_session *s, int mode);
 /* Asynchronous pieces of the call above, for timing: set the device-side
  * (token, position), then enqueue steps on the session stream. */

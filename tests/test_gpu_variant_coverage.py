@@ -19,7 +19,8 @@ import oracle_lib
 from buddy_mlir_amd import ops, synthetic
 from buddy_mlir_amd.session import Shape
 from parity import check_close
-from test_gpu_prefill import SCALE, SILU_PAIR_SHAPES, bf16_round, run_attn, silu_pair_case
+from test_gpu_prefill import (SCALE, SILU_PAIR_SHAPES, bf16_round, fixed_point_round, run_attn,
+                              silu_pair_case)
 
 pytestmark = pytest.mark.gpu
 
@@ -190,10 +191,13 @@ def gemm_case(oracle, M, K, N, mode):
     q, s = synthetic.quantized_linear(K, N, M + K + N)
     g = torch.Generator(device="cuda").manual_seed(M)
     x = torch.randn((M, K), generator=g, device="cuda")
-    y = ops.gemm_w8a32(x, ops.pack_w8(q), s, K, N, exact=mode == "exact", digits=mode == "digits")
+    y = ops.gemm_w8a32(x, ops.pack_w8(q), s, K, N, exact=mode == "exact",
+                       digits={"digits": 3, "digits2": 2}.get(mode, False))
     torch.cuda.synchronize()
     xh = x.cpu().numpy()
     a_in = bf16_round(xh) if mode == "bf16" else xh
+    if mode == "digits2":
+        a_in, _ = fixed_point_round(xh, digits=2)
     want = oracle.blis_gemm_w8a32(a_in, q.cpu().numpy(), s.cpu().numpy())
     got = y.cpu().numpy()
     for m in range(M):
@@ -222,9 +226,11 @@ def test_every_int8_prefill_matmul_variant(bh, oracle):
     bh.buddy_hip_variant_reset()
     for M, K, N in GEMM_I8_SHAPES:
         gemm_case(oracle, M, K, N, "digits")
+        gemm_case(oracle, M, K, N, "digits2")  # the two-plane variants
         w8a8_case(bh, oracle, M, K, N)  # the one-plane variants of the same tile shapes
     for M, K, N in SILU_PAIR_SHAPES[1:5]:  # the paired variants
         silu_pair_case(oracle, M, K, N)
+        silu_pair_case(oracle, M, K, N, digits=2)
     for fam in ("gemm_w8_i8_wide_kernel", "gemm_w8_i8_kernel"):
         assert launched(bh, fam) == compiled(bh, fam), compiled(bh, fam) - launched(bh, fam)
 
