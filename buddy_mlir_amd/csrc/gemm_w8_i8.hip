@@ -33,6 +33,7 @@
 #include "gemm.h"
 
 #include <algorithm>
+#include <cstdlib>
 #include <map>
 #include <mutex>
 
@@ -1041,6 +1042,11 @@ int launch_gemm_w8_digits_d(const GemmW8Args &in, const void *planes, hipStream_
   //    partial sums, and the second kernel (3 us + its bytes at 3 TB/s);
   //  * 64 x 64 tiles, K split over the wavefronts: bound by L2 -> CU traffic,
   //    16 KiB per workgroup and chunk at about 6 TB/s.
+  // A norm that is to follow (then_norm_w) costs a launch of its own, about
+  // 5 us, unless the kernel that adds K slices writes its planes (it holds whole
+  // rows, up to kRowCache columns).
+  const double pending_norm = in.then_norm_w ? 5.0 : 0.0;
+  const bool slices_fuse_norm = gemm_staging_layout(in.M, in.N).cols_padded <= kRowCache;
   int best_gpw = 0, best_rb = 0, best_s = 0;
   double best_cost = 0;
   for (int gpw : {5, 4})
@@ -1059,6 +1065,8 @@ int launch_gemm_w8_digits_d(const GemmW8Args &in, const void *planes, hipStream_
         double cost = (double)ceil_div(per_xcd, 32) * wg;
         if (s > 1)
           cost += 3.0 + 4.0 * (double)(ncols * rows * s) * (kSlices * rb * 16 * gpw * 16) / 3e6;
+        if (s == 1 || !slices_fuse_norm)
+          cost += pending_norm;
         if (!best_gpw || cost < best_cost - 1e-9) {
           best_gpw = gpw;
           best_rb = rb;
@@ -1075,8 +1083,15 @@ int launch_gemm_w8_digits_d(const GemmW8Args &in, const void *planes, hipStream_
     return launch_rmsnorm_to_digits(in.C, in.ldc, in.then_norm_w, (int)in.M, (int)in.N,
                                     in.then_norm_eps, in.digits, in.then_norm_staged, stream);
   };
+  // The 64 x 64 kernel: two workgroups fit a compute unit, and a workgroup takes
+  // about 6 us for its first chunk per wavefront and 2 us for every further one
+  // (measured: 17.3 us for q|k|v, 18.6 us for o_proj at 512 rows, 72 us for
+  // down).  Neither it nor the unsplit wide kernel holds whole rows, so a norm
+  // that is to follow costs them a launch of its own.
   const int64_t split_wgs = ceil_div(a.groups, kSplitGroups) * (a.Mp / 64);
-  const double split_cost = 1.0 + (double)split_wgs * a.chunks * 16384.0 / 6e6;
+  const double split_cost =
+      1.0 + (double)ceil_div(split_wgs, 512) * (6.2 + 2.0 * (double)(ceil_div(a.chunks, kSlices) - 1)) +
+      pending_norm;
   if (split_cost < best_cost) {
     a.ncols = (int)ceil_div(a.groups, kSplitGroups);
     a.cols_padded = (int)round_up(a.ncols, 8);
@@ -1105,7 +1120,7 @@ int launch_gemm_w8_digits_d(const GemmW8Args &in, const void *planes, hipStream_
   if (best_s == 1)
     return then_norm();
   const GemmStagingLayout next = gemm_staging_layout(in.M, in.N);
-  if (in.then_norm_w && next.cols_padded <= kRowCache) {
+  if (in.then_norm_w && slices_fuse_norm) {
     // the kernel that adds the slices holds whole rows: it writes the planes too
     const size_t row_lds = 2 * sizeof(float) * (size_t)next.cols_padded;
     if (row_lds > 48 * 1024) { // up to 96 KiB at kRowCache columns

@@ -122,6 +122,7 @@ struct Session {
   float *kv_rows = nullptr; // staging of get_kv_rows, grown on demand
   size_t kv_rows_cap = 0;
   unsigned short *pf_xn_bf = nullptr, *pf_g_bf = nullptr; // bf16 matmul inputs
+  unsigned short *pf_att_dg = nullptr; // digit planes of the attention output (o_proj's input)
   int gemm_terms = 3; // bf16 terms per activation in the prefill matmuls (3 = exact)
   int gemm_digits = 3; // int8 digit planes instead of bf16 terms when not 0
 
@@ -312,7 +313,7 @@ struct Session {
       (void)hipFree(pf_tokens);
       pf_tokens = nullptr;
     }
-    for (unsigned short **p : {&pf_xn_bf, &pf_g_bf})
+    for (unsigned short **p : {&pf_xn_bf, &pf_g_bf, &pf_att_dg})
       if (*p) {
         (void)hipFree(*p);
         *p = nullptr;
@@ -332,6 +333,7 @@ struct Session {
                             lg = gemm_staging_layout(rows, S.inter);
     BH_CHECK_HIP(hipMalloc((void **)&pf_xn_bf, std::max(lx.bytes(3), lx.bytes_digits(3))));
     BH_CHECK_HIP(hipMalloc((void **)&pf_g_bf, std::max(lg.bytes(3), lg.bytes_digits(3))));
+    BH_CHECK_HIP(hipMalloc((void **)&pf_att_dg, gemm_staging_layout(rows, QN).bytes_digits(3)));
     pf_rows = rows;
     return BUDDY_HIP_OK;
   }
@@ -448,10 +450,23 @@ struct Session {
       a.scale = scale;
       if ((rc = launch_attn_prefill(a, stream)))
         return rc;
-      if ((rc = gemm(pf_att, L.o, pf_x, n, true)))
-        return rc;
-      if ((rc = norm_to_staging(pf_x, L.ln2, n, pf_xn_bf)))
-        return rc;
+      if (gemm_digits) {
+        // o_proj's finished rows go on as the normed input of gate and up: where
+        // the matmul splits K over workgroups, the kernel that adds the slices
+        // holds whole rows and writes those digit planes itself
+        if ((rc = launch_activations_to_digits(pf_att, (int64_t)S.heads * S.head_dim, n,
+                                               (int64_t)S.heads * S.head_dim, gemm_digits,
+                                               pf_att_dg, stream)))
+          return rc;
+        if ((rc = gemm_staged(reinterpret_cast<const unsigned short *>(pf_att_dg), L.o, pf_x, n,
+                              true, 0, L.ln2, pf_xn_bf)))
+          return rc;
+      } else {
+        if ((rc = gemm(pf_att, L.o, pf_x, n, true)))
+          return rc;
+        if ((rc = norm_to_staging(pf_x, L.ln2, n, pf_xn_bf)))
+          return rc;
+      }
       const int64_t ld_gu = 2 * (int64_t)S.inter;
       if (L.gate_up_joint && gemm_digits) {
         // gate and up in one launch whose workgroups hold matching tiles of
@@ -680,7 +695,7 @@ void buddy_hip_session_destroy(buddy_hip_session *hs) try {
     (void)hipFree(p);
   for (void *p : {(void *)s->pf_x, (void *)s->pf_xn, (void *)s->pf_qkv, (void *)s->pf_att,
                   (void *)s->pf_g, (void *)s->pf_tokens, (void *)s->kv_rows,
-                  (void *)s->pf_xn_bf, (void *)s->pf_g_bf})
+                  (void *)s->pf_xn_bf, (void *)s->pf_g_bf, (void *)s->pf_att_dg})
     if (p)
       (void)hipFree(p);
   if (s->host_state)
