@@ -65,6 +65,30 @@ def gate_up_traffic(collecting: bool = False):
     return int(m.group(2).replace(",", "")), TRAFFIC_PROFILE
 
 
+TRACE_PROFILE = "profiles/decode_step_qwen2_1p5b_ctx1024_kernel_trace.md"
+
+
+def gate_up_rocprof_us():
+    """Average duration of the dominant kernel in the timed replay of the loop
+    below, as rocprofv3's kernel trace of this same command recorded it (the
+    summary under profiles/): the second clock on `roofline.avg_launch_us`, so
+    that the fraction can be recomputed from the line alone.  None when the
+    summary is missing or was taken for another kernel."""
+    import re
+
+    path = ROOT / TRACE_PROFILE
+    if not path.exists():
+        return None, f"{TRACE_PROFILE} not found"
+    text = path.read_text()
+    m = re.search(r"## Dominant kernel: `([^`]+)`", text)
+    t = re.search(r"timed replay of the roofline loop.*?average ([0-9.]+) us", text, re.S)
+    if not m or not t:
+        return None, f"no dominant-kernel figures in {TRACE_PROFILE}"
+    if m.group(1) != GATE_UP_KERNEL:
+        return None, f"{TRACE_PROFILE} was taken for `{m.group(1)}`"
+    return float(t.group(1)), TRACE_PROFILE
+
+
 def gate_up_bytes(hidden: int, inter: int) -> int:
     """Algorithmic bytes of one fused RMSNorm + gate|up GEMV + SiLU*mul launch:
     two int8 matrices, their scales, the activation row, the norm weight and
@@ -962,6 +986,7 @@ def main():
     achieved = gu_b / gu_s / 1e9
     step_b = decode_step_bytes(shape, CONTEXT + W + K // 2)
     traffic, traffic_source = gate_up_traffic(collecting=args.calibrate_copy)
+    prof_us, prof_source = gate_up_rocprof_us()
 
     out = {
         "metric": "decode_tokens_per_s",
@@ -1003,6 +1028,11 @@ def main():
             "avg_launch_us": gu_s * 1e6,
             "traffic": traffic,
             "traffic_source": traffic_source,
+            # the same launches under rocprofv3 --kernel-trace (durations under the
+            # profiler come out a few per cent longer than HIP events without it)
+            "rocprof_avg_launch_us": prof_us,
+            "frac_rocprof": (gu_b / (prof_us * 1e-6) / 1e9 / HBM_PEAK_GBPS) if prof_us else None,
+            "rocprof_source": prof_source,
         },
     }
     if args.calibrate_copy:
