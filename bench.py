@@ -402,8 +402,9 @@ def bench_gemv(bh, args):
 
 
 def bench_mlp(bh, args):
-    """configs[1]: h = SiLU(x G) * (x U), y = h D at M in {1, 4, 16} (--mlp-rows): two launches
-    (fused gate|up, then down), 12 rotating weight sets (496 MB)."""
+    """configs[1]: h = SiLU(x G) * (x U), y = h D at M in {1, 4, 16} (--mlp-rows): one call of
+    buddy_hip_mlp_block_w8a32 (two launches: fused gate|up, then down), 12
+    rotating weight sets (496 MB)."""
     import torch
 
     H, I = 1536, 8960
@@ -420,15 +421,28 @@ def bench_mlp(bh, args):
         f1 = _linear_fn(bh, [(gu[2 * i], gu[2 * i + 1]) for i in range(12)], x, h, H, I, M, True, None, 2)
         f2 = _linear_fn(bh, [(w,) for w in dn], h, y, I, H, M, False, None, 0)
 
-        def fn(i):
+        def two_calls(i):
             f1(i)
             f2(i)
-        t = _time_launches(fn, 480)
+        # the block as one call (buddy_hip_mlp_block_w8a32)
+        from buddy_mlir_amd import ops
+        sc_i = torch.full((I,), 1e-3, device="cuda")
+        sc_h = torch.full((H,), 1e-3, device="cuda")
+        stream = torch.cuda.current_stream().cuda_stream
+        descs = [ops.mlp_block_desc(x, gu[2 * i], sc_i, gu[2 * i + 1], sc_i, dn[i], sc_h, y, H, I)
+                 for i in range(12)]
+
+        def block(i):
+            if bh.buddy_hip_mlp_block_w8a32(ctypes.byref(descs[i % 12][0]), stream):
+                raise RuntimeError("mlp_block_w8a32 failed")
+        t = _time_launches(block, 480)
         # three int8 matrices, their scales, M rows in and M rows out
         by = 3 * H * I + 4 * (2 * I + H) + 4 * M * 2 * H
         res[f"M={M}"] = {"us": t * 1e6, "gbps": by / t / 1e9,
                          "frac": by / t / 1e9 / HBM_PEAK_GBPS,
-                         # each launch on its own, same rotation
+                         # the same two matmuls as two buddy_hip_linear_w8a32 calls (f32
+                         # rows between them), and each of those on its own
+                         "two_linear_calls_us": _time_launches(two_calls, 480) * 1e6,
                          "gate_up_us": _time_launches(f1, 240) * 1e6,
                          "down_us": _time_launches(f2, 240) * 1e6}
     t = res["M=1"]["us"] * 1e-6

@@ -97,6 +97,8 @@ def _declare(lib):
         "buddy_hip_gemv_w8a32": (c_int, [vp, vp, vp, vp, i64, i64, i64, c_uint,
                                          vp]),
         "buddy_hip_linear_w8a32": (c_int, [vp, vp]),
+        "buddy_hip_mlp_block_workspace_bytes": (sz, [i64, i64]),
+        "buddy_hip_mlp_block_w8a32": (c_int, [vp, vp]),
         "buddy_hip_gemm_w8a32": (c_int, [vp, vp, vp, vp, i64, i64, i64, c_uint, vp]),
         "buddy_hip_rmsnorm": (c_int, [vp, vp, vp, c_int, c_int, c_float, vp]),
         "buddy_hip_rope": (c_int, [vp, vp, vp, c_int, c_int, vp]),

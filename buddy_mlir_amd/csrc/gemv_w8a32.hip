@@ -1716,6 +1716,59 @@ int buddy_hip_linear_w8a32(const buddy_hip_linear_desc *d,
   return bh::launch_gemv(a, bh::as_stream(stream));
 } BH_CATCH_INT("buddy_hip_linear_w8a32")
 
+size_t buddy_hip_mlp_block_workspace_bytes(int64_t M, int64_t inter) {
+  if (M < 1 || M > 16 || inter < 1)
+    return 0;
+  return (sizeof(float) * (size_t)M * (size_t)inter + 255) & ~(size_t)255;
+}
+
+int buddy_hip_mlp_block_w8a32(const buddy_hip_mlp_block_desc *d, buddy_hip_stream stream) try {
+  BH_REQUIRE(d, "mlp_block_w8a32: null descriptor");
+  BH_REQUIRE(d->x && d->gate && d->gate_scale && d->up && d->up_scale && d->down &&
+                 d->down_scale && d->y && d->workspace,
+             "mlp_block_w8a32: null pointer");
+  BH_REQUIRE(d->M >= 1 && d->M <= 16, "mlp_block_w8a32: M=%lld outside 1..16", (long long)d->M);
+  BH_REQUIRE(d->hidden > 0 && d->inter > 0 && d->ldx >= d->hidden && d->ldy >= d->hidden,
+             "mlp_block_w8a32: bad shape or row stride");
+  BH_REQUIRE(d->workspace_bytes >= buddy_hip_mlp_block_workspace_bytes(d->M, d->inter) &&
+                 (reinterpret_cast<uintptr_t>(d->workspace) & 15) == 0,
+             "mlp_block_w8a32: workspace of %zu bytes (16-byte aligned) needed, %zu given",
+             buddy_hip_mlp_block_workspace_bytes(d->M, d->inter), d->workspace_bytes);
+  hipStream_t s = bh::as_stream(stream);
+  float *h = static_cast<float *>(d->workspace); // [M, inter] between the two launches
+  bh::GemvArgs g;
+  g.A = d->x;
+  g.lda = d->ldx;
+  g.W0 = d->gate;
+  g.s0 = d->gate_scale;
+  g.W1 = d->up;
+  g.s1 = d->up_scale;
+  g.norm_w = d->norm_w;
+  g.norm_eps = d->norm_eps;
+  g.norm_inv_k = 1.0f / (float)d->hidden;
+  g.C = h;
+  g.ldc = d->inter;
+  g.M = (int)d->M;
+  g.K = d->hidden;
+  g.N = d->inter;
+  g.epilogue = bh::kEpiSiluMul;
+  int rc = bh::launch_gemv(g, s);
+  if (rc)
+    return rc;
+  bh::GemvArgs w;
+  w.A = h;
+  w.lda = d->inter;
+  w.W0 = d->down;
+  w.s0 = d->down_scale;
+  w.C = d->y;
+  w.ldc = d->ldy;
+  w.M = (int)d->M;
+  w.K = d->inter;
+  w.N = d->hidden;
+  w.epilogue = (d->flags & BUDDY_HIP_GEMV_ACCUMULATE) ? bh::kEpiAccum : bh::kEpiStore;
+  return bh::launch_gemv(w, s);
+} BH_CATCH_INT("buddy_hip_mlp_block_w8a32")
+
 int buddy_hip_gemv_w8a32(const float *A, const int8_t *packed,
                          const float *scale, float *C, int64_t M, int64_t K,
                          int64_t N, unsigned flags, buddy_hip_stream stream) try {

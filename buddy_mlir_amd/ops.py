@@ -42,6 +42,55 @@ def linear_w8a32(stream=None, **kw):
           "linear_w8a32")
 
 
+class MlpBlockDesc(ctypes.Structure):
+    """ctypes mirror of buddy_hip_mlp_block_desc."""
+    _fields_ = [("x", ctypes.c_void_p), ("ldx", ctypes.c_int64),
+                ("norm_w", ctypes.c_void_p), ("norm_eps", ctypes.c_float),
+                ("gate", ctypes.c_void_p), ("gate_scale", ctypes.c_void_p),
+                ("up", ctypes.c_void_p), ("up_scale", ctypes.c_void_p),
+                ("down", ctypes.c_void_p), ("down_scale", ctypes.c_void_p),
+                ("y", ctypes.c_void_p), ("ldy", ctypes.c_int64),
+                ("M", ctypes.c_int64), ("hidden", ctypes.c_int64), ("inter", ctypes.c_int64),
+                ("flags", ctypes.c_uint), ("workspace", ctypes.c_void_p),
+                ("workspace_bytes", ctypes.c_size_t)]
+
+
+def mlp_block_desc(x, gate, gate_scale, up, up_scale, down, down_scale, y, hidden: int,
+                   inter: int, norm_w=None, norm_eps: float = 0.0, accumulate: bool = False,
+                   workspace=None):
+    """Descriptor of buddy_hip_mlp_block_w8a32 over torch device tensors, plus
+    the workspace tensor it points into (keep it alive)."""
+    M = x.shape[0]
+    if workspace is None:
+        workspace = torch.empty(lib().buddy_hip_mlp_block_workspace_bytes(M, inter),
+                                dtype=torch.uint8, device=x.device)
+    d = MlpBlockDesc()
+    d.x, d.ldx = x.data_ptr(), x.stride(0)
+    d.norm_w = norm_w.data_ptr() if norm_w is not None else None
+    d.norm_eps = norm_eps
+    d.gate, d.gate_scale = gate.data_ptr(), gate_scale.data_ptr()
+    d.up, d.up_scale = up.data_ptr(), up_scale.data_ptr()
+    d.down, d.down_scale = down.data_ptr(), down_scale.data_ptr()
+    d.y, d.ldy = y.data_ptr(), y.stride(0)
+    d.M, d.hidden, d.inter = M, hidden, inter
+    d.flags = GEMV_ACCUMULATE if accumulate else 0
+    d.workspace, d.workspace_bytes = workspace.data_ptr(), workspace.numel()
+    return d, workspace
+
+
+def mlp_block_w8a32(x, gate, gate_scale, up, up_scale, down, down_scale, hidden: int,
+                    inter: int, y=None, stream=None, **kw):
+    """y (+)= (SiLU(x' . gate) * (x' . up)) . down for 1..16 rows (two launches)."""
+    if y is None:
+        y = torch.empty((x.shape[0], hidden), dtype=torch.float32, device=x.device)
+    d, ws = mlp_block_desc(x, gate, gate_scale, up, up_scale, down, down_scale, y, hidden,
+                           inter, **kw)
+    check(lib().buddy_hip_mlp_block_w8a32(ctypes.byref(d),
+                                          _stream() if stream is None else stream),
+          "mlp_block_w8a32")
+    return y
+
+
 def pack_w8_tiles(q: torch.Tensor, tile_n: int) -> torch.Tensor:
     _dev(q, torch.int8)
     K, N = q.shape

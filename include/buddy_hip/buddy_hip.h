@@ -198,6 +198,36 @@ int buddy_hip_gemv_w8a32(const float *A, const int8_t *packed,
                          const float *scale, float *C, int64_t M, int64_t K,
                          int64_t N, unsigned flags, buddy_hip_stream stream);
 
+/* One MLP block of a decoder layer at a decode batch of M = 1..16 rows:
+ *   y (+)= (SiLU(x' . gate) * (x' . up)) . down,   x' = RMSNorm(x) * norm_w or x
+ * (subgraph0_decode_simplify.mlir:210-260 over M rows): the two launches of
+ * buddy_hip_linear_w8a32 that make it (gate and up fused with SiLU * mul, then
+ * down) behind one call, with the same kernels and roundings.  All three
+ * matrices are wave-tile packed ([hidden, inter] twice, [inter, hidden]).  The
+ * intermediate rows [M, inter] f32 live in `workspace`
+ * (buddy_hip_mlp_block_workspace_bytes(M, inter) bytes, 16-byte aligned).  No
+ * counterpart in the reference, whose decode kernels are m == 1 only. */
+typedef struct buddy_hip_mlp_block_desc {
+  const float *x;          /* [M, hidden], row stride ldx */
+  int64_t ldx;
+  const float *norm_w;     /* [hidden] or NULL; 16-byte aligned */
+  float norm_eps;
+  const int8_t *gate;      /* packed [hidden, inter] */
+  const float *gate_scale; /* [inter] */
+  const int8_t *up;
+  const float *up_scale;
+  const int8_t *down;      /* packed [inter, hidden] */
+  const float *down_scale; /* [hidden] */
+  float *y;                /* [M, hidden], row stride ldy */
+  int64_t ldy;
+  int64_t M, hidden, inter;
+  unsigned flags;          /* BUDDY_HIP_GEMV_ACCUMULATE: y += ... (the residual) */
+  void *workspace;
+  size_t workspace_bytes;
+} buddy_hip_mlp_block_desc;
+size_t buddy_hip_mlp_block_workspace_bytes(int64_t M, int64_t inter);
+int buddy_hip_mlp_block_w8a32(const buddy_hip_mlp_block_desc *d, buddy_hip_stream stream);
+
 /* Full form of the kernel above with the fusions a decoder layer uses.
  * Every pointer is device memory. */
 typedef struct buddy_hip_linear_desc {

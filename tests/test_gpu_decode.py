@@ -28,6 +28,100 @@ def linear(bh, **kw):
     torch.cuda.synchronize()
 
 
+def mlp_block_oracle(oracle, xh, qg, sg, qu, su, qd, sd, norm_w=None, eps=None, y0=None):
+    """The block on the CPU: M = 1 follows the decode GEMV kernel, more rows the
+    BLIS kernel (the only vectorised reference kernel for M > 1)."""
+    M = xh.shape[0]
+    if norm_w is not None:
+        xh = np.stack([oracle.rmsnorm(r, norm_w, eps, np.float32(1.0) / np.float32(xh.shape[1]))
+                       for r in xh])
+    if M == 1:
+        g = oracle.dequant_gemv(xh[0], qg, sg)[None]
+        u = oracle.dequant_gemv(xh[0], qu, su)[None]
+    else:
+        g = oracle.blis_gemm_w8a32(xh, qg, sg)
+        u = oracle.blis_gemm_w8a32(xh, qu, su)
+    hh = np.stack([oracle.silu_mul(g[m], u[m]) for m in range(M)])
+    if M == 1:
+        return oracle.dequant_gemv(hh[0], qd, sd, None if y0 is None else y0[0])[None]
+    return oracle.blis_gemm_w8a32(hh, qd, sd, None if y0 is None else y0.copy())
+
+
+@pytest.mark.parametrize("M", [1, 4, 5, 8, 9, 13, 16])
+def test_mlp_block_entry_point_matches_oracle(bh, oracle, M):
+    """BASELINE configs[1] through the one call made for it: 1536 <-> 8960,
+    plain, and with the RMSNorm in front and the residual behind that a decoder
+    layer has."""
+    H, I = 1536, 8960
+    qg, sg = synthetic.quantized_linear(H, I, 11)
+    qu, su = synthetic.quantized_linear(H, I, 12)
+    qd, sd = synthetic.quantized_linear(I, H, 13)
+    g = torch.Generator(device="cuda").manual_seed(M)
+    x = torch.randn((M, H), generator=g, device="cuda")
+    if M > 2:
+        x[1] *= 1e-6   # rows of very different size (h goes with the square): the
+        x[2] *= 1e5    # steps are per row
+    w = 1 + 0.1 * torch.randn(H, generator=g, device="cuda")
+    y0 = torch.randn((M, H), generator=g, device="cuda")
+    pg, pu, pd = ops.pack_w8(qg), ops.pack_w8(qu), ops.pack_w8(qd)
+    torch.cuda.synchronize()
+    y = ops.mlp_block_w8a32(x, pg, sg, pu, su, pd, sd, H, I)
+    y2 = y0.clone()
+    ops.mlp_block_w8a32(x, pg, sg, pu, su, pd, sd, H, I, y=y2, norm_w=w, norm_eps=1e-6,
+                        accumulate=True)
+    torch.cuda.synchronize()
+    hq = [t.cpu().numpy() for t in (qg, sg, qu, su, qd, sd)]
+    want = mlp_block_oracle(oracle, x.cpu().numpy(), *hq)
+    want2 = mlp_block_oracle(oracle, x.cpu().numpy(), *hq, norm_w=w.cpu().numpy(),
+                             eps=np.float32(1e-6), y0=y0.cpu().numpy())
+    got, got2 = y.cpu().numpy(), y2.cpu().numpy()
+    for m in range(M):
+        check_close(got[m], want[m])
+        check_close(got2[m], want2[m])
+
+
+@pytest.mark.parametrize("M,H,I", [(7, 256, 100), (16, 64, 33), (5, 192, 70), (11, 320, 1000),
+                                   (8, 128, 64), (16, 1536, 96)])
+def test_mlp_block_ragged_shapes(bh, oracle, M, H, I):
+    """Intermediate sizes that end inside a tile of 64 k or inside a channel
+    group."""
+    qg, sg = synthetic.quantized_linear(H, I, 21)
+    qu, su = synthetic.quantized_linear(H, I, 22)
+    qd, sd = synthetic.quantized_linear(I, H, 23)
+    x = torch.randn((M, H), generator=torch.Generator(device="cuda").manual_seed(M + I),
+                    device="cuda") * 3
+    y = ops.mlp_block_w8a32(x, ops.pack_w8(qg), sg, ops.pack_w8(qu), su, ops.pack_w8(qd), sd, H, I)
+    torch.cuda.synchronize()
+    want = mlp_block_oracle(oracle, x.cpu().numpy(),
+                            *[t.cpu().numpy() for t in (qg, sg, qu, su, qd, sd)])
+    got = y.cpu().numpy()
+    for m in range(M):
+        check_close(got[m], want[m])
+
+
+def test_mlp_block_non_finite_rows_and_refusals(bh, oracle):
+    H, I, M = 256, 512, 9
+    qg, sg = synthetic.quantized_linear(H, I, 31)
+    qu, su = synthetic.quantized_linear(H, I, 32)
+    qd, sd = synthetic.quantized_linear(I, H, 33)
+    pg, pu, pd = ops.pack_w8(qg), ops.pack_w8(qu), ops.pack_w8(qd)
+    x = torch.randn((M, H), generator=torch.Generator(device="cuda").manual_seed(3), device="cuda")
+    clean = ops.mlp_block_w8a32(x, pg, sg, pu, su, pd, sd, H, I).cpu().numpy()
+    x[2, 5] = float("nan")
+    x[7, 0] = float("inf")
+    got = ops.mlp_block_w8a32(x, pg, sg, pu, su, pd, sd, H, I).cpu().numpy()
+    assert np.isnan(got[[2, 7]]).all()
+    rest = [m for m in range(M) if m not in (2, 7)]
+    np.testing.assert_array_equal(got[rest], clean[rest])
+    # a workspace that is too small, and too many rows
+    y = torch.empty((M, H), device="cuda")
+    d, ws = ops.mlp_block_desc(x, pg, sg, pu, su, pd, sd, y, H, I)
+    d.workspace_bytes = 16
+    assert bh.buddy_hip_mlp_block_w8a32(ctypes.byref(d), None) != 0
+    assert b"workspace" in bh.buddy_hip_last_error()
+    assert bh.buddy_hip_mlp_block_workspace_bytes(17, I) == 0
+
+
 @pytest.mark.parametrize("M", [1, 4, 16])
 def test_mlp_block_matches_oracle(bh, oracle, M):
     """h = SiLU(x.G) * (x.U); y = h.D -- the fused gate|up kernel and the down
