@@ -348,6 +348,28 @@ def test_prefill_in_two_blocks_and_after_decode_steps(oracle):
     sess.close()
 
 
+def test_wide_hidden_size_through_the_slice_adding_norm_kernel(oracle):
+    """hidden = 9216: the kernel that adds the K slices of o_proj / down and
+    writes the next RMSNorm's digit planes keeps two copies of a row in LDS,
+    72 KiB here -- more than the 64 KiB a kernel gets without asking.  A
+    prompt of 64 tokens (one row tile: the matmuls then split K over
+    workgroups) against 64 oracle decode steps."""
+    shape = Shape(layers=2, hidden=9216, heads=8, kv_heads=2, head_dim=128, inter=2048,
+                  vocab=512, max_len=128, rms_eps=1e-6)
+    sess, host = synthetic.build_session(shape, context=0, keep_host=True, ln_jitter=0.1)
+    om = oracle_model(oracle, shape, host)
+    kv = [a.copy() for a in host["kv"]]
+    toks = synthetic.first_tokens(shape, 64, seed=23).tolist()
+    for pos, t in enumerate(toks):
+        otok, ologits = om.decode_step(t, pos, kv)
+    nxt, logits = sess.prefill(toks, 0)
+    check_close(logits, ologits)
+    assert nxt == otok
+    for j in range(2 * shape.layers):
+        check_close(sess.get_kv(j)[:, :64, :], kv[j][:, :64, :])
+    sess.close()
+
+
 @pytest.mark.timeout(900)
 def test_qwen2_1p5b_shape_512_token_prefill(oracle):
     """The full 28-layer shape, a prompt of 512 tokens as one block (digit-plane
