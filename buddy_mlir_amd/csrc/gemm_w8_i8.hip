@@ -1061,7 +1061,13 @@ int launch_gemm_w8_digits_d(const GemmW8Args &in, const void *planes, hipStream_
         const int64_t cps = ceil_div(a.chunks, s);
         if (ceil_div(a.chunks, cps) != s)
           continue; // the last slice would be empty
-        const double wg = 0.0125 * (double)(cps * gpw * rb * in.digits) + 7.0 + (s > 1 ? 2.0 : 0.0);
+        // (with the whole K in one workgroup a chunk of the pipelined loop takes
+        // 0.55 us however few matrix instructions it holds -- its barrier, staging
+        // and waits: 512 x 1536 x 2048 on two planes as 88 tiles of 48 x 256 took
+        // 19.4 us where 24 x 0.3 + 7 would be 14.2)
+        const double chunk_us =
+            std::max(0.0125 * (double)(gpw * rb * in.digits), s == 1 ? 0.55 : 0.0);
+        const double wg = chunk_us * (double)cps + 7.0 + (s > 1 ? 2.0 : 0.0);
         double cost = (double)ceil_div(per_xcd, 32) * wg;
         if (s > 1)
           cost += 3.0 + 4.0 * (double)(ncols * rows * s) * (kSlices * rb * 16 * gpw * 16) / 3e6;

@@ -184,6 +184,10 @@ def test_row_gemv_random_shapes(bh, oracle):
 # ---- prefill matmul: the tile shape comes out of the launch's cost model -------
 GEMM_I8_SHAPES = [(144, 256, 16384), (300, 256, 10240), (200, 192, 16384), (512, 192, 8960),
                   (17, 64, 64)]
+# with two planes every unsplit tile costs the loop's floor per chunk, so the
+# widest tile wins there; the other tile shapes are reached with K split over
+# workgroups
+GEMM_I8_SPLIT_K_SHAPES = [(17, 1536, 256), (100, 4096, 8192), (100, 4096, 12288)]
 GEMM_BF16_SHAPES = [(512, 64, 8960), (300, 64, 10240), (17, 64, 64)]
 
 
@@ -228,6 +232,9 @@ def test_every_int8_prefill_matmul_variant(bh, oracle):
         gemm_case(oracle, M, K, N, "digits")
         gemm_case(oracle, M, K, N, "digits2")  # the two-plane variants
         w8a8_case(bh, oracle, M, K, N)  # the one-plane variants of the same tile shapes
+    for M, K, N in GEMM_I8_SPLIT_K_SHAPES:
+        gemm_case(oracle, M, K, N, "digits")
+        gemm_case(oracle, M, K, N, "digits2")
     for M, K, N in SILU_PAIR_SHAPES[1:5]:  # the paired variants
         silu_pair_case(oracle, M, K, N)
         silu_pair_case(oracle, M, K, N, digits=2)
