@@ -20,9 +20,13 @@ namespace bh {
 namespace {
 
 constexpr int kD = 128;
-constexpr int kQB = 16;            // query rows per workgroup
+constexpr int kQB = 16;            // query rows per block
 constexpr int kKB = 16;            // key positions per step of a wavefront
-constexpr int kAttnWaves = 4;      // wavefronts per workgroup; they split the keys
+constexpr int kAttnWaves = 8;      // wavefronts per workgroup; they split the keys
+constexpr int kKPitch = kD + 4;    // floats per key row in LDS (fragment reads hit every bank once)
+constexpr int kOutPitch = kWave + 1;      // floats per accumulator register row of a partial output in LDS
+constexpr int kSlotFloats = kKB * kKPitch; // a wavefront's part of LDS: a K block, later its partial output
+static_assert(32 * kOutPitch <= kSlotFloats, "partial output must fit the slot");
 constexpr float kSeedM = -1.0e30f; // tosa.py:4383
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
@@ -34,90 +38,84 @@ struct PrefillArgs {
   float *out;         // token t, head h at out + t*o_stride + h*o_hstride
   int64_t q_stride, q_hstride, o_stride, o_hstride, kv_stride;
   int heads, group, q_len, k_len, q_offset; // query i sits at key position q_offset + i
+  int nqb;                                  // query blocks of kQB rows
   float scale;
 };
 
-// One workgroup: 16 query rows of one head.  Its four wavefronts take the 16-key
-// blocks round robin, each with its own running (max, sum, output), and merge
-// at the end.  All products run on the f32 matrix cores (16x16x4), operands
-// straight from global memory in fragment layout:
+// LDS of a workgroup, in floats: the Q fragments of its two query blocks, one
+// slot per wavefront, the (max, sum) pairs of the partial results and which part
+// each wavefront worked on.
+constexpr int kQFloats = 2 * 8 * kWave * 4;
+constexpr int kLdsFloats = kQFloats + kAttnWaves * kSlotFloats + 2 * kAttnWaves * kQB + kAttnWaves;
+
+// One workgroup: two blocks of 16 query rows of one head, block j from the start
+// and block j from the end, so that under the causal mask every workgroup has the
+// same number of 16-key blocks before it (one query block alone would have
+// between 1 and q_len / 16 of them, and the launch would last as long as the
+// longest).  The eight wavefronts are dealt to the two query blocks in proportion
+// to their key blocks; those of a query block split its key blocks into equal
+// contiguous shares, each with its own running (max, sum, output), and the
+// partial results meet in LDS at the end.
+// All products run on the f32 matrix cores (16x16x4):
 //   S^T[key, query] = K . Q^T   (contraction over d; in step 4J + e a lane
 //                                supplies d = 16 J + 4 (lane/16) + e, for K and
-//                                Q alike: the four lane groups of a load read 64
-//                                contiguous bytes of a row, so a K load touches
-//                                16 pieces of memory and not 64)
+//                                Q alike)
 //   O^T[d, query]  += V^T . P^T (contraction over the key; the S^T accumulator
 //                                registers ARE the P^T operand of step r: a
 //                                lane holds keys 4*(lane/16) + r of query lane%16)
 // so the scores never leave the registers between the two products.
 __global__ void __launch_bounds__(kAttnWaves *kWave) __attribute__((amdgpu_waves_per_eu(2, 2)))
 attn_prefill_kernel(PrefillArgs a) {
-  __shared__ float o_s[kAttnWaves][32][kWave];
-  __shared__ float m_s[kAttnWaves][kQB], l_s[kAttnWaves][kQB];
+  extern __shared__ __attribute__((aligned(16))) float lds[];
+  f32x4 *q_s = reinterpret_cast<f32x4 *>(lds);          // [2][8][64]: part, J, lane
+  float *slot_s = lds + kQFloats;                  // [kAttnWaves][kSlotFloats]
+  float *m_s = slot_s + kAttnWaves * kSlotFloats;  // [kAttnWaves][kQB]
+  float *l_s = m_s + kAttnWaves * kQB;
+  int *part_s = reinterpret_cast<int *>(l_s + kAttnWaves * kQB); // [kAttnWaves]: part, or -1
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  // workgroups start in id order: the last query blocks, which see the most
-  // keys, come first for every head, the short ones fill the gaps at the end
   const int h = blockIdx.x, kvh = h / a.group;
-  const int q0 = ((int)gridDim.y - 1 - (int)blockIdx.y) * kQB;
-  const int nq = min(kQB, a.q_len - q0);
   const int qi = lane & 15, lg = lane >> 4; // query of this lane; lane group
-  const int qrow = q0 + min(qi, nq - 1);    // rows past the end repeat the last
-
-  // Q^T fragment: qf[4J + e] is d = 16 J + 4 lg + e
-  float qf[32];
-  {
-    const float *src = a.q + (int64_t)qrow * a.q_stride + (int64_t)h * a.q_hstride + lg * 4;
+  // part 0: query block blockIdx.y, part 1: its mirror image (the same block in
+  // the middle of an odd number of blocks: then part 0 is empty)
+  const int qb1 = a.nqb - 1 - (int)blockIdx.y;
+  const bool single = qb1 == (int)blockIdx.y;
+  int q0[2], nq[2], nb[2];
 #pragma unroll
-    for (int j = 0; j < 32; j += 4) {
-      const float4 v = *reinterpret_cast<const float4 *>(src + 4 * j);
-      qf[j] = v.x;
-      qf[j + 1] = v.y;
-      qf[j + 2] = v.z;
-      qf[j + 3] = v.w;
-    }
+  for (int p = 0; p < 2; ++p) {
+    q0[p] = (p ? qb1 : (int)blockIdx.y) * kQB;
+    nq[p] = min(kQB, a.q_len - q0[p]);
+    // last key any query of the block may see
+    const int k_last = a.mask ? a.k_len - 1 : min(a.k_len - 1, a.q_offset + q0[p] + nq[p] - 1);
+    nb[p] = k_last / kKB + 1;
   }
-  // last key any query of this workgroup may see
-  const int k_last = a.mask ? a.k_len - 1
-                            : min(a.k_len - 1, a.q_offset + q0 + nq - 1);
-  const int nblocks = k_last / kKB + 1;
+  if (single)
+    nb[0] = 0;
+  const int total = nb[0] + nb[1];
+  // wavefronts [0, wa) work on part 0, the others on part 1
+  const int wa = nb[0] ? max(1, min(kAttnWaves - 1, (kAttnWaves * nb[0] + total / 2) / total)) : 0;
+  // key blocks [b0, b1) of its part (fewer than 2^16 blocks, at most 8 shares)
+  const int part = wave < wa ? 0 : 1;
+  const unsigned sn = part ? kAttnWaves - wa : wa, si = part ? wave - wa : wave;
+  const int b0 = (int)((unsigned)nb[part] * si / sn), b1 = (int)((unsigned)nb[part] * (si + 1) / sn);
+  const int pq0 = q0[part], pnq = nq[part];
+
   const float *kbase = a.k + (int64_t)kvh * a.kv_stride * kD;
   const float *vbase = a.v + (int64_t)kvh * a.kv_stride * kD;
-
-  float m_run = kSeedM, l_run = 0.f; // l_run: this lane's share of the row sum
-  f32x4 acc[8]; // O^T: acc[2*e + half][r] is d = 64*half + 4*(4*lg + r) + e
-#pragma unroll
-  for (int i = 0; i < 8; ++i)
-    acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+  float *ks = slot_s + wave * kSlotFloats;
 
   // K and V of a key block: 16 loads, issued by hand one block ahead of the
   // block being multiplied (the compiler sinks ordinary loads down to their
   // first use, which leaves the matrix cores waiting out every L2 round trip).
-  // A fetch is always exactly 16 loads -- blocks past the end fetch the last
-  // block again -- so that vmcnt(16) means "everything but the newest fetch has
-  // arrived".  The registers of a fetch are only read after such a wait names
-  // them; the build refuses scratch use in this file.
+  // A fetch is always exactly 16 loads, so that vmcnt(16) means "everything but
+  // the newest fetch has arrived".  The registers of a fetch are only read after
+  // such a wait names them; the build refuses scratch use in this file.
   struct Frag {
     f32x4 k[8], v[8];
   };
   auto issue = [](f32x4 &dst, const float *p) {
     asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(dst) : "v"(p) : "memory");
-  };
-  auto fetch = [&](int b, Frag &f) {
-    const int p0 = min(b, nblocks - 1) * kKB;
-    // K fragment: key p0 + lane%16, k[J] is d = 16 J + 4 lg + 0..3
-    const float *ks = kbase + (int64_t)min(p0 + qi, a.k_len - 1) * kD + lg * 4;
-#pragma unroll
-    for (int j = 0; j < 8; ++j)
-      issue(f.k[j], ks + 16 * j);
-    // V^T fragments: key p0 + 4*lg + r, d = 64*half + 4*(lane%16) + 0..3
-#pragma unroll
-    for (int r = 0; r < 4; ++r) {
-      const float *vs = vbase + (int64_t)min(p0 + 4 * lg + r, a.k_len - 1) * kD + 4 * qi;
-      issue(f.v[2 * r], vs);
-      issue(f.v[2 * r + 1], vs + 64);
-    }
   };
   auto arrived = [](Frag &f, auto n_in_flight) { // at most N loads still in flight
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"(decltype(n_in_flight)::value) : "memory");
@@ -127,7 +125,62 @@ attn_prefill_kernel(PrefillArgs a) {
       asm volatile("" : "+v"(f.v[j])::"memory");
     }
   };
+  auto fetch = [&](int b, Frag &f) {
+    const int p0 = b * kKB;
+    // K rows as they lie: load i is keys p0 + 2 i and p0 + 2 i + 1, a lane's four
+    // values d = 4 (lane % 32) + 0..3 (half a wavefront reads one whole row)
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+      issue(f.k[i], kbase + (int64_t)min(p0 + 2 * i + (lane >> 5), a.k_len - 1) * kD +
+                        (lane & 31) * 4);
+    // V^T fragments: key p0 + 4*lg + r, d = 64*half + 4*(lane%16) + 0..3
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const float *vs = vbase + (int64_t)min(p0 + 4 * lg + r, a.k_len - 1) * kD + 4 * qi;
+      issue(f.v[2 * r], vs);
+      issue(f.v[2 * r + 1], vs + 64);
+    }
+  };
+  Frag fa, fb;
+  if (b0 < b1)
+    fetch(b0, fa); // on its way while the queries are staged
+
+  { // Q^T fragments into LDS: wavefront w loads J = 2 (w % 4), + 1 of part w / 4
+    const int p = wave >> 2;
+    const int qrow = q0[p] + min(qi, nq[p] - 1); // rows past the end repeat the last
+    const float *src = a.q + (int64_t)qrow * a.q_stride + (int64_t)h * a.q_hstride + lg * 4;
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      const int J = 2 * (wave & 3) + t;
+      q_s[(p * 8 + J) * kWave + lane] = *reinterpret_cast<const f32x4 *>(src + 16 * J);
+    }
+  }
+  __syncthreads();
+
+  float qf[32]; // Q^T fragment: qf[4J + e] is d = 16 J + 4 lg + e of this lane's query
+#pragma unroll
+  for (int J = 0; J < 8; ++J) {
+    const f32x4 v = q_s[(part * 8 + J) * kWave + lane];
+    qf[4 * J] = v[0];
+    qf[4 * J + 1] = v[1];
+    qf[4 * J + 2] = v[2];
+    qf[4 * J + 3] = v[3];
+  }
+  float m_run = kSeedM, l_run = 0.f; // l_run: this lane's share of the row sum
+  f32x4 acc[8]; // O^T: acc[2*e + half][r] is d = 64*half + 4*(4*lg + r) + e
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+    acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
   auto block = [&](const Frag &f, int b) {
+    // The K rows turn into fragments through this wavefront's part of LDS: lane
+    // (qi, lg) reads d = 16 J + 4 lg + 0..3 of key p0 + qi.  (Fetched in that
+    // layout straight from memory, a load touches 16 rows with every 16 lanes.)
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+      *reinterpret_cast<f32x4 *>(ks + (2 * i + (lane >> 5)) * kKPitch + (lane & 31) * 4) = f.k[i];
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
     // ---- S^T block: keys x queries ------------------------------------------
     // four independent partial sums: a matrix instruction that adds to the
     // result of the one before it cannot issue until that one has finished
@@ -136,39 +189,45 @@ attn_prefill_kernel(PrefillArgs a) {
     for (int e = 0; e < 4; ++e)
       sp[e] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int j = 0; j < 8; ++j)
+    for (int j = 0; j < 8; ++j) {
+      const f32x4 kf = *reinterpret_cast<const f32x4 *>(ks + qi * kKPitch + 16 * j + 4 * lg);
 #pragma unroll
       for (int e = 0; e < 4; ++e)
-        sp[e] = __builtin_amdgcn_mfma_f32_16x16x4f32(f.k[j][e], qf[4 * j + e], sp[e], 0, 0, 0);
+        sp[e] = __builtin_amdgcn_mfma_f32_16x16x4f32(kf[e], qf[4 * j + e], sp[e], 0, 0, 0);
+    }
+    // (the next block's rows are written after these reads: one wavefront's LDS
+    // operations complete in order)
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
     const f32x4 st = (sp[0] + sp[1]) + (sp[2] + sp[3]);
-    // lane holds keys p0 + 4*lg + r of query q0 + qi
+    // lane holds keys p0 + 4*lg + r of query pq0 + qi
     const int p0 = b * kKB;
     float sc[4];
     float m_blk = -INFINITY;
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
       const int kp = p0 + 4 * lg + r;
-      float v = st[r] * a.scale;
-      bool ok = qi < nq && kp < a.k_len;
+      float x = st[r] * a.scale;
+      bool ok = qi < pnq && kp < a.k_len;
       if (ok) {
         if (a.mask)
-          v += a.mask[(int64_t)(q0 + qi) * a.k_len + kp];
+          x += a.mask[(int64_t)(pq0 + qi) * a.k_len + kp];
         else
-          ok = kp <= a.q_offset + q0 + qi;
+          ok = kp <= a.q_offset + pq0 + qi;
       }
-      sc[r] = ok ? v : -INFINITY;
+      sc[r] = ok ? x : -INFINITY;
       m_blk = fmaxf(m_blk, sc[r]);
     }
     m_blk = fmaxf(m_blk, __shfl_xor(m_blk, 16, 64));
     m_blk = fmaxf(m_blk, __shfl_xor(m_blk, 32, 64));
     const float m_new = fmaxf(m_run, m_blk); // m_run is finite, so m_new is
     const float alpha = expf(m_run - m_new);
-    float p[4];
+    float pr[4];
     float l_blk = 0.f;
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
-      p[r] = expf(sc[r] - m_new);
-      l_blk += p[r];
+      pr[r] = expf(sc[r] - m_new);
+      l_blk += pr[r];
     }
     l_run = l_run * alpha + l_blk;
     m_run = m_new;
@@ -181,69 +240,93 @@ attn_prefill_kernel(PrefillArgs a) {
 #pragma unroll
       for (int half = 0; half < 2; ++half) {
         const f32x4 vv = f.v[2 * r + half];
-        acc[0 + half] = __builtin_amdgcn_mfma_f32_16x16x4f32(vv[0], p[r], acc[0 + half], 0, 0, 0);
-        acc[2 + half] = __builtin_amdgcn_mfma_f32_16x16x4f32(vv[1], p[r], acc[2 + half], 0, 0, 0);
-        acc[4 + half] = __builtin_amdgcn_mfma_f32_16x16x4f32(vv[2], p[r], acc[4 + half], 0, 0, 0);
-        acc[6 + half] = __builtin_amdgcn_mfma_f32_16x16x4f32(vv[3], p[r], acc[6 + half], 0, 0, 0);
+        acc[0 + half] = __builtin_amdgcn_mfma_f32_16x16x4f32(vv[0], pr[r], acc[0 + half], 0, 0, 0);
+        acc[2 + half] = __builtin_amdgcn_mfma_f32_16x16x4f32(vv[1], pr[r], acc[2 + half], 0, 0, 0);
+        acc[4 + half] = __builtin_amdgcn_mfma_f32_16x16x4f32(vv[2], pr[r], acc[4 + half], 0, 0, 0);
+        acc[6 + half] = __builtin_amdgcn_mfma_f32_16x16x4f32(vv[3], pr[r], acc[6 + half], 0, 0, 0);
       }
     }
   };
-  Frag fa, fb;
-  fetch(wave, fa);
-  for (int b = wave; b < nblocks; b += 2 * kAttnWaves) {
-    fetch(b + kAttnWaves, fb);
-    arrived(fa, std::integral_constant<int, 16>{});
-    block(fa, b);
-    fetch(b + 2 * kAttnWaves, fa);
-    arrived(fb, std::integral_constant<int, 16>{});
-    if (b + kAttnWaves < nblocks)
-      block(fb, b + kAttnWaves);
-  }
-  // the last fetch (a repeated block) may still be in flight: its registers stay
-  // allocated until it has landed
-  arrived(fa, std::integral_constant<int, 0>{});
-  arrived(fb, std::integral_constant<int, 0>{});
-  // this wavefront's row sums: the four lane groups hold different keys
-  l_run += __shfl_xor(l_run, 16, 64);
-  l_run += __shfl_xor(l_run, 32, 64);
-
-  // ---- merge the wavefronts (the reference's combine rule, in wave order) ----
+  if (b0 < b1) {
+    // fa holds (in flight) block b; nothing is fetched past the end of the share
+    int b = b0;
+    for (; b + 2 < b1; b += 2) {
+      fetch(b + 1, fb);
+      arrived(fa, std::integral_constant<int, 16>{});
+      block(fa, b);
+      fetch(b + 2, fa);
+      arrived(fb, std::integral_constant<int, 16>{});
+      block(fb, b + 1);
+    }
+    if (b + 1 < b1) {
+      fetch(b + 1, fb);
+      arrived(fa, std::integral_constant<int, 16>{});
+      block(fa, b);
+      arrived(fb, std::integral_constant<int, 0>{});
+      block(fb, b + 1);
+    } else {
+      arrived(fa, std::integral_constant<int, 0>{});
+      block(fa, b);
+    }
+    // this wavefront's row sums: the four lane groups hold different keys
+    l_run += __shfl_xor(l_run, 16, 64);
+    l_run += __shfl_xor(l_run, 32, 64);
+    // (rows of kWave + 1 floats: the merge reads them by column)
 #pragma unroll
-  for (int i = 0; i < 8; ++i)
+    for (int i = 0; i < 8; ++i)
 #pragma unroll
-    for (int r = 0; r < 4; ++r)
-      o_s[wave][i * 4 + r][lane] = acc[i][r];
-  if (lg == 0) {
-    m_s[wave][qi] = m_run;
-    l_s[wave][qi] = l_run;
+      for (int r = 0; r < 4; ++r)
+        ks[(i * 4 + r) * kOutPitch + lane] = acc[i][r];
+    if (lg == 0) {
+      m_s[wave * kQB + qi] = m_run;
+      l_s[wave * kQB + qi] = l_run;
+    }
   }
+  if (lane == 0)
+    part_s[wave] = b0 < b1 ? part : -1;
   __syncthreads();
-  float m_all = m_s[0][qi];
+
+  // ---- merge the partial results (the reference's combine rule, in wave order).
+  // A thread finishes four consecutive d of one query per part, so that a
+  // wavefront writes two whole rows of the output: value d = 64 half + 16 lg +
+  // 4 r + e of query q is accumulator 2 e + half, register r of lane 16 lg + q.
+  const int c = lane & 31, mq = 2 * wave + (lane >> 5);
+  const int m_half = c >> 4, m_lg = (c >> 2) & 3, m_r = c & 3;
 #pragma unroll
-  for (int w = 1; w < kAttnWaves; ++w)
-    m_all = fmaxf(m_all, m_s[w][qi]);
-  float wgt[kAttnWaves], l_all = 0.f;
+  for (int p = 0; p < 2; ++p) {
+    if ((single && p == 0) || mq >= nq[p])
+      continue;
+    float wgt[kAttnWaves], m_w[kAttnWaves], m_all = kSeedM, l_all = 0.f;
+    bool has[kAttnWaves];
 #pragma unroll
-  for (int w = 0; w < kAttnWaves; ++w) {
-    wgt[w] = expf(m_s[w][qi] - m_all);
-    l_all = fmaf(l_s[w][qi], wgt[w], l_all);
-  }
-  if (qi >= nq)
-    return;
-  const float inv = 1.0f / l_all;
-  float *o = a.out + (int64_t)(q0 + qi) * a.o_stride + (int64_t)h * a.o_hstride;
-  // wavefront w finishes accumulators 2w and 2w+1 (e = w, both halves)
+    for (int w = 0; w < kAttnWaves; ++w) {
+      // (what a wavefront of the other part, or one without a share, left in its
+      // slot is not a number to be multiplied by zero: it is not looked at)
+      has[w] = part_s[w] == p;
+      m_w[w] = has[w] ? m_s[w * kQB + mq] : kSeedM;
+      m_all = fmaxf(m_all, m_w[w]);
+    }
 #pragma unroll
-  for (int half = 0; half < 2; ++half) {
-    const int i = 2 * wave + half;
+    for (int w = 0; w < kAttnWaves; ++w) {
+      wgt[w] = has[w] ? expf(m_w[w] - m_all) : 0.f;
+      const float l = has[w] ? l_s[w * kQB + mq] : 0.f;
+      l_all = fmaf(l, wgt[w], l_all);
+    }
+    const float inv = 1.0f / l_all;
+    f32x4 o;
 #pragma unroll
-    for (int r = 0; r < 4; ++r) {
+    for (int e = 0; e < 4; ++e) {
       float sum = 0.f;
 #pragma unroll
-      for (int w = 0; w < kAttnWaves; ++w)
-        sum = fmaf(o_s[w][i * 4 + r][lane], wgt[w], sum);
-      o[64 * half + 4 * (4 * lg + r) + wave] = sum * inv;
+      for (int w = 0; w < kAttnWaves; ++w) {
+        const float x = slot_s[w * kSlotFloats + ((2 * e + m_half) * 4 + m_r) * kOutPitch +
+                               16 * m_lg + mq];
+        sum = fmaf(has[w] ? x : 0.f, wgt[w], sum);
+      }
+      o[e] = sum * inv;
     }
+    *reinterpret_cast<f32x4 *>(a.out + (int64_t)(q0[p] + mq) * a.o_stride +
+                               (int64_t)h * a.o_hstride + 4 * c) = o;
   }
 }
 
@@ -300,6 +383,9 @@ int launch_attn_prefill(const AttnPrefillArgs &in, hipStream_t stream) {
                  in.o_hstride >= kD && in.q_stride % 4 == 0 && in.o_stride % 4 == 0 &&
                  in.q_hstride % 4 == 0 && in.o_hstride % 4 == 0,
              "attn_prefill: bad strides");
+  BH_REQUIRE(((reinterpret_cast<uintptr_t>(in.q) | reinterpret_cast<uintptr_t>(in.k) |
+               reinterpret_cast<uintptr_t>(in.v) | reinterpret_cast<uintptr_t>(in.out)) & 15) == 0,
+             "attn_prefill: q, k, v and out must be 16-byte aligned");
   PrefillArgs a;
   a.q = in.q;
   a.k = in.k;
@@ -317,10 +403,15 @@ int launch_attn_prefill(const AttnPrefillArgs &in, hipStream_t stream) {
   a.k_len = in.k_len;
   a.q_offset = in.k_len - in.q_len; // the last query sees every key
   a.scale = in.scale;
-  BH_REQUIRE(ceil_div(in.q_len, kQB) <= 65535, "attn_prefill: q_len %d too long", in.q_len);
+  a.nqb = (int)ceil_div(in.q_len, kQB);
+  const int pairs = (a.nqb + 1) / 2;
+  BH_REQUIRE(pairs <= 65535, "attn_prefill: q_len %d too long", in.q_len);
+  static DynLdsOnce dyn_lds;
+  BH_CHECK_HIP(ensure_dyn_lds(dyn_lds, reinterpret_cast<const void *>(attn_prefill_kernel),
+                              (int)(kLdsFloats * sizeof(float))));
   BH_NOTE_VARIANT(AttnPrefillFamily);
-  hipLaunchKernelGGL(attn_prefill_kernel, dim3(in.heads, (unsigned)ceil_div(in.q_len, kQB)),
-                     dim3(kAttnWaves * kWave), 0, stream, a);
+  hipLaunchKernelGGL(attn_prefill_kernel, dim3(in.heads, (unsigned)pairs),
+                     dim3(kAttnWaves * kWave), kLdsFloats * sizeof(float), stream, a);
   BH_CHECK_HIP(hipGetLastError());
   return BUDDY_HIP_OK;
 }

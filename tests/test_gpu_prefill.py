@@ -283,6 +283,35 @@ def test_prefill_attention_gqa_and_longer_keys(bh, oracle):
     check_close(run_attn(bh, q, k, v, None, H, HKV, Lq, Lk), want)
 
 
+@pytest.mark.parametrize("Lq,Lk", [(1, 1), (5, 5), (17, 17), (33, 33), (95, 95), (129, 129),
+                                   (1, 300), (16, 130), (50, 51), (200, 333)])
+def test_prefill_attention_ragged_lengths(bh, oracle, Lq, Lk):
+    """A workgroup takes a query block and its mirror image, and its wavefronts
+    split the key blocks of the two: one query block alone, an odd number of
+    them (the middle one on its own), a last block of 1 row, fewer key blocks than
+    wavefronts, and prompts that continue behind cached positions -- with the
+    implicit causal mask and with the same mask passed as a tensor."""
+    H, HKV = 4, 2
+    g = torch.Generator(device="cuda").manual_seed(1000 * Lq + Lk)
+    q = torch.randn((H, Lq, 128), generator=g, device="cuda")
+    k = torch.randn((HKV, Lk, 128), generator=g, device="cuda")
+    v = torch.randn((HKV, Lk, 128), generator=g, device="cuda")
+    kk = k.repeat_interleave(H // HKV, dim=0).cpu().numpy()
+    vv = v.repeat_interleave(H // HKV, dim=0).cpu().numpy()
+    qi = np.arange(Lq)[:, None] + (Lk - Lq)
+    mh = np.where(np.arange(Lk)[None, :] <= qi, 0.0, -np.inf).astype(np.float32)
+    want = oracle.prefill_flash_attention(q.cpu().numpy(), kk, vv, mh, SCALE)
+    check_close(run_attn(bh, q, k, v, None, H, HKV, Lq, Lk), want)
+    check_close(run_attn(bh, q, k, v, torch.from_numpy(mh).cuda(), H, HKV, Lq, Lk), want)
+
+
+def test_prefill_attention_refuses_unaligned_operands(bh):
+    t = torch.zeros(4 * 16 * 128 + 4, device="cuda")
+    p = t.data_ptr()
+    rc = bh.buddy_hip_prefill_attention(p + 4, p, p, None, p, 4, 4, 128, 16, 16, float(SCALE), None)
+    assert rc == 1 and b"16-byte aligned" in bh.buddy_hip_last_error()
+
+
 @pytest.mark.parametrize("precision", ["digits", "exact", "bf16", "digits2"])
 def test_small_model_block_prefill_equals_token_by_token(oracle, precision):
     """Prefill of 40 prompt tokens as one block against 40 oracle decode steps:
