@@ -403,7 +403,8 @@ def test_wide_hidden_size_through_the_slice_adding_norm_kernel(oracle):
 def test_qwen2_1p5b_shape_512_token_prefill(oracle):
     """The full 28-layer shape, a prompt of 512 tokens as one block (digit-plane
     matmuls, the default) against 512 oracle decode steps: last-row logits, the
-    greedy token, and the cache rows of the first and the last layer."""
+    greedy token, and the cache rows of the first and the last layer; then the
+    last-row logits of the three other activation modes."""
     shape = Shape()
     sess, host = synthetic.build_session(shape, context=0, keep_host=True)
     om = oracle_model(oracle, shape, host)
@@ -422,6 +423,21 @@ def test_qwen2_1p5b_shape_512_token_prefill(oracle):
     t2, olg = om.decode_step(otok, 512, kv)
     check_close(lg, olg)
     assert n2 == t2
+    # the same prompt in the other activation modes, at the bound each one's
+    # rounding allows over 28 layers: every f32 bit (three bf16 terms) at the f32
+    # bar, two digit planes (2^-15 of a row's maximum per matmul), activations cast
+    # to bf16 (2^-9 per element: the precision BASELINE's prefill case names)
+    _, exact = sess.prefill(toks, 0, precision="exact")
+    check_close(exact, ologits)
+    _, two = sess.prefill(toks, 0, precision="digits2")
+    nw2 = check_close(two, ologits, rtol=2e-2, atol_frac=3e-3, normwise=3e-3)
+    _, cast = sess.prefill(toks, 0, precision="bf16")
+    nwc = check_close(cast, ologits, rtol=5e-2, atol_frac=2e-2, normwise=2e-2)
+    print(f"norm-wise error of the last-row logits: two planes {nw2:.2e}, bf16 cast {nwc:.2e}")
+    assert nw2 < nwc
+    for lg_mode in (exact, two, cast):
+        assert int(np.argmax(lg_mode)) == otok or float(top2[1] - top2[0]) < 0.05 * float(
+            np.abs(ologits).max())
     sess.close()
 
 
