@@ -22,7 +22,6 @@ namespace {
 constexpr int kD = 128;
 constexpr int kQB = 16;            // query rows per block
 constexpr int kKB = 16;            // key positions per step of a wavefront
-constexpr int kAttnWaves = 8;      // wavefronts per workgroup; they split the keys
 constexpr int kKPitch = kD + 4;    // floats per key row in LDS (fragment reads hit every bank once)
 constexpr int kOutPitch = kWave + 1;      // floats per accumulator register row of a partial output in LDS
 constexpr int kSlotFloats = kKB * kKPitch; // a wavefront's part of LDS: a K block, later its partial output
@@ -39,6 +38,7 @@ struct PrefillArgs {
   int64_t q_stride, q_hstride, o_stride, o_hstride, kv_stride;
   int heads, group, q_len, k_len, q_offset; // query i sits at key position q_offset + i
   int nqb;                                  // query blocks of kQB rows
+  int paired;                               // a workgroup takes a query block and its mirror image
   float scale;
 };
 
@@ -46,16 +46,20 @@ struct PrefillArgs {
 // slot per wavefront, the (max, sum) pairs of the partial results and which part
 // each wavefront worked on.
 constexpr int kQFloats = 2 * 8 * kWave * 4;
-constexpr int kLdsFloats = kQFloats + kAttnWaves * kSlotFloats + 2 * kAttnWaves * kQB + kAttnWaves;
+constexpr int lds_floats(int waves) { return kQFloats + waves * kSlotFloats + 2 * waves * kQB + waves; }
 
 // One workgroup: two blocks of 16 query rows of one head, block j from the start
 // and block j from the end, so that under the causal mask every workgroup has the
 // same number of 16-key blocks before it (one query block alone would have
-// between 1 and q_len / 16 of them, and the launch would last as long as the
-// longest).  The eight wavefronts are dealt to the two query blocks in proportion
-// to their key blocks; those of a query block split its key blocks into equal
-// contiguous shares, each with its own running (max, sum, output), and the
-// partial results meet in LDS at the end.
+// between 1 and q_len / 16 of them, and a launch of one round would last as long
+// as the longest).  The W wavefronts are dealt to the two query blocks in
+// proportion to their key blocks; those of a query block split its key blocks
+// into equal contiguous shares, each with its own running (max, sum, output), and
+// the partial results meet in LDS at the end.  W = 8 and pairs while the launch
+// is at most one workgroup per compute unit.  A longer launch balances itself
+// better with many workgroups of unequal length, the longest first: then a
+// workgroup takes one query block (part 0 empty), W = 4, two workgroups per
+// compute unit, so that one's staging and merge overlap the other's key loop.
 // All products run on the f32 matrix cores (16x16x4):
 //   S^T[key, query] = K . Q^T   (contraction over d; in step 4J + e a lane
 //                                supplies d = 16 J + 4 (lane/16) + e, for K and
@@ -64,8 +68,10 @@ constexpr int kLdsFloats = kQFloats + kAttnWaves * kSlotFloats + 2 * kAttnWaves 
 //                                registers ARE the P^T operand of step r: a
 //                                lane holds keys 4*(lane/16) + r of query lane%16)
 // so the scores never leave the registers between the two products.
+template <int kAttnWaves>
 __global__ void __launch_bounds__(kAttnWaves *kWave) __attribute__((amdgpu_waves_per_eu(2, 2)))
 attn_prefill_kernel(PrefillArgs a) {
+  static_assert(kAttnWaves == 4 || kAttnWaves == 8, "wavefronts per workgroup");
   extern __shared__ __attribute__((aligned(16))) float lds[];
   f32x4 *q_s = reinterpret_cast<f32x4 *>(lds);          // [2][8][64]: part, J, lane
   float *slot_s = lds + kQFloats;                  // [kAttnWaves][kSlotFloats]
@@ -79,8 +85,11 @@ attn_prefill_kernel(PrefillArgs a) {
   const int qi = lane & 15, lg = lane >> 4; // query of this lane; lane group
   // part 0: query block blockIdx.y, part 1: its mirror image (the same block in
   // the middle of an odd number of blocks: then part 0 is empty)
+  // (unpaired launches: one query block per workgroup, part 0 stays empty; ids
+  // start in order, so the blocks that see the most keys come first and the
+  // short ones fill the gaps at the end)
   const int qb1 = a.nqb - 1 - (int)blockIdx.y;
-  const bool single = qb1 == (int)blockIdx.y;
+  const bool single = !a.paired || qb1 == (int)blockIdx.y;
   int q0[2], nq[2], nb[2];
 #pragma unroll
   for (int p = 0; p < 2; ++p) {
@@ -145,13 +154,13 @@ attn_prefill_kernel(PrefillArgs a) {
   if (b0 < b1)
     fetch(b0, fa); // on its way while the queries are staged
 
-  { // Q^T fragments into LDS: wavefront w loads J = 2 (w % 4), + 1 of part w / 4
-    const int p = wave >> 2;
-    const int qrow = q0[p] + min(qi, nq[p] - 1); // rows past the end repeat the last
-    const float *src = a.q + (int64_t)qrow * a.q_stride + (int64_t)h * a.q_hstride + lg * 4;
+  { // Q^T fragments into LDS: the 16 (part, J) pieces are dealt to the wavefronts
+    constexpr int kPieces = 16 / kAttnWaves;
 #pragma unroll
-    for (int t = 0; t < 2; ++t) {
-      const int J = 2 * (wave & 3) + t;
+    for (int t = 0; t < kPieces; ++t) {
+      const int piece = wave * kPieces + t, p = piece >> 3, J = piece & 7;
+      const int qrow = q0[p] + min(qi, nq[p] - 1); // rows past the end repeat the last
+      const float *src = a.q + (int64_t)qrow * a.q_stride + (int64_t)h * a.q_hstride + lg * 4;
       q_s[(p * 8 + J) * kWave + lane] = *reinterpret_cast<const f32x4 *>(src + 16 * J);
     }
   }
@@ -288,12 +297,14 @@ attn_prefill_kernel(PrefillArgs a) {
 
   // ---- merge the partial results (the reference's combine rule, in wave order).
   // A thread finishes four consecutive d of one query per part, so that a
-  // wavefront writes two whole rows of the output: value d = 64 half + 16 lg +
+  // wavefront writes two whole rows of the output at a time: value d = 64 half + 16 lg +
   // 4 r + e of query q is accumulator 2 e + half, register r of lane 16 lg + q.
-  const int c = lane & 31, mq = 2 * wave + (lane >> 5);
+  const int c = lane & 31;
   const int m_half = c >> 4, m_lg = (c >> 2) & 3, m_r = c & 3;
 #pragma unroll
-  for (int p = 0; p < 2; ++p) {
+  for (int it = 0; it < 2 * (8 / kAttnWaves); ++it) {
+    const int p = it & 1;
+    const int mq = (2 * wave + (lane >> 5)) * (8 / kAttnWaves) + (it >> 1);
     if ((single && p == 0) || mq >= nq[p])
       continue;
     float wgt[kAttnWaves], m_w[kAttnWaves], m_all = kSeedM, l_all = 0.f;
@@ -406,12 +417,24 @@ int launch_attn_prefill(const AttnPrefillArgs &in, hipStream_t stream) {
   a.nqb = (int)ceil_div(in.q_len, kQB);
   const int pairs = (a.nqb + 1) / 2;
   BH_REQUIRE(pairs <= 65535, "attn_prefill: q_len %d too long", in.q_len);
-  static DynLdsOnce dyn_lds;
-  BH_CHECK_HIP(ensure_dyn_lds(dyn_lds, reinterpret_cast<const void *>(attn_prefill_kernel),
-                              (int)(kLdsFloats * sizeof(float))));
-  BH_NOTE_VARIANT(AttnPrefillFamily);
-  hipLaunchKernelGGL(attn_prefill_kernel, dim3(in.heads, (unsigned)pairs),
-                     dim3(kAttnWaves * kWave), kLdsFloats * sizeof(float), stream, a);
+  constexpr int kComputeUnits = 256; // MI355X
+  a.paired = (int64_t)in.heads * pairs <= kComputeUnits;
+  if (a.paired) {
+    static DynLdsOnce dyn_lds;
+    BH_CHECK_HIP(ensure_dyn_lds(dyn_lds, reinterpret_cast<const void *>(attn_prefill_kernel<8>),
+                                (int)(lds_floats(8) * sizeof(float))));
+    BH_NOTE_VARIANT(AttnPrefillFamily, 8);
+    hipLaunchKernelGGL(attn_prefill_kernel<8>, dim3(in.heads, (unsigned)pairs), dim3(8 * kWave),
+                       lds_floats(8) * sizeof(float), stream, a);
+  } else {
+    BH_REQUIRE(a.nqb <= 65535, "attn_prefill: q_len %d too long", in.q_len);
+    static DynLdsOnce dyn_lds;
+    BH_CHECK_HIP(ensure_dyn_lds(dyn_lds, reinterpret_cast<const void *>(attn_prefill_kernel<4>),
+                                (int)(lds_floats(4) * sizeof(float))));
+    BH_NOTE_VARIANT(AttnPrefillFamily, 4);
+    hipLaunchKernelGGL(attn_prefill_kernel<4>, dim3(in.heads, (unsigned)a.nqb), dim3(4 * kWave),
+                       lds_floats(4) * sizeof(float), stream, a);
+  }
   BH_CHECK_HIP(hipGetLastError());
   return BUDDY_HIP_OK;
 }

@@ -305,6 +305,22 @@ def test_prefill_attention_ragged_lengths(bh, oracle, Lq, Lk):
     check_close(run_attn(bh, q, k, v, torch.from_numpy(mh).cuda(), H, HKV, Lq, Lk), want)
 
 
+@pytest.mark.parametrize("H,HKV,Lq,Lk", [(32, 8, 272, 272), (12, 2, 600, 700)])
+def test_prefill_attention_launches_of_several_rounds(bh, oracle, H, HKV, Lq, Lk):
+    """More workgroups than compute units: the launch takes the form with four
+    wavefronts per workgroup (two workgroups per compute unit)."""
+    g = torch.Generator(device="cuda").manual_seed(H + Lq)
+    q = torch.randn((H, Lq, 128), generator=g, device="cuda")
+    k = torch.randn((HKV, Lk, 128), generator=g, device="cuda")
+    v = torch.randn((HKV, Lk, 128), generator=g, device="cuda")
+    kk = k.repeat_interleave(H // HKV, dim=0).cpu().numpy()
+    vv = v.repeat_interleave(H // HKV, dim=0).cpu().numpy()
+    qi = np.arange(Lq)[:, None] + (Lk - Lq)
+    mh = np.where(np.arange(Lk)[None, :] <= qi, 0.0, -np.inf).astype(np.float32)
+    want = oracle.prefill_flash_attention(q.cpu().numpy(), kk, vv, mh, SCALE)
+    check_close(run_attn(bh, q, k, v, None, H, HKV, Lq, Lk), want)
+
+
 def test_prefill_attention_refuses_unaligned_operands(bh):
     t = torch.zeros(4 * 16 * 128 + 4, device="cuda")
     p = t.data_ptr()

@@ -265,6 +265,17 @@ def test_prefill_attention_and_no_unlisted_family(bh, oracle):
     mask = np.triu(np.full((L, L), -np.inf, np.float32), 1)
     want = oracle.prefill_flash_attention(q.cpu().numpy(), kk, vv, mask, SCALE)
     check_close(got, want)
+    # more workgroups than compute units: four wavefronts per workgroup
+    heads, kv_heads, L = 32, 8, 272
+    q = torch.randn((heads, L, D), generator=g, device="cuda")
+    k = torch.randn((kv_heads, L, D), generator=g, device="cuda")
+    v = torch.randn((kv_heads, L, D), generator=g, device="cuda")
+    got = run_attn(bh, q, k, v, None, heads, kv_heads, L, L)
+    rep = heads // kv_heads
+    mask = np.triu(np.full((L, L), -np.inf, np.float32), 1)
+    want = oracle.prefill_flash_attention(q.cpu().numpy(), np.repeat(k.cpu().numpy(), rep, axis=0),
+                                          np.repeat(v.cpu().numpy(), rep, axis=0), mask, SCALE)
+    check_close(got, want)
     assert launched(bh, "attn_prefill_kernel") == compiled(bh, "attn_prefill_kernel")
     # every family the library lists is one of those this file drives
     known = ("gemv_w8a32_i8_kernel", "gemv_w8a32_mfma_kernel", "gemm_w8_i8_wide_kernel",
