@@ -319,6 +319,7 @@ def test_prefill_attention_launches_of_several_rounds(bh, oracle, H, HKV, Lq, Lk
     mh = np.where(np.arange(Lk)[None, :] <= qi, 0.0, -np.inf).astype(np.float32)
     want = oracle.prefill_flash_attention(q.cpu().numpy(), kk, vv, mh, SCALE)
     check_close(run_attn(bh, q, k, v, None, H, HKV, Lq, Lk), want)
+    check_close(run_attn(bh, q, k, v, torch.from_numpy(mh).cuda(), H, HKV, Lq, Lk), want)
 
 
 def test_prefill_attention_refuses_unaligned_operands(bh):
