@@ -346,6 +346,7 @@ def bench_gemv(bh, args):
     wscale = torch.full((N,), 1e-3, device="cuda")
     ws_bytes = bh.buddy_hip_w8a8_workspace_bytes(1, K)
     ws = torch.empty((ws_bytes,), dtype=torch.int8, device="cuda")
+    stream = torch.cuda.current_stream().cuda_stream
 
     def make_w8a8(stream):
         def w8a8(i):
