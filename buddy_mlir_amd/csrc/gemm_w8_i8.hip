@@ -247,6 +247,7 @@ struct GemmI8Args {
   float *partial;     // [tile][slice][wavefront][row block][16][16 GPW]
   int accumulate;
   int32_t *sums;      // one plane only: the int32 sums themselves, dense [M, N], or null
+  int int_partials;   // one plane, K split: the slices leave their int32 sums as they are
 };
 
 // sum_j 256^j acc_j as f32 (each int32 sum is exact; the conversions round to 24
@@ -603,8 +604,13 @@ __global__ void __launch_bounds__(kSlices *kWave) gemm_w8_i8_wide_kernel(GemmI8A
     for (int rb = 0; rb < RB; ++rb) {
 #pragma unroll
       for (int g = 0; g < GPW; ++g) {
-        const float4 o = make_float4(combine<D>(acc[g][rb], 0), combine<D>(acc[g][rb], 1),
-                                     combine<D>(acc[g][rb], 2), combine<D>(acc[g][rb], 3));
+        float4 o = make_float4(combine<D>(acc[g][rb], 0), combine<D>(acc[g][rb], 1),
+                               combine<D>(acc[g][rb], 2), combine<D>(acc[g][rb], 3));
+        if constexpr (D == 1) {
+          if (a.int_partials) // exact beyond 2^24: the bits travel as they are
+            o = make_float4(__int_as_float(acc[g][rb][0][0]), __int_as_float(acc[g][rb][0][1]),
+                            __int_as_float(acc[g][rb][0][2]), __int_as_float(acc[g][rb][0][3]));
+        }
         *reinterpret_cast<float4 *>(tile + (lane & 15) * kPad + g * 16 + (lane >> 4) * 4) = o;
       }
 #pragma unroll
@@ -791,6 +797,45 @@ reduce_slices_kernel(GemmI8Args a, int rb_per_tile, int gpw) {
     if (n + r < a.N) {
       const float o = (a.bias ? a.bias[n + r] : 0.f) + (v[r] * step) * a.scale[n + r];
       c[r] = a.accumulate ? c[r] + o : o;
+    }
+}
+
+// One plane (the w8a8 matmul): the slices hold int32 sums, added exactly; then
+// C = f32(sum) * (step * scale[n]) in that order (linalg.py:12833-12845), and the
+// sums themselves where the caller asked for them.
+__global__ void __launch_bounds__(256)
+reduce_slices_i32_kernel(GemmI8Args a, int rb_per_tile, int gpw) {
+  const int n4 = (a.N + 3) / 4;
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= (int64_t)a.M * n4)
+    return;
+  const int m = (int)(i / n4), n = (int)(i % n4) * 4;
+  const int span = 16 * gpw;
+  const int rbk = m / (16 * rb_per_tile), rb = (m / 16) % rb_per_tile, row = m % 16;
+  const int col = n / (kSlices * span), wave = (n / span) % kSlices, ch = n % span;
+  const int sub = 16 * span;
+  const size_t slice_stride = (size_t)kSlices * rb_per_tile * sub;
+  const float *p = a.partial + ((size_t)(rbk * a.ncols + col) * a.slices) * slice_stride +
+                   ((size_t)wave * rb_per_tile + rb) * sub + row * span + ch;
+  int v[4] = {0, 0, 0, 0};
+  for (int sl = 0; sl < a.slices; sl += 4) {
+    v4i32 q[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+      q[u] = *reinterpret_cast<const v4i32 *>(p + (size_t)min(sl + u, a.slices - 1) * slice_stride);
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+      if (sl + u < a.slices) {
+        v[0] += q[u][0]; v[1] += q[u][1]; v[2] += q[u][2]; v[3] += q[u][3];
+      }
+  }
+  const float step = a.steps[m];
+#pragma unroll
+  for (int r = 0; r < 4; ++r)
+    if (n + r < a.N) {
+      a.C[(int64_t)m * a.ldc + n + r] = scaled<1>((float)v[r], step, a.scale[n + r]);
+      if (a.sums)
+        a.sums[(int64_t)m * a.N + n + r] = v[r];
     }
 }
 
@@ -1001,6 +1046,7 @@ int launch_gemm_w8_digits_d(const GemmW8Args &in, const void *planes, hipStream_
   a.accumulate = in.accumulate ? 1 : 0;
   a.partial = nullptr;
   a.sums = nullptr;
+  a.int_partials = 0;
   a.slices = 1;
   if (in.silu_pair) {
     // two matrices of N / 2 channels, result SiLU(first) * second: wide tiles of
@@ -1158,9 +1204,9 @@ int launch_gemm_w8_digits(const GemmW8Args &in, const void *planes, hipStream_t 
 
 // The w8a8 matmul for more than 16 rows: `plane` holds the int8 activations as
 // one plane ([rows_padded][cols_padded], zero padded) followed by the row steps,
-// every one of them the per-tensor activation scale.  K stays within one
-// workgroup, so the int32 sums are whole and exact (K <= 2^17: 2^17 * 127 * 128
-// is below 2^31).
+// every one of them the per-tensor activation scale.  The int32 sums are exact
+// whether K stays within one workgroup or is split over several (K <= 2^17:
+// 2^17 * 127 * 128 is below 2^31).
 int launch_gemm_w8a8_plane(const void *plane, const int8_t *W, const float *wscale, float *C,
                            int32_t *sums, int64_t M, int64_t K, int64_t N,
                            hipStream_t stream) {
@@ -1183,27 +1229,59 @@ int launch_gemm_w8a8_plane(const void *plane, const int8_t *W, const float *wsca
   a.accumulate = 0;
   a.partial = nullptr;
   a.sums = sums;
-  a.slices = 1;
-  a.chunks_per_slice = a.chunks;
-  // the same cost model as above, whole K per workgroup only
-  int best_gpw = 0, best_rb = 0;
+  a.int_partials = 0;
+  // the cost model of the digit-plane launch with one plane; K slices leave int32
+  // sums in the workspace (f32 ones would round above 2^24) and a second kernel
+  // adds them exactly
+  int best_gpw = 0, best_rb = 0, best_s = 0;
   double best_cost = 0;
+  const int64_t reduce_wgs = ceil_div(M * ceil_div(N, 4), 256);
   for (int gpw : {5, 4})
     for (int rb : {4, 3}) {
       const int64_t ncols = ceil_div(a.groups, gpw * kSlices), rows = ceil_div(M, 16 * rb);
-      const int64_t per_xcd = ceil_div(ncols, 8) * rows;
-      const double wg = 0.0125 * (double)(a.chunks * gpw * rb) + 7.0;
-      const double cost = (double)ceil_div(per_xcd, 32) * wg;
-      if (!best_gpw || cost < best_cost - 1e-9) {
-        best_gpw = gpw;
-        best_rb = rb;
-        best_cost = cost;
+      for (int s = 1; s <= 16; ++s) {
+        const int64_t per_xcd = ceil_div(ncols * s, 8) * rows;
+        if (s > 1 && per_xcd > 32)
+          break;
+        const int64_t cps = ceil_div(a.chunks, s);
+        if (ceil_div(a.chunks, cps) != s)
+          continue; // the last slice would be empty
+        const double chunk_us = std::max(0.0125 * (double)(gpw * rb), s == 1 ? 0.55 : 0.0);
+        const double wg = chunk_us * (double)cps + 7.0 + (s > 1 ? 2.0 : 0.0);
+        double cost = (double)ceil_div(per_xcd, 32) * wg;
+        if (s > 1)
+          cost += 3.0 + 4.0 * (double)(ncols * rows * s) * (kSlices * rb * 16 * gpw * 16) / 3e6 +
+                  0.002 * (double)reduce_wgs;
+        if (!best_gpw || cost < best_cost - 1e-9) {
+          best_gpw = gpw;
+          best_rb = rb;
+          best_s = s;
+          best_cost = cost;
+        }
       }
     }
   a.ncols = (int)ceil_div(a.groups, best_gpw * kSlices);
-  a.cols_padded = (int)round_up((int64_t)a.ncols, 8);
+  a.cols_padded = (int)round_up((int64_t)a.ncols * best_s, 8);
   const int row_tiles = (int)ceil_div(M, 16 * best_rb);
-  return launch_shape<1>(best_rb, best_gpw, a, (unsigned)(a.cols_padded * row_tiles), stream);
+  a.slices = best_s;
+  a.chunks_per_slice = (int)ceil_div(a.chunks, best_s);
+  if (best_s > 1) {
+    const size_t tile_floats = (size_t)kSlices * best_rb * 16 * best_gpw * 16;
+    const size_t bytes = sizeof(float) * tile_floats * best_s * (size_t)a.ncols * row_tiles;
+    char *ws = nullptr;
+    if (int rc = workspace_for(stream, bytes, &ws))
+      return rc;
+    a.partial = reinterpret_cast<float *>(ws);
+    a.int_partials = 1;
+  }
+  if (int rc = launch_shape<1>(best_rb, best_gpw, a, (unsigned)(a.cols_padded * row_tiles), stream))
+    return rc;
+  if (best_s > 1) {
+    hipLaunchKernelGGL(reduce_slices_i32_kernel, dim3((unsigned)reduce_wgs), dim3(256), 0, stream, a,
+                       best_rb, best_gpw);
+    BH_CHECK_HIP(hipGetLastError());
+  }
+  return BUDDY_HIP_OK;
 }
 
 } // namespace bh

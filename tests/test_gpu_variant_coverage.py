@@ -188,6 +188,8 @@ GEMM_I8_SHAPES = [(144, 256, 16384), (300, 256, 10240), (200, 192, 16384), (512,
 # widest tile wins there; the other tile shapes are reached with K split over
 # workgroups
 GEMM_I8_SPLIT_K_SHAPES = [(17, 1536, 256), (100, 4096, 8192), (100, 4096, 12288)]
+# one plane (w8a8): the same, the K slices leaving int32 sums
+W8A8_SPLIT_K_SHAPES = [(17, 1536, 256), (100, 4096, 12288), (300, 4096, 5120)]
 GEMM_BF16_SHAPES = [(512, 64, 8960), (300, 64, 10240), (17, 64, 64)]
 
 
@@ -235,6 +237,8 @@ def test_every_int8_prefill_matmul_variant(bh, oracle):
     for M, K, N in GEMM_I8_SPLIT_K_SHAPES:
         gemm_case(oracle, M, K, N, "digits")
         gemm_case(oracle, M, K, N, "digits2")
+    for M, K, N in W8A8_SPLIT_K_SHAPES:
+        w8a8_case(bh, oracle, M, K, N)
     for M, K, N in SILU_PAIR_SHAPES[1:5]:  # the paired variants
         silu_pair_case(oracle, M, K, N)
         silu_pair_case(oracle, M, K, N, digits=2)
