@@ -5,7 +5,21 @@
 
 namespace bh {
 
-constexpr int kAttnChunk = 64; // cache positions per flash-decoding partial
+constexpr int kAttnChunk = 64; // cache positions per flash-decoding partial (the default)
+// A decode step far into a long cache takes larger chunks (128 or 256 positions,
+// 8 or 16 wavefronts of 16 positions per workgroup): the consumer that folds the
+// partials reads one per chunk, and beyond ~18 of them that fold, not the scan of
+// the cache, is what the step waits for.
+inline int attn_chunk_for_position(int pos) {
+  return pos < 18 * 64 ? 64 : pos < 18 * 128 ? 128 : 256;
+}
+// Chunks a step at `pos` launches and folds: those up to the position, in
+// batches of 18 (what the fold requests at once), never more than the cache has.
+inline int attn_chunks_for_position(int pos, int chunk, int max_len) {
+  const int all = (max_len + chunk - 1) / chunk, need = pos / chunk + 1;
+  const int batches = (need + 17) / 18;
+  return batches * 18 < all ? batches * 18 : all;
+}
 constexpr int kAttnHeadDim = 128; // the head size the decode kernel is written for
 
 struct AttnDecodeArgs {
@@ -24,6 +38,10 @@ struct AttnDecodeArgs {
   void *workspace = nullptr; // flash-decoding partials
   size_t workspace_bytes = 0;
   bool combine = true; // false: leave the partials for the consumer to fold
+  int chunk = kAttnChunk; // cache positions per partial: 64, 128 or 256
+  // partials to produce (the first ones; the caller knows the position lies in
+  // them); 0: one for every chunk of the cache
+  int chunks_used = 0;
 };
 
 // Where the partials live inside the workspace.
@@ -32,7 +50,8 @@ struct AttnPartials {
   float *ml;  // [heads, nchunks, 2] = (max, sum)
   int nchunks;
 };
-AttnPartials attn_partials(void *workspace, int heads, int head_dim, int max_len);
+AttnPartials attn_partials(void *workspace, int heads, int head_dim, int max_len,
+                           int chunk = kAttnChunk);
 
 struct AttnPrefillArgs {
   const float *q = nullptr;   // token t, head h at q + t*q_stride + h*q_hstride

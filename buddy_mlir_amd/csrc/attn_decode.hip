@@ -30,8 +30,7 @@ namespace bh {
 namespace {
 
 
-constexpr int kChunk = kAttnChunk; // cache positions per workgroup
-constexpr int kThreads = 256;
+constexpr int kPW = 16;           // cache positions per wavefront
 constexpr int kMaxGroup = 8;     // query heads per KV head
 constexpr int kD = kAttnHeadDim; // head_dim this kernel is written for
 constexpr float kSeedM = -1.0e30f; // tosa.py:13971
@@ -46,12 +45,13 @@ struct AttnArgs {
   float *part_ml;        // [heads, nchunks, 2]
   float *out;            // [heads*D]
   float *lse;            // [heads] or null: m + log l of the whole softmax
-  int heads, kv_heads, group, max_len, nchunks;
+  int heads, kv_heads, group, max_len, nchunks, chunk;
+  int used; // chunks this launch covers (the first ones of nchunks)
   float scale;
   int pairs_padded; // (chunk, kv head) pairs rounded up to the XCD count
 };
 
-// One workgroup: 64 cache positions x one query head.  The workgroups that
+// One workgroup: 16 kWaves cache positions (64 by default) x one query head.  The workgroups that
 // share a chunk (the query heads of one KV head: same K/V rows) get linear ids
 // that are equal modulo 8, so they run on the same XCD and the rows come out of
 // that XCD's L2 after the first of them has fetched them.
@@ -60,12 +60,12 @@ struct AttnArgs {
 // behind the arrival of its K/V rows: the small operands (q, the token's own
 // k and v, the RoPE table) are requested first, the K/V rows right behind
 // them, and q is rotated into LDS while the rows are still on their way -- the
-// one barrier before the merge.  Each of the four wavefronts then handles 16
+// one barrier before the merge.  Each of the wavefronts then handles 16
 // positions entirely on its own (scores, its own max / exp / sum, its share of
-// P.V) in registers and cross-lane operations, and the four meet once in LDS.
-__global__ void __launch_bounds__(kThreads) attn_decode_partial(AttnArgs a) {
-  constexpr int kWaves = kThreads / 64;
-  constexpr int kPW = kChunk / kWaves; // positions per wavefront: 16
+// P.V) in registers and cross-lane operations, and they meet once in LDS.
+template <int kWaves>
+__global__ void __launch_bounds__(kWaves * 64) attn_decode_partial(AttnArgs a) {
+  constexpr int kChunk = kWaves * kPW; // cache positions per workgroup: 64, 128 or 256
   constexpr int kR = kPW / 2;          // rows per lane: 8
   __shared__ __attribute__((aligned(16))) float q_s[kD], knew_s[kD], vnew_s[kD];
   __shared__ __attribute__((aligned(16))) float accw_s[kWaves][kD];
@@ -74,9 +74,9 @@ __global__ void __launch_bounds__(kThreads) attn_decode_partial(AttnArgs a) {
   const int tid = threadIdx.x;
   const int wave = tid >> 6, lane = tid & 63;
   const int hb = blockIdx.x / a.pairs_padded, ckv = blockIdx.x % a.pairs_padded;
-  if (ckv >= a.nchunks * a.kv_heads)
+  if (ckv >= a.used * a.kv_heads)
     return; // padding id
-  const int chunk = ckv % a.nchunks, kvh = ckv / a.nchunks;
+  const int chunk = ckv % a.used, kvh = ckv / a.used;
   const int p0 = chunk * kChunk;
   const int h = kvh * a.group + hb; // this workgroup's query head
 
@@ -213,7 +213,7 @@ __global__ void __launch_bounds__(kThreads) attn_decode_partial(AttnArgs a) {
   }
   __syncthreads();
 
-  // ---- the four wavefronts meet: one partial per (head, chunk) --------------
+  // ---- the wavefronts meet: one partial per (head, chunk) -------------------
   if (tid < kD) {
     float m = mw_s[0];
 #pragma unroll
@@ -240,7 +240,7 @@ __global__ void __launch_bounds__(kThreads) attn_decode_partial(AttnArgs a) {
 __global__ void __launch_bounds__(kD) attn_decode_combine(AttnArgs a) {
   const int h = blockIdx.x, d = threadIdx.x;
   const int pos = min(max(*a.pos_ptr, 0), a.max_len - 1);
-  const int used = min(a.nchunks, pos / kChunk + 1);
+  const int used = min(a.nchunks, pos / a.chunk + 1);
   float m_run = kSeedM, l_run = 0.f, acc = 0.f;
   for (int s = 0; s < used; ++s) {
     const float m_c = a.part_ml[((size_t)h * a.nchunks + s) * 2 + 0];
@@ -302,13 +302,13 @@ int static_scratch(float **out, hipStream_t stream) {
 } // namespace
 
 size_t attn_decode_workspace_bytes(int heads, int max_len) {
-  const int nchunks = (int)ceil_div(max_len, kChunk);
+  const int nchunks = (int)ceil_div(max_len, kAttnChunk); // the smallest chunk: the most partials
   return sizeof(float) * (size_t)heads * nchunks * (kD + 2);
 }
 
-AttnPartials attn_partials(void *workspace, int heads, int head_dim, int max_len) {
+AttnPartials attn_partials(void *workspace, int heads, int head_dim, int max_len, int chunk) {
   AttnPartials p;
-  p.nchunks = (int)ceil_div(max_len, kChunk);
+  p.nchunks = (int)ceil_div(max_len, chunk);
   p.acc = static_cast<float *>(workspace);
   p.ml = p.acc + (size_t)heads * p.nchunks * head_dim;
   return p;
@@ -342,16 +342,27 @@ int launch_attn_decode(const AttnDecodeArgs &in, hipStream_t stream) {
   a.kv_heads = in.kv_heads;
   a.group = in.heads / in.kv_heads;
   a.max_len = in.max_len;
-  a.nchunks = (int)ceil_div(in.max_len, kChunk);
+  BH_REQUIRE(in.chunk == 64 || in.chunk == 128 || in.chunk == 256, "attn_decode: chunk %d",
+             in.chunk);
+  a.chunk = in.chunk;
+  a.nchunks = (int)ceil_div(in.max_len, in.chunk);
   a.scale = in.scale;
-  const AttnPartials parts = attn_partials(in.workspace, in.heads, kD, in.max_len);
+  const AttnPartials parts = attn_partials(in.workspace, in.heads, kD, in.max_len, in.chunk);
   a.part_acc = parts.acc;
   a.part_ml = parts.ml;
   a.out = in.out;
   a.lse = in.lse;
-  a.pairs_padded = (int)round_up((int64_t)a.nchunks * in.kv_heads, 8);
-  hipLaunchKernelGGL(attn_decode_partial, dim3(a.pairs_padded * a.group),
-                     dim3(kThreads), 0, stream, a);
+  a.used = in.chunks_used > 0 ? std::min(in.chunks_used, a.nchunks) : a.nchunks;
+  BH_REQUIRE(!in.combine || a.used == a.nchunks,
+             "attn_decode: the combine pass needs a partial for every chunk");
+  a.pairs_padded = (int)round_up((int64_t)a.used * in.kv_heads, 8);
+  const dim3 grid(a.pairs_padded * a.group);
+  if (in.chunk == 64)
+    hipLaunchKernelGGL(attn_decode_partial<4>, grid, dim3(4 * 64), 0, stream, a);
+  else if (in.chunk == 128)
+    hipLaunchKernelGGL(attn_decode_partial<8>, grid, dim3(8 * 64), 0, stream, a);
+  else
+    hipLaunchKernelGGL(attn_decode_partial<16>, grid, dim3(16 * 64), 0, stream, a);
   if (in.combine)
     hipLaunchKernelGGL(attn_decode_combine, dim3(in.heads), dim3(kD), 0, stream, a);
   BH_CHECK_HIP(hipGetLastError());

@@ -33,6 +33,7 @@ struct GemvArgs {
   const float *attn_acc = nullptr, *attn_ml = nullptr;
   const int *pos_ptr = nullptr;
   int attn_nchunks = 0, attn_chunk = 0, head_dim = 0;
+  int attn_used = 0; // chunks to fold (the first ones); 0: all attn_nchunks
   int tile_n = 16; // channels per packed tile: 16 (default), 8 or 4
   // One row with the STORE epilogue, optional: the first maximum of every
   // channel group's 16 results, (value, index) at [group] of these two arrays

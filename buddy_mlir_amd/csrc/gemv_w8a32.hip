@@ -135,7 +135,7 @@ struct KernelArgs {
   // activation provider 2: fold flash-decoding partials while staging
   const float *attn_acc, *attn_ml;
   const int *pos_ptr;
-  int attn_nchunks, attn_chunk, head_dim;
+  int attn_nchunks, attn_chunk, head_dim, attn_used;
   // one row, STORE: per channel group the first maximum of its results, or null
   float *cand_v;
   int *cand_i;
@@ -249,10 +249,10 @@ __device__ __forceinline__ void emit_group_maximum(const KernelArgs &a, int g, i
 __device__ __forceinline__ float4 attn_combined(const KernelArgs &a, int k) {
   constexpr int B = 9; // partials fetched per batch (two batches at 18 chunks)
   const int h = k / a.head_dim, d = k % a.head_dim;
-  // every chunk is folded: the ones beyond the position hold (m, l, acc) =
-  // (-1e30, 0, 0) and drop out with weight exp(-1e30 - m) = 0, so the loop does
-  // not have to wait for the position
-  const int used = a.attn_nchunks;
+  // every chunk the launch was given is folded: the ones beyond the position
+  // hold (m, l, acc) = (-1e30, 0, 0) and drop out with weight exp(-1e30 - m) = 0,
+  // so the loop does not have to wait for the position
+  const int used = a.attn_used;
   const float2 *ml = reinterpret_cast<const float2 *>(a.attn_ml) +
                      (size_t)h * a.attn_nchunks;
   const float *acc = a.attn_acc + (size_t)h * a.attn_nchunks * a.head_dim + d;
@@ -622,7 +622,7 @@ template <int U>
 __device__ __forceinline__ void attn_fold_tiles(const KernelArgs &a, int t0, int t1,
                                                 int lane, float (&x)[U]) {
   constexpr int B = 18;
-  const int used = a.attn_nchunks;
+  const int used = a.attn_used;
   const float2 *ml[U];
   const float *acc[U];
   float r[U], m[U], l[U];
@@ -1634,6 +1634,7 @@ int launch_gemv(const GemvArgs &a, hipStream_t stream) {
   ka.pos_ptr = a.pos_ptr;
   ka.attn_nchunks = a.attn_nchunks;
   ka.attn_chunk = a.attn_chunk;
+  ka.attn_used = a.attn_used > 0 ? std::min(a.attn_used, a.attn_nchunks) : a.attn_nchunks;
   ka.head_dim = a.head_dim;
   switch (mt) {
   case 1: return launch_m<1>(a, ka, p, stream);

@@ -27,6 +27,7 @@
 #include <cmath>
 #include <cstring>
 #include <new>
+#include <map>
 #include <vector>
 
 namespace bh {
@@ -110,8 +111,14 @@ struct Session {
   // step will use.  -1 until set_state; every step advances both on the device,
   // so the host can refuse steps that would leave the cache or the token log.
   int next_pos = -1, next_step = 0;
-  hipGraph_t graph = nullptr;
-  hipGraphExec_t graph_exec = nullptr;
+  // One captured step per (attention chunk size, chunks covered): the host knows
+  // the position of the step it launches and picks the graph.  A cache of up to
+  // 1152 positions only ever has one.
+  struct StepGraph {
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t exec = nullptr;
+  };
+  std::map<std::pair<int, int>, StepGraph> graphs;
   bool use_graph = true;
   std::vector<void *> owned;
   // prefill activations, grown on demand: rows = tokens per prefill call
@@ -162,12 +169,13 @@ struct Session {
   }
 
   void drop_graph() {
-    if (graph_exec)
-      (void)hipGraphExecDestroy(graph_exec);
-    if (graph)
-      (void)hipGraphDestroy(graph);
-    graph_exec = nullptr;
-    graph = nullptr;
+    for (auto &kv : graphs) {
+      if (kv.second.exec)
+        (void)hipGraphExecDestroy(kv.second.exec);
+      if (kv.second.graph)
+        (void)hipGraphDestroy(kv.second.graph);
+    }
+    graphs.clear();
   }
 
   int gemv(const float *A, const PackedLinear &W0, const PackedLinear *W1,
@@ -194,8 +202,10 @@ struct Session {
     return launch_gemv(g, stream);
   }
 
-  // Enqueues one decode step (reads token/pos from device state).
-  int enqueue_step() {
+  // Enqueues one decode step (reads token/pos from device state); attn_chunk:
+  // cache positions per attention partial, attn_used: partials covered, both
+  // chosen by the host from the position.
+  int enqueue_step(int attn_chunk, int attn_used) {
     // x and the RoPE table were prepared by the previous step's last kernel (or
     // by prepare_step after the host set token and position)
     const auto &S = shape;
@@ -226,16 +236,19 @@ struct Session {
       a.workspace = attn_ws;
       a.workspace_bytes = attn_ws_bytes;
       a.combine = false; // o_proj folds the partials while staging its input
+      a.chunk = attn_chunk;
+      a.chunks_used = attn_used;
       if ((rc = launch_attn_decode(a, stream)))
         return rc;
       {
         const AttnPartials parts =
-            attn_partials(attn_ws, S.heads, S.head_dim, S.max_len);
+            attn_partials(attn_ws, S.heads, S.head_dim, S.max_len, attn_chunk);
         GemvArgs g;
         g.attn_acc = parts.acc;
         g.attn_ml = parts.ml;
         g.attn_nchunks = parts.nchunks;
-        g.attn_chunk = kAttnChunk;
+        g.attn_chunk = attn_chunk;
+        g.attn_used = attn_used;
         g.head_dim = S.head_dim;
         g.pos_ptr = state + 1;
         g.W0 = L.o.w;
@@ -544,24 +557,26 @@ struct Session {
     int rc = check_steps(1, "decode step");
     if (rc)
       return rc;
+    const int attn_chunk = attn_chunk_for_position(next_pos);
+    const int attn_used = attn_chunks_for_position(next_pos, attn_chunk, shape.max_len);
     if (!use_graph) {
-      rc = enqueue_step();
+      rc = enqueue_step(attn_chunk, attn_used);
     } else {
-      if (!graph_exec) {
+      StepGraph &g = graphs[{attn_chunk, attn_used}];
+      if (!g.exec) {
         BH_CHECK_HIP(hipStreamBeginCapture(stream, hipStreamCaptureModeThreadLocal));
-        rc = enqueue_step();
-        hipError_t e = hipStreamEndCapture(stream, &graph);
+        rc = enqueue_step(attn_chunk, attn_used);
+        hipError_t e = hipStreamEndCapture(stream, &g.graph);
         if (!rc && e != hipSuccess)
           rc = fail(BUDDY_HIP_ERR_HIP, "hipStreamEndCapture: %s", hipGetErrorString(e));
-        if (!rc && (e = hipGraphInstantiate(&graph_exec, graph, nullptr, nullptr, 0)) !=
-                       hipSuccess)
+        if (!rc && (e = hipGraphInstantiate(&g.exec, g.graph, nullptr, nullptr, 0)) != hipSuccess)
           rc = fail(BUDDY_HIP_ERR_HIP, "hipGraphInstantiate: %s", hipGetErrorString(e));
         if (rc) {
           drop_graph(); // a half-built graph is not kept
           return rc;
         }
       }
-      BH_CHECK_HIP(hipGraphLaunch(graph_exec, stream));
+      BH_CHECK_HIP(hipGraphLaunch(g.exec, stream));
     }
     if (!rc) {
       ++next_pos;
@@ -574,7 +589,7 @@ struct Session {
   // pointers): whoever may change one of them drops the graph first, and the
   // next step captures a new one.
   int invalidate_graph() {
-    if (graph_exec || graph) {
+    if (!graphs.empty()) {
       BH_CHECK_HIP(hipStreamSynchronize(stream));
       drop_graph();
     }

@@ -392,6 +392,37 @@ def test_small_model_decodes_at_long_context(oracle):
     sess.close()
 
 
+@pytest.mark.parametrize("start", [100, 1140, 2296])
+def test_small_model_steps_across_the_attention_chunk_sizes(oracle, start):
+    """A step far into a long cache takes attention chunks of 128 or 256 positions
+    (from positions 1152 and 2304 on) and covers only the chunks up to its
+    position: greedy steps that cross each boundary, and a short context in a
+    large cache, against the oracle -- every step's logits and the token fed back
+    on the device."""
+    shape = Shape(layers=2, hidden=256, heads=4, kv_heads=2, head_dim=128, inter=512,
+                  vocab=1024, max_len=4352, rms_eps=1e-6)
+    sess, host = synthetic.build_session(shape, context=start, keep_host=True, ln_jitter=0.1)
+    om = oracle_model(oracle, shape, host)
+    kv = [a.copy() for a in host["kv"]]
+    tok = 7
+    for step in range(20):
+        nxt, logits = sess.decode(tok, start + step)
+        otok, ologits = om.decode_step(tok, start + step, kv)
+        check_close(logits, ologits)
+        assert nxt == otok
+        tok = otok
+    # the same stretch again as one call (the cache rows are rewritten with the
+    # same values)
+    toks = sess.decode_greedy(7, start, 20)
+    kv2 = [a.copy() for a in host["kv"]]
+    t, want = 7, []
+    for step in range(20):
+        t, _ = om.decode_step(t, start + step, kv2)
+        want.append(t)
+    assert toks.tolist() == want
+    sess.close()
+
+
 def test_small_model_greedy_feedback_matches_stepwise(oracle):
     sess, host = synthetic.build_session(SMALL, context=16, keep_host=True, ln_jitter=0.1)
     toks = sess.decode_greedy(5, 16, 24)
