@@ -6,19 +6,36 @@
 namespace bh {
 
 constexpr int kAttnChunk = 64; // cache positions per flash-decoding partial (the default)
-// A decode step far into a long cache takes larger chunks (128 or 256 positions,
-// 8 or 16 wavefronts of 16 positions per workgroup): the consumer that folds the
-// partials reads one per chunk, and beyond ~18 of them that fold, not the scan of
-// the cache, is what the step waits for.
-inline int attn_chunk_for_position(int pos) {
-  return pos < 18 * 64 ? 64 : pos < 18 * 128 ? 128 : 256;
-}
-// Chunks a step at `pos` launches and folds: those up to the position, in
-// batches of 18 (what the fold requests at once), never more than the cache has.
-inline int attn_chunks_for_position(int pos, int chunk, int max_len) {
-  const int all = (max_len + chunk - 1) / chunk, need = pos / chunk + 1;
+// How a decode step at position `pos` cuts its attention.  Up to 18 partials per
+// head the o_proj launch folds them in one trip to memory: chunks of 64 positions
+// up to position 1152, 128 up to 2304, 256 up to 4608 (8 or 16 wavefronts of 16
+// positions per workgroup).  Beyond that the partials are folded by a launch of
+// their own and one workgroup takes all the query heads of a KV head (a K/V row
+// then leaves L2 once, not once per head); its chunks are the largest that still
+// give the launch about 200 workgroups.  Attention and fold cover only the
+// chunks up to the position, in batches of 18, whatever the cache's capacity.
+struct AttnStepPlan {
+  int chunk;     // cache positions per partial: 64, 128 or 256
+  int used;      // partials per head the step produces and folds
+  bool own_fold; // a launch of its own folds them; workgroups take whole head groups
+};
+inline AttnStepPlan attn_step_plan(int pos, int max_len, int kv_heads) {
+  AttnStepPlan p;
+  p.own_fold = pos >= 18 * 256;
+  if (!p.own_fold) {
+    p.chunk = pos < 18 * 64 ? 64 : pos < 18 * 128 ? 128 : 256;
+  } else {
+    p.chunk = 64;
+    for (int c : {256, 128})
+      if ((pos / c + 1) * kv_heads >= 192) {
+        p.chunk = c;
+        break;
+      }
+  }
+  const int all = (max_len + p.chunk - 1) / p.chunk, need = pos / p.chunk + 1;
   const int batches = (need + 17) / 18;
-  return batches * 18 < all ? batches * 18 : all;
+  p.used = batches * 18 < all ? batches * 18 : all;
+  return p;
 }
 constexpr int kAttnHeadDim = 128; // the head size the decode kernel is written for
 
@@ -38,6 +55,10 @@ struct AttnDecodeArgs {
   void *workspace = nullptr; // flash-decoding partials
   size_t workspace_bytes = 0;
   bool combine = true; // false: leave the partials for the consumer to fold
+  // with combine: the form for a step far into a long cache -- one workgroup
+  // per (chunk, KV head) for all its query heads, then a fold with all partials
+  // in flight instead of chunk by chunk (covers chunks_used partials, no lse)
+  bool wide_combine = false;
   int chunk = kAttnChunk; // cache positions per partial: 64, 128 or 256
   // partials to produce (the first ones; the caller knows the position lies in
   // them); 0: one for every chunk of the cache

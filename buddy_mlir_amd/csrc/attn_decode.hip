@@ -234,6 +234,164 @@ __global__ void __launch_bounds__(kWaves * 64) attn_decode_partial(AttnArgs a) {
   }
 }
 
+// The same for a step far into a long cache, where the rows of a chunk coming
+// out of L2 once per query head (six times for this model) is what the launch
+// waits for: one workgroup takes all the query heads of a KV head, so that a K/V
+// row is loaded once and multiplied with every head's query.
+template <int kWaves>
+__global__ void __launch_bounds__(kWaves * 64) attn_decode_partial_group(AttnArgs a) {
+  constexpr int kChunk = kWaves * kPW;
+  constexpr int kR = kPW / 2;
+  __shared__ __attribute__((aligned(16))) float q_s[kMaxGroup][kD], knew_s[kD], vnew_s[kD];
+  // what the wavefronts leave for the merge, every head of the group at once
+  extern __shared__ __attribute__((aligned(16))) float accw_s[]; // [group][kWaves][kD]
+  __shared__ float mw_s[kMaxGroup][kWaves], lw_s[kMaxGroup][kWaves];
+
+  const int tid = threadIdx.x;
+  const int wave = tid >> 6, lane = tid & 63;
+  const int ckv = blockIdx.x;
+  if (ckv >= a.used * a.kv_heads)
+    return; // padding id
+  const int chunk = ckv % a.used, kvh = ckv / a.used;
+  const int p0 = chunk * kChunk;
+  const int c4 = lane & 31, par = lane >> 5;
+  const int pw0 = p0 + wave * kPW;
+  float4 kreg[kR], vreg[kR];
+#pragma unroll
+  for (int i = 0; i < kR; ++i) {
+    const int row = min(pw0 + par + 2 * i, a.max_len - 1);
+    kreg[i] = *reinterpret_cast<const float4 *>(
+        a.kcache + ((size_t)kvh * a.max_len + row) * kD + c4 * 4);
+  }
+#pragma unroll
+  for (int i = 0; i < kR; ++i) {
+    const int row = min(pw0 + par + 2 * i, a.max_len - 1);
+    vreg[i] = *reinterpret_cast<const float4 *>(
+        a.vcache + ((size_t)kvh * a.max_len + row) * kD + c4 * 4);
+  }
+  const int pos_raw = *a.pos_ptr;
+  const bool pos_ok = pos_raw >= 0 && pos_raw < a.max_len;
+  const int pos = min(max(pos_raw, 0), a.max_len - 1);
+  if (p0 > pos) { // nothing visible in this chunk: empty partials
+    for (int i = tid; i < a.group * kD; i += kWaves * 64) {
+      const int h = kvh * a.group + i / kD;
+      a.part_acc[((size_t)h * a.nchunks + chunk) * kD + i % kD] = 0.f;
+    }
+    if (tid < a.group) {
+      const int h = kvh * a.group + tid;
+      a.part_ml[((size_t)h * a.nchunks + chunk) * 2 + 0] = kSeedM;
+      a.part_ml[((size_t)h * a.nchunks + chunk) * 2 + 1] = 0.f;
+    }
+    return;
+  }
+  const bool has_new = pos < p0 + kChunk;
+  // ---- RoPE of every query of the group and of the token's key --------------
+  for (int i = tid; i < (a.group + 1) * kD; i += kWaves * 64) {
+    const int hh = i / kD, j = i % kD, jj = j & (kD / 2 - 1);
+    float cs, sn;
+    if (a.rope_table) {
+      cs = a.rope_table[jj];
+      sn = a.rope_table[kD / 2 + jj];
+    } else {
+      sincosf(a.inv_freq[jj] * (float)pos, &sn, &cs);
+    }
+    // the queries of the group, then (hh == group) the token's own key
+    const float *src = hh < a.group ? a.qkv + (size_t)(kvh * a.group + hh) * kD
+                                    : a.qkv + (size_t)a.heads * kD + (size_t)kvh * kD;
+    const float raw = src[j];
+    const float pair = j < kD / 2 ? -src[j + kD / 2] : src[j - kD / 2];
+    const float rot = raw * cs + pair * sn;
+    if (hh < a.group) {
+      q_s[hh][j] = rot;
+    } else if (has_new) {
+      const float vraw = src[(size_t)a.kv_heads * kD + j];
+      knew_s[j] = rot;
+      vnew_s[j] = vraw;
+      if (pos_ok) {
+        a.kcache[((size_t)kvh * a.max_len + pos) * kD + j] = rot;
+        a.vcache[((size_t)kvh * a.max_len + pos) * kD + j] = vraw;
+      }
+    }
+  }
+  __syncthreads();
+  // the token's own rows replace what the cache holds at its position
+#pragma unroll
+  for (int i = 0; i < kR; ++i)
+    if (pw0 + par + 2 * i == pos) {
+      kreg[i] = *reinterpret_cast<const float4 *>(knew_s + c4 * 4);
+      vreg[i] = *reinterpret_cast<const float4 *>(vnew_s + c4 * 4);
+    }
+  for (int hh = 0; hh < a.group; ++hh) {
+    const int h = kvh * a.group + hh;
+    const float4 q4 = *reinterpret_cast<const float4 *>(q_s[hh] + c4 * 4);
+    float sc[kR];
+#pragma unroll
+    for (int i = 0; i < kR; ++i) {
+      const int p = pw0 + par + 2 * i;
+      const float4 k4 = kreg[i];
+      float d = fmaf(q4.x, k4.x, fmaf(q4.y, k4.y, fmaf(q4.z, k4.z, q4.w * k4.w)));
+      d = row16_sum(d);
+      d += __shfl_xor(d, 16, 64);
+      sc[i] = p <= pos ? d * a.scale : -INFINITY;
+    }
+    float m_w = kSeedM;
+#pragma unroll
+    for (int i = 0; i < kR; ++i)
+      m_w = fmaxf(m_w, sc[i]);
+    m_w = fmaxf(m_w, __shfl_xor(m_w, 32, 64));
+    float l_w = 0.f;
+#pragma unroll
+    for (int i = 0; i < kR; ++i) {
+      sc[i] = fast_exp(sc[i] - m_w);
+      l_w += sc[i];
+    }
+    l_w += __shfl_xor(l_w, 32, 64);
+    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+    for (int i = 0; i < kR; ++i) {
+      const int p = pw0 + par + 2 * i;
+      const float4 v = vreg[i];
+      if (p <= pos) { // rows beyond the position may hold anything
+        acc.x = fmaf(v.x, sc[i], acc.x);
+        acc.y = fmaf(v.y, sc[i], acc.y);
+        acc.z = fmaf(v.z, sc[i], acc.z);
+        acc.w = fmaf(v.w, sc[i], acc.w);
+      }
+    }
+    acc.x += __shfl_xor(acc.x, 32, 64);
+    acc.y += __shfl_xor(acc.y, 32, 64);
+    acc.z += __shfl_xor(acc.z, 32, 64);
+    acc.w += __shfl_xor(acc.w, 32, 64);
+    if (lane < 32)
+      *reinterpret_cast<float4 *>(&accw_s[((size_t)hh * kWaves + wave) * kD + c4 * 4]) = acc;
+    if (lane == 0) {
+      mw_s[hh][wave] = m_w;
+      lw_s[hh][wave] = l_w;
+    }
+  }
+  __syncthreads();
+  // ---- the wavefronts meet, once for all heads: one partial per (head, chunk) --
+  for (int i = tid; i < a.group * kD; i += kWaves * 64) {
+    const int hh = i / kD, d = i % kD, h = kvh * a.group + hh;
+    float m = mw_s[hh][0];
+#pragma unroll
+    for (int w = 1; w < kWaves; ++w)
+      m = fmaxf(m, mw_s[hh][w]);
+    float o = 0.f, l = 0.f;
+#pragma unroll
+    for (int w = 0; w < kWaves; ++w) {
+      const float f = fast_exp(mw_s[hh][w] - m);
+      o = fmaf(accw_s[((size_t)hh * kWaves + w) * kD + d], f, o);
+      l = fmaf(lw_s[hh][w], f, l);
+    }
+    a.part_acc[((size_t)h * a.nchunks + chunk) * kD + d] = o;
+    if (d == 0) {
+      a.part_ml[((size_t)h * a.nchunks + chunk) * 2 + 0] = m;
+      a.part_ml[((size_t)h * a.nchunks + chunk) * 2 + 1] = l;
+    }
+  }
+}
+
 // Folds the partials of one head in chunk order with the reference's combine
 // (tosa.py:14485-14568): m_new = max(m_run, m_s); a = exp(m_run - m_new);
 // b = exp(m_s - m_new); l = l*a + l_s*b; acc = acc_s*b + acc*a; out = acc / l.
@@ -256,6 +414,75 @@ __global__ void __launch_bounds__(kD) attn_decode_combine(AttnArgs a) {
   a.out[(size_t)h * kD + d] = acc / l_run;
   if (a.lse && d == 0) // tosa.py:14576-14580
     a.lse[h] = m_run + logf(l_run);
+}
+
+// The same fold for a step far into a long cache, where one partial after the
+// other would take a trip to memory each: a workgroup of 32 x 32 threads per head,
+// thread (q, g) gathers d = 4 q .. 4 q + 3 of the chunks s = g, g + 32, ... with
+// every load in flight at once, every wavefront works out the common maximum and
+// the weights exp(m_s - max m) for itself, and the 32 groups meet in LDS.  The
+// sums are those of the chunk-by-chunk rule in another order.
+constexpr int kWideChunks = 1024; // partials per head it takes (256 k positions at 256 per chunk)
+
+__global__ void __launch_bounds__(1024) attn_decode_combine_wide(AttnArgs a) {
+  constexpr int kPer = kWideChunks / 32; // chunks per thread at most
+  __shared__ float w_s[kWideChunks];
+  __shared__ __attribute__((aligned(16))) float4 red_s[32][32];
+  const int h = blockIdx.x, tid = threadIdx.x, lane = tid & 63;
+  const int q = tid & 31, g = tid >> 5;
+  const int used = a.used;
+  const float2 *ml = reinterpret_cast<const float2 *>(a.part_ml) + (size_t)h * a.nchunks;
+  const float *acc = a.part_acc + (size_t)h * a.nchunks * kD + q * 4;
+  // the partial sums of this thread's chunks, requested before anything is known
+  // of their weights (chunks past the last repeat it and are not added)
+  float4 v[4];
+  float4 sum = make_float4(0.f, 0.f, 0.f, 0.f);
+  // the weights: every wavefront computes all of them (64 chunks per pass) and
+  // wavefront 0 leaves them in LDS
+  float m_all = kSeedM;
+  for (int s0 = 0; s0 < used; s0 += 64)
+    m_all = fmaxf(m_all, wave_max(s0 + lane < used ? ml[s0 + lane].x : kSeedM));
+  float l_all = 0.f;
+  for (int s0 = 0; s0 < used; s0 += 64) {
+    const bool in = s0 + lane < used;
+    const float2 mine = ml[min(s0 + lane, used - 1)];
+    const float w = in ? fast_exp(mine.x - m_all) : 0.f;
+    l_all += wave_sum(mine.y * w);
+    if (tid < 64 && in)
+      w_s[s0 + lane] = w;
+  }
+  __syncthreads();
+  for (int i0 = 0; i0 < kPer; i0 += 4) {
+    if (g + 32 * i0 >= used)
+      break;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      v[i] = *reinterpret_cast<const float4 *>(acc + (size_t)min(g + 32 * (i0 + i), used - 1) * kD);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int c = g + 32 * (i0 + i);
+      if (c < used) {
+        const float w = w_s[c];
+        sum.x = fmaf(v[i].x, w, sum.x);
+        sum.y = fmaf(v[i].y, w, sum.y);
+        sum.z = fmaf(v[i].z, w, sum.z);
+        sum.w = fmaf(v[i].w, w, sum.w);
+      }
+    }
+  }
+  red_s[g][q] = sum;
+  __syncthreads();
+  if (tid < 32) {
+    float4 o = red_s[0][tid];
+#pragma unroll 8
+    for (int gg = 1; gg < 32; ++gg) {
+      const float4 r = red_s[gg][tid];
+      o.x += r.x; o.y += r.y; o.z += r.z; o.w += r.w;
+    }
+    const float inv = 1.0f / l_all;
+    *reinterpret_cast<float4 *>(a.out + (size_t)h * kD + tid * 4) =
+        make_float4(o.x * inv, o.y * inv, o.z * inv, o.w * inv);
+  }
 }
 
 // ---- scratch of the entry point that allocates nothing --------------------
@@ -353,9 +580,32 @@ int launch_attn_decode(const AttnDecodeArgs &in, hipStream_t stream) {
   a.out = in.out;
   a.lse = in.lse;
   a.used = in.chunks_used > 0 ? std::min(in.chunks_used, a.nchunks) : a.nchunks;
-  BH_REQUIRE(!in.combine || a.used == a.nchunks,
+  BH_REQUIRE(!in.combine || in.wide_combine || a.used == a.nchunks,
              "attn_decode: the combine pass needs a partial for every chunk");
+  BH_REQUIRE(!in.wide_combine || (in.combine && !in.lse && a.used <= kWideChunks),
+             "attn_decode: the wide combine takes up to %d partials per head and returns no lse",
+             kWideChunks);
   a.pairs_padded = (int)round_up((int64_t)a.used * in.kv_heads, 8);
+  if (in.wide_combine) {
+    // far into a long cache: one workgroup per (chunk, KV head) for all its heads
+    const dim3 grid(a.used * in.kv_heads);
+    const size_t lds = sizeof(float) * (size_t)a.group * (in.chunk / kPW) * kD; // <= 64 KiB
+    if (in.chunk == 64) {
+      hipLaunchKernelGGL(attn_decode_partial_group<4>, grid, dim3(4 * 64), lds, stream, a);
+    } else if (in.chunk == 128) {
+      hipLaunchKernelGGL(attn_decode_partial_group<8>, grid, dim3(8 * 64), lds, stream, a);
+    } else {
+      // with 8 heads per KV head the 64 KiB of dynamic LDS come on top of 6 KiB
+      static DynLdsOnce dyn_lds;
+      BH_CHECK_HIP(ensure_dyn_lds(dyn_lds,
+                                  reinterpret_cast<const void *>(attn_decode_partial_group<16>),
+                                  (int)(sizeof(float) * kMaxGroup * 16 * kD)));
+      hipLaunchKernelGGL(attn_decode_partial_group<16>, grid, dim3(16 * 64), lds, stream, a);
+    }
+    hipLaunchKernelGGL(attn_decode_combine_wide, dim3(in.heads), dim3(1024), 0, stream, a);
+    BH_CHECK_HIP(hipGetLastError());
+    return BUDDY_HIP_OK;
+  }
   const dim3 grid(a.pairs_padded * a.group);
   if (in.chunk == 64)
     hipLaunchKernelGGL(attn_decode_partial<4>, grid, dim3(4 * 64), 0, stream, a);
@@ -363,7 +613,9 @@ int launch_attn_decode(const AttnDecodeArgs &in, hipStream_t stream) {
     hipLaunchKernelGGL(attn_decode_partial<8>, grid, dim3(8 * 64), 0, stream, a);
   else
     hipLaunchKernelGGL(attn_decode_partial<16>, grid, dim3(16 * 64), 0, stream, a);
-  if (in.combine)
+  if (in.combine && in.wide_combine)
+    hipLaunchKernelGGL(attn_decode_combine_wide, dim3(in.heads), dim3(1024), 0, stream, a);
+  else if (in.combine)
     hipLaunchKernelGGL(attn_decode_combine, dim3(in.heads), dim3(kD), 0, stream, a);
   BH_CHECK_HIP(hipGetLastError());
   return BUDDY_HIP_OK;

@@ -202,10 +202,10 @@ struct Session {
     return launch_gemv(g, stream);
   }
 
-  // Enqueues one decode step (reads token/pos from device state); attn_chunk:
-  // cache positions per attention partial, attn_used: partials covered, both
-  // chosen by the host from the position.
-  int enqueue_step(int attn_chunk, int attn_used) {
+  // Enqueues one decode step (reads token/pos from device state) with the cut
+  // of the attention the host chose from the position.
+  int enqueue_step(const AttnStepPlan &plan) {
+    const int attn_chunk = plan.chunk, attn_used = plan.used;
     // x and the RoPE table were prepared by the previous step's last kernel (or
     // by prepare_step after the host set token and position)
     const auto &S = shape;
@@ -235,12 +235,21 @@ struct Session {
       a.scale = scale;
       a.workspace = attn_ws;
       a.workspace_bytes = attn_ws_bytes;
-      a.combine = false; // o_proj folds the partials while staging its input
+      // o_proj folds the partials while staging its input -- up to the 18 it
+      // requests in one trip; beyond that (positions from 4608 on) every one of
+      // its workgroups would repeat a fold that outgrows the matrix, and a
+      // launch of its own folds them once
+      const bool own_fold = plan.own_fold;
+      a.combine = own_fold;
+      a.wide_combine = own_fold;
       a.chunk = attn_chunk;
       a.chunks_used = attn_used;
       if ((rc = launch_attn_decode(a, stream)))
         return rc;
-      {
+      if (own_fold) {
+        if ((rc = gemv(att, L.o, nullptr, nullptr, x, kEpiAccum)))
+          return rc;
+      } else {
         const AttnPartials parts =
             attn_partials(attn_ws, S.heads, S.head_dim, S.max_len, attn_chunk);
         GemvArgs g;
@@ -557,15 +566,14 @@ struct Session {
     int rc = check_steps(1, "decode step");
     if (rc)
       return rc;
-    const int attn_chunk = attn_chunk_for_position(next_pos);
-    const int attn_used = attn_chunks_for_position(next_pos, attn_chunk, shape.max_len);
+    const AttnStepPlan plan = attn_step_plan(next_pos, shape.max_len, shape.kv_heads);
     if (!use_graph) {
-      rc = enqueue_step(attn_chunk, attn_used);
+      rc = enqueue_step(plan);
     } else {
-      StepGraph &g = graphs[{attn_chunk, attn_used}];
+      StepGraph &g = graphs[{plan.chunk, plan.own_fold ? -plan.used : plan.used}];
       if (!g.exec) {
         BH_CHECK_HIP(hipStreamBeginCapture(stream, hipStreamCaptureModeThreadLocal));
-        rc = enqueue_step(attn_chunk, attn_used);
+        rc = enqueue_step(plan);
         hipError_t e = hipStreamEndCapture(stream, &g.graph);
         if (!rc && e != hipSuccess)
           rc = fail(BUDDY_HIP_ERR_HIP, "hipStreamEndCapture: %s", hipGetErrorString(e));

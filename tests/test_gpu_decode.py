@@ -392,15 +392,16 @@ def test_small_model_decodes_at_long_context(oracle):
     sess.close()
 
 
-@pytest.mark.parametrize("start", [100, 1140, 2296])
+@pytest.mark.parametrize("start", [100, 1140, 2296, 4596, 9400])
 def test_small_model_steps_across_the_attention_chunk_sizes(oracle, start):
     """A step far into a long cache takes attention chunks of 128 or 256 positions
-    (from positions 1152 and 2304 on) and covers only the chunks up to its
-    position: greedy steps that cross each boundary, and a short context in a
-    large cache, against the oracle -- every step's logits and the token fed back
-    on the device."""
+    (from positions 1152 and 2304 on), covers only the chunks up to its position,
+    and from position 4608 on folds the partials in a launch of its own instead of
+    in the o_proj launch: greedy steps that cross each boundary, a short context
+    in a large cache and a step with 37 partials per head, against the oracle --
+    every step's logits and the token fed back on the device."""
     shape = Shape(layers=2, hidden=256, heads=4, kv_heads=2, head_dim=128, inter=512,
-                  vocab=1024, max_len=4352, rms_eps=1e-6)
+                  vocab=1024, max_len=9472 if start > 4400 else 4352, rms_eps=1e-6)
     sess, host = synthetic.build_session(shape, context=start, keep_host=True, ln_jitter=0.1)
     om = oracle_model(oracle, shape, host)
     kv = [a.copy() for a in host["kv"]]
