@@ -392,16 +392,18 @@ def test_small_model_decodes_at_long_context(oracle):
     sess.close()
 
 
-@pytest.mark.parametrize("start", [100, 1140, 2296, 4596, 9400])
+@pytest.mark.parametrize("start", [100, 1140, 2296, 4596, 9400, 12280, 24310])
 def test_small_model_steps_across_the_attention_chunk_sizes(oracle, start):
     """A step far into a long cache takes attention chunks of 128 or 256 positions
     (from positions 1152 and 2304 on), covers only the chunks up to its position,
     and from position 4608 on folds the partials in a launch of its own instead of
     in the o_proj launch: greedy steps that cross each boundary, a short context
-    in a large cache and a step with 37 partials per head, against the oracle --
-    every step's logits and the token fed back on the device."""
+    in a large cache, and the lengths at which the launches of all heads of a KV
+    head go from chunks of 64 to 128 and to 256 positions (12288, 24320), against
+    the oracle -- every step's logits and the token fed back on the device."""
     shape = Shape(layers=2, hidden=256, heads=4, kv_heads=2, head_dim=128, inter=512,
-                  vocab=1024, max_len=9472 if start > 4400 else 4352, rms_eps=1e-6)
+                  vocab=1024, max_len=(start + 100 + 63) // 64 * 64 if start > 4400 else 4352,
+                  rms_eps=1e-6)
     sess, host = synthetic.build_session(shape, context=start, keep_host=True, ln_jitter=0.1)
     om = oracle_model(oracle, shape, host)
     kv = [a.copy() for a in host["kv"]]
