@@ -6,14 +6,15 @@
 namespace bh {
 
 constexpr int kAttnChunk = 64; // cache positions per flash-decoding partial (the default)
-// How a decode step at position `pos` cuts its attention.  Up to 18 partials per
-// head the o_proj launch folds them in one trip to memory: chunks of 64 positions
-// up to position 1152, 128 up to 2304, 256 up to 4608 (8 or 16 wavefronts of 16
-// positions per workgroup).  Beyond that the partials are folded by a launch of
-// their own and one workgroup takes all the query heads of a KV head (a K/V row
-// then leaves L2 once, not once per head); its chunks are the largest that still
-// give the launch about 200 workgroups.  Attention and fold cover only the
-// chunks up to the position, in batches of 18, whatever the cache's capacity.
+// How a decode step at position `pos` cuts its attention.  The o_proj launch
+// folds up to 36 partials per head in one trip to memory (18 at its best):
+// chunks of 64 positions up to position 1152, 128 up to 2304, 256 up to 9216 (8
+// or 16 wavefronts of 16 positions per workgroup).  Beyond that the partials are
+// folded by a launch of their own and one workgroup takes all the query heads of
+// a KV head (a K/V row then leaves L2 once, not once per head); its chunks are
+// the largest that still give the launch about 200 workgroups.  Attention and
+// fold cover only the chunks up to the position, in batches of 18, whatever the
+// cache's capacity.
 struct AttnStepPlan {
   int chunk;     // cache positions per partial: 64, 128 or 256
   int used;      // partials per head the step produces and folds
@@ -21,7 +22,7 @@ struct AttnStepPlan {
 };
 inline AttnStepPlan attn_step_plan(int pos, int max_len, int kv_heads) {
   AttnStepPlan p;
-  p.own_fold = pos >= 18 * 256;
+  p.own_fold = pos >= 36 * 256;
   if (!p.own_fold) {
     p.chunk = pos < 18 * 64 ? 64 : pos < 18 * 128 ? 128 : 256;
   } else {

@@ -637,21 +637,23 @@ __device__ __forceinline__ void attn_fold_tiles(const KernelArgs &a, int t0, int
     m[u] = -1.0e30f;
     l[u] = 0.f;
   }
-  if (used <= B) {
-    // The usual case (a cache of up to 18 chunks = 1152 positions): one batch,
-    // and nothing in it depends on anything loaded -- the (max, sum) pair of
-    // every chunk and the partial sums of every tile are requested together, so
-    // the fold costs one trip to memory, not two.  Slots past the last chunk
-    // repeat it (a valid, finite partial) and get weight 0.
+  // The usual case (up to 18 chunks: a cache of 1152 positions, or a step whose
+  // chunks are 128 or 256 positions), and up to 36: one batch, and nothing in it
+  // depends on anything loaded -- the (max, sum) pair of every chunk and the
+  // partial sums of every tile are requested together, so the fold costs one trip
+  // to memory, not two.  Slots past the last chunk repeat it (a valid, finite
+  // partial) and get weight 0.
+  auto one_batch = [&](auto batch) {
+    constexpr int BB = decltype(batch)::value;
     float2 mine[U];
-    float v[U][B];
+    float v[U][BB];
 #pragma unroll
     for (int u = 0; u < U; ++u)
       mine[u] = ml[u][min(lane, used - 1)];
 #pragma unroll
     for (int u = 0; u < U; ++u)
 #pragma unroll
-      for (int j = 0; j < B; ++j)
+      for (int j = 0; j < BB; ++j)
         v[u][j] = acc[u][(size_t)min(j, used - 1) * a.head_dim];
     const bool valid = lane < used;
 #pragma unroll
@@ -660,9 +662,14 @@ __device__ __forceinline__ void attn_fold_tiles(const KernelArgs &a, int t0, int
       const float w = valid ? fast_exp(mine[u].x - mb) : 0.f;
       l[u] = wave_sum(mine[u].y * w);
 #pragma unroll
-      for (int j = 0; j < B; ++j)
+      for (int j = 0; j < BB; ++j)
         r[u] = fmaf(v[u][j], lane_f(w, j), r[u]);
     }
+  };
+  if (used <= B) {
+    one_batch(std::integral_constant<int, B>{});
+  } else if (used <= 2 * B && U <= 2) {
+    one_batch(std::integral_constant<int, 2 * B>{});
   } else {
   for (int c0 = 0; c0 < used; c0 += kWave) { // 64 chunks per pass
     const int cnt = min(kWave, used - c0);

@@ -392,11 +392,11 @@ def test_small_model_decodes_at_long_context(oracle):
     sess.close()
 
 
-@pytest.mark.parametrize("start", [100, 1140, 2296, 4596, 9400, 12280, 24310])
+@pytest.mark.parametrize("start", [100, 1140, 2296, 4596, 9206, 12280, 24310])
 def test_small_model_steps_across_the_attention_chunk_sizes(oracle, start):
     """A step far into a long cache takes attention chunks of 128 or 256 positions
     (from positions 1152 and 2304 on), covers only the chunks up to its position,
-    and from position 4608 on folds the partials in a launch of its own instead of
+    and from position 9216 on folds the partials in a launch of its own instead of
     in the o_proj launch: greedy steps that cross each boundary, a short context
     in a large cache, and the lengths at which the launches of all heads of a KV
     head go from chunks of 64 to 128 and to 256 positions (12288, 24320), against
