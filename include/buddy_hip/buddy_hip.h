@@ -379,7 +379,10 @@ int buddy_hip_matmul_f32(const float *A, const float *B, float *C, int64_t M,
  * 4986-5004) and runs the greedy part of runtime/llm/TextGeneration.cpp:215-266
  * on the device.  Field names follow the HF config, not the reference's
  * (its `head_num` is kv_heads and its `hidden_size` is head_dim:
- * tools/buddy-codegen/gen_config.py:288-299).  Not re-entrant per session. */
+ * tools/buddy-codegen/gen_config.py:288-299).  Not re-entrant per session.
+ * max_len is the capacity of the cache only: what a decode step costs follows
+ * its position (the attention is cut by it: larger chunks far into a long
+ * cache, only the chunks up to the position; one captured graph per cut). */
 typedef struct buddy_hip_model_shape {
   int layers, hidden, heads, kv_heads, head_dim, inter, vocab;
   int max_len;    /* KV cache capacity in positions */
