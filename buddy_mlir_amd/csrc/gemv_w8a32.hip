@@ -1112,7 +1112,8 @@ __global__ void __launch_bounds__(kMaxWaves *kWave)
         float v = in ? x[m][q][e] : 0.f;
         if (NORM) {
           ss[m] = fmaf(v, v, ss[m]);
-          v *= nw[q][e];
+          // (the weight's 16 bytes may reach past its end, where anything lies)
+          v = in ? v * nw[q][e] : 0.f;
         }
         x[m][q][e] = v;
         mb = max(mb, __float_as_uint(v) & 0x7fffffffu);

@@ -195,7 +195,7 @@ def test_norm_weight_alignment_and_ragged_k(bh, oracle, M):
     """RMSNorm fused into the GEMV with K not a multiple of 4: the kernels read
     the norm weight in 16-byte pieces, so one that is not 16-byte aligned (a
     piece could run past its end) is refused; an aligned one gives the oracle's
-    result."""
+    result whatever lies behind its last value."""
     K, N = 1001, 272
     eps = np.float32(1e-6)
     g = torch.Generator(device="cuda").manual_seed(70 + M)
@@ -207,7 +207,12 @@ def test_norm_weight_alignment_and_ragged_k(bh, oracle, M):
     with pytest.raises(bma.BuddyHipError, match="16-byte aligned"):
         ops.linear_w8a32(A=x, lda=K, W0=ops.pack_w8(q), scale0=s, norm_w=wbuf[1:],
                          norm_eps=float(eps), C=out, ldc=N, M=M, K=K, N=N, epilogue=0)
-    w = wbuf[:K].clone()
+    # the weight's last 16-byte piece reaches past its K values, and what lies
+    # there (NaNs here) must not reach the result
+    wpad = torch.full((K + 7,), float("nan"), device="cuda")
+    wpad[:K] = wbuf[:K]
+    w = wpad[:K]
+    assert w.data_ptr() % 16 == 0
     ops.linear_w8a32(A=x, lda=K, W0=ops.pack_w8(q), scale0=s, norm_w=w, norm_eps=float(eps),
                      C=out, ldc=N, M=M, K=K, N=N, epilogue=0)
     torch.cuda.synchronize()
