@@ -89,10 +89,20 @@ def test_fast_kernel_against_the_real_number_sum(bh, oracle, K, N):
     dot = a.astype(np.float64) @ qh.astype(np.float64)
     exact = c0.astype(np.float64) + dot * scale.astype(np.float64)
     # the best an f16 result can be: half a unit in the last place of the exact
-    # value (plus the f32 roundings of the finishing multiply-add)
+    # value (plus the f32 roundings of the finishing multiply-add).  The sums of
+    # a wavefront's run (exact integers) and of the k-slices meet in f32: where an
+    # outlier makes a slice's sum large and the result is a cancellation, those
+    # roundings (2^-24 of the largest partial sum each) show.  With that term at
+    # its worst case over the whole row the bound holds for every element; without
+    # it for all but a few in a thousand.
     ulp = np.spacing(np.abs(exact).astype(np.float16)).astype(np.float64)
     slack = 4e-7 * (np.abs(c0.astype(np.float64)) + np.abs(dot * scale.astype(np.float64)))
-    assert (np.abs(got - exact) <= 0.5 * ulp * (1 + 2.0 ** -9) + slack).all()
+    tight = 0.5 * ulp * (1 + 2.0 ** -9) + slack
+    fixed = (float(np.abs(a.astype(np.float64)).max()) * 2.0 ** -23 *
+             (np.abs(qh.astype(np.float64)).sum(axis=0) * scale.astype(np.float64)))
+    err = np.abs(got - exact)
+    assert (err <= tight + fixed).all()
+    assert (err > tight).sum() <= max(1, N // 300), int((err > tight).sum())
     # and no further from it than the reference's f16 chain
     ref = oracle.w4a16_gemv(a, ph, scale, c0).astype(np.float64)
     assert np.linalg.norm(got - exact) <= np.linalg.norm(ref - exact) + 1e-12
