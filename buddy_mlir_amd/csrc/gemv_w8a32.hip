@@ -1025,8 +1025,13 @@ __global__ void __launch_bounds__(kMaxWaves *kWave)
     for (int q = 0; q < XV; ++q) {
       const int kc = min(t0 * kTileK + q * 256 + 4 * lane, klast);
       if (NORM) {
+        // (the weight's last 16 bytes may reach past its end, where anything
+        // lies -- a NaN there would turn the zero it meets into a NaN)
         const float4 v = *reinterpret_cast<const float4 *>(a.norm_w + kc);
-        nw[q][0] = v.x, nw[q][1] = v.y, nw[q][2] = v.z, nw[q][3] = v.w;
+        nw[q][0] = v.x;
+        nw[q][1] = kc + 1 < a.K ? v.y : 0.f;
+        nw[q][2] = kc + 2 < a.K ? v.z : 0.f;
+        nw[q][3] = kc + 3 < a.K ? v.w : 0.f;
       }
 #pragma unroll
       for (int m = 0; m < M; ++m) { // rows past the batch repeat its last row; never stored
@@ -1112,8 +1117,7 @@ __global__ void __launch_bounds__(kMaxWaves *kWave)
         float v = in ? x[m][q][e] : 0.f;
         if (NORM) {
           ss[m] = fmaf(v, v, ss[m]);
-          // (the weight's 16 bytes may reach past its end, where anything lies)
-          v = in ? v * nw[q][e] : 0.f;
+          v *= nw[q][e];
         }
         x[m][q][e] = v;
         mb = max(mb, __float_as_uint(v) & 0x7fffffffu);
