@@ -134,6 +134,7 @@ def _declare(lib):
         "buddy_hip_w8a32_blob_layout": (i64, [vp, vp, i64]),
         "buddy_hip_set_gemv_batch_kernel": (c_int, [c_int]),
         "buddy_hip_gemv_w8a32_plan": (c_int, [i64, i64, i64, c_uint, vp]),
+        "buddy_hip_attn_step_plan": (c_int, [c_int, c_int, c_int, vp, vp, vp]),
         "buddy_hip_session_create_from_w8a32_blobs": (vp, [vp, vp, i64, vp, i64]),
         "_mlir_ciface_forward_prefill": (None, [vp, vp, vp, vp]),
         "_mlir_ciface_forward_decode": (None, [vp] * 88),

@@ -38,6 +38,8 @@ inline AttnStepPlan attn_step_plan(int pos, int max_len, int kv_heads) {
   p.used = batches * 18 < all ? batches * 18 : all;
   return p;
 }
+// partials per head the fold of its own takes: 2^20 positions at 256 per chunk
+constexpr int kAttnWideChunks = 4096;
 constexpr int kAttnHeadDim = 128; // the head size the decode kernel is written for
 
 struct AttnDecodeArgs {

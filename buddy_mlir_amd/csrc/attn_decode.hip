@@ -422,7 +422,7 @@ __global__ void __launch_bounds__(kD) attn_decode_combine(AttnArgs a) {
 // every load in flight at once, every wavefront works out the common maximum and
 // the weights exp(m_s - max m) for itself, and the 32 groups meet in LDS.  The
 // sums are those of the chunk-by-chunk rule in another order.
-constexpr int kWideChunks = 1024; // partials per head it takes (256 k positions at 256 per chunk)
+constexpr int kWideChunks = kAttnWideChunks; // partials per head it takes
 
 __global__ void __launch_bounds__(1024) attn_decode_combine_wide(AttnArgs a) {
   constexpr int kPer = kWideChunks / 32; // chunks per thread at most
@@ -628,6 +628,18 @@ extern "C" {
 size_t buddy_hip_attn_decode_workspace_bytes(int heads, int max_len) {
   return bh::attn_decode_workspace_bytes(heads, max_len);
 }
+
+int buddy_hip_attn_step_plan(int pos, int max_len, int kv_heads, int *chunk, int *partials,
+                             int *own_fold) try {
+  BH_REQUIRE(chunk && partials && own_fold, "attn_step_plan: null argument");
+  BH_REQUIRE(max_len > 0 && pos >= 0 && pos < max_len && kv_heads > 0,
+             "attn_step_plan: pos=%d max_len=%d kv_heads=%d", pos, max_len, kv_heads);
+  const bh::AttnStepPlan p = bh::attn_step_plan(pos, max_len, kv_heads);
+  *chunk = p.chunk;
+  *partials = p.used;
+  *own_fold = p.own_fold ? 1 : 0;
+  return BUDDY_HIP_OK;
+} BH_CATCH_INT("buddy_hip_attn_step_plan")
 
 int buddy_hip_gqa_decode_attention(const float *qkv, const float *inv_freq,
                                    const int *pos, float *kcache, float *vcache,

@@ -646,6 +646,11 @@ buddy_hip_session *buddy_hip_session_create(const buddy_hip_model_shape *shape,
     bh::fail(BUDDY_HIP_ERR_NO_DEVICE, "session_create: no HIP device");
     return nullptr;
   }
+  if (S.max_len > bh::kAttnWideChunks * 256) {
+    bh::fail(BUDDY_HIP_ERR_ARG, "session_create: max_len %d above %d positions", S.max_len,
+             bh::kAttnWideChunks * 256);
+    return nullptr;
+  }
   Session *s = new (std::nothrow) Session();
   if (!s)
     return nullptr;

@@ -317,6 +317,14 @@ int buddy_hip_argmax(const float *x, int n, void *workspace, int *out_index,
  * (tosa.py:14576-14594).  head_dim must be 128.  *pos must lie in
  * 0..max_len-1; a position outside writes no cache row. */
 size_t buddy_hip_attn_decode_workspace_bytes(int heads, int max_len);
+/* How the session cuts the attention of a decode step at position `pos` (host
+ * arithmetic, no device needed): cache positions per partial (64, 128 or 256),
+ * partials per head the step produces and folds (they cover the position), and
+ * whether a launch of its own folds them (1) or the o_proj launch does (0).
+ * No counterpart in the reference (its cache length is a compile-time tier,
+ * tools/buddy-codegen/gen_session.py:358-379). */
+int buddy_hip_attn_step_plan(int pos, int max_len, int kv_heads, int *chunk, int *partials,
+                             int *own_fold);
 int buddy_hip_gqa_decode_attention(const float *qkv, const float *inv_freq,
                                    const int *pos, float *kcache, float *vcache,
                                    float *out, float *lse, int heads,
