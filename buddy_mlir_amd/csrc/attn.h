@@ -19,17 +19,24 @@ struct AttnStepPlan {
   int chunk;     // cache positions per partial: 64, 128 or 256
   int used;      // partials per head the step produces and folds
   bool own_fold; // a launch of its own folds them; workgroups take whole head groups
+  int head_split; // ... or (2) half a head group each
 };
 inline AttnStepPlan attn_step_plan(int pos, int max_len, int kv_heads) {
   AttnStepPlan p;
+  p.head_split = 1;
   p.own_fold = pos >= 36 * 256;
   if (!p.own_fold) {
     p.chunk = pos < 18 * 64 ? 64 : pos < 18 * 128 ? 128 : 256;
   } else {
-    p.chunk = 64;
+    // Whole head groups on the largest chunks that still give ~200 workgroups; where that
+    // would take chunks of 64, chunks of 128 with half a head group per workgroup instead
+    // (measured: 128 x 2 beats 64 x 1, and 128 x 1 beats 256 x 2).
+    p.chunk = 128;
+    p.head_split = 2;
     for (int c : {256, 128})
       if ((pos / c + 1) * kv_heads >= 192) {
         p.chunk = c;
+        p.head_split = 1;
         break;
       }
   }
@@ -62,6 +69,7 @@ struct AttnDecodeArgs {
   // per (chunk, KV head) for all its query heads, then a fold with all partials
   // in flight instead of chunk by chunk (covers chunks_used partials, no lse)
   bool wide_combine = false;
+  int head_split = 1; // with wide_combine: 2 = two workgroups per (chunk, KV head), half its heads each
   int chunk = kAttnChunk; // cache positions per partial: 64, 128 or 256
   // partials to produce (the first ones; the caller knows the position lies in
   // them); 0: one for every chunk of the cache

@@ -47,6 +47,7 @@ struct AttnArgs {
   float *lse;            // [heads] or null: m + log l of the whole softmax
   int heads, kv_heads, group, max_len, nchunks, chunk;
   int used; // chunks this launch covers (the first ones of nchunks)
+  int head_split; // grouped launches: workgroups per (chunk, KV head), each a share of its heads
   float scale;
   int pairs_padded; // (chunk, kv head) pairs rounded up to the XCD count
 };
@@ -249,10 +250,13 @@ __global__ void __launch_bounds__(kWaves * 64) attn_decode_partial_group(AttnArg
 
   const int tid = threadIdx.x;
   const int wave = tid >> 6, lane = tid & 63;
-  const int ckv = blockIdx.x;
+  const int ckv = blockIdx.x / a.head_split, hs = blockIdx.x % a.head_split;
   if (ckv >= a.used * a.kv_heads)
     return; // padding id
   const int chunk = ckv % a.used, kvh = ckv / a.used;
+  // this workgroup's share of the group's query heads
+  const int per = (a.group + a.head_split - 1) / a.head_split;
+  const int h_lo = hs * per, h_hi = min(a.group, h_lo + per);
   const int p0 = chunk * kChunk;
   const int c4 = lane & 31, par = lane >> 5;
   const int pw0 = p0 + wave * kPW;
@@ -273,12 +277,12 @@ __global__ void __launch_bounds__(kWaves * 64) attn_decode_partial_group(AttnArg
   const bool pos_ok = pos_raw >= 0 && pos_raw < a.max_len;
   const int pos = min(max(pos_raw, 0), a.max_len - 1);
   if (p0 > pos) { // nothing visible in this chunk: empty partials
-    for (int i = tid; i < a.group * kD; i += kWaves * 64) {
-      const int h = kvh * a.group + i / kD;
+    for (int i = tid; i < (h_hi - h_lo) * kD; i += kWaves * 64) {
+      const int h = kvh * a.group + h_lo + i / kD;
       a.part_acc[((size_t)h * a.nchunks + chunk) * kD + i % kD] = 0.f;
     }
-    if (tid < a.group) {
-      const int h = kvh * a.group + tid;
+    if (tid < h_hi - h_lo) {
+      const int h = kvh * a.group + h_lo + tid;
       a.part_ml[((size_t)h * a.nchunks + chunk) * 2 + 0] = kSeedM;
       a.part_ml[((size_t)h * a.nchunks + chunk) * 2 + 1] = 0.f;
     }
@@ -307,7 +311,7 @@ __global__ void __launch_bounds__(kWaves * 64) attn_decode_partial_group(AttnArg
       const float vraw = src[(size_t)a.kv_heads * kD + j];
       knew_s[j] = rot;
       vnew_s[j] = vraw;
-      if (pos_ok) {
+      if (pos_ok && hs == 0) { // one writer per cache row
         a.kcache[((size_t)kvh * a.max_len + pos) * kD + j] = rot;
         a.vcache[((size_t)kvh * a.max_len + pos) * kD + j] = vraw;
       }
@@ -321,8 +325,7 @@ __global__ void __launch_bounds__(kWaves * 64) attn_decode_partial_group(AttnArg
       kreg[i] = *reinterpret_cast<const float4 *>(knew_s + c4 * 4);
       vreg[i] = *reinterpret_cast<const float4 *>(vnew_s + c4 * 4);
     }
-  for (int hh = 0; hh < a.group; ++hh) {
-    const int h = kvh * a.group + hh;
+  for (int hh = h_lo; hh < h_hi; ++hh) {
     const float4 q4 = *reinterpret_cast<const float4 *>(q_s[hh] + c4 * 4);
     float sc[kR];
 #pragma unroll
@@ -371,8 +374,8 @@ __global__ void __launch_bounds__(kWaves * 64) attn_decode_partial_group(AttnArg
   }
   __syncthreads();
   // ---- the wavefronts meet, once for all heads: one partial per (head, chunk) --
-  for (int i = tid; i < a.group * kD; i += kWaves * 64) {
-    const int hh = i / kD, d = i % kD, h = kvh * a.group + hh;
+  for (int i = tid; i < (h_hi - h_lo) * kD; i += kWaves * 64) {
+    const int hh = h_lo + i / kD, d = i % kD, h = kvh * a.group + hh;
     float m = mw_s[hh][0];
 #pragma unroll
     for (int w = 1; w < kWaves; ++w)
@@ -580,6 +583,7 @@ int launch_attn_decode(const AttnDecodeArgs &in, hipStream_t stream) {
   a.out = in.out;
   a.lse = in.lse;
   a.used = in.chunks_used > 0 ? std::min(in.chunks_used, a.nchunks) : a.nchunks;
+  a.head_split = 1;
   BH_REQUIRE(!in.combine || in.wide_combine || a.used == a.nchunks,
              "attn_decode: the combine pass needs a partial for every chunk");
   BH_REQUIRE(!in.wide_combine || (in.combine && !in.lse && a.used <= kWideChunks),
@@ -588,7 +592,10 @@ int launch_attn_decode(const AttnDecodeArgs &in, hipStream_t stream) {
   a.pairs_padded = (int)round_up((int64_t)a.used * in.kv_heads, 8);
   if (in.wide_combine) {
     // far into a long cache: one workgroup per (chunk, KV head) for all its heads
-    const dim3 grid(a.used * in.kv_heads);
+    BH_REQUIRE(in.head_split == 1 || in.head_split == 2, "attn_decode: head_split %d",
+               in.head_split);
+    a.head_split = std::min(in.head_split, a.group); // a group of one head has nothing to share out
+    const dim3 grid(a.used * in.kv_heads * a.head_split);
     const size_t lds = sizeof(float) * (size_t)a.group * (in.chunk / kPW) * kD; // <= 64 KiB
     if (in.chunk == 64) {
       hipLaunchKernelGGL(attn_decode_partial_group<4>, grid, dim3(4 * 64), lds, stream, a);

@@ -244,6 +244,7 @@ struct Session {
       a.wide_combine = own_fold;
       a.chunk = attn_chunk;
       a.chunks_used = attn_used;
+      a.head_split = plan.head_split;
       if ((rc = launch_attn_decode(a, stream)))
         return rc;
       if (own_fold) {
@@ -570,7 +571,7 @@ struct Session {
     if (!use_graph) {
       rc = enqueue_step(plan);
     } else {
-      StepGraph &g = graphs[{plan.chunk, plan.own_fold ? -plan.used : plan.used}];
+      StepGraph &g = graphs[{plan.chunk * 4 + plan.head_split, plan.own_fold ? -plan.used : plan.used}];
       if (!g.exec) {
         BH_CHECK_HIP(hipStreamBeginCapture(stream, hipStreamCaptureModeThreadLocal));
         rc = enqueue_step(plan);
