@@ -68,7 +68,6 @@ template <int kWaves>
 __global__ void __launch_bounds__(kWaves * 64) attn_decode_partial(AttnArgs a) {
   constexpr int kChunk = kWaves * kPW; // cache positions per workgroup: 64, 128 or 256
   constexpr int kR = kPW / 2;          // rows per lane: 8
-  __shared__ __attribute__((aligned(16))) float q_s[kD], knew_s[kD], vnew_s[kD];
   __shared__ __attribute__((aligned(16))) float accw_s[kWaves][kD];
   __shared__ float mw_s[kWaves], lw_s[kWaves];
 
@@ -81,26 +80,28 @@ __global__ void __launch_bounds__(kWaves * 64) attn_decode_partial(AttnArgs a) {
   const int p0 = chunk * kChunk;
   const int h = kvh * a.group + hb; // this workgroup's query head
 
-  // ---- small operands first: they are what the barrier below waits for ----
-  // thread j < 128 rotates element j of q and of the token's k, with the angle
-  // of j mod 64
-  const int j = tid & (kD - 1), jj = j & (kD / 2 - 1);
-  float qraw = 0.f, qpair = 0.f, kraw = 0.f, kpair = 0.f, vraw = 0.f;
-  float inv_f = 0.f, cs = 0.f, sn = 0.f;
-  if (tid < kD) {
-    const float *q = a.qkv + (size_t)h * kD;
-    qraw = q[j];
-    qpair = j < kD / 2 ? -q[j + kD / 2] : q[j - kD / 2];
-    const float *k = a.qkv + (size_t)a.heads * kD + (size_t)kvh * kD;
-    kraw = k[j];
-    kpair = j < kD / 2 ? -k[j + kD / 2] : k[j - kD / 2];
-    vraw = k[(size_t)a.kv_heads * kD + j];
-    if (a.rope_table) {
-      cs = a.rope_table[jj];
-      sn = a.rope_table[kD / 2 + jj];
-    } else {
-      inv_f = a.inv_freq[jj];
-    }
+  // ---- small operands first ----------------------------------------------
+  // Every lane asks for what its own four dims (c4) need: q, the new k and v,
+  // their rotation partners 64 dims away and the angles of (dim mod 64).  The
+  // rotation then happens in registers: no wavefront waits for another before
+  // the scores.
+  const int j = tid & (kD - 1);
+  const int c4 = lane & 31, par = lane >> 5;
+  const int d0 = c4 * 4, dp = d0 ^ (kD / 2), ja = d0 & (kD / 2 - 1);
+  const float *qh = a.qkv + (size_t)h * kD;
+  const float *kh = a.qkv + (size_t)a.heads * kD + (size_t)kvh * kD;
+  const float4 q_raw = *reinterpret_cast<const float4 *>(qh + d0);
+  float4 q_pair = *reinterpret_cast<const float4 *>(qh + dp);
+  const float4 k_raw = *reinterpret_cast<const float4 *>(kh + d0);
+  float4 k_pair = *reinterpret_cast<const float4 *>(kh + dp);
+  const float4 v_new = *reinterpret_cast<const float4 *>(kh + (size_t)a.kv_heads * kD + d0);
+  float4 cs4, sn4; // without the table: cs4 holds the inverse frequencies for now
+  if (a.rope_table) {
+    cs4 = *reinterpret_cast<const float4 *>(a.rope_table + ja);
+    sn4 = *reinterpret_cast<const float4 *>(a.rope_table + kD / 2 + ja);
+  } else {
+    cs4 = *reinterpret_cast<const float4 *>(a.inv_freq + ja);
+    sn4 = make_float4(0.f, 0.f, 0.f, 0.f);
   }
   // ---- then this wavefront's 16 K rows and 16 V rows -----------------------
   // One lane mapping for both: lane = (float4 column c4 of the 128 dims, row
@@ -109,7 +110,6 @@ __global__ void __launch_bounds__(kWaves * 64) attn_decode_partial(AttnArgs a) {
   // whatever the position is (rows beyond it hold zeros or stale data and are
   // masked by select, never multiplied in), so nothing here waits for the
   // position to arrive.
-  const int c4 = lane & 31, par = lane >> 5;
   const int pw0 = p0 + wave * kPW; // first position of this wavefront
   float4 kreg[kR], vreg[kR];
 #pragma unroll
@@ -142,32 +142,35 @@ __global__ void __launch_bounds__(kWaves * 64) attn_decode_partial(AttnArgs a) {
   const bool has_new = pos < p0 + kChunk; // the token's own row lies in this chunk
 
   // ---- RoPE: q' = q*cos + cat(-q[64:], q[:64])*sin, same for the new k ------
-  if (tid < kD) {
-    if (!a.rope_table)
-      sincosf(inv_f * (float)pos, &sn, &cs);
-    q_s[j] = qraw * cs + qpair * sn;
-    if (has_new) {
-      const float kn = kraw * cs + kpair * sn;
-      knew_s[j] = kn;
-      vnew_s[j] = vraw;
-      if (hb == 0 && pos_ok) { // one writer per cache row
-        a.kcache[((size_t)kvh * a.max_len + pos) * kD + j] = kn;
-        a.vcache[((size_t)kvh * a.max_len + pos) * kD + j] = vraw;
-      }
-    }
+  if (!a.rope_table) {
+    const float4 f = cs4;
+    sincosf(f.x * (float)pos, &sn4.x, &cs4.x);
+    sincosf(f.y * (float)pos, &sn4.y, &cs4.y);
+    sincosf(f.z * (float)pos, &sn4.z, &cs4.z);
+    sincosf(f.w * (float)pos, &sn4.w, &cs4.w);
   }
-  __syncthreads();
+  if (d0 < kD / 2) {
+    q_pair = make_float4(-q_pair.x, -q_pair.y, -q_pair.z, -q_pair.w);
+    k_pair = make_float4(-k_pair.x, -k_pair.y, -k_pair.z, -k_pair.w);
+  }
+  const float4 q4 = make_float4(q_raw.x * cs4.x + q_pair.x * sn4.x, q_raw.y * cs4.y + q_pair.y * sn4.y,
+                                q_raw.z * cs4.z + q_pair.z * sn4.z, q_raw.w * cs4.w + q_pair.w * sn4.w);
+  const float4 k_new = make_float4(k_raw.x * cs4.x + k_pair.x * sn4.x, k_raw.y * cs4.y + k_pair.y * sn4.y,
+                                   k_raw.z * cs4.z + k_pair.z * sn4.z, k_raw.w * cs4.w + k_pair.w * sn4.w);
+  if (has_new && hb == 0 && pos_ok && tid < 32) { // one writer per cache row
+    *reinterpret_cast<float4 *>(a.kcache + ((size_t)kvh * a.max_len + pos) * kD + d0) = k_new;
+    *reinterpret_cast<float4 *>(a.vcache + ((size_t)kvh * a.max_len + pos) * kD + d0) = v_new;
+  }
 
   // ---- scores of this wavefront's 16 positions ------------------------------
   // every lane of a half ends up with the 8 scores of its half's rows
-  const float4 q4 = *reinterpret_cast<const float4 *>(q_s + c4 * 4);
   float sc[kR];
 #pragma unroll
   for (int i = 0; i < kR; ++i) {
     const int p = pw0 + par + 2 * i;
     float4 k4 = kreg[i];
     if (p == pos) // the token's own key is not in the cache yet
-      k4 = *reinterpret_cast<const float4 *>(knew_s + c4 * 4);
+      k4 = k_new;
     float d = fmaf(q4.x, k4.x, fmaf(q4.y, k4.y, fmaf(q4.z, k4.z, q4.w * k4.w)));
     d = row16_sum(d);               // the 16 lanes of a row
     d += __shfl_xor(d, 16, 64);     // the two rows of a half: all 128 dims
@@ -194,7 +197,7 @@ __global__ void __launch_bounds__(kWaves * 64) attn_decode_partial(AttnArgs a) {
     const int p = pw0 + par + 2 * i;
     float4 v = vreg[i];
     if (p == pos) // the token's own value row
-      v = *reinterpret_cast<const float4 *>(vnew_s + c4 * 4);
+      v = v_new;
     if (p <= pos) { // rows beyond the position may hold anything
       acc.x = fmaf(v.x, sc[i], acc.x);
       acc.y = fmaf(v.y, sc[i], acc.y);
@@ -260,6 +263,28 @@ __global__ void __launch_bounds__(kWaves * 64) attn_decode_partial_group(AttnArg
   const int p0 = chunk * kChunk;
   const int c4 = lane & 31, par = lane >> 5;
   const int pw0 = p0 + wave * kPW;
+  // ---- small operands first: the queries of the group and the token's key, an
+  // element and its rotation partner per thread and pass, with their angles ----
+  constexpr int kPasses = ((kMaxGroup + 1) * kD + kWaves * 64 - 1) / (kWaves * 64);
+  float raw[kPasses], pair[kPasses], cs[kPasses], sn[kPasses], vraw[kPasses];
+#pragma unroll
+  for (int u = 0; u < kPasses; ++u) {
+    const int i = min(tid + u * kWaves * 64, (a.group + 1) * kD - 1); // past the end: repeats
+    const int hh = i / kD, j = i % kD, jj = j & (kD / 2 - 1);
+    // the queries of the group, then (hh == group) the token's own key
+    const float *src = hh < a.group ? a.qkv + (size_t)(kvh * a.group + hh) * kD
+                                    : a.qkv + (size_t)a.heads * kD + (size_t)kvh * kD;
+    raw[u] = src[j];
+    pair[u] = j < kD / 2 ? -src[j + kD / 2] : src[j - kD / 2];
+    vraw[u] = hh < a.group ? 0.f : src[(size_t)a.kv_heads * kD + j];
+    if (a.rope_table) {
+      cs[u] = a.rope_table[jj];
+      sn[u] = a.rope_table[kD / 2 + jj];
+    } else {
+      cs[u] = a.inv_freq[jj]; // the angle needs the position
+      sn[u] = 0.f;
+    }
+  }
   float4 kreg[kR], vreg[kR];
 #pragma unroll
   for (int i = 0; i < kR; ++i) {
@@ -290,30 +315,23 @@ __global__ void __launch_bounds__(kWaves * 64) attn_decode_partial_group(AttnArg
   }
   const bool has_new = pos < p0 + kChunk;
   // ---- RoPE of every query of the group and of the token's key --------------
-  for (int i = tid; i < (a.group + 1) * kD; i += kWaves * 64) {
-    const int hh = i / kD, j = i % kD, jj = j & (kD / 2 - 1);
-    float cs, sn;
-    if (a.rope_table) {
-      cs = a.rope_table[jj];
-      sn = a.rope_table[kD / 2 + jj];
-    } else {
-      sincosf(a.inv_freq[jj] * (float)pos, &sn, &cs);
-    }
-    // the queries of the group, then (hh == group) the token's own key
-    const float *src = hh < a.group ? a.qkv + (size_t)(kvh * a.group + hh) * kD
-                                    : a.qkv + (size_t)a.heads * kD + (size_t)kvh * kD;
-    const float raw = src[j];
-    const float pair = j < kD / 2 ? -src[j + kD / 2] : src[j - kD / 2];
-    const float rot = raw * cs + pair * sn;
-    if (hh < a.group) {
-      q_s[hh][j] = rot;
-    } else if (has_new) {
-      const float vraw = src[(size_t)a.kv_heads * kD + j];
-      knew_s[j] = rot;
-      vnew_s[j] = vraw;
-      if (pos_ok && hs == 0) { // one writer per cache row
-        a.kcache[((size_t)kvh * a.max_len + pos) * kD + j] = rot;
-        a.vcache[((size_t)kvh * a.max_len + pos) * kD + j] = vraw;
+#pragma unroll
+  for (int u = 0; u < kPasses; ++u) {
+    const int i = tid + u * kWaves * 64;
+    if (i < (a.group + 1) * kD) {
+      const int hh = i / kD, j = i % kD;
+      if (!a.rope_table)
+        sincosf(cs[u] * (float)pos, &sn[u], &cs[u]);
+      const float rot = raw[u] * cs[u] + pair[u] * sn[u];
+      if (hh < a.group) {
+        q_s[hh][j] = rot;
+      } else if (has_new) {
+        knew_s[j] = rot;
+        vnew_s[j] = vraw[u];
+        if (pos_ok && hs == 0) { // one writer per cache row
+          a.kcache[((size_t)kvh * a.max_len + pos) * kD + j] = rot;
+          a.vcache[((size_t)kvh * a.max_len + pos) * kD + j] = vraw[u];
+        }
       }
     }
   }
@@ -548,6 +566,10 @@ int launch_attn_decode(const AttnDecodeArgs &in, hipStream_t stream) {
   BH_REQUIRE(in.qkv && in.inv_freq && in.pos_ptr && in.kcache && in.vcache &&
                  (in.out || !in.combine) && in.workspace,
              "attn_decode: null pointer");
+  auto aligned16 = [](const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
+  BH_REQUIRE(aligned16(in.qkv) && aligned16(in.inv_freq) && aligned16(in.rope_table) &&
+                 aligned16(in.kcache) && aligned16(in.vcache),
+             "attn_decode: qkv, inv_freq, the RoPE table and the caches must be 16-byte aligned");
   BH_REQUIRE(in.head_dim == kD, "attn_decode: head_dim %d (only %d is built)",
              in.head_dim, kD);
   BH_REQUIRE(in.kv_heads > 0 && in.heads % in.kv_heads == 0 &&

@@ -315,7 +315,9 @@ int buddy_hip_argmax(const float *x, int n, void *workspace, int *out_index,
  * and attends over rows 0..*pos.  out: [heads*head_dim].  lse: [heads] or NULL,
  * the op's second result, max + log(sum) of each head's scaled scores
  * (tosa.py:14576-14594).  head_dim must be 128.  *pos must lie in
- * 0..max_len-1; a position outside writes no cache row. */
+ * 0..max_len-1; a position outside writes no cache row.  qkv, inv_freq and the
+ * caches must be 16-byte aligned (the kernels read them four floats at a time);
+ * other addresses are refused. */
 size_t buddy_hip_attn_decode_workspace_bytes(int heads, int max_len);
 /* How the session cuts the attention of a decode step at position `pos` (host
  * arithmetic, no device needed): cache positions per partial (64, 128 or 256),

@@ -266,6 +266,22 @@ def test_standalone_elementwise_and_argmax(bh, oracle):
     assert int(out.item()) == 100 == oracle.argmax_first(v.cpu().numpy())
 
 
+def test_decode_attention_refuses_unaligned_operands(bh):
+    """The kernels read qkv, inv_freq and the caches four floats at a time."""
+    H, HKV, D, L = 4, 2, 128, 64
+    t = torch.zeros((H + 2 * HKV) * D + 2 * HKV * L * D + D + 8, device="cuda")
+    pos_t = torch.zeros(1, dtype=torch.int32, device="cuda")
+    nb = bh.buddy_hip_attn_decode_workspace_bytes(H, L)
+    ws = torch.empty(nb, dtype=torch.uint8, device="cuda")
+    out = torch.empty(H * D, device="cuda")
+    p = t.data_ptr()
+    for off in ((4, 0, 0), (0, 4, 0), (0, 0, 4)):
+        rc = bh.buddy_hip_gqa_decode_attention(
+            p + off[0], p + off[1], pos_t.data_ptr(), p + off[2], p, out.data_ptr(), None,
+            H, HKV, D, L, 0.088, ws.data_ptr(), nb, None)
+        assert rc == 1 and b"16-byte aligned" in bh.buddy_hip_last_error()
+
+
 @pytest.mark.parametrize("pos", [0, 8, 31, 32, 36, 612, 1023, 1087])
 def test_decode_attention_with_rope_and_kv_write(bh, oracle, pos):
     """valid lengths 9/37/613/1024 are the reference's own check points
