@@ -442,6 +442,29 @@ def test_small_model_steps_across_the_attention_chunk_sizes(oracle, start):
     sess.close()
 
 
+@pytest.mark.parametrize("heads,kv_heads", [(1, 1), (3, 1), (5, 1), (6, 1), (8, 1), (12, 2), (8, 4)])
+def test_long_context_steps_for_every_size_of_head_group(oracle, heads, kv_heads):
+    """From position 9216 on a workgroup takes all the query heads of a KV head, or,
+    where there are few KV heads, half of them (a group of 3 or 5 splits unevenly, a
+    group of one not at all): steps that cross that position against the oracle."""
+    start = 9210
+    shape = Shape(layers=1, hidden=256, heads=heads, kv_heads=kv_heads, head_dim=128, inter=256,
+                  vocab=512, max_len=9280, rms_eps=1e-6)
+    sess, host = synthetic.build_session(shape, context=start, keep_host=True, ln_jitter=0.1)
+    om = oracle_model(oracle, shape, host)
+    kv = [a.copy() for a in host["kv"]]
+    tok = 3
+    for step in range(12):
+        nxt, logits = sess.decode(tok, start + step)
+        otok, ologits = om.decode_step(tok, start + step, kv)
+        check_close(logits, ologits)
+        assert nxt == otok
+        tok = otok
+    for j in range(2):
+        check_close(sess.get_kv(j)[:, start:start + 12, :], kv[j][:, start:start + 12, :])
+    sess.close()
+
+
 def test_small_model_greedy_feedback_matches_stepwise(oracle):
     sess, host = synthetic.build_session(SMALL, context=16, keep_host=True, ln_jitter=0.1)
     toks = sess.decode_greedy(5, 16, 24)
