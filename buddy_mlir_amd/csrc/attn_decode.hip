@@ -73,10 +73,17 @@ __global__ void __launch_bounds__(kWaves * 64) attn_decode_partial(AttnArgs a) {
 
   const int tid = threadIdx.x;
   const int wave = tid >> 6, lane = tid & 63;
-  const int hb = blockIdx.x / a.pairs_padded, ckv = blockIdx.x % a.pairs_padded;
-  if (ckv >= a.used * a.kv_heads)
+  // grid (pairs_padded, group): the workgroups of a (chunk, KV head) pair have
+  // linear ids equal modulo 8.  No division ahead of the first load: a pair's KV
+  // head is found by counting (there are few)
+  const int hb = blockIdx.y;
+  int chunk = blockIdx.x, kvh = 0;
+  if (chunk >= a.used * a.kv_heads)
     return; // padding id
-  const int chunk = ckv % a.used, kvh = ckv / a.used;
+  while (chunk >= a.used) {
+    chunk -= a.used;
+    ++kvh;
+  }
   const int p0 = chunk * kChunk;
   const int h = kvh * a.group + hb; // this workgroup's query head
 
@@ -253,12 +260,18 @@ __global__ void __launch_bounds__(kWaves * 64) attn_decode_partial_group(AttnArg
 
   const int tid = threadIdx.x;
   const int wave = tid >> 6, lane = tid & 63;
-  const int ckv = blockIdx.x / a.head_split, hs = blockIdx.x % a.head_split;
-  if (ckv >= a.used * a.kv_heads)
+  // grid (pairs_padded, head_split): the workgroups that share a (chunk, KV head)
+  // pair have linear ids equal modulo 8 -- one XCD, one L2 for the pair's rows
+  const int hs = blockIdx.y;
+  int chunk = blockIdx.x, kvh = 0;
+  if (chunk >= a.used * a.kv_heads)
     return; // padding id
-  const int chunk = ckv % a.used, kvh = ckv / a.used;
-  // this workgroup's share of the group's query heads
-  const int per = (a.group + a.head_split - 1) / a.head_split;
+  while (chunk >= a.used) { // no division ahead of the first load
+    chunk -= a.used;
+    ++kvh;
+  }
+  // this workgroup's share of the group's query heads (head_split is 1 or 2)
+  const int per = (a.group + a.head_split - 1) >> (a.head_split - 1);
   const int h_lo = hs * per, h_hi = min(a.group, h_lo + per);
   const int p0 = chunk * kChunk;
   const int c4 = lane & 31, par = lane >> 5;
@@ -617,7 +630,7 @@ int launch_attn_decode(const AttnDecodeArgs &in, hipStream_t stream) {
     BH_REQUIRE(in.head_split == 1 || in.head_split == 2, "attn_decode: head_split %d",
                in.head_split);
     a.head_split = std::min(in.head_split, a.group); // a group of one head has nothing to share out
-    const dim3 grid(a.used * in.kv_heads * a.head_split);
+    const dim3 grid(a.pairs_padded, a.head_split);
     const size_t lds = sizeof(float) * (size_t)a.group * (in.chunk / kPW) * kD; // <= 64 KiB
     if (in.chunk == 64) {
       hipLaunchKernelGGL(attn_decode_partial_group<4>, grid, dim3(4 * 64), lds, stream, a);
@@ -635,7 +648,7 @@ int launch_attn_decode(const AttnDecodeArgs &in, hipStream_t stream) {
     BH_CHECK_HIP(hipGetLastError());
     return BUDDY_HIP_OK;
   }
-  const dim3 grid(a.pairs_padded * a.group);
+  const dim3 grid(a.pairs_padded, a.group);
   if (in.chunk == 64)
     hipLaunchKernelGGL(attn_decode_partial<4>, grid, dim3(4 * 64), 0, stream, a);
   else if (in.chunk == 128)

@@ -101,7 +101,14 @@ template <typename Family, int... P> struct Variant {
 inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 inline int64_t round_up(int64_t a, int64_t b) { return ceil_div(a, b) * b; }
 
+// The k-slices per channel group are a power of two (the planners only double or
+// halve them), so a wavefront finds its slice with a shift and a mask instead of
+// the forty-odd scalar instructions of a division ahead of its first load.
+inline bool is_pow2(int v) { return v > 0 && (v & (v - 1)) == 0; }
+
 #if defined(__HIPCC__)
+__device__ __forceinline__ int shift_of(int pow2) { return __builtin_ctz((unsigned)pow2); }
+
 // One-instruction transcendental forms (v_exp_f32, v_rcp_f32, v_rsq_f32: 1 ulp)
 // for the epilogues of the decode kernels, where a single wavefront finishes a
 // tile alone and the library routines' twenty-odd dependent instructions each

@@ -78,10 +78,11 @@ __global__ void __launch_bounds__(kFastMaxWaves *kWave)
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
   const int nwaves = a.G * a.KS;
-  const int gl = wave / a.KS, ks = wave % a.KS;
+  const int ksh = shift_of(a.KS);
+  const int gl = wave >> ksh, ks = wave & (a.KS - 1);
   const int g = blockIdx.x * a.G + gl;
   const bool live = g < a.groups;
-  const int per = (a.chunks + a.KS - 1) / a.KS;
+  const int per = (a.chunks + a.KS - 1) >> ksh;
   const int t0 = min(ks * per, a.chunks), t1 = min(t0 + per, a.chunks);
   const int4 *w = a.W + ((size_t)(live ? g : 0) * a.chunks) * 64 + lane;
   const int n = g * kTileN + lane;
@@ -259,6 +260,7 @@ pack_w4_tiles_kernel(const int8_t *__restrict__ packed, int K, int N, int chunks
 }
 
 template <int U> int launch_fast(const FastArgs &a, unsigned blocks, size_t lds, hipStream_t s) {
+  BH_REQUIRE(is_pow2(a.KS), "w4a16: %d k-slices (the kernel shifts by their count)", a.KS);
   hipLaunchKernelGGL(w4a16_fast_kernel<U>, dim3(blocks), dim3(a.G * a.KS * kWave), lds, s, a.A,
                      a.W, a.scale, a.C, a.K, a.N, a.groups, a.chunks, a.G, a.KS);
   BH_CHECK_HIP(hipGetLastError());

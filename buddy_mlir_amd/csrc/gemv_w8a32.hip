@@ -248,7 +248,7 @@ __device__ __forceinline__ void emit_group_maximum(const KernelArgs &a, int g, i
 // time so that their loads are in flight together).
 __device__ __forceinline__ float4 attn_combined(const KernelArgs &a, int k) {
   constexpr int B = 9; // partials fetched per batch (two batches at 18 chunks)
-  const int h = k / a.head_dim, d = k % a.head_dim;
+  const int h = k >> shift_of(a.head_dim), d = k & (a.head_dim - 1); // a power of two
   // every chunk the launch was given is folded: the ones beyond the position
   // hold (m, l, acc) = (-1e30, 0, 0) and drop out with weight exp(-1e30 - m) = 0,
   // so the loop does not have to wait for the position
@@ -309,11 +309,12 @@ __global__ void __launch_bounds__(kMaxWaves *kWave)
   const int tid = threadIdx.x;
   const int wave = tid >> 6, lane = tid & 63;
   const int nwaves = a.G * a.KS;
-  const int gl = wave / a.KS, ks = wave % a.KS;
+  const int ksh = shift_of(a.KS);
+  const int gl = wave >> ksh, ks = wave & (a.KS - 1);
   const int g = blockIdx.x * a.G + gl;
   const bool live = g < a.groups;
   // this wavefront's contiguous run of tiles
-  const int per = (a.chunks + a.KS - 1) / a.KS;
+  const int per = (a.chunks + a.KS - 1) >> ksh;
   const int t0 = min(ks * per, a.chunks);
   const int t1 = min(t0 + per, a.chunks);
   const int TR = a.tiles_per_round;
@@ -630,7 +631,8 @@ __device__ __forceinline__ void attn_fold_tiles(const KernelArgs &a, int t0, int
   for (int u = 0; u < U; ++u) {
     const int t = min(t0 + u, t1 - 1); // slots past the run repeat its last tile
     const int k = min(t * kTileK + lane, a.K - 1);
-    const int h = __builtin_amdgcn_readfirstlane(k / a.head_dim), d = k % a.head_dim;
+    const int h = __builtin_amdgcn_readfirstlane(k >> shift_of(a.head_dim)),
+              d = k & (a.head_dim - 1); // a power of two
     ml[u] = reinterpret_cast<const float2 *>(a.attn_ml) + (size_t)h * a.attn_nchunks;
     acc[u] = a.attn_acc + (size_t)h * a.attn_nchunks * a.head_dim + d;
     r[u] = 0.f;
@@ -775,11 +777,12 @@ __global__ void __launch_bounds__(kMaxWaves *kWave)
   extern __shared__ float lds[]; // only the meeting place of the k-slices
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
-  const int gl = wave / a.KS, ks = wave % a.KS;
+  const int ksh = shift_of(a.KS);
+  const int gl = wave >> ksh, ks = wave & (a.KS - 1);
   const int gi = blockIdx.x * a.G + gl;
   const int g = gi >> hs, half = gi & hs;
   const bool live = g < a.groups;
-  const int per = (a.chunks + a.KS - 1) / a.KS;
+  const int per = (a.chunks + a.KS - 1) >> ksh;
   const int t0 = min(ks * per, a.chunks);
   const int t1 = min(t0 + per, a.chunks);
 
@@ -999,11 +1002,12 @@ __global__ void __launch_bounds__(kMaxWaves *kWave)
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
   const int nwaves = a.G * a.KS;
-  const int gl = wave / a.KS, ks = wave % a.KS;
+  const int ksh = shift_of(a.KS);
+  const int gl = wave >> ksh, ks = wave & (a.KS - 1);
   const int gi = blockIdx.x * a.G + gl;
   const int g = gi >> hs, half = gi & hs;
   const bool live = g < a.groups;
-  const int per = (a.chunks + a.KS - 1) / a.KS;
+  const int per = (a.chunks + a.KS - 1) >> ksh;
   const int t0 = min(ks * per, a.chunks);
   const int t1 = min(t0 + per, a.chunks);
 
@@ -1572,7 +1576,8 @@ int launch_gemv(const GemvArgs &a, hipStream_t stream) {
   BH_REQUIRE((a.A || a.attn_acc) && a.W0 && a.s0 && a.C, "gemv: null pointer");
   BH_REQUIRE(!a.attn_acc || (a.attn_ml && a.pos_ptr && a.attn_nchunks > 0 &&
                              a.attn_chunk > 0 && a.head_dim > 0 &&
-                             a.head_dim % 4 == 0 && a.K % a.head_dim == 0),
+                             a.head_dim % 4 == 0 && is_pow2(a.head_dim) &&
+                             a.K % a.head_dim == 0),
              "gemv: incomplete attention-partials input");
   BH_REQUIRE(a.M >= 1 && a.M <= 16, "gemv: M=%d outside 1..16", a.M);
   BH_REQUIRE(a.K > 0 && a.N > 0 && a.K < (1 << 30) && a.N < (1 << 30),
@@ -1629,6 +1634,7 @@ int launch_gemv(const GemvArgs &a, hipStream_t stream) {
   ka.groups = (int)p.groups;
   ka.chunks = (int)p.chunks;
   ka.G = p.G;
+  BH_REQUIRE(is_pow2(p.KS), "gemv: %d k-slices (the kernels shift by their count)", p.KS);
   ka.KS = p.KS;
   ka.tiles_per_round = p.tiles_per_round;
   ka.tile_n = a.tile_n;

@@ -219,7 +219,8 @@ __global__ void __launch_bounds__(kMaxWavesI8 *kWave, 3) // 3 wavefronts per SIM
   extern __shared__ __attribute__((aligned(16))) float red[];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int sl = wave / a.KS, ks = wave % a.KS;
+  const int ksh = shift_of(a.KS);
+  const int sl = wave >> ksh, ks = wave & (a.KS - 1);
   const int row_half = a.row_split ? blockIdx.x & 1 : 0;
   if (a.row_split) { // this workgroup's rows: the first eight or the rest
     a.A += (int64_t)row_half * 8 * a.lda;
@@ -232,7 +233,7 @@ __global__ void __launch_bounds__(kMaxWavesI8 *kWave, 3) // 3 wavefronts per SIM
   // what a wavefront's slice is cut from and a fetch brings: chunks, or pairs of
   // chunks with T2
   const int units = T2 ? (a.chunks + 1) / 2 : a.chunks;
-  const int per = (units + a.KS - 1) / a.KS;
+  const int per = (units + a.KS - 1) >> ksh;
   const int c0 = min(ks * per, units), c1 = min(c0 + per, units);
   const int kg = lane >> 4;
   const int col = lane & 15;          // column of the activation operand
@@ -566,6 +567,7 @@ int launch_kernel(I8Args ka, int ks_forced, hipStream_t stream) {
   }
   if (ks_forced)
     ks = ks_forced;
+  BH_REQUIRE(is_pow2(ks), "gemv: %d k-slices (the kernels shift by their count)", ks);
   ka.KS = ks;
   ka.GS = ks < 4 ? 4 / ks : 1;
   const int waves = ka.GS * ka.KS;

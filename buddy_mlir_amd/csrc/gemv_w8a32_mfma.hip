@@ -201,11 +201,12 @@ __global__ void __launch_bounds__(kMaxWavesMfma *kWave)
   extern __shared__ __attribute__((aligned(16))) float red[];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int sl = wave / a.KS, ks = wave % a.KS;
+  const int ksh = shift_of(a.KS);
+  const int sl = wave >> ksh, ks = wave & (a.KS - 1);
   const int span = blockIdx.x * a.GS + sl;
   const bool live = span < a.spans;
   const int g0 = (live ? span : 0) * SPAN;
-  const int per = (a.chunks + a.KS - 1) / a.KS;
+  const int per = (a.chunks + a.KS - 1) >> ksh;
   const int c0 = min(ks * per, a.chunks), c1 = min(c0 + per, a.chunks);
   const int m = lane & 15, kg = lane >> 4;
 
@@ -452,6 +453,7 @@ int launch_gemv_mfma(const GemvArgs &a, hipStream_t stream) {
   const int ks_max = dual && span == 4 ? 8 : kMaxWavesMfma;
   while (ks < ks_max && (int64_t)ka.spans * ks < 2048 && ka.chunks / (ks * 2) >= 2)
     ks *= 2;
+  BH_REQUIRE(is_pow2(ks), "gemv: %d k-slices (the kernels shift by their count)", ks);
   ka.KS = ks;
   ka.GS = ks < 4 ? 4 / ks : 1;
   const int blocks = (int)ceil_div(ka.spans, ka.GS);
