@@ -60,12 +60,34 @@ struct AttnArgs {
 // The step is latency bound, so the kernel is built to have almost nothing
 // behind the arrival of its K/V rows: the small operands (q, the token's own
 // k and v, the RoPE table) are requested first, the K/V rows right behind
-// them, and q is rotated into LDS while the rows are still on their way -- the
-// one barrier before the merge.  Each of the wavefronts then handles 16
-// positions entirely on its own (scores, its own max / exp / sum, its share of
-// P.V) in registers and cross-lane operations, and they meet once in LDS.
+// them, and every lane rotates its own four dims of q in registers.  Each of the
+// wavefronts then handles 16 positions entirely on its own (scores, its own
+// max / exp / sum, its share of P.V) in registers and cross-lane operations, and
+// they meet once in LDS.
+//
+// What a wavefront needs before its first load -- five pointers and four
+// integers, 14 argument words -- are separate leading parameters: this file is
+// built with -amdgpu-kernarg-preload-count=14, so they arrive in SGPRs and the
+// loads do not wait for a scalar load of the argument block.
+__host__ __device__ constexpr int pack_heads(int heads, int kv_heads, int group) {
+  return heads | kv_heads << 12 | group << 24; // heads, kv_heads < 4096, group <= 8
+}
 template <int kWaves>
-__global__ void __launch_bounds__(kWaves * 64) attn_decode_partial(AttnArgs a) {
+__global__ void __launch_bounds__(kWaves * 64)
+    attn_decode_partial(const float *p_qkv, float *p_kcache, float *p_vcache,
+                        const float *p_rope_table, const int *p_pos, int p_used, int p_max_len,
+                        int p_heads, int p_unused, AttnArgs rest) {
+  AttnArgs a = rest;
+  a.qkv = p_qkv;
+  a.kcache = p_kcache;
+  a.vcache = p_vcache;
+  a.rope_table = p_rope_table;
+  a.pos_ptr = p_pos;
+  a.used = p_used;
+  a.max_len = p_max_len;
+  a.heads = p_heads & 0xfff;
+  a.kv_heads = (p_heads >> 12) & 0xfff;
+  a.group = p_heads >> 24;
   constexpr int kChunk = kWaves * kPW; // cache positions per workgroup: 64, 128 or 256
   constexpr int kR = kPW / 2;          // rows per lane: 8
   __shared__ __attribute__((aligned(16))) float accw_s[kWaves][kD];
@@ -250,7 +272,22 @@ __global__ void __launch_bounds__(kWaves * 64) attn_decode_partial(AttnArgs a) {
 // waits for: one workgroup takes all the query heads of a KV head, so that a K/V
 // row is loaded once and multiplied with every head's query.
 template <int kWaves>
-__global__ void __launch_bounds__(kWaves * 64) attn_decode_partial_group(AttnArgs a) {
+__global__ void __launch_bounds__(kWaves * 64)
+    attn_decode_partial_group(const float *p_qkv, float *p_kcache, float *p_vcache,
+                              const float *p_rope_table, const int *p_pos, int p_used,
+                              int p_max_len, int p_heads, int p_head_split, AttnArgs rest) {
+  AttnArgs a = rest; // the leading parameters arrive in SGPRs (see attn_decode_partial)
+  a.qkv = p_qkv;
+  a.kcache = p_kcache;
+  a.vcache = p_vcache;
+  a.rope_table = p_rope_table;
+  a.pos_ptr = p_pos;
+  a.used = p_used;
+  a.max_len = p_max_len;
+  a.heads = p_heads & 0xfff;
+  a.kv_heads = (p_heads >> 12) & 0xfff;
+  a.group = p_heads >> 24;
+  a.head_split = p_head_split;
   constexpr int kChunk = kWaves * kPW;
   constexpr int kR = kPW / 2;
   __shared__ __attribute__((aligned(16))) float q_s[kMaxGroup][kD], knew_s[kD], vnew_s[kD];
@@ -631,30 +668,43 @@ int launch_attn_decode(const AttnDecodeArgs &in, hipStream_t stream) {
                in.head_split);
     a.head_split = std::min(in.head_split, a.group); // a group of one head has nothing to share out
     const dim3 grid(a.pairs_padded, a.head_split);
+    BH_REQUIRE(in.heads < 4096, "attn_decode: %d heads", in.heads);
+    const int hp = pack_heads(a.heads, a.kv_heads, a.group);
     const size_t lds = sizeof(float) * (size_t)a.group * (in.chunk / kPW) * kD; // <= 64 KiB
     if (in.chunk == 64) {
-      hipLaunchKernelGGL(attn_decode_partial_group<4>, grid, dim3(4 * 64), lds, stream, a);
+      hipLaunchKernelGGL(attn_decode_partial_group<4>, grid, dim3(4 * 64), lds, stream, a.qkv,
+                         a.kcache, a.vcache, a.rope_table, a.pos_ptr, a.used, a.max_len, hp,
+                         a.head_split, a);
     } else if (in.chunk == 128) {
-      hipLaunchKernelGGL(attn_decode_partial_group<8>, grid, dim3(8 * 64), lds, stream, a);
+      hipLaunchKernelGGL(attn_decode_partial_group<8>, grid, dim3(8 * 64), lds, stream, a.qkv,
+                         a.kcache, a.vcache, a.rope_table, a.pos_ptr, a.used, a.max_len, hp,
+                         a.head_split, a);
     } else {
       // with 8 heads per KV head the 64 KiB of dynamic LDS come on top of 6 KiB
       static DynLdsOnce dyn_lds;
       BH_CHECK_HIP(ensure_dyn_lds(dyn_lds,
                                   reinterpret_cast<const void *>(attn_decode_partial_group<16>),
                                   (int)(sizeof(float) * kMaxGroup * 16 * kD)));
-      hipLaunchKernelGGL(attn_decode_partial_group<16>, grid, dim3(16 * 64), lds, stream, a);
+      hipLaunchKernelGGL(attn_decode_partial_group<16>, grid, dim3(16 * 64), lds, stream, a.qkv,
+                         a.kcache, a.vcache, a.rope_table, a.pos_ptr, a.used, a.max_len, hp,
+                         a.head_split, a);
     }
     hipLaunchKernelGGL(attn_decode_combine_wide, dim3(in.heads), dim3(1024), 0, stream, a);
     BH_CHECK_HIP(hipGetLastError());
     return BUDDY_HIP_OK;
   }
   const dim3 grid(a.pairs_padded, a.group);
+  BH_REQUIRE(in.heads < 4096, "attn_decode: %d heads", in.heads);
+  const int hp = pack_heads(a.heads, a.kv_heads, a.group);
   if (in.chunk == 64)
-    hipLaunchKernelGGL(attn_decode_partial<4>, grid, dim3(4 * 64), 0, stream, a);
+    hipLaunchKernelGGL(attn_decode_partial<4>, grid, dim3(4 * 64), 0, stream, a.qkv, a.kcache,
+                       a.vcache, a.rope_table, a.pos_ptr, a.used, a.max_len, hp, 0, a);
   else if (in.chunk == 128)
-    hipLaunchKernelGGL(attn_decode_partial<8>, grid, dim3(8 * 64), 0, stream, a);
+    hipLaunchKernelGGL(attn_decode_partial<8>, grid, dim3(8 * 64), 0, stream, a.qkv, a.kcache,
+                       a.vcache, a.rope_table, a.pos_ptr, a.used, a.max_len, hp, 0, a);
   else
-    hipLaunchKernelGGL(attn_decode_partial<16>, grid, dim3(16 * 64), 0, stream, a);
+    hipLaunchKernelGGL(attn_decode_partial<16>, grid, dim3(16 * 64), 0, stream, a.qkv, a.kcache,
+                       a.vcache, a.rope_table, a.pos_ptr, a.used, a.max_len, hp, 0, a);
   if (in.combine && in.wide_combine)
     hipLaunchKernelGGL(attn_decode_combine_wide, dim3(in.heads), dim3(1024), 0, stream, a);
   else if (in.combine)
