@@ -495,40 +495,66 @@ __global__ void __launch_bounds__(kD) attn_decode_combine(AttnArgs a) {
 // sums are those of the chunk-by-chunk rule in another order.
 constexpr int kWideChunks = kAttnWideChunks; // partials per head it takes
 
-__global__ void __launch_bounds__(1024) attn_decode_combine_wide(AttnArgs a) {
+__global__ void __launch_bounds__(1024)
+    attn_decode_combine_wide(const float *p_acc, const float *p_ml, float *p_out, int p_nchunks,
+                             int p_used) { // (arguments preloaded into SGPRs)
   constexpr int kPer = kWideChunks / 32; // chunks per thread at most
+  constexpr int kFast = 4;               // passes of 64 chunks whose (max, sum) pairs stay in registers
   __shared__ float w_s[kWideChunks];
   __shared__ __attribute__((aligned(16))) float4 red_s[32][32];
   const int h = blockIdx.x, tid = threadIdx.x, lane = tid & 63;
   const int q = tid & 31, g = tid >> 5;
-  const int used = a.used;
-  const float2 *ml = reinterpret_cast<const float2 *>(a.part_ml) + (size_t)h * a.nchunks;
-  const float *acc = a.part_acc + (size_t)h * a.nchunks * kD + q * 4;
-  // the partial sums of this thread's chunks, requested before anything is known
-  // of their weights (chunks past the last repeat it and are not added)
+  const int used = p_used;
+  const float2 *ml = reinterpret_cast<const float2 *>(p_ml) + (size_t)h * p_nchunks;
+  const float *acc = p_acc + (size_t)h * p_nchunks * kD + q * 4;
+  // the partial sums of this thread's first four chunks and the (max, sum) pairs
+  // are requested together, before anything is known of the weights: one trip
+  // (chunks past the last repeat it and are not added)
   float4 v[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+    v[i] = *reinterpret_cast<const float4 *>(acc + (size_t)min(g + 32 * i, used - 1) * kD);
   float4 sum = make_float4(0.f, 0.f, 0.f, 0.f);
   // the weights: every wavefront computes all of them (64 chunks per pass) and
   // wavefront 0 leaves them in LDS
-  float m_all = kSeedM;
-  for (int s0 = 0; s0 < used; s0 += 64)
-    m_all = fmaxf(m_all, wave_max(s0 + lane < used ? ml[s0 + lane].x : kSeedM));
-  float l_all = 0.f;
-  for (int s0 = 0; s0 < used; s0 += 64) {
-    const bool in = s0 + lane < used;
-    const float2 mine = ml[min(s0 + lane, used - 1)];
-    const float w = in ? fast_exp(mine.x - m_all) : 0.f;
-    l_all += wave_sum(mine.y * w);
-    if (tid < 64 && in)
-      w_s[s0 + lane] = w;
+  float m_all = kSeedM, l_all = 0.f;
+  if (used <= 64 * kFast) {
+    float2 mine[kFast];
+#pragma unroll
+    for (int p = 0; p < kFast; ++p)
+      mine[p] = ml[min(64 * p + lane, used - 1)];
+#pragma unroll
+    for (int p = 0; p < kFast; ++p)
+      m_all = fmaxf(m_all, wave_max(64 * p + lane < used ? mine[p].x : kSeedM));
+#pragma unroll
+    for (int p = 0; p < kFast; ++p) {
+      const bool in = 64 * p + lane < used;
+      const float w = in ? fast_exp(mine[p].x - m_all) : 0.f;
+      l_all += wave_sum(mine[p].y * w);
+      if (tid < 64 && in)
+        w_s[64 * p + lane] = w;
+    }
+  } else {
+    for (int s0 = 0; s0 < used; s0 += 64)
+      m_all = fmaxf(m_all, wave_max(s0 + lane < used ? ml[s0 + lane].x : kSeedM));
+    for (int s0 = 0; s0 < used; s0 += 64) {
+      const bool in = s0 + lane < used;
+      const float2 mine = ml[min(s0 + lane, used - 1)];
+      const float w = in ? fast_exp(mine.x - m_all) : 0.f;
+      l_all += wave_sum(mine.y * w);
+      if (tid < 64 && in)
+        w_s[s0 + lane] = w;
+    }
   }
   __syncthreads();
   for (int i0 = 0; i0 < kPer; i0 += 4) {
     if (g + 32 * i0 >= used)
       break;
+    if (i0 > 0) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
-      v[i] = *reinterpret_cast<const float4 *>(acc + (size_t)min(g + 32 * (i0 + i), used - 1) * kD);
+      for (int i = 0; i < 4; ++i)
+        v[i] = *reinterpret_cast<const float4 *>(acc + (size_t)min(g + 32 * (i0 + i), used - 1) * kD);
+    }
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int c = g + 32 * (i0 + i);
@@ -551,7 +577,7 @@ __global__ void __launch_bounds__(1024) attn_decode_combine_wide(AttnArgs a) {
       o.x += r.x; o.y += r.y; o.z += r.z; o.w += r.w;
     }
     const float inv = 1.0f / l_all;
-    *reinterpret_cast<float4 *>(a.out + (size_t)h * kD + tid * 4) =
+    *reinterpret_cast<float4 *>(p_out + (size_t)h * kD + tid * 4) =
         make_float4(o.x * inv, o.y * inv, o.z * inv, o.w * inv);
   }
 }
@@ -689,7 +715,8 @@ int launch_attn_decode(const AttnDecodeArgs &in, hipStream_t stream) {
                          a.kcache, a.vcache, a.rope_table, a.pos_ptr, a.used, a.max_len, hp,
                          a.head_split, a);
     }
-    hipLaunchKernelGGL(attn_decode_combine_wide, dim3(in.heads), dim3(1024), 0, stream, a);
+    hipLaunchKernelGGL(attn_decode_combine_wide, dim3(in.heads), dim3(1024), 0, stream, a.part_acc,
+                       a.part_ml, a.out, a.nchunks, a.used);
     BH_CHECK_HIP(hipGetLastError());
     return BUDDY_HIP_OK;
   }
@@ -706,7 +733,8 @@ int launch_attn_decode(const AttnDecodeArgs &in, hipStream_t stream) {
     hipLaunchKernelGGL(attn_decode_partial<16>, grid, dim3(16 * 64), 0, stream, a.qkv, a.kcache,
                        a.vcache, a.rope_table, a.pos_ptr, a.used, a.max_len, hp, 0, a);
   if (in.combine && in.wide_combine)
-    hipLaunchKernelGGL(attn_decode_combine_wide, dim3(in.heads), dim3(1024), 0, stream, a);
+    hipLaunchKernelGGL(attn_decode_combine_wide, dim3(in.heads), dim3(1024), 0, stream, a.part_acc,
+                       a.part_ml, a.out, a.nchunks, a.used);
   else if (in.combine)
     hipLaunchKernelGGL(attn_decode_combine, dim3(in.heads), dim3(kD), 0, stream, a);
   BH_CHECK_HIP(hipGetLastError());
