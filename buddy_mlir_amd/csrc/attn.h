@@ -6,15 +6,15 @@
 namespace bh {
 
 constexpr int kAttnChunk = 64; // cache positions per flash-decoding partial (the default)
-// How a decode step at position `pos` cuts its attention.  The o_proj launch
-// folds up to 36 partials per head in one trip to memory (18 at its best):
-// chunks of 64 positions up to position 1152, 128 up to 2304, 256 up to 9216 (8
-// or 16 wavefronts of 16 positions per workgroup).  Beyond that the partials are
-// folded by a launch of their own and one workgroup takes all the query heads of
-// a KV head (a K/V row then leaves L2 once, not once per head); its chunks are
-// the largest that still give the launch about 200 workgroups.  Attention and
-// fold cover only the chunks up to the position, in batches of 18, whatever the
-// cache's capacity.
+// How a decode step at position `pos` cuts its attention.  Up to position 5120
+// the o_proj launch folds the partials, up to 36 per head in one trip to memory
+// (18 at its best): chunks of 64 positions up to position 1152, 128 up to 2304,
+// 256 beyond (8 or 16 wavefronts of 16 positions per workgroup).  From 5120 on
+// (where those launches would outgrow one workgroup per compute unit) the
+// partials are folded by a launch of their own and one workgroup takes all the
+// query heads of a KV head, or half of them (a K/V row then leaves L2 once or
+// twice, not once per head).  Attention and fold cover only the chunks up to the
+// position, in batches of 18, whatever the cache's capacity.
 struct AttnStepPlan {
   int chunk;     // cache positions per partial: 64, 128 or 256
   int used;      // partials per head the step produces and folds
@@ -24,21 +24,20 @@ struct AttnStepPlan {
 inline AttnStepPlan attn_step_plan(int pos, int max_len, int kv_heads) {
   AttnStepPlan p;
   p.head_split = 1;
-  p.own_fold = pos >= 36 * 256;
+  p.own_fold = pos >= 20 * 256;
   if (!p.own_fold) {
     p.chunk = pos < 18 * 64 ? 64 : pos < 18 * 128 ? 128 : 256;
   } else {
-    // Whole head groups on the largest chunks that still give ~200 workgroups; where that
-    // would take chunks of 64, chunks of 128 with half a head group per workgroup instead
-    // (measured: 128 x 2 beats 64 x 1, and 128 x 1 beats 256 x 2).
-    p.chunk = 128;
-    p.head_split = 2;
-    for (int c : {256, 128})
-      if ((pos / c + 1) * kv_heads >= 192) {
-        p.chunk = c;
-        p.head_split = 1;
-        break;
-      }
+    // Measured on a 12-head, 2-KV-head model from 5 k to 32 k positions (ms per step
+    // for chunk x split): workgroups of 16 wavefronts (chunks of 256) must not
+    // outnumber the 256 compute units, and want at least ~150 of them busy.
+    const int n256 = (pos / 256 + 1) * kv_heads; // workgroups of whole head groups on chunks of 256
+    if (2 * n256 <= 256) {
+      p.chunk = n256 >= 100 ? 256 : 128; // 16 k: 1.005 (256 x 2) vs 1.027; 12 k: 0.986 (128 x 2) vs 0.995
+      p.head_split = 2;
+    } else {
+      p.chunk = 256; // 20 k: 1.138 (256 x 1) vs 1.159 (128 x 1); 17.5 k: 1.147 with 128 x 1
+    }
   }
   const int all = (max_len + p.chunk - 1) / p.chunk, need = pos / p.chunk + 1;
   const int batches = (need + 17) / 18;

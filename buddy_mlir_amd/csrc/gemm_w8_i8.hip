@@ -317,7 +317,22 @@ __device__ __forceinline__ void load_chunk(const v4i32 *const (&wp)[kSplitGroups
 // 64 rows x 64 channels per workgroup; the four wavefronts split K and meet in
 // LDS in slice order.
 template <int D>
-__global__ void __launch_bounds__(kSlices *kWave) gemm_w8_i8_kernel(GemmI8Args a) {
+__global__ void __launch_bounds__(kSlices *kWave) gemm_w8_i8_kernel(
+    const int8_t *p_planes, const int4 *p_W, int p_Mp, int p_Kp, int p_groups, int p_chunks,
+    int p_ncols, int p_cols_padded, int p_slices, int p_chunks_per_slice, GemmI8Args rest) {
+  // what a wavefront needs before its first fetch arrives in SGPRs (this file is
+  // built with -amdgpu-kernarg-preload-count); the rest is loaded behind the fetch
+  GemmI8Args a = rest;
+  a.planes = p_planes;
+  a.W = p_W;
+  a.Mp = p_Mp;
+  a.Kp = p_Kp;
+  a.groups = p_groups;
+  a.chunks = p_chunks;
+  a.ncols = p_ncols;
+  a.cols_padded = p_cols_padded;
+  a.slices = p_slices;
+  a.chunks_per_slice = p_chunks_per_slice;
   extern __shared__ __attribute__((aligned(16))) float red[]; // [slice][64][lane]
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -460,7 +475,22 @@ __device__ __forceinline__ void wait_loads(FetchRegs<D, GPW> &f) {
 // through LDS in the epilogue, so only half as much is stored and no launch
 // reads both results again.
 template <int D, int RB, int GPW, bool PAIR>
-__global__ void __launch_bounds__(kSlices *kWave) gemm_w8_i8_wide_kernel(GemmI8Args a) {
+__global__ void __launch_bounds__(kSlices *kWave) gemm_w8_i8_wide_kernel(
+    const int8_t *p_planes, const int4 *p_W, int p_Mp, int p_Kp, int p_groups, int p_chunks,
+    int p_ncols, int p_cols_padded, int p_slices, int p_chunks_per_slice, GemmI8Args rest) {
+  // what a wavefront needs before its first fetch arrives in SGPRs (this file is
+  // built with -amdgpu-kernarg-preload-count); the rest is loaded behind the fetch
+  GemmI8Args a = rest;
+  a.planes = p_planes;
+  a.W = p_W;
+  a.Mp = p_Mp;
+  a.Kp = p_Kp;
+  a.groups = p_groups;
+  a.chunks = p_chunks;
+  a.ncols = p_ncols;
+  a.cols_padded = p_cols_padded;
+  a.slices = p_slices;
+  a.chunks_per_slice = p_chunks_per_slice;
   constexpr int kRing = RingDepth<GPW>::value;
   constexpr int L = GPW + D; // loads per fetch
   // chunks per unrolled pass: a multiple of the ring, and an even number of
@@ -909,7 +939,9 @@ int launch_wide(const GemmI8Args &a, unsigned blocks, hipStream_t stream) {
                                 (int)lds));
   }
   BH_NOTE_VARIANT(WideFamily, D, RB, GPW, (int)PAIR);
-  hipLaunchKernelGGL(kernel, dim3(blocks), dim3(kSlices * kWave), lds, stream, a);
+  hipLaunchKernelGGL(kernel, dim3(blocks), dim3(kSlices * kWave), lds, stream, a.planes, a.W, a.Mp,
+                     a.Kp, a.groups, a.chunks, a.ncols, a.cols_padded, a.slices, a.chunks_per_slice,
+                     a);
   BH_CHECK_HIP(hipGetLastError());
   return BUDDY_HIP_OK;
 }
@@ -994,7 +1026,9 @@ template <int D> int launch_split(const GemmI8Args &a, unsigned blocks, hipStrea
   BH_CHECK_HIP(ensure_dyn_lds(dyn_lds, reinterpret_cast<const void *>(kernel),
                               (int)lds));
   BH_NOTE_VARIANT(SplitFamily, D);
-  hipLaunchKernelGGL(kernel, dim3(blocks), dim3(kSlices * kWave), lds, stream, a);
+  hipLaunchKernelGGL(kernel, dim3(blocks), dim3(kSlices * kWave), lds, stream, a.planes, a.W, a.Mp,
+                     a.Kp, a.groups, a.chunks, a.ncols, a.cols_padded, a.slices, a.chunks_per_slice,
+                     a);
   BH_CHECK_HIP(hipGetLastError());
   return BUDDY_HIP_OK;
 }

@@ -22,7 +22,8 @@ def test_partials_cover_the_position_and_fit(bh, kv_heads):
     rng = np.random.default_rng(kv_heads)
     cases = [(p, m) for m in (1, 64, 65, 1088, 1152, 1153, 4352, 9472, 32768, 131072, 262144, 1 << 20)
              for p in {0, m - 1, m // 2, min(m - 1, 1151), min(m - 1, 1152), min(m - 1, 2303),
-                       min(m - 1, 2304), min(m - 1, 9215), min(m - 1, 9216)}]
+                       min(m - 1, 2304), min(m - 1, 5119), min(m - 1, 5120), min(m - 1, 12544),
+                       min(m - 1, 16384)}]
     cases += [(int(p), int(m)) for m in rng.integers(1, 1 << 20, 300)
               for p in rng.integers(0, m, 3)]
     for pos, max_len in cases:

@@ -408,15 +408,16 @@ def test_small_model_decodes_at_long_context(oracle):
     sess.close()
 
 
-@pytest.mark.parametrize("start", [100, 1140, 2296, 4596, 9206, 12280, 24310])
+@pytest.mark.parametrize("start", [100, 1140, 2296, 4596, 5110, 12535, 16375])
 def test_small_model_steps_across_the_attention_chunk_sizes(oracle, start):
     """A step far into a long cache takes attention chunks of 128 or 256 positions
     (from positions 1152 and 2304 on), covers only the chunks up to its position,
-    and from position 9216 on folds the partials in a launch of its own instead of
+    and from position 5120 on folds the partials in a launch of its own instead of
     in the o_proj launch: greedy steps that cross each boundary, a short context
-    in a large cache, and the lengths at which the launches of all heads of a KV
-    head go from chunks of 64 to 128 and to 256 positions (12288, 24320), against
-    the oracle -- every step's logits and the token fed back on the device."""
+    in a large cache, and the positions at which the launches that take the heads
+    of a KV head together change their cut (12544 and 16384 with two KV
+    heads), against the oracle -- every step's logits and the token fed back on
+    the device."""
     shape = Shape(layers=2, hidden=256, heads=4, kv_heads=2, head_dim=128, inter=512,
                   vocab=1024, max_len=(start + 100 + 63) // 64 * 64 if start > 4400 else 4352,
                   rms_eps=1e-6)
@@ -444,12 +445,12 @@ def test_small_model_steps_across_the_attention_chunk_sizes(oracle, start):
 
 @pytest.mark.parametrize("heads,kv_heads", [(1, 1), (3, 1), (5, 1), (6, 1), (8, 1), (12, 2), (8, 4)])
 def test_long_context_steps_for_every_size_of_head_group(oracle, heads, kv_heads):
-    """From position 9216 on a workgroup takes all the query heads of a KV head, or,
+    """From position 5120 on a workgroup takes all the query heads of a KV head, or,
     where there are few KV heads, half of them (a group of 3 or 5 splits unevenly, a
     group of one not at all): steps that cross that position against the oracle."""
-    start = 9210
+    start = 5114
     shape = Shape(layers=1, hidden=256, heads=heads, kv_heads=kv_heads, head_dim=128, inter=256,
-                  vocab=512, max_len=9280, rms_eps=1e-6)
+                  vocab=512, max_len=5184, rms_eps=1e-6)
     sess, host = synthetic.build_session(shape, context=start, keep_host=True, ln_jitter=0.1)
     om = oracle_model(oracle, shape, host)
     kv = [a.copy() for a in host["kv"]]
