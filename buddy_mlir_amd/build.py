@@ -61,7 +61,8 @@ def _check_no_scratch(src: Path, remarks: str) -> None:
 # Files whose kernels take their leading pointer arguments preloaded into SGPRs
 # by the command processor (the count is in argument words).
 KERNARG_PRELOAD = {"gemv_w8a32.hip": 14, "gemv_w4a16_fast.hip": 14, "attn_decode.hip": 14,
-                   "elementwise.hip": 14, "gemm_w8_i8.hip": 14}
+                   "elementwise.hip": 14, "gemm_w8_i8.hip": 14,
+                   "attn_prefill.hip": 14}
 
 
 def _hipcc() -> str:

@@ -70,8 +70,24 @@ constexpr int lds_floats(int waves) { return kQFloats + waves * kSlotFloats + 2 
 // so the scores never leave the registers between the two products.
 template <int kAttnWaves>
 __global__ void __launch_bounds__(kAttnWaves *kWave) __attribute__((amdgpu_waves_per_eu(2, 2)))
-attn_prefill_kernel(PrefillArgs a) {
+attn_prefill_kernel(const float *p_k, const float *p_v, const float *p_mask, int64_t p_kv_stride,
+                    int p_group, int p_nqb, int p_q_len, int p_k_len, int p_q_offset,
+                    PrefillArgs rest) {
   static_assert(kAttnWaves == 4 || kAttnWaves == 8, "wavefronts per workgroup");
+  // what comes before the first fetch arrives in SGPRs (this file is built with
+  // -amdgpu-kernarg-preload-count); p_group carries the group size, whether the
+  // launch is paired and the multiplier that divides a head index by the group
+  PrefillArgs a = rest;
+  a.k = p_k;
+  a.v = p_v;
+  a.mask = p_mask;
+  a.kv_stride = p_kv_stride;
+  a.group = p_group & 0xfff;
+  a.paired = (p_group >> 12) & 1;
+  a.nqb = p_nqb;
+  a.q_len = p_q_len;
+  a.k_len = p_k_len;
+  a.q_offset = p_q_offset;
   extern __shared__ __attribute__((aligned(16))) float lds[];
   f32x4 *q_s = reinterpret_cast<f32x4 *>(lds);          // [2][8][64]: part, J, lane
   float *slot_s = lds + kQFloats;                  // [kAttnWaves][kSlotFloats]
@@ -81,7 +97,7 @@ attn_prefill_kernel(PrefillArgs a) {
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int h = blockIdx.x, kvh = h / a.group;
+  const int h = blockIdx.x, kvh = (int)(((unsigned)h * (unsigned)(p_group >> 13)) >> 16); // h / group
   const int qi = lane & 15, lg = lane >> 4; // query of this lane; lane group
   // part 0: query block blockIdx.y, part 1: its mirror image (the same block in
   // the middle of an odd number of blocks: then part 0 is empty)
@@ -419,13 +435,19 @@ int launch_attn_prefill(const AttnPrefillArgs &in, hipStream_t stream) {
   BH_REQUIRE(pairs <= 65535, "attn_prefill: q_len %d too long", in.q_len);
   constexpr int kComputeUnits = 256; // MI355X
   a.paired = (int64_t)in.heads * pairs <= kComputeUnits;
+  // group | paired << 12 | (65536 / group + 1) << 13: (h * multiplier) >> 16 == h / group
+  // while heads * group < 65536
+  BH_REQUIRE(a.group >= 1 && a.group < 4096 && (int64_t)in.heads * a.group < 65536,
+             "attn_prefill: heads=%d group=%d", in.heads, a.group);
+  const int gp = a.group | a.paired << 12 | (65536 / a.group + 1) << 13;
   if (a.paired) {
     static DynLdsOnce dyn_lds;
     BH_CHECK_HIP(ensure_dyn_lds(dyn_lds, reinterpret_cast<const void *>(attn_prefill_kernel<8>),
                                 (int)(lds_floats(8) * sizeof(float))));
     BH_NOTE_VARIANT(AttnPrefillFamily, 8);
     hipLaunchKernelGGL(attn_prefill_kernel<8>, dim3(in.heads, (unsigned)pairs), dim3(8 * kWave),
-                       lds_floats(8) * sizeof(float), stream, a);
+                       lds_floats(8) * sizeof(float), stream, a.k, a.v, a.mask, a.kv_stride, gp, a.nqb,
+                       a.q_len, a.k_len, a.q_offset, a);
   } else {
     BH_REQUIRE(a.nqb <= 65535, "attn_prefill: q_len %d too long", in.q_len);
     static DynLdsOnce dyn_lds;
@@ -433,7 +455,8 @@ int launch_attn_prefill(const AttnPrefillArgs &in, hipStream_t stream) {
                                 (int)(lds_floats(4) * sizeof(float))));
     BH_NOTE_VARIANT(AttnPrefillFamily, 4);
     hipLaunchKernelGGL(attn_prefill_kernel<4>, dim3(in.heads, (unsigned)a.nqb), dim3(4 * kWave),
-                       lds_floats(4) * sizeof(float), stream, a);
+                       lds_floats(4) * sizeof(float), stream, a.k, a.v, a.mask, a.kv_stride, gp, a.nqb,
+                       a.q_len, a.k_len, a.q_offset, a);
   }
   BH_CHECK_HIP(hipGetLastError());
   return BUDDY_HIP_OK;

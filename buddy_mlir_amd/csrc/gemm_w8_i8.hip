@@ -874,9 +874,16 @@ reduce_slices_i32_kernel(GemmI8Args a, int rb_per_tile, int gpw) {
 // rmsnorm_to_digits_kernel would read back from C): lds = [Kp2] cache of
 // row_to_digits, then [Kp2] the row.
 __global__ void __launch_bounds__(kRowThreads)
-reduce_slices_norm_kernel(GemmI8Args a, int rb_per_tile, int gpw,
+reduce_slices_norm_kernel(const float *p_partial, const float *p_steps, int p_N, int p_ncols,
+                          int p_slices, int rb_per_tile, int gpw, GemmI8Args rest,
                           const float *__restrict__ norm_w, float inv_n, float eps, int D,
                           int Mp2, int Kp2, int8_t *__restrict__ planes) {
+  GemmI8Args a = rest; // the leading parameters arrive in SGPRs, ahead of the first load
+  a.partial = const_cast<float *>(p_partial);
+  a.steps = p_steps;
+  a.N = p_N;
+  a.ncols = p_ncols;
+  a.slices = p_slices;
   __shared__ float red[kRowThreads / 64];
   extern __shared__ __attribute__((aligned(16))) float row_lds[];
   float *xrow = row_lds + Kp2;
@@ -1216,8 +1223,8 @@ int launch_gemm_w8_digits_d(const GemmW8Args &in, const void *planes, hipStream_
                                   (int)(2 * sizeof(float) * kRowCache)));
     }
     hipLaunchKernelGGL(reduce_slices_norm_kernel, dim3((unsigned)a.M), dim3(kRowThreads),
-                       row_lds, stream, a, best_rb,
-                       best_gpw, in.then_norm_w, 1.0f / (float)in.N, in.then_norm_eps,
+                       row_lds, stream, a.partial, a.steps, a.N, a.ncols, a.slices, best_rb,
+                       best_gpw, a, in.then_norm_w, 1.0f / (float)in.N, in.then_norm_eps,
                        in.digits, next.rows_padded, next.cols_padded,
                        static_cast<int8_t *>(in.then_norm_staged));
     BH_CHECK_HIP(hipGetLastError());
