@@ -58,11 +58,11 @@ def _check_no_scratch(src: Path, remarks: str) -> None:
             + "\n  ".join(bad))
 
 
-# Files whose kernels take their leading pointer arguments preloaded into SGPRs
-# by the command processor (the count is in argument words).
-KERNARG_PRELOAD = {"gemv_w8a32.hip": 14, "gemv_w4a16_fast.hip": 14, "attn_decode.hip": 14,
-                   "elementwise.hip": 14, "gemm_w8_i8.hip": 14,
-                   "attn_prefill.hip": 14}
+# Every kernel takes its leading scalar and pointer arguments preloaded into SGPRs by
+# the command processor (up to this many argument words; arguments behind a
+# struct passed by value are loaded as usual): a wavefront's first loads then do
+# not wait for a scalar load of the argument block.
+KERNARG_PRELOAD = 14
 
 
 def _hipcc() -> str:
@@ -89,8 +89,8 @@ def _compile(src: Path, force: bool) -> Path:
     cmd = [_hipcc(), *COMMON, "-x", "hip", "-c", str(src), "-o", str(obj)]
     if src.name in NO_SCRATCH:
         cmd.append("-Rpass-analysis=kernel-resource-usage")
-    if src.name in KERNARG_PRELOAD:
-        cmd += ["-mllvm", f"-amdgpu-kernarg-preload-count={KERNARG_PRELOAD[src.name]}"]
+    if src.suffix == ".hip":
+        cmd += ["-mllvm", f"-amdgpu-kernarg-preload-count={KERNARG_PRELOAD}"]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError(f"hipcc failed on {src.name}:\n{r.stdout}\n{r.stderr}")
