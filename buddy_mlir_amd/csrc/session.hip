@@ -236,9 +236,9 @@ struct Session {
       a.workspace = attn_ws;
       a.workspace_bytes = attn_ws_bytes;
       // o_proj folds the partials while staging its input -- up to the 36 it
-      // requests in one trip; beyond that (positions from 9216 on) every one of
-      // its workgroups would repeat a fold that outgrows the matrix, and a
-      // launch of its own folds them once
+      // requests in one trip; far into a long cache (the plan says from where)
+      // every one of its workgroups would repeat a fold that outgrows the
+      // matrix, and a launch of its own folds them once
       const bool own_fold = plan.own_fold;
       a.combine = own_fold;
       a.wide_combine = own_fold;
