@@ -14,7 +14,8 @@ constexpr int kAttnChunk = 64; // cache positions per flash-decoding partial (th
 // partials are folded by a launch of their own and one workgroup takes all the
 // query heads of a KV head, or half of them (a K/V row then leaves L2 once or
 // twice, not once per head).  Attention and fold cover only the chunks up to the
-// position, in batches of 18, whatever the cache's capacity.
+// position (rounded up to a multiple of four; 18 with chunks of 64), whatever the
+// cache's capacity.
 struct AttnStepPlan {
   int chunk;     // cache positions per partial: 64, 128 or 256
   int used;      // partials per head the step produces and folds
@@ -40,8 +41,13 @@ inline AttnStepPlan attn_step_plan(int pos, int max_len, int kv_heads) {
     }
   }
   const int all = (max_len + p.chunk - 1) / p.chunk, need = pos / p.chunk + 1;
-  const int batches = (need + 17) / 18;
-  p.used = batches * 18 < all ? batches * 18 : all;
+  // 18 for chunks of 64 (one captured step serves a cache of 1152 positions, and
+  // the fold's first trip takes 18 anyway); with larger chunks the next multiple
+  // of four: every chunk past the position costs workgroups that find nothing to do
+  int want = (need + 3) / 4 * 4;
+  if (need <= 18)
+    want = p.chunk == 64 || want > 18 ? 18 : want;
+  p.used = want < all ? want : all;
   return p;
 }
 // partials per head the fold of its own takes: 2^20 positions at 256 per chunk

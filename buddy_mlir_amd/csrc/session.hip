@@ -119,6 +119,7 @@ struct Session {
     hipGraphExec_t exec = nullptr;
   };
   std::map<std::pair<int, int>, StepGraph> graphs;
+  static constexpr size_t kMaxStepGraphs = 8;
   bool use_graph = true;
   std::vector<void *> owned;
   // prefill activations, grown on demand: rows = tokens per prefill call
@@ -571,7 +572,19 @@ struct Session {
     if (!use_graph) {
       rc = enqueue_step(plan);
     } else {
-      StepGraph &g = graphs[{plan.chunk * 4 + plan.head_split, plan.own_fold ? -plan.used : plan.used}];
+      // one captured step per cut of the attention; positions only move forward,
+      // so a session far into a long cache keeps the last few and lets the rest go
+      const std::pair<int, int> key{plan.chunk * 4 + plan.head_split,
+                                    plan.own_fold ? -plan.used : plan.used};
+      auto it = graphs.find(key);
+      if (it == graphs.end()) {
+        if (graphs.size() >= kMaxStepGraphs) {
+          BH_CHECK_HIP(hipStreamSynchronize(stream)); // a replay may still be running
+          drop_graph();
+        }
+        it = graphs.emplace(key, StepGraph{}).first;
+      }
+      StepGraph &g = it->second;
       if (!g.exec) {
         BH_CHECK_HIP(hipStreamBeginCapture(stream, hipStreamCaptureModeThreadLocal));
         rc = enqueue_step(plan);

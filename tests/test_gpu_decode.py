@@ -466,6 +466,23 @@ def test_long_context_steps_for_every_size_of_head_group(oracle, heads, kv_heads
     sess.close()
 
 
+def test_a_long_generation_outlives_the_captured_steps_it_keeps():
+    """A session keeps a captured step per cut of the attention and lets the oldest
+    go after eight: 5200 greedy steps from position 5000 pass more cuts than that
+    (a new one every 512 positions), and must give the tokens of the same steps
+    launched one by one without a graph."""
+    shape = Shape(layers=1, hidden=256, heads=4, kv_heads=2, head_dim=128, inter=256,
+                  vocab=512, max_len=10368, rms_eps=1e-6)
+    start, steps = 5000, 5200
+    toks = []
+    for graph in (True, False):
+        sess, _ = synthetic.build_session(shape, context=start, ln_jitter=0.1)
+        sess.use_graph(graph)
+        toks.append(sess.decode_greedy(3, start, steps))
+        sess.close()
+    assert toks[0].tolist() == toks[1].tolist()
+
+
 def test_small_model_greedy_feedback_matches_stepwise(oracle):
     sess, host = synthetic.build_session(SMALL, context=16, keep_host=True, ln_jitter=0.1)
     toks = sess.decode_greedy(5, 16, 24)
