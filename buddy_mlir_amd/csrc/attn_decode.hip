@@ -24,6 +24,8 @@
 // folds them in chunk order with the reference's own combine rule.
 #include "attn.h"
 
+#include <type_traits>
+
 #include <atomic>
 
 namespace bh {
@@ -393,53 +395,63 @@ __global__ void __launch_bounds__(kWaves * 64)
       kreg[i] = *reinterpret_cast<const float4 *>(knew_s + c4 * 4);
       vreg[i] = *reinterpret_cast<const float4 *>(vnew_s + c4 * 4);
     }
-  for (int hh = h_lo; hh < h_hi; ++hh) {
-    const float4 q4 = *reinterpret_cast<const float4 *>(q_s[hh] + c4 * 4);
-    float sc[kR];
+  // The launch is bound by its vector instructions at long contexts, and every
+  // chunk but the one the position lies in is visible whole: those run without the
+  // comparisons and selects of the mask.
+  auto heads_pass = [&](auto whole_chunk) {
+    constexpr bool kWhole = decltype(whole_chunk)::value;
+    for (int hh = h_lo; hh < h_hi; ++hh) {
+      const float4 q4 = *reinterpret_cast<const float4 *>(q_s[hh] + c4 * 4);
+      float sc[kR];
 #pragma unroll
-    for (int i = 0; i < kR; ++i) {
-      const int p = pw0 + par + 2 * i;
-      const float4 k4 = kreg[i];
-      float d = fmaf(q4.x, k4.x, fmaf(q4.y, k4.y, fmaf(q4.z, k4.z, q4.w * k4.w)));
-      d = row16_sum(d);
-      d += __shfl_xor(d, 16, 64);
-      sc[i] = p <= pos ? d * a.scale : -INFINITY;
-    }
-    float m_w = kSeedM;
+      for (int i = 0; i < kR; ++i) {
+        const int p = pw0 + par + 2 * i;
+        const float4 k4 = kreg[i];
+        float d = fmaf(q4.x, k4.x, fmaf(q4.y, k4.y, fmaf(q4.z, k4.z, q4.w * k4.w)));
+        d = row16_sum(d);
+        d += __shfl_xor(d, 16, 64);
+        sc[i] = kWhole || p <= pos ? d * a.scale : -INFINITY;
+      }
+      float m_w = kSeedM;
 #pragma unroll
-    for (int i = 0; i < kR; ++i)
-      m_w = fmaxf(m_w, sc[i]);
-    m_w = fmaxf(m_w, __shfl_xor(m_w, 32, 64));
-    float l_w = 0.f;
+      for (int i = 0; i < kR; ++i)
+        m_w = fmaxf(m_w, sc[i]);
+      m_w = fmaxf(m_w, __shfl_xor(m_w, 32, 64));
+      float l_w = 0.f;
 #pragma unroll
-    for (int i = 0; i < kR; ++i) {
-      sc[i] = fast_exp(sc[i] - m_w);
-      l_w += sc[i];
-    }
-    l_w += __shfl_xor(l_w, 32, 64);
-    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+      for (int i = 0; i < kR; ++i) {
+        sc[i] = fast_exp(sc[i] - m_w);
+        l_w += sc[i];
+      }
+      l_w += __shfl_xor(l_w, 32, 64);
+      float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
 #pragma unroll
-    for (int i = 0; i < kR; ++i) {
-      const int p = pw0 + par + 2 * i;
-      const float4 v = vreg[i];
-      if (p <= pos) { // rows beyond the position may hold anything
+      for (int i = 0; i < kR; ++i) {
+        const int p = pw0 + par + 2 * i;
+        float4 v = vreg[i];
+        if (!kWhole && p > pos) // rows beyond the position may hold anything
+          v = make_float4(0.f, 0.f, 0.f, 0.f);
         acc.x = fmaf(v.x, sc[i], acc.x);
         acc.y = fmaf(v.y, sc[i], acc.y);
         acc.z = fmaf(v.z, sc[i], acc.z);
         acc.w = fmaf(v.w, sc[i], acc.w);
       }
+      acc.x += __shfl_xor(acc.x, 32, 64);
+      acc.y += __shfl_xor(acc.y, 32, 64);
+      acc.z += __shfl_xor(acc.z, 32, 64);
+      acc.w += __shfl_xor(acc.w, 32, 64);
+      if (lane < 32)
+        *reinterpret_cast<float4 *>(&accw_s[((size_t)hh * kWaves + wave) * kD + c4 * 4]) = acc;
+      if (lane == 0) {
+        mw_s[hh][wave] = m_w;
+        lw_s[hh][wave] = l_w;
+      }
     }
-    acc.x += __shfl_xor(acc.x, 32, 64);
-    acc.y += __shfl_xor(acc.y, 32, 64);
-    acc.z += __shfl_xor(acc.z, 32, 64);
-    acc.w += __shfl_xor(acc.w, 32, 64);
-    if (lane < 32)
-      *reinterpret_cast<float4 *>(&accw_s[((size_t)hh * kWaves + wave) * kD + c4 * 4]) = acc;
-    if (lane == 0) {
-      mw_s[hh][wave] = m_w;
-      lw_s[hh][wave] = l_w;
-    }
-  }
+  };
+  if (p0 + kChunk - 1 <= pos)
+    heads_pass(std::true_type{});
+  else
+    heads_pass(std::false_type{});
   __syncthreads();
   // ---- the wavefronts meet, once for all heads: one partial per (head, chunk) --
   for (int i = tid; i < (h_hi - h_lo) * kD; i += kWaves * 64) {
