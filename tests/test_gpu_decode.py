@@ -466,6 +466,27 @@ def test_long_context_steps_for_every_size_of_head_group(oracle, heads, kv_heads
     sess.close()
 
 
+@pytest.mark.parametrize("start", [17000, 66000])
+def test_fold_of_more_partials_than_one_pass_takes(oracle, start):
+    """The launch that folds the partials far into a long cache takes 128 of them
+    per head in its first pass and keeps the (max, sum) pairs of up to 256 in
+    registers: with one KV head 17000 positions are 136 partials of 128
+    positions, 66000 are 260 of 256."""
+    shape = Shape(layers=1, hidden=256, heads=2, kv_heads=1, head_dim=128, inter=256,
+                  vocab=512, max_len=start + 64, rms_eps=1e-6)
+    sess, host = synthetic.build_session(shape, context=start, keep_host=True, ln_jitter=0.1)
+    om = oracle_model(oracle, shape, host)
+    kv = [a.copy() for a in host["kv"]]
+    tok = 3
+    for step in range(4):
+        nxt, logits = sess.decode(tok, start + step)
+        otok, ologits = om.decode_step(tok, start + step, kv)
+        check_close(logits, ologits)
+        assert nxt == otok
+        tok = otok
+    sess.close()
+
+
 def test_a_long_generation_outlives_the_captured_steps_it_keeps():
     """A session keeps a captured step per cut of the attention and lets the oldest
     go after eight: 5200 greedy steps from position 5000 pass more cuts than that
