@@ -378,25 +378,32 @@ __global__ void __launch_bounds__(kSlices *kWave) gemm_w8_i8_kernel(
       cur = nxt;
   }
 
-  float *mine = red + (size_t)wave * 64 * kWave;
-#pragma unroll
-  for (int g = 0; g < kSplitGroups; ++g)
-#pragma unroll
-    for (int rb = 0; rb < 4; ++rb)
-#pragma unroll
-      for (int r = 0; r < 4; ++r)
-        mine[((g * 4 + rb) * 4 + r) * kWave + lane] = combine<D>(acc[g][rb], r);
-  __syncthreads();
-  const int g = wave; // wavefront w finishes channel group w
-  if (g0 + g >= a.groups)
-    return;
+  // wavefront w finishes channel group w: its scales, bias and the steps of the
+  // rows are asked for here, ahead of the meeting in LDS, not at their use
+  const int g = wave;
   const int n = (g0 + g) * kTileN + (lane >> 4) * 4;
-  float s[4], b[4];
+  float s[4], b[4], row_step[4];
 #pragma unroll
   for (int r = 0; r < 4; ++r) {
     s[r] = n + r < a.N ? a.scale[n + r] : 0.f;
     b[r] = (a.bias && n + r < a.N) ? a.bias[n + r] : 0.f;
   }
+#pragma unroll
+  for (int rb = 0; rb < 4; ++rb) {
+    const int m = m0 + rb * 16 + (lane & 15);
+    row_step[rb] = m < a.M ? a.steps[m] : 0.f;
+  }
+  float *mine = red + (size_t)wave * 64 * kWave;
+#pragma unroll
+  for (int gg = 0; gg < kSplitGroups; ++gg)
+#pragma unroll
+    for (int rb = 0; rb < 4; ++rb)
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        mine[((gg * 4 + rb) * 4 + r) * kWave + lane] = combine<D>(acc[gg][rb], r);
+  __syncthreads();
+  if (g0 + g >= a.groups)
+    return;
   const bool vec = n + 3 < a.N && (a.ldc & 3) == 0 &&
                    (reinterpret_cast<uintptr_t>(a.C) & 15) == 0;
 #pragma unroll
@@ -413,7 +420,7 @@ __global__ void __launch_bounds__(kSlices *kWave) gemm_w8_i8_kernel(
     }
     if (m >= a.M)
       continue;
-    store_row(a, m, n, a.steps[m], v, s, b, vec);
+    store_row(a, m, n, row_step[rb], v, s, b, vec);
   }
 }
 
@@ -448,8 +455,28 @@ __global__ void __launch_bounds__(kSlices *kWave) gemm_w8_i8_kernel(
 // invalidate a whole L2 each time and slowed the running workgroups threefold.)
 template <int GPW> struct RingDepth { static constexpr int value = GPW > 4 ? 4 : 5; };
 
+// LDS of the wide kernel: three fragment buffers in the loop, four output tiles in
+// the epilogue (and with PAIR the values that cross from wavefronts 2 and 3 to 0
+// and 1); behind them, with PAIR, the scales of the workgroup's channels of both
+// matrices and the steps of its rows, fetched once as the launch starts (loaded
+// at their use, every one of them was an L2 round trip the epilogue waited out).
+template <int D, int RB, int GPW, bool PAIR> constexpr size_t wide_main_lds_bytes() {
+  const size_t loop = sizeof(v4i32) * 3 * D * RB * kWave;
+  const size_t epi = sizeof(float) * kSlices * 16 * (GPW * 16 + 4) +
+                     (PAIR ? sizeof(float4) * kSlices * ((RB + 1) / 2) * GPW * kWave : 0);
+  return loop > epi ? loop : epi;
+}
+template <int RB, int GPW> constexpr int wide_epi_scales() { return 2 * 2 * GPW * 16; }
+template <int D, int RB, int GPW, bool PAIR> constexpr size_t wide_lds_bytes() {
+  return wide_main_lds_bytes<D, RB, GPW, PAIR>() +
+         (PAIR ? sizeof(float) * (wide_epi_scales<RB, GPW>() + RB * 16) : 0);
+}
+
 __device__ __forceinline__ void issue_load(v4i32 &dst, const void *p) {
   asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(dst) : "v"(p) : "memory");
+}
+__device__ __forceinline__ void issue_load_f32(float &dst, const void *p) {
+  asm volatile("global_load_dword %0, %1, off" : "=v"(dst) : "v"(p) : "memory");
 }
 template <int D, int GPW> struct FetchRegs {
   v4i32 w[GPW];
@@ -559,10 +586,47 @@ __global__ void __launch_bounds__(kSlices *kWave) gemm_w8_i8_wide_kernel(
     for (int rb = 0; rb < RB; ++rb)
       dst[rb] = frag_s[(((size_t)buf * D + j) * RB + rb) * kWave + lane];
   };
+  // PAIR: the epilogue's scales (both matrices, this workgroup's 64 GPW channels)
+  // and row steps, two per thread, requested ahead of the stream (so the counted
+  // waits below cover them) and parked in LDS for the epilogue
+  constexpr int kEpiScales = wide_epi_scales<RB, GPW>(); // [matrix][32 GPW channels]
+  float *epi_s = reinterpret_cast<float *>(frag_s) +
+                 wide_main_lds_bytes<D, RB, GPW, PAIR>() / sizeof(float);
+  float epi_v[2] = {0.f, 0.f};
+  bool epi_ok[2] = {false, false};
+  if constexpr (PAIR) {
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      const int idx = tid + u * kSlices * kWave;
+      const float *src = a.scale; // a valid address for the slots past the end
+      if (idx < kEpiScales) {
+        const int mtx = idx / (kEpiScales / 2), ch = idx % (kEpiScales / 2);
+        const int n = col * (kEpiScales / 2) + ch;
+        epi_ok[u] = n < a.N;
+        if (epi_ok[u])
+          src = a.scale + (size_t)mtx * a.N + n;
+      } else if (idx < kEpiScales + RB * 16) {
+        const int mr = m0 + idx - kEpiScales;
+        epi_ok[u] = mr < a.M;
+        if (epi_ok[u])
+          src = a.steps + mr;
+      }
+      issue_load_f32(epi_v[u], src);
+    }
+  }
 #pragma unroll
   for (int u = 0; u < kRing; ++u)
     fetch(u, ring[u]);
   wait_loads<(kRing - 1) * L, D, GPW>(ring[0]); // chunk 0 has arrived
+  if constexpr (PAIR) {
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      asm volatile("" : "+v"(epi_v[u])::"memory"); // older than chunk 0: landed
+      const int idx = tid + u * kSlices * kWave;
+      if (idx < kEpiScales + RB * 16)
+        epi_s[idx] = epi_ok[u] ? epi_v[u] : 0.f;
+    }
+  }
   stage(ring[0], 0);
   wait_loads<(kRing - 2) * L, D, GPW>(ring[1]);
   stage(ring[1], 1);
@@ -672,10 +736,9 @@ __global__ void __launch_bounds__(kSlices *kWave) gemm_w8_i8_wide_kernel(
   auto finished = [&](int g, int rb, float step) {
     float4 o;
     if constexpr (PAIR) {
-      const int n = (g0 + g) * kTileN + (lane >> 4) * 4;
-      float4 sc = make_float4(0.f, 0.f, 0.f, 0.f);
-      if (n < a.N)
-        sc = *reinterpret_cast<const float4 *>(a.scale + (wave >> 1) * a.N + n);
+      const float4 sc = *reinterpret_cast<const float4 *>(
+          epi_s + (wave >> 1) * (kEpiScales / 2) + ((wave & 1) * GPW + g) * kTileN +
+          (lane >> 4) * 4);
       o.x = scaled<D>(combine<D>(acc[g][rb], 0), step, sc.x);
       o.y = scaled<D>(combine<D>(acc[g][rb], 1), step, sc.y);
       o.z = scaled<D>(combine<D>(acc[g][rb], 2), step, sc.z);
@@ -701,8 +764,7 @@ __global__ void __launch_bounds__(kSlices *kWave) gemm_w8_i8_wide_kernel(
     for (int rb = 0; rb < RB; ++rb) {
       if (second ? rb >= kUpper : rb < kUpper)
         continue; // stays here
-      const int mr = m0 + rb * 16 + (lane & 15);
-      const float step = mr < a.M ? a.steps[mr] : 0.f;
+      const float step = epi_s[kEpiScales + rb * 16 + (lane & 15)];
       const int slot = rb < kUpper ? rb : rb - kUpper;
 #pragma unroll
       for (int g = 0; g < GPW; ++g)
@@ -715,7 +777,11 @@ __global__ void __launch_bounds__(kSlices *kWave) gemm_w8_i8_wide_kernel(
     if (PAIR && (second ? rb < kUpper : rb >= kUpper))
       continue; // the partner wavefront finishes this row block
     const int mr = m0 + rb * 16 + (lane & 15);
-    const float step = mr < a.M ? a.steps[mr] : 0.f;
+    float step;
+    if constexpr (PAIR)
+      step = epi_s[kEpiScales + rb * 16 + (lane & 15)];
+    else
+      step = mr < a.M ? a.steps[mr] : 0.f;
 #pragma unroll
     for (int g = 0; g < GPW; ++g) {
       float4 o = finished(g, rb, step);
@@ -803,6 +869,25 @@ __device__ __forceinline__ void sum_slices(const float *p, size_t slice_stride, 
   }
 }
 
+// What finishes four neighbouring outputs: scales, bias and (accumulating) the old
+// values, asked for in one go before the slices are summed -- loaded at their
+// use, each was an L2 round trip of its own behind the sum.
+struct FinishOperands {
+  float scale[4], bias[4], old[4];
+};
+__device__ __forceinline__ FinishOperands load_finish_operands(const GemmI8Args &a, const float *c,
+                                                              int n) {
+  FinishOperands f;
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const bool in = n + r < a.N;
+    f.scale[r] = in ? a.scale[n + r] : 0.f;
+    f.bias[r] = (in && a.bias) ? a.bias[n + r] : 0.f;
+    f.old[r] = (in && a.accumulate) ? c[r] : 0.f;
+  }
+  return f;
+}
+
 // C (+)= step[m] * scale[n] * sum over slices of the unscaled sums, slice order.
 __global__ void __launch_bounds__(256)
 reduce_slices_kernel(GemmI8Args a, int rb_per_tile, int gpw) {
@@ -818,15 +903,16 @@ reduce_slices_kernel(GemmI8Args a, int rb_per_tile, int gpw) {
   const size_t slice_stride = (size_t)kSlices * rb_per_tile * sub;
   const float *p = a.partial + ((size_t)(rbk * a.ncols + col) * a.slices) * slice_stride +
                    ((size_t)wave * rb_per_tile + rb) * sub + row * span + ch;
-  float v[4];
-  sum_slices(p, slice_stride, a.slices, v);
   const float step = a.steps[m];
   float *c = a.C + (int64_t)m * a.ldc + n;
+  const FinishOperands f = load_finish_operands(a, c, n);
+  float v[4];
+  sum_slices(p, slice_stride, a.slices, v);
 #pragma unroll
   for (int r = 0; r < 4; ++r)
     if (n + r < a.N) {
-      const float o = (a.bias ? a.bias[n + r] : 0.f) + (v[r] * step) * a.scale[n + r];
-      c[r] = a.accumulate ? c[r] + o : o;
+      const float o = f.bias[r] + (v[r] * step) * f.scale[r];
+      c[r] = a.accumulate ? f.old[r] + o : o;
     }
 }
 
@@ -899,15 +985,16 @@ reduce_slices_norm_kernel(const float *p_partial, const float *p_steps, int p_N,
     const int col = n / (kSlices * span), wave = (n / span) % kSlices, ch = n % span;
     const float *p = a.partial + ((size_t)(rbk * a.ncols + col) * a.slices) * slice_stride +
                      ((size_t)wave * rb_per_tile + rb) * sub + row * span + ch;
+    float *c = a.C + (int64_t)m * a.ldc + n;
+    const FinishOperands f = load_finish_operands(a, c, n);
     float v[4];
     sum_slices(p, slice_stride, a.slices, v);
-    float *c = a.C + (int64_t)m * a.ldc + n;
 #pragma unroll
     for (int r = 0; r < 4; ++r)
       if (n + r < a.N) {
-        float o = (a.bias ? a.bias[n + r] : 0.f) + (v[r] * step) * a.scale[n + r];
+        float o = f.bias[r] + (v[r] * step) * f.scale[r];
         if (a.accumulate)
-          o += c[r];
+          o += f.old[r];
         c[r] = o;
         xrow[n + r] = o;
       }
@@ -933,12 +1020,7 @@ BH_VARIANT_FAMILY(SplitFamily, "gemm_w8_i8_kernel");
 
 template <int D, int RB, int GPW, bool PAIR = false>
 int launch_wide(const GemmI8Args &a, unsigned blocks, hipStream_t stream) {
-  // three fragment buffers in the loop, four output tiles in the epilogue (and
-  // with PAIR the values that cross from wavefronts 2 and 3 to 0 and 1)
-  constexpr size_t lds =
-      std::max(sizeof(v4i32) * 3 * D * RB * kWave,
-               sizeof(float) * kSlices * 16 * (GPW * 16 + 4) +
-                   (PAIR ? sizeof(float4) * kSlices * ((RB + 1) / 2) * GPW * kWave : 0));
+  constexpr size_t lds = wide_lds_bytes<D, RB, GPW, PAIR>();
   auto kernel = gemm_w8_i8_wide_kernel<D, RB, GPW, PAIR>;
   if (lds > 48 * 1024) {
     static DynLdsOnce dyn_lds;
