@@ -147,6 +147,9 @@ w8a8_gemv_kernel(const int4 *__restrict__ W, const int8_t *__restrict__ xq,
   const int g = blockIdx.x;
   const int per = (chunks + 3) / 4;
   const int t0 = min(wave * per, chunks), t1 = min(t0 + per, chunks);
+  // the two scales of the result: asked for with the first loads, not at the
+  // very end of the launch behind the meeting of the wavefronts
+  const float comb = *a_scale * wscale[min(g * 16 + (lane & 15), N - 1)];
   int acc[M];
 #pragma unroll
   for (int m = 0; m < M; ++m)
@@ -182,14 +185,12 @@ w8a8_gemv_kernel(const int4 *__restrict__ W, const int8_t *__restrict__ xq,
   if (wave == 0 && lane < 16) {
     const int n = g * 16 + lane;
     if (n < N) {
-      const float sa = *a_scale;
 #pragma unroll
       for (int m = 0; m < M; ++m) {
         if (m < rows) {
           const int tot = red[0][m][lane] + red[1][m][lane] + red[2][m][lane] + red[3][m][lane];
           if (acc_out)
             acc_out[(size_t)m * N + n] = tot;
-          const float comb = sa * wscale[n];
           C[(size_t)m * N + n] = (float)tot * comb;
         }
       }
