@@ -148,6 +148,14 @@ finish_step_kernel(const float *__restrict__ pv, const int *__restrict__ pi,
   __shared__ int si[16];
   __shared__ int s_tok, s_pos;
   const int threads = blockDim.x; // 256, or 1024 for thousands of candidates
+  // token, position and step count: asked for with the first loads, not behind
+  // the pick (only thread 0 uses them)
+  int st_tok = 0, st_pos = 0, st_step = 0;
+  if (threadIdx.x == 0) {
+    st_tok = state[0];
+    st_pos = state[1];
+    st_step = state[2];
+  }
   if (nparts > 0) {
     float v = -INFINITY;
     int idx = 0x7fffffff;
@@ -182,18 +190,21 @@ finish_step_kernel(const float *__restrict__ pv, const int *__restrict__ pi,
       if (idx == 0x7fffffff)
         idx = 0;
       // the host bounds the step count; a counter outside the log writes nothing
-      if ((unsigned)state[2] < (unsigned)log_cap)
-        token_log[state[2]] = idx;
+      if ((unsigned)st_step < (unsigned)log_cap)
+        token_log[st_step] = idx;
       state[0] = idx;
+      st_tok = idx;
     }
   }
   if (threadIdx.x == 0) {
     if (advance) {
-      state[1] += 1;
-      state[2] += 1;
+      st_pos += 1;
+      st_step += 1;
+      state[1] = st_pos;
+      state[2] = st_step;
     }
-    s_tok = state[0];
-    s_pos = state[1];
+    s_tok = st_tok;
+    s_pos = st_pos;
   }
   __syncthreads();
   int64_t t = s_tok;
